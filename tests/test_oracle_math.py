@@ -1,0 +1,243 @@
+"""Pins the CPU oracle where the ONNX vectors leave it open: against independent
+numpy restatements (different code, different loop structure), closed forms and
+invariants.  A dropped term, a wrong sign, a transposed operand or a wrong pad
+side fails at least one test here."""
+import numpy as np
+import pytest
+
+
+def np_quantize(x, scale, zp, lo, hi):
+    """quantize_array (runtime/ops/quantize.cc:16-35) spelled in numpy fp32 ops."""
+    s = x.astype(np.float32) / np.float32(scale)
+    if zp != 0:
+        s = s + np.float32(zp)
+    s = np.maximum(np.float32(lo), np.minimum(s, np.float32(hi))) + np.float32(0.5)
+    return np.trunc(s).astype(np.int64)
+
+
+@pytest.mark.parametrize("dtype,zp,scale", [(np.uint8, 128, 0.02), (np.uint8, 0, 1.0 / 255), (np.int8, 0, 0.05),
+                                            (np.int8, -7, 0.3), (np.uint8, 255, 3.0), (np.int8, 127, 1e-3)])
+def test_quantize_vs_numpy(oracle, dtype, zp, scale):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 10,
+                        np.array([0, -0.0, 1e-30, -1e-30, 1e30, -1e30, 0.5 * scale, 1.5 * scale, 2.5 * scale,
+                                  -0.5 * scale, -1.5 * scale], np.float32),
+                        (np.arange(-300, 300, dtype=np.float32) + 0.5) * np.float32(scale)])
+    lo, hi = (0, 255) if dtype == np.uint8 else (-128, 127)
+    got = oracle.quantize_linear(x, scale, zp, dtype)
+    np.testing.assert_array_equal(got.astype(np.int64), np_quantize(x, scale, zp, lo, hi))
+    # range + monotone non-decreasing in x
+    order = np.argsort(x, kind="stable")
+    assert np.all(np.diff(got[order].astype(np.int64)) >= 0)
+    assert got.min() >= lo and got.max() <= hi
+
+
+def test_quantize_int8_truncation_quirk(oracle):
+    # +0.5f then a truncating cast rounds negative values toward zero-ish:
+    # -1.7 -> -1.2 -> -1 (a round-to-nearest would give -2).  runtime/ops/quantize.cc:34.
+    y = oracle.quantize_linear(np.array([-1.7, -1.2, -0.6, 1.7], np.float32), 1.0, 0, np.int8)
+    assert y.tolist() == [-1, 0, 0, 2]
+    y = oracle.quantize_linear(np.array([-1.7, 2.5, 3.5], np.float32), 1.0, 0, np.int8, round_mode=oracle.ROUND_ONNX_RNE)
+    assert y.tolist() == [-2, 2, 4]
+    # -128 is unreachable for int8 under the reference rule (clip to -128, +0.5, truncate -> -127)
+    assert oracle.quantize_linear(np.array([-1e9], np.float32), 1.0, 0, np.int8).tolist() == [-127]
+
+
+@pytest.mark.parametrize("dtype,zp", [(np.uint8, 0), (np.uint8, 128), (np.uint8, 255)])
+@pytest.mark.parametrize("scale", [0.05, 1.0 / 255, 2.0, 0.00369204697])
+def test_quantize_of_dequantize_is_identity(oracle, dtype, zp, scale):
+    q = np.arange(0, 256).astype(dtype)
+    x = oracle.dequantize_linear(q, scale, zp)
+    np.testing.assert_array_equal(x, ((q.astype(np.float32) - np.float32(zp)) * np.float32(scale)))
+    np.testing.assert_array_equal(oracle.quantize_linear(x, scale, zp, dtype), q)
+
+
+def test_dequantize_exhaustive_int8(oracle):
+    q = np.arange(-128, 128).astype(np.int8)
+    for zp in (0, -5, 127):
+        x = oracle.dequantize_linear(q, 0.1, zp)
+        want = (q.astype(np.float64) - zp) * float(np.float32(0.1))
+        np.testing.assert_array_equal(x, want.astype(np.float32))  # exact product fits? compare after fp32 rounding
+        np.testing.assert_array_equal(x, oracle.dequantize_linear(q, 0.1, zp, multipass=True))
+
+
+@pytest.mark.parametrize("adt,bdt", [(np.uint8, np.int8), (np.uint8, np.uint8), (np.int8, np.int8)])
+def test_matmul_integer_vs_int64(oracle, adt, bdt):
+    rng = np.random.default_rng(2)
+    lo_a, hi_a = (0, 256) if adt == np.uint8 else (-128, 128)
+    lo_b, hi_b = (0, 256) if bdt == np.uint8 else (-128, 128)
+    a = rng.integers(lo_a, hi_a, size=(3, 5, 37)).astype(adt)
+    b = rng.integers(lo_b, hi_b, size=(3, 37, 11)).astype(bdt)
+    bz = rng.integers(lo_b, hi_b, size=11).astype(bdt)
+    az = np.array([7]).astype(adt)
+    want = np.einsum("bmk,bkn->bmn", a.astype(np.int64) - int(az[0]), b.astype(np.int64) - bz.astype(np.int64)[None, None, :])
+    np.testing.assert_array_equal(oracle.matmul_integer(a, b, az, bz), want)
+    np.testing.assert_array_equal(oracle.matmul_integer(a[0], b[0], None, None), a[0].astype(np.int64) @ b[0].astype(np.int64))
+
+
+
+def np_conv_int64(x, w, strides, pads4, group):
+    """Independent int64 convolution: explicit zero padding + window slicing."""
+    N, C, H, W = x.shape
+    OC, Cg, KH, KW = w.shape
+    ph0, pw0, ph1, pw1 = pads4
+    xp = np.zeros((N, C, H + ph0 + ph1, W + pw0 + pw1), np.int64)
+    xp[:, :, ph0:ph0 + H, pw0:pw0 + W] = x
+    OH = (H + ph0 + ph1 - KH) // strides[0] + 1
+    OW = (W + pw0 + pw1 - KW) // strides[1] + 1
+    y = np.zeros((N, OC, OH, OW), np.int64)
+    OCg = OC // group
+    for g in range(group):
+        xs = xp[:, g * Cg:(g + 1) * Cg]
+        ws = w[g * OCg:(g + 1) * OCg]
+        for oh in range(OH):
+            for ow in range(OW):
+                win = xs[:, :, oh * strides[0]:oh * strides[0] + KH, ow * strides[1]:ow * strides[1] + KW]
+                y[:, g * OCg:(g + 1) * OCg, oh, ow] = np.tensordot(win, ws, axes=([1, 2, 3], [1, 2, 3]))
+    return y
+
+
+CONV_CASES = [
+    # N, C, H, W, OC, KH, KW, strides, pads, group
+    (2, 4, 7, 6, 6, 3, 3, (1, 1), (1, 1), 1),
+    (1, 6, 9, 8, 4, 3, 2, (2, 1), (0, 1), 2),
+    (2, 8, 5, 5, 8, 3, 3, (1, 1), (1, 1), 8),     # depthwise
+    (1, 3, 11, 11, 5, 7, 7, (2, 2), (3, 3), 1),   # stem-like
+    (1, 5, 6, 7, 3, 1, 1, (2, 2), (0, 0), 1),     # strided pointwise
+    (1, 2, 5, 4, 2, 3, 3, (2, 2), (0, 0, 1, 1), 1),  # asymmetric (what SAME_UPPER produces)
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("wdt", [np.int8, np.uint8])
+def test_conv_integer_vs_int64(oracle, case, wdt):
+    N, C, H, W, OC, KH, KW, strides, pads, group = case
+    rng = np.random.default_rng(3)
+    x = rng.integers(0, 256, size=(N, C, H, W)).astype(np.uint8)
+    lo, hi = (0, 256) if wdt == np.uint8 else (-128, 128)
+    w = rng.integers(lo, hi, size=(OC, C // group, KH, KW)).astype(wdt)
+    wz = rng.integers(lo, hi, size=OC).astype(wdt)
+    xz = 131
+    pads4 = pads if len(pads) == 4 else (pads[0], pads[1], pads[0], pads[1])
+    want = np_conv_int64(x.astype(np.int64) - xz, w.astype(np.int64) - wz.astype(np.int64)[:, None, None, None],
+                         strides, pads4, group)
+    got = oracle.conv_integer(x, w, xz, wz, strides=strides, pads=pads, group=group)
+    np.testing.assert_array_equal(got, want)
+    # scalar w zero point and none
+    want0 = np_conv_int64(x.astype(np.int64), w.astype(np.int64) - int(wz[0]), strides, pads4, group)
+    np.testing.assert_array_equal(oracle.conv_integer(x, w, None, wz[:1], strides=strides, pads=pads, group=group), want0)
+
+
+def test_same_upper_autopad(oracle):
+    # CalculateAutoPad (runtime/chainerx_util.cc:276-311): out = ceil(in/stride); extra pad goes to the END
+    assert oracle.same_upper_pads(5, 2, 3) == (1, 1)
+    assert oracle.same_upper_pads(4, 2, 3) == (0, 1)
+    assert oracle.same_upper_pads(28, 1, 3) == (1, 1)
+    assert oracle.same_upper_pads(224, 2, 7) == (2, 3)
+    rng = np.random.default_rng(4)
+    x = rng.integers(0, 256, size=(1, 2, 4, 4)).astype(np.uint8)
+    w = rng.integers(-128, 128, size=(3, 2, 3, 3)).astype(np.int8)
+    got = oracle.conv_integer(x, w, 3, None, strides=(2, 2), pads=(0, 0), auto_pad="SAME_UPPER")
+    want = np_conv_int64(x.astype(np.int64) - 3, w.astype(np.int64), (2, 2), (0, 0, 1, 1), 1)
+    assert got.shape == (1, 3, 2, 2)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("bias_mode", ["none", "reference_float", "onnx_int32"])
+def test_qlinear_conv_int_equals_literal_on_power_of_two_scales(oracle, case, bias_mode):
+    """With power-of-two scales and |acc| < 2^24 every fp32 product and partial sum
+    of the literal path is exact, so both oracles must agree bit for bit."""
+    N, C, H, W, OC, KH, KW, strides, pads, group = case
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 256, size=(N, C, H, W)).astype(np.uint8)
+    w = rng.integers(-127, 128, size=(OC, C // group, KH, KW)).astype(np.int8)
+    ws = (2.0 ** rng.integers(-9, -5, size=OC)).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-1000, 1001, size=OC).astype(np.int32)
+    kw = dict(strides=strides, pads=pads, group=group)
+    if bias_mode == "none":
+        kw.update(bias=None)
+    elif bias_mode == "reference_float":
+        kw.update(bias=bias, bias_mode=oracle.BIAS_REFERENCE_FLOAT)
+    else:
+        kw.update(bias=bias, bias_mode=oracle.BIAS_ONNX_INT32)
+    args = (x, 2.0 ** -6, 128, w, ws, wz, 2.0 ** -3, 128)
+    a = oracle.qlinear_conv_int(*args, **kw)
+    b = oracle.qlinear_conv_literal(*args, **kw)
+    np.testing.assert_array_equal(a, b)
+    assert a.min() < a.max()  # not saturated into a constant
+
+
+def test_qlinear_conv_int_closed_form_1x1(oracle):
+    """1x1 conv, one channel: y = Q((x - xz) * (w - wz) * xs * ws) element by element."""
+    x = np.arange(256, dtype=np.uint8).reshape(1, 1, 16, 16)
+    w = np.array([[[[-3]]]], np.int8)
+    xs, ws, ys, xz, yz = np.float32(0.02), np.float32(0.007), np.float32(0.05), 128, 128
+    acc = (x.astype(np.int64) - xz) * -3
+    v = acc.astype(np.float32) * np.float32(xs * ws)
+    want = np_quantize(v, ys, yz, 0, 255)
+    got = oracle.qlinear_conv_int(x, xs, xz, w, np.array([ws]), np.array([0], np.int8), ys, yz)
+    np.testing.assert_array_equal(got.astype(np.int64), want)
+
+
+def test_qlinear_matmul_relu_and_bias(oracle):
+    rng = np.random.default_rng(6)
+    a = rng.integers(0, 256, size=(32, 100)).astype(np.uint8)
+    b = rng.integers(-127, 128, size=(100, 10)).astype(np.int8)
+    bias = rng.integers(-500, 500, size=10).astype(np.int32)
+    s_a, s_b, s_y = np.float32(1 / 255), np.float32(0.004), np.float32(0.02)
+    acc = (a.astype(np.int64) - 128) @ b.astype(np.int64) + bias
+    v = acc.astype(np.float32) * np.float32(s_a * s_b)
+    want = np_quantize(v, s_y, 128, 0, 255)
+    got = oracle.qlinear_matmul_int(a, s_a, 128, b, s_b, 0, s_y, 128, bias=bias)
+    np.testing.assert_array_equal(got.astype(np.int64), want)
+    got_relu = oracle.qlinear_matmul_int(a, s_a, 128, b, s_b, 0, s_y, 128, bias=bias, relu=True)
+    np.testing.assert_array_equal(got_relu.astype(np.int64), np.maximum(want, 128))
+    # fused Relu == Q(Relu(DQ(q))) spelled out with the element-wise oracle
+    dq = oracle.dequantize_linear(got, s_y, 128)
+    np.testing.assert_array_equal(oracle.quantize_linear(oracle.relu(dq), s_y, 128), got_relu)
+
+
+def ulp_diff(a, b):
+    a = np.asarray(a, np.float32).view(np.int32).astype(np.int64)
+    b = np.asarray(b, np.float32).view(np.int32).astype(np.int64)
+    a = np.where(a < 0, -(a & 0x7FFFFFFF), a)
+    b = np.where(b < 0, -(b & 0x7FFFFFFF), b)
+    return np.abs(a - b)
+
+
+def test_elementwise_ops_against_float64(oracle):
+    rng = np.random.default_rng(7)
+    x = np.concatenate([rng.standard_normal(100000).astype(np.float32) * 3,
+                        np.array([0, 1e-8, -1e-8, 0.5, 1, 21.9, 22, 30, -30, 88, -88, -104], np.float32)])
+    x64 = x.astype(np.float64)
+    assert ulp_diff(oracle.tanh(x), np.tanh(x64).astype(np.float32)).max() <= 2
+    assert ulp_diff(oracle.exp(x), np.exp(x64).astype(np.float32)).max() <= 1
+    assert ulp_diff(oracle.sigmoid(x), (1 / (1 + np.exp(-x64))).astype(np.float32)).max() <= 2
+    np.testing.assert_array_equal(oracle.relu(x), np.maximum(x, 0))
+    np.testing.assert_array_equal(oracle.clip(x, 0, 6), np.clip(x, 0, 6))
+    a = rng.standard_normal(1024).astype(np.float32)
+    x2 = rng.standard_normal((3, 5, 1024)).astype(np.float32)
+    np.testing.assert_array_equal(oracle.binary(oracle.MUL, x2, a), x2 * a)
+    np.testing.assert_array_equal(oracle.binary(oracle.ADD, x2, np.float32(2.5)), x2 + np.float32(2.5))
+    np.testing.assert_array_equal(oracle.binary(oracle.SUB, a, x2), a - x2)
+    col = rng.standard_normal((3, 5, 1)).astype(np.float32)   # not a trailing-axis broadcast: materialised
+    np.testing.assert_array_equal(oracle.binary(oracle.DIV, x2, col), x2 / col)
+    np.testing.assert_array_equal(oracle.round_half_even(np.array([0.5, 1.5, 2.5, -0.5, -1.5], np.float32)),
+                                  np.array([0, 2, 2, -0, -2], np.float32))
+
+
+def test_chain_matches_stepwise_numpy(oracle):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((4, 8, 64)).astype(np.float32)
+    c = rng.standard_normal((4, 8, 64)).astype(np.float32)
+    a = rng.standard_normal(64).astype(np.float32)
+    b = rng.standard_normal(64).astype(np.float32)
+    prog = [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+            ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")]
+    env = oracle.run_chain(prog, dict(x=x, a=a, b=b, c=c))
+    t1 = x * a + b  # numpy rounds after each op as well
+    np.testing.assert_array_equal(env["t1"], t1)
+    want = np.maximum(oracle.tanh(t1) * oracle.sigmoid(c) + x, 0)
+    np.testing.assert_array_equal(env["y"], want)
