@@ -1,0 +1,113 @@
+"""ctypes binding of include/chx_hip.h.  Torch is used for device memory and the
+current stream only; every computation goes through libchx_hip.so, and a missing
+library is an error (there is no fallback path)."""
+import ctypes
+import os
+
+import torch
+
+MAX_NDIM = 10
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libchx_hip.so")
+
+# ChainerX dtype codes (compiler/dtype.h:14-25 of the reference tree)
+BOOL, INT8, INT16, INT32, INT64, UINT8, FLOAT16, FLOAT32, FLOAT64 = 1, 2, 3, 4, 5, 6, 7, 8, 9
+_TORCH_TO_CHX = {
+    torch.bool: BOOL, torch.int8: INT8, torch.int16: INT16, torch.int32: INT32, torch.int64: INT64,
+    torch.uint8: UINT8, torch.float16: FLOAT16, torch.float32: FLOAT32, torch.float64: FLOAT64,
+}
+
+ROUND_REFERENCE = 0
+ROUND_ONNX_RNE = 1
+BIAS_REFERENCE_FLOAT = 0
+BIAS_ONNX_INT32 = 2
+FUSE_RELU = 4
+
+EXPORTS = [
+    "chx_hip_init", "chx_hip_last_error", "chx_hip_version", "chx_hip_get_device_props", "chx_hip_malloc",
+    "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
+    "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
+    "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
+    "chx_hip_qlinear_matmul", "chx_hip_elementwise",
+]
+
+
+class Tensor(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("dtype", ctypes.c_int32), ("ndim", ctypes.c_int32),
+                ("shape", ctypes.c_int64 * MAX_NDIM), ("strides", ctypes.c_int64 * MAX_NDIM)]
+
+
+class ConvParams(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "stride_h", "stride_w", "pad_h_begin", "pad_w_begin", "pad_h_end", "pad_w_end", "group")]
+
+
+class DeviceProps(ctypes.Structure):
+    _fields_ = [("compute_units", ctypes.c_int32), ("clock_khz", ctypes.c_int32),
+                ("memory_clock_khz", ctypes.c_int32), ("memory_bus_bits", ctypes.c_int32),
+                ("total_memory", ctypes.c_int64), ("arch", ctypes.c_char * 64), ("name", ctypes.c_char * 128)]
+
+
+class ChxHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("chx_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(there is no CPU fallback for the device ops)" % LIB_PATH)
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.chx_hip_last_error.restype = ctypes.c_char_p
+        _lib.chx_hip_version.restype = ctypes.c_char_p
+        _lib.chx_hip_qconv_plan_destroy.restype = None
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise ChxHipError(rc, lib().chx_hip_last_error().decode("utf-8", "replace"))
+
+
+def desc(t):
+    """chx_hip_tensor for a torch device tensor (byte strides, like ChainerX)."""
+    d = Tensor()
+    d.data = t.data_ptr()
+    d.dtype = _TORCH_TO_CHX[t.dtype]
+    d.ndim = t.dim()
+    es = t.element_size()
+    for i in range(t.dim()):
+        d.shape[i] = t.shape[i]
+        d.strides[i] = t.stride(i) * es
+    return d
+
+
+def ref(t):
+    return None if t is None else ctypes.byref(desc(t))
+
+
+def stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def init(device=0):
+    check(lib().chx_hip_init(ctypes.c_int(device)))
+
+
+def device_props():
+    p = DeviceProps()
+    check(lib().chx_hip_get_device_props(ctypes.byref(p)))
+    return dict(compute_units=p.compute_units, clock_khz=p.clock_khz, memory_clock_khz=p.memory_clock_khz,
+                memory_bus_bits=p.memory_bus_bits, total_memory=p.total_memory, arch=p.arch.decode(),
+                name=p.name.decode())
+
+
+def conv_params(strides, pads_begin, pads_end, group):
+    return ConvParams(strides[0], strides[1], pads_begin[0], pads_begin[1], pads_end[0], pads_end[1], group)

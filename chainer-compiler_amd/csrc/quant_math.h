@@ -1,0 +1,79 @@
+// Device-side scalar arithmetic of the quantized ops, shared by every kernel that
+// quantizes, dequantizes or requantizes.  Each function is the reference's fp32
+// operation sequence; translation units including this header are compiled with
+// -ffp-contract=off so that no two operations merge into a fused multiply-add.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace chx {
+
+struct QuantParams {
+    float scale;  // y_scale
+    float zpf;    // float(y_zero_point); 0.0f when the reference skips the addition
+    float lo;     // 0 or -128
+    float hi;     // 255 or 127
+};
+
+inline QuantParams make_quant_params(float scale, int32_t zero_point, bool int8_out) {
+    QuantParams q;
+    q.scale = scale;
+    q.zpf = (float)zero_point;
+    q.lo = int8_out ? -128.f : 0.f;
+    q.hi = int8_out ? 127.f : 255.f;
+    return q;
+}
+
+// quantize_array, runtime/ops/quantize.cc:29-34:
+//   scaled = v / y_scale; if (zp != 0) scaled += zp;
+//   AsType(Maximum(lo, Minimum(scaled, hi)) + 0.5f)          (AsType truncates)
+// Adding zpf == 0.0f is the identity on every finite value except that it turns -0.0
+// into +0.0, which the clamp, the +0.5f and the truncation cannot tell apart, so the
+// reference's "skip when zero" needs no branch.
+// kRne selects the ONNX operator text instead: saturate(rint(v / y_scale) + zp).
+template <bool kRne>
+__device__ __forceinline__ int32_t quantize_value(float v, const QuantParams& q) {
+    float s = v / q.scale;  // IEEE-754 correctly rounded division
+    if (kRne) {
+        s = rintf(s) + q.zpf;
+        s = s < q.hi ? s : q.hi;
+        s = q.lo < s ? s : q.lo;
+        return (int32_t)s;
+    }
+    s = s + q.zpf;
+    s = s < q.hi ? s : q.hi;
+    s = q.lo < s ? s : q.lo;
+    s = s + 0.5f;
+    return (int32_t)s;  // v_cvt_i32_f32 truncates toward zero
+}
+
+// dequantize_array, runtime/ops/quantize.cc:37-44: (float(x) - zp) * scale.
+// Subtracting 0.0f is exact, so the "skip when zero" needs no branch either.
+__device__ __forceinline__ float dequantize_value(int32_t q, float zpf, float scale) {
+    float f = (float)q;
+    f = f - zpf;
+    return f * scale;
+}
+
+template <bool kSigned>
+__device__ __forceinline__ int32_t byte_of(uint32_t word, int i) {
+    const uint32_t b = (word >> (8 * i)) & 0xffu;
+    return kSigned ? (int32_t)(int8_t)b : (int32_t)b;
+}
+
+__device__ __forceinline__ uint32_t pack4(int32_t a, int32_t b, int32_t c, int32_t d) {
+    return ((uint32_t)a & 0xffu) | (((uint32_t)b & 0xffu) << 8) | (((uint32_t)c & 0xffu) << 16) |
+           (((uint32_t)d & 0xffu) << 24);
+}
+
+// Requantizing epilogue of the contractions: int32 accumulator -> 8-bit code.
+//   v = float(acc) * (x_scale * w_scale[oc])      (combined = fp32 product of the scales)
+//   bias per mode, then quantize_value.
+struct RequantParams {
+    QuantParams q;
+    int32_t relu_floor;  // lower clamp applied to the code (y_zero_point when Relu is fused, else INT32_MIN)
+};
+
+}  // namespace chx

@@ -1,0 +1,210 @@
+/*
+ * chx_hip.h -- C ABI of the MI355X (gfx950) quantized-inference kernels that sit
+ * under chainer-compiler's ChxVM op layer.
+ *
+ * Every entry point is what a ChxVM op's RunImpl body binds for this path; the
+ * reference interface each one replaces is cited as file:line of the
+ * chainer-compiler tree.  Plain pointers and sizes only; no C++ or torch types.
+ *
+ * Conventions
+ *   - Return value: 0 on success, a CHX_HIP_E* code otherwise; the message for
+ *     the calling thread's last failure is chx_hip_last_error().  No exceptions
+ *     cross this boundary and nothing aborts the process (the reference's
+ *     CHECK macros do, common/log.h:31-44; the RunImpl wrappers keep that
+ *     behaviour by CHECKing the return code).
+ *   - Tensors are described by chx_hip_tensor: device pointer, ChainerX dtype
+ *     code (compiler/dtype.h:14-25), shape and strides IN BYTES (ChainerX
+ *     arrays carry byte strides).  The caller allocates outputs; shape
+ *     inference stays in the RunImpl wrappers.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Calls only enqueue work; they synchronize with the host where the comment
+ *     of an entry point says so and nowhere else.
+ *   - Scales and zero points that ChxVM hands over as StrictScalar
+ *     (runtime/strict_scalar.h:8-34) are host values here.
+ *   - Activations may be given either NCHW-contiguous or as NCHW-shaped views of
+ *     channels-last (NHWC) memory; both are valid ChainerX arrays.  Channels-last
+ *     is the layout the MFMA kernels read and write without a transposition.
+ */
+#ifndef CHX_HIP_H_
+#define CHX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CHX_HIP_MAX_NDIM 10 /* chainerx::kMaxNdim */
+
+/* ChainerX dtype codes, compiler/dtype.h:14-25 */
+enum {
+    CHX_HIP_BOOL = 1,
+    CHX_HIP_INT8 = 2,
+    CHX_HIP_INT16 = 3,
+    CHX_HIP_INT32 = 4,
+    CHX_HIP_INT64 = 5,
+    CHX_HIP_UINT8 = 6,
+    CHX_HIP_FLOAT16 = 7,
+    CHX_HIP_FLOAT32 = 8,
+    CHX_HIP_FLOAT64 = 9
+};
+
+enum {
+    CHX_HIP_OK = 0,
+    CHX_HIP_EINVAL = 1,      /* bad argument: dtype, shape, stride, null pointer */
+    CHX_HIP_EUNSUPPORTED = 2,/* valid for the reference op but not implemented on the device */
+    CHX_HIP_ERUNTIME = 3,    /* a HIP / hiprtc call failed */
+    CHX_HIP_ECOMPILE = 4     /* run-time compilation of a fused kernel failed */
+};
+
+/* Behaviour switches.  0 is always the reference's behaviour. */
+enum {
+    /* rounding of QuantizeLinear and of every requantizing epilogue */
+    CHX_HIP_ROUND_REFERENCE = 0u,     /* AsType(clip(v/scale + zp) + 0.5f): runtime/ops/quantize.cc:29-34 */
+    CHX_HIP_ROUND_ONNX_RNE = 1u,      /* saturate(round_half_even(v/scale) + zp): the ONNX operator text */
+    /* how a QLinearConv bias enters */
+    CHX_HIP_BIAS_REFERENCE_FLOAT = 0u,/* float(b) added unscaled to the fp32 result: runtime/ops/quantize.cc:93 */
+    CHX_HIP_BIAS_ONNX_INT32 = 2u,     /* b added to the int32 accumulator (scale x_scale*w_scale) */
+    /* Q(Relu(DQ(q))) folded into the epilogue: output clamped below at y_zero_point */
+    CHX_HIP_FUSE_RELU = 4u
+};
+
+typedef struct chx_hip_tensor {
+    void* data;                        /* device address of element [0,0,...] */
+    int32_t dtype;                     /* CHX_HIP_* dtype code */
+    int32_t ndim;
+    int64_t shape[CHX_HIP_MAX_NDIM];
+    int64_t strides[CHX_HIP_MAX_NDIM]; /* bytes */
+} chx_hip_tensor;
+
+/* Convolution attributes after the RunImpl wrapper has completed them
+ * (ComplementStride/ComplementPad runtime/chainerx_util.cc:180-200 and
+ * CalculateAutoPad :276-311): explicit begin and end pads per spatial axis. */
+typedef struct chx_hip_conv_params {
+    int32_t stride_h, stride_w;
+    int32_t pad_h_begin, pad_w_begin;
+    int32_t pad_h_end, pad_w_end;
+    int32_t group;
+} chx_hip_conv_params;
+
+typedef struct chx_hip_device_props {
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int64_t total_memory;
+    char arch[64];
+    char name[128];
+} chx_hip_device_props;
+
+/* ---- library state ----------------------------------------------------------------- */
+
+/* Selects `device` for the calling thread and checks that it is a gfx950 part.
+ * Replaces nothing in the reference (ChainerX owns device selection there,
+ * tools/run_onnx.cc:343-357). */
+int chx_hip_init(int device);
+const char* chx_hip_last_error(void);
+const char* chx_hip_version(void);
+int chx_hip_get_device_props(chx_hip_device_props* out);
+
+/* Thin device-memory helpers for hosts that have no allocator of their own (the
+ * C++ ChxVM runtime mirror uses them where the reference uses chainerx::Empty /
+ * Device::MakeDataFromForeignPointer, runtime/chainerx_util.cc:60-120). */
+int chx_hip_malloc(void** ptr, size_t bytes);
+int chx_hip_free(void* ptr);
+int chx_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream); /* synchronizes the stream */
+int chx_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream); /* synchronizes the stream */
+int chx_hip_memset(void* dst, int value, size_t bytes, void* stream);
+int chx_hip_stream_synchronize(void* stream);
+
+/* ---- QuantizeLinear / DequantizeLinear ------------------------------------------------ */
+
+/* QuantizeLinearOp::RunImpl -> quantize_array, runtime/ops/quantize.cc:16-35,48-53.
+ * x float32; y uint8 or int8 (the dtype the zero point has in the reference),
+ * same shape.  One pass: y = cast(max(lo, min(x / y_scale + zp, hi)) + 0.5f). */
+int chx_hip_quantize_linear(
+        const chx_hip_tensor* x, float y_scale, int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
+
+/* DequantizeLinearOp::RunImpl -> dequantize_array, runtime/ops/quantize.cc:37-44,55-60.
+ * x uint8 or int8; y float32: y = (float(x) - zp) * x_scale. */
+int chx_hip_dequantize_linear(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, chx_hip_tensor* y, void* stream);
+
+/* ---- QLinearConv ---------------------------------------------------------------------- */
+
+/* QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94 (+ GroupedConv,
+ * runtime/chainerx_util.cc:313-340).
+ *   x uint8/int8 [N,C,H,W]; w int8/uint8 [OC,C/group,KH,KW]; w_scale float32 0-d or
+ *   [OC]; w_zero_point same element count as w_scale, dtype of w; bias int32 [OC] or
+ *   NULL; y uint8/int8 [N,OC,OH,OW].
+ * The contraction accumulates exactly in int32 and the epilogue evaluates
+ *   v = float(acc) * (x_scale * w_scale[oc]);  (+ bias per `flags`);  quantize_array(v)
+ * in that fp32 operation order.  Reads w_zero_point back to the host once per call
+ * (a stream synchronization) to pick the kernel; use a plan to avoid that. */
+int chx_hip_qlinear_conv(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
+        const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_params* params, uint32_t flags, chx_hip_tensor* y, void* stream);
+
+/* The same op with the weight-side work (repacking for the MFMA kernel, per-channel
+ * sums, the zero-point read-back) done once.  The reference redoes its weight
+ * dequantization on every call (runtime/ops/quantize.cc:76-88); a ChxVM op object
+ * lives as long as the program, so the wrapper keeps one plan per QLinearConv
+ * instruction, in the manner of the stateful backend ops (runtime/ops/tvm.cc:90-158).
+ * create() synchronizes the stream; run() does not.  The plan keeps pointers to
+ * w_scale and bias: they must stay alive and unchanged. */
+typedef struct chx_hip_qconv_plan chx_hip_qconv_plan;
+int chx_hip_qconv_plan_create(
+        const chx_hip_tensor* w, const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_params* params, void* stream, chx_hip_qconv_plan** plan);
+int chx_hip_qconv_plan_run(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
+        int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
+void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan);
+
+/* ---- integer contractions ------------------------------------------------------------- */
+
+/* ConvIntegerOp::RunImpl, runtime/ops/quantize.cc:116-146.  y int32 [N,OC,OH,OW].
+ * w_zero_point: NULL, 0-d or [OC]. */
+int chx_hip_conv_integer(
+        const chx_hip_tensor* x, const chx_hip_tensor* w, int32_t x_zero_point, const chx_hip_tensor* w_zero_point,
+        const chx_hip_conv_params* params, chx_hip_tensor* y, void* stream);
+
+/* MatMulIntegerOp::RunImpl, runtime/ops/quantize.cc:96-114 with NumpyMatMul,
+ * runtime/chainerx_util.cc:210-230.  a [..,M,K], b [..,K,N] with equal leading
+ * dims, y int32 [..,M,N].  Zero points: NULL, or arrays of ndim <= 1 subtracted by
+ * numpy broadcasting (a 1-D one lines up with the last axis: K for a, N for b). */
+int chx_hip_matmul_integer(
+        const chx_hip_tensor* a, const chx_hip_tensor* b, const chx_hip_tensor* a_zero_point,
+        const chx_hip_tensor* b_zero_point, chx_hip_tensor* y, void* stream);
+
+/* The instruction sequence DequantizeLinear, DequantizeLinear, MatMul, QuantizeLinear
+ * that ReplaceQLinearMatMul (compiler/simplifier.cc:675-694) leaves for an ONNX
+ * QLinearMatMul node, as one kernel.  Per-tensor scales and zero points.
+ * `bias` (int32 [N], added to the accumulator) and CHX_HIP_FUSE_RELU are
+ * extensions used by the MLP configuration; pass NULL / 0 for the reference op. */
+int chx_hip_qlinear_matmul(
+        const chx_hip_tensor* a, float a_scale, int32_t a_zero_point, const chx_hip_tensor* b, float b_scale,
+        int32_t b_zero_point, float y_scale, int32_t y_zero_point, const chx_hip_tensor* bias, uint32_t flags,
+        chx_hip_tensor* y, void* stream);
+
+/* ---- fused element-wise chains ---------------------------------------------------------- */
+
+/* ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161.  `code` is the program
+ * text the hip fusion builder emits for a FusionGroup (the counterpart of the CUDA
+ * source from compiler/nvrtc_builder.cc:91-206): one SSA statement per node in
+ * topological order.  All inputs must have one dtype; the result shape is the
+ * broadcast of the input shapes; inputs are read through their strides (nothing is
+ * materialised).  The kernel is generated and compiled with hiprtc on first use
+ * and cached by program text and operand layout, like the reference's two-level
+ * cache (runtime/ops/nvrtc.cc:41-84). */
+int chx_hip_elementwise(
+        const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
+        chx_hip_tensor* const* outputs, int32_t n_outputs, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CHX_HIP_H_ */
