@@ -28,7 +28,7 @@ EXPORTS = [
     "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
-    "chx_hip_qlinear_matmul", "chx_hip_elementwise",
+    "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source",
 ]
 
 
@@ -111,3 +111,33 @@ def device_props():
 
 def conv_params(strides, pads_begin, pads_end, group):
     return ConvParams(strides[0], strides[1], pads_begin[0], pads_begin[1], pads_end[0], pads_end[1], group)
+
+
+def tensor_array(descs):
+    """Array of pointers to chx_hip_tensor (keeps the descriptors alive on the result)."""
+    arr = (ctypes.POINTER(Tensor) * len(descs))(*[ctypes.pointer(d) for d in descs])
+    arr._keep = descs
+    return arr
+
+
+def make_desc(data_ptr, dtype, shape, strides_bytes):
+    d = Tensor()
+    d.data = data_ptr
+    d.dtype = dtype
+    d.ndim = len(shape)
+    for i, (n, st) in enumerate(zip(shape, strides_bytes)):
+        d.shape[i] = n
+        d.strides[i] = st
+    return d
+
+
+def elementwise_source(code, fusion_id, in_descs, out_descs, compile=False):
+    """Generated HIP source for a fusion program and operand layouts (no GPU needed)."""
+    ins, outs = tensor_array(in_descs), tensor_array(out_descs)
+    needed = ctypes.c_size_t(0)
+    args = (code.encode(), ctypes.c_int32(fusion_id), ins, ctypes.c_int32(len(in_descs)), outs,
+            ctypes.c_int32(len(out_descs)), ctypes.c_int32(1 if compile else 0))
+    check(lib().chx_hip_elementwise_source(*args, None, ctypes.c_size_t(0), ctypes.byref(needed)))
+    buf = ctypes.create_string_buffer(needed.value)
+    check(lib().chx_hip_elementwise_source(*args, buf, ctypes.c_size_t(needed.value), None))
+    return buf.value.decode()

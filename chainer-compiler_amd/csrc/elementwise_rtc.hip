@@ -1,0 +1,769 @@
+// Fused element-wise chains (the FusionGroup kernels).
+//
+// The reference lowers a FusionGroup on the GPU by generating CUDA source at compile
+// time (compiler/nvrtc_builder.cc:91-206), compiling it with NVRTC on first use and
+// launching one thread per element over inputs that were first broadcast and copied
+// (runtime/ops/nvrtc.cc:90-161).  Here the FusionGroup travels as a small SSA program
+// text; the HIP source is generated at run time, when the operand layouts are known,
+// so that
+//   - broadcast operands are read through their strides (a [1024] vector against a
+//     [64,1024,1024] tensor costs 4 KiB of traffic, not 256 MiB),
+//   - every full-size operand moves in 128-bit accesses,
+//   - the arithmetic is the CPU path's: one IEEE operation per node in topological
+//     order, no contraction, tanh/exp as the host C library computes them
+//     (faithful_math.h), sigmoid as 1/(1+exp(-x)).
+// Compiled code objects are cached by generated source text; loaded kernels by the
+// same key (the reference's two-level cache, runtime/ops/nvrtc.cc:41-84, here under a
+// mutex).
+//
+// Program text (one statement per line, '#' starts a comment):
+//   chxhip-fusion 1
+//   in  <name>:<dtype> ...            dtype: float32 | uint8 | int8
+//   <name> = <Op> <operand> ...       operands are earlier names or, where noted, literals
+//   out <name>:<dtype> ...
+// Ops: Identity a | Neg a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
+//      Tanh a | Sigmoid a | Exp a | Relu a | Clip a <lo> <hi> | Const <value>
+//      QuantizeLinear a <scale> <zero_point> <uint8|int8> [rne]   (float -> 8-bit code)
+//      DequantizeLinear q <scale> <zero_point>                    (8-bit code -> float)
+// Float literals are decimal or 0x######## (the bit pattern of the float32).
+#include <hip/hiprtc.h>
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "chx_internal.h"
+
+namespace chx {
+namespace {
+
+const char* kFaithfulMathText =
+#include "faithful_math_text.inc"
+        ;
+
+struct Stmt {
+    std::string out, op;
+    std::vector<std::string> args;
+};
+
+struct Port {
+    std::string name;
+    int32_t dtype;
+};
+
+struct Program {
+    std::vector<Port> inputs, outputs;
+    std::vector<Stmt> stmts;
+};
+
+bool parse_dtype(const std::string& s, int32_t* dt) {
+    if (s == "float32") *dt = CHX_HIP_FLOAT32;
+    else if (s == "uint8") *dt = CHX_HIP_UINT8;
+    else if (s == "int8") *dt = CHX_HIP_INT8;
+    else return false;
+    return true;
+}
+
+std::vector<std::string> split_ws(const std::string& line) {
+    std::vector<std::string> out;
+    std::istringstream iss(line);
+    std::string tok;
+    while (iss >> tok) out.push_back(tok);
+    return out;
+}
+
+int parse_port(const std::string& tok, Port* p) {
+    const size_t c = tok.find(':');
+    CHX_REQUIRE(c != std::string::npos, "fusion program: expected name:dtype, got '%s'", tok.c_str());
+    p->name = tok.substr(0, c);
+    CHX_REQUIRE(parse_dtype(tok.substr(c + 1), &p->dtype), "fusion program: unsupported dtype in '%s'", tok.c_str());
+    return CHX_HIP_OK;
+}
+
+int parse_program(const char* code, Program* prog) {
+    CHX_REQUIRE(code != nullptr, "fusion program: null code");
+    std::istringstream iss(code);
+    std::string line;
+    bool header = false;
+    while (std::getline(iss, line)) {
+        const size_t hash = line.find('#');
+        if (hash != std::string::npos) line.resize(hash);
+        std::vector<std::string> t = split_ws(line);
+        if (t.empty()) continue;
+        if (!header) {
+            CHX_REQUIRE(t.size() == 2 && t[0] == "chxhip-fusion" && t[1] == "1",
+                        "fusion program: missing 'chxhip-fusion 1' header (is this NVRTC source?)");
+            header = true;
+            continue;
+        }
+        if (t[0] == "in" || t[0] == "out") {
+            for (size_t i = 1; i < t.size(); ++i) {
+                Port p;
+                CHX_PROPAGATE(parse_port(t[i], &p));
+                (t[0] == "in" ? prog->inputs : prog->outputs).push_back(p);
+            }
+            continue;
+        }
+        CHX_REQUIRE(t.size() >= 3 && t[1] == "=", "fusion program: cannot parse statement '%s'", line.c_str());
+        Stmt s;
+        s.out = t[0];
+        s.op = t[2];
+        s.args.assign(t.begin() + 3, t.end());
+        prog->stmts.push_back(s);
+    }
+    CHX_REQUIRE(header, "fusion program: empty");
+    CHX_REQUIRE(!prog->inputs.empty(), "fusion program: no inputs");
+    CHX_REQUIRE(!prog->outputs.empty(), "fusion program: no outputs");
+    return CHX_HIP_OK;
+}
+
+std::string ident(const std::string& s) {
+    std::string o = "v_";
+    for (char c : s) o += (isalnum((unsigned char)c) ? c : '_');
+    return o;
+}
+
+int float_literal(const std::string& tok, std::string* out) {
+    float f;
+    if (tok.size() == 10 && tok[0] == '0' && (tok[1] == 'x' || tok[1] == 'X')) {
+        char* end = nullptr;
+        const unsigned long u = strtoul(tok.c_str(), &end, 16);
+        CHX_REQUIRE(end && *end == 0, "fusion program: bad float bit pattern '%s'", tok.c_str());
+        const uint32_t u32 = (uint32_t)u;
+        memcpy(&f, &u32, 4);
+    } else {
+        char* end = nullptr;
+        const double d = strtod(tok.c_str(), &end);
+        CHX_REQUIRE(end && *end == 0 && end != tok.c_str(), "fusion program: bad float literal '%s'", tok.c_str());
+        f = (float)d;
+    }
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    char buf[64];
+    snprintf(buf, sizeof(buf), "__builtin_bit_cast(float, 0x%08xu)", bits);
+    *out = buf;
+    return CHX_HIP_OK;
+}
+
+// Emits the per-element device function:  elem(in..., &out...).
+// Value kinds: 'f' float32 value, 'q' 8-bit code held in an int.
+int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* uses_exp_table) {
+    std::map<std::string, char> kind;
+    os << "__device__ __forceinline__ void elem(";
+    bool first = true;
+    for (const Port& p : prog.inputs) {
+        CHX_REQUIRE(!kind.count(p.name), "fusion program: duplicate input '%s'", p.name.c_str());
+        kind[p.name] = p.dtype == CHX_HIP_FLOAT32 ? 'f' : 'q';
+        os << (first ? "" : ", ") << (p.dtype == CHX_HIP_FLOAT32 ? "const float " : "const int ") << ident(p.name);
+        first = false;
+    }
+    for (size_t i = 0; i < prog.outputs.size(); ++i)
+        os << ", " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float& " : "int& ") << "o_" << i;
+    os << ") {\n";
+    const char* fma = use_fma ? "true" : "false";
+    for (const Stmt& s : prog.stmts) {
+        CHX_REQUIRE(!kind.count(s.out), "fusion program: '%s' assigned twice", s.out.c_str());
+        auto need = [&](size_t n) -> int {
+            CHX_REQUIRE(s.args.size() == n, "fusion program: %s takes %zu operands, got %zu", s.op.c_str(), n,
+                        s.args.size());
+            return CHX_HIP_OK;
+        };
+        auto val = [&](size_t i, char k, std::string* out) -> int {
+            auto it = kind.find(s.args[i]);
+            CHX_REQUIRE(it != kind.end(), "fusion program: '%s' used before definition in '%s'", s.args[i].c_str(),
+                        s.op.c_str());
+            CHX_REQUIRE(it->second == k, "fusion program: operand '%s' of %s has the wrong kind (%s expected)",
+                        s.args[i].c_str(), s.op.c_str(), k == 'f' ? "float" : "8-bit code");
+            *out = ident(s.args[i]);
+            return CHX_HIP_OK;
+        };
+        const std::string o = ident(s.out);
+        std::string a, b, l0, l1;
+        char out_kind = 'f';
+        static const std::map<std::string, const char*> binops = {{"Add", "+"}, {"Sub", "-"}, {"Mul", "*"}, {"Div", "/"}};
+        if (binops.count(s.op)) {
+            CHX_PROPAGATE(need(2));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            CHX_PROPAGATE(val(1, 'f', &b));
+            os << "  const float " << o << " = " << a << " " << binops.at(s.op) << " " << b << ";\n";
+        } else if (s.op == "Max" || s.op == "Min") {
+            CHX_PROPAGATE(need(2));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            CHX_PROPAGATE(val(1, 'f', &b));
+            if (s.op == "Max")
+                os << "  const float " << o << " = " << a << " < " << b << " ? " << b << " : " << a << ";\n";
+            else
+                os << "  const float " << o << " = " << b << " < " << a << " ? " << b << " : " << a << ";\n";
+        } else if (s.op == "Identity") {
+            CHX_PROPAGATE(need(1));
+            auto it = kind.find(s.args[0]);
+            CHX_REQUIRE(it != kind.end(), "fusion program: '%s' used before definition", s.args[0].c_str());
+            out_kind = it->second;
+            os << "  const " << (out_kind == 'f' ? "float " : "int ") << o << " = " << ident(s.args[0]) << ";\n";
+        } else if (s.op == "Neg") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = -" << a << ";\n";
+        } else if (s.op == "Tanh") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = chx_fm::tanhf_faithful(" << a << ");\n";
+        } else if (s.op == "Exp") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = chx_fm::expf_faithful<" << fma << ">(" << a << ");\n";
+            *uses_exp_table = true;
+        } else if (s.op == "Sigmoid") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = chx_fm::sigmoid_faithful<" << fma << ">(" << a << ");\n";
+            *uses_exp_table = true;
+        } else if (s.op == "Relu") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = " << a << " < 0.0f ? 0.0f : " << a << ";\n";
+        } else if (s.op == "Clip") {
+            CHX_PROPAGATE(need(3));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            CHX_PROPAGATE(float_literal(s.args[1], &l0));
+            CHX_PROPAGATE(float_literal(s.args[2], &l1));
+            os << "  const float " << o << "_lo = " << a << " < " << l0 << " ? " << l0 << " : " << a << ";\n";
+            os << "  const float " << o << " = " << o << "_lo < " << l1 << " ? " << o << "_lo : " << l1 << ";\n";
+        } else if (s.op == "Const") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(float_literal(s.args[0], &l0));
+            os << "  const float " << o << " = " << l0 << ";\n";
+        } else if (s.op == "QuantizeLinear") {
+            CHX_REQUIRE(s.args.size() == 4 || (s.args.size() == 5 && s.args[4] == "rne"),
+                        "fusion program: QuantizeLinear a scale zero_point dtype [rne]");
+            CHX_PROPAGATE(val(0, 'f', &a));
+            CHX_PROPAGATE(float_literal(s.args[1], &l0));
+            char* end = nullptr;
+            const long zp = strtol(s.args[2].c_str(), &end, 10);
+            CHX_REQUIRE(end && *end == 0, "fusion program: bad zero point '%s'", s.args[2].c_str());
+            int32_t dt;
+            CHX_REQUIRE(parse_dtype(s.args[3], &dt) && is_q8(dt), "fusion program: QuantizeLinear dtype must be uint8 or int8");
+            const bool i8 = dt == CHX_HIP_INT8;
+            CHX_REQUIRE(zp >= (i8 ? -128 : 0) && zp <= (i8 ? 127 : 255), "fusion program: zero point %ld out of range", zp);
+            const char* lo = i8 ? "-128.0f" : "0.0f";
+            const char* hi = i8 ? "127.0f" : "255.0f";
+            // quantize_array, runtime/ops/quantize.cc:29-34
+            os << "  float " << o << "_s = " << a << " / " << l0 << ";\n";
+            if (s.args.size() == 5) {
+                os << "  " << o << "_s = __builtin_rintf(" << o << "_s) + " << zp << ".0f;\n";
+                os << "  " << o << "_s = " << o << "_s < " << hi << " ? " << o << "_s : " << hi << ";\n";
+                os << "  " << o << "_s = " << lo << " < " << o << "_s ? " << o << "_s : " << lo << ";\n";
+            } else {
+                os << "  " << o << "_s = " << o << "_s + " << zp << ".0f;\n";
+                os << "  " << o << "_s = " << o << "_s < " << hi << " ? " << o << "_s : " << hi << ";\n";
+                os << "  " << o << "_s = " << lo << " < " << o << "_s ? " << o << "_s : " << lo << ";\n";
+                os << "  " << o << "_s = " << o << "_s + 0.5f;\n";
+            }
+            os << "  const int " << o << " = (int)" << o << "_s;\n";
+            out_kind = 'q';
+        } else if (s.op == "DequantizeLinear") {
+            CHX_PROPAGATE(need(3));
+            CHX_PROPAGATE(val(0, 'q', &a));
+            CHX_PROPAGATE(float_literal(s.args[1], &l0));
+            char* end = nullptr;
+            const long zp = strtol(s.args[2].c_str(), &end, 10);
+            CHX_REQUIRE(end && *end == 0, "fusion program: bad zero point '%s'", s.args[2].c_str());
+            // dequantize_array, runtime/ops/quantize.cc:37-44
+            os << "  const float " << o << "_f = (float)" << a << " - " << zp << ".0f;\n";
+            os << "  const float " << o << " = " << o << "_f * " << l0 << ";\n";
+        } else {
+            CHX_FAIL(CHX_HIP_EUNSUPPORTED, "fusion program: op '%s' is not in the fusable set", s.op.c_str());
+        }
+        kind[s.out] = out_kind;
+    }
+    for (size_t i = 0; i < prog.outputs.size(); ++i) {
+        auto it = kind.find(prog.outputs[i].name);
+        CHX_REQUIRE(it != kind.end(), "fusion program: output '%s' is never defined", prog.outputs[i].name.c_str());
+        const char want = prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? 'f' : 'q';
+        CHX_REQUIRE(it->second == want, "fusion program: output '%s' is declared %s but computed as %s",
+                    prog.outputs[i].name.c_str(), dtype_name(prog.outputs[i].dtype), it->second == 'f' ? "float" : "code");
+        os << "  o_" << i << " = " << ident(prog.outputs[i].name) << ";\n";
+    }
+    os << "}\n";
+    return CHX_HIP_OK;
+}
+
+enum Mode : char { kFull = 'F', kScalar = 'S', kPeriodic = 'P' };
+
+const char* ctype_of(int32_t dt) {
+    return dt == CHX_HIP_FLOAT32 ? "float" : (dt == CHX_HIP_INT8 ? "signed char" : "unsigned char");
+}
+
+// Source of both kernels for one (program, operand modes) combination.
+//   <name>_vec : V elements per thread through 128-bit accesses; operands are full
+//                (same flat index as the output), scalar, or periodic (index modulo a
+//                period that is a multiple of V).
+//   <name>_gen : one element per thread, operands addressed through per-axis strides.
+int generate_source(
+        const Program& prog, const std::string& name, const std::string& modes, const std::vector<uint32_t>& periods,
+        int vec, bool use_fma, std::string* out) {
+    std::ostringstream os;
+    os << "#pragma clang fp contract(off)\n";
+    os << "#define FM_FN __device__ __forceinline__\n";
+    os << "#define FM_TABLE_QUALIFIER static __device__ const\n";
+    std::ostringstream body;
+    bool uses_table = false;
+    CHX_PROPAGATE(emit_elem(prog, use_fma, body, &uses_table));
+    os << kFaithfulMathText << "\n";
+    os << "typedef float v4f __attribute__((ext_vector_type(4)));\n";
+    os << "typedef unsigned int v4u __attribute__((ext_vector_type(4)));\n";
+    os << "namespace {\n" << body.str() << "}\n";
+    const size_t nin = prog.inputs.size(), nout = prog.outputs.size();
+
+    // ---- vector kernel ----
+    os << "extern \"C\" __global__ __launch_bounds__(256) void " << name << "_vec(unsigned int n_vec";
+    for (size_t i = 0; i < nin; ++i) os << ", const " << ctype_of(prog.inputs[i].dtype) << "* __restrict__ i" << i;
+    for (size_t i = 0; i < nout; ++i) os << ", " << ctype_of(prog.outputs[i].dtype) << "* __restrict__ o" << i;
+    os << ") {\n";
+    os << "  const unsigned int gid = blockIdx.x * 256u + threadIdx.x;\n";
+    os << "  if (gid >= n_vec) return;\n";
+    os << "  const unsigned int base = gid * " << vec << "u;  // fewer than 2^31 elements\n";
+    for (size_t i = 0; i < nin; ++i) {
+        const bool f32 = prog.inputs[i].dtype == CHX_HIP_FLOAT32;
+        const bool sgn = prog.inputs[i].dtype == CHX_HIP_INT8;
+        os << "  " << (f32 ? "float" : "int") << " x" << i << "[" << vec << "];\n";
+        if (modes[i] == kScalar) {
+            os << "  for (int e = 0; e < " << vec << "; ++e) x" << i << "[e] = i" << i << "[0];\n";
+            continue;
+        }
+        std::string idx = "base";
+        if (modes[i] == kPeriodic) idx = "(base % " + std::to_string(periods[i]) + "u)";
+        const bool nt = modes[i] == kFull;
+        if (f32) {
+            os << "  { const v4f* src = (const v4f*)(i" << i << " + " << idx << ");\n";
+            for (int j = 0; j < vec / 4; ++j) {
+                os << "    const v4f t" << j << " = " << (nt ? "__builtin_nontemporal_load(src + " : "*(src + ") << j << ");\n";
+                for (int k = 0; k < 4; ++k) os << "    x" << i << "[" << (j * 4 + k) << "] = t" << j << "[" << k << "];\n";
+            }
+            os << "  }\n";
+        } else {
+            // vec == 16: one 128-bit load of 16 codes
+            os << "  { const v4u t = " << (nt ? "__builtin_nontemporal_load((const v4u*)(i" : "*((const v4u*)(i") << i
+               << " + " << idx << "));\n";
+            for (int e = 0; e < vec; ++e) {
+                os << "    x" << i << "[" << e << "] = ";
+                if (sgn)
+                    os << "(int)(signed char)((t[" << (e / 4) << "] >> " << (8 * (e % 4)) << ") & 0xffu);\n";
+                else
+                    os << "(int)((t[" << (e / 4) << "] >> " << (8 * (e % 4)) << ") & 0xffu);\n";
+            }
+            os << "  }\n";
+        }
+    }
+    for (size_t i = 0; i < nout; ++i)
+        os << "  " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float" : "int") << " y" << i << "[" << vec << "];\n";
+    os << "#pragma unroll\n  for (int e = 0; e < " << vec << "; ++e) elem(";
+    for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "x" << i << "[e]";
+    for (size_t i = 0; i < nout; ++i) os << ", y" << i << "[e]";
+    os << ");\n";
+    for (size_t i = 0; i < nout; ++i) {
+        if (prog.outputs[i].dtype == CHX_HIP_FLOAT32) {
+            os << "  { v4f* dst = (v4f*)(o" << i << " + base);\n";
+            for (int j = 0; j < vec / 4; ++j) {
+                os << "    v4f t" << j << ";\n";
+                for (int k = 0; k < 4; ++k) os << "    t" << j << "[" << k << "] = y" << i << "[" << (j * 4 + k) << "];\n";
+                os << "    __builtin_nontemporal_store(t" << j << ", dst + " << j << ");\n";
+            }
+            os << "  }\n";
+        } else {
+            os << "  { v4u t;\n";
+            for (int w = 0; w < 4; ++w) {
+                os << "    t[" << w << "] = ";
+                for (int k = 0; k < 4; ++k)
+                    os << (k ? " | " : "") << "(((unsigned int)y" << i << "[" << (w * 4 + k) << "] & 0xffu) << " << (8 * k) << ")";
+                os << ";\n";
+            }
+            os << "    __builtin_nontemporal_store(t, (v4u*)(o" << i << " + base));\n  }\n";
+        }
+    }
+    os << "}\n";
+
+    // ---- general kernel ----
+    os << "struct GenDesc { int ndim; int pad; long long shape[" << CHX_HIP_MAX_NDIM << "]; long long istr[" << nin << "]["
+       << CHX_HIP_MAX_NDIM << "]; };\n";
+    os << "extern \"C\" __global__ __launch_bounds__(256) void " << name
+       << "_gen(unsigned long long begin, unsigned long long n";
+    for (size_t i = 0; i < nin; ++i) os << ", const " << ctype_of(prog.inputs[i].dtype) << "* __restrict__ i" << i;
+    for (size_t i = 0; i < nout; ++i) os << ", " << ctype_of(prog.outputs[i].dtype) << "* __restrict__ o" << i;
+    os << ", GenDesc d) {\n";
+    os << "  const unsigned long long idx = begin + (unsigned long long)blockIdx.x * 256ull + threadIdx.x;\n";
+    os << "  if (idx >= n) return;\n";
+    os << "  long long off[" << nin << "];\n";
+    os << "  for (int i = 0; i < " << nin << "; ++i) off[i] = 0;\n";
+    os << "  unsigned long long rest = idx;\n";
+    os << "  for (int a = d.ndim - 1; a >= 0; --a) {\n";
+    os << "    const unsigned long long q = rest / (unsigned long long)d.shape[a];\n";
+    os << "    const long long r = (long long)(rest - q * (unsigned long long)d.shape[a]);\n";
+    os << "    for (int i = 0; i < " << nin << "; ++i) off[i] += r * d.istr[i][a];\n";
+    os << "    rest = q;\n  }\n";
+    for (size_t i = 0; i < nout; ++i)
+        os << "  " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float" : "int") << " r" << i << ";\n";
+    os << "  elem(";
+    for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "i" << i << "[off[" << i << "]]";
+    for (size_t i = 0; i < nout; ++i) os << ", r" << i;
+    os << ");\n";
+    for (size_t i = 0; i < nout; ++i) {
+        if (prog.outputs[i].dtype == CHX_HIP_FLOAT32)
+            os << "  o" << i << "[idx] = r" << i << ";\n";
+        else
+            os << "  o" << i << "[idx] = (" << ctype_of(prog.outputs[i].dtype) << ")r" << i << ";\n";
+    }
+    os << "}\n";
+    *out = os.str();
+    return CHX_HIP_OK;
+}
+
+struct CompiledKernels {
+    std::vector<char> code;
+    hipModule_t module = nullptr;  // loaded lazily, per process (one GPU)
+    hipFunction_t vec = nullptr, gen = nullptr;
+};
+
+std::mutex g_cache_mutex;
+std::map<std::string, std::shared_ptr<CompiledKernels>> g_cache;  // key: generated source
+
+int compile_source(const std::string& src, const std::string& name, std::vector<char>* code) {
+    hiprtcProgram p;
+    if (hiprtcCreateProgram(&p, src.c_str(), (name + ".hip").c_str(), 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+        CHX_FAIL(CHX_HIP_ERUNTIME, "hiprtcCreateProgram failed for %s", name.c_str());
+    const char* opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-Xclang", "-target-feature",
+                          "-Xclang", "-packed-fp32-ops"};
+    const hiprtcResult r = hiprtcCompileProgram(p, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t ls = 0;
+        hiprtcGetProgramLogSize(p, &ls);
+        std::string log(ls, '\0');
+        if (ls) hiprtcGetProgramLog(p, &log[0]);
+        hiprtcDestroyProgram(&p);
+        CHX_FAIL(CHX_HIP_ECOMPILE, "hiprtc could not compile %s: %s\n%s", name.c_str(), hiprtcGetErrorString(r),
+                 log.c_str());
+    }
+    size_t cs = 0;
+    hiprtcGetCodeSize(p, &cs);
+    code->resize(cs);
+    hiprtcGetCode(p, code->data());
+    hiprtcDestroyProgram(&p);
+    return CHX_HIP_OK;
+}
+
+// Which operation grouping of expf the host C library uses (see faithful_math.h):
+// the two groupings differ on exactly two inputs, so evaluating one of them tells.
+bool host_libm_uses_fma() {
+    static const bool v = [] {
+        volatile float x = 0.0f;
+        const uint32_t bits = 0x4202422fu;
+        float xf;
+        memcpy(&xf, &bits, 4);
+        x = xf;
+        const float e = expf(x);
+        uint32_t eb;
+        memcpy(&eb, &e, 4);
+        return eb == 0x56fc9f1cu;  // 0x1.f93e38p+46: the fused-reduction result
+    }();
+    return v;
+}
+
+struct Plan {
+    std::string modes;             // per input
+    bool vector_ok = false;
+    int vec = 4;
+    int64_t n = 0;
+    int ndim = 0;
+    int64_t shape[CHX_HIP_MAX_NDIM];
+    std::vector<std::vector<int64_t>> istr;  // element strides per input, per collapsed axis
+    std::vector<uint32_t> periods;
+};
+
+int make_plan(
+        const Program& prog, const chx_hip_tensor* const* inputs, int32_t n_inputs, chx_hip_tensor* const* outputs,
+        int32_t n_outputs, Plan* plan) {
+    CHX_REQUIRE((size_t)n_inputs == prog.inputs.size(), "fusion: program declares %zu inputs, %d given",
+                prog.inputs.size(), n_inputs);
+    CHX_REQUIRE((size_t)n_outputs == prog.outputs.size(), "fusion: program declares %zu outputs, %d given",
+                prog.outputs.size(), n_outputs);
+    int nd = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        CHX_PROPAGATE(check_tensor(inputs[i], "fusion input"));
+        CHX_REQUIRE(inputs[i]->dtype == prog.inputs[i].dtype, "fusion: input %d is %s, program says %s", i,
+                    dtype_name(inputs[i]->dtype), dtype_name(prog.inputs[i].dtype));
+        nd = inputs[i]->ndim > nd ? inputs[i]->ndim : nd;
+    }
+    // BroadcastShapes over all inputs, runtime/ops/nvrtc.cc:100-104
+    int64_t shape[CHX_HIP_MAX_NDIM];
+    for (int a = 0; a < nd; ++a) shape[a] = 1;
+    for (int i = 0; i < n_inputs; ++i) {
+        const chx_hip_tensor& t = *inputs[i];
+        for (int a = 0; a < t.ndim; ++a) {
+            const int oa = nd - t.ndim + a;
+            if (t.shape[a] == 1) continue;
+            CHX_REQUIRE(shape[oa] == 1 || shape[oa] == t.shape[a], "fusion: input %d does not broadcast (axis %d: %lld vs %lld)",
+                        i, a, (long long)t.shape[a], (long long)shape[oa]);
+            shape[oa] = t.shape[a];
+        }
+    }
+    int64_t n = 1;
+    for (int a = 0; a < nd; ++a) n *= shape[a];
+    plan->n = n;
+    for (int i = 0; i < n_outputs; ++i) {
+        CHX_PROPAGATE(check_tensor(outputs[i], "fusion output"));
+        const chx_hip_tensor& t = *outputs[i];
+        CHX_REQUIRE(t.dtype == prog.outputs[i].dtype, "fusion: output %d is %s, program says %s", i, dtype_name(t.dtype),
+                    dtype_name(prog.outputs[i].dtype));
+        CHX_REQUIRE(t.ndim == nd, "fusion: output %d has ndim %d, the broadcast result has %d", i, t.ndim, nd);
+        for (int a = 0; a < nd; ++a)
+            CHX_REQUIRE(t.shape[a] == shape[a], "fusion: output %d has extent %lld on axis %d, expected %lld", i,
+                        (long long)t.shape[a], a, (long long)shape[a]);
+    }
+    // Iteration order: axes of output 0 by decreasing stride; every output must be dense in
+    // that order with the same element strides.
+    int order[CHX_HIP_MAX_NDIM];
+    int na = 0;
+    const chx_hip_tensor& o0 = *outputs[0];
+    const int64_t es0 = dtype_size(o0.dtype);
+    for (int a = 0; a < nd; ++a)
+        if (shape[a] != 1) order[na++] = a;
+    for (int i = 0; i < na; ++i)
+        for (int j = i + 1; j < na; ++j)
+            if (o0.strides[order[j]] > o0.strides[order[i]]) {
+                const int t = order[i];
+                order[i] = order[j];
+                order[j] = t;
+            }
+    {
+        int64_t expect = 1;
+        for (int i = na - 1; i >= 0; --i) {
+            for (int k = 0; k < n_outputs; ++k) {
+                const int64_t es = dtype_size(outputs[k]->dtype);
+                CHX_REQUIRE(outputs[k]->strides[order[i]] == expect * es,
+                            "fusion: output %d is not dense, or outputs differ in layout", k);
+            }
+            expect *= shape[order[i]];
+        }
+        (void)es0;
+    }
+    // Element strides of every input along the ordered axes (0 where it broadcasts).
+    std::vector<std::vector<int64_t>> istr(n_inputs, std::vector<int64_t>(na, 0));
+    for (int i = 0; i < n_inputs; ++i) {
+        const chx_hip_tensor& t = *inputs[i];
+        const int64_t es = dtype_size(t.dtype);
+        for (int k = 0; k < na; ++k) {
+            const int ia = order[k] - (nd - t.ndim);
+            if (ia < 0 || t.shape[ia] == 1) continue;
+            CHX_REQUIRE(t.strides[ia] % es == 0, "fusion: input %d has a stride that is not a multiple of its element size", i);
+            istr[i][k] = t.strides[ia] / es;
+        }
+    }
+    // Collapse neighbouring axes that every operand walks contiguously.
+    std::vector<int64_t> cshape;
+    std::vector<std::vector<int64_t>> cstr(n_inputs);
+    for (int k = 0; k < na; ++k) {
+        const int64_t ext = shape[order[k]];
+        bool merge = !cshape.empty();
+        if (merge)
+            for (int i = 0; i < n_inputs; ++i)
+                if (cstr[i].back() != istr[i][k] * ext) merge = false;
+        if (merge) {
+            cshape.back() *= ext;
+            for (int i = 0; i < n_inputs; ++i) cstr[i].back() = istr[i][k];
+        } else {
+            cshape.push_back(ext);
+            for (int i = 0; i < n_inputs; ++i) cstr[i].push_back(istr[i][k]);
+        }
+    }
+    plan->ndim = (int)cshape.size();
+    for (int a = 0; a < plan->ndim; ++a) plan->shape[a] = cshape[a];
+    plan->istr = cstr;
+
+    bool any8 = false;
+    for (const Port& p : prog.inputs) any8 = any8 || p.dtype != CHX_HIP_FLOAT32;
+    for (const Port& p : prog.outputs) any8 = any8 || p.dtype != CHX_HIP_FLOAT32;
+    plan->vec = any8 ? 16 : 4;
+    plan->modes.assign(n_inputs, kFull);
+    plan->periods.assign(n_inputs, 0);
+    bool ok = n < (int64_t(1) << 31);  // CHECK_GT(1 << 31, size), runtime/ops/nvrtc.cc:127
+    // dense inner strides of the output in collapsed axes
+    std::vector<int64_t> dense(plan->ndim, 1);
+    for (int a = plan->ndim - 2; a >= 0; --a) dense[a] = dense[a + 1] * cshape[a + 1];
+    for (int i = 0; i < n_inputs; ++i) {
+        bool all_zero = true, full = true;
+        for (int a = 0; a < plan->ndim; ++a) {
+            if (cstr[i][a] != 0) all_zero = false;
+            if (cstr[i][a] != dense[a]) full = false;
+        }
+        const int64_t es = dtype_size(inputs[i]->dtype);
+        if (plan->ndim == 0 || all_zero) {
+            plan->modes[i] = kScalar;
+        } else if (full) {
+            plan->modes[i] = kFull;
+            if (!aligned(inputs[i]->data, 16)) ok = false;
+        } else {
+            // periodic: zero strides on the outer axes, dense strides on the inner ones
+            int a = 0;
+            while (a < plan->ndim && cstr[i][a] == 0) ++a;
+            bool inner_dense = a > 0;
+            for (int b = a; b < plan->ndim; ++b)
+                if (cstr[i][b] != dense[b]) inner_dense = false;
+            const int64_t period = a > 0 ? dense[a - 1] : 0;
+            if (inner_dense && period % plan->vec == 0 && period < (int64_t(1) << 31) && aligned(inputs[i]->data, 16)) {
+                plan->modes[i] = kPeriodic;
+                plan->periods[i] = (uint32_t)period;
+            } else {
+                ok = false;
+            }
+        }
+        (void)es;
+    }
+    for (int k = 0; k < n_outputs; ++k)
+        if (!aligned(outputs[k]->data, 16)) ok = false;
+    plan->vector_ok = ok && n >= plan->vec;
+    if (!plan->vector_ok) {
+        // the general kernel ignores modes; use one canonical key
+        plan->modes.assign(n_inputs, kFull);
+        plan->periods.assign(n_inputs, 0);
+    }
+    return CHX_HIP_OK;
+}
+
+struct ArgPacker {
+    std::vector<char> buf;
+    template <typename T>
+    void push(const T& v) {
+        const size_t a = alignof(T);
+        const size_t off = (buf.size() + a - 1) / a * a;
+        buf.resize(off + sizeof(T));
+        memcpy(buf.data() + off, &v, sizeof(T));
+    }
+    void push_bytes(const void* p, size_t n, size_t a) {
+        const size_t off = (buf.size() + a - 1) / a * a;
+        buf.resize(off + n);
+        memcpy(buf.data() + off, p, n);
+    }
+};
+
+int prepare(
+        const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
+        chx_hip_tensor* const* outputs, int32_t n_outputs, Program* prog, Plan* plan, std::string* name,
+        std::string* src) {
+    CHX_REQUIRE(inputs != nullptr && n_inputs > 0, "fusion: no inputs");  // CHECK(!inputs.empty()), nvrtc.cc:93
+    CHX_REQUIRE(outputs != nullptr && n_outputs > 0, "fusion: no outputs");
+    CHX_PROPAGATE(parse_program(code, prog));
+    CHX_PROPAGATE(make_plan(*prog, inputs, n_inputs, outputs, n_outputs, plan));
+    *name = "fusion" + std::to_string(fusion_id < 0 ? 0 : fusion_id);
+    CHX_PROPAGATE(generate_source(*prog, *name, plan->modes, plan->periods, plan->vec, host_libm_uses_fma(), src));
+    return CHX_HIP_OK;
+}
+
+int get_compiled(const std::string& src, const std::string& name, std::shared_ptr<CompiledKernels>* out) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_cache.find(src);
+    if (it != g_cache.end()) {
+        *out = it->second;
+        return CHX_HIP_OK;
+    }
+    auto ck = std::make_shared<CompiledKernels>();
+    CHX_PROPAGATE(compile_source(src, name, &ck->code));
+    g_cache.emplace(src, ck);
+    *out = ck;
+    return CHX_HIP_OK;
+}
+
+int load_kernels(CompiledKernels* ck, const std::string& name) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    if (ck->module) return CHX_HIP_OK;
+    hipModule_t m;
+    CHX_HIP_CALL(hipModuleLoadData(&m, ck->code.data()));
+    CHX_HIP_CALL(hipModuleGetFunction(&ck->vec, m, (name + "_vec").c_str()));
+    CHX_HIP_CALL(hipModuleGetFunction(&ck->gen, m, (name + "_gen").c_str()));
+    ck->module = m;
+    return CHX_HIP_OK;
+}
+
+int launch(hipFunction_t f, unsigned grid, ArgPacker& args, hipStream_t s) {
+    size_t size = args.buf.size();
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.buf.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                     HIP_LAUNCH_PARAM_END};
+    CHX_HIP_CALL(hipModuleLaunchKernel(f, grid, 1, 1, 256, 1, 1, 0, s, nullptr, extra));
+    return CHX_HIP_OK;
+}
+
+}  // namespace
+}  // namespace chx
+
+using namespace chx;
+
+extern "C" int chx_hip_elementwise_source(
+        const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
+        chx_hip_tensor* const* outputs, int32_t n_outputs, int32_t compile, char* buffer, size_t buffer_size,
+        size_t* needed) {
+    Program prog;
+    Plan plan;
+    std::string name, src;
+    CHX_PROPAGATE(prepare(code, fusion_id, inputs, n_inputs, outputs, n_outputs, &prog, &plan, &name, &src));
+    if (compile) {
+        std::shared_ptr<CompiledKernels> ck;
+        CHX_PROPAGATE(get_compiled(src, name, &ck));
+    }
+    std::string text = std::string("// modes=") + plan.modes + (plan.vector_ok ? " vector" : " general") + "\n" + src;
+    if (needed) *needed = text.size() + 1;
+    if (buffer && buffer_size) {
+        const size_t n = text.size() < buffer_size - 1 ? text.size() : buffer_size - 1;
+        memcpy(buffer, text.data(), n);
+        buffer[n] = 0;
+    }
+    return CHX_HIP_OK;
+}
+
+extern "C" int chx_hip_elementwise(
+        const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
+        chx_hip_tensor* const* outputs, int32_t n_outputs, void* stream) {
+    Program prog;
+    Plan plan;
+    std::string name, src;
+    CHX_PROPAGATE(prepare(code, fusion_id, inputs, n_inputs, outputs, n_outputs, &prog, &plan, &name, &src));
+    if (plan.n == 0) return CHX_HIP_OK;
+    std::shared_ptr<CompiledKernels> ck;
+    CHX_PROPAGATE(get_compiled(src, name, &ck));
+    CHX_PROPAGATE(load_kernels(ck.get(), name));
+    hipStream_t s = as_stream(stream);
+
+    int64_t done = 0;
+    if (plan.vector_ok) {
+        const int64_t n_vec = plan.n / plan.vec;
+        ArgPacker a;
+        a.push((uint32_t)n_vec);
+        for (int i = 0; i < n_inputs; ++i) a.push(inputs[i]->data);
+        for (int i = 0; i < n_outputs; ++i) a.push(outputs[i]->data);
+        CHX_PROPAGATE(launch(ck->vec, (unsigned)((n_vec + 255) / 256), a, s));
+        done = n_vec * plan.vec;
+    }
+    if (done < plan.n) {
+        CHX_REQUIRE(plan.n - done < (int64_t(1) << 39), "fusion: %lld elements is beyond what the general kernel covers",
+                    (long long)(plan.n - done));
+        ArgPacker a;
+        a.push((unsigned long long)done);
+        a.push((unsigned long long)plan.n);
+        for (int i = 0; i < n_inputs; ++i) a.push(inputs[i]->data);
+        for (int i = 0; i < n_outputs; ++i) a.push(outputs[i]->data);
+        // GenDesc { int ndim; int pad; long long shape[MAX]; long long istr[nin][MAX]; }
+        std::vector<long long> d(1 + CHX_HIP_MAX_NDIM + (size_t)n_inputs * CHX_HIP_MAX_NDIM, 0);
+        int32_t head[2] = {plan.ndim, 0};
+        memcpy(&d[0], head, 8);
+        for (int k = 0; k < plan.ndim; ++k) d[1 + k] = plan.shape[k];
+        for (int k = plan.ndim; k < CHX_HIP_MAX_NDIM; ++k) d[1 + k] = 1;
+        for (int i = 0; i < n_inputs; ++i)
+            for (int k = 0; k < plan.ndim; ++k) d[1 + CHX_HIP_MAX_NDIM + (size_t)i * CHX_HIP_MAX_NDIM + k] = plan.istr[i][k];
+        a.push_bytes(d.data(), d.size() * sizeof(long long), 8);
+        CHX_PROPAGATE(launch(ck->gen, (unsigned)((plan.n - done + 255) / 256), a, s));
+    }
+    return CHX_HIP_OK;
+}

@@ -1,0 +1,233 @@
+// fp32 exp and tanh that reproduce the host C library bit for bit.
+//
+// On the CPU a fused group runs as separate ChxVM ops, and ChainerX's native Tanh
+// and Exp kernels call std::tanh / std::exp on float, i.e. the C library's tanhf and
+// expf.  Inside a chain (tanh(..) * sigmoid(..) + x) a one-ulp difference in a
+// transcendental survives cancellation as a large relative error, so the device
+// code does not approximate these functions on its own terms: it carries out the
+// same sequence of IEEE operations as the C library the oracle runs on
+// (GNU libc 2.35, x86-64):
+//   expf   the table-driven double-precision algorithm of Szabolcs Nagy's
+//          optimized routines (glibc sysdeps/ieee754/flt-32/e_expf.c): N = 32 table
+//          entries of 2^(i/N), a cubic in double, one final rounding to float.
+//   tanhf  the fdlibm algorithm (Sun Microsystems; glibc
+//          sysdeps/ieee754/flt-32/s_tanhf.c) on top of fdlibm's expm1f
+//          (s_expm1f.c), all in fp32.
+// Every operation below is a single correctly rounded IEEE operation; the file
+// must be compiled with floating-point contraction off, except where an explicit
+// fma is written.  tests/test_faithful_math.py checks the host build of this very
+// header against the C library over all 2^32 inputs, and the device build against
+// the host build.
+//
+// The header has no includes so that it can be handed to the run-time compiler as
+// text; FM_FN supplies the function qualifiers.
+#pragma once
+
+#ifndef FM_FN
+#define FM_FN inline
+#endif
+
+namespace chx_fm {
+
+typedef unsigned int fm_u32;
+typedef unsigned long long fm_u64;
+typedef int fm_i32;
+
+FM_FN fm_u32 f2u(float f) {
+    return __builtin_bit_cast(fm_u32, f);
+}
+FM_FN float u2f(fm_u32 u) {
+    return __builtin_bit_cast(float, u);
+}
+FM_FN fm_u64 d2u(double d) {
+    return __builtin_bit_cast(fm_u64, d);
+}
+FM_FN double u2d(fm_u64 u) {
+    return __builtin_bit_cast(double, u);
+}
+
+// tab[i] = bits(2^(i/32)) - (i << 47)
+#ifdef FM_TABLE_QUALIFIER
+FM_TABLE_QUALIFIER
+#else
+static const
+#endif
+fm_u64 kExp2fTab[32] = {
+        0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+        0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+        0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+        0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+        0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+        0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+        0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+        0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
+};
+
+// expf.  kUseFma selects the operation grouping of the C library build that is
+// dispatched on x86-64 CPUs with FMA3: there the compiler contracted the reduction
+// r = InvLn2N*x - kd into one fused multiply-add (and the cubic's multiply-adds,
+// which changes no result).  Without it every multiply and add rounds on its own.
+// Over all 2^32 inputs the two groupings differ on exactly two, 0x4202422f and
+// 0xc27c65d9, which is how a host's variant can be told.
+template <bool kUseFma>
+FM_FN float expf_faithful(float x) {
+    const fm_u32 ux = f2u(x);
+    const fm_u32 abstop = (ux >> 20) & 0x7ff;
+    if (abstop >= 0x42b) {  // |x| >= 88 or NaN
+        if (ux == 0xff800000u) return 0.0f;
+        if (abstop >= 0x7f8) return x + x;
+        if (x > 0x1.62e42ep6f) return u2f(0x7f800000u);  // overflow
+        if (x < -0x1.9fe368p6f) return 0.0f;             // underflow
+    }
+    const double xd = (double)x;
+    const double InvLn2N = 0x1.71547652b82fep+0 * 32.0;
+    const double Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    double z = InvLn2N * xd;
+    double kd = z + Shift;
+    const fm_u64 ki = d2u(kd);
+    kd = kd - Shift;
+    const double r = kUseFma ? __builtin_fma(InvLn2N, xd, -kd) : z - kd;
+    fm_u64 t = kExp2fTab[ki & 31];
+    t += ki << 47;
+    const double s = u2d(t);
+    double y;
+    if (kUseFma) {
+        z = __builtin_fma(C0, r, C1);
+        const double r2 = r * r;
+        y = __builtin_fma(C2, r, 1.0);
+        y = __builtin_fma(z, r2, y);
+    } else {
+        z = C0 * r + C1;
+        const double r2 = r * r;
+        y = C2 * r + 1.0;
+        y = z * r2 + y;
+    }
+    y = y * s;
+    return (float)y;
+}
+
+// expm1f, fdlibm.
+FM_FN float expm1f_faithful(float x) {
+    const float one = 1.0f, huge = 1.0e+30f, tiny = 1.0e-30f;
+    const float o_threshold = u2f(0x42b17180u);
+    const float ln2_hi = u2f(0x3f317180u);
+    const float ln2_lo = u2f(0x3717f7d1u);
+    const float invln2 = u2f(0x3fb8aa3bu);
+    const float Q1 = u2f(0xbd088889u);
+    const float Q2 = u2f(0x3ad00d01u);
+    const float Q3 = u2f(0xb8a670cdu);
+    const float Q4 = u2f(0x36867e54u);
+    const float Q5 = u2f(0xb457edbbu);
+
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    fm_i32 k;
+    fm_u32 hx = f2u(x);
+    const fm_u32 xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+
+    if (hx >= 0x4195b844u) {      // |x| >= 27 ln2
+        if (hx >= 0x42b17218u) {  // |x| >= 88.721...
+            if (hx > 0x7f800000u) return x + x;
+            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) return tiny - one;
+    }
+
+    if (hx > 0x3eb17218u) {       // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {   // |x| < 1.5 ln2
+            if (xsb == 0) {
+                hi = x - ln2_hi;
+                lo = ln2_lo;
+                k = 1;
+            } else {
+                hi = x + ln2_hi;
+                lo = -ln2_lo;
+                k = -1;
+            }
+        } else {
+            k = (fm_i32)(invln2 * x + (xsb == 0 ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {  // |x| < 2^-25
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = u2f(f2u(y) + ((fm_u32)k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = u2f(0x3f800000u - (0x1000000u >> k));  // 1 - 2^-k
+        y = t - (e - x);
+        y = u2f(f2u(y) + ((fm_u32)k << 23));
+    } else {
+        t = u2f((fm_u32)(0x7f - k) << 23);  // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = u2f(f2u(y) + ((fm_u32)k << 23));
+    }
+    return y;
+}
+
+// tanhf, fdlibm.
+FM_FN float tanhf_faithful(float x) {
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    float t, z;
+    const fm_u32 jx = f2u(x);
+    const fm_u32 ix = jx & 0x7fffffffu;
+    if (ix >= 0x7f800000u) {
+        if ((jx >> 31) == 0) return one / x + one;
+        return one / x - one;
+    }
+    const float ax = u2f(ix);
+    if (ix < 0x41b00000u) {  // |x| < 22
+        if (ix == 0) return x;
+        if (ix < 0x24000000u) return x * (one + x);  // |x| < 2^-55
+        if (ix >= 0x3f800000u) {                      // |x| >= 1
+            t = expm1f_faithful(two * ax);
+            z = one - two / (t + two);
+        } else {
+            t = expm1f_faithful(-two * ax);
+            z = -t / (t + two);
+        }
+    } else {
+        z = one - tiny;
+    }
+    return (jx >> 31) == 0 ? z : -z;
+}
+
+// ChainerX's Sigmoid routine as the oracle restates it: Reciprocal(1 + Exp(-x)),
+// one rounding per operation.
+template <bool kUseFma>
+FM_FN float sigmoid_faithful(float x) {
+    const float e = expf_faithful<kUseFma>(-x);
+    const float d = 1.0f + e;
+    return 1.0f / d;
+}
+
+}  // namespace chx_fm

@@ -36,8 +36,4 @@ int chx_hip_qlinear_matmul(
         const chx_hip_tensor*, uint32_t, chx_hip_tensor*, void*) {
     CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_qlinear_matmul: not implemented");
 }
-int chx_hip_elementwise(
-        const char*, int32_t, const chx_hip_tensor* const*, int32_t, chx_hip_tensor* const*, int32_t, void*) {
-    CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_elementwise: not implemented");
-}
 }

@@ -203,6 +203,17 @@ int chx_hip_elementwise(
         const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
         chx_hip_tensor* const* outputs, int32_t n_outputs, void* stream);
 
+/* Diagnostics for the same op: writes the HIP source that chx_hip_elementwise would
+ * generate for these operands into `buffer` (truncated to buffer_size, always
+ * terminated; *needed receives the full size) and, when `compile` is non-zero, also
+ * runs it through hiprtc.  Touches no device memory and needs no GPU, so it is what
+ * a build machine uses to validate a program.  Counterpart of the reference's source
+ * dumps (runtime/ops/nvrtc.cc:118-123, compiler/chxvm/emitter.cc:625-627). */
+int chx_hip_elementwise_source(
+        const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
+        chx_hip_tensor* const* outputs, int32_t n_outputs, int32_t compile, char* buffer, size_t buffer_size,
+        size_t* needed);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,92 @@
+"""Host logic of the fused element-wise path, exercised without a GPU: program
+parsing, operand-layout planning, source generation and hiprtc compilation for
+gfx950 (hiprtc cross-compiles without a device)."""
+import pytest
+import torch
+
+import __graft_entry__ as entry
+
+pkg = entry.load_package()
+capi, ops = pkg.capi, pkg.ops
+
+F32 = torch.float32
+CHAIN = ops.fusion_program(
+    [("x", F32), ("a", F32), ("b", F32), ("c", F32)],
+    [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+     ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")],
+    [("y", F32)])
+
+
+def fake(shape, dtype=capi.FLOAT32, es=4, addr=0x10000000, strides=None):
+    if strides is None:
+        strides, acc = [], es
+        for n in reversed(shape):
+            strides.insert(0, acc)
+            acc *= n
+    return capi.make_desc(addr, dtype, shape, strides)
+
+
+def test_chain_plans_vector_kernel_with_periodic_broadcast():
+    full = (64, 1024, 1024)
+    src = capi.elementwise_source(CHAIN, 7, [fake(full), fake((1024,)), fake((1024,)), fake(full)], [fake(full)],
+                                  compile=True)
+    head = src.splitlines()[0]
+    assert "modes=FPPF vector" in head
+    assert "fusion7_vec" in src and "fusion7_gen" in src
+    assert "base % 1024u" in src                 # the [1024] operands are read in place, not materialised
+    assert "tanhf_faithful" in src and "sigmoid_faithful" in src
+    assert "#pragma clang fp contract(off)" in src
+
+
+def test_scalar_and_general_modes():
+    full = (8, 30)
+    src = capi.elementwise_source(CHAIN, 1, [fake(full), fake(()), fake((1,)), fake(full)], [fake(full)])
+    assert "modes=FSSF vector" in src.splitlines()[0]
+    # a column operand [8,1] is neither full, scalar nor periodic -> general kernel
+    src = capi.elementwise_source(CHAIN, 1, [fake(full), fake((8, 1)), fake((30,)), fake(full)], [fake(full)])
+    assert "general" in src.splitlines()[0]
+    # misaligned full operand -> general kernel
+    src = capi.elementwise_source(CHAIN, 1, [fake(full, addr=0x10000004), fake(()), fake(()), fake(full)], [fake(full)])
+    assert "general" in src.splitlines()[0]
+
+
+def test_quantized_chain_uses_16_wide_vectors():
+    prog = ops.fusion_program(
+        [("qa", torch.uint8), ("qb", torch.uint8)],
+        [("a", "DequantizeLinear", "qa", 0.05, 128), ("b", "DequantizeLinear", "qb", 0.02, 120),
+         ("s", "Add", "a", "b"), ("r", "Relu", "s"), ("q", "QuantizeLinear", "r", 0.06, 0, "uint8")],
+        [("q", torch.uint8)])
+    shp = (4, 64, 14, 14)
+    u8 = dict(dtype=capi.UINT8, es=1)
+    src = capi.elementwise_source(prog, 2, [fake(shp, **u8), fake(shp, **u8)], [fake(shp, **u8)], compile=True)
+    assert "modes=FF vector" in src.splitlines()[0]
+    assert "int x0[16]" in src
+
+
+@pytest.mark.parametrize("prog,msg", [
+    ("extern \"C\" __global__ void fusion0() {}", "header"),
+    ("chxhip-fusion 1\nin x:float32\ny = Cosh x\nout y:float32\n", "not in the fusable set"),
+    ("chxhip-fusion 1\nin x:float32\ny = Add x z\nout y:float32\n", "before definition"),
+    ("chxhip-fusion 1\nin x:float32\ny = Add x\nout y:float32\n", "takes 2 operands"),
+    ("chxhip-fusion 1\nin x:float32\ny = Tanh x\nout y:uint8\n", "declared uint8"),
+    ("chxhip-fusion 1\nin x:float64\ny = Tanh x\nout y:float32\n", "unsupported dtype"),
+    ("chxhip-fusion 1\nin x:uint8\ny = Tanh x\nout y:float32\n", "wrong kind"),
+    ("chxhip-fusion 1\nin x:float32\ny = QuantizeLinear x 0.1 300 uint8\nout y:uint8\n", "out of range"),
+])
+def test_program_errors(prog, msg):
+    with pytest.raises(capi.ChxHipError, match=msg):
+        u8 = dict(dtype=capi.UINT8, es=1)
+        capi.elementwise_source(prog, 0, [fake((16,), **(u8 if "x:uint8" in prog else {}))],
+                                [fake((16,), **(u8 if "y:uint8" in prog else {}))])
+
+
+def test_operand_errors():
+    with pytest.raises(capi.ChxHipError, match="does not broadcast"):
+        capi.elementwise_source(CHAIN, 0, [fake((4, 5)), fake((3,)), fake(()), fake((4, 5))], [fake((4, 5))])
+    with pytest.raises(capi.ChxHipError, match="extent"):
+        capi.elementwise_source(CHAIN, 0, [fake((4, 5)), fake(()), fake(()), fake((4, 5))], [fake((4, 6))])
+    with pytest.raises(capi.ChxHipError, match="program declares 4 inputs"):
+        capi.elementwise_source(CHAIN, 0, [fake((4, 5))], [fake((4, 5))])
+    with pytest.raises(capi.ChxHipError, match="is uint8, program says float32"):
+        capi.elementwise_source(CHAIN, 0, [fake((4, 5), dtype=capi.UINT8), fake(()), fake(()), fake((4, 5))],
+                                [fake((4, 5))])

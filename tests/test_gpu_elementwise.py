@@ -1,0 +1,161 @@
+"""Fused element-wise chains on the MI355X through the C ABI against the op-by-op
+CPU oracle (compiler/chxvm/emitter.cc:697-726: on the CPU a FusionGroup runs as its
+individual ops, one fp32 rounding each).
+
+Tolerance: the requirement is 2 ulp or 1e-6 relative per element.  The device code
+reproduces the host C library's tanhf/expf operation by operation, so the tests
+assert the stronger property, bit equality, and state the tolerance where a looser
+comparison is made on purpose."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+F32 = torch.float32
+ULP_TOL = 2
+REL_TOL = 1e-6
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+def chain_program(ops):
+    return ops.fusion_program(
+        [("x", F32), ("a", F32), ("b", F32), ("c", F32)],
+        [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+         ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")],
+        [("y", F32)])
+
+
+ORACLE_CHAIN = [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+                ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")]
+
+
+def within_tolerance(got, want):
+    ulp = np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))
+    rel = np.abs(got.astype(np.float64) - want) <= REL_TOL * np.abs(want.astype(np.float64))
+    return (ulp <= ULP_TOL) | rel | (got == want)
+
+
+def unary_program(ops, op):
+    return ops.fusion_program([("x", F32)], [("y", op, "x")], [("y", F32)])
+
+
+@pytest.mark.parametrize("op", ["Tanh", "Exp", "Sigmoid"])
+def test_transcendentals_bit_exact_over_strided_float_space(g, oracle, op):
+    # every 251st fp32 bit pattern (17.1 M inputs) plus the neighbourhoods where the
+    # algorithms switch branches
+    bits = np.arange(0, 1 << 32, 251, dtype=np.uint64).astype(np.uint32)
+    edges = np.array([0x3f800000, 0x41b00000, 0x24000000, 0x3eb17218, 0x3F851592, 0x33000000, 0x4195b844,
+                      0x42b17218, 0x42b00000, 0x42cff1b5, 0x4202422f, 0xc27c65d9, 0x7f800000, 0x00800000],
+                     dtype=np.uint32)
+    near = (edges[:, None].astype(np.int64) + np.arange(-64, 65)[None, :]).astype(np.uint32).reshape(-1)
+    bits = np.concatenate([bits, near, near | np.uint32(0x80000000)])
+    x = bits.view(np.float32)
+    want = {"Tanh": oracle.tanh, "Exp": oracle.exp, "Sigmoid": oracle.sigmoid}[op](x)
+    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, unary_program(g.ops, op))[0])
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    mism = (got.view(np.uint32) != want.view(np.uint32)) & ~nan
+    assert mism.sum() == 0, "%d of %d differ, first x=%r" % (mism.sum(), x.size, x[mism][:4])
+
+
+@pytest.mark.parametrize("shape,vec_shape", [((8, 64, 256), (256,)), ((3, 5, 7), (7,)), ((2, 1000), (1000,)),
+                                            ((1, 4), (4,)), ((5,), (1,))])
+def test_chain_matches_oracle(g, oracle, shape, vec_shape):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(shape).astype(np.float32)
+    c = rng.standard_normal(shape).astype(np.float32)
+    a = rng.standard_normal(vec_shape).astype(np.float32)
+    b = rng.standard_normal(vec_shape).astype(np.float32)
+    want = oracle.run_chain(ORACLE_CHAIN, dict(x=x, a=a, b=b, c=c))["y"]
+    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x), g.dev(a), g.dev(b), g.dev(c)], 1, chain_program(g.ops), 3)[0])
+    assert got.shape == want.shape
+    assert within_tolerance(got, want).all()          # the stated requirement
+    np.testing.assert_array_equal(got, want)          # what the implementation actually delivers
+
+
+def test_general_broadcast_and_multiple_outputs(g, oracle):
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((6, 1, 33)).astype(np.float32)
+    col = rng.standard_normal((1, 9, 1)).astype(np.float32)   # broadcasts on the outer AND the inner axis
+    prog = g.ops.fusion_program([("x", F32), ("k", F32)],
+                                [("h", "Const", 0.5), ("s", "Sub", "x", "k"), ("e", "Exp", "s"), ("d", "Div", "e", "h"),
+                                 ("m", "Max", "d", "x"), ("n", "Neg", "m"), ("cl", "Clip", "n", -3.0, 0.25)],
+                                [("d", F32), ("cl", F32)])
+    d, cl = g.ops.ElementWiseNvrtc([g.dev(x), g.dev(col)], 2, prog, 4)
+    env = oracle.run_chain([("s", "Sub", "x", "k"), ("e", "Exp", "s")], dict(x=x, k=col))
+    want_d = oracle.binary(oracle.DIV, env["e"], np.float32(0.5))
+    want_cl = oracle.clip(-np.maximum(want_d, np.broadcast_to(x, want_d.shape)), -3.0, 0.25)
+    assert d.shape == (6, 9, 33)
+    np.testing.assert_array_equal(g.host(d), want_d)
+    np.testing.assert_array_equal(g.host(cl), want_cl)
+
+
+def test_quantized_residual_add_relu(g, oracle):
+    """DequantizeLinear x2 -> Add -> Relu -> QuantizeLinear as one kernel on uint8 tensors, NCHW and
+    channels-last."""
+    rng = np.random.default_rng(13)
+    qa = rng.integers(0, 256, size=(2, 24, 9, 9)).astype(np.uint8)
+    qb = rng.integers(0, 256, size=(2, 24, 9, 9)).astype(np.uint8)
+    prog = g.ops.fusion_program(
+        [("qa", torch.uint8), ("qb", torch.uint8)],
+        [("a", "DequantizeLinear", "qa", 0.05, 128), ("b", "DequantizeLinear", "qb", 0.02, 120),
+         ("s", "Add", "a", "b"), ("r", "Relu", "s"), ("q", "QuantizeLinear", "r", 0.06, 3, "uint8")],
+        [("q", torch.uint8)])
+    s = oracle.binary(oracle.ADD, oracle.dequantize_linear(qa, 0.05, 128), oracle.dequantize_linear(qb, 0.02, 120))
+    want = oracle.quantize_linear(oracle.relu(s), 0.06, 3, np.uint8)
+    got = g.ops.ElementWiseNvrtc([g.dev(qa), g.dev(qb)], 1, prog, 5)[0]
+    np.testing.assert_array_equal(g.host(got), want)
+    cl = g.ops.ElementWiseNvrtc([g.to_channels_last(g.dev(qa)), g.to_channels_last(g.dev(qb))], 1, prog, 5)[0]
+    assert cl.stride() == g.to_channels_last(g.dev(qa)).stride()
+    np.testing.assert_array_equal(g.host(cl), want)
+
+
+def test_fused_quantize_dequantize_round_trip(g, oracle):
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal((4, 1024)) * 3).astype(np.float32)
+    prog = g.ops.fusion_program([("x", F32)], [("q", "QuantizeLinear", "x", 0.05, 0, "int8"),
+                                               ("y", "DequantizeLinear", "q", 0.05, 0)], [("y", F32)])
+    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, prog, 6)[0])
+    np.testing.assert_array_equal(got, oracle.dequantize_linear(oracle.quantize_linear(x, 0.05, 0, np.int8), 0.05, 0))
+
+
+def test_full_size_chain(g, oracle):
+    """x, c [64,1024,1024], a, b [1024]: sampled rows against the oracle plus properties that do
+    not depend on the size."""
+    torch.manual_seed(1)
+    x = torch.randn(64, 1024, 1024, device="cuda")
+    c = torch.randn(64, 1024, 1024, device="cuda")
+    a = torch.randn(1024, device="cuda")
+    b = torch.randn(1024, device="cuda")
+    y = g.ops.ElementWiseNvrtc([x, a, b, c], 1, chain_program(g.ops), 3)[0]
+    torch.cuda.synchronize()
+    assert y.shape == x.shape and float(y.min()) >= 0.0            # Relu
+    assert bool(((y == 0) | (y > 0)).all())
+    # |tanh * sigmoid| < 1, so y <= max(x + 1, 0)
+    assert bool((y <= torch.clamp(x + 1, min=0)).all())
+    rows = torch.randint(0, 64 * 1024, (96,), device="cuda")
+    xs, cs = x.view(-1, 1024)[rows].cpu().numpy(), c.view(-1, 1024)[rows].cpu().numpy()
+    want = oracle.run_chain(ORACLE_CHAIN, dict(x=xs, a=a.cpu().numpy(), b=b.cpu().numpy(), c=cs))["y"]
+    np.testing.assert_array_equal(y.view(-1, 1024)[rows].cpu().numpy(), want)
+
+
+def test_kernel_cache_and_errors(g):
+    x = torch.randn(1000, device="cuda")
+    prog = unary_program(g.ops, "Tanh")
+    y1 = g.ops.ElementWiseNvrtc([x], 1, prog)[0]
+    y2 = g.ops.ElementWiseNvrtc([x], 1, prog)[0]       # second call hits the cache
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2)
+    with pytest.raises(g.capi.ChxHipError, match="fusable set"):
+        g.ops.ElementWiseNvrtc([x], 1, unary_program(g.ops, "Erf"))
+    with pytest.raises(g.capi.ChxHipError, match="does not broadcast"):
+        g.ops.ElementWiseNvrtc([x, torch.randn(7, device="cuda")], 1,
+                               g.ops.fusion_program([("x", F32), ("z", F32)], [("y", "Add", "x", "z")], [("y", F32)]),
+                               outs=[torch.empty(1000, device="cuda")])

@@ -95,10 +95,13 @@ def test_full_size_round_trip_properties(g, oracle):
     d = g.ops.DequantizeLinear(q, 0.05, 0)
     q2 = g.ops.QuantizeLinear(d, 0.05, 0, torch.int8)
     torch.cuda.synchronize()
-    assert torch.equal(q, q2)                       # Q(DQ(q)) == q
+    # Q(DQ(q)) == q for q >= 0; for q < 0 the reference's "+0.5f then truncate" lands on q + 1
+    assert torch.equal(q2, torch.where(q < 0, q + 1, q))
     assert int(q.min()) >= -127 and int(q.max()) <= 127
     err = (d - x).abs().max().item()
     assert err <= 0.05 * 1.0001                     # |DQ(Q(x)) - x| <= scale under half-up/truncate
+    u = g.ops.QuantizeLinear(x, 0.05, 128, torch.uint8)
+    assert torch.equal(g.ops.QuantizeLinear(g.ops.DequantizeLinear(u, 0.05, 128), 0.05, 128, torch.uint8), u)
     idx = torch.randint(0, 64 * 1024 * 1024 // 4096, (257,), device="cuda")
     rows = x.view(-1, 4096)[idx]
     np.testing.assert_array_equal(q.view(-1, 4096)[idx].cpu().numpy(),
