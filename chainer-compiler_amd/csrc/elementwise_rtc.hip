@@ -321,13 +321,20 @@ int generate_source(
     const size_t nin = prog.inputs.size(), nout = prog.outputs.size();
 
     // ---- vector kernel ----
+    // `vec` elements per lane and step: 4 when any full-size operand is float32 (float32
+    // moves as one 128-bit access per lane, 8-bit codes as one 32-bit access), 16 when all
+    // of them are 8-bit (one 128-bit access each).  kSteps steps per thread at a stride of
+    // one block keep every access instruction of a wavefront on one contiguous span.
+    const int steps = 2;
     os << "extern \"C\" __global__ __launch_bounds__(256) void " << name << "_vec(unsigned int n_vec";
     for (size_t i = 0; i < nin; ++i) os << ", const " << ctype_of(prog.inputs[i].dtype) << "* __restrict__ i" << i;
     for (size_t i = 0; i < nout; ++i) os << ", " << ctype_of(prog.outputs[i].dtype) << "* __restrict__ o" << i;
     os << ") {\n";
-    os << "  const unsigned int gid = blockIdx.x * 256u + threadIdx.x;\n";
-    os << "  if (gid >= n_vec) return;\n";
-    os << "  const unsigned int base = gid * " << vec << "u;  // fewer than 2^31 elements\n";
+    os << "  const unsigned int vid0 = blockIdx.x * " << 256 * steps << "u + threadIdx.x;\n";
+    os << "#pragma unroll\n  for (int st = 0; st < " << steps << "; ++st) {\n";
+    os << "  const unsigned int vid = vid0 + st * 256u;\n";
+    os << "  if (vid < n_vec) {\n";
+    os << "  const unsigned int base = vid * " << vec << "u;  // fewer than 2^31 elements\n";
     for (size_t i = 0; i < nin; ++i) {
         const bool f32 = prog.inputs[i].dtype == CHX_HIP_FLOAT32;
         const bool sgn = prog.inputs[i].dtype == CHX_HIP_INT8;
@@ -339,17 +346,23 @@ int generate_source(
         std::string idx = "base";
         if (modes[i] == kPeriodic) idx = "(base % " + std::to_string(periods[i]) + "u)";
         const bool nt = modes[i] == kFull;
+        const char* ld0 = nt ? "__builtin_nontemporal_load(" : "*(";
         if (f32) {
             os << "  { const v4f* src = (const v4f*)(i" << i << " + " << idx << ");\n";
             for (int j = 0; j < vec / 4; ++j) {
-                os << "    const v4f t" << j << " = " << (nt ? "__builtin_nontemporal_load(src + " : "*(src + ") << j << ");\n";
+                os << "    const v4f t" << j << " = " << ld0 << "src + " << j << ");\n";
                 for (int k = 0; k < 4; ++k) os << "    x" << i << "[" << (j * 4 + k) << "] = t" << j << "[" << k << "];\n";
             }
             os << "  }\n";
         } else {
-            // vec == 16: one 128-bit load of 16 codes
-            os << "  { const v4u t = " << (nt ? "__builtin_nontemporal_load((const v4u*)(i" : "*((const v4u*)(i") << i
-               << " + " << idx << "));\n";
+            const int words = vec / 4;
+            os << "  { unsigned int t[" << words << "];\n";
+            if (words == 4) {
+                os << "    const v4u tv = " << ld0 << "(const v4u*)(i" << i << " + " << idx << "));\n";
+                os << "    t[0] = tv[0]; t[1] = tv[1]; t[2] = tv[2]; t[3] = tv[3];\n";
+            } else {
+                os << "    t[0] = " << ld0 << "(const unsigned int*)(i" << i << " + " << idx << "));\n";
+            }
             for (int e = 0; e < vec; ++e) {
                 os << "    x" << i << "[" << e << "] = ";
                 if (sgn)
@@ -376,17 +389,23 @@ int generate_source(
             }
             os << "  }\n";
         } else {
-            os << "  { v4u t;\n";
-            for (int w = 0; w < 4; ++w) {
+            const int words = vec / 4;
+            os << "  { unsigned int t[" << words << "];\n";
+            for (int w = 0; w < words; ++w) {
                 os << "    t[" << w << "] = ";
                 for (int k = 0; k < 4; ++k)
                     os << (k ? " | " : "") << "(((unsigned int)y" << i << "[" << (w * 4 + k) << "] & 0xffu) << " << (8 * k) << ")";
                 os << ";\n";
             }
-            os << "    __builtin_nontemporal_store(t, (v4u*)(o" << i << " + base));\n  }\n";
+            if (words == 4) {
+                os << "    v4u tv; tv[0] = t[0]; tv[1] = t[1]; tv[2] = t[2]; tv[3] = t[3];\n";
+                os << "    __builtin_nontemporal_store(tv, (v4u*)(o" << i << " + base));\n  }\n";
+            } else {
+                os << "    __builtin_nontemporal_store(t[0], (unsigned int*)(o" << i << " + base));\n  }\n";
+            }
         }
     }
-    os << "}\n";
+    os << "  }\n  }\n}\n";
 
     // ---- general kernel ----
     os << "struct GenDesc { int ndim; int pad; long long shape[" << CHX_HIP_MAX_NDIM << "]; long long istr[" << nin << "]["
@@ -584,10 +603,10 @@ int make_plan(
     for (int a = 0; a < plan->ndim; ++a) plan->shape[a] = cshape[a];
     plan->istr = cstr;
 
-    bool any8 = false;
-    for (const Port& p : prog.inputs) any8 = any8 || p.dtype != CHX_HIP_FLOAT32;
-    for (const Port& p : prog.outputs) any8 = any8 || p.dtype != CHX_HIP_FLOAT32;
-    plan->vec = any8 ? 16 : 4;
+    bool any32 = false;
+    for (const Port& p : prog.inputs) any32 = any32 || p.dtype == CHX_HIP_FLOAT32;
+    for (const Port& p : prog.outputs) any32 = any32 || p.dtype == CHX_HIP_FLOAT32;
+    plan->vec = any32 ? 4 : 16;
     plan->modes.assign(n_inputs, kFull);
     plan->periods.assign(n_inputs, 0);
     bool ok = n < (int64_t(1) << 31);  // CHECK_GT(1 << 31, size), runtime/ops/nvrtc.cc:127
@@ -743,7 +762,7 @@ extern "C" int chx_hip_elementwise(
         a.push((uint32_t)n_vec);
         for (int i = 0; i < n_inputs; ++i) a.push(inputs[i]->data);
         for (int i = 0; i < n_outputs; ++i) a.push(outputs[i]->data);
-        CHX_PROPAGATE(launch(ck->vec, (unsigned)((n_vec + 255) / 256), a, s));
+        CHX_PROPAGATE(launch(ck->vec, (unsigned)((n_vec + 511) / 512), a, s));
         done = n_vec * plan.vec;
     }
     if (done < plan.n) {

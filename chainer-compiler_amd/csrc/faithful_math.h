@@ -194,31 +194,79 @@ FM_FN float expm1f_faithful(float x) {
     return y;
 }
 
-// tanhf, fdlibm.
+// tanhf, fdlibm, written without data-dependent branches so that a 64-wide wavefront
+// does not serialise the algorithm's many cases: every lane evaluates the one shared
+// expm1f core (argument reduction, polynomial, one division) on the argument its case
+// calls for, all reconstruction formulas, and selects.  Each selected value is produced
+// by exactly the operations fdlibm's tanhf -> expm1f performs for that input:
+//   |x| >= 1 : t = expm1f( 2|x|), z = 1 - 2/(t+2)      (k = 3..63 in expm1f)
+//   |x| <  1 : t = expm1f(-2|x|), z = -t/(t+2)         (k = 0, -1, -2, -3)
+// with k*ln2_hi == +-ln2_hi exactly for k == +-1 and hi == x, lo == 0 for k == 0, so the
+// reduction needs no case split either.
 FM_FN float tanhf_faithful(float x) {
-    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    float t, z;
+    const float one = 1.0f, two = 2.0f;
+    const float ln2_hi = u2f(0x3f317180u);
+    const float ln2_lo = u2f(0x3717f7d1u);
+    const float invln2 = u2f(0x3fb8aa3bu);
+    const float Q1 = u2f(0xbd088889u);
+    const float Q2 = u2f(0x3ad00d01u);
+    const float Q3 = u2f(0xb8a670cdu);
+    const float Q4 = u2f(0x36867e54u);
+    const float Q5 = u2f(0xb457edbbu);
+
     const fm_u32 jx = f2u(x);
     const fm_u32 ix = jx & 0x7fffffffu;
-    if (ix >= 0x7f800000u) {
-        if ((jx >> 31) == 0) return one / x + one;
-        return one / x - one;
-    }
     const float ax = u2f(ix);
-    if (ix < 0x41b00000u) {  // |x| < 22
-        if (ix == 0) return x;
-        if (ix < 0x24000000u) return x * (one + x);  // |x| < 2^-55
-        if (ix >= 0x3f800000u) {                      // |x| >= 1
-            t = expm1f_faithful(two * ax);
-            z = one - two / (t + two);
-        } else {
-            t = expm1f_faithful(-two * ax);
-            z = -t / (t + two);
-        }
-    } else {
-        z = one - tiny;
-    }
-    return (jx >> 31) == 0 ? z : -z;
+    const bool big = ix >= 0x3f800000u;  // |x| >= 1
+    const float arg = big ? two * ax : -two * ax;
+
+    // expm1f(arg)
+    const fm_u32 hx = f2u(arg) & 0x7fffffffu;
+    fm_i32 k = (fm_i32)(invln2 * arg + (big ? 0.5f : -0.5f));
+    k = hx < 0x3F851592u ? (big ? 1 : -1) : k;  // |arg| < 1.5 ln2
+    k = hx > 0x3eb17218u ? k : 0;               // |arg| <= 0.5 ln2
+    const float tk = (float)k;
+    const float hi = arg - tk * ln2_hi;
+    const float lo = tk * ln2_lo;
+    const float xr = hi - lo;
+    const float c = (hi - xr) - lo;
+    const float hfx = 0.5f * xr;
+    const float hxs = xr * hfx;
+    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    const float t3 = 3.0f - r1 * hfx;
+    const float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+    const float y_k0 = xr - (xr * e - hxs);
+    float e2 = (xr * (e - c) - c);
+    e2 -= hxs;
+    const float y_km1 = 0.5f * (xr - e2) - 0.5f;
+    const float emx = e2 - xr;
+    const fm_u32 kshift = (fm_u32)k << 23;
+    // k <= -2 or k > 56
+    float ya = one - emx;
+    ya = u2f(f2u(ya) + kshift);
+    ya = ya - one;
+    // 1 < k < 23
+    const float tb = u2f(0x3f800000u - (0x1000000u >> ((fm_u32)k & 31u)));
+    float yb = tb - emx;
+    yb = u2f(f2u(yb) + kshift);
+    // 23 <= k <= 56
+    const float tc = u2f((fm_u32)(0x7f - k) << 23);
+    float yc = xr - (e2 + tc);
+    yc += one;
+    yc = u2f(f2u(yc) + kshift);
+    float t = k < 23 ? yb : yc;
+    t = (k <= -2 || k > 56) ? ya : t;
+    t = k == -1 ? y_km1 : t;
+    t = k == 0 ? y_k0 : t;
+    t = hx < 0x33000000u ? arg : t;  // |arg| < 2^-25: expm1f returns its argument
+
+    const float q = (big ? two : t) / (t + two);
+    float z = big ? one - q : -q;
+    z = ix >= 0x41b00000u ? one : z;           // |x| >= 22 (and +-inf): one - tiny
+    float r = (jx >> 31) == 0 ? z : -z;
+    r = ix < 0x24000000u ? x : r;              // |x| < 2^-55: x*(1+x) == x; also +-0
+    r = ix > 0x7f800000u ? x + x : r;          // NaN
+    return r;
 }
 
 // ChainerX's Sigmoid routine as the oracle restates it: Reciprocal(1 + Exp(-x)),

@@ -13,27 +13,30 @@ constexpr int kThreads = 256;
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
-// 16 elements per thread: 4 x 128-bit loads, 1 x 128-bit store.
+// One 128-bit load and one 32-bit store per lane and step, kUnroll steps per thread at
+// a stride of one block, so that every access instruction of a wavefront covers one
+// contiguous span (1 KiB in, 256 B out).
+constexpr int kUnroll = 4;
+
 template <bool kRne>
 __global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
-        const v4f* __restrict__ x, v4u* __restrict__ y, int64_t n_vec, QuantParams qp) {
-    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (i >= n_vec) return;
-    const v4f* src = x + i * 4;
-    v4f v0 = __builtin_nontemporal_load(src + 0);
-    v4f v1 = __builtin_nontemporal_load(src + 1);
-    v4f v2 = __builtin_nontemporal_load(src + 2);
-    v4f v3 = __builtin_nontemporal_load(src + 3);
-    v4u out;
-    out.x = pack4(quantize_value<kRne>(v0.x, qp), quantize_value<kRne>(v0.y, qp), quantize_value<kRne>(v0.z, qp),
-                  quantize_value<kRne>(v0.w, qp));
-    out.y = pack4(quantize_value<kRne>(v1.x, qp), quantize_value<kRne>(v1.y, qp), quantize_value<kRne>(v1.z, qp),
-                  quantize_value<kRne>(v1.w, qp));
-    out.z = pack4(quantize_value<kRne>(v2.x, qp), quantize_value<kRne>(v2.y, qp), quantize_value<kRne>(v2.z, qp),
-                  quantize_value<kRne>(v2.w, qp));
-    out.w = pack4(quantize_value<kRne>(v3.x, qp), quantize_value<kRne>(v3.y, qp), quantize_value<kRne>(v3.z, qp),
-                  quantize_value<kRne>(v3.w, qp));
-    __builtin_nontemporal_store(out, y + i);
+        const v4f* __restrict__ x, uint32_t* __restrict__ y, int64_t n_vec, QuantParams qp) {
+    const int64_t first = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+    v4f v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = first + u * kThreads;
+        if (i < n_vec) v[u] = __builtin_nontemporal_load(x + i);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = first + u * kThreads;
+        if (i < n_vec) {
+            const uint32_t out = pack4(quantize_value<kRne>(v[u].x, qp), quantize_value<kRne>(v[u].y, qp),
+                                       quantize_value<kRne>(v[u].z, qp), quantize_value<kRne>(v[u].w, qp));
+            __builtin_nontemporal_store(out, y + i);
+        }
+    }
 }
 
 // Remainder elements and unaligned buffers: one element per thread.
@@ -78,15 +81,19 @@ __device__ __forceinline__ v4f dequant4(uint32_t w, float zpf, float scale) {
 
 template <bool kSigned>
 __global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
-        const v4u* __restrict__ x, v4f* __restrict__ y, int64_t n_vec, float zpf, float scale) {
-    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    if (i >= n_vec) return;
-    const v4u q = __builtin_nontemporal_load(x + i);
-    v4f* dst = y + i * 4;
-    __builtin_nontemporal_store(dequant4<kSigned>(q.x, zpf, scale), dst + 0);
-    __builtin_nontemporal_store(dequant4<kSigned>(q.y, zpf, scale), dst + 1);
-    __builtin_nontemporal_store(dequant4<kSigned>(q.z, zpf, scale), dst + 2);
-    __builtin_nontemporal_store(dequant4<kSigned>(q.w, zpf, scale), dst + 3);
+        const uint32_t* __restrict__ x, v4f* __restrict__ y, int64_t n_vec, float zpf, float scale) {
+    const int64_t first = (int64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+    uint32_t q[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = first + u * kThreads;
+        if (i < n_vec) q[u] = __builtin_nontemporal_load(x + i);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = first + u * kThreads;
+        if (i < n_vec) __builtin_nontemporal_store(dequant4<kSigned>(q[u], zpf, scale), y + i);
+    }
 }
 
 template <bool kSigned>
@@ -111,6 +118,10 @@ __global__ __launch_bounds__(kThreads) void dequantize_strided_kernel(
 
 inline unsigned blocks_for(int64_t n) {
     return (unsigned)((n + kThreads - 1) / kThreads);
+}
+
+inline unsigned flat_blocks_for(int64_t n_vec) {
+    return (unsigned)((n_vec + kThreads * kUnroll - 1) / (kThreads * kUnroll));
 }
 
 StridedDesc make_desc(const chx_hip_tensor& t) {
@@ -150,17 +161,17 @@ extern "C" int chx_hip_quantize_linear(
         const float* xp = static_cast<const float*>(x->data);
         uint8_t* yp = static_cast<uint8_t*>(y->data);
         int64_t n_vec = 0;
-        if (aligned(xp, 16) && aligned(yp, 16)) n_vec = n / 16;
+        if (aligned(xp, 16) && aligned(yp, 16)) n_vec = n / 4;
         if (n_vec > 0) {
             if (rne)
-                quantize_flat_kernel<true><<<blocks_for(n_vec), kThreads, 0, s>>>(
-                        reinterpret_cast<const v4f*>(xp), reinterpret_cast<v4u*>(yp), n_vec, qp);
+                quantize_flat_kernel<true><<<flat_blocks_for(n_vec), kThreads, 0, s>>>(
+                        reinterpret_cast<const v4f*>(xp), reinterpret_cast<uint32_t*>(yp), n_vec, qp);
             else
-                quantize_flat_kernel<false><<<blocks_for(n_vec), kThreads, 0, s>>>(
-                        reinterpret_cast<const v4f*>(xp), reinterpret_cast<v4u*>(yp), n_vec, qp);
+                quantize_flat_kernel<false><<<flat_blocks_for(n_vec), kThreads, 0, s>>>(
+                        reinterpret_cast<const v4f*>(xp), reinterpret_cast<uint32_t*>(yp), n_vec, qp);
             CHX_PROPAGATE(launch_check("quantize_flat_kernel"));
         }
-        const int64_t done = n_vec * 16;
+        const int64_t done = n_vec * 4;
         if (done < n) {
             if (rne)
                 quantize_scalar_kernel<true><<<blocks_for(n - done), kThreads, 0, s>>>(xp, yp, done, n, qp);
@@ -198,17 +209,17 @@ extern "C" int chx_hip_dequantize_linear(
         const uint8_t* xp = static_cast<const uint8_t*>(x->data);
         float* yp = static_cast<float*>(y->data);
         int64_t n_vec = 0;
-        if (aligned(xp, 16) && aligned(yp, 16)) n_vec = n / 16;
+        if (aligned(xp, 16) && aligned(yp, 16)) n_vec = n / 4;
         if (n_vec > 0) {
             if (i8)
-                dequantize_flat_kernel<true><<<blocks_for(n_vec), kThreads, 0, s>>>(
-                        reinterpret_cast<const v4u*>(xp), reinterpret_cast<v4f*>(yp), n_vec, zpf, x_scale);
+                dequantize_flat_kernel<true><<<flat_blocks_for(n_vec), kThreads, 0, s>>>(
+                        reinterpret_cast<const uint32_t*>(xp), reinterpret_cast<v4f*>(yp), n_vec, zpf, x_scale);
             else
-                dequantize_flat_kernel<false><<<blocks_for(n_vec), kThreads, 0, s>>>(
-                        reinterpret_cast<const v4u*>(xp), reinterpret_cast<v4f*>(yp), n_vec, zpf, x_scale);
+                dequantize_flat_kernel<false><<<flat_blocks_for(n_vec), kThreads, 0, s>>>(
+                        reinterpret_cast<const uint32_t*>(xp), reinterpret_cast<v4f*>(yp), n_vec, zpf, x_scale);
             CHX_PROPAGATE(launch_check("dequantize_flat_kernel"));
         }
-        const int64_t done = n_vec * 16;
+        const int64_t done = n_vec * 4;
         if (done < n) {
             if (i8)
                 dequantize_scalar_kernel<true><<<blocks_for(n - done), kThreads, 0, s>>>(xp, yp, done, n, zpf, x_scale);

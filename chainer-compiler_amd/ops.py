@@ -81,10 +81,10 @@ def ElementWiseNvrtc(inputs, num_outputs, code, fusion_id=0, outs=None):
     broadcast of the input shapes; `num_outputs` arrays of that shape are allocated.
     When every full-shape input is channels-last the outputs are allocated
     channels-last too, so chains between convolutions never transpose."""
-    shape = torch.broadcast_shapes(*[tuple(t.shape) for t in inputs])
     out_dtypes = _program_output_dtypes(code)
     assert len(out_dtypes) == num_outputs
     if outs is None:
+        shape = torch.broadcast_shapes(*[tuple(t.shape) for t in inputs])
         full = [t for t in inputs if tuple(t.shape) == tuple(shape)]
         cl = len(shape) == 4 and full and all(
             t.permute(0, 2, 3, 1).is_contiguous() and not t.is_contiguous() for t in full)
