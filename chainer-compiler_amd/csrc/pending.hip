@@ -4,11 +4,6 @@
 
 extern "C" {
 
-int chx_hip_qlinear_conv(
-        const chx_hip_tensor*, float, int32_t, const chx_hip_tensor*, const chx_hip_tensor*, const chx_hip_tensor*,
-        float, int32_t, const chx_hip_tensor*, const chx_hip_conv_params*, uint32_t, chx_hip_tensor*, void*) {
-    CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_qlinear_conv: not implemented");
-}
 int chx_hip_qconv_plan_create(
         const chx_hip_tensor*, const chx_hip_tensor*, const chx_hip_tensor*, const chx_hip_tensor*,
         const chx_hip_conv_params*, void*, chx_hip_qconv_plan**) {
@@ -20,20 +15,5 @@ int chx_hip_qconv_plan_run(
     CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_qconv_plan_run: not implemented");
 }
 void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan*) {
-}
-int chx_hip_conv_integer(
-        const chx_hip_tensor*, const chx_hip_tensor*, int32_t, const chx_hip_tensor*, const chx_hip_conv_params*,
-        chx_hip_tensor*, void*) {
-    CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_conv_integer: not implemented");
-}
-int chx_hip_matmul_integer(
-        const chx_hip_tensor*, const chx_hip_tensor*, const chx_hip_tensor*, const chx_hip_tensor*, chx_hip_tensor*,
-        void*) {
-    CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_matmul_integer: not implemented");
-}
-int chx_hip_qlinear_matmul(
-        const chx_hip_tensor*, float, int32_t, const chx_hip_tensor*, float, int32_t, float, int32_t,
-        const chx_hip_tensor*, uint32_t, chx_hip_tensor*, void*) {
-    CHX_FAIL(CHX_HIP_EUNSUPPORTED, "chx_hip_qlinear_matmul: not implemented");
 }
 }

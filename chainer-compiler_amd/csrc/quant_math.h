@@ -68,12 +68,28 @@ __device__ __forceinline__ uint32_t pack4(int32_t a, int32_t b, int32_t c, int32
            (((uint32_t)d & 0xffu) << 24);
 }
 
-// Requantizing epilogue of the contractions: int32 accumulator -> 8-bit code.
-//   v = float(acc) * (x_scale * w_scale[oc])      (combined = fp32 product of the scales)
-//   bias per mode, then quantize_value.
+// Requantizing epilogue of the contractions: exact int32 accumulator -> 8-bit code.
+//   acc (+ bias, ONNX mode)                         int32
+//   v = float(acc) * (x_scale * w_scale[oc])        the scales' fp32 product first
+//   v = v + float(bias)                             (reference mode: runtime/ops/quantize.cc:93)
+//   code = quantize_value(v);  code = max(code, relu_floor)
 struct RequantParams {
     QuantParams q;
-    int32_t relu_floor;  // lower clamp applied to the code (y_zero_point when Relu is fused, else INT32_MIN)
+    float x_scale;
+    int32_t bias_mode;   // 0 none, 1 reference float, 2 ONNX int32
+    int32_t relu_floor;  // y_zero_point when Relu is fused, else INT32_MIN
 };
+
+enum { kBiasNone = 0, kBiasReferenceFloat = 1, kBiasOnnxInt32 = 2 };
+
+template <bool kRne>
+__device__ __forceinline__ int32_t requantize_value(int32_t acc, float w_scale, int32_t bias, const RequantParams& rp) {
+    if (rp.bias_mode == kBiasOnnxInt32) acc += bias;
+    const float s = rp.x_scale * w_scale;
+    float v = (float)acc * s;
+    if (rp.bias_mode == kBiasReferenceFloat) v = v + (float)bias;
+    const int32_t code = quantize_value<kRne>(v, rp.q);
+    return code < rp.relu_floor ? rp.relu_floor : code;
+}
 
 }  // namespace chx

@@ -98,3 +98,90 @@ def ElementWiseNvrtc(inputs, num_outputs, code, fusion_id=0, outs=None):
                                               ctypes.c_int32(len(inputs)), outp, ctypes.c_int32(len(outs)),
                                               capi.stream_ptr()))
     return outs
+
+
+# --- convolution attribute handling (runtime/chainerx_util.cc:180-200, 276-311) -----------------
+
+def _complement(values, ndim_spatial, default):
+    """ComplementStride / ComplementPad: an empty attribute means `default` per spatial axis."""
+    values = list(values)
+    return values if values else [default] * ndim_spatial
+
+
+def _auto_pad(auto_pad, in_shape, kernel, strides, pads):
+    """CalculateAutoPad: only '' (NOTSET) and 'SAME_UPPER'; the extra padding goes to the end."""
+    begin, end = list(pads), list(pads)
+    if auto_pad:
+        if auto_pad != "SAME_UPPER":
+            raise ValueError("auto_pad must be '' or 'SAME_UPPER', got %r" % auto_pad)
+        for i in range(len(pads)):
+            target = (in_shape[i] + strides[i] - 1) // strides[i]
+            need = (target - 1) * strides[i] + kernel[i] - in_shape[i]
+            begin[i] = need // 2
+            end[i] = need - begin[i]
+    return begin, end
+
+
+def _conv_setup(x, w, strides, pads, group, auto_pad):
+    strides = _complement(strides, x.dim() - 2, 1)
+    pads = _complement(pads, x.dim() - 2, 0)
+    if len(pads) == 2 * (x.dim() - 2):    # explicit begin/end list (what ApplyAsymmetricPad handles)
+        begin, end = pads[:x.dim() - 2], pads[x.dim() - 2:]
+    else:
+        begin, end = _auto_pad(auto_pad, x.shape[2:], w.shape[2:], strides, pads)
+    oh = (x.shape[2] + begin[0] + end[0] - w.shape[2]) // strides[0] + 1
+    ow = (x.shape[3] + begin[1] + end[1] - w.shape[3]) // strides[1] + 1
+    return capi.conv_params(strides, begin, end, group), (x.shape[0], w.shape[0], oh, ow)
+
+
+def _alloc_like_input_layout(x, shape, dtype):
+    if x.dim() == 4 and not x.is_contiguous() and x.permute(0, 2, 3, 1).is_contiguous():
+        return _channels_last_empty(shape, dtype, x.device)
+    return torch.empty(shape, dtype=dtype, device=x.device)
+
+
+def QLinearConv(x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_zero_point, b=None, strides=(),
+                pads=(), group=1, auto_pad="", zero_point_dtype=torch.uint8, flags=0, out=None):
+    """QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94.  The output dtype is the
+    dtype of y_zero_point."""
+    params, shape = _conv_setup(x, w, strides, pads, group, auto_pad)
+    if out is None:
+        out = _alloc_like_input_layout(x, shape, zero_point_dtype)
+    capi.check(capi.lib().chx_hip_qlinear_conv(
+        capi.ref(x), _f(x_scale), _i(x_zero_point), capi.ref(w), capi.ref(w_scale), capi.ref(w_zero_point),
+        _f(y_scale), _i(y_zero_point), capi.ref(b), ctypes.byref(params), ctypes.c_uint32(flags), capi.ref(out),
+        capi.stream_ptr()))
+    return out
+
+
+def ConvInteger(x, w, x_zero_point=None, w_zero_point=None, strides=(), pads=(), group=1, auto_pad="", out=None):
+    """ConvIntegerOp::RunImpl, runtime/ops/quantize.cc:116-146."""
+    params, shape = _conv_setup(x, w, strides, pads, group, auto_pad)
+    if out is None:
+        out = _alloc_like_input_layout(x, shape, torch.int32)
+    capi.check(capi.lib().chx_hip_conv_integer(
+        capi.ref(x), capi.ref(w), _i(0 if x_zero_point is None else x_zero_point), capi.ref(w_zero_point),
+        ctypes.byref(params), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
+def MatMulInteger(a, b, a_zero_point=None, b_zero_point=None, out=None):
+    """MatMulIntegerOp::RunImpl, runtime/ops/quantize.cc:96-114."""
+    if out is None:
+        out = torch.empty(tuple(a.shape[:-1]) + (b.shape[-1],), dtype=torch.int32, device=a.device)
+    capi.check(capi.lib().chx_hip_matmul_integer(capi.ref(a), capi.ref(b), capi.ref(a_zero_point),
+                                                 capi.ref(b_zero_point), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
+def QLinearMatMul(a, a_scale, a_zero_point, b, b_scale, b_zero_point, y_scale, y_zero_point, bias=None,
+                  zero_point_dtype=torch.uint8, flags=0, out=None):
+    """The DequantizeLinear, DequantizeLinear, MatMul, QuantizeLinear sequence that
+    ReplaceQLinearMatMul (compiler/simplifier.cc:675-694) leaves for a QLinearMatMul
+    node, as one call."""
+    if out is None:
+        out = torch.empty(tuple(a.shape[:-1]) + (b.shape[-1],), dtype=zero_point_dtype, device=a.device)
+    capi.check(capi.lib().chx_hip_qlinear_matmul(
+        capi.ref(a), _f(a_scale), _i(a_zero_point), capi.ref(b), _f(b_scale), _i(b_zero_point), _f(y_scale),
+        _i(y_zero_point), capi.ref(bias), ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
+    return out

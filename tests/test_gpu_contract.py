@@ -1,0 +1,231 @@
+"""QLinearConv, ConvInteger, MatMulInteger and QLinearMatMul on the MI355X through the
+C ABI, bit-exact against the integer-accumulating CPU oracle; the literal fp32 oracle
+is compared where both are provably identical and reported otherwise."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TDT = {np.uint8: torch.uint8, np.int8: torch.int8}
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+def rand_q(rng, shape, dtype):
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    return rng.integers(lo, hi, size=shape).astype(dtype)
+
+
+# ---- known-answer vectors of the ONNX node tests --------------------------------------------
+
+def test_onnx_qlinearconv(g, onnx_vectors):
+    t = onnx_vectors["test_qlinearconv"]
+    x = g.dev(np.array(t["x"], np.uint8).reshape(t["x_shape"]))
+    w = g.dev(np.array(t["w"], np.uint8).reshape(t["w_shape"]))
+    y = g.ops.QLinearConv(x, t["x_scale"], t["x_zero_point"], w, g.dev(np.array(t["w_scale"], np.float32)),
+                          g.dev(np.array(t["w_zero_point"], np.uint8)), t["y_scale"], t["y_zero_point"])
+    assert g.host(y).reshape(7, 7).tolist() == t["y"]
+
+
+@pytest.mark.parametrize("name", ["test_qlinearmatmul_2D", "test_qlinearmatmul_3D"])
+def test_onnx_qlinearmatmul(g, onnx_vectors, name):
+    t = onnx_vectors[name]
+    y = g.ops.QLinearMatMul(g.dev(np.array(t["a"], np.uint8)), t["a_scale"], t["a_zero_point"],
+                            g.dev(np.array(t["b"], np.uint8)), t["b_scale"], t["b_zero_point"], t["y_scale"],
+                            t["y_zero_point"])
+    assert g.host(y).tolist() == t["y"]
+
+
+def test_onnx_matmulinteger(g, onnx_vectors):
+    t = onnx_vectors["test_matmulinteger"]
+    y = g.ops.MatMulInteger(g.dev(np.array(t["a"], np.uint8)), g.dev(np.array(t["b"], np.uint8)),
+                            g.dev(np.array([t["a_zero_point"]], np.uint8)), g.dev(np.array([t["b_zero_point"]], np.uint8)))
+    assert y.dtype == torch.int32 and g.host(y).tolist() == t["y"]
+
+
+@pytest.mark.parametrize("name", ["test_basic_convinteger", "test_convinteger_with_padding"])
+def test_onnx_convinteger(g, onnx_vectors, name):
+    t = onnx_vectors[name]
+    x = g.dev(np.array(t["x"], np.uint8).reshape(t["x_shape"]))
+    w = g.dev(np.array(t["w"], np.uint8).reshape(t["w_shape"]))
+    y = g.ops.ConvInteger(x, w, t["x_zero_point"], None, pads=t["pads"])
+    assert list(y.shape) == t["y_shape"] and g.host(y).reshape(-1).tolist() == t["y"]
+
+
+# ---- random cases against the oracle ---------------------------------------------------------
+
+CONV_CASES = [
+    # N, C, H, W, OC, KH, KW, strides, pads, group, auto_pad
+    (2, 4, 7, 6, 6, 3, 3, (1, 1), (1, 1), 1, ""),
+    (1, 6, 9, 8, 4, 3, 2, (2, 1), (0, 1), 2, ""),
+    (2, 8, 5, 5, 8, 3, 3, (1, 1), (1, 1), 8, ""),        # depthwise
+    (1, 3, 23, 23, 5, 7, 7, (2, 2), (3, 3), 1, ""),      # stem-like
+    (1, 5, 6, 7, 3, 1, 1, (2, 2), (0, 0), 1, ""),        # strided pointwise
+    (1, 2, 5, 4, 2, 3, 3, (2, 2), (0, 0), 1, "SAME_UPPER"),  # asymmetric end padding
+    (2, 16, 6, 6, 32, 3, 3, (1, 1), (), 1, ""),          # empty pads attribute -> 0
+    (1, 64, 8, 8, 64, 3, 3, (), (1, 1), 1, ""),          # empty strides attribute -> 1
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("xdt,wdt", [(np.uint8, np.int8), (np.uint8, np.uint8), (np.int8, np.int8)])
+def test_conv_integer(g, oracle, case, xdt, wdt):
+    N, C, H, W, OC, KH, KW, strides, pads, group, auto_pad = case
+    rng = np.random.default_rng(21)
+    x, w = rand_q(rng, (N, C, H, W), xdt), rand_q(rng, (OC, C // group, KH, KW), wdt)
+    wz = rand_q(rng, (OC,), wdt)
+    xz = int(rand_q(rng, (1,), xdt)[0])
+    kw = dict(strides=strides or (1, 1), pads=pads or (0, 0), group=group, auto_pad=auto_pad)
+    want = oracle.conv_integer(x, w, xz, wz, **kw)
+    got = g.ops.ConvInteger(g.dev(x), g.dev(w), xz, g.dev(wz), strides=strides, pads=pads, group=group, auto_pad=auto_pad)
+    np.testing.assert_array_equal(g.host(got), want)
+    # scalar weight zero point, channels-last input view
+    want = oracle.conv_integer(x, w, xz, wz[:1], **kw)
+    got = g.ops.ConvInteger(g.to_channels_last(g.dev(x)), g.dev(w), xz, g.dev(wz[:1].reshape(())), strides=strides,
+                            pads=pads, group=group, auto_pad=auto_pad)
+    np.testing.assert_array_equal(g.host(got), want)
+    # no zero points at all
+    np.testing.assert_array_equal(
+        g.host(g.ops.ConvInteger(g.dev(x), g.dev(w), strides=strides, pads=pads, group=group, auto_pad=auto_pad)),
+        oracle.conv_integer(x, w, None, None, **kw))
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("bias_mode", ["none", "reference_float", "onnx_int32"])
+@pytest.mark.parametrize("ydt", [np.uint8, np.int8])
+def test_qlinear_conv(g, oracle, case, bias_mode, ydt):
+    N, C, H, W, OC, KH, KW, strides, pads, group, auto_pad = case
+    rng = np.random.default_rng(22)
+    x = rand_q(rng, (N, C, H, W), np.uint8)
+    w = rng.integers(-127, 128, size=(OC, C // group, KH, KW)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-1000, 1001, size=OC).astype(np.int32)
+    K = (C // group) * KH * KW
+    ys = np.float32(0.02 * 0.005 * 128 * 64 * np.sqrt(K) / 100)
+    yz = 128 if ydt == np.uint8 else -3
+    okw = dict(strides=strides or (1, 1), pads=pads or (0, 0), group=group, auto_pad=auto_pad)
+    flags, b = 0, None
+    if bias_mode == "reference_float":
+        b, okw["bias"], okw["bias_mode"] = bias, bias, oracle.BIAS_REFERENCE_FLOAT
+    elif bias_mode == "onnx_int32":
+        b, okw["bias"], okw["bias_mode"] = bias, bias, oracle.BIAS_ONNX_INT32
+        flags = g.capi.BIAS_ONNX_INT32
+    want = oracle.qlinear_conv_int(x, 0.02, 128, w, ws, wz, ys, yz, ydt, **okw)
+    got = g.ops.QLinearConv(g.dev(x), 0.02, 128, g.dev(w), g.dev(ws), g.dev(wz), ys, yz,
+                            None if b is None else g.dev(b), strides=strides, pads=pads, group=group,
+                            auto_pad=auto_pad, zero_point_dtype=TDT[ydt], flags=flags)
+    np.testing.assert_array_equal(g.host(got), want)
+    if bias_mode != "reference_float":
+        assert want.min() < want.max()
+    # channels-last in -> channels-last out, fused Relu, ONNX rounding
+    fl = flags | g.capi.FUSE_RELU | g.capi.ROUND_ONNX_RNE
+    want2 = np.maximum(oracle.qlinear_conv_int(x, 0.02, 128, w, ws, wz, ys, yz, ydt, round_mode=oracle.ROUND_ONNX_RNE,
+                                               **okw), yz).astype(ydt)
+    got2 = g.ops.QLinearConv(g.to_channels_last(g.dev(x)), 0.02, 128, g.dev(w), g.dev(ws), g.dev(wz), ys, yz,
+                             None if b is None else g.dev(b), strides=strides, pads=pads, group=group,
+                             auto_pad=auto_pad, zero_point_dtype=TDT[ydt], flags=fl)
+    assert got2.permute(0, 2, 3, 1).is_contiguous()
+    np.testing.assert_array_equal(g.host(got2), want2)
+
+
+def test_qlinear_conv_per_tensor_and_weight_zero_points(g, oracle):
+    rng = np.random.default_rng(23)
+    x = rand_q(rng, (2, 8, 9, 9), np.int8)
+    w = rand_q(rng, (12, 8, 3, 3), np.uint8)
+    for ws, wz in ((np.float32(0.004), np.uint8(131)),
+                   (rng.uniform(0.001, 0.01, size=12).astype(np.float32), rand_q(rng, (12,), np.uint8))):
+        want = oracle.qlinear_conv_int(x, 0.03, -5, w, ws, wz, 0.9, 100, np.uint8, pads=(1, 1))
+        got = g.ops.QLinearConv(g.dev(x), 0.03, -5, g.dev(w), g.dev(np.asarray(ws)), g.dev(np.asarray(wz)), 0.9, 100,
+                                pads=(1, 1))
+        np.testing.assert_array_equal(g.host(got), want)
+        assert want.min() < want.max()
+
+
+def test_qlinear_conv_equals_literal_reference_on_power_of_two_scales(g, oracle):
+    """Where the reference's fp32 contraction is exact (power-of-two scales, |acc| < 2^24) the
+    device result must equal the literal restatement of QLinearConvOp bit for bit, including
+    the reference's unscaled float bias."""
+    rng = np.random.default_rng(24)
+    x = rand_q(rng, (2, 16, 10, 10), np.uint8)
+    w = rng.integers(-127, 128, size=(24, 16, 3, 3)).astype(np.int8)
+    ws = (2.0 ** rng.integers(-9, -5, size=24)).astype(np.float32)
+    wz = np.zeros(24, np.int8)
+    bias = rng.integers(-20, 21, size=24).astype(np.int32)
+    want = oracle.qlinear_conv_literal(x, 2.0 ** -6, 128, w, ws, wz, 2.0 ** -2, 128, np.uint8, bias=bias, pads=(1, 1))
+    got = g.ops.QLinearConv(g.dev(x), 2.0 ** -6, 128, g.dev(w), g.dev(ws), g.dev(wz), 2.0 ** -2, 128, g.dev(bias),
+                            pads=(1, 1))
+    np.testing.assert_array_equal(g.host(got), want)
+    assert want.min() < want.max()
+
+
+@pytest.mark.parametrize("adt,bdt", [(np.uint8, np.int8), (np.uint8, np.uint8), (np.int8, np.int8)])
+@pytest.mark.parametrize("shape", [((5, 37), (37, 11)), ((3, 5, 37), (3, 37, 11)), ((32, 784), (784, 100)),
+                                   ((2, 2, 4, 16), (2, 2, 16, 8))])
+def test_matmul_integer(g, oracle, adt, bdt, shape):
+    rng = np.random.default_rng(25)
+    a, b = rand_q(rng, shape[0], adt), rand_q(rng, shape[1], bdt)
+    az, bz = rand_q(rng, (1,), adt), rand_q(rng, (shape[1][-1],), bdt)
+    want = oracle.matmul_integer(a, b, az, bz)
+    got = g.ops.MatMulInteger(g.dev(a), g.dev(b), g.dev(az), g.dev(bz))
+    np.testing.assert_array_equal(g.host(got), want)
+    ak = rand_q(rng, (shape[0][-1],), adt)   # 1-D a zero point lines up with K (plain broadcasting)
+    np.testing.assert_array_equal(g.host(g.ops.MatMulInteger(g.dev(a), g.dev(b), g.dev(ak), None)),
+                                  oracle.matmul_integer(a, b, ak, None))
+    # transposed (strided) operand
+    bt = g.dev(np.ascontiguousarray(np.swapaxes(b, -1, -2))).transpose(-1, -2)
+    np.testing.assert_array_equal(g.host(g.ops.MatMulInteger(g.dev(a), bt, None, g.dev(bz))),
+                                  oracle.matmul_integer(a, b, None, bz))
+
+
+def test_mlp_configuration(g, oracle):
+    """MLP 784-100-100-10, batch 32: QuantizeLinear -> (QLinearMatMul + bias + Relu) x2 ->
+    QLinearMatMul -> DequantizeLinear; uint8 activations zp 128 scale 1/255, int8 symmetric
+    per-tensor weights from N(0, 0.05), int32 bias."""
+    rng = np.random.default_rng(0)
+    x = rng.uniform(0, 1, size=(32, 784)).astype(np.float32)
+    dims = [784, 100, 100, 10]
+    s_act = np.float32(1 / 255)
+    h_d = g.ops.QuantizeLinear(g.dev(x), s_act, 128, torch.uint8)
+    h_o = oracle.quantize_linear(x, s_act, 128, np.uint8)
+    for i in range(3):
+        wf = (rng.standard_normal((dims[i], dims[i + 1])) * 0.05).astype(np.float32)
+        # compiler/quantize.cc:77-81: scale = 2 max|w| / 254, q = rint(w / scale)
+        s_w = np.float32(np.float32(np.abs(wf).max() * 2) / np.float32(254))
+        wq = np.rint(wf / s_w).astype(np.int8)
+        bias = rng.integers(-2000, 2000, size=dims[i + 1]).astype(np.int32)
+        relu = i < 2
+        s_y = np.float32(s_act * 8)
+        h_o = oracle.qlinear_matmul_int(h_o, s_act if i == 0 else s_prev, 128, wq, s_w, 0, s_y, 128, bias=bias, relu=relu)
+        h_d = g.ops.QLinearMatMul(h_d, s_act if i == 0 else s_prev, 128, g.dev(wq), s_w, 0, s_y, 128, g.dev(bias),
+                                  flags=g.capi.FUSE_RELU if relu else 0)
+        s_prev = s_y
+        np.testing.assert_array_equal(g.host(h_d), h_o)
+        assert h_o.min() < h_o.max()
+    out = g.ops.DequantizeLinear(h_d, s_prev, 128)
+    np.testing.assert_array_equal(g.host(out), oracle.dequantize_linear(h_o, s_prev, 128))
+
+
+def test_errors(g):
+    x = torch.zeros((1, 4, 5, 5), dtype=torch.uint8, device="cuda")
+    w = torch.zeros((6, 4, 3, 3), dtype=torch.int8, device="cuda")
+    ws = torch.ones(6, device="cuda")
+    wz = torch.zeros(6, dtype=torch.int8, device="cuda")
+    with pytest.raises(g.capi.ChxHipError, match="expected \\[1,6,3,3\\]"):
+        g.ops.QLinearConv(x, 1.0, 0, w, ws, wz, 1.0, 0, out=torch.zeros((1, 6, 5, 5), dtype=torch.uint8, device="cuda"))
+    with pytest.raises(g.capi.ChxHipError, match="channels"):
+        g.ops.QLinearConv(x, 1.0, 0, w, ws, wz, 1.0, 0, group=2)
+    with pytest.raises(g.capi.ChxHipError, match="same shape"):
+        g.ops.QLinearConv(x, 1.0, 0, w, ws, wz[:1], 1.0, 0)
+    with pytest.raises(g.capi.ChxHipError, match="bias must be int32"):
+        g.ops.QLinearConv(x, 1.0, 0, w, ws, wz, 1.0, 0, torch.zeros(6, device="cuda"))
+    with pytest.raises(g.capi.ChxHipError, match="inner dimensions"):
+        g.ops.MatMulInteger(torch.zeros((2, 3), dtype=torch.uint8, device="cuda"),
+                            torch.zeros((4, 5), dtype=torch.uint8, device="cuda"),
+                            out=torch.zeros((2, 5), dtype=torch.int32, device="cuda"))
