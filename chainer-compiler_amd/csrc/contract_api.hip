@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "contract.h"
+#include "conv_mfma.h"
 
 namespace chx {
 namespace {
@@ -159,10 +160,407 @@ void fill_matmul_args(
     m->b_signed = b.dtype == CHX_HIP_INT8;
 }
 
+
+// ---- MFMA path -------------------------------------------------------------------------------
+
+inline int round_up(int v, int m) {
+    return (v + m - 1) / m * m;
+}
+
+// Packed weights for the MFMA kernel (see conv_mfma.hip).
+struct PackedWeights {
+    int8_t* wp = nullptr;
+    int32_t* wsum = nullptr;
+    int C64 = 0, OCpad = 0, KP = 0;
+};
+
+size_t packed_bytes(int OC, int C, int KH, int KW, PackedWeights* pw) {
+    pw->C64 = round_up(C, 64);
+    pw->OCpad = round_up(OC, 128);
+    pw->KP = KH * KW * pw->C64;
+    return (size_t)pw->OCpad * pw->KP;
+}
+
+// The weights qualify for the MFMA kernel: one group, int8, accumulator cannot overflow.
+bool weights_fit_mfma(const chx_hip_tensor& w, int group) {
+    if (group != 1 || w.dtype != CHX_HIP_INT8) return false;
+    const int64_t K = (int64_t)round_up((int)w.shape[1], 64) * w.shape[2] * w.shape[3];
+    return K * 128 * 128 < (int64_t(1) << 31) && w.shape[0] < (1 << 24);
+}
+
+// Tile shape: the largest tile that still gives every compute unit about two work-groups.
+void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px) {
+    static const int cand[4][2] = {{128, 128}, {64, 128}, {128, 64}, {64, 64}};
+    const int64_t want = 2 * 256;
+    for (int i = 0; i < 4; ++i) {
+        int toc = cand[i][0], tpx = cand[i][1];
+        if (OC <= 64 && toc > 64) continue;
+        const int64_t blocks = (int64_t)((OC + toc - 1) / toc) * ((M + tpx - 1) / tpx);
+        *tile_oc = toc;
+        *tile_px = tpx;
+        if (blocks >= want) return;
+    }
+}
+
+struct XLayout {
+    const char* ptr;
+    int64_t n_stride, h_stride, w_stride;
+    bool direct;  // usable as is
+};
+
+// channels-last view with 16-byte aligned pixels whose pitch covers round_up(C, 16) bytes
+bool x_is_mfma_ready(const chx_hip_tensor& x) {
+    const int64_t C = x.shape[1];
+    if (C != 1 && x.strides[1] != 1) return false;
+    const int64_t c16 = (C + 15) / 16 * 16;
+    if (!aligned(x.data, 16)) return false;
+    for (int ax : {0, 2, 3}) {
+        if (x.shape[ax] == 1) continue;
+        if (x.strides[ax] % 16 != 0 || x.strides[ax] < c16) return false;
+    }
+    // reading c16 bytes of the last pixel must stay inside the allocation: guaranteed when every
+    // pixel pitch covers c16 bytes, which the loop above checked for all axes of extent > 1
+    if (x.shape[3] == 1 && x.shape[2] == 1 && x.shape[0] == 1) return C == c16;
+    return true;
+}
+
+// pixel-major output: (n, oh, ow) collapse to one index with a single stride, channels unit stride
+bool y_is_pixel_major(const chx_hip_tensor& y, int64_t* px_stride) {
+    const int64_t es = dtype_size(y.dtype);
+    if (y.shape[1] != 1 && y.strides[1] != es) return false;
+    int64_t stride = -1, expect = -1;
+    for (int ax : {3, 2, 0}) {
+        if (y.shape[ax] == 1) continue;
+        if (stride < 0) {
+            stride = y.strides[ax];
+            expect = stride * y.shape[ax];
+        } else {
+            if (y.strides[ax] != expect) return false;
+            expect *= y.shape[ax];
+        }
+    }
+    if (stride < 0) stride = y.shape[1] * es;
+    if (stride < y.shape[1] * es) return false;
+    *px_stride = stride;
+    return true;
+}
+
+struct ConvCall {
+    const chx_hip_tensor* x;
+    chx_hip_tensor* y;
+    const chx_hip_conv_params* p;
+    ConvShape cs;
+    int32_t x_zp;
+    bool out_int32;
+    bool rne;
+    const float* w_scale;
+    int32_t w_scale_len;
+    const int32_t* bias;
+    RequantParams rq;
+};
+
+// Runs the MFMA kernel on packed weights.  x may be channels-last (used in place) or
+// NCHW-contiguous (transposed into scratch first); y may be pixel-major (written in place) or
+// NCHW-contiguous 8-bit (written to scratch, then transposed).  Returns EUNSUPPORTED when the
+// operand layouts fit neither, so that the caller can fall back to the direct kernel.
+int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
+    const chx_hip_tensor& x = *c.x;
+    chx_hip_tensor& y = *c.y;
+    const ConvShape& cs = c.cs;
+    const int C16 = round_up(cs.C, 16);
+    void* x_scratch = nullptr;
+    void* y_scratch = nullptr;
+    ConvMfmaArgs a;
+    memset(&a, 0, sizeof(a));
+    if (x_is_mfma_ready(x)) {
+        a.x = static_cast<const char*>(x.data);
+        a.x_n_stride = x.strides[0];
+        a.x_h_stride = x.strides[2];
+        a.x_w_stride = x.strides[3];
+    } else if (is_contiguous(x)) {
+        const int64_t HW = (int64_t)cs.H * cs.W;
+        CHX_PROPAGATE(scratch_alloc(&x_scratch, (size_t)cs.N * HW * C16, s));
+        CHX_PROPAGATE(launch_nchw_to_nhwc_u8(static_cast<const char*>(x.data), static_cast<char*>(x_scratch), cs.N, cs.C,
+                                             HW, C16, s));
+        a.x = static_cast<const char*>(x_scratch);
+        a.x_w_stride = C16;
+        a.x_h_stride = (int64_t)cs.W * C16;
+        a.x_n_stride = HW * C16;
+    } else {
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "x layout is neither channels-last nor NCHW-contiguous");
+    }
+    const int64_t es = c.out_int32 ? 4 : 1;
+    int64_t y_px = 0;
+    bool y_post = false;
+    if (y_is_pixel_major(y, &y_px)) {
+        a.y = static_cast<char*>(y.data);
+        a.y_px_stride = y_px;
+    } else if (is_contiguous(y) && !c.out_int32) {
+        const int64_t OHW = (int64_t)cs.OH * cs.OW;
+        const int pitch = round_up(cs.OC, 16);
+        if (scratch_alloc(&y_scratch, (size_t)cs.N * OHW * pitch, s) != CHX_HIP_OK) {
+            scratch_free(x_scratch, s);
+            return CHX_HIP_ERUNTIME;
+        }
+        a.y = static_cast<char*>(y_scratch);
+        a.y_px_stride = pitch;
+        y_post = true;
+    } else {
+        scratch_free(x_scratch, s);
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "y layout is neither pixel-major nor NCHW-contiguous 8-bit");
+    }
+    a.y_vec_ok = aligned(a.y, 16) && (a.y_px_stride % 16 == 0) ? 1 : 0;
+    (void)es;
+    a.C16 = C16;
+    a.C64 = pw.C64;
+    a.H = cs.H; a.W = cs.W; a.OH = cs.OH; a.OW = cs.OW; a.KH = cs.KH; a.KW = cs.KW;
+    a.sh = c.p->stride_h; a.sw = c.p->stride_w; a.ph = c.p->pad_h_begin; a.pw = c.p->pad_w_begin;
+    a.M = (int64_t)cs.N * cs.OH * cs.OW;
+    a.OC = cs.OC;
+    a.KP = pw.KP;
+    a.nk = pw.KP / 64;
+    a.wp = pw.wp;
+    a.wsum = pw.wsum;
+    a.x_zp = c.x_zp;
+    const bool xu = x.dtype == CHX_HIP_UINT8;
+    a.corr_mult = xu ? 128 - c.x_zp : -c.x_zp;
+    a.w_scale = c.w_scale;
+    a.w_scale_len = c.w_scale_len;
+    a.bias = c.bias;
+    a.rq = c.rq;
+    int toc = 64, tpx = 64;
+    pick_tile(cs.OC, a.M, &toc, &tpx);
+    int rc = launch_conv_mfma(a, toc, tpx, xu, c.out_int32, c.rne, s);
+    if (rc == CHX_HIP_OK && y_post) {
+        rc = launch_nhwc_to_nchw_u8(static_cast<const char*>(y_scratch), static_cast<char*>(y.data), cs.N, cs.OC,
+                                    (int64_t)cs.OH * cs.OW, (int)a.y_px_stride, s);
+    }
+    scratch_free(x_scratch, s);
+    scratch_free(y_scratch, s);
+    return rc;
+}
+
+// Reads a small parameter vector back to the host (synchronizes the stream).
+int read_back(const chx_hip_tensor& t, std::vector<uint8_t>* out, hipStream_t s) {
+    const int64_t n = numel(t);
+    out->resize((size_t)n);
+    if (n == 0) return CHX_HIP_OK;
+    if (t.ndim == 0 || t.strides[0] == 1 || n == 1) {
+        CHX_HIP_CALL(hipMemcpyAsync(out->data(), t.data, (size_t)n, hipMemcpyDeviceToHost, s));
+    } else {
+        CHX_HIP_CALL(hipMemcpy2DAsync(out->data(), 1, t.data, (size_t)t.strides[0], 1, (size_t)n, hipMemcpyDeviceToHost, s));
+    }
+    CHX_HIP_CALL(hipStreamSynchronize(s));
+    return CHX_HIP_OK;
+}
+
+bool all_zero(const std::vector<uint8_t>& v) {
+    for (uint8_t b : v)
+        if (b) return false;
+    return true;
+}
+
 }  // namespace
 }  // namespace chx
 
 using namespace chx;
+
+
+namespace chx {
+namespace {
+
+// Allocates and fills packed weights.  With `persistent` the buffers come from hipMalloc and
+// live until release_packed(); otherwise they are stream-ordered scratch.
+int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedWeights* pw) {
+    const size_t bytes = packed_bytes((int)w.shape[0], (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], pw);
+    void* p0 = nullptr;
+    void* p1 = nullptr;
+    if (persistent) {
+        CHX_HIP_CALL(hipMalloc(&p0, bytes));
+        if (hipMalloc(&p1, sizeof(int32_t) * pw->OCpad) != hipSuccess) {
+            (void)hipFree(p0);
+            CHX_FAIL(CHX_HIP_ERUNTIME, "hipMalloc failed for the per-channel weight sums");
+        }
+    } else {
+        CHX_PROPAGATE(scratch_alloc(&p0, bytes, s));
+        if (scratch_alloc(&p1, sizeof(int32_t) * pw->OCpad, s) != CHX_HIP_OK) {
+            scratch_free(p0, s);
+            return CHX_HIP_ERUNTIME;
+        }
+    }
+    pw->wp = static_cast<int8_t*>(p0);
+    pw->wsum = static_cast<int32_t*>(p1);
+    return pack_weights(w, pw->C64, pw->OCpad, pw->wp, pw->wsum, s);
+}
+
+void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
+    if (persistent) {
+        if (pw->wp) (void)hipFree(pw->wp);
+        if (pw->wsum) (void)hipFree(pw->wsum);
+    } else {
+        scratch_free(pw->wp, s);
+        scratch_free(pw->wsum, s);
+    }
+    pw->wp = nullptr;
+    pw->wsum = nullptr;
+}
+
+struct QConvChecked {
+    ConvShape cs;
+    ConvDirectArgs direct;
+};
+
+// Validation shared by the one-shot call and the plan: everything QLinearConvOp::RunImpl CHECKs.
+int check_qconv(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
+        const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_params* params, uint32_t flags, chx_hip_tensor* y, QConvChecked* out) {
+    CHX_PROPAGATE(check_tensor(x, "QLinearConv x"));
+    CHX_PROPAGATE(check_tensor(w, "QLinearConv w"));
+    CHX_PROPAGATE(check_tensor(w_scale, "QLinearConv w_scale"));
+    CHX_PROPAGATE(check_tensor(w_zero_point, "QLinearConv w_zero_point"));
+    CHX_PROPAGATE(check_tensor(y, "QLinearConv y"));
+    CHX_REQUIRE(params != nullptr, "QLinearConv: null params");
+    ConvShape& cs = out->cs;
+    CHX_PROPAGATE(conv_shape(*x, *w, *params, *y, "QLinearConv", &cs));
+    CHX_REQUIRE(w_scale->dtype == CHX_HIP_FLOAT32, "QLinearConv: w_scale must be float32");
+    CHX_REQUIRE(w_zero_point->dtype == w->dtype, "QLinearConv: w_zero_point must have the dtype of w");
+    // CHECK_EQ(w_scale.GetTotalSize(), w_zero_point.GetTotalSize()), runtime/ops/quantize.cc:76-77
+    int64_t slen, sstride, zlen, zstride;
+    CHX_PROPAGATE(param_vector(*w_scale, cs.OC, "QLinearConv w_scale", &slen, &sstride));
+    CHX_PROPAGATE(param_vector(*w_zero_point, cs.OC, "QLinearConv w_zero_point", &zlen, &zstride));
+    CHX_REQUIRE(slen == zlen && w_scale->ndim == w_zero_point->ndim,
+                "QLinearConv: w_scale and w_zero_point must have the same shape");
+    CHX_REQUIRE(slen == 1 || sstride == 4, "QLinearConv: w_scale must be contiguous");
+    ConvDirectArgs& a = out->direct;
+    fill_conv_args(*x, *w, *params, *y, cs, &a);
+    a.x_zp = x_zero_point;
+    a.w_zp = static_cast<const char*>(w_zero_point->data);
+    a.w_zp_len = (int32_t)zlen;
+    a.w_zp_stride = zstride;
+    a.requant = 1;
+    a.w_scale = static_cast<const float*>(w_scale->data);
+    a.w_scale_len = (int32_t)slen;
+    CHX_PROPAGATE(fill_requant(x_scale, y_scale, y_zero_point, *y, bias, cs.OC, flags, "QLinearConv", &a.rq, &a.bias));
+    return CHX_HIP_OK;
+}
+
+ConvCall conv_call_from(const QConvChecked& q, const chx_hip_tensor* x, chx_hip_tensor* y, const chx_hip_conv_params* p,
+                        bool rne) {
+    ConvCall c;
+    c.x = x;
+    c.y = y;
+    c.p = p;
+    c.cs = q.cs;
+    c.x_zp = q.direct.x_zp;
+    c.out_int32 = false;
+    c.rne = rne;
+    c.w_scale = q.direct.w_scale;
+    c.w_scale_len = q.direct.w_scale_len;
+    c.bias = q.direct.bias;
+    c.rq = q.direct.rq;
+    return c;
+}
+
+}  // namespace
+}  // namespace chx
+
+struct chx_hip_qconv_plan {
+    chx_hip_tensor w, w_scale, w_zero_point, bias;
+    bool has_bias;
+    chx_hip_conv_params params;
+    bool mfma;
+    chx::PackedWeights pw;
+};
+
+extern "C" int chx_hip_qlinear_conv(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
+        const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_params* params, uint32_t flags, chx_hip_tensor* y, void* stream) {
+    QConvChecked q;
+    CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_zero_point, bias, params,
+                              flags, y, &q));
+    hipStream_t s = as_stream(stream);
+    const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
+    if (weights_fit_mfma(*w, params->group)) {
+        std::vector<uint8_t> zp;
+        CHX_PROPAGATE(read_back(*w_zero_point, &zp, s));
+        if (all_zero(zp)) {
+            PackedWeights pw;
+            CHX_PROPAGATE(make_packed(*w, false, s, &pw));
+            const int rc = run_conv_mfma(conv_call_from(q, x, y, params, rne), pw, s);
+            release_packed(&pw, false, s);
+            if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        }
+    }
+    return launch_conv_direct(q.direct, rne, s);
+}
+
+extern "C" int chx_hip_qconv_plan_create(
+        const chx_hip_tensor* w, const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_params* params, void* stream, chx_hip_qconv_plan** plan) {
+    CHX_REQUIRE(plan != nullptr, "QLinearConv plan: null output");
+    *plan = nullptr;
+    CHX_PROPAGATE(check_tensor(w, "QLinearConv w"));
+    CHX_PROPAGATE(check_tensor(w_scale, "QLinearConv w_scale"));
+    CHX_PROPAGATE(check_tensor(w_zero_point, "QLinearConv w_zero_point"));
+    CHX_REQUIRE(params != nullptr, "QLinearConv plan: null params");
+    CHX_REQUIRE(w->ndim == 4 && is_q8(w->dtype), "QLinearConv plan: w must be a 4-D uint8/int8 tensor");
+    if (bias) CHX_PROPAGATE(check_tensor(bias, "QLinearConv bias"));
+    hipStream_t s = as_stream(stream);
+    chx_hip_qconv_plan* p = new chx_hip_qconv_plan();
+    p->w = *w;
+    p->w_scale = *w_scale;
+    p->w_zero_point = *w_zero_point;
+    p->has_bias = bias != nullptr;
+    if (bias) p->bias = *bias;
+    p->params = *params;
+    p->mfma = false;
+    if (weights_fit_mfma(*w, params->group) && w_zero_point->dtype == w->dtype && w_zero_point->ndim <= 1) {
+        std::vector<uint8_t> zp;
+        int rc = read_back(*w_zero_point, &zp, s);
+        if (rc == CHX_HIP_OK && all_zero(zp)) {
+            rc = make_packed(*w, true, s, &p->pw);
+            if (rc == CHX_HIP_OK) {
+                hipError_t e = hipStreamSynchronize(s);
+                if (e != hipSuccess) {
+                    set_error("hipStreamSynchronize failed: %s", hipGetErrorString(e));
+                    rc = CHX_HIP_ERUNTIME;
+                }
+            }
+            if (rc == CHX_HIP_OK) p->mfma = true;
+        }
+        if (rc != CHX_HIP_OK) {
+            release_packed(&p->pw, true, s);
+            delete p;
+            return rc;
+        }
+    }
+    *plan = p;
+    return CHX_HIP_OK;
+}
+
+extern "C" int chx_hip_qconv_plan_run(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
+        int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream) {
+    CHX_REQUIRE(plan != nullptr, "QLinearConv plan: null plan");
+    QConvChecked q;
+    CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, &plan->w, &plan->w_scale, &plan->w_zero_point, y_scale,
+                              y_zero_point, plan->has_bias ? &plan->bias : nullptr, &plan->params, flags, y, &q));
+    hipStream_t s = as_stream(stream);
+    const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
+    if (plan->mfma) {
+        const int rc = run_conv_mfma(conv_call_from(q, x, y, &plan->params, rne), plan->pw, s);
+        if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+    }
+    return launch_conv_direct(q.direct, rne, s);
+}
+
+extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {
+    if (!plan) return;
+    chx::release_packed(&plan->pw, true, nullptr);
+    delete plan;
+}
 
 extern "C" int chx_hip_conv_integer(
         const chx_hip_tensor* x, const chx_hip_tensor* w, int32_t x_zero_point, const chx_hip_tensor* w_zero_point,
@@ -186,8 +584,114 @@ extern "C" int chx_hip_conv_integer(
         a.w_zp_len = (int32_t)len;
         a.w_zp_stride = stride;
     }
-    return launch_conv_direct(a, false, as_stream(stream));
+    hipStream_t s = as_stream(stream);
+    if (weights_fit_mfma(*w, params->group)) {
+        bool zero = true;
+        if (w_zero_point) {
+            std::vector<uint8_t> zp;
+            CHX_PROPAGATE(read_back(*w_zero_point, &zp, s));
+            zero = all_zero(zp);
+        }
+        if (zero) {
+            ConvCall c;
+            memset(&c, 0, sizeof(c));
+            c.x = x;
+            c.y = y;
+            c.p = params;
+            c.cs = cs;
+            c.x_zp = x_zero_point;
+            c.out_int32 = true;
+            PackedWeights pw;
+            CHX_PROPAGATE(make_packed(*w, false, s, &pw));
+            const int rc = run_conv_mfma(c, pw, s);
+            release_packed(&pw, false, s);
+            if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        }
+    }
+    return launch_conv_direct(a, false, s);
 }
+
+namespace chx {
+namespace {
+
+// A 2-D matrix product as a 1x1 convolution over M "pixels": a [M,K] is a channels-last
+// activation row per pixel, b [K,N] the weights of N output channels.
+int matmul_via_mfma(
+        const chx_hip_tensor& a, const chx_hip_tensor& b, chx_hip_tensor& y, const MatMulShape& ms, int32_t a_zp,
+        bool out_int32, bool rne, float b_scale, const int32_t* bias, const RequantParams& rq, hipStream_t s) {
+    const int nd = a.ndim;
+    if (ms.batch != 1 || b.dtype != CHX_HIP_INT8 || ms.M > INT32_MAX || ms.K > (1 << 20) || ms.N >= (1 << 24))
+        return CHX_HIP_EUNSUPPORTED;
+    chx_hip_tensor x4, w4, y4;
+    memset(&x4, 0, sizeof(x4));
+    memset(&w4, 0, sizeof(w4));
+    memset(&y4, 0, sizeof(y4));
+    x4.data = a.data; x4.dtype = a.dtype; x4.ndim = 4;
+    x4.shape[0] = 1; x4.shape[1] = ms.K; x4.shape[2] = 1; x4.shape[3] = ms.M;
+    x4.strides[0] = 0; x4.strides[1] = a.strides[nd - 1]; x4.strides[2] = 0; x4.strides[3] = a.strides[nd - 2];
+    w4.data = b.data; w4.dtype = b.dtype; w4.ndim = 4;
+    w4.shape[0] = ms.N; w4.shape[1] = ms.K; w4.shape[2] = 1; w4.shape[3] = 1;
+    w4.strides[0] = b.strides[nd - 1]; w4.strides[1] = b.strides[nd - 2]; w4.strides[2] = 0; w4.strides[3] = 0;
+    y4.data = y.data; y4.dtype = y.dtype; y4.ndim = 4;
+    y4.shape[0] = 1; y4.shape[1] = ms.N; y4.shape[2] = 1; y4.shape[3] = ms.M;
+    y4.strides[0] = 0; y4.strides[1] = y.strides[nd - 1]; y4.strides[2] = 0; y4.strides[3] = y.strides[nd - 2];
+    if (!weights_fit_mfma(w4, 1) || !x_is_mfma_ready(x4)) return CHX_HIP_EUNSUPPORTED;
+    int64_t px;
+    if (!y_is_pixel_major(y4, &px)) return CHX_HIP_EUNSUPPORTED;
+    chx_hip_conv_params p = {1, 1, 0, 0, 0, 0, 1};
+    ConvCall c;
+    memset(&c, 0, sizeof(c));
+    c.x = &x4;
+    c.y = &y4;
+    c.p = &p;
+    c.cs.N = 1; c.cs.C = (int32_t)ms.K; c.cs.H = 1; c.cs.W = (int32_t)ms.M;
+    c.cs.OC = (int32_t)ms.N; c.cs.Cg = (int32_t)ms.K; c.cs.KH = 1; c.cs.KW = 1; c.cs.OH = 1; c.cs.OW = (int32_t)ms.M;
+    c.x_zp = a_zp;
+    c.out_int32 = out_int32;
+    c.rne = rne;
+    static const float kOne = 0.f;
+    (void)kOne;
+    c.w_scale = nullptr;
+    c.w_scale_len = 1;
+    c.bias = bias;
+    c.rq = rq;
+    PackedWeights pw;
+    CHX_PROPAGATE(make_packed(w4, false, s, &pw));
+    // the per-tensor b_scale is a host value; the kernel reads scales from device memory
+    void* scale_dev = nullptr;
+    int rc = CHX_HIP_OK;
+    if (!out_int32) {
+        rc = scratch_alloc(&scale_dev, sizeof(float), s);
+        if (rc == CHX_HIP_OK && hipMemcpyAsync(scale_dev, &b_scale, sizeof(float), hipMemcpyHostToDevice, s) != hipSuccess) {
+            set_error("hipMemcpyAsync of the weight scale failed");
+            rc = CHX_HIP_ERUNTIME;
+        }
+        c.w_scale = static_cast<const float*>(scale_dev);
+    }
+    if (rc == CHX_HIP_OK) rc = run_conv_mfma(c, pw, s);
+    scratch_free(scale_dev, s);
+    release_packed(&pw, false, s);
+    return rc;
+}
+
+// Scalar zero point held in a device array of one element (or absent): host value, via a
+// synchronizing read.  Returns false when the array is a per-axis vector.
+int scalar_zero_point(const chx_hip_tensor* zp, hipStream_t s, bool* is_scalar, int32_t* value) {
+    *is_scalar = true;
+    *value = 0;
+    if (!zp) return CHX_HIP_OK;
+    if (numel(*zp) != 1) {
+        *is_scalar = false;
+        return CHX_HIP_OK;
+    }
+    std::vector<uint8_t> v;
+    CHX_PROPAGATE(read_back(*zp, &v, s));
+    *value = zp->dtype == CHX_HIP_INT8 ? (int32_t)(int8_t)v[0] : (int32_t)v[0];
+    return CHX_HIP_OK;
+}
+
+}  // namespace
+}  // namespace chx
 
 extern "C" int chx_hip_matmul_integer(
         const chx_hip_tensor* a, const chx_hip_tensor* b, const chx_hip_tensor* a_zero_point,
@@ -221,7 +725,20 @@ extern "C" int chx_hip_matmul_integer(
         m.b_zp_stride = stride;
         m.b_zp_signed = b_zero_point->dtype == CHX_HIP_INT8;
     }
-    return launch_matmul_direct(m, false, as_stream(stream));
+    hipStream_t s = as_stream(stream);
+    if (ms.batch == 1 && b->dtype == CHX_HIP_INT8 && ms.M * ms.N * ms.K >= (int64_t(1) << 22)) {
+        bool a_scalar, b_scalar;
+        int32_t az, bz;
+        CHX_PROPAGATE(scalar_zero_point(a_zero_point, s, &a_scalar, &az));
+        CHX_PROPAGATE(scalar_zero_point(b_zero_point, s, &b_scalar, &bz));
+        if (a_scalar && b_scalar && bz == 0) {
+            RequantParams rq;
+            memset(&rq, 0, sizeof(rq));
+            const int rc = matmul_via_mfma(*a, *b, *y, ms, az, true, false, 0.f, nullptr, rq, s);
+            if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        }
+    }
+    return launch_matmul_direct(m, false, s);
 }
 
 extern "C" int chx_hip_qlinear_matmul(
@@ -243,39 +760,12 @@ extern "C" int chx_hip_qlinear_matmul(
     // the extension's bias is always the ONNX kind: int32, added to the accumulator
     CHX_PROPAGATE(fill_requant(a_scale, y_scale, y_zero_point, *y, bias, ms.N, flags | CHX_HIP_BIAS_ONNX_INT32,
                                "QLinearMatMul", &m.rq, &m.bias));
-    return launch_matmul_direct(m, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0, as_stream(stream));
+    hipStream_t s = as_stream(stream);
+    const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
+    if (b_zero_point == 0) {
+        const int rc = matmul_via_mfma(*a, *b, *y, ms, a_zero_point, false, rne, b_scale, m.bias, m.rq, s);
+        if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+    }
+    return launch_matmul_direct(m, rne, s);
 }
 
-extern "C" int chx_hip_qlinear_conv(
-        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
-        const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
-        const chx_hip_tensor* bias, const chx_hip_conv_params* params, uint32_t flags, chx_hip_tensor* y, void* stream) {
-    CHX_PROPAGATE(check_tensor(x, "QLinearConv x"));
-    CHX_PROPAGATE(check_tensor(w, "QLinearConv w"));
-    CHX_PROPAGATE(check_tensor(w_scale, "QLinearConv w_scale"));
-    CHX_PROPAGATE(check_tensor(w_zero_point, "QLinearConv w_zero_point"));
-    CHX_PROPAGATE(check_tensor(y, "QLinearConv y"));
-    CHX_REQUIRE(params != nullptr, "QLinearConv: null params");
-    ConvShape cs;
-    CHX_PROPAGATE(conv_shape(*x, *w, *params, *y, "QLinearConv", &cs));
-    CHX_REQUIRE(w_scale->dtype == CHX_HIP_FLOAT32, "QLinearConv: w_scale must be float32");
-    CHX_REQUIRE(w_zero_point->dtype == w->dtype, "QLinearConv: w_zero_point must have the dtype of w");
-    // CHECK_EQ(w_scale.GetTotalSize(), w_zero_point.GetTotalSize()), runtime/ops/quantize.cc:76-77
-    int64_t slen, sstride, zlen, zstride;
-    CHX_PROPAGATE(param_vector(*w_scale, cs.OC, "QLinearConv w_scale", &slen, &sstride));
-    CHX_PROPAGATE(param_vector(*w_zero_point, cs.OC, "QLinearConv w_zero_point", &zlen, &zstride));
-    CHX_REQUIRE(slen == zlen && w_scale->ndim == w_zero_point->ndim,
-                "QLinearConv: w_scale and w_zero_point must have the same shape");
-    CHX_REQUIRE(slen == 1 || sstride == 4, "QLinearConv: w_scale must be contiguous");
-    ConvDirectArgs a;
-    fill_conv_args(*x, *w, *params, *y, cs, &a);
-    a.x_zp = x_zero_point;
-    a.w_zp = static_cast<const char*>(w_zero_point->data);
-    a.w_zp_len = (int32_t)zlen;
-    a.w_zp_stride = zstride;
-    a.requant = 1;
-    a.w_scale = static_cast<const float*>(w_scale->data);
-    a.w_scale_len = (int32_t)slen;
-    CHX_PROPAGATE(fill_requant(x_scale, y_scale, y_zero_point, *y, bias, cs.OC, flags, "QLinearConv", &a.rq, &a.bias));
-    return launch_conv_direct(a, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0, as_stream(stream));
-}

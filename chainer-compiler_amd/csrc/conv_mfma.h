@@ -1,0 +1,44 @@
+// Interface of the MFMA implicit-GEMM kernel (conv_mfma.hip) and the layout helpers
+// (layout.hip) towards the entry points.
+#pragma once
+
+#include "chx_internal.h"
+#include "quant_math.h"
+
+namespace chx {
+
+struct ConvMfmaArgs {
+    // activations, channels-last: element (n, c, ih, iw) at x + n*x_n_stride + ih*x_h_stride + iw*x_w_stride + c
+    const char* x;
+    int64_t x_n_stride, x_h_stride, x_w_stride;
+    int32_t C16;  // channels rounded up to 16; the pixel pitch covers at least this many bytes
+    int32_t C64;  // channels rounded up to 64 (K bytes per filter tap in the packed weights)
+    int32_t H, W, OH, OW, KH, KW, sh, sw, ph, pw;
+    int64_t M;    // N * OH * OW
+    int32_t OC;
+    int32_t nk;   // K steps: KH * KW * C64 / 64
+    int32_t KP;   // packed row length: KH * KW * C64
+    const int8_t* wp;     // [OCpad][KP]
+    const int32_t* wsum;  // [OCpad]
+    int32_t x_zp;
+    int32_t corr_mult;    // (128 - x_zp) for uint8 x, (-x_zp) for int8 x
+    // output, pixel-major: element (m, oc) at y + m*y_px_stride + oc*elemsize
+    char* y;
+    int64_t y_px_stride;
+    int32_t y_vec_ok;     // 16-byte stores allowed (base and pitch aligned)
+    // epilogue
+    const float* w_scale;
+    int32_t w_scale_len;
+    const int32_t* bias;
+    RequantParams rq;
+    int32_t tiles_oc, tiles_px;  // filled by the launcher
+};
+
+int pack_weights(const chx_hip_tensor& w, int C64, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, bool x_unsigned, bool out_int32, bool rne, hipStream_t s);
+
+// [N][C][HW] bytes -> [N][HW][pitch] bytes (lanes c >= C of a pixel are zero filled) and back
+int launch_nchw_to_nhwc_u8(const char* src, char* dst, int N, int C, int64_t HW, int pitch, hipStream_t s);
+int launch_nhwc_to_nchw_u8(const char* src, char* dst, int N, int C, int64_t HW, int pitch, hipStream_t s);
+
+}  // namespace chx

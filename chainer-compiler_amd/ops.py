@@ -185,3 +185,45 @@ def QLinearMatMul(a, a_scale, a_zero_point, b, b_scale, b_zero_point, y_scale, y
         capi.ref(a), _f(a_scale), _i(a_zero_point), capi.ref(b), _f(b_scale), _i(b_zero_point), _f(y_scale),
         _i(y_zero_point), capi.ref(bias), ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
     return out
+
+
+class QLinearConvPlan(object):
+    """Weight-side state of one QLinearConv instruction (chx_hip_qconv_plan): repacked
+    weights and per-channel sums, built once and reused by every run."""
+
+    def __init__(self, w, w_scale, w_zero_point, b=None, strides=(), pads=(), group=1, auto_pad=""):
+        self._keep = (w, w_scale, w_zero_point, b)
+        self.w, self.strides, self.pads, self.group, self.auto_pad = w, strides, pads, group, auto_pad
+        self._plans = {}
+
+    def _plan_for(self, x):
+        params, shape = _conv_setup(x, self.w, self.strides, self.pads, self.group, self.auto_pad)
+        key = tuple(getattr(params, f) for f, _ in params._fields_)
+        if key not in self._plans:
+            handle = ctypes.c_void_p()
+            w, w_scale, w_zero_point, b = self._keep
+            capi.check(capi.lib().chx_hip_qconv_plan_create(
+                capi.ref(w), capi.ref(w_scale), capi.ref(w_zero_point), capi.ref(b), ctypes.byref(params),
+                capi.stream_ptr(), ctypes.byref(handle)))
+            self._plans[key] = handle
+        return self._plans[key], shape
+
+    def run(self, x, x_scale, x_zero_point, y_scale, y_zero_point, zero_point_dtype=torch.uint8, flags=0, out=None):
+        handle, shape = self._plan_for(x)
+        if out is None:
+            out = _alloc_like_input_layout(x, shape, zero_point_dtype)
+        capi.check(capi.lib().chx_hip_qconv_plan_run(
+            handle, capi.ref(x), _f(x_scale), _i(x_zero_point), _f(y_scale), _i(y_zero_point),
+            ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
+        return out
+
+    def close(self):
+        for handle in self._plans.values():
+            capi.lib().chx_hip_qconv_plan_destroy(handle)
+        self._plans = {}
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
