@@ -1,0 +1,299 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|conv3x3|fusion|qdq]
+
+Default workload: ResNet-50 v1 int8 QDQ inference, batch 64, 224x224 (the configuration the
+headline metric is quoted on).  One step = one pass of the whole op program over one batch
+that is already resident in HBM (fp32 NCHW input; QuantizeLinear is part of the step).
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the int8 MFMA implicit-GEMM
+convolution for resnet50 / conv3x3, the fused element-wise kernel for fusion / qdq), timed
+live with events on the launch stream inside the timed region.  `cpu_baseline` times the
+restated reference CPU op sequence (the oracle's literal fp32 path) on the host cores for a
+bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8, published
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "conv3x3", "fusion", "qdq"])
+    ap.add_argument("--batch", type=int, default=0, help="override the batch size (changes the workload; for experiments)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline")
+    return ap.parse_args()
+
+
+def timed_steps(torch, step, steps, warmup, instrument=None):
+    """W untimed steps, then exactly K timed steps between two synchronizations."""
+    for _ in range(warmup):
+        step(None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(instrument)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+class KernelTimer(object):
+    """Event pairs around chosen launches on the current (launch) stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = []
+
+    def wrap(self, tag, fn):
+        a = self.torch.cuda.Event(enable_timing=True)
+        b = self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        r = fn()
+        b.record()
+        self.pairs.append((tag, a, b))
+        return r
+
+    def totals(self):
+        out = {}
+        for tag, a, b in self.pairs:
+            ms = a.elapsed_time(b)
+            cnt, tot = out.get(tag, (0, 0.0))
+            out[tag] = (cnt + 1, tot + ms)
+        return out
+
+
+def cpu_info():
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return model, os.cpu_count() or 1
+
+
+# ------------------------------------------------------------------------------------------------
+
+def bench_resnet50(args, torch, pkg):
+    wl = pkg.workloads
+    batch = args.batch or 64
+    model = wl.build_resnet50(batch=batch, seed=3)
+    runner = wl.DeviceRunner(model, pkg)
+    x = torch.from_numpy(model["input"]).cuda()
+    ops, capi = pkg.ops, pkg.capi
+    conv_ops = 2.0 * model["macs"]
+
+    def step(timer):
+        if timer is None:
+            runner.run(x)
+            return
+        # same program, with event pairs around every QLinearConv launch
+        q, m = model["qparams"], model
+        v = {"x": x}
+        for fid, ins in enumerate(m["program"]):
+            kind, out = ins[0], ins[1]
+            buf = runner.bufs[out]
+            if kind == "QLinearConv":
+                c = m["convs"][ins[3]]
+                timer.wrap("conv", lambda: runner.plans[ins[3]].run(
+                    v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8, flags=capi.BIAS_ONNX_INT32, out=buf))
+            elif kind == "QuantizeLinear":
+                ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
+            elif kind == "MaxPool":
+                ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
+            elif kind == "AddRelu":
+                ops.ElementWiseNvrtc([v[ins[2]], v[ins[3]]], 1, runner.fusion[out], fid, outs=[buf])
+            elif kind == "AveragePool":
+                ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
+                                  q[out][1], out=buf)
+            elif kind == "DequantizeLinear":
+                ops.DequantizeLinear(v[ins[2]], ins[3], ins[4], out=buf)
+            v[out] = buf
+
+    timer = KernelTimer(torch)
+    sec = timed_steps(torch, step, args.steps, args.warmup, timer)
+    tot = timer.totals()["conv"]
+    n_launch = tot[0] / args.steps
+    conv_ms_per_step = tot[1] / args.steps
+    achieved = conv_ops / (conv_ms_per_step * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % round(n_launch),
+                    achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
+                    ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
+    res = dict(metric="images/sec ResNet-50 int8 bs64 @1 GPU", value=batch / sec, unit="images/sec",
+               ms_per_step=sec * 1e3, dtype="int8",
+               config=dict(workload="resnet50_v1_int8_qdq", batch=batch, image=224, layout="channels_last",
+                           conv_gmac_per_image=model["macs"] / batch / 1e9))
+
+    def cpu():
+        from oracle import oracle as orc
+        lit = _literal_executor(orc)
+        small = wl.build_resnet50(batch=1, seed=3)
+        cores = orc.max_threads()
+        orc.set_threads(cores)
+        t0 = time.perf_counter()
+        wl.run_reference(small, lit, small["input"])
+        dt = time.perf_counter() - t0
+        orc.set_threads(1)
+        return dict(value=1.0 / dt, unit="images/sec", cores=cores, kind="port",
+                    sample="1 image (batch 1 of the same network), restated reference op sequence: fp32 dequantize, "
+                           "im2col + sequential-k GEMM, multi-pass quantize; OpenMP over %d threads; %.1f s" % (cores, dt))
+    runner_close = runner.close
+    return res, roofline, cpu, runner_close
+
+
+def _literal_executor(orc):
+    """The oracle with QLinearConv routed to the literal fp32 restatement of the reference."""
+    class Lit(object):
+        def __getattr__(self, name):
+            return getattr(orc, name)
+
+        def qlinear_conv_int(self, *a, **k):
+            return orc.qlinear_conv_literal(*a, **k)
+    return Lit()
+
+
+def bench_conv3x3(args, torch, pkg):
+    import numpy as np
+    ops, capi = pkg.ops, pkg.capi
+    n = args.batch or 32
+    rng = np.random.default_rng(2)
+    x = rng.integers(0, 256, size=(n, 128, 28, 28)).astype(np.uint8)
+    w = rng.integers(-127, 128, size=(128, 128, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, size=128).astype(np.float32)
+    wz = np.zeros(128, np.int8)
+    bias = rng.integers(-1000, 1001, size=128).astype(np.int32)
+    xd = torch.from_numpy(x).cuda().permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)
+    plan = ops.QLinearConvPlan(*[torch.from_numpy(a).cuda() for a in (w, ws, wz, bias)], pads=(1, 1))
+    y = plan.run(xd, 0.02, 128, 0.05, 128, flags=capi.BIAS_ONNX_INT32)
+    mac = n * 28 * 28 * 128 * 128 * 9
+
+    def step(timer):
+        fn = lambda: plan.run(xd, 0.02, 128, 0.05, 128, flags=capi.BIAS_ONNX_INT32, out=y)
+        timer.wrap("conv", fn) if timer else fn()
+
+    timer = KernelTimer(torch)
+    sec = timed_steps(torch, step, args.steps, args.warmup, timer)
+    cnt, ms = timer.totals()["conv"]
+    achieved = 2.0 * mac / (ms / cnt * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel="conv_mfma_kernel", achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s",
+                    frac=achieved / INT8_PEAK_TOPS, traffic=None, ops_per_launch=2.0 * mac, launch_us=ms / cnt * 1e3)
+    res = dict(metric="images/sec QLinearConv 3x3 128->128 @28x28 (ResNet-50 stage 3), 1 GPU", value=n / sec,
+               unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
+               config=dict(workload="qlinearconv_3x3_c128_28x28", batch=n, layout="channels_last"))
+
+    def cpu():
+        from oracle import oracle as orc
+        cores = orc.max_threads()
+        orc.set_threads(cores)
+        k = 4
+        t0 = time.perf_counter()
+        orc.qlinear_conv_literal(x[:k], 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1),
+                                 bias_mode=orc.BIAS_ONNX_INT32)
+        dt = time.perf_counter() - t0
+        orc.set_threads(1)
+        return dict(value=k / dt, unit="images/sec", cores=cores, kind="port",
+                    sample="%d of %d images, literal fp32 restatement of QLinearConvOp, %d threads, %.2f s" % (k, n, cores, dt))
+    return res, roofline, cpu, plan.close
+
+
+def bench_fusion(args, torch, pkg, qdq=False):
+    import numpy as np
+    ops = pkg.ops
+    f32 = torch.float32
+    torch.manual_seed(1)
+    x = torch.randn(64, 1024, 1024, device="cuda")
+    y = torch.empty_like(x)
+    if qdq:
+        prog = ops.fusion_program([("x", f32)], [("q", "QuantizeLinear", "x", 0.05, 0, "int8"),
+                                                  ("y", "DequantizeLinear", "q", 0.05, 0)], [("y", f32)])
+        ins, nbytes, name = [x], 2 * x.numel() * 4, "quantize_dequantize_fused"
+    else:
+        c = torch.randn_like(x)
+        a = torch.randn(1024, device="cuda")
+        b = torch.randn(1024, device="cuda")
+        prog = ops.fusion_program(
+            [("x", f32), ("a", f32), ("b", f32), ("c", f32)],
+            [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+             ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")], [("y", f32)])
+        ins, nbytes, name = [x, a, b, c], 3 * x.numel() * 4 + 2 * 1024 * 4, "relu(tanh(x*a+b)*sigmoid(c)+x)"
+
+    def step(timer):
+        fn = lambda: ops.ElementWiseNvrtc(ins, 1, prog, 3, outs=[y])
+        timer.wrap("ew", fn) if timer else fn()
+
+    timer = KernelTimer(torch)
+    sec = timed_steps(torch, step, args.steps, args.warmup, timer)
+    cnt, ms = timer.totals()["ew"]
+    achieved = nbytes / (ms / cnt * 1e-3) / 1e9
+    roofline = dict(bound="hbm", kernel="fusion3_vec", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=achieved / HBM_PEAK_GBS, traffic=None, bytes_per_launch=nbytes, launch_us=ms / cnt * 1e3)
+    res = dict(metric="GB/s FusionGroup %s fp32 [64,1024,1024] @1 GPU" % name, value=nbytes / sec / 1e9, unit="GB/s",
+               ms_per_step=sec * 1e3, dtype="f32", config=dict(workload="fusion_" + ("qdq" if qdq else "chain"), elements=x.numel()))
+
+    def cpu():
+        from oracle import oracle as orc
+        cores = orc.max_threads()
+        orc.set_threads(cores)
+        rows = 2 * 1024
+        xs = x.view(-1, 1024)[:rows].cpu().numpy()
+        t0 = time.perf_counter()
+        if qdq:
+            orc.dequantize_linear(orc.quantize_linear_multipass(xs, 0.05, 0, np.int8), 0.05, 0, multipass=True)
+        else:
+            cs = ins[3].view(-1, 1024)[:rows].cpu().numpy()
+            orc.run_chain([("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"),
+                           ("t3", "Sigmoid", "c"), ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"),
+                           ("y", "Relu", "t5")], dict(x=xs, a=ins[1].cpu().numpy(), b=ins[2].cpu().numpy(), c=cs))
+        dt = time.perf_counter() - t0
+        orc.set_threads(1)
+        frac = rows * 1024 / x.numel()
+        return dict(value=nbytes * frac / dt / 1e9, unit="GB/s", cores=cores, kind="port",
+                    sample="%d of %d rows, op-by-op fp32 passes with temporaries, %d threads, %.2f s" % (
+                        rows, x.numel() // 1024, cores, dt))
+    return res, roofline, cpu, (lambda: None)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; this path has no multi-GPU leg (inference is data parallel over the "
+              "batch and every GPU box here has one GPU).  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    pkg.capi.init(0)
+    if args.workload == "resnet50":
+        res, roofline, cpu, close = bench_resnet50(args, torch, pkg)
+    elif args.workload == "conv3x3":
+        res, roofline, cpu, close = bench_conv3x3(args, torch, pkg)
+    else:
+        res, roofline, cpu, close = bench_fusion(args, torch, pkg, qdq=args.workload == "qdq")
+    out = dict(res)
+    out.update(n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak", vs_baseline=None,
+               data="synthetic", roofline=roofline)
+    if not args.no_cpu_baseline:
+        model, ncpu = cpu_info()
+        cb = cpu()
+        cb["host"] = "%s, %d logical CPUs visible" % (model, ncpu)
+        out["cpu_baseline"] = cb
+    close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

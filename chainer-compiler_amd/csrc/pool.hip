@@ -1,0 +1,214 @@
+// Pooling on 8-bit quantized tensors, for running whole quantized networks without
+// leaving the 8-bit domain.  In a ChxVM program these appear as
+//   DequantizeLinear -> MaxPool / AveragePool (runtime/ops/pooling.cc:47-75) -> QuantizeLinear;
+// the hip backend lowers each such triple to one of these kernels.
+//   max:     with the same scale and zero point on both sides the triple equals the
+//            maximum of the codes (dequantization is increasing, Q(DQ(q)) == q).
+//   average: y = Q( (sum of DQ(x) over the window, fp32, in (kh, kw) order) / count ).
+// Both are bandwidth-bound; channels-last tensors move 16 channels per lane.
+#include <cstring>
+
+#include "chx_internal.h"
+#include "quant_math.h"
+
+namespace chx {
+namespace {
+
+constexpr int kThreads = 256;
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+struct PoolArgs {
+    const char* x;
+    char* y;
+    int64_t xs[4], ys[4];  // byte strides of N, C, H, W
+    int32_t N, C, H, W, OH, OW, kh, kw, sh, sw, ph, pw;
+    int32_t is_signed;
+    int64_t total;
+};
+
+__device__ __forceinline__ uint32_t max4_u8(uint32_t a, uint32_t b) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t x = (a >> (8 * i)) & 0xffu, y = (b >> (8 * i)) & 0xffu;
+        r |= (x > y ? x : y) << (8 * i);
+    }
+    return r;
+}
+
+// channels-last, C % 16 == 0: one lane = 16 channels of one output pixel.  int8 codes are
+// compared as unsigned after flipping the sign bit.
+__global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= a.total) return;
+    const int cgroups = a.C / 16;
+    const int cg = (int)(idx % cgroups);
+    int64_t r = idx / cgroups;
+    const int ow = (int)(r % a.OW);
+    r /= a.OW;
+    const int oh = (int)(r % a.OH);
+    const int n = (int)(r / a.OH);
+    const uint32_t flip = a.is_signed ? 0x80808080u : 0u;
+    v4u m = {0, 0, 0, 0};
+    for (int i = 0; i < a.kh; ++i) {
+        const int ih = oh * a.sh - a.ph + i;
+        if ((unsigned)ih >= (unsigned)a.H) continue;
+        for (int j = 0; j < a.kw; ++j) {
+            const int iw = ow * a.sw - a.pw + j;
+            if ((unsigned)iw >= (unsigned)a.W) continue;
+            v4u v = *reinterpret_cast<const v4u*>(a.x + n * a.xs[0] + ih * a.xs[2] + iw * a.xs[3] + cg * 16);
+            m[0] = max4_u8(m[0], v[0] ^ flip);
+            m[1] = max4_u8(m[1], v[1] ^ flip);
+            m[2] = max4_u8(m[2], v[2] ^ flip);
+            m[3] = max4_u8(m[3], v[3] ^ flip);
+        }
+    }
+    m[0] ^= flip; m[1] ^= flip; m[2] ^= flip; m[3] ^= flip;
+    *reinterpret_cast<v4u*>(a.y + n * a.ys[0] + oh * a.ys[2] + ow * a.ys[3] + cg * 16) = m;
+}
+
+// any strides: one lane = one output element, channel index fastest
+__global__ __launch_bounds__(kThreads) void max_pool_generic_kernel(PoolArgs a) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= a.total) return;
+    const int c = (int)(idx % a.C);
+    int64_t r = idx / a.C;
+    const int ow = (int)(r % a.OW);
+    r /= a.OW;
+    const int oh = (int)(r % a.OH);
+    const int n = (int)(r / a.OH);
+    int32_t m = -1000;
+    for (int i = 0; i < a.kh; ++i) {
+        const int ih = oh * a.sh - a.ph + i;
+        if ((unsigned)ih >= (unsigned)a.H) continue;
+        for (int j = 0; j < a.kw; ++j) {
+            const int iw = ow * a.sw - a.pw + j;
+            if ((unsigned)iw >= (unsigned)a.W) continue;
+            const uint8_t raw = *reinterpret_cast<const uint8_t*>(a.x + n * a.xs[0] + c * a.xs[1] + ih * a.xs[2] + iw * a.xs[3]);
+            const int32_t v = a.is_signed ? (int32_t)(int8_t)raw : (int32_t)raw;
+            m = v > m ? v : m;
+        }
+    }
+    *reinterpret_cast<uint8_t*>(a.y + n * a.ys[0] + c * a.ys[1] + oh * a.ys[2] + ow * a.ys[3]) = (uint8_t)m;
+}
+
+struct AvgArgs {
+    PoolArgs p;
+    float x_scale, x_zpf;
+    int32_t count_include_pad;
+    QuantParams q;
+};
+
+template <bool kRne>
+__global__ __launch_bounds__(kThreads) void average_pool_kernel(AvgArgs a) {
+    const PoolArgs& p = a.p;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= p.total) return;
+    const int c = (int)(idx % p.C);
+    int64_t r = idx / p.C;
+    const int ow = (int)(r % p.OW);
+    r /= p.OW;
+    const int oh = (int)(r % p.OH);
+    const int n = (int)(r / p.OH);
+    float sum = 0.f;
+    int32_t cnt = 0;
+    for (int i = 0; i < p.kh; ++i) {
+        const int ih = oh * p.sh - p.ph + i;
+        if ((unsigned)ih >= (unsigned)p.H) continue;
+        for (int j = 0; j < p.kw; ++j) {
+            const int iw = ow * p.sw - p.pw + j;
+            if ((unsigned)iw >= (unsigned)p.W) continue;
+            const uint8_t raw = *reinterpret_cast<const uint8_t*>(p.x + n * p.xs[0] + c * p.xs[1] + ih * p.xs[2] + iw * p.xs[3]);
+            const int32_t v = p.is_signed ? (int32_t)(int8_t)raw : (int32_t)raw;
+            sum = sum + dequantize_value(v, a.x_zpf, a.x_scale);
+            ++cnt;
+        }
+    }
+    if (a.count_include_pad) cnt = p.kh * p.kw;
+    const float mean = sum / (float)cnt;
+    *reinterpret_cast<uint8_t*>(p.y + n * p.ys[0] + c * p.ys[1] + oh * p.ys[2] + ow * p.ys[3]) =
+            (uint8_t)quantize_value<kRne>(mean, a.q);
+}
+
+int fill_pool_args(
+        const chx_hip_tensor* x, chx_hip_tensor* y, int kh, int kw, int sh, int sw, int ph0, int pw0, int ph1, int pw1,
+        int cover_all, const char* op, PoolArgs* a) {
+    CHX_PROPAGATE(check_tensor(x, op));
+    CHX_PROPAGATE(check_tensor(y, op));
+    CHX_REQUIRE(x->ndim == 4 && y->ndim == 4, "%s: x and y must be 4-D", op);
+    CHX_REQUIRE(is_q8(x->dtype) && is_q8(y->dtype), "%s: x and y must be uint8 or int8", op);
+    CHX_REQUIRE(kh >= 1 && kw >= 1 && sh >= 1 && sw >= 1 && ph0 >= 0 && pw0 >= 0 && ph1 >= 0 && pw1 >= 0,
+                "%s: bad kernel, stride or padding", op);
+    const int64_t H = x->shape[2], W = x->shape[3];
+    CHX_REQUIRE(H + ph0 + ph1 >= kh && W + pw0 + pw1 >= kw, "%s: kernel larger than the padded input", op);
+    const int64_t OH = cover_all ? (H + ph0 + ph1 - kh + sh - 1) / sh + 1 : (H + ph0 + ph1 - kh) / sh + 1;
+    const int64_t OW = cover_all ? (W + pw0 + pw1 - kw + sw - 1) / sw + 1 : (W + pw0 + pw1 - kw) / sw + 1;
+    CHX_REQUIRE(y->shape[0] == x->shape[0] && y->shape[1] == x->shape[1] && y->shape[2] == OH && y->shape[3] == OW,
+                "%s: y is [%lld,%lld,%lld,%lld], expected [%lld,%lld,%lld,%lld]", op, (long long)y->shape[0],
+                (long long)y->shape[1], (long long)y->shape[2], (long long)y->shape[3], (long long)x->shape[0],
+                (long long)x->shape[1], (long long)OH, (long long)OW);
+    memset(a, 0, sizeof(*a));
+    a->x = static_cast<const char*>(x->data);
+    a->y = static_cast<char*>(y->data);
+    for (int i = 0; i < 4; ++i) {
+        a->xs[i] = x->strides[i];
+        a->ys[i] = y->strides[i];
+    }
+    a->N = (int32_t)x->shape[0]; a->C = (int32_t)x->shape[1]; a->H = (int32_t)H; a->W = (int32_t)W;
+    a->OH = (int32_t)OH; a->OW = (int32_t)OW;
+    a->kh = kh; a->kw = kw; a->sh = sh; a->sw = sw; a->ph = ph0; a->pw = pw0;
+    a->is_signed = x->dtype == CHX_HIP_INT8;
+    a->total = (int64_t)a->N * a->C * OH * OW;
+    return CHX_HIP_OK;
+}
+
+}  // namespace
+}  // namespace chx
+
+using namespace chx;
+
+extern "C" int chx_hip_max_pool_q8(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+        int32_t pad_h_begin, int32_t pad_w_begin, int32_t pad_h_end, int32_t pad_w_end, int32_t cover_all,
+        chx_hip_tensor* y, void* stream) {
+    PoolArgs a;
+    CHX_PROPAGATE(fill_pool_args(x, y, kernel_h, kernel_w, stride_h, stride_w, pad_h_begin, pad_w_begin, pad_h_end,
+                                 pad_w_end, cover_all, "MaxPool", &a));
+    CHX_REQUIRE(x->dtype == y->dtype, "MaxPool: x and y must have the same dtype");
+    if (a.total == 0) return CHX_HIP_OK;
+    hipStream_t s = as_stream(stream);
+    int64_t px, py;
+    const bool cl16 = a.C % 16 == 0 && is_channels_last(*x, &px) && is_channels_last(*y, &py) && aligned(x->data, 16) &&
+                      aligned(y->data, 16) && px % 16 == 0 && py % 16 == 0;
+    if (cl16) {
+        a.total = (int64_t)a.N * a.OH * a.OW * (a.C / 16);
+        max_pool_cl16_kernel<<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
+        return launch_check("max_pool_cl16_kernel");
+    }
+    max_pool_generic_kernel<<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
+    return launch_check("max_pool_generic_kernel");
+}
+
+extern "C" int chx_hip_average_pool_q8(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, int32_t kernel_h, int32_t kernel_w,
+        int32_t stride_h, int32_t stride_w, int32_t pad_h, int32_t pad_w, int32_t count_include_pad, float y_scale,
+        int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream) {
+    AvgArgs a;
+    CHX_PROPAGATE(fill_pool_args(x, y, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, 0,
+                                 "AveragePool", &a.p));
+    const bool i8 = y->dtype == CHX_HIP_INT8;
+    CHX_REQUIRE(y_zero_point >= (i8 ? -128 : 0) && y_zero_point <= (i8 ? 127 : 255),
+                "AveragePool: zero point %d outside the range of %s", y_zero_point, dtype_name(y->dtype));
+    if (a.p.total == 0) return CHX_HIP_OK;
+    a.x_scale = x_scale;
+    a.x_zpf = (float)x_zero_point;
+    a.count_include_pad = count_include_pad;
+    a.q = make_quant_params(y_scale, y_zero_point, i8);
+    hipStream_t s = as_stream(stream);
+    const unsigned blocks = (unsigned)((a.p.total + kThreads - 1) / kThreads);
+    if (flags & CHX_HIP_ROUND_ONNX_RNE)
+        average_pool_kernel<true><<<blocks, kThreads, 0, s>>>(a);
+    else
+        average_pool_kernel<false><<<blocks, kThreads, 0, s>>>(a);
+    return launch_check("average_pool_kernel");
+}

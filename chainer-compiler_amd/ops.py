@@ -227,3 +227,40 @@ class QLinearConvPlan(object):
             self.close()
         except Exception:
             pass
+
+
+def _pool_out(in_dim, p0, p1, k, s, cover_all):
+    if cover_all:
+        return (in_dim + p0 + p1 - k + s - 1) // s + 1
+    return (in_dim + p0 + p1 - k) // s + 1
+
+
+def MaxPoolQ8(x, kernel_shape, strides=(), pads=(), cover_all=False, out=None):
+    """DequantizeLinear -> MaxPool (runtime/ops/pooling.cc:47-61) -> QuantizeLinear with equal
+    quantization parameters, on the 8-bit codes."""
+    strides = _complement(strides, 2, 1)
+    pads = _complement(pads, 2, 0)
+    if out is None:
+        shape = (x.shape[0], x.shape[1], _pool_out(x.shape[2], pads[0], pads[0], kernel_shape[0], strides[0], cover_all),
+                 _pool_out(x.shape[3], pads[1], pads[1], kernel_shape[1], strides[1], cover_all))
+        out = _alloc_like_input_layout(x, shape, x.dtype)
+    capi.check(capi.lib().chx_hip_max_pool_q8(
+        capi.ref(x), _i(kernel_shape[0]), _i(kernel_shape[1]), _i(strides[0]), _i(strides[1]), _i(pads[0]), _i(pads[1]),
+        _i(pads[0]), _i(pads[1]), _i(1 if cover_all else 0), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
+def AveragePoolQ8(x, x_scale, x_zero_point, kernel_shape, strides, pads, y_scale, y_zero_point,
+                  count_include_pad=False, zero_point_dtype=torch.uint8, flags=0, out=None):
+    """DequantizeLinear -> AveragePool (runtime/ops/pooling.cc:63-75) -> QuantizeLinear."""
+    strides = _complement(strides, 2, 1)
+    pads = _complement(pads, 2, 0)
+    if out is None:
+        shape = (x.shape[0], x.shape[1], _pool_out(x.shape[2], pads[0], pads[0], kernel_shape[0], strides[0], False),
+                 _pool_out(x.shape[3], pads[1], pads[1], kernel_shape[1], strides[1], False))
+        out = _alloc_like_input_layout(x, shape, zero_point_dtype)
+    capi.check(capi.lib().chx_hip_average_pool_q8(
+        capi.ref(x), _f(x_scale), _i(x_zero_point), _i(kernel_shape[0]), _i(kernel_shape[1]), _i(strides[0]),
+        _i(strides[1]), _i(pads[0]), _i(pads[1]), _i(1 if count_include_pad else 0), _f(y_scale), _i(y_zero_point),
+        ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
+    return out

@@ -1,0 +1,280 @@
+"""Quantized networks as hand-built ChxVM-style programs: the ResNet-50 int8 QDQ
+configuration the headline metric is quoted on, in the op vocabulary of this path.
+
+A program is a list of instructions over named values; every instruction is one op
+of the path (QuantizeLinear, QLinearConv, MaxPool, FusionGroup Add+Relu, AveragePool,
+DequantizeLinear).  `build_resnet50` only constructs data (weights, scales, the
+instruction list); executing it is the job of `DeviceRunner` (MI355X, through the C
+ABI) or of a reference executor supplied by the tests and the benchmark.
+
+Construction follows the reference where it defines the step:
+  architecture            scripts/resnet50.py:10-107 (stride on the first 1x1 of a
+                          down-sampling bottleneck, 7x7/2 stem with bias, 3x3/2
+                          max-pool with cover_all, 7x7 average pool, FC 2048->1000)
+  BatchNorm folding       compiler/merge.cc:142-211: s = gamma / sqrt(var + eps),
+                          w' = w * s, b' = (b - mean) * s + beta
+  weight quantization     compiler/quantize.cc:77-81, per output channel:
+                          scale = 2 max|w| / 254, q = rint(w / scale), zero point 0
+  activation quantization compiler/quantize.cc:84-86 on the min/max of one seeded
+                          batch: scale = (max - min) / 255 with min <= 0 <= max,
+                          zero_point = rint(-min / scale), uint8
+Bias is int32 at scale x_scale * w_scale[oc] (the ONNX QLinearConv definition).
+A Relu after a convolution is folded into the convolution's output quantization:
+the calibrated post-Relu range starts at 0, so the zero point is 0 and the uint8
+saturation of QLinearConv is the Relu (Q(Relu(DQ(q))) == q for every code).
+"""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+EPS = 2e-5  # chainer.links.BatchNormalization default
+
+
+def _he_normal(rng, shape):
+    fan_in = int(np.prod(shape[1:]))
+    return (rng.standard_normal(shape) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+
+
+def _fold_bn(rng, w, b):
+    oc = w.shape[0]
+    gamma = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    beta = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    mean = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    s = (gamma / np.sqrt(var + np.float32(EPS))).astype(np.float32)
+    w2 = (w * s[:, None, None, None]).astype(np.float32)
+    b0 = np.zeros(oc, np.float32) if b is None else b
+    b2 = ((b0 - mean) * s + beta).astype(np.float32)
+    return w2, b2
+
+
+def quantize_weights_per_channel(w):
+    """compiler/quantize.cc:77-81 applied per output channel (QuantizeWeightConvolution)."""
+    oc = w.shape[0]
+    flat = w.reshape(oc, -1)
+    rmin = np.minimum(flat.min(axis=1), 0).astype(np.float32)
+    rmax = np.maximum(flat.max(axis=1), 0).astype(np.float32)
+    max_range = np.maximum(np.abs(rmin), np.abs(rmax)).astype(np.float32)
+    scale = (max_range * np.float32(2) / np.float32(254)).astype(np.float32)
+    scale = np.where(scale == 0, np.float32(1), scale).astype(np.float32)
+    q = np.rint(w / scale[:, None, None, None]).astype(np.int8)
+    return q, scale
+
+
+def activation_qparams(t):
+    """compiler/quantize.cc:84-86: uint8, range widened to contain 0."""
+    rmin = min(float(t.min()), 0.0)
+    rmax = max(float(t.max()), 0.0)
+    scale = np.float32((np.float32(rmax) - np.float32(rmin)) / np.float32(255)) if rmin != rmax else np.float32(1)
+    zp = int(np.rint((0 - np.float32(rmin)) / scale))
+    return scale, zp
+
+
+class ConvLayer(object):
+    def __init__(self, name, w, b, stride, pad):
+        self.name, self.wf, self.bf, self.stride, self.pad = name, w, b, stride, pad
+        self.wq, self.w_scale = quantize_weights_per_channel(w)
+        self.w_zp = np.zeros(w.shape[0], np.int8)
+        self.x_scale = self.x_zp = self.y_scale = self.y_zp = None
+        self.bias_q = None
+
+    def finish(self):
+        s = (np.float32(self.x_scale) * self.w_scale).astype(np.float32)
+        self.bias_q = np.rint(self.bf / s).astype(np.int64).clip(-2 ** 31, 2 ** 31 - 1).astype(np.int32)
+
+    def macs(self, out_shape):
+        n, oc, oh, ow = out_shape
+        return n * oh * ow * oc * int(np.prod(self.wf.shape[1:]))
+
+
+def build_resnet50(batch=64, image=224, seed=3, width=64, blocks=(3, 4, 6, 3), classes=1000, device=None):
+    """Returns a dict: program (instruction list), convs (name -> ConvLayer), qparams
+    (value name -> (scale, zero_point)), input (the seeded fp32 batch), shapes, macs.
+
+    `width`, `blocks`, `image`, `classes` shrink the network for tests; the defaults are
+    ResNet-50 v1."""
+    rng = np.random.default_rng(seed)
+    dev = device or ("cuda" if torch.cuda.is_available() else "cpu")
+    x = rng.standard_normal((batch, 3, image, image)).astype(np.float32)
+    program, convs, qparams, shapes = [], {}, {}, {}
+    fvals = {"x": torch.from_numpy(x).to(dev)}
+
+    def note(name):
+        qparams[name] = activation_qparams(fvals[name])
+        shapes[name] = tuple(fvals[name].shape)
+
+    def conv(name, src, dst, cin, cout, k, stride, pad, relu, bias=False):
+        w = _he_normal(rng, (cout, cin, k, k))
+        b = (rng.standard_normal(cout) * 0.1).astype(np.float32) if bias else None
+        w, b = _fold_bn(rng, w, b)
+        layer = ConvLayer(name, w, b, stride, pad)
+        convs[name] = layer
+        # calibration runs the float network with the weights the quantized one represents
+        wd = torch.from_numpy(layer.wq.astype(np.float32) * layer.w_scale[:, None, None, None]).to(dev)
+        y = F.conv2d(fvals[src], wd, torch.from_numpy(b).to(dev), stride=stride, padding=pad)
+        fvals[dst] = F.relu(y) if relu else y
+        note(dst)
+        layer.x_scale, layer.x_zp = qparams[src]
+        layer.y_scale, layer.y_zp = qparams[dst]
+        layer.finish()
+        program.append(("QLinearConv", dst, src, name))
+
+    note("x")
+    program.append(("QuantizeLinear", "x_q", "x") + qparams["x"])
+    fvals["x_q"] = fvals["x"]
+    qparams["x_q"], shapes["x_q"] = qparams["x"], shapes["x"]
+    conv("conv1", "x_q", "stem", 3, width, 7, 2, 3, relu=True, bias=True)
+    fvals["pool1"] = F.max_pool2d(fvals["stem"], 3, 2, 0, ceil_mode=True)
+    qparams["pool1"], shapes["pool1"] = qparams["stem"], tuple(fvals["pool1"].shape)
+    program.append(("MaxPool", "pool1", "stem", 3, 2, 0, True))
+
+    cur, cin = "pool1", width
+    for si, nblk in enumerate(blocks):
+        ch = width * (2 ** si)
+        cout = ch * 4
+        for bi in range(nblk):
+            p = "res%d_%d" % (si + 2, bi)
+            stride = 2 if (bi == 0 and si > 0) else 1
+            conv(p + "_c1", cur, p + "_a", cin, ch, 1, stride, 0, relu=True)
+            conv(p + "_c2", p + "_a", p + "_b", ch, ch, 3, 1, 1, relu=True)
+            conv(p + "_c3", p + "_b", p + "_c", ch, cout, 1, 1, 0, relu=False)
+            if bi == 0:
+                conv(p + "_c4", cur, p + "_s", cin, cout, 1, stride, 0, relu=False)
+                short = p + "_s"
+            else:
+                short = cur
+            fvals[p] = F.relu(fvals[p + "_c"] + fvals[short])
+            note(p)
+            program.append(("AddRelu", p, p + "_c", short))
+            for tmp in (p + "_a", p + "_b", p + "_c", p + "_s", cur):
+                fvals.pop(tmp, None)   # calibration activations no longer needed
+            cur, cin = p, cout
+    k = fvals[cur].shape[2]
+    fvals["gap"] = F.avg_pool2d(fvals[cur], k, 1)
+    note("gap")
+    program.append(("AveragePool", "gap", cur, int(k)))
+    conv("fc", "gap", "logits_q", cin, classes, 1, 1, 0, relu=False, bias=True)
+    program.append(("DequantizeLinear", "logits", "logits_q") + qparams["logits_q"])
+    shapes["logits"] = shapes["logits_q"]
+    total_macs = 0
+    for ins in program:
+        if ins[0] == "QLinearConv":
+            total_macs += convs[ins[3]].macs(shapes[ins[1]])
+    return dict(program=program, convs=convs, qparams=qparams, shapes=shapes, input=x, macs=total_macs,
+                float_logits=fvals["logits_q"].detach().cpu().numpy())
+
+
+def add_relu_program(ops, qa, qb, qy):
+    """FusionGroup text for Q(Relu(DQ(a) + DQ(b))) on uint8 tensors."""
+    u8 = torch.uint8
+    return ops.fusion_program(
+        [("a", u8), ("b", u8)],
+        [("fa", "DequantizeLinear", "a", "0x%08x" % np.float32(qa[0]).view(np.uint32), qa[1]),
+         ("fb", "DequantizeLinear", "b", "0x%08x" % np.float32(qb[0]).view(np.uint32), qb[1]),
+         ("s", "Add", "fa", "fb"), ("r", "Relu", "s"),
+         ("q", "QuantizeLinear", "r", "0x%08x" % np.float32(qy[0]).view(np.uint32), qy[1], "uint8")],
+        [("q", u8)])
+
+
+class DeviceRunner(object):
+    """Runs a program on the MI355X: weights resident, one plan per QLinearConv, every
+    activation channels-last, all intermediate buffers allocated once."""
+
+    def __init__(self, model, pkg):
+        self.m, self.ops, self.capi = model, pkg.ops, pkg.capi
+        self.dev = {}
+        self.plans = {}
+        self.bufs = {}
+        self.fusion = {}
+        for name, c in model["convs"].items():
+            t = [torch.from_numpy(a).cuda() for a in (c.wq, c.w_scale, c.w_zp, c.bias_q)]
+            self.dev[name] = t
+            self.plans[name] = self.ops.QLinearConvPlan(t[0], t[1], t[2], t[3], strides=(c.stride, c.stride),
+                                                        pads=(c.pad, c.pad))
+        for ins in model["program"]:
+            out = ins[1]
+            shp = model["shapes"][out]
+            if ins[0] == "DequantizeLinear":
+                self.bufs[out] = torch.empty(shp, dtype=torch.float32, device="cuda")
+            else:
+                n, c, h, w = shp
+                self.bufs[out] = torch.empty((n, h, w, c), dtype=torch.uint8, device="cuda").permute(0, 3, 1, 2)
+            if ins[0] == "AddRelu":
+                q = model["qparams"]
+                self.fusion[out] = add_relu_program(self.ops, q[ins[2]], q[ins[3]], q[out])
+
+    def run(self, x):
+        ops, q, m = self.ops, self.m["qparams"], self.m
+        v = {"x": x}
+        for fid, ins in enumerate(m["program"]):
+            kind, out = ins[0], ins[1]
+            buf = self.bufs[out]
+            if kind == "QuantizeLinear":
+                ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
+            elif kind == "QLinearConv":
+                c = m["convs"][ins[3]]
+                self.plans[ins[3]].run(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
+                                       flags=self.capi.BIAS_ONNX_INT32, out=buf)
+            elif kind == "MaxPool":
+                ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
+            elif kind == "AddRelu":
+                ops.ElementWiseNvrtc([v[ins[2]], v[ins[3]]], 1, self.fusion[out], fid, outs=[buf])
+            elif kind == "AveragePool":
+                ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
+                                  q[out][1], out=buf)
+            elif kind == "DequantizeLinear":
+                ops.DequantizeLinear(v[ins[2]], ins[3], ins[4], out=buf)
+            else:
+                raise ValueError(kind)
+            v[out] = buf
+        return v
+
+    def close(self):
+        for p in self.plans.values():
+            p.close()
+
+
+def run_reference(model, orc, x, keep=None):
+    """Executes the program with a CPU executor `orc` that offers the oracle's functions
+    (quantize_linear, qlinear_conv_int, max_pool_q8, ...).  Test and benchmark code passes
+    the oracle module in; this module itself never imports it."""
+    q = model["qparams"]
+    v = {"x": x}
+    for ins in model["program"]:
+        kind, out = ins[0], ins[1]
+        if kind == "QuantizeLinear":
+            v[out] = orc.quantize_linear(v[ins[2]], ins[3], ins[4], np.uint8)
+        elif kind == "QLinearConv":
+            c = model["convs"][ins[3]]
+            v[out] = orc.qlinear_conv_int(v[ins[2]], c.x_scale, c.x_zp, c.wq, c.w_scale, c.w_zp, c.y_scale, c.y_zp,
+                                          np.uint8, bias=c.bias_q, strides=(c.stride, c.stride), pads=(c.pad, c.pad),
+                                          bias_mode=orc.BIAS_ONNX_INT32)
+        elif kind == "MaxPool":
+            v[out] = orc.max_pool_q8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6])
+        elif kind == "AddRelu":
+            a = orc.dequantize_linear(v[ins[2]], *q[ins[2]])
+            b = orc.dequantize_linear(v[ins[3]], *q[ins[3]])
+            v[out] = orc.quantize_linear(orc.relu(orc.binary(orc.ADD, a, b)), q[out][0], q[out][1], np.uint8)
+        elif kind == "AveragePool":
+            v[out] = orc.average_pool_q8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0),
+                                         q[out][0], q[out][1], np.uint8)
+        elif kind == "DequantizeLinear":
+            v[out] = orc.dequantize_linear(v[ins[2]], ins[3], ins[4])
+        else:
+            raise ValueError(kind)
+        if keep is not None:
+            for name in list(v):
+                if name not in keep and name != out and not _still_needed(model["program"], ins, name):
+                    del v[name]
+    return v
+
+
+def _still_needed(program, current, name):
+    seen = False
+    for ins in program:
+        if ins is current:
+            seen = True
+            continue
+        if seen and name in ins[2:]:
+            return True
+    return False

@@ -189,6 +189,26 @@ int chx_hip_qlinear_matmul(
         int32_t b_zero_point, float y_scale, int32_t y_zero_point, const chx_hip_tensor* bias, uint32_t flags,
         chx_hip_tensor* y, void* stream);
 
+/* ---- pooling on quantized tensors ------------------------------------------------------ */
+
+/* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized
+ * network: DequantizeLinear -> MaxPool -> QuantizeLinear with one scale and zero
+ * point on both sides, which equals the maximum of the 8-bit codes.  x, y uint8 or
+ * int8 (same dtype), [N,C,H,W].  cover_all as in ChainerX: the output extent is
+ * ceil((in + pads - k) / s) + 1 and overhanging windows see only the image. */
+int chx_hip_max_pool_q8(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+        int32_t pad_h_begin, int32_t pad_w_begin, int32_t pad_h_end, int32_t pad_w_end, int32_t cover_all,
+        chx_hip_tensor* y, void* stream);
+
+/* AveragePoolOp::RunImpl, runtime/ops/pooling.cc:63-75, between a DequantizeLinear
+ * (x_scale, x_zero_point) and a QuantizeLinear (y_scale, y_zero_point):
+ * y = Q(sum_{window} DQ(x) / count), fp32 sum in (kh, kw) order. */
+int chx_hip_average_pool_q8(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, int32_t kernel_h, int32_t kernel_w,
+        int32_t stride_h, int32_t stride_w, int32_t pad_h, int32_t pad_w, int32_t count_include_pad, float y_scale,
+        int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
+
 /* ---- fused element-wise chains ---------------------------------------------------------- */
 
 /* ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161.  `code` is the program

@@ -517,3 +517,81 @@ void orc_round_f32(const float* x, int64_t n, float* y) {
     for (int64_t i = 0; i < n; ++i) y[i] = (float)rint((double)x[i]);
 }
 
+
+/* ------------------------------------------------------------------------- */
+/* Pooling between a DequantizeLinear and a QuantizeLinear, as a quantized network
+ * runs it (MaxPoolOp / AveragePoolOp::RunImpl, runtime/ops/pooling.cc:47-75).
+ *
+ * orc_max_pool_q8: DequantizeLinear -> MaxPool -> QuantizeLinear with the same scale
+ * and zero point on both sides equals the maximum of the codes, because the
+ * dequantization map is increasing and Q(DQ(q)) == q for uint8 (checked exhaustively
+ * in the tests).  Out-of-image taps never win (ChainerX pads max-pooling with the
+ * lowest value); cover_all makes the last window start inside the image even when
+ * it overhangs: out = ceil((in + p0 + p1 - k) / s) + 1 instead of floor.
+ *
+ * orc_average_pool_q8: y = Q( (sum over the window of DQ(x)) / count ), the sum taken
+ * in fp32 in (kh, kw) order starting from 0.  PARITY UNPINNED for that order and for
+ * "divide by count" (ChainerX's AveragePool kernel is not in the tree); padding taps
+ * add 0 and count toward `count` when count_include_pad. */
+static int64_t pool_out_dim(int64_t in, int64_t p0, int64_t p1, int64_t k, int64_t s, int cover_all) {
+    if (cover_all) return (in + p0 + p1 - k + s - 1) / s + 1;
+    return (in + p0 + p1 - k) / s + 1;
+}
+
+int64_t orc_pool_out_dim(int64_t in, int64_t p0, int64_t p1, int64_t k, int64_t s, int cover_all) {
+    return pool_out_dim(in, p0, p1, k, s, cover_all);
+}
+
+void orc_max_pool_q8(
+        const void* x, int x_is_int8, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw, int64_t sh,
+        int64_t sw, int64_t ph0, int64_t pw0, int64_t ph1, int64_t pw1, int cover_all, void* y) {
+    const int64_t OH = pool_out_dim(H, ph0, ph1, kh, sh, cover_all), OW = pool_out_dim(W, pw0, pw1, kw, sw, cover_all);
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t nc = 0; nc < N * C; ++nc) {
+        for (int64_t oh = 0; oh < OH; ++oh)
+            for (int64_t ow = 0; ow < OW; ++ow) {
+                int32_t m = -1000;
+                for (int64_t i = 0; i < kh; ++i)
+                    for (int64_t j = 0; j < kw; ++j) {
+                        const int64_t ih = oh * sh - ph0 + i, iw = ow * sw - pw0 + j;
+                        if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                        const int32_t v = load_q(x, x_is_int8, (nc * H + ih) * W + iw);
+                        if (v > m) m = v;
+                    }
+                if (x_is_int8)
+                    ((int8_t*)y)[(nc * OH + oh) * OW + ow] = (int8_t)m;
+                else
+                    ((uint8_t*)y)[(nc * OH + oh) * OW + ow] = (uint8_t)m;
+            }
+    }
+}
+
+void orc_average_pool_q8(
+        const void* x, int x_is_int8, float x_scale, int32_t x_zp, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh,
+        int64_t kw, int64_t sh, int64_t sw, int64_t ph, int64_t pw, int count_include_pad, float y_scale, int32_t y_zp,
+        int y_is_int8, int round_mode, void* y) {
+    const int64_t OH = pool_out_dim(H, ph, ph, kh, sh, 0), OW = pool_out_dim(W, pw, pw, kw, sw, 0);
+    const float lo = y_is_int8 ? -128.f : 0.f, hi = y_is_int8 ? 127.f : 255.f;
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t nc = 0; nc < N * C; ++nc) {
+        for (int64_t oh = 0; oh < OH; ++oh)
+            for (int64_t ow = 0; ow < OW; ++ow) {
+                float sum = 0.f;
+                int32_t cnt = 0;
+                for (int64_t i = 0; i < kh; ++i)
+                    for (int64_t j = 0; j < kw; ++j) {
+                        const int64_t ih = oh * sh - ph + i, iw = ow * sw - pw + j;
+                        if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                        sum = sum + dequantize_one(load_q(x, x_is_int8, (nc * H + ih) * W + iw), x_scale, x_zp);
+                        ++cnt;
+                    }
+                if (count_include_pad) cnt = (int32_t)(kh * kw);
+                volatile float mean = sum / (float)cnt;
+                const int32_t q = quantize_one(mean, y_scale, y_zp, lo, hi, round_mode);
+                if (y_is_int8)
+                    ((int8_t*)y)[(nc * OH + oh) * OW + ow] = (int8_t)q;
+                else
+                    ((uint8_t*)y)[(nc * OH + oh) * OW + ow] = (uint8_t)q;
+            }
+    }
+}

@@ -340,3 +340,38 @@ def run_chain(program, inputs):
         else:
             raise ValueError("op not in the fusable set: %s" % op)
     return env
+
+
+# --- pooling on quantized tensors (runtime/ops/pooling.cc:47-75 between DQ and Q) -----------------
+
+def pool_out_dim(in_dim, p0, p1, k, s, cover_all=False):
+    lib().orc_pool_out_dim.restype = ctypes.c_int64
+    return int(lib().orc_pool_out_dim(*[ctypes.c_int64(v) for v in (in_dim, p0, p1, k, s)], ctypes.c_int(int(cover_all))))
+
+
+def max_pool_q8(x, kernel, strides, pads=(0, 0), cover_all=False):
+    x = _c(x)
+    N, C, H, W = x.shape
+    OH = pool_out_dim(H, pads[0], pads[0], kernel[0], strides[0], cover_all)
+    OW = pool_out_dim(W, pads[1], pads[1], kernel[1], strides[1], cover_all)
+    y = np.empty((N, C, OH, OW), dtype=x.dtype)
+    i64 = ctypes.c_int64
+    lib().orc_max_pool_q8(_p(x), _i8flag(x), i64(N), i64(C), i64(H), i64(W), i64(kernel[0]), i64(kernel[1]),
+                          i64(strides[0]), i64(strides[1]), i64(pads[0]), i64(pads[1]), i64(pads[0]), i64(pads[1]),
+                          ctypes.c_int(int(cover_all)), _p(y))
+    return y
+
+
+def average_pool_q8(x, x_scale, x_zero_point, kernel, strides, pads, y_scale, y_zero_point, y_dtype=np.uint8,
+                    count_include_pad=False, round_mode=ROUND_REFERENCE):
+    x = _c(x)
+    N, C, H, W = x.shape
+    OH = pool_out_dim(H, pads[0], pads[0], kernel[0], strides[0])
+    OW = pool_out_dim(W, pads[1], pads[1], kernel[1], strides[1])
+    y = np.empty((N, C, OH, OW), dtype=y_dtype)
+    i64 = ctypes.c_int64
+    lib().orc_average_pool_q8(_p(x), _i8flag(x), _f(x_scale), ctypes.c_int32(int(x_zero_point)), i64(N), i64(C), i64(H),
+                              i64(W), i64(kernel[0]), i64(kernel[1]), i64(strides[0]), i64(strides[1]), i64(pads[0]),
+                              i64(pads[1]), ctypes.c_int(int(count_include_pad)), _f(y_scale),
+                              ctypes.c_int32(int(y_zero_point)), ctypes.c_int(_i8flag(y)), ctypes.c_int(round_mode), _p(y))
+    return y

@@ -7,6 +7,7 @@ import __graft_entry__ as entry
 pkg = entry.load_package()
 capi = pkg.capi
 ops = pkg.ops
+workloads = pkg.workloads
 
 
 def dev(a):

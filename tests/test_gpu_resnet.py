@@ -1,0 +1,69 @@
+"""Whole quantized networks on the MI355X against the CPU oracle executing the same
+op program: every intermediate tensor must be bit-identical (uint8), the final
+DequantizeLinear output identical as fp32."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+def check_model(g, oracle, model, threads=16):
+    wl = g.pkg.workloads
+    runner = wl.DeviceRunner(model, g.pkg)
+    dev = runner.run(torch.from_numpy(model["input"]).cuda())
+    torch.cuda.synchronize()
+    oracle.set_threads(threads)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"])
+    finally:
+        oracle.set_threads(1)
+    for ins in model["program"]:
+        name = ins[1]
+        got = dev[name].cpu().numpy()
+        np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s" % (name, ins[0]))
+    runner.close()
+    return ref
+
+
+def test_pooling_ops(g, oracle):
+    rng = np.random.default_rng(41)
+    x = rng.integers(0, 256, size=(2, 32, 13, 12)).astype(np.uint8)
+    for cover_all in (False, True):
+        want = oracle.max_pool_q8(x, (3, 3), (2, 2), (0, 0), cover_all)
+        for xd in (g.dev(x), g.to_channels_last(g.dev(x))):
+            np.testing.assert_array_equal(g.host(g.ops.MaxPoolQ8(xd, (3, 3), (2, 2), (0, 0), cover_all)), want)
+    xi = rng.integers(-128, 128, size=(1, 16, 9, 9)).astype(np.int8)
+    np.testing.assert_array_equal(g.host(g.ops.MaxPoolQ8(g.to_channels_last(g.dev(xi)), (2, 2), (2, 2), (1, 1))),
+                                  oracle.max_pool_q8(xi, (2, 2), (2, 2), (1, 1)))
+    want = oracle.average_pool_q8(x, 0.05, 30, (7, 7), (1, 1), (0, 0), 0.02, 7)
+    np.testing.assert_array_equal(g.host(g.ops.AveragePoolQ8(g.to_channels_last(g.dev(x)), 0.05, 30, (7, 7), (1, 1), (0, 0),
+                                                             0.02, 7)), want)
+    assert want.min() < want.max()
+    # max of the codes == Q(MaxPool(DQ(x))) spelled out on the CPU
+    dq = oracle.dequantize_linear(x, 0.05, 30)
+    pooled = np.stack([[dq[n, c, i:i + 3, j:j + 3].max() for i in range(0, 11, 2) for j in range(0, 10, 2)]
+                       for n in range(2) for c in range(32)]).reshape(2, 32, 6, 5)
+    np.testing.assert_array_equal(oracle.quantize_linear(pooled, 0.05, 30), oracle.max_pool_q8(x, (3, 3), (2, 2)))
+
+
+def test_small_resnet_every_value(g, oracle):
+    model = g.pkg.workloads.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
+    ref = check_model(g, oracle, model)
+    # the quantized network tracks the float one it was calibrated on
+    err = np.abs(ref["logits"].reshape(2, 10) - model["float_logits"].reshape(2, 10)).max()
+    assert err < 0.25 * np.abs(model["float_logits"]).max() + 0.5
+
+
+def test_resnet50_batch1(g, oracle):
+    """The real architecture (ResNet-50 v1, 224x224) on one image."""
+    model = g.pkg.workloads.build_resnet50(batch=1, seed=3)
+    assert 3.8e9 < model["macs"] < 4.2e9
+    check_model(g, oracle, model)
