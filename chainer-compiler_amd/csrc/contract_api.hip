@@ -3,6 +3,8 @@
 // (runtime/ops/quantize.cc:62-146) and GroupedConv (runtime/chainerx_util.cc:313-340);
 // the arithmetic is in the kernels.
 #include <climits>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -172,26 +174,49 @@ struct PackedWeights {
     int8_t* wp = nullptr;
     int32_t* wsum = nullptr;
     int C64 = 0, OCpad = 0, KP = 0;
+    bool dense = false;  // taps packed densely; activations go through an explicit im2col
 };
 
+// Dense packing pays when per-tap padding to 64 channels would at least double the K extent.
+bool prefer_dense(int C, int KH, int KW) {
+    return KH * KW > 1 && round_up(C, 64) * KH * KW >= 2 * round_up(C * KH * KW, 64);
+}
+
 size_t packed_bytes(int OC, int C, int KH, int KW, PackedWeights* pw) {
-    pw->C64 = round_up(C, 64);
     pw->OCpad = round_up(OC, 128);
-    pw->KP = KH * KW * pw->C64;
+    pw->dense = prefer_dense(C, KH, KW);
+    if (pw->dense) {
+        pw->KP = round_up(C * KH * KW, 64);
+        pw->C64 = pw->KP;
+    } else {
+        pw->C64 = round_up(C, 64);
+        pw->KP = KH * KW * pw->C64;
+    }
     return (size_t)pw->OCpad * pw->KP;
 }
 
 // The weights qualify for the MFMA kernel: one group, int8, accumulator cannot overflow.
 bool weights_fit_mfma(const chx_hip_tensor& w, int group) {
     if (group != 1 || w.dtype != CHX_HIP_INT8) return false;
-    const int64_t K = (int64_t)round_up((int)w.shape[1], 64) * w.shape[2] * w.shape[3];
-    return K * 128 * 128 < (int64_t(1) << 31) && w.shape[0] < (1 << 24);
+    if (w.shape[1] > (1 << 20) || w.shape[2] * w.shape[3] > 64) return false;  // one mask bit per filter tap
+    PackedWeights pw;
+    packed_bytes(1, (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], &pw);
+    return (int64_t)pw.KP * 128 * 128 < (int64_t(1) << 31) && w.shape[0] < (1 << 24);
 }
 
-// Tile shape: the largest tile that still gives every compute unit about two work-groups.
+// Tile shape: the largest tile that still gives every compute unit a work-group.
 void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px) {
+    // CHX_HIP_TILE=<oc>,<px> forces a tile shape (tuning aid)
+    if (const char* env = getenv("CHX_HIP_TILE")) {
+        int toc = 0, tpx = 0;
+        if (sscanf(env, "%d,%d", &toc, &tpx) == 2 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128)) {
+            *tile_oc = toc;
+            *tile_px = tpx;
+            return;
+        }
+    }
     static const int cand[4][2] = {{128, 128}, {64, 128}, {128, 64}, {64, 64}};
-    const int64_t want = 2 * 256;
+    const int64_t want = 256;
     for (int i = 0; i < 4; ++i) {
         int toc = cand[i][0], tpx = cand[i][1];
         if (OC <= 64 && toc > 64) continue;
@@ -245,7 +270,15 @@ bool y_is_pixel_major(const chx_hip_tensor& y, int64_t* px_stride) {
     return true;
 }
 
+// Scratch buffers that outlive a call: a plan keeps its transposition / im2col space so that
+// repeated runs allocate nothing (and can be captured into a HIP graph).  Grow-only.
+struct ScratchCache {
+    void* ptr[2] = {nullptr, nullptr};
+    size_t size[2] = {0, 0};
+};
+
 struct ConvCall {
+    ScratchCache* cache;  // null: stream-ordered scratch for this call only
     const chx_hip_tensor* x;
     chx_hip_tensor* y;
     const chx_hip_conv_params* p;
@@ -263,6 +296,25 @@ struct ConvCall {
 // NCHW-contiguous (transposed into scratch first); y may be pixel-major (written in place) or
 // NCHW-contiguous 8-bit (written to scratch, then transposed).  Returns EUNSUPPORTED when the
 // operand layouts fit neither, so that the caller can fall back to the direct kernel.
+int acquire_scratch(ScratchCache* cache, int slot, size_t bytes, hipStream_t s, void** out) {
+    if (!cache) return scratch_alloc(out, bytes, s);
+    if (cache->size[slot] < bytes) {
+        // the old buffer may still be in use by work queued on the stream
+        CHX_HIP_CALL(hipStreamSynchronize(s));
+        if (cache->ptr[slot]) CHX_HIP_CALL(hipFree(cache->ptr[slot]));
+        cache->ptr[slot] = nullptr;
+        cache->size[slot] = 0;
+        CHX_HIP_CALL(hipMalloc(&cache->ptr[slot], bytes));
+        cache->size[slot] = bytes;
+    }
+    *out = cache->ptr[slot];
+    return CHX_HIP_OK;
+}
+
+void release_scratch(ScratchCache* cache, void* p, hipStream_t s) {
+    if (!cache) scratch_free(p, s);
+}
+
 int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     const chx_hip_tensor& x = *c.x;
     chx_hip_tensor& y = *c.y;
@@ -272,14 +324,42 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     void* y_scratch = nullptr;
     ConvMfmaArgs a;
     memset(&a, 0, sizeof(a));
-    if (x_is_mfma_ready(x)) {
+    int KH = cs.KH, KW = cs.KW, H = cs.H, W = cs.W, sh = c.p->stride_h, sw = c.p->stride_w, ph = c.p->pad_h_begin,
+        pw_ = c.p->pad_w_begin, C16eff = C16;
+    if (pw.dense) {
+        // explicit im2col: [M][Kd] bytes, then a 1x1 convolution over Kd channels and M pixels in a row
+        const int64_t M = (int64_t)cs.N * cs.OH * cs.OW;
+        CHX_REQUIRE(M <= INT32_MAX, "QLinearConv: too many output pixels for the im2col path");
+        CHX_PROPAGATE(acquire_scratch(c.cache, 0, (size_t)M * pw.KP, s, &x_scratch));
+        Im2colArgs ia;
+        memset(&ia, 0, sizeof(ia));
+        ia.x = static_cast<const char*>(x.data);
+        for (int i = 0; i < 4; ++i) ia.xs[i] = x.strides[i];
+        ia.C = cs.C; ia.H = cs.H; ia.W = cs.W; ia.OH = cs.OH; ia.OW = cs.OW; ia.KH = cs.KH; ia.KW = cs.KW;
+        ia.sh = sh; ia.sw = sw; ia.ph = ph; ia.pw = pw_;
+        ia.Kd = pw.KP;
+        ia.fill = c.x_zp;
+        ia.M = M;
+        ia.col = static_cast<char*>(x_scratch);
+        const int rc = launch_im2col_dense(ia, s);
+        if (rc != CHX_HIP_OK) {
+            release_scratch(c.cache, x_scratch, s);
+            return rc;
+        }
+        a.x = static_cast<const char*>(x_scratch);
+        a.x_w_stride = pw.KP;
+        a.x_h_stride = 0;
+        a.x_n_stride = 0;
+        KH = KW = 1; H = 1; W = (int)M; sh = sw = 1; ph = pw_ = 0;
+        C16eff = pw.KP;
+    } else if (x_is_mfma_ready(x)) {
         a.x = static_cast<const char*>(x.data);
         a.x_n_stride = x.strides[0];
         a.x_h_stride = x.strides[2];
         a.x_w_stride = x.strides[3];
     } else if (is_contiguous(x)) {
         const int64_t HW = (int64_t)cs.H * cs.W;
-        CHX_PROPAGATE(scratch_alloc(&x_scratch, (size_t)cs.N * HW * C16, s));
+        CHX_PROPAGATE(acquire_scratch(c.cache, 0, (size_t)cs.N * HW * C16, s, &x_scratch));
         CHX_PROPAGATE(launch_nchw_to_nhwc_u8(static_cast<const char*>(x.data), static_cast<char*>(x_scratch), cs.N, cs.C,
                                              HW, C16, s));
         a.x = static_cast<const char*>(x_scratch);
@@ -298,23 +378,25 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     } else if (is_contiguous(y) && !c.out_int32) {
         const int64_t OHW = (int64_t)cs.OH * cs.OW;
         const int pitch = round_up(cs.OC, 16);
-        if (scratch_alloc(&y_scratch, (size_t)cs.N * OHW * pitch, s) != CHX_HIP_OK) {
-            scratch_free(x_scratch, s);
+        if (acquire_scratch(c.cache, 1, (size_t)cs.N * OHW * pitch, s, &y_scratch) != CHX_HIP_OK) {
+            release_scratch(c.cache, x_scratch, s);
             return CHX_HIP_ERUNTIME;
         }
         a.y = static_cast<char*>(y_scratch);
         a.y_px_stride = pitch;
         y_post = true;
     } else {
-        scratch_free(x_scratch, s);
+        release_scratch(c.cache, x_scratch, s);
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "y layout is neither pixel-major nor NCHW-contiguous 8-bit");
     }
     a.y_vec_ok = aligned(a.y, 16) && (a.y_px_stride % 16 == 0) ? 1 : 0;
     (void)es;
-    a.C16 = C16;
+    a.C16 = C16eff;
     a.C64 = pw.C64;
-    a.H = cs.H; a.W = cs.W; a.OH = cs.OH; a.OW = cs.OW; a.KH = cs.KH; a.KW = cs.KW;
-    a.sh = c.p->stride_h; a.sw = c.p->stride_w; a.ph = c.p->pad_h_begin; a.pw = c.p->pad_w_begin;
+    a.H = H; a.W = W; a.KH = KH; a.KW = KW;
+    a.OH = pw.dense ? 1 : cs.OH;
+    a.OW = pw.dense ? (int)((int64_t)cs.N * cs.OH * cs.OW) : cs.OW;
+    a.sh = sh; a.sw = sw; a.ph = ph; a.pw = pw_;
     a.M = (int64_t)cs.N * cs.OH * cs.OW;
     a.OC = cs.OC;
     a.KP = pw.KP;
@@ -328,6 +410,8 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.w_scale_len = c.w_scale_len;
     a.bias = c.bias;
     a.rq = c.rq;
+    a.inv_y_scale = c.out_int32 ? 0.f : 1.0f / c.rq.q.scale;
+    CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64;
     pick_tile(cs.OC, a.M, &toc, &tpx);
     int rc = launch_conv_mfma(a, toc, tpx, xu, c.out_int32, c.rne, s);
@@ -335,8 +419,8 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
         rc = launch_nhwc_to_nchw_u8(static_cast<const char*>(y_scratch), static_cast<char*>(y.data), cs.N, cs.OC,
                                     (int64_t)cs.OH * cs.OW, (int)a.y_px_stride, s);
     }
-    scratch_free(x_scratch, s);
-    scratch_free(y_scratch, s);
+    release_scratch(c.cache, x_scratch, s);
+    release_scratch(c.cache, y_scratch, s);
     return rc;
 }
 
@@ -390,6 +474,7 @@ int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedW
     }
     pw->wp = static_cast<int8_t*>(p0);
     pw->wsum = static_cast<int32_t*>(p1);
+    if (pw->dense) return pack_weights_dense(w, pw->KP, pw->OCpad, pw->wp, pw->wsum, s);
     return pack_weights(w, pw->C64, pw->OCpad, pw->wp, pw->wsum, s);
 }
 
@@ -448,6 +533,7 @@ int check_qconv(
 ConvCall conv_call_from(const QConvChecked& q, const chx_hip_tensor* x, chx_hip_tensor* y, const chx_hip_conv_params* p,
                         bool rne) {
     ConvCall c;
+    c.cache = nullptr;
     c.x = x;
     c.y = y;
     c.p = p;
@@ -471,6 +557,7 @@ struct chx_hip_qconv_plan {
     chx_hip_conv_params params;
     bool mfma;
     chx::PackedWeights pw;
+    chx::ScratchCache scratch;  // makes run() unsafe to call concurrently on one plan
 };
 
 extern "C" int chx_hip_qlinear_conv(
@@ -550,7 +637,9 @@ extern "C" int chx_hip_qconv_plan_run(
     hipStream_t s = as_stream(stream);
     const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
     if (plan->mfma) {
-        const int rc = run_conv_mfma(conv_call_from(q, x, y, &plan->params, rne), plan->pw, s);
+        ConvCall call = conv_call_from(q, x, y, &plan->params, rne);
+        call.cache = const_cast<ScratchCache*>(&plan->scratch);
+        const int rc = run_conv_mfma(call, plan->pw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
     return launch_conv_direct(q.direct, rne, s);
@@ -559,6 +648,8 @@ extern "C" int chx_hip_qconv_plan_run(
 extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {
     if (!plan) return;
     chx::release_packed(&plan->pw, true, nullptr);
+    for (int i = 0; i < 2; ++i)
+        if (plan->scratch.ptr[i]) (void)hipFree(plan->scratch.ptr[i]);
     delete plan;
 }
 

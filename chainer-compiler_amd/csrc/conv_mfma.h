@@ -31,9 +31,22 @@ struct ConvMfmaArgs {
     int32_t w_scale_len;
     const int32_t* bias;
     RequantParams rq;
+    float inv_y_scale;           // 1 / y_scale, for the guarded fast requantization
     int32_t tiles_oc, tiles_px;  // filled by the launcher
 };
 
+struct Im2colArgs {
+    const char* x;
+    int64_t xs[4];  // byte strides of N, C, H, W
+    int32_t C, H, W, OH, OW, KH, KW, sh, sw, ph, pw;
+    int32_t Kd;     // row length of the expanded matrix, a multiple of 64
+    int32_t fill;   // the activation zero point (raw code)
+    int64_t M;
+    char* col;      // [M][Kd]
+};
+
+int pack_weights_dense(const chx_hip_tensor& w, int Kd, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+int launch_im2col_dense(const Im2colArgs& a, hipStream_t s);
 int pack_weights(const chx_hip_tensor& w, int C64, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, bool x_unsigned, bool out_int32, bool rne, hipStream_t s);
 

@@ -196,6 +196,10 @@ class DeviceRunner(object):
             shp = model["shapes"][out]
             if ins[0] == "DequantizeLinear":
                 self.bufs[out] = torch.empty(shp, dtype=torch.float32, device="cuda")
+            elif ins[0] == "QuantizeLinear":
+                # the network input stays NCHW like the fp32 tensor it is quantized from (one flat,
+                # fully coalesced pass); the 3-channel stem reads it through its im2col step
+                self.bufs[out] = torch.empty(shp, dtype=torch.uint8, device="cuda")
             else:
                 n, c, h, w = shp
                 self.bufs[out] = torch.empty((n, h, w, c), dtype=torch.uint8, device="cuda").permute(0, 3, 1, 2)
@@ -229,7 +233,24 @@ class DeviceRunner(object):
             v[out] = buf
         return v
 
+    def capture(self, x):
+        """Records one pass of the program into a HIP graph (after a warm-up pass that
+        compiles the fused kernels and sizes every plan's scratch) and returns a callable that
+        replays it: the launch-bound instruction sequence then costs one graph launch."""
+        self.run(x)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            values = self.run(x)
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return values
+        return replay
+
     def close(self):
+        self._graph = None
         for p in self.plans.values():
             p.close()
 

@@ -152,8 +152,11 @@ int chx_hip_qlinear_conv(
  * dequantization on every call (runtime/ops/quantize.cc:76-88); a ChxVM op object
  * lives as long as the program, so the wrapper keeps one plan per QLinearConv
  * instruction, in the manner of the stateful backend ops (runtime/ops/tvm.cc:90-158).
- * create() synchronizes the stream; run() does not.  The plan keeps pointers to
- * w_scale and bias: they must stay alive and unchanged. */
+ * create() synchronizes the stream; run() does not, and allocates nothing once the plan
+ * has seen its largest input (it keeps its own transposition / im2col space), so a
+ * sequence of runs can be captured into a HIP graph.  One plan must not be run from two
+ * threads or streams at once.  The plan keeps pointers to w_scale and bias: they must
+ * stay alive and unchanged. */
 typedef struct chx_hip_qconv_plan chx_hip_qconv_plan;
 int chx_hip_qconv_plan_create(
         const chx_hip_tensor* w, const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point,

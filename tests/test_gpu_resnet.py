@@ -67,3 +67,24 @@ def test_resnet50_batch1(g, oracle):
     model = g.pkg.workloads.build_resnet50(batch=1, seed=3)
     assert 3.8e9 < model["macs"] < 4.2e9
     check_model(g, oracle, model)
+
+
+def test_hip_graph_replay_matches_eager(g, oracle):
+    """The program captured into a HIP graph: several replays, with eager work and
+    synchronizations in between, must each reproduce the eager result bit for bit."""
+    wl = g.pkg.workloads
+    model = wl.build_resnet50(batch=2, image=64, seed=6, width=16, blocks=(1, 1, 1, 1), classes=10)
+    runner = wl.DeviceRunner(model, g.pkg)
+    x = torch.from_numpy(model["input"]).cuda()
+    eager = {k: v.clone() for k, v in runner.run(x).items()}
+    torch.cuda.synchronize()
+    replay = runner.capture(x)
+    for i in range(4):
+        for buf in runner.bufs.values():
+            buf.zero_()                       # eager work between replays; also proves the replay recomputes
+        torch.cuda.synchronize()
+        out = replay()
+        torch.cuda.synchronize()
+        for ins in model["program"]:
+            assert torch.equal(out[ins[1]], eager[ins[1]]), "replay %d: %s" % (i, ins[1])
+    runner.close()
