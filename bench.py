@@ -8,7 +8,9 @@ headline metric is quoted on).  One step = one pass of the whole op program over
 that is already resident in HBM (fp32 NCHW input; QuantizeLinear is part of the step).
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the int8 MFMA implicit-GEMM
 convolution for resnet50 / conv3x3, the fused element-wise kernel for fusion / qdq), timed
-live with events on the launch stream inside the timed region.  `cpu_baseline` times the
+live with events on the launch stream: around every launch of the timed region for the
+single-kernel workloads, and for resnet50 (whose timed region is a HIP graph replay) around
+back-to-back repeats of each convolution launch right after it.  `cpu_baseline` times the
 restated reference CPU op sequence (the oracle's literal fp32 path) on the host cores for a
 bounded sample of the same workload.
 """
@@ -98,52 +100,51 @@ def bench_resnet50(args, torch, pkg):
     ops, capi = pkg.ops, pkg.capi
     conv_ops = 2.0 * model["macs"]
 
-    def step(timer):
-        if timer is None:
-            runner.run(x)
-            return
-        # Same program, with event pairs around every QLinearConv launch.  A sleeping kernel goes
-        # first so that the host finishes submitting the step while the GPU is still held back:
-        # the event pairs then measure back-to-back execution, not gaps in submission.
-        torch.cuda._sleep(int(2.4e9 * 0.012))
-        q, m = model["qparams"], model
-        v = {"x": x}
-        for fid, ins in enumerate(m["program"]):
-            kind, out = ins[0], ins[1]
-            buf = runner.bufs[out]
-            if kind == "QLinearConv":
-                c = m["convs"][ins[3]]
-                timer.wrap("conv", lambda: runner.plans[ins[3]].run(
-                    v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8, flags=capi.BIAS_ONNX_INT32, out=buf))
-            elif kind == "QuantizeLinear":
-                ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
-            elif kind == "MaxPool":
-                ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
-            elif kind == "AddRelu":
-                ops.ElementWiseNvrtc([v[ins[2]], v[ins[3]]], 1, runner.fusion[out], fid, outs=[buf])
-            elif kind == "AveragePool":
-                ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
-                                  q[out][1], out=buf)
-            elif kind == "DequantizeLinear":
-                ops.DequantizeLinear(v[ins[2]], ins[3], ins[4], out=buf)
-            v[out] = buf
+    def step(_timer):
+        runner.run(x)
 
     # The timed region replays the whole program as one HIP graph (about 125 launches per step
-    # would otherwise be bound by the host).  The per-kernel event pairs cannot be recorded inside
-    # a graph, so the convolution launches are timed in the same number of eagerly launched,
-    # instrumented steps right after.
-    timer = KernelTimer(torch)
+    # would otherwise be bound by the host); --no-graph launches every op from the host instead.
     if args.no_graph:
-        sec = timed_steps(torch, step, args.steps, args.warmup, timer)
+        sec = timed_steps(torch, step, args.steps, args.warmup)
     else:
         replay = runner.capture(x)
         sec = timed_steps(torch, lambda _t: replay(), args.steps, args.warmup)
-        timed_steps(torch, step, args.steps, 1, timer)
-    tot = timer.totals()["conv"]
-    n_launch = tot[0] / args.steps
-    conv_ms_per_step = tot[1] / args.steps
+
+    # Launch duration of the dominant kernel: event pairs cannot be recorded inside a graph
+    # replay, and around single 15-60 us launches they mostly measure submission gaps.  So each
+    # QLinearConv instruction of the program is launched REP times back to back between one
+    # event pair on the launch stream, on the buffers of the step just timed; a sleeping kernel
+    # goes first so that the host is done submitting before the GPU starts.  The per-step
+    # kernel time is the sum of the per-instruction averages.
+    REP = 20
+    vals = runner.run(x)
+    torch.cuda.synchronize()
+    conv_ms_per_step, n_launch = 0.0, 0
+    pairs = []
+    for ins in model["program"]:
+        if ins[0] != "QLinearConv":
+            continue
+        c = model["convs"][ins[3]]
+        fn = lambda: runner.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
+                                              flags=capi.BIAS_ONNX_INT32, out=runner.bufs[ins[1]])
+        torch.cuda._sleep(int(2.4e9 * 0.002))
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(REP):
+            fn()
+        b.record()
+        pairs.append((ins[3], a, b))
+        n_launch += 1
+    torch.cuda.synchronize()
+    per_layer = {}
+    for name, a, b in pairs:
+        ms = a.elapsed_time(b) / REP
+        per_layer[name] = ms
+        conv_ms_per_step += ms
     achieved = conv_ops / (conv_ms_per_step * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % round(n_launch),
+    roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % n_launch,
                     achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
                     ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
     res = dict(metric="images/sec ResNet-50 int8 bs64 @1 GPU", value=batch / sec, unit="images/sec",
@@ -203,13 +204,22 @@ def bench_conv3x3(args, torch, pkg):
     y = plan.run(xd, 0.02, 128, 0.05, 128, flags=capi.BIAS_ONNX_INT32)
     mac = n * 28 * 28 * 128 * 128 * 9
 
-    def step(timer):
-        fn = lambda: plan.run(xd, 0.02, 128, 0.05, 128, flags=capi.BIAS_ONNX_INT32, out=y)
-        timer.wrap("conv", fn) if timer else fn()
+    fn = lambda: plan.run(xd, 0.02, 128, 0.05, 128, flags=capi.BIAS_ONNX_INT32, out=y)
 
-    timer = KernelTimer(torch)
-    sec = timed_steps(torch, step, args.steps, args.warmup, timer)
-    cnt, ms = timer.totals()["conv"]
+    def step(_timer):
+        fn()
+
+    sec = timed_steps(torch, step, args.steps, args.warmup)
+    # Launch duration: one event pair around K more launches, queued behind a sleeping kernel so
+    # that the GPU runs them back to back (a pair around one 16 us launch measures submission).
+    torch.cuda._sleep(int(2.4e9 * 0.002))
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(args.steps):
+        fn()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms, cnt = ev0.elapsed_time(ev1), args.steps
     achieved = 2.0 * mac / (ms / cnt * 1e-3) / 1e12
     roofline = dict(bound="mfma", kernel="conv_mfma_kernel", achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s",
                     frac=achieved / INT8_PEAK_TOPS, traffic=None, ops_per_launch=2.0 * mac, launch_us=ms / cnt * 1e3)
@@ -221,14 +231,21 @@ def bench_conv3x3(args, torch, pkg):
         from oracle import oracle as orc
         cores = orc.max_threads()
         orc.set_threads(cores)
-        k = 4
+        reps = 30
         t0 = time.perf_counter()
-        orc.qlinear_conv_literal(x[:k], 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1),
-                                 bias_mode=orc.BIAS_ONNX_INT32)
+        for _ in range(reps):
+            orc.qlinear_conv_literal(x, 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1),
+                                     bias_mode=orc.BIAS_ONNX_INT32)
         dt = time.perf_counter() - t0
         orc.set_threads(1)
-        return dict(value=k / dt, unit="images/sec", cores=cores, kind="port",
-                    sample="%d of %d images, literal fp32 restatement of QLinearConvOp, %d threads, %.2f s" % (k, n, cores, dt))
+        t1 = time.perf_counter()
+        orc.qlinear_conv_literal(x, 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1),
+                                 bias_mode=orc.BIAS_ONNX_INT32)
+        dt1 = time.perf_counter() - t1
+        return dict(value=reps * n / dt, unit="images/sec", cores=cores, kind="port", single_thread_value=n / dt1,
+                    sample="%d passes over all %d images, literal fp32 restatement of QLinearConvOp (dequantize, im2col + "
+                           "sequential-k GEMM, quantize), %d threads: %.1f s; one pass single-threaded: %.1f s" % (
+                               reps, n, cores, dt, dt1))
     return res, roofline, cpu, plan.close
 
 
@@ -270,7 +287,7 @@ def bench_fusion(args, torch, pkg, qdq=False):
         from oracle import oracle as orc
         cores = orc.max_threads()
         orc.set_threads(cores)
-        rows = 2 * 1024
+        rows = 16 * 1024
         xs = x.view(-1, 1024)[:rows].cpu().numpy()
         t0 = time.perf_counter()
         if qdq:
