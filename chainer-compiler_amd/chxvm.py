@@ -1,0 +1,427 @@
+"""Python face of the hip ChxVM runtime (lib/libchxvm_hip_runtime.so).
+
+Three parts, all used by the tests and by hosts that drive the VM from Python:
+
+  * a writer of the ChxVMProgramProto wire format (field numbers of runtime/chxvm.proto.tmpl:1-65
+    of the chainer-compiler tree) and `ProgramBuilder`, which plays the part of the generated
+    `AddXxxOp(prog, ...)` emitters (compiler/chxvm/gen_chxvm_codegen.py:18-101): operands are
+    checked against the op table `runtime/chxvm_ops.idl` and encoded by their declared type;
+  * `Program`: load a serialized program into the C++ VM and run it on device tensors;
+  * `BackendConfig` queries (configs/backend_config.h of the chainer-compiler tree).
+"""
+import ctypes
+import os
+import struct
+
+import numpy as np
+
+from . import capi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+RUNTIME_LIB = os.path.join(_HERE, "lib", "libchxvm_hip_runtime.so")
+IDL_PATH = os.path.join(_HERE, "runtime", "chxvm_ops.idl")
+
+RUNTIME_EXPORTS = [
+    "chxvm_last_error", "chxvm_num_ops", "chxvm_op_name", "chxvm_op_number", "chxvm_proto_roundtrip", "chxvm_free",
+    "chxvm_program_create", "chxvm_program_destroy", "chxvm_program_num_instructions", "chxvm_program_num_inputs",
+    "chxvm_program_input_name", "chxvm_program_run", "chxvm_outputs_count", "chxvm_outputs_name", "chxvm_outputs_get",
+    "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name",
+]
+
+# ChxVMValueProto.Type
+VALUE_TYPE = {"ARRAY": 1, "OPTIONAL_ARRAY": 2, "ARRAY_LIST": 3, "SEQUENCE": 4, "OPAQUE": 5, "INT": 6, "FLOAT": 7,
+              "INTS": 8, "STRING": 9, "LONGS": 10, "DOUBLES": 11, "INT_VALUES": 12, "SHAPE": 13, "SCALAR": 14,
+              "OPTIONAL_SCALAR": 15, "STRINGS": 16}
+
+# IDL operand type -> (Type enum name, encoder)
+_SLOT_TYPES = ("Array", "OptionalArray", "ArrayList", "Scalar", "OptionalScalar", "Shape")
+
+
+class ChxVMError(RuntimeError):
+    pass
+
+
+_rt = None
+
+
+def runtime():
+    """The loaded runtime library; raises when it has not been built (no fallback)."""
+    global _rt
+    if _rt is None:
+        if not os.path.exists(RUNTIME_LIB):
+            raise ChxVMError("%s is missing: build it with `make -C chainer-compiler_amd/runtime`" % RUNTIME_LIB)
+        capi.lib()  # libchx_hip.so first, so that the dependency resolves to the in-tree build
+        rt = ctypes.CDLL(RUNTIME_LIB)
+        rt.chxvm_last_error.restype = ctypes.c_char_p
+        rt.chxvm_op_name.restype = ctypes.c_char_p
+        rt.chxvm_op_name.argtypes = [ctypes.c_int32]
+        rt.chxvm_op_number.argtypes = [ctypes.c_char_p]
+        rt.chxvm_proto_roundtrip.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p),
+                                             ctypes.POINTER(ctypes.c_size_t)]
+        rt.chxvm_free.argtypes = [ctypes.c_void_p]
+        rt.chxvm_free.restype = None
+        rt.chxvm_program_create.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+        rt.chxvm_program_destroy.argtypes = [ctypes.c_void_p]
+        rt.chxvm_program_destroy.restype = None
+        rt.chxvm_program_num_instructions.argtypes = [ctypes.c_void_p]
+        rt.chxvm_program_num_inputs.argtypes = [ctypes.c_void_p]
+        rt.chxvm_program_input_name.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+        rt.chxvm_program_input_name.restype = ctypes.c_char_p
+        rt.chxvm_program_run.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(capi.Tensor),
+                                         ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_void_p)]
+        rt.chxvm_outputs_count.argtypes = [ctypes.c_void_p]
+        rt.chxvm_outputs_name.argtypes = [ctypes.c_void_p, ctypes.c_int32]
+        rt.chxvm_outputs_name.restype = ctypes.c_char_p
+        rt.chxvm_outputs_get.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(capi.Tensor)]
+        rt.chxvm_outputs_destroy.argtypes = [ctypes.c_void_p]
+        rt.chxvm_outputs_destroy.restype = None
+        rt.chxvm_backend_config_has.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_char_p,
+                                                ctypes.POINTER(ctypes.c_int32)]
+        rt.chxvm_backend_config_name.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
+        _rt = rt
+    return _rt
+
+
+def _check(rc):
+    if rc != 0:
+        raise ChxVMError(runtime().chxvm_last_error().decode("utf-8", "replace"))
+
+
+# ---------------------------------------------------------------------------------------------
+# wire format
+# ---------------------------------------------------------------------------------------------
+
+def _varint(v):
+    v &= (1 << 64) - 1  # negative int32/int64 values take ten bytes, as protobuf writes them
+    out = bytearray()
+    while True:
+        b = v & 0x7F
+        v >>= 7
+        if v:
+            out.append(b | 0x80)
+        else:
+            out.append(b)
+            return bytes(out)
+
+
+def _f_varint(field, v):
+    return _varint(field << 3) + _varint(v)
+
+
+def _f_bytes(field, b):
+    if isinstance(b, str):
+        b = b.encode()
+    return _varint((field << 3) | 2) + _varint(len(b)) + b
+
+
+def _f_double(field, v):
+    return _varint((field << 3) | 1) + struct.pack("<d", v)
+
+
+def encode_value(type_name, v):
+    """One ChxVMValueProto (runtime/chxvm.proto.tmpl:1-36)."""
+    out = _f_varint(1, VALUE_TYPE[type_name])
+    if type_name in ("ARRAY", "OPTIONAL_ARRAY"):
+        out += _f_varint(2, v)
+    elif type_name == "INT":
+        out += _f_varint(3, v)
+    elif type_name == "FLOAT":
+        out += _f_double(4, v)
+    elif type_name in ("INTS", "INT_VALUES", "LONGS"):
+        out += b"".join(_f_varint(5, x) for x in v)
+    elif type_name == "STRING":
+        out += _f_bytes(6, v)
+    elif type_name == "ARRAY_LIST":
+        out += b"".join(_f_varint(7, x) for x in v)
+    elif type_name == "SEQUENCE":
+        out += _f_varint(8, v)
+    elif type_name == "DOUBLES":
+        out += b"".join(_f_double(10, x) for x in v)
+    elif type_name == "OPAQUE":
+        out += _f_varint(11, v)
+    elif type_name == "SHAPE":
+        out += _f_varint(12, v)
+    elif type_name in ("SCALAR", "OPTIONAL_SCALAR"):
+        out += _f_varint(13, v)
+    elif type_name == "STRINGS":
+        out += b"".join(_f_bytes(14, x) for x in v)
+    else:
+        raise ValueError(type_name)
+    return out
+
+
+def encode_type(dtype, shape):
+    return _f_varint(1, dtype) + b"".join(_f_varint(2, d) for d in shape)
+
+
+def encode_instruction(op, inputs, outputs, debug_info="", id=0, output_types=(), output_names=(), flops=None):
+    """inputs: list of (type_name, value); outputs: list of slot numbers."""
+    out = _f_varint(1, op)
+    out += b"".join(_f_bytes(2, encode_value(t, v)) for t, v in inputs)
+    out += b"".join(_f_varint(3, o) for o in outputs)
+    if debug_info:
+        out += _f_bytes(4, debug_info)
+    out += _f_varint(5, id)
+    out += b"".join(_f_bytes(6, encode_type(*t)) for t in output_types)
+    out += b"".join(_f_bytes(7, n) for n in output_names)
+    if flops is not None:
+        out += _f_varint(8, flops)
+    return out
+
+
+def encode_program(instructions, input_names=(), input_types=()):
+    out = b"".join(_f_bytes(1, i) for i in instructions)
+    out += b"".join(_f_bytes(2, n) for n in input_names)
+    out += b"".join(_f_bytes(3, encode_type(*t)) for t in input_types)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# op table and program builder
+# ---------------------------------------------------------------------------------------------
+
+_IDL_TO_VALUE = {"Array": "ARRAY", "OptionalArray": "ARRAY", "ArrayList": "ARRAY_LIST", "Scalar": "SCALAR",
+                 "OptionalScalar": "SCALAR", "Shape": "SHAPE", "Int": "INT", "Float": "FLOAT", "Ints": "INTS",
+                 "IntValues": "INT_VALUES", "Doubles": "DOUBLES", "String": "STRING", "Strings": "STRINGS"}
+
+
+def read_op_table(path=IDL_PATH):
+    """[(name, inputs or None, outputs or None)] in op-number order (number = index + 1)."""
+    table = []
+    for raw in open(path):
+        line = raw.split("#")[0].strip()
+        if not line:
+            continue
+        if ":" not in line:
+            table.append((line, None, None))
+            continue
+        head, sig = line.split(":", 1)
+        ins, outs = sig.split("->")
+        parse = lambda t: [tuple(p.split()) for p in (q.strip() for q in t.split(",")) if p]
+        table.append((head.split()[0], parse(ins), parse(outs)))
+    return table
+
+
+# ChainerX dtype numbers (compiler/dtype.h:14-25)
+DTYPE = {"bool": 1, "int8": 2, "int16": 3, "int32": 4, "int64": 5, "uint8": 6, "float16": 7, "float32": 8, "float64": 9}
+
+
+class ProgramBuilder:
+    """Assembles a ChxVMProgramProto instruction by instruction.
+
+    `b.QuantizeLinear(x, scale, zp)` appends the instruction and returns the slot number(s) of
+    its result(s); slot operands take slot numbers (-1 for an absent optional one), field
+    operands take Python values.  `new_slot()` hands out fresh variable ids.
+    """
+
+    def __init__(self, table=None):
+        self.table = table or read_op_table()
+        self.index = {name: (i + 1, ins, outs) for i, (name, ins, outs) in enumerate(self.table)}
+        self.instructions = []
+        self.input_names = []
+        self.input_types = []
+        self.next_slot = 1
+        self.next_id = 1
+
+    def new_slot(self):
+        s = self.next_slot
+        self.next_slot += 1
+        return s
+
+    def __getattr__(self, name):
+        if name.startswith("_") or name not in self.index:
+            raise AttributeError(name)
+        return lambda *args, **kw: self.add(name, *args, **kw)
+
+    def add(self, name, *args, outputs=None, debug_info="", num_list_outputs=None):
+        number, ins, outs = self.index[name]
+        if ins is None:
+            raise ChxVMError("op %s has no signature in the op table of this runtime" % name)
+        if len(args) != len(ins):
+            raise ChxVMError("%s takes %d operands (%s), got %d" % (name, len(ins), ", ".join(n for _, n in ins), len(args)))
+        enc = []
+        for (typ, opname), v in zip(ins, args):
+            if typ in ("OptionalArray", "OptionalScalar") and v is None:
+                v = -1
+            if typ in ("Ints", "IntValues", "ArrayList"):
+                v = [int(x) for x in v]
+            elif typ == "Doubles":
+                v = [float(x) for x in v]
+            elif typ == "Float":
+                v = float(v)
+            elif typ not in ("String", "Strings"):
+                v = int(v)
+            enc.append((_IDL_TO_VALUE[typ], v))
+        if outputs is None:
+            outputs = []
+            for typ, _ in outs:
+                if typ == "ArrayList":
+                    outputs.append([self.new_slot() for _ in range(num_list_outputs)])
+                else:
+                    outputs.append(self.new_slot())
+        flat = []
+        for o in outputs:
+            flat.extend(o if isinstance(o, (list, tuple)) else [o])
+        self.instructions.append(encode_instruction(number, enc, flat, debug_info=debug_info, id=self.next_id))
+        self.next_id += 1
+        if not outputs:
+            return None
+        return outputs[0] if len(outputs) == 1 else tuple(outputs)
+
+    # conveniences -----------------------------------------------------------------------
+    def input(self, name, dtype="float32", shape=()):
+        self.input_names.append(name)
+        self.input_types.append((DTYPE[dtype], list(shape)))
+        return self.add("In", name)
+
+    def output(self, name, slot):
+        self.add("Out", name, slot)
+
+    def scalar(self, value, dtype):
+        if dtype.startswith("float"):
+            return self.add("FloatScalarConstant", value, DTYPE[dtype], 0)
+        return self.add("IntScalarConstant", value, DTYPE[dtype], 0)
+
+    def constant(self, array):
+        a = np.asarray(array)
+        dt = DTYPE[str(a.dtype)]
+        if a.dtype.kind == "f":
+            return self.add("FloatConstant", a.ravel().tolist(), dt, a.shape, 0)
+        return self.add("IntConstant", a.ravel().tolist(), dt, a.shape, 0)
+
+    def serialize(self):
+        return encode_program(self.instructions, self.input_names, self.input_types)
+
+
+# ---------------------------------------------------------------------------------------------
+# running
+# ---------------------------------------------------------------------------------------------
+
+_NP_OF_CODE = {1: np.bool_, 2: np.int8, 3: np.int16, 4: np.int32, 5: np.int64, 6: np.uint8, 7: np.float16, 8: np.float32,
+               9: np.float64}
+
+
+def _to_numpy(desc):
+    """Host copy of the device array a descriptor names, with its shape and element order."""
+    dt = np.dtype(_NP_OF_CODE[desc.dtype])
+    nd = desc.ndim
+    shape = [desc.shape[i] for i in range(nd)]
+    strides = [desc.strides[i] for i in range(nd)]
+    span = dt.itemsize + sum((s - 1) * st for s, st in zip(shape, strides)) if all(shape) else 0
+    buf = np.empty(max(span, 1), dtype=np.uint8)
+    if span:
+        capi.check(capi.lib().chx_hip_memcpy_d2h(buf.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(desc.data),
+                                                 ctypes.c_size_t(span), None))
+    view = np.lib.stride_tricks.as_strided(buf[:dt.itemsize].view(dt), shape=shape, strides=strides) if span else \
+        np.empty(shape, dt)
+    return np.ascontiguousarray(view)
+
+
+class Program:
+    """A serialized ChxVMProgramProto loaded into the C++ VM."""
+
+    def __init__(self, serialized):
+        self._h = ctypes.c_void_p()
+        self.serialized = bytes(serialized)
+        _check(runtime().chxvm_program_create(self.serialized, len(self.serialized), ctypes.byref(self._h)))
+
+    @property
+    def num_instructions(self):
+        return runtime().chxvm_program_num_instructions(self._h)
+
+    @property
+    def input_names(self):
+        rt = runtime()
+        return [rt.chxvm_program_input_name(self._h, i).decode() for i in range(rt.chxvm_program_num_inputs(self._h))]
+
+    def run(self, inputs, trace_level=0):
+        """inputs: {name: torch device tensor}.  Returns {name: numpy array}."""
+        rt = runtime()
+        names = list(inputs)
+        c_names = (ctypes.c_char_p * len(names))(*[n.encode() for n in names])
+        descs = (capi.Tensor * len(names))(*[capi.desc(inputs[n]) for n in names])
+        out = ctypes.c_void_p()
+        _check(rt.chxvm_program_run(self._h, c_names, descs, len(names), trace_level, ctypes.byref(out)))
+        try:
+            result = {}
+            for i in range(rt.chxvm_outputs_count(out)):
+                d = capi.Tensor()
+                _check(rt.chxvm_outputs_get(out, i, ctypes.byref(d)))
+                result[rt.chxvm_outputs_name(out, i).decode()] = _to_numpy(d)
+            return result
+        finally:
+            rt.chxvm_outputs_destroy(out)
+
+    def close(self):
+        if self._h:
+            runtime().chxvm_program_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def proto_roundtrip(serialized):
+    """Parse with the C++ reader and serialize again with the C++ writer."""
+    rt = runtime()
+    out = ctypes.c_void_p()
+    n = ctypes.c_size_t()
+    _check(rt.chxvm_proto_roundtrip(bytes(serialized), len(serialized), ctypes.byref(out), ctypes.byref(n)))
+    try:
+        return ctypes.string_at(out, n.value)
+    finally:
+        rt.chxvm_free(out)
+
+
+def op_name(number):
+    return runtime().chxvm_op_name(number).decode()
+
+
+def op_number(name):
+    return runtime().chxvm_op_number(name.encode())
+
+
+def num_ops():
+    return runtime().chxvm_num_ops()
+
+
+class BackendConfig:
+    """BackendConfig.FromName / FromJSON of the C++ runtime."""
+
+    def __init__(self, config, is_json):
+        self._config = config.encode()
+        self._is_json = 1 if is_json else 0
+        buf = ctypes.create_string_buffer(256)
+        _check(runtime().chxvm_backend_config_name(self._config, self._is_json, buf, 256))
+        self.name = buf.value.decode()
+
+    @classmethod
+    def FromName(cls, name):
+        return cls(name, False)
+
+    @classmethod
+    def FromJSON(cls, text):
+        return cls(text, True)
+
+    def _has(self, section, key):
+        out = ctypes.c_int32()
+        _check(runtime().chxvm_backend_config_has(self._config, self._is_json, section.encode(), key.encode(), ctypes.byref(out)))
+        return out.value
+
+    def simplify_preproc_count(self, key):
+        return self._has("simplify_preproc", key)
+
+    def simplify_count(self, key):
+        return self._has("simplify", key)
+
+    def merge_count(self, key):
+        return self._has("merge", key)
+
+    def expanding_functions_count(self, key):
+        return self._has("expanding_functions", key)
+
+    def HasOp(self, key):
+        return bool(self._has("supported_ops", key))

@@ -1,0 +1,172 @@
+#include "chxvm_capi.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+#include "chxvm.h"
+#include "configs/backend_config.h"
+
+using chainer_compiler::BackendConfig;
+using namespace chainer_compiler::runtime;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+template <class Fn>
+int32_t Guard(Fn fn) {
+    try {
+        fn();
+        return 0;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        return 1;
+    }
+}
+
+}  // namespace
+
+struct chxvm_program {
+    std::unique_ptr<ChxVM> vm;
+};
+
+struct chxvm_outputs {
+    std::vector<std::string> names;
+    std::vector<chainerx::Array> arrays;
+    InOuts keep_inputs;
+};
+
+extern "C" {
+
+const char* chxvm_last_error(void) {
+    return g_last_error.c_str();
+}
+
+int32_t chxvm_num_ops(void) {
+    return NumOps();
+}
+
+const char* chxvm_op_name(int32_t op) {
+    return OpName(op);
+}
+
+int32_t chxvm_op_number(const char* name) {
+    return OpNumber(name);
+}
+
+int32_t chxvm_proto_roundtrip(const void* bytes, size_t size, void** out, size_t* out_size) {
+    return Guard([&] {
+        const ChxVMProgramProto program = ChxVMProgramProto::ParseFromString(std::string(static_cast<const char*>(bytes), size));
+        const std::string again = program.SerializeAsString();
+        *out = std::malloc(again.size() ? again.size() : 1);
+        std::memcpy(*out, again.data(), again.size());
+        *out_size = again.size();
+    });
+}
+
+void chxvm_free(void* p) {
+    std::free(p);
+}
+
+int32_t chxvm_program_create(const void* bytes, size_t size, chxvm_program** out) {
+    return Guard([&] {
+        const ChxVMProgramProto program = ChxVMProgramProto::ParseFromString(std::string(static_cast<const char*>(bytes), size));
+        std::unique_ptr<chxvm_program> p(new chxvm_program());
+        p->vm.reset(new ChxVM(program));
+        *out = p.release();
+    });
+}
+
+void chxvm_program_destroy(chxvm_program* program) {
+    delete program;
+}
+
+int32_t chxvm_program_num_instructions(const chxvm_program* program) {
+    return static_cast<int32_t>(program->vm->num_instructions());
+}
+
+int32_t chxvm_program_num_inputs(const chxvm_program* program) {
+    return static_cast<int32_t>(program->vm->input_names().size());
+}
+
+const char* chxvm_program_input_name(const chxvm_program* program, int32_t i) {
+    return program->vm->input_names()[static_cast<size_t>(i)].c_str();
+}
+
+int32_t chxvm_program_run(
+        chxvm_program* program,
+        const char* const* input_names,
+        const chx_hip_tensor* inputs,
+        int32_t num_inputs,
+        int32_t trace_level,
+        chxvm_outputs** out) {
+    return Guard([&] {
+        InOuts in;
+        for (int32_t i = 0; i < num_inputs; ++i) {
+            const chx_hip_tensor& t = inputs[i];
+            chainerx::Shape shape;
+            chainerx::Strides strides;
+            for (int d = 0; d < t.ndim; ++d) {
+                shape.push_back(t.shape[d]);
+                strides.push_back(t.strides[d]);
+            }
+            std::shared_ptr<void> borrowed(t.data, [](void*) {});
+            chainerx::Array a = chainerx::Array::MakeOwned(borrowed, static_cast<chainerx::Dtype>(t.dtype), shape, strides);
+            CHECK(in.emplace(input_names[i], std::make_shared<ChxVMVar>(a)).second) << "duplicate input " << input_names[i];
+        }
+        ChxVMOptions options;
+        options.trace_level = trace_level;
+        InOuts result = program->vm->Run(in, options);
+        std::unique_ptr<chxvm_outputs> o(new chxvm_outputs());
+        for (const auto& p : result) {
+            o->names.push_back(p.first);
+            o->arrays.push_back(p.second->GetArray());
+        }
+        o->keep_inputs = in;
+        CHXVM_HIP_CALL(chx_hip_stream_synchronize(nullptr));  // device sync at the end of a run (tools/run_onnx.cc:462)
+        *out = o.release();
+    });
+}
+
+int32_t chxvm_outputs_count(const chxvm_outputs* outputs) {
+    return static_cast<int32_t>(outputs->arrays.size());
+}
+
+const char* chxvm_outputs_name(const chxvm_outputs* outputs, int32_t i) {
+    return outputs->names[static_cast<size_t>(i)].c_str();
+}
+
+int32_t chxvm_outputs_get(const chxvm_outputs* outputs, int32_t i, chx_hip_tensor* out) {
+    return Guard([&] {
+        CHECK_LT(static_cast<size_t>(i), outputs->arrays.size());
+        *out = outputs->arrays[static_cast<size_t>(i)].hip();
+    });
+}
+
+void chxvm_outputs_destroy(chxvm_outputs* outputs) {
+    delete outputs;
+}
+
+int32_t chxvm_backend_config_has(const char* config, int32_t is_json, const char* section, const char* key, int32_t* out) {
+    return Guard([&] {
+        std::unique_ptr<BackendConfig> c = is_json ? BackendConfig::FromJSON(config) : BackendConfig::FromName(config);
+        const std::string s = section;
+        if (s == "simplify_preproc") *out = static_cast<int32_t>(c->GetSimplifyPreproc().count(key));
+        else if (s == "simplify") *out = static_cast<int32_t>(c->GetSimplify().count(key));
+        else if (s == "merge") *out = static_cast<int32_t>(c->GetMerge().count(key));
+        else if (s == "expanding_functions") *out = static_cast<int32_t>(c->GetExpandingFunctions().count(key));
+        else if (s == "supported_ops") *out = c->HasOp(key) ? 1 : 0;
+        else CHECK(false) << "unknown section " << s;
+    });
+}
+
+int32_t chxvm_backend_config_name(const char* config, int32_t is_json, char* buf, size_t buf_size) {
+    return Guard([&] {
+        std::unique_ptr<BackendConfig> c = is_json ? BackendConfig::FromJSON(config) : BackendConfig::FromName(config);
+        CHECK_LT(c->name().size(), buf_size);
+        std::strcpy(buf, c->name().c_str());
+    });
+}
+
+}  // extern "C"

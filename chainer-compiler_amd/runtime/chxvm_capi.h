@@ -1,0 +1,63 @@
+/* C face of the hip ChxVM runtime (libchxvm_hip_runtime.so), for hosts that embed the VM without
+ * C++ linkage -- the role of the pybind module `chainer_compiler_core` in the chainer-compiler tree
+ * (tools/run_onnx_core.cc, python/chainer_compiler_core.cc).  Programs are serialized
+ * ChxVMProgramProto messages (runtime/chxvm.proto.tmpl); arrays are device memory described by
+ * chx_hip_tensor.  Every function returns 0 on success; after a failure chxvm_last_error() holds
+ * the message of the failed CHECK (this thread's last one). */
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "chx_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct chxvm_program chxvm_program;
+typedef struct chxvm_outputs chxvm_outputs;
+
+const char* chxvm_last_error(void);
+
+/* op enum: 1-based position in the op table; name of 0 or of an unknown number is "?" */
+int32_t chxvm_num_ops(void);
+const char* chxvm_op_name(int32_t op);
+int32_t chxvm_op_number(const char* name);
+
+/* Parses and re-serializes a program (wire-format round trip); *out is malloc'ed, free with chxvm_free. */
+int32_t chxvm_proto_roundtrip(const void* bytes, size_t size, void** out, size_t* out_size);
+void chxvm_free(void* p);
+
+/* Builds the instruction objects (constants are uploaded, InitImpl runs). */
+int32_t chxvm_program_create(const void* bytes, size_t size, chxvm_program** out);
+void chxvm_program_destroy(chxvm_program* program);
+int32_t chxvm_program_num_instructions(const chxvm_program* program);
+int32_t chxvm_program_num_inputs(const chxvm_program* program);
+const char* chxvm_program_input_name(const chxvm_program* program, int32_t i);
+
+/* Runs the program.  inputs[i] describes device memory the caller keeps alive until the outputs
+ * are destroyed.  trace_level: 0 silent, 1 one line per instruction on stderr, 2 adds values. */
+int32_t chxvm_program_run(
+        chxvm_program* program,
+        const char* const* input_names,
+        const chx_hip_tensor* inputs,
+        int32_t num_inputs,
+        int32_t trace_level,
+        chxvm_outputs** out);
+int32_t chxvm_outputs_count(const chxvm_outputs* outputs);
+const char* chxvm_outputs_name(const chxvm_outputs* outputs, int32_t i);
+/* Descriptor of output i (device memory owned by `outputs`). */
+int32_t chxvm_outputs_get(const chxvm_outputs* outputs, int32_t i, chx_hip_tensor* out);
+void chxvm_outputs_destroy(chxvm_outputs* outputs);
+
+/* BackendConfig queries.  `config` is a built-in name ("chxvm", "chxvm_test", "hip") or, with
+ * is_json != 0, a JSON document.  section: "simplify_preproc", "simplify", "merge",
+ * "expanding_functions" (membership) or "supported_ops" (HasOp).  *out = 0 or 1. */
+int32_t chxvm_backend_config_has(const char* config, int32_t is_json, const char* section, const char* key, int32_t* out);
+/* Name of the configuration ("custom" for a JSON document) into buf. */
+int32_t chxvm_backend_config_name(const char* config, int32_t is_json, char* buf, size_t buf_size);
+
+#ifdef __cplusplus
+}
+#endif

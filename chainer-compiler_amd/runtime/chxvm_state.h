@@ -1,0 +1,92 @@
+// ChxVMState: the variable slots of one run, with the accessors the generated Run() glue uses
+// (runtime/chxvm_state.h:21-106, runtime/chxvm_state.cc of the chainer-compiler tree).
+#pragma once
+
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "chxvm_var.h"
+
+namespace chainer_compiler {
+namespace runtime {
+
+typedef std::map<std::string, std::shared_ptr<ChxVMVar>> InOuts;
+
+struct ChxVMOptions {
+    int trace_level = 0;
+    bool is_training = false;
+    bool check_nans = false;
+    bool check_infs = false;
+};
+
+class ChxVMState {
+public:
+    ChxVMState(const ChxVMOptions& options, int num_variables, const InOuts& inputs);
+
+    int pc() const {
+        return pc_;
+    }
+    void set_pc(int pc) {
+        pc_ = pc;
+    }
+
+    chainerx::Array GetArray(int index);
+    absl::optional<chainerx::Array> GetOptionalArray(int index);
+    void SetArray(int index, const chainerx::Array& value);
+    void FreeVar(int index);
+
+    std::vector<chainerx::Array> GetArrayList(const std::vector<int>& index);
+    void SetArrayList(const std::vector<int>& index, const std::vector<chainerx::Array>& vars);
+
+    ChxVMVar* GetVar(int index);
+    void SetVar(int index, const ChxVMVar& var);
+
+    const chainerx::Shape& GetShape(int index);
+    void SetShape(int index, chainerx::Shape s);
+
+    const StrictScalar& GetScalar(int index);
+    absl::optional<StrictScalar> GetOptionalScalar(int index);
+    void SetScalar(int index, StrictScalar s);
+
+    std::string GetVarString(int index);
+    std::string GetVarListString(const std::vector<int>& indices);
+
+    void Input(const std::string& name, int index);
+    void Output(const std::string& name, int index);
+
+    const InOuts& GetOutputs() const {
+        return outputs_;
+    }
+
+    // NaN/Inf scans of the reference (runtime/chxvm_state.cc:245-263) are float-only debugging
+    // aids; the quantized path keeps the switches but has nothing to scan.
+    void CheckNans(const std::vector<int>&, const std::vector<int>&) {
+    }
+    void CheckInfs(const std::vector<int>&, const std::vector<int>&) {
+    }
+
+    int trace_level() const {
+        return options_.trace_level;
+    }
+    bool is_training() const {
+        return options_.is_training;
+    }
+    bool check_nans() const {
+        return options_.check_nans;
+    }
+    bool check_infs() const {
+        return options_.check_infs;
+    }
+
+private:
+    int pc_ = 0;
+    std::vector<std::unique_ptr<ChxVMVar>> variables_;
+    InOuts inputs_;
+    InOuts outputs_;
+    ChxVMOptions options_;
+};
+
+}  // namespace runtime
+}  // namespace chainer_compiler

@@ -1,0 +1,67 @@
+// ElementWiseNvrtcOp::RunImpl on the hip backend (runtime/ops/nvrtc.cc:90-161 of the
+// chainer-compiler tree): result shape = broadcast of the inputs, outputs allocated here, the
+// kernel generated, compiled, cached and launched behind chx_hip_elementwise.  The inputs are
+// handed over as they are; nothing is broadcast or copied first.
+#include <sstream>
+
+#include "../gen/gen_chxvm_ops.h"
+
+namespace chainer_compiler {
+namespace runtime {
+
+namespace {
+
+// dtypes of the outputs, from the program's `out name:dtype ...` line
+std::vector<chainerx::Dtype> OutputDtypes(const std::string& code) {
+    std::vector<chainerx::Dtype> out;
+    std::istringstream iss(code);
+    std::string line;
+    while (std::getline(iss, line)) {
+        std::istringstream ls(line);
+        std::string tok;
+        if (!(ls >> tok) || tok != "out") continue;
+        while (ls >> tok) {
+            const size_t c = tok.find(':');
+            CHECK(c != std::string::npos) << "bad output declaration in fusion program: " << tok;
+            const std::string dt = tok.substr(c + 1);
+            if (dt == "float32") out.push_back(chainerx::Dtype::kFloat32);
+            else if (dt == "uint8") out.push_back(chainerx::Dtype::kUInt8);
+            else if (dt == "int8") out.push_back(chainerx::Dtype::kInt8);
+            else CHECK(false) << "unsupported dtype in fusion program: " << dt;
+        }
+    }
+    return out;
+}
+
+}  // namespace
+
+std::vector<chainerx::Array> ElementWiseNvrtcOp::RunImpl(ChxVMState* st, const std::vector<chainerx::Array>& orig_inputs) {
+    CHECK(!orig_inputs.empty());
+    chainerx::Shape shape = orig_inputs[0].shape();
+    for (const chainerx::Array& input : orig_inputs) shape = chainerx::internal::BroadcastShapes(shape, input.shape());
+    const std::vector<chainerx::Dtype> dtypes = OutputDtypes(code);
+    CHECK_EQ(static_cast<size_t>(num_outputs), dtypes.size()) << "fusion program declares a different number of outputs";
+
+    // channels-last operands give channels-last results, so chains between convolutions never transpose
+    bool channels_last = shape.size() == 4;
+    for (const chainerx::Array& input : orig_inputs)
+        if (input.shape() == shape && (input.IsContiguous() || input.strides()[1] != input.GetItemSize())) channels_last = false;
+
+    std::vector<chainerx::Array> outputs;
+    std::vector<chx_hip_tensor> in_desc, out_desc;
+    for (const chainerx::Array& input : orig_inputs) in_desc.push_back(input.hip());
+    for (int i = 0; i < num_outputs; ++i) {
+        outputs.push_back(channels_last ? chainerx::EmptyChannelsLast(shape, dtypes[i]) : chainerx::Empty(shape, dtypes[i]));
+        out_desc.push_back(outputs.back().hip());
+    }
+    std::vector<const chx_hip_tensor*> in_ptr;
+    std::vector<chx_hip_tensor*> out_ptr;
+    for (chx_hip_tensor& t : in_desc) in_ptr.push_back(&t);
+    for (chx_hip_tensor& t : out_desc) out_ptr.push_back(&t);
+    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), fusion_id, in_ptr.data(), static_cast<int32_t>(in_ptr.size()), out_ptr.data(),
+                                       static_cast<int32_t>(out_ptr.size()), nullptr));
+    return outputs;
+}
+
+}  // namespace runtime
+}  // namespace chainer_compiler

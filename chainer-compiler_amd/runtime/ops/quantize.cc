@@ -1,0 +1,144 @@
+// RunImpl bodies of the quantized ops on the hip backend: the signatures of
+// runtime/ops/quantize.cc:48-146 of the chainer-compiler tree, each body a shape inference, an
+// output allocation and one call into the C ABI (include/chx_hip.h).
+#include "../chainerx_util.h"
+#include "../gen/gen_chxvm_ops.h"
+
+namespace chainer_compiler {
+namespace runtime {
+
+namespace {
+
+StrictScalar DefaultZeroPoint() {
+    // an absent zero point is uint8 0 (runtime/ops/quantize.cc:50-51,57-58)
+    return StrictScalar(chainerx::Dtype::kUInt8, chainerx::Scalar(0u), false);
+}
+
+void CheckQuantizedDtype(chainerx::Dtype dt, const char* what) {
+    CHECK(dt == chainerx::Dtype::kUInt8 || dt == chainerx::Dtype::kInt8) << what << " must be uint8 or int8, got " << dt;
+}
+
+// outputs follow the input's layout: channels-last in, channels-last out
+chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& shape, chainerx::Dtype dtype) {
+    const bool channels_last = x.ndim() == 4 && !x.IsContiguous() && x.strides()[1] == x.GetItemSize();
+    return channels_last ? chainerx::EmptyChannelsLast(shape, dtype) : chainerx::Empty(shape, dtype);
+}
+
+}  // namespace
+
+chainerx::Array QuantizeLinearOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& x, const StrictScalar& y_scale, const absl::optional<StrictScalar>& y_zero_point_opt) {
+    const StrictScalar y_zero_point = y_zero_point_opt.has_value() ? *y_zero_point_opt : DefaultZeroPoint();
+    CheckQuantizedDtype(y_zero_point.dtype(), "QuantizeLinear zero point");  // CHECK_EQ(kUInt8, ...), quantize.cc:24
+    chainerx::Array y = EmptyLike4d(x, x.shape(), y_zero_point.dtype());
+    chx_hip_tensor xt = x.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_quantize_linear(&xt, static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)),
+                                           CHX_HIP_ROUND_REFERENCE, &yt, nullptr));
+    return y;
+}
+
+chainerx::Array DequantizeLinearOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& x, const StrictScalar& x_scale, const absl::optional<StrictScalar>& x_zero_point_opt) {
+    const StrictScalar x_zero_point = x_zero_point_opt.has_value() ? *x_zero_point_opt : DefaultZeroPoint();
+    chainerx::Array y = EmptyLike4d(x, x.shape(), chainerx::Dtype::kFloat32);
+    chx_hip_tensor xt = x.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_dequantize_linear(&xt, static_cast<float>(x_scale),
+                                             static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &yt, nullptr));
+    return y;
+}
+
+// Per-instruction state: the plan holds the weights repacked for the MFMA kernel.  The
+// reference re-dequantizes the weights on every call (quantize.cc:76-88); an op object lives as
+// long as the program, so the repacking is done once.
+class QLinearConvOp::QLinearConvImpl {
+public:
+    chx_hip_qconv_plan* plan = nullptr;
+    chx_hip_conv_params params;
+    void* w_data = nullptr;
+};
+
+void QLinearConvOp::InitImpl() {
+    impl_ = new QLinearConvImpl();
+}
+
+QLinearConvOp::~QLinearConvOp() {
+    if (impl_) chx_hip_qconv_plan_destroy(impl_->plan);
+    delete impl_;
+}
+
+chainerx::Array QLinearConvOp::RunImpl(
+        ChxVMState* st,
+        const chainerx::Array& q_x,
+        const StrictScalar& x_scale,
+        const StrictScalar& x_zero_point,
+        const chainerx::Array& q_w,
+        const chainerx::Array& w_scale,
+        const chainerx::Array& w_zero_point,
+        const StrictScalar& y_scale,
+        const StrictScalar& y_zero_point,
+        const absl::optional<chainerx::Array>& b) {
+    CHECK_EQ(w_scale.GetTotalSize(), w_zero_point.GetTotalSize());
+    CHECK_EQ(w_scale.shape().size(), w_zero_point.shape().size());
+    CheckQuantizedDtype(y_zero_point.dtype(), "QLinearConv y_zero_point");
+    const chx_hip_conv_params p = MakeConvParams(q_x, q_w, strides, pads, group, auto_pad);
+    // the plan is keyed on the weight array and the completed attributes; both are constants
+    // of the instruction in every program the compiler emits
+    if (impl_->plan && (impl_->w_data != q_w.raw_data() || memcmp(&impl_->params, &p, sizeof(p)) != 0)) {
+        chx_hip_qconv_plan_destroy(impl_->plan);
+        impl_->plan = nullptr;
+    }
+    if (!impl_->plan) {
+        chx_hip_tensor wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), bt;
+        if (b.has_value()) bt = b->hip();
+        CHXVM_HIP_CALL(chx_hip_qconv_plan_create(&wt, &st2, &zt, b.has_value() ? &bt : nullptr, &p, nullptr, &impl_->plan));
+        impl_->params = p;
+        impl_->w_data = q_w.raw_data();
+    }
+    chainerx::Array y = EmptyLike4d(q_x, ConvOutputShape(q_x, q_w, p), y_zero_point.dtype());
+    chx_hip_tensor xt = q_x.hip(), yt = y.hip();
+    // the reference hands the raw bias to the fp32 convolution (quantize.cc:93)
+    CHXVM_HIP_CALL(chx_hip_qconv_plan_run(
+            impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
+            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)),
+            CHX_HIP_ROUND_REFERENCE | CHX_HIP_BIAS_REFERENCE_FLOAT, &yt, nullptr));
+    return y;
+}
+
+chainerx::Array MatMulIntegerOp::RunImpl(
+        ChxVMState* st,
+        const chainerx::Array& q_a,
+        const chainerx::Array& q_b,
+        const absl::optional<chainerx::Array>& a_zero_point,
+        const absl::optional<chainerx::Array>& b_zero_point) {
+    if (a_zero_point.has_value()) CHECK_GE(1, a_zero_point->shape().size());
+    if (b_zero_point.has_value()) CHECK_GE(1, b_zero_point->shape().size());
+    CHECK_LE(2, q_a.ndim());
+    CHECK_EQ(q_a.ndim(), q_b.ndim()) << "MatMulInteger operands must have the same rank on the hip backend";
+    chainerx::Shape shape(q_a.shape().begin(), q_a.shape().end() - 1);
+    shape.push_back(q_b.shape()[q_b.ndim() - 1]);
+    chainerx::Array y = chainerx::Empty(shape, chainerx::Dtype::kInt32);
+    chx_hip_tensor at = q_a.hip(), bt = q_b.hip(), yt = y.hip(), azt, bzt;
+    if (a_zero_point.has_value()) azt = a_zero_point->hip();
+    if (b_zero_point.has_value()) bzt = b_zero_point->hip();
+    CHXVM_HIP_CALL(chx_hip_matmul_integer(&at, &bt, a_zero_point.has_value() ? &azt : nullptr,
+                                          b_zero_point.has_value() ? &bzt : nullptr, &yt, nullptr));
+    return y;
+}
+
+chainerx::Array ConvIntegerOp::RunImpl(
+        ChxVMState* st,
+        const chainerx::Array& q_x,
+        const chainerx::Array& q_w,
+        const absl::optional<StrictScalar>& x_zero_point,
+        const absl::optional<chainerx::Array>& w_zero_point_opt) {
+    const chx_hip_conv_params p = MakeConvParams(q_x, q_w, strides, pads, group, auto_pad);
+    chainerx::Array y = EmptyLike4d(q_x, ConvOutputShape(q_x, q_w, p), chainerx::Dtype::kInt32);
+    chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), yt = y.hip(), zt;
+    if (w_zero_point_opt.has_value()) zt = w_zero_point_opt->hip();
+    const int32_t xz = x_zero_point.has_value() ? static_cast<int32_t>(static_cast<int64_t>(*x_zero_point)) : 0;
+    CHXVM_HIP_CALL(chx_hip_conv_integer(&xt, &wt, xz, w_zero_point_opt.has_value() ? &zt : nullptr, &p, &yt, nullptr));
+    return y;
+}
+
+}  // namespace runtime
+}  // namespace chainer_compiler

@@ -1,0 +1,202 @@
+"""Serialized ChxVM programs run by the C++ VM of the hip runtime (proto reader -> generated op
+classes -> RunImpl bodies -> C ABI), compared with the CPU oracle: bit-exact for the 8-bit and
+int32 results, and for the fused fp32 chain (the device code restates the host libm bit for bit;
+the stated bar is 2 ulp or 1e-6 relative)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+@pytest.fixture(scope="module")
+def vm(g):
+    from importlib import import_module
+    return import_module(g.pkg.__name__ + ".chxvm")
+
+
+def rand_q(rng, shape, dtype):
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    return rng.integers(lo, hi, size=shape).astype(dtype)
+
+
+def test_quantize_dequantize_program(g, vm, oracle):
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (3, 5, 7))
+    s = b.scalar(0.037, "float32")
+    z = b.scalar(131, "uint8")
+    q = b.QuantizeLinear(x, s, z)
+    d = b.DequantizeLinear(q, s, z)
+    q0 = b.QuantizeLinear(x, s, None)          # absent zero point: uint8 0
+    b.output("q", q)
+    b.output("d", d)
+    b.output("q0", q0)
+    prog = vm.Program(b.serialize())
+    assert prog.num_instructions == 9 and prog.input_names == ["x"]
+    rng = np.random.default_rng(3)
+    xv = (rng.standard_normal((3, 5, 7)) * 3).astype(np.float32)
+    out = prog.run({"x": g.dev(xv)})
+    want_q = oracle.quantize_linear(xv, np.float32(0.037), 131, np.uint8)
+    np.testing.assert_array_equal(out["q"], want_q)
+    np.testing.assert_array_equal(out["d"].view(np.int32), oracle.dequantize_linear(want_q, np.float32(0.037), 131).view(np.int32))
+    np.testing.assert_array_equal(out["q0"], oracle.quantize_linear(xv, np.float32(0.037), 0, np.uint8))
+    assert out["q"].dtype == np.uint8 and out["d"].dtype == np.float32
+    # a second run of the same program object gives the same values
+    np.testing.assert_array_equal(prog.run({"x": g.dev(xv)})["q"], want_q)
+
+
+def test_int8_zero_point_selects_int8_output(g, vm, oracle):
+    b = vm.ProgramBuilder()
+    x = b.input("x")
+    q = b.QuantizeLinear(x, b.scalar(0.5, "float32"), b.scalar(-7, "int8"))
+    b.output("q", q)
+    xv = np.linspace(-80, 80, 1001).astype(np.float32)
+    out = vm.Program(b.serialize()).run({"x": g.dev(xv)})
+    assert out["q"].dtype == np.int8
+    np.testing.assert_array_equal(out["q"], oracle.quantize_linear(xv, np.float32(0.5), -7, np.int8))
+
+
+@pytest.mark.parametrize("auto_pad,pads,strides", [("", [1, 1], [1, 1]), ("SAME_UPPER", [], [2, 2]), ("", [], [])])
+def test_qlinear_conv_program(g, vm, oracle, auto_pad, pads, strides):
+    """In -> QuantizeLinear -> QLinearConv (constants as instructions, bias added the reference's
+    way) -> DequantizeLinear -> Out, twice through the same program (the plan is built once)."""
+    rng = np.random.default_rng(11)
+    N, C, H, W, OC = 2, 16, 9, 10, 24
+    w = rng.integers(-127, 128, size=(OC, C, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-5, 6, size=OC).astype(np.int32)
+    xs, xz, ys, yz = np.float32(0.02), 128, np.float32(0.11), 120
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (N, C, H, W))
+    s_x, z_x = b.scalar(float(xs), "float32"), b.scalar(xz, "uint8")
+    q = b.QuantizeLinear(x, s_x, z_x)
+    y = b.QLinearConv(q, s_x, z_x, b.constant(w), b.constant(ws), b.constant(wz), b.scalar(float(ys), "float32"),
+                      b.scalar(yz, "uint8"), b.constant(bias), strides, pads, 1, auto_pad)
+    d = b.DequantizeLinear(y, b.scalar(float(ys), "float32"), b.scalar(yz, "uint8"))
+    b.Free(q)
+    b.output("y", y)
+    b.output("d", d)
+    prog = vm.Program(b.serialize())
+    for seed in (0, 1):
+        xv = np.random.default_rng(seed).uniform(-2.5, 2.5, size=(N, C, H, W)).astype(np.float32)
+        out = prog.run({"x": g.dev(xv)})
+        qx = oracle.quantize_linear(xv, xs, xz, np.uint8)
+        want = oracle.qlinear_conv_int(qx, xs, xz, w, ws, wz, ys, yz, np.uint8, bias=bias,
+                                       bias_mode=oracle.BIAS_REFERENCE_FLOAT, strides=tuple(strides) or (1, 1),
+                                       pads=tuple(pads) or (0, 0), auto_pad=auto_pad)
+        np.testing.assert_array_equal(out["y"], want)
+        assert want.min() < want.max()
+        np.testing.assert_array_equal(out["d"].view(np.int32), oracle.dequantize_linear(want, ys, yz).view(np.int32))
+
+
+def test_qlinear_conv_onnx_vector_through_vm(g, vm, onnx_vectors):
+    t = onnx_vectors["test_qlinearconv"]
+    b = vm.ProgramBuilder()
+    x = b.input("x", "uint8", t["x_shape"])
+    y = b.QLinearConv(x, b.scalar(t["x_scale"], "float32"), b.scalar(t["x_zero_point"], "uint8"),
+                      b.constant(np.array(t["w"], np.uint8).reshape(t["w_shape"])),
+                      b.constant(np.array(t["w_scale"], np.float32)), b.constant(np.array(t["w_zero_point"], np.uint8)),
+                      b.scalar(t["y_scale"], "float32"), b.scalar(t["y_zero_point"], "uint8"), None, [], [], 1, "")
+    b.output("y", y)
+    out = vm.Program(b.serialize()).run({"x": g.dev(np.array(t["x"], np.uint8).reshape(t["x_shape"]))})
+    assert out["y"].reshape(7, 7).tolist() == t["y"]
+
+
+def test_conv_integer_and_matmul_integer_programs(g, vm, oracle, onnx_vectors):
+    rng = np.random.default_rng(5)
+    x, w = rand_q(rng, (2, 6, 9, 8), np.uint8), rand_q(rng, (4, 3, 3, 2), np.int8)
+    wz = rand_q(rng, (4,), np.int8)
+    b = vm.ProgramBuilder()
+    xi = b.input("x", "uint8", x.shape)
+    y = b.ConvInteger(xi, b.constant(w), b.scalar(77, "uint8"), b.constant(wz), [2, 1], [0, 1], 2, "")
+    y2 = b.ConvInteger(xi, b.constant(w), None, None, [2, 1], [0, 1], 2, "")
+    b.output("y", y)
+    b.output("y2", y2)
+    out = vm.Program(b.serialize()).run({"x": g.dev(x)})
+    np.testing.assert_array_equal(out["y"], oracle.conv_integer(x, w, 77, wz, strides=(2, 1), pads=(0, 1), group=2))
+    np.testing.assert_array_equal(out["y2"], oracle.conv_integer(x, w, None, None, strides=(2, 1), pads=(0, 1), group=2))
+    assert out["y"].dtype == np.int32
+
+    t = onnx_vectors["test_matmulinteger"]
+    b = vm.ProgramBuilder()
+    a, bb = b.input("a", "uint8"), b.input("b", "uint8")
+    y = b.MatMulInteger(a, bb, b.constant(np.array([t["a_zero_point"]], np.uint8)),
+                        b.constant(np.array([t["b_zero_point"]], np.uint8)))
+    b.output("y", y)
+    out = vm.Program(b.serialize()).run({"a": g.dev(np.array(t["a"], np.uint8)), "b": g.dev(np.array(t["b"], np.uint8))})
+    assert out["y"].tolist() == t["y"]
+    a_, b_ = rand_q(rng, (3, 5, 37), np.uint8), rand_q(rng, (3, 37, 11), np.int8)
+    b = vm.ProgramBuilder()
+    y = b.MatMulInteger(b.input("a", "uint8"), b.input("b", "int8"), None, None)
+    b.output("y", y)
+    out = vm.Program(b.serialize()).run({"a": g.dev(a_), "b": g.dev(b_)})
+    np.testing.assert_array_equal(out["y"], oracle.matmul_integer(a_, b_, None, None))
+
+
+def test_fusion_group_program(g, vm, oracle):
+    """ElementWiseNvrtc with the chain Mul, Add, Tanh, Sigmoid, Mul, Add, Relu and broadcast
+    [C] operands; two outputs."""
+    chain = [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "t2"),
+             ("t4", "Mul", "t3", "x"), ("t5", "Add", "t4", "c"), ("y", "Relu", "t5")]
+    code = g.ops.fusion_program(
+        [("x", torch.float32), ("a", torch.float32), ("b", torch.float32), ("c", torch.float32)], chain,
+        [("y", torch.float32), ("t2", torch.float32)])
+    b = vm.ProgramBuilder()
+    ins = [b.input(n) for n in ("x", "a", "b", "c")]
+    y, t2 = b.ElementWiseNvrtc(ins, 2, code, 3, num_list_outputs=2)
+    b.output("y", y)
+    b.output("t2", t2)
+    prog = vm.Program(b.serialize())
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((4, 33, 65)).astype(np.float32) * 2
+    a, bb = rng.standard_normal(65).astype(np.float32), rng.standard_normal(65).astype(np.float32)
+    c = rng.standard_normal((4, 33, 65)).astype(np.float32)
+    out = prog.run({"x": g.dev(x), "a": g.dev(a), "b": g.dev(bb), "c": g.dev(c)})
+    env = oracle.run_chain(chain, {"x": x, "a": a, "b": bb, "c": c})
+    t2w, yw = env["t2"], env["y"]
+    # bar: 2 ulp or 1e-6 relative; the device code is written to give 0
+    assert g.ulp_diff(out["t2"], t2w).max() == 0
+    assert g.ulp_diff(out["y"], yw).max() == 0
+
+
+def test_null_operand_skips_the_op(g, vm):
+    """An op with a null array operand is skipped and its outputs become null
+    (runtime/gen_chxvm.py:240-253); reading such an output as an array fails."""
+    b = vm.ProgramBuilder()
+    n = b.NullConstant()
+    q = b.QuantizeLinear(n, b.scalar(1.0, "float32"), None)
+    i = b.new_slot()
+    b.add("Identity", q, outputs=[i])
+    b.output("q", i)
+    prog = vm.Program(b.serialize())
+    with pytest.raises(vm.ChxVMError):
+        prog.run({})
+
+
+def test_errors_name_the_instruction(g, vm):
+    b = vm.ProgramBuilder()
+    x = b.input("x")
+    b.output("y", b.QuantizeLinear(x, b.scalar(1.0, "float32"), b.scalar(3, "int32"), debug_info="node quant0"))
+    prog = vm.Program(b.serialize())
+    with pytest.raises(vm.ChxVMError) as e:
+        prog.run({"x": g.dev(np.zeros(4, np.float32))})
+    assert "uint8 or int8" in str(e.value)
+    with pytest.raises(vm.ChxVMError) as e:
+        prog.run({})
+    assert "Input 'x' not found" in str(e.value)
+    # writing a slot twice is refused (runtime/chxvm_state.cc:171-176)
+    b = vm.ProgramBuilder()
+    x = b.input("x")
+    s = b.scalar(1.0, "float32")
+    q = b.QuantizeLinear(x, s, None)
+    b.add("QuantizeLinear", x, s, -1, outputs=[q])
+    with pytest.raises(vm.ChxVMError):
+        vm.Program(b.serialize()).run({"x": g.dev(np.zeros(4, np.float32))})
