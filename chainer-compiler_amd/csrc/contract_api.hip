@@ -411,6 +411,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.bias = c.bias;
     a.rq = c.rq;
     a.inv_y_scale = c.out_int32 ? 0.f : 1.0f / c.rq.q.scale;
+    a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64;
     pick_tile(cs.OC, a.M, &toc, &tpx);

@@ -31,7 +31,8 @@ struct ConvMfmaArgs {
     int32_t w_scale_len;
     const int32_t* bias;
     RequantParams rq;
-    float inv_y_scale;           // 1 / y_scale, for the guarded fast requantization
+    float inv_y_scale;           // 1 / y_scale, for the division-free requantization
+    float lo_folded;             // lower clamp bound with the fused Relu folded in (fold_relu_floor)
     int32_t tiles_oc, tiles_px;  // filled by the launcher
 };
 

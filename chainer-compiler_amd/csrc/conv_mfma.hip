@@ -26,6 +26,8 @@
 // channels at a time, transposed through LDS into [pixel][oc] rows and written as
 // 128-bit stores to the channels-last output.  With an int32 output (ConvInteger,
 // MatMulInteger) the accumulators are stored directly.
+#include <type_traits>
+
 #include "contract.h"
 #include "conv_mfma.h"
 
@@ -34,6 +36,7 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kBK = 64;  // K bytes per step
 
@@ -148,37 +151,82 @@ __device__ __forceinline__ int lds_chunk_offset(int row, int kc) {
     return row * kBK + ((kc ^ ((row >> 2) & 3)) << 4);
 }
 
+// Row b (64 bytes) holds the byte b in every position.  A filter tap outside the image fetches
+// the row of the activation zero point, so padding needs no data-dependent fix-up.
+#define CHX_B16(v) v, v, v, v, v, v, v, v, v, v, v, v, v, v, v, v
+#define CHX_ROW(v) CHX_B16(v), CHX_B16(v), CHX_B16(v), CHX_B16(v)
+#define CHX_ROWS16(h)                                                                                     \
+    CHX_ROW((h) * 16 + 0), CHX_ROW((h) * 16 + 1), CHX_ROW((h) * 16 + 2), CHX_ROW((h) * 16 + 3),           \
+    CHX_ROW((h) * 16 + 4), CHX_ROW((h) * 16 + 5), CHX_ROW((h) * 16 + 6), CHX_ROW((h) * 16 + 7),           \
+    CHX_ROW((h) * 16 + 8), CHX_ROW((h) * 16 + 9), CHX_ROW((h) * 16 + 10), CHX_ROW((h) * 16 + 11),         \
+    CHX_ROW((h) * 16 + 12), CHX_ROW((h) * 16 + 13), CHX_ROW((h) * 16 + 14), CHX_ROW((h) * 16 + 15)
+__device__ __attribute__((aligned(64))) const unsigned char g_fill_rows[256 * 64] = {
+        CHX_ROWS16(0), CHX_ROWS16(1), CHX_ROWS16(2),  CHX_ROWS16(3),  CHX_ROWS16(4),  CHX_ROWS16(5),  CHX_ROWS16(6),  CHX_ROWS16(7),
+        CHX_ROWS16(8), CHX_ROWS16(9), CHX_ROWS16(10), CHX_ROWS16(11), CHX_ROWS16(12), CHX_ROWS16(13), CHX_ROWS16(14), CHX_ROWS16(15)};
+#undef CHX_ROWS16
+#undef CHX_ROW
+#undef CHX_B16
+
+// Asynchronous copy of 16 bytes per lane from global memory straight into LDS: lane i of the
+// wavefront writes LDS bytes [lds_addr + 16*i, lds_addr + 16*i + 16).  lds_addr must be the
+// same for all lanes (it travels in M0).  Completion is tracked by the wave's vector-memory
+// counter like any load; nothing passes through registers.
+__device__ __forceinline__ void async_copy16(const void* src, uint32_t lds_addr) {
+    asm volatile(
+            "s_mov_b32 m0, %1\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, off"
+            :
+            : "v"(src), "s"(lds_addr)
+            : "memory", "m0");
+}
+
+// Wait until at most N of this wave's vector-memory operations are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 // FM x FN MFMA tiles (32x32) per wavefront; four wavefronts in a 2x2 grid per work-group.
 // Tile = (64*FM) output channels x (64*FN) pixels.
 //
 // Work-groups are persistent: each owns one output-channel tile and walks over pixel tiles
 // px_first, px_first + px_step, ...  The sequence of (pixel tile, K step) pairs is one flat
-// pipeline: global loads run D steps ahead of the MFMAs and cross tile boundaries, so the
-// loads of the next tile are in flight while the current tile is finished and written out.
+// pipeline over a ring of NS LDS stages: the asynchronous copies run NS-1 steps ahead of the
+// MFMAs and cross tile boundaries, so the operands of the next tile are in flight while the
+// current tile is requantized and written out.  Per K step a wave issues FM + FN copy
+// instructions, reads its fragments back with 128-bit LDS loads, flips the sign bits of uint8
+// activations on the fragments, and feeds 2*FM*FN MFMAs; one barrier per step.
+//
+// LDS stage: rows of 64 K-bytes, weight rows first, then pixel rows.  A copy instruction fills
+// 1 KB = 16 consecutive rows; lane l lands in row l/4, slot l%4 and therefore fetches K chunk
+// (l%4) ^ ((l/16)%4) of that row, which is the XOR swizzle lds_chunk_offset() undoes on the
+// read side (bank-conflict-free 128-bit fragment reads).
 //
 // kPad: some filter tap can fall outside the image, or the channel count is not a multiple
 // of 64.  Then each staged row carries a bit mask of its valid taps (computed once per pixel
-// tile) and invalid chunks are replaced by the zero point on their way into LDS.  Without
-// kPad (1x1 and other unpadded convolutions on 64-multiple channels, matrix products) every
-// load is valid and the per-step work on the vector ALU is one address add and the sign flip.
+// tile) and an invalid chunk is fetched from a 64-byte row holding the zero point instead
+// (g_fill_rows), which makes it contribute (zp - zp) * w = 0.  Without kPad (1x1 and other
+// unpadded convolutions on 64-multiple channels, matrix products) every chunk is valid.
 template <int FM, int FN, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv_mfma_kernel(ConvMfmaArgs a) {
     constexpr int T = 256;
     constexpr int TM = 64 * FM;  // output channels per tile
     constexpr int TN = 64 * FN;  // pixels per tile
-    constexpr int D = 3;         // K steps in flight between global memory and LDS
+    constexpr int NS = 3;        // LDS stages
     constexpr int STAGE_BYTES = (TM + TN) * kBK;
+    constexpr int COPIES = FM + FN;     // copy instructions per wave and stage
     constexpr int OUT_PITCH = TM + 16;  // staging row pitch in bytes, keeps 16-byte alignment
     constexpr int LDS_OUT = kOutInt32 ? 16 : TN * OUT_PITCH;
-    __shared__ __attribute__((aligned(16))) char lds[2 * STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) char lds_out[LDS_OUT];
-    __shared__ float s_scale[TM];
-    __shared__ int32_t s_add[TM];
-    __shared__ float s_fbias[TM];
+    __shared__ __attribute__((aligned(16))) float s_scale[TM];
+    __shared__ __attribute__((aligned(16))) int32_t s_add[TM];
+    __shared__ __attribute__((aligned(16))) float s_fbias[TM];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
     // Work-group ids go round-robin over the 8 XCDs, each with its own L2.  Every XCD gets one
@@ -198,40 +246,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     const int my_tiles = px_first < px_hi ? (px_hi - px_first + px_step - 1) / px_step : 0;
     const int nk = a.nk;
     const int total_stages = my_tiles * nk;
+    if (total_stages == 0) return;
 
-    // per-channel epilogue constants
-    for (int i = tid; i < TM; i += T) {
-        const int oc = oc0 + i;
-        float sc = 0.f, fb = 0.f;
-        int32_t add = 0;
-        if (oc < a.OC) {
-            add = a.corr_mult * a.wsum[oc];
-            if (!kOutInt32) {
-                const float wsc = a.w_scale_len > 1 ? a.w_scale[oc] : a.w_scale[0];
-                sc = a.rq.x_scale * wsc;
-                if (a.bias) {
-                    if (a.rq.bias_mode == kBiasOnnxInt32) add += a.bias[oc];
-                    if (a.rq.bias_mode == kBiasReferenceFloat) fb = (float)a.bias[oc];
-                }
-            }
-        }
-        s_scale[i] = sc;
-        s_add[i] = add;
-        s_fbias[i] = fb;
-    }
-
-    // chunks this thread stages per K step: FM of the weight tile, FN of the activation tile;
-    // chunk q = tid + j*256 -> row q/4, 16-byte K chunk q%4
-    const int kc = tid & 3;
-    const int row0 = tid >> 2;  // rows row0 + 64*j
+    // rows this thread copies per stage: row0 + 64*j of the weight tile and of the pixel tile,
+    // K chunk kc of each
+    const int row0 = tid >> 2;
+    const int kc = (lane & 3) ^ ((lane >> 4) & 3);
     const int8_t* wp_row[FM];
 #pragma unroll
     for (int j = 0; j < FM; ++j) wp_row[j] = a.wp + (int64_t)(oc0 + row0 + 64 * j) * a.KP + kc * 16;
+    const char* fill_src = reinterpret_cast<const char*>(g_fill_rows) + (a.x_zp & 0xff) * 64 + kc * 16;
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)ring + (uint32_t)wave * 1024u;  // LDS byte address
 
-    const int fill_byte = kXUnsigned ? ((a.x_zp ^ 0x80) & 0xff) : (a.x_zp & 0xff);
-    const int fill_word = (int)((unsigned)fill_byte * 0x01010101u);
-
-    // ---- load side state: which (pixel tile, K step) the next global load fetches ----
+    // ---- copy side state: which (pixel tile, K step) the next stage fetches ----
     const char* xb[FN];
     int ld_tile = px_first;
     int ld_k = 0, kh = 0, kw = 0, c0 = 0, kofs = 0;
@@ -269,31 +296,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     };
     set_load_tile();
 
-    // Loads are unconditional (an invalid chunk reads the tensor's first bytes instead) and
-    // nothing consumes a loaded value here; the fill value and the sign flip are applied when
-    // the stage is written to LDS, several K steps later, so the loads stay in flight.
-    auto load_global = [&](v4i* pa, v4i* pb, uint32_t& okmask) {
+    // Every stage issues the same number of copies and none is conditional, so a fixed
+    // vector-memory count identifies the stage about to be consumed.  Stages past the end of
+    // this work-group's list re-read the last K step into a ring slot nobody reads again.
+    auto issue_stage = [&](int buf) {
+        const uint32_t dst = ring_addr + (uint32_t)buf * STAGE_BYTES;
 #pragma unroll
-        for (int j = 0; j < FM; ++j) pa[j] = *reinterpret_cast<const v4i*>(wp_row[j] + kofs);
-        okmask = 0;
+        for (int j = 0; j < FM; ++j) async_copy16(wp_row[j] + kofs, dst + j * 4096);
         if (kPad) {
             const bool c_ok = c0 + kc * 16 < a.C16;
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const bool ok = c_ok && ((tapmask[j] >> tap) & 1u);
-                const char* src = ok ? xb[j] + tap_off + c0 : a.x;
-                pb[j] = *reinterpret_cast<const v4i*>(src);
-                okmask |= (ok ? 1u : 0u) << j;
+                async_copy16(ok ? xb[j] + tap_off + c0 : fill_src, dst + TM * kBK + j * 4096);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < FN; ++j) pb[j] = *reinterpret_cast<const v4i*>(xb[j] + tap_off + c0);
+            for (int j = 0; j < FN; ++j) async_copy16(xb[j] + tap_off + c0, dst + TM * kBK + j * 4096);
         }
         // advance to the next K step, or to the first K step of this work-group's next pixel tile
         if (++ld_k == nk) {
-            ld_k = 0; kh = 0; kw = 0; c0 = 0; kofs = 0; tap_off = 0; tap = 0;
-            ld_tile += px_step;
-            set_load_tile();
+            if (ld_tile + px_step < px_hi) {
+                ld_k = 0; kh = 0; kw = 0; c0 = 0; kofs = 0; tap_off = 0; tap = 0;
+                ld_tile += px_step;
+                set_load_tile();
+            } else {
+                --ld_k;  // nothing follows: keep fetching the last step
+            }
         } else {
             kofs += kBK;
             c0 += kBK;
@@ -309,40 +338,51 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             }
         }
     };
-    auto store_lds = [&](int buf, const v4i* pa, const v4i* pb, uint32_t okmask) {
-        char* sa = lds + buf * STAGE_BYTES;
-        char* sb = sa + TM * kBK;
-#pragma unroll
-        for (int j = 0; j < FM; ++j) *reinterpret_cast<v4i*>(sa + lds_chunk_offset(row0 + 64 * j, kc)) = pa[j];
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            v4i v = pb[j];
-            if (kXUnsigned) v ^= (int)0x80808080;
-            if (kPad) {
-                const bool ok = (okmask >> j) & 1u;
-                v[0] = ok ? v[0] : fill_word;
-                v[1] = ok ? v[1] : fill_word;
-                v[2] = ok ? v[2] : fill_word;
-                v[3] = ok ? v[3] : fill_word;
-            }
-            *reinterpret_cast<v4i*>(sb + lds_chunk_offset(row0 + 64 * j, kc)) = v;
-        }
-    };
 
+    // the first NS-1 stages go out before anything else touches memory
+#pragma unroll
+    for (int d = 0; d < NS - 1; ++d) issue_stage(d);
+
+    // per-channel epilogue constants; s_add seeds the accumulators
+    for (int i = tid; i < TM; i += T) {
+        const int oc = oc0 + i;
+        float sc = 0.f, fb = 0.f;
+        int32_t add = 0;
+        if (oc < a.OC) {
+            add = a.corr_mult * a.wsum[oc];
+            if (!kOutInt32) {
+                const float wsc = a.w_scale_len > 1 ? a.w_scale[oc] : a.w_scale[0];
+                sc = a.rq.x_scale * wsc;
+                if (a.bias) {
+                    if (a.rq.bias_mode == kBiasOnnxInt32) add += a.bias[oc];
+                    if (a.rq.bias_mode == kBiasReferenceFloat) fb = (float)a.bias[oc];
+                }
+            }
+        }
+        s_scale[i] = sc;
+        s_add[i] = add;
+        s_fbias[i] = fb;
+    }
+    __syncthreads();
+
+    // lane holds, per 32x32 MFMA tile: pixel column (lane & 31), output-channel rows
+    // (v / 4) * 8 + (lane >> 5) * 4 + (v % 4)
     v16i acc[FM][FN];
-    auto zero_acc = [&]() {
+    auto seed_acc = [&]() {
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+            for (int g = 0; g < 4; ++g) {
+                const v4i ad = *reinterpret_cast<const v4i*>(&s_add[wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4]);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] = ad[e];
+            }
     };
-    zero_acc();
+    seed_acc();
 
     // ---- epilogue of one finished pixel tile ----
-    // lane holds, per 32x32 MFMA tile: pixel column (lane & 31), output-channel rows
-    // (v / 4) * 8 + (lane >> 5) * 4 + (v % 4)
     auto epilogue = [&](int px_tile) {
         const int64_t m0 = (int64_t)px_tile * TN;
         if (kOutInt32) {
@@ -359,7 +399,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                         const int oc = oc0 + ocl;
                         v4i out;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) out[e] = acc[i][j][g * 4 + e] + s_add[ocl + e];
+                        for (int e = 0; e < 4; ++e) out[e] = acc[i][j][g * 4 + e];
                         if (a.y_vec_ok && oc + 4 <= a.OC) {
                             *reinterpret_cast<v4i*>(yrow + (int64_t)oc * 4) = out;
                         } else {
@@ -371,39 +411,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                 }
             return;
         }
-        const bool float_bias = a.rq.bias_mode == kBiasReferenceFloat;  // uniform
+        // requantize: one instance of the element loop per bias mode (the branch is uniform)
+        auto requantize_tile = [&](auto float_bias_tag) {
+            constexpr bool kFloatBias = decltype(float_bias_tag)::value;
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
-                float sc[4], fb[4];
-                int32_t ad[4];
+                for (int g = 0; g < 4; ++g) {
+                    const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
+                    const v4f sc = *reinterpret_cast<const v4f*>(&s_scale[ocl]);
+                    v4f fb = {0.f, 0.f, 0.f, 0.f};
+                    if (kFloatBias) fb = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    sc[e] = s_scale[ocl + e];
-                    ad[e] = s_add[ocl + e];
-                    fb[e] = float_bias ? s_fbias[ocl + e] : 0.f;
-                }
+                    for (int j = 0; j < FN; ++j) {
+                        const int pxl = wn * 32 * FN + j * 32 + (lane & 31);
+                        int32_t code[4];
 #pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    const int pxl = wn * 32 * FN + j * 32 + (lane & 31);
-                    int32_t code[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int32_t accv = acc[i][j][g * 4 + e] + ad[e];
-                        float v = (float)accv * sc[e];
-                        // the reference adds a float bias after the scale multiply; x + 0.0f
-                        // changes nothing the quantization can see, so no branch is needed
-                        v = v + fb[e];
-                        const int32_t c = quantize_value_fast<kRne>(v, a.rq.q, a.inv_y_scale);
-                        code[e] = c < a.rq.relu_floor ? a.rq.relu_floor : c;
+                        for (int e = 0; e < 4; ++e) {
+                            float v = (float)acc[i][j][g * 4 + e] * sc[e];
+                            if (kFloatBias) v = v + fb[e];  // reference mode: float bias after the scale multiply
+                            code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                        }
+                        *reinterpret_cast<uint32_t*>(lds_out + pxl * OUT_PITCH + ocl) = pack4(code[0], code[1], code[2], code[3]);
                     }
-                    const uint32_t packed = ((uint32_t)code[0] & 0xffu) | (((uint32_t)code[1] & 0xffu) << 8) |
-                                            (((uint32_t)code[2] & 0xffu) << 16) | ((uint32_t)code[3] << 24);
-                    *reinterpret_cast<uint32_t*>(lds_out + pxl * OUT_PITCH + ocl) = packed;
                 }
-            }
+        };
+        if (a.rq.bias_mode == kBiasReferenceFloat) requantize_tile(std::true_type());
+        else requantize_tile(std::false_type());
         __syncthreads();
         constexpr int CHUNKS_PER_ROW = TM / 16;
         for (int q = tid; q < TN * CHUNKS_PER_ROW; q += T) {
@@ -424,63 +458,54 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         }
     };
 
-    if (total_stages == 0) return;
-    v4i ra[D][FM], rb[D][FN];
-    uint32_t okm[D];
-    // Every iteration issues the same number of loads and none of it is conditional, so the
-    // compiler can wait for exactly the stage it is about to store (vmcnt counts in order) and
-    // leave the younger stages in flight.  Iterations past the end (the loop runs a multiple
-    // of D) recompute a finished tile's stale LDS contents into accumulators nobody reads and
-    // load from valid addresses; a tile boundary they reach belongs to no tile of this work-group and is skipped.
-    // prologue: stages 0 .. D-1 in flight, stage 0 into LDS, its registers refilled with stage D
-#pragma unroll
-    for (int d = 0; d < D; ++d) load_global(ra[d], rb[d], okm[d]);
-    store_lds(0, ra[0], rb[0], okm[0]);
-    load_global(ra[0], rb[0], okm[0]);
-    __syncthreads();
-
     const int frag_row = lane & 31;
     const int frag_kc = lane >> 5;
-    int ck = 0;               // K step within the tile being computed
-    int c_tile = px_first;    // pixel tile being computed
-    const int iters = (total_stages + D - 1) / D * D;
-    for (int s0 = 0; s0 < iters; s0 += D) {
+    int ck = 0;             // K step within the tile being computed
+    int c_tile = px_first;  // pixel tile being computed
+    int cbuf = 0;           // ring slot being computed
+    int lbuf = NS - 1;      // ring slot the next copy fills
+    for (int s = 0; s < total_stages; ++s) {
+        // this wave's copies of stage s have landed when at most the NS-2 younger stages are
+        // outstanding; the barrier extends that to every wave's copies, and also says that
+        // everybody is done reading the slot the next copies overwrite
+        wait_vmcnt<(NS - 2) * COPIES>();
+        __syncthreads();
+        issue_stage(lbuf);
+        lbuf = lbuf + 1 == NS ? 0 : lbuf + 1;
+
+        const char* sa = ring + cbuf * STAGE_BYTES;
+        const char* sb = sa + TM * kBK;
+        cbuf = cbuf + 1 == NS ? 0 : cbuf + 1;
+        v4i fa[2][FM], fb[2][FN];
 #pragma unroll
-        for (int u = 0; u < D; ++u) {
-            const int cur = (s0 + u) & 1;
-            const char* sa = lds + cur * STAGE_BYTES;
-            const char* sb = sa + TM * kBK;
-            v4i fa[2][FM], fb[2][FN];
+        for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
+            for (int i = 0; i < FM; ++i)
+                fa[sub][i] = *reinterpret_cast<const v4i*>(
+                        sa + lds_chunk_offset(wm * 32 * FM + i * 32 + frag_row, sub * 2 + frag_kc));
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
-                    fa[sub][i] = *reinterpret_cast<const v4i*>(
-                            sa + lds_chunk_offset(wm * 32 * FM + i * 32 + frag_row, sub * 2 + frag_kc));
+            for (int j = 0; j < FN; ++j) {
+                v4i v = *reinterpret_cast<const v4i*>(
+                        sb + lds_chunk_offset(wn * 32 * FN + j * 32 + frag_row, sub * 2 + frag_kc));
+                if (kXUnsigned) v ^= (int)0x80808080;  // uint8 code - 128 as int8
+                fb[sub][j] = v;
+            }
+        }
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
-                    fb[sub][j] = *reinterpret_cast<const v4i*>(
-                            sb + lds_chunk_offset(wn * 32 * FN + j * 32 + frag_row, sub * 2 + frag_kc));
-            }
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[sub][i], fb[sub][j], acc[i][j], 0, 0, 0);
-            const int nxt = (u + 1) % D;  // register set holding the next stage (static after unrolling)
-            store_lds(cur ^ 1, ra[nxt], rb[nxt], okm[nxt]);
-            load_global(ra[nxt], rb[nxt], okm[nxt]);
-            if (++ck == nk) {
-                if (c_tile < px_hi) epilogue(c_tile);  // iterations past the end own no tile
-                zero_acc();
-                ck = 0;
-                c_tile += px_step;
-            }
-            __syncthreads();
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[sub][i], fb[sub][j], acc[i][j], 0, 0, 0);
+        if (++ck == nk) {
+            epilogue(c_tile);
+            seed_acc();
+            ck = 0;
+            c_tile += px_step;
         }
     }
+    wait_vmcnt<0>();  // the copies past the end still target this work-group's LDS
 }
 
 template <int FM, int FN>

@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <cstdint>
 
 namespace chx {
@@ -71,6 +72,36 @@ __device__ __forceinline__ int32_t quantize_value_fast(float v, const QuantParam
     s = s + q.zpf;
     s = __builtin_fminf(s, q.hi);
     s = __builtin_fmaxf(s, q.lo);
+    s = s + 0.5f;
+    return (int32_t)s;
+}
+
+// The fused Relu (code = max(code, floor), floor = the output zero point) folded into the lower
+// clamp bound: for a floor f >= 0 clamping to max(lo, f) gives f + 0.5 -> f for everything
+// below, and what the truncation makes of values in [f - 0.5, f) is f either way; for f < 0
+// the bound is f - 0.5, which the + 0.5 turns into exactly f, while values in [f - 0.5, f)
+// keep the reference's truncation toward zero.  In ONNX rounding mode the clamp acts on
+// integers and the bound is simply max(lo, f).
+inline float fold_relu_floor(const QuantParams& q, int32_t relu_floor, bool rne) {
+    if (relu_floor == INT32_MIN) return q.lo;
+    const float f = (float)relu_floor;
+    const float bound = (rne || relu_floor >= 0) ? f : f - 0.5f;
+    return bound > q.lo ? bound : q.lo;
+}
+
+// quantize_value_fast with the lower bound of fold_relu_floor and the clamp as one median
+// instruction (the same function as min/max for every non-NaN value).
+template <bool kRne>
+__device__ __forceinline__ int32_t quantize_value_folded(float v, const QuantParams& q, float inv_scale, float lo_folded) {
+    const float q0 = v * inv_scale;
+    const float r = __builtin_fmaf(-q0, q.scale, v);
+    float s = __builtin_fmaf(r, inv_scale, q0);
+    if (kRne) {
+        s = rintf(s) + q.zpf;
+        return (int32_t)__builtin_amdgcn_fmed3f(s, lo_folded, q.hi);
+    }
+    s = s + q.zpf;
+    s = __builtin_amdgcn_fmed3f(s, lo_folded, q.hi);
     s = s + 0.5f;
     return (int32_t)s;
 }
