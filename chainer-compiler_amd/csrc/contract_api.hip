@@ -227,6 +227,74 @@ void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px) {
     }
 }
 
+// Launch configurations measured for the input shapes a plan has seen: the first eager call on
+// a new shape times every tile shape and occupancy cap on the call's own operands (every
+// configuration writes the same bytes) and later calls reuse the fastest.
+struct TunedConfig {
+    int64_t M;
+    int32_t H, W, OH, OW;
+    int tile_oc, tile_px, max_wgs_per_cu;
+};
+struct TuneCache {
+    std::vector<TunedConfig> entries;
+};
+
+bool autotune_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("CHX_HIP_AUTOTUNE");  // CHX_HIP_AUTOTUNE=0 keeps the heuristic
+        return !(e && e[0] == '0') && !getenv("CHX_HIP_TILE");
+    }();
+    return on;
+}
+
+bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;  // when in doubt, do not time
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
+// Times every launch configuration on the call's operands and keeps the fastest in *best.
+int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hipStream_t s, TunedConfig* best) {
+    static const int tiles[4][2] = {{128, 128}, {64, 128}, {128, 64}, {64, 64}};
+    static const int caps[3] = {0, 2, 1};
+    hipEvent_t e0, e1;
+    CHX_HIP_CALL(hipEventCreate(&e0));
+    CHX_HIP_CALL(hipEventCreate(&e1));
+    float best_ms = -1.f;
+    int rc = CHX_HIP_OK;
+    for (int t = 0; t < 4 && rc == CHX_HIP_OK; ++t) {
+        if (a.OC <= 64 && tiles[t][0] > 64) continue;
+        for (int c = 0; c < 3 && rc == CHX_HIP_OK; ++c) {
+            const int reps = 3;
+            rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], xu, out_int32, rne, s);  // warm
+            if (rc != CHX_HIP_OK) break;
+            if (hipEventRecord(e0, s) != hipSuccess) rc = CHX_HIP_ERUNTIME;
+            for (int r = 0; r < reps && rc == CHX_HIP_OK; ++r)
+                rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], xu, out_int32, rne, s);
+            if (rc != CHX_HIP_OK) break;
+            float ms = 0.f;
+            if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                hipEventElapsedTime(&ms, e0, e1) != hipSuccess) {
+                rc = CHX_HIP_ERUNTIME;
+                break;
+            }
+            if (best_ms < 0.f || ms < best_ms) {
+                best_ms = ms;
+                best->tile_oc = tiles[t][0];
+                best->tile_px = tiles[t][1];
+                best->max_wgs_per_cu = caps[c];
+            }
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != CHX_HIP_OK) CHX_FAIL(rc, "timing the convolution launch configurations failed: %s", chx_hip_last_error());
+    return CHX_HIP_OK;
+}
+
 struct XLayout {
     const char* ptr;
     int64_t n_stride, h_stride, w_stride;
@@ -278,6 +346,7 @@ struct ScratchCache {
 };
 
 struct ConvCall {
+    TuneCache* tune;      // null: heuristic tile choice
     ScratchCache* cache;  // null: stream-ordered scratch for this call only
     const chx_hip_tensor* x;
     chx_hip_tensor* y;
@@ -413,9 +482,28 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.inv_y_scale = c.out_int32 ? 0.f : 1.0f / c.rq.q.scale;
     a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
-    int toc = 64, tpx = 64;
+    int toc = 64, tpx = 64, cap = 0;
     pick_tile(cs.OC, a.M, &toc, &tpx);
-    int rc = launch_conv_mfma(a, toc, tpx, xu, c.out_int32, c.rne, s);
+    int rc = CHX_HIP_OK;
+    const TunedConfig* tuned = nullptr;
+    if (c.tune) {
+        for (const TunedConfig& t : c.tune->entries)
+            if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW) tuned = &t;
+        if (!tuned && autotune_enabled() && !stream_is_capturing(s)) {
+            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0};
+            rc = tune_conv_mfma(a, xu, c.out_int32, c.rne, s, &best);
+            if (rc == CHX_HIP_OK) {
+                c.tune->entries.push_back(best);
+                tuned = &c.tune->entries.back();
+            }
+        }
+    }
+    if (tuned) {
+        toc = tuned->tile_oc;
+        tpx = tuned->tile_px;
+        cap = tuned->max_wgs_per_cu;
+    }
+    if (rc == CHX_HIP_OK) rc = launch_conv_mfma(a, toc, tpx, cap, xu, c.out_int32, c.rne, s);
     if (rc == CHX_HIP_OK && y_post) {
         rc = launch_nhwc_to_nchw_u8(static_cast<const char*>(y_scratch), static_cast<char*>(y.data), cs.N, cs.OC,
                                     (int64_t)cs.OH * cs.OW, (int)a.y_px_stride, s);
@@ -535,6 +623,7 @@ ConvCall conv_call_from(const QConvChecked& q, const chx_hip_tensor* x, chx_hip_
                         bool rne) {
     ConvCall c;
     c.cache = nullptr;
+    c.tune = nullptr;
     c.x = x;
     c.y = y;
     c.p = p;
@@ -559,6 +648,7 @@ struct chx_hip_qconv_plan {
     bool mfma;
     chx::PackedWeights pw;
     chx::ScratchCache scratch;  // makes run() unsafe to call concurrently on one plan
+    chx::TuneCache tune;
 };
 
 extern "C" int chx_hip_qlinear_conv(
@@ -640,6 +730,7 @@ extern "C" int chx_hip_qconv_plan_run(
     if (plan->mfma) {
         ConvCall call = conv_call_from(q, x, y, &plan->params, rne);
         call.cache = const_cast<ScratchCache*>(&plan->scratch);
+        call.tune = const_cast<TuneCache*>(&plan->tune);
         const int rc = run_conv_mfma(call, plan->pw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }

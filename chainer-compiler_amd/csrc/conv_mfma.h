@@ -34,6 +34,7 @@ struct ConvMfmaArgs {
     float inv_y_scale;           // 1 / y_scale, for the division-free requantization
     float lo_folded;             // lower clamp bound with the fused Relu folded in (fold_relu_floor)
     int32_t tiles_oc, tiles_px;  // filled by the launcher
+    uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
 };
 
 struct Im2colArgs {
@@ -46,10 +47,20 @@ struct Im2colArgs {
     char* col;      // [M][Kd]
 };
 
+// Multiplier and shift with n / d == (mulhi(n, mul) + n) >> shift for every n < 2^31 (d >= 1).
+inline void magic_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
+    uint32_t l = 0;
+    while ((uint64_t(1) << l) < d) ++l;
+    *mul = (uint32_t)((((uint64_t(1) << l) - d) << 32) / d + 1);
+    *shift = l;
+}
+
 int pack_weights_dense(const chx_hip_tensor& w, int Kd, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 int launch_im2col_dense(const Im2colArgs& a, hipStream_t s);
 int pack_weights(const chx_hip_tensor& w, int C64, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
-int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, bool x_unsigned, bool out_int32, bool rne, hipStream_t s);
+// max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once)
+int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
+                     hipStream_t s);
 
 // [N][C][HW] bytes -> [N][HW][pitch] bytes (lanes c >= C of a pixel are zero filled) and back
 int launch_nchw_to_nhwc_u8(const char* src, char* dst, int N, int C, int64_t HW, int pitch, hipStream_t s);

@@ -167,6 +167,11 @@ __device__ __attribute__((aligned(64))) const unsigned char g_fill_rows[256 * 64
 #undef CHX_ROW
 #undef CHX_B16
 
+// n / d for n < 2^31 with the multiplier and shift of magic_divisor() (conv_mfma.h).
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t mul, uint32_t shift) {
+    return (__umulhi(n, mul) + n) >> shift;
+}
+
 // Asynchronous copy of 16 bytes per lane from global memory straight into LDS: lane i of the
 // wavefront writes LDS bytes [lds_addr + 16*i, lds_addr + 16*i + 16).  lds_addr must be the
 // same for all lanes (it travels in M0).  Completion is tracked by the wave's vector-memory
@@ -275,22 +280,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             const bool row_ok = m < a.M && ld_tile < px_hi;
             // rows past the end re-read the last pixel; they are never written back
             const uint32_t mm = m < a.M ? (uint32_t)m : (uint32_t)(a.M - 1);  // M fits 31 bits (checked on the host)
-            const uint32_t ow = mm % (uint32_t)a.OW;
-            const uint32_t r = mm / (uint32_t)a.OW;
-            const uint32_t oh = r % (uint32_t)a.OH;
-            const uint32_t n = r / (uint32_t)a.OH;
+            const uint32_t r = fast_div(mm, a.ow_mul, a.ow_shift);
+            const uint32_t ow = mm - r * (uint32_t)a.OW;
+            const uint32_t n = fast_div(r, a.oh_mul, a.oh_shift);
+            const uint32_t oh = r - n * (uint32_t)a.OH;
             const int ih0 = (int)oh * a.sh - a.ph;
             const int iw0 = (int)ow * a.sw - a.pw;
             xb[j] = a.x + (int64_t)n * a.x_n_stride + (int64_t)ih0 * a.x_h_stride + (int64_t)iw0 * a.x_w_stride + kc * 16;
             if (kPad) {
+                // taps (i, jj) inside the image: i in [r_lo, r_hi), jj in [c_lo, c_hi)
+                const int c_lo = min(max(-iw0, 0), a.KW), c_hi = min(max(a.W - iw0, 0), a.KW);
+                const int r_lo = min(max(-ih0, 0), a.KH), r_hi = min(max(a.H - ih0, 0), a.KH);
+                const uint64_t below_hi = c_hi >= 64 ? ~(uint64_t)0 : ((uint64_t)1 << c_hi) - 1;  // a 1x64 filter fills the mask
+                const uint64_t cols = c_hi > c_lo ? below_hi & ~(((uint64_t)1 << c_lo) - 1) : 0;
                 uint64_t mask = 0;
-                if (row_ok) {
-                    for (int t = 0, i = 0; i < a.KH; ++i)
-                        for (int jj = 0; jj < a.KW; ++jj, ++t)
-                            if ((unsigned)(ih0 + i) < (unsigned)a.H && (unsigned)(iw0 + jj) < (unsigned)a.W)
-                                mask |= (uint64_t)1 << t;
-                }
-                tapmask[j] = mask;
+                for (int i = 0; i < a.KH; ++i)
+                    if (i >= r_lo && i < r_hi) mask |= cols << (i * a.KW);
+                tapmask[j] = row_ok ? mask : 0;
             }
         }
     };
@@ -509,12 +515,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 }
 
 template <int FM, int FN>
-int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool rne, hipStream_t s) {
+int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool rne, int max_wgs_per_cu, hipStream_t s) {
     // persistent work-groups: as many as the device holds at once, a whole number per
     // output-channel tile
-    static int resident = 0;  // per (FM, FN); the variants of one tile shape use about the same resources
-    if (resident == 0) {
-        int dev = 0, cus = 256, per_cu = 2;
+    static int cus = 256, per_cu = 0;  // per (FM, FN); the variants of one tile shape use about the same resources
+    if (per_cu == 0) {
+        int dev = 0;
+        per_cu = 2;
         if (hipGetDevice(&dev) == hipSuccess) {
             hipDeviceProp_t prop;
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
@@ -524,8 +531,8 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
                     hipSuccess ||
             per_cu < 1)
             per_cu = 2;
-        resident = cus * per_cu;
     }
+    const int resident = cus * (max_wgs_per_cu > 0 && max_wgs_per_cu < per_cu ? max_wgs_per_cu : per_cu);
     int slots = (a.tiles_px + 7) / 8;  // pixel-tile slots per XCD
     const int cap = resident / (8 * a.tiles_oc) > 0 ? resident / (8 * a.tiles_oc) : 1;
     if (slots > cap) slots = cap;
@@ -578,14 +585,17 @@ int launch_im2col_dense(const Im2colArgs& a, hipStream_t s) {
     return launch_check("im2col_dense_kernel");
 }
 
-int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, bool x_unsigned, bool out_int32, bool rne, hipStream_t s) {
+int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
+                     hipStream_t s) {
     a.tiles_oc = (a.OC + tile_oc - 1) / tile_oc;
     a.tiles_px = (int)((a.M + tile_px - 1) / tile_px);
     if (a.M == 0 || a.OC == 0) return CHX_HIP_OK;
-    if (tile_oc == 128 && tile_px == 128) return launch_config<2, 2>(a, x_unsigned, out_int32, rne, s);
-    if (tile_oc == 64 && tile_px == 128) return launch_config<1, 2>(a, x_unsigned, out_int32, rne, s);
-    if (tile_oc == 128 && tile_px == 64) return launch_config<2, 1>(a, x_unsigned, out_int32, rne, s);
-    if (tile_oc == 64 && tile_px == 64) return launch_config<1, 1>(a, x_unsigned, out_int32, rne, s);
+    magic_divisor((uint32_t)a.OW, &a.ow_mul, &a.ow_shift);
+    magic_divisor((uint32_t)a.OH, &a.oh_mul, &a.oh_shift);
+    if (tile_oc == 128 && tile_px == 128) return launch_config<2, 2>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 64 && tile_px == 128) return launch_config<1, 2>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 128 && tile_px == 64) return launch_config<2, 1>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 64 && tile_px == 64) return launch_config<1, 1>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
     CHX_FAIL(CHX_HIP_EINVAL, "conv_mfma: no kernel for a %dx%d tile", tile_oc, tile_px);
 }
 
