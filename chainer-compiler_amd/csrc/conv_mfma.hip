@@ -146,6 +146,73 @@ __global__ __launch_bounds__(256) void im2col_dense_kernel(Im2colArgs a) {
     *reinterpret_cast<v4i*>(a.col + m * a.Kd + ch * 16) = o;
 }
 
+// The same matrix, staged through LDS: a work-group takes kIm2colPx consecutive output pixels of
+// one output row, copies the C x KH input row segments they touch into LDS once (coalesced,
+// out-of-image bytes replaced by the zero point), and then every lane assembles 16-byte chunks
+// of the [M][Kd] rows from LDS bytes; consecutive lanes write consecutive chunks.  A table maps
+// k = (kh*KW + kw)*C + c to the LDS offset of the pixel-independent part of the address.
+constexpr int kIm2colPx = 64;
+constexpr int kIm2colPatchMax = 24 * 1024;  // bytes of LDS for the input patch
+
+__global__ __launch_bounds__(256) void im2col_dense_lds_kernel(Im2colArgs a, int row_len) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char im2col_lds[];
+    const int K = a.KH * a.KW * a.C;
+    uint16_t* tab = reinterpret_cast<uint16_t*>(im2col_lds);  // [Kd]
+    unsigned char* patch = im2col_lds + a.Kd * 2;             // [C*KH][row_len]
+    const int tid = threadIdx.x;
+    const int ow0 = blockIdx.x * kIm2colPx;
+    const int oh = blockIdx.y;
+    const int n = blockIdx.z;
+    for (int k = tid; k < a.Kd; k += 256) {
+        int v = 0xffff;
+        if (k < K) {
+            const int c = k % a.C, pos = k / a.C;
+            const int kh = pos / a.KW, kw = pos % a.KW;
+            v = (c * a.KH + kh) * row_len + kw;
+        }
+        tab[k] = (uint16_t)v;
+    }
+    const int ih0 = oh * a.sh - a.ph, iw0 = ow0 * a.sw - a.pw;
+    const char* xn = a.x + (int64_t)n * a.xs[0];
+    const int rows = a.C * a.KH;
+    for (int idx = tid; idx < rows * row_len; idx += 256) {
+        const int rr = idx / row_len, col = idx - rr * row_len;
+        const int c = rr / a.KH, kh = rr - c * a.KH;
+        const int ih = ih0 + kh, iw = iw0 + col;
+        unsigned char v = (unsigned char)a.fill;
+        if ((unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W)
+            v = *reinterpret_cast<const unsigned char*>(xn + (int64_t)c * a.xs[1] + (int64_t)ih * a.xs[2] + (int64_t)iw * a.xs[3]);
+        patch[idx] = v;
+    }
+    __syncthreads();
+    const int chunks = a.Kd / 16;
+    const int npx = min(kIm2colPx, a.OW - ow0);
+    const int64_t m0 = ((int64_t)n * a.OH + oh) * a.OW + ow0;
+    const uint32_t fill = (uint32_t)a.fill & 0xffu;
+    for (int q = tid; q < npx * chunks; q += 256) {
+        const int p = q / chunks, ch = q - p * chunks;
+        const unsigned char* src = patch + p * a.sw;
+        const v4i t0 = *reinterpret_cast<const v4i*>(tab + ch * 16);
+        const v4i t1 = *reinterpret_cast<const v4i*>(tab + ch * 16 + 8);
+        uint32_t out[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int k = d * 4 + e;  // two 16-bit offsets per dword of the table
+                const uint32_t pair = (uint32_t)(k < 8 ? t0[k >> 1] : t1[(k - 8) >> 1]);
+                const uint32_t off = (k & 1) ? pair >> 16 : pair & 0xffffu;
+                const uint32_t v = off == 0xffffu ? fill : (uint32_t)src[off];
+                word |= v << (8 * e);
+            }
+            out[d] = word;
+        }
+        const v4i o = {(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
+        *reinterpret_cast<v4i*>(a.col + (m0 + p) * a.Kd + ch * 16) = o;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ int lds_chunk_offset(int row, int kc) {
     return row * kBK + ((kc ^ ((row >> 2) & 3)) << 4);
@@ -581,6 +648,15 @@ int pack_weights_dense(const chx_hip_tensor& w, int Kd, int OCpad, int8_t* wp, i
 int launch_im2col_dense(const Im2colArgs& a, hipStream_t s) {
     const int64_t total = a.M * (a.Kd / 16);
     if (total == 0) return CHX_HIP_OK;
+    // LDS-staged variant when the input patch of a pixel group fits (the offsets are 16-bit)
+    const int row_len = (kIm2colPx - 1) * a.sw + a.KW;
+    const int64_t patch = (int64_t)a.C * a.KH * row_len;
+    const int64_t N = a.M / ((int64_t)a.OH * a.OW);
+    if (patch <= kIm2colPatchMax && patch < 0xffff && a.OH <= 65535 && N <= 65535) {
+        const dim3 grid((unsigned)((a.OW + kIm2colPx - 1) / kIm2colPx), (unsigned)a.OH, (unsigned)N);
+        im2col_dense_lds_kernel<<<grid, 256, (size_t)(a.Kd * 2 + patch), s>>>(a, row_len);
+        return launch_check("im2col_dense_lds_kernel");
+    }
     im2col_dense_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a);
     return launch_check("im2col_dense_kernel");
 }

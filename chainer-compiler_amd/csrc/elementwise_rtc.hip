@@ -128,7 +128,20 @@ std::string ident(const std::string& s) {
     return o;
 }
 
+int float_value(const std::string& tok, float* value);
+
 int float_literal(const std::string& tok, std::string* out) {
+    float f;
+    CHX_PROPAGATE(float_value(tok, &f));
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    char buf[64];
+    snprintf(buf, sizeof(buf), "__builtin_bit_cast(float, 0x%08xu)", bits);
+    *out = buf;
+    return CHX_HIP_OK;
+}
+
+int float_value(const std::string& tok, float* value) {
     float f;
     if (tok.size() == 10 && tok[0] == '0' && (tok[1] == 'x' || tok[1] == 'X')) {
         char* end = nullptr;
@@ -142,11 +155,7 @@ int float_literal(const std::string& tok, std::string* out) {
         CHX_REQUIRE(end && *end == 0 && end != tok.c_str(), "fusion program: bad float literal '%s'", tok.c_str());
         f = (float)d;
     }
-    uint32_t bits;
-    memcpy(&bits, &f, 4);
-    char buf[64];
-    snprintf(buf, sizeof(buf), "__builtin_bit_cast(float, 0x%08xu)", bits);
-    *out = buf;
+    *value = f;
     return CHX_HIP_OK;
 }
 
@@ -252,8 +261,28 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             CHX_REQUIRE(zp >= (i8 ? -128 : 0) && zp <= (i8 ? 127 : 255), "fusion program: zero point %ld out of range", zp);
             const char* lo = i8 ? "-128.0f" : "0.0f";
             const char* hi = i8 ? "127.0f" : "255.0f";
-            // quantize_array, runtime/ops/quantize.cc:29-34
-            os << "  float " << o << "_s = " << a << " / " << l0 << ";\n";
+            // quantize_array, runtime/ops/quantize.cc:29-34.  The correctly rounded quotient comes from
+            // three multiply-adds with the rounded reciprocal (q0 within an ulp, exact residual, one
+            // correction) instead of the ten-instruction IEEE division.  The dividend is first limited
+            // to +-2^40 * scale: beyond that both the true quotient and the limited one are far outside
+            // the 8-bit range and saturate alike, and no intermediate can overflow.
+            float scale_value;
+            CHX_PROPAGATE(float_value(s.args[1], &scale_value));
+            if (scale_value >= 0x1p-60f && scale_value <= 0x1p60f) {
+                const float inv = 1.0f / scale_value, big = 0x1p40f * scale_value;
+                uint32_t inv_bits, big_bits;
+                memcpy(&inv_bits, &inv, 4);
+                memcpy(&big_bits, &big, 4);
+                char inv_lit[64], big_lit[64];
+                snprintf(inv_lit, sizeof(inv_lit), "__builtin_bit_cast(float, 0x%08xu)", inv_bits);
+                snprintf(big_lit, sizeof(big_lit), "__builtin_bit_cast(float, 0x%08xu)", big_bits);
+                os << "  const float " << o << "_v = __builtin_amdgcn_fmed3f(" << a << ", -" << big_lit << ", " << big_lit << ");\n";
+                os << "  const float " << o << "_q0 = " << o << "_v * " << inv_lit << ";\n";
+                os << "  const float " << o << "_r = __builtin_fmaf(-" << o << "_q0, " << l0 << ", " << o << "_v);\n";
+                os << "  float " << o << "_s = __builtin_fmaf(" << o << "_r, " << inv_lit << ", " << o << "_q0);\n";
+            } else {
+                os << "  float " << o << "_s = " << a << " / " << l0 << ";\n";
+            }
             if (s.args.size() == 5) {
                 os << "  " << o << "_s = __builtin_rintf(" << o << "_s) + " << zp << ".0f;\n";
                 os << "  " << o << "_s = " << o << "_s < " << hi << " ? " << o << "_s : " << hi << ";\n";
