@@ -10,6 +10,7 @@
 
 #include "contract.h"
 #include "conv_mfma.h"
+#include "depthwise.h"
 
 namespace chx {
 namespace {
@@ -579,6 +580,56 @@ void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
     pw->wsum = nullptr;
 }
 
+// Depthwise 3x3 on int8 weights with zero weight zero points: paired weights and per-channel
+// sums, plus the per-run parameter vectors (they depend on the activation scale and zero point).
+struct DepthwiseState {
+    int C = 0;
+    void* block = nullptr;  // one allocation: pairs | wsum | seed | scale | fbias
+    int32_t* pairs = nullptr;
+    int32_t* wsum = nullptr;
+    int32_t* seed = nullptr;
+    float* scale = nullptr;
+    float* fbias = nullptr;
+};
+
+bool weights_fit_depthwise(const chx_hip_tensor& w, int group) {
+    return w.dtype == CHX_HIP_INT8 && group > 1 && w.shape[0] == group && w.shape[1] == 1 && w.shape[2] == 3 &&
+           w.shape[3] == 3 && group % 16 == 0;
+}
+
+int make_depthwise(const chx_hip_tensor& w, bool persistent, hipStream_t s, DepthwiseState* st) {
+    const int C = (int)w.shape[0];
+    const size_t pairs_bytes = (size_t)(C / 16) * 5 * 16 * sizeof(int32_t);
+    const size_t total = pairs_bytes + (size_t)C * 16;
+    void* p = nullptr;
+    if (persistent) CHX_HIP_CALL(hipMalloc(&p, total));
+    else CHX_PROPAGATE(scratch_alloc(&p, total, s));
+    st->C = C;
+    st->block = p;
+    char* b = static_cast<char*>(p);
+    st->pairs = reinterpret_cast<int32_t*>(b);
+    st->wsum = reinterpret_cast<int32_t*>(b + pairs_bytes);
+    st->seed = st->wsum + C;
+    st->scale = reinterpret_cast<float*>(st->seed + C);
+    st->fbias = st->scale + C;
+    return pack_depthwise(w, st->pairs, st->wsum, s);
+}
+
+void release_depthwise(DepthwiseState* st, bool persistent, hipStream_t s) {
+    if (!st->block) return;
+    if (persistent) (void)hipFree(st->block);
+    else scratch_free(st->block, s);
+    st->block = nullptr;
+}
+
+// channels-last 8-bit tensor whose pixels are 16-byte aligned vectors of C bytes
+bool is_depthwise_layout(const chx_hip_tensor& t) {
+    if (!is_q8(t.dtype) || t.strides[1] != 1 || !aligned(t.data, 16)) return false;
+    for (int ax : {0, 2, 3})
+        if (t.shape[ax] != 1 && (t.strides[ax] % 16 != 0 || t.strides[ax] < t.shape[1])) return false;
+    return true;
+}
+
 struct QConvChecked {
     ConvShape cs;
     ConvDirectArgs direct;
@@ -638,6 +689,40 @@ ConvCall conv_call_from(const QConvChecked& q, const chx_hip_tensor* x, chx_hip_
     return c;
 }
 
+// Runs the depthwise kernel; EUNSUPPORTED when the operand layouts are not channels-last.
+int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
+    const chx_hip_tensor& x = *c.x;
+    const chx_hip_tensor& y = *c.y;
+    if (!is_depthwise_layout(x) || !is_depthwise_layout(y))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel needs channels-last 8-bit operands with 16-byte aligned pixels");
+    const bool xs = x.dtype == CHX_HIP_INT8;
+    const int32_t zp_u = xs ? c.x_zp + 128 : c.x_zp;
+    CHX_PROPAGATE(launch_depthwise_params(st.C, st.wsum, zp_u, c.w_scale, c.w_scale_len, c.rq.x_scale, c.bias, c.rq.bias_mode,
+                                          st.seed, st.scale, st.fbias, s));
+    DepthwiseArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = static_cast<const char*>(x.data);
+    a.x_n_stride = x.strides[0];
+    a.x_h_stride = x.strides[2];
+    a.x_w_stride = x.strides[3];
+    a.y = static_cast<char*>(y.data);
+    a.y_n_stride = y.strides[0];
+    a.y_h_stride = y.strides[2];
+    a.y_w_stride = y.strides[3];
+    a.N = c.cs.N; a.C = c.cs.C; a.H = c.cs.H; a.W = c.cs.W; a.OH = c.cs.OH; a.OW = c.cs.OW;
+    a.sh = c.p->stride_h; a.sw = c.p->stride_w; a.ph = c.p->pad_h_begin; a.pw = c.p->pad_w_begin;
+    a.x_signed = xs ? 1 : 0;
+    a.x_zp_u = zp_u;
+    a.pairs = st.pairs;
+    a.seed = st.seed;
+    a.scale = st.scale;
+    a.fbias = (c.bias && c.rq.bias_mode == kBiasReferenceFloat) ? st.fbias : nullptr;
+    a.q = c.rq.q;
+    a.inv_y_scale = 1.0f / c.rq.q.scale;
+    a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
+    return launch_depthwise3x3(a, c.rne, s);
+}
+
 }  // namespace
 }  // namespace chx
 
@@ -646,6 +731,8 @@ struct chx_hip_qconv_plan {
     bool has_bias;
     chx_hip_conv_params params;
     bool mfma;
+    bool depthwise;
+    chx::DepthwiseState dw;
     chx::PackedWeights pw;
     chx::ScratchCache scratch;  // makes run() unsafe to call concurrently on one plan
     chx::TuneCache tune;
@@ -668,6 +755,17 @@ extern "C" int chx_hip_qlinear_conv(
             CHX_PROPAGATE(make_packed(*w, false, s, &pw));
             const int rc = run_conv_mfma(conv_call_from(q, x, y, params, rne), pw, s);
             release_packed(&pw, false, s);
+            if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        }
+    }
+    if (weights_fit_depthwise(*w, params->group)) {
+        std::vector<uint8_t> zp;
+        CHX_PROPAGATE(read_back(*w_zero_point, &zp, s));
+        if (all_zero(zp)) {
+            DepthwiseState st;
+            CHX_PROPAGATE(make_depthwise(*w, false, s, &st));
+            const int rc = run_depthwise(conv_call_from(q, x, y, params, rne), st, s);
+            release_depthwise(&st, false, s);
             if (rc != CHX_HIP_EUNSUPPORTED) return rc;
         }
     }
@@ -694,6 +792,21 @@ extern "C" int chx_hip_qconv_plan_create(
     if (bias) p->bias = *bias;
     p->params = *params;
     p->mfma = false;
+    p->depthwise = false;
+    if (weights_fit_depthwise(*w, params->group) && w_zero_point->dtype == w->dtype && w_zero_point->ndim <= 1) {
+        std::vector<uint8_t> zp;
+        int rc = read_back(*w_zero_point, &zp, s);
+        if (rc == CHX_HIP_OK && all_zero(zp)) {
+            rc = make_depthwise(*w, true, s, &p->dw);
+            if (rc == CHX_HIP_OK && hipStreamSynchronize(s) != hipSuccess) rc = CHX_HIP_ERUNTIME;
+            if (rc == CHX_HIP_OK) p->depthwise = true;
+        }
+        if (rc != CHX_HIP_OK) {
+            release_depthwise(&p->dw, true, s);
+            delete p;
+            return rc;
+        }
+    }
     if (weights_fit_mfma(*w, params->group) && w_zero_point->dtype == w->dtype && w_zero_point->ndim <= 1) {
         std::vector<uint8_t> zp;
         int rc = read_back(*w_zero_point, &zp, s);
@@ -734,12 +847,17 @@ extern "C" int chx_hip_qconv_plan_run(
         const int rc = run_conv_mfma(call, plan->pw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
+    if (plan->depthwise) {
+        const int rc = run_depthwise(conv_call_from(q, x, y, &plan->params, rne), plan->dw, s);
+        if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+    }
     return launch_conv_direct(q.direct, rne, s);
 }
 
 extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {
     if (!plan) return;
     chx::release_packed(&plan->pw, true, nullptr);
+    chx::release_depthwise(&plan->dw, true, nullptr);
     for (int i = 0; i < 2; ++i)
         if (plan->scratch.ptr[i]) (void)hipFree(plan->scratch.ptr[i]);
     delete plan;

@@ -1,0 +1,35 @@
+// Interface of the depthwise 3x3 kernel (depthwise.hip) towards the entry points.
+#pragma once
+
+#include "chx_internal.h"
+#include "quant_math.h"
+
+namespace chx {
+
+struct DepthwiseArgs {
+    // activations, channels-last: element (n, c, ih, iw) at x + n*x_n_stride + ih*x_h_stride + iw*x_w_stride + c
+    const char* x;
+    int64_t x_n_stride, x_h_stride, x_w_stride;
+    char* y;  // same convention
+    int64_t y_n_stride, y_h_stride, y_w_stride;
+    int32_t N, C, H, W, OH, OW, sh, sw, ph, pw;
+    int32_t x_signed;       // int8 activations: codes and zero point are shifted by 128
+    int32_t x_zp_u;         // zero point in the unsigned range (zp, or zp + 128 for int8)
+    const int32_t* pairs;   // [C/16][5][16] paired weights (pack_depthwise)
+    const int32_t* seed;    // [C] accumulator start
+    const float* scale;     // [C] x_scale * w_scale[c]
+    const float* fbias;     // [C] or null: float bias added after the scale multiply (reference mode)
+    QuantParams q;
+    float inv_y_scale;
+    float lo_folded;
+    int32_t ow_blocks;      // filled by the launcher
+    int64_t total;          // filled by the launcher
+};
+
+int pack_depthwise(const chx_hip_tensor& w, int32_t* pairs, int32_t* wsum, hipStream_t s);
+int launch_depthwise_params(
+        int C, const int32_t* wsum, int32_t zp_u, const float* w_scale, int w_scale_len, float x_scale, const int32_t* bias,
+        int bias_mode, int32_t* seed, float* scale, float* fbias, hipStream_t s);
+int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s);
+
+}  // namespace chx

@@ -283,14 +283,14 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             } else {
                 os << "  float " << o << "_s = " << a << " / " << l0 << ";\n";
             }
+            // the clamp is one median instruction: the same function as Maximum(lo, Minimum(s, hi))
+            // for every value that is not a NaN
             if (s.args.size() == 5) {
                 os << "  " << o << "_s = __builtin_rintf(" << o << "_s) + " << zp << ".0f;\n";
-                os << "  " << o << "_s = " << o << "_s < " << hi << " ? " << o << "_s : " << hi << ";\n";
-                os << "  " << o << "_s = " << lo << " < " << o << "_s ? " << o << "_s : " << lo << ";\n";
+                os << "  " << o << "_s = __builtin_amdgcn_fmed3f(" << o << "_s, " << lo << ", " << hi << ");\n";
             } else {
                 os << "  " << o << "_s = " << o << "_s + " << zp << ".0f;\n";
-                os << "  " << o << "_s = " << o << "_s < " << hi << " ? " << o << "_s : " << hi << ";\n";
-                os << "  " << o << "_s = " << lo << " < " << o << "_s ? " << o << "_s : " << lo << ";\n";
+                os << "  " << o << "_s = __builtin_amdgcn_fmed3f(" << o << "_s, " << lo << ", " << hi << ");\n";
                 os << "  " << o << "_s = " << o << "_s + 0.5f;\n";
             }
             os << "  const int " << o << " = (int)" << o << "_s;\n";

@@ -1,5 +1,6 @@
 """Quantized networks as hand-built ChxVM-style programs: the ResNet-50 int8 QDQ
-configuration the headline metric is quoted on, in the op vocabulary of this path.
+configuration the headline metric is quoted on and the MobileNetV2 configuration with its
+depthwise convolutions, in the op vocabulary of this path.
 
 A program is a list of instructions over named values; every instruction is one op
 of the path (QuantizeLinear, QLinearConv, MaxPool, FusionGroup Add+Relu, AveragePool,
@@ -71,8 +72,8 @@ def activation_qparams(t):
 
 
 class ConvLayer(object):
-    def __init__(self, name, w, b, stride, pad):
-        self.name, self.wf, self.bf, self.stride, self.pad = name, w, b, stride, pad
+    def __init__(self, name, w, b, stride, pad, group=1):
+        self.name, self.wf, self.bf, self.stride, self.pad, self.group = name, w, b, stride, pad, group
         self.wq, self.w_scale = quantize_weights_per_channel(w)
         self.w_zp = np.zeros(w.shape[0], np.int8)
         self.x_scale = self.x_zp = self.y_scale = self.y_zp = None
@@ -164,6 +165,105 @@ def build_resnet50(batch=64, image=224, seed=3, width=64, blocks=(3, 4, 6, 3), c
                 float_logits=fvals["logits_q"].detach().cpu().numpy())
 
 
+# MobileNetV2-1.0 (Sandler et al. 2018, table 2): expansion t, output channels c, repeats n, stride s
+MOBILENETV2_BLOCKS = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2),
+                      (6, 320, 1, 1))
+
+
+def build_mobilenetv2(batch=128, image=224, seed=4, blocks=MOBILENETV2_BLOCKS, stem=32, head=1280, classes=1000,
+                      device=None):
+    """MobileNetV2 as a QDQ program: 3x3/2 stem, inverted residual blocks (1x1 expansion,
+    depthwise 3x3, linear 1x1 projection, residual Add where shapes agree), 1x1 head, global
+    average pool, classifier.  Kaiming-normal weights with BatchNorm folded; every ReLU6 is
+    folded into the output quantization of its convolution (the calibrated range of a
+    post-ReLU6 tensor is [0, <=6], zero point 0, so uint8 saturation is the clipping); the
+    linear projections and the residual sums get asymmetric uint8 ranges.  `blocks`, `stem`,
+    `head`, `image`, `classes` shrink the network for tests."""
+    rng = np.random.default_rng(seed)
+    dev = device or ("cuda" if torch.cuda.is_available() else "cpu")
+    x = rng.standard_normal((batch, 3, image, image)).astype(np.float32)
+    program, convs, qparams, shapes = [], {}, {}, {}
+    fvals = {"x": torch.from_numpy(x).to(dev)}
+
+    def note(name):
+        qparams[name] = activation_qparams(fvals[name])
+        shapes[name] = tuple(fvals[name].shape)
+
+    def conv(name, src, dst, cin, cout, k, stride, pad, relu6, group=1, bias=False):
+        w = _he_normal(rng, (cout, cin // group, k, k))
+        b = (rng.standard_normal(cout) * 0.1).astype(np.float32) if bias else None
+        w, b = _fold_bn(rng, w, b)
+        layer = ConvLayer(name, w, b, stride, pad, group)
+        convs[name] = layer
+        wd = torch.from_numpy(layer.wq.astype(np.float32) * layer.w_scale[:, None, None, None]).to(dev)
+        y = F.conv2d(fvals[src], wd, torch.from_numpy(b).to(dev), stride=stride, padding=pad, groups=group)
+        fvals[dst] = F.relu6(y) if relu6 else y
+        note(dst)
+        layer.x_scale, layer.x_zp = qparams[src]
+        layer.y_scale, layer.y_zp = qparams[dst]
+        layer.finish()
+        program.append(("QLinearConv", dst, src, name))
+
+    note("x")
+    program.append(("QuantizeLinear", "x_q", "x") + qparams["x"])
+    fvals["x_q"] = fvals["x"]
+    qparams["x_q"], shapes["x_q"] = qparams["x"], shapes["x"]
+    conv("stem", "x_q", "f0", 3, stem, 3, 2, 1, relu6=True)
+    cur, cin, bi = "f0", stem, 0
+    for t, c, n, s_ in blocks:
+        for i in range(n):
+            bi += 1
+            p = "b%d" % bi
+            stride = s_ if i == 0 else 1
+            hidden = cin * t
+            src = cur
+            if t != 1:
+                conv(p + "_expand", src, p + "_e", cin, hidden, 1, 1, 0, relu6=True)
+                src = p + "_e"
+            conv(p + "_dw", src, p + "_d", hidden, hidden, 3, stride, 1, relu6=True, group=hidden)
+            conv(p + "_project", p + "_d", p + "_p", hidden, c, 1, 1, 0, relu6=False)
+            out = p + "_p"
+            if stride == 1 and cin == c:
+                fvals[p] = fvals[p + "_p"] + fvals[cur]
+                note(p)
+                program.append(("Add", p, p + "_p", cur))
+                out = p
+            for tmp in (p + "_e", p + "_d", cur) + ((p + "_p",) if out != p + "_p" else ()):
+                fvals.pop(tmp, None)
+            cur, cin = out, c
+    conv("head", cur, "head", cin, head, 1, 1, 0, relu6=True)
+    k = fvals["head"].shape[2]
+    fvals["gap"] = F.avg_pool2d(fvals["head"], k, 1)
+    note("gap")
+    program.append(("AveragePool", "gap", "head", int(k)))
+    conv("fc", "gap", "logits_q", head, classes, 1, 1, 0, relu6=False, bias=True)
+    program.append(("DequantizeLinear", "logits", "logits_q") + qparams["logits_q"])
+    shapes["logits"] = shapes["logits_q"]
+    total_macs = 0
+    dw_bytes = 0
+    for ins in program:
+        if ins[0] == "QLinearConv":
+            layer = convs[ins[3]]
+            total_macs += layer.macs(shapes[ins[1]])
+            if layer.group > 1:
+                # algorithmic bytes of a depthwise layer: activations in and out once, nine weights per channel
+                dw_bytes += int(np.prod(shapes[ins[2]])) + int(np.prod(shapes[ins[1]])) + 9 * layer.group
+    return dict(program=program, convs=convs, qparams=qparams, shapes=shapes, input=x, macs=total_macs,
+                depthwise_bytes=dw_bytes, float_logits=fvals["logits_q"].detach().cpu().numpy())
+
+
+def add_program(ops, qa, qb, qy):
+    """FusionGroup text for Q(DQ(a) + DQ(b)) on uint8 tensors (a residual sum without Relu)."""
+    u8 = torch.uint8
+    return ops.fusion_program(
+        [("a", u8), ("b", u8)],
+        [("fa", "DequantizeLinear", "a", "0x%08x" % np.float32(qa[0]).view(np.uint32), qa[1]),
+         ("fb", "DequantizeLinear", "b", "0x%08x" % np.float32(qb[0]).view(np.uint32), qb[1]),
+         ("s", "Add", "fa", "fb"),
+         ("q", "QuantizeLinear", "s", "0x%08x" % np.float32(qy[0]).view(np.uint32), qy[1], "uint8")],
+        [("q", u8)])
+
+
 def add_relu_program(ops, qa, qb, qy):
     """FusionGroup text for Q(Relu(DQ(a) + DQ(b))) on uint8 tensors."""
     u8 = torch.uint8
@@ -186,11 +286,12 @@ class DeviceRunner(object):
         self.plans = {}
         self.bufs = {}
         self.fusion = {}
+        self.full = {}
         for name, c in model["convs"].items():
             t = [torch.from_numpy(a).cuda() for a in (c.wq, c.w_scale, c.w_zp, c.bias_q)]
             self.dev[name] = t
             self.plans[name] = self.ops.QLinearConvPlan(t[0], t[1], t[2], t[3], strides=(c.stride, c.stride),
-                                                        pads=(c.pad, c.pad))
+                                                        pads=(c.pad, c.pad), group=c.group)
         for ins in model["program"]:
             out = ins[1]
             shp = model["shapes"][out]
@@ -201,11 +302,19 @@ class DeviceRunner(object):
                 # fully coalesced pass); the 3-channel stem reads it through its im2col step
                 self.bufs[out] = torch.empty(shp, dtype=torch.uint8, device="cuda")
             else:
+                # channels-last with the pixel pitch rounded up to 16 bytes, so that every pixel is a
+                # whole number of aligned 16-byte vectors also for channel counts like 24
                 n, c, h, w = shp
-                self.bufs[out] = torch.empty((n, h, w, c), dtype=torch.uint8, device="cuda").permute(0, 3, 1, 2)
+                pitch = (c + 15) // 16 * 16
+                full = torch.zeros((n, h, w, pitch), dtype=torch.uint8, device="cuda")
+                self.bufs[out] = full[..., :c].permute(0, 3, 1, 2)
+                # element-wise groups run over the padded pixels as they lie in memory (dense)
+                self.full[out] = full.permute(0, 3, 1, 2)
+            q = model["qparams"]
             if ins[0] == "AddRelu":
-                q = model["qparams"]
                 self.fusion[out] = add_relu_program(self.ops, q[ins[2]], q[ins[3]], q[out])
+            if ins[0] == "Add":
+                self.fusion[out] = add_program(self.ops, q[ins[2]], q[ins[3]], q[out])
 
     def run(self, x):
         ops, q, m = self.ops, self.m["qparams"], self.m
@@ -221,8 +330,8 @@ class DeviceRunner(object):
                                        flags=self.capi.BIAS_ONNX_INT32, out=buf)
             elif kind == "MaxPool":
                 ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
-            elif kind == "AddRelu":
-                ops.ElementWiseNvrtc([v[ins[2]], v[ins[3]]], 1, self.fusion[out], fid, outs=[buf])
+            elif kind in ("AddRelu", "Add"):
+                ops.ElementWiseNvrtc([self.full[ins[2]], self.full[ins[3]]], 1, self.fusion[out], fid, outs=[self.full[out]])
             elif kind == "AveragePool":
                 ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
                                   q[out][1], out=buf)
@@ -269,13 +378,17 @@ def run_reference(model, orc, x, keep=None):
             c = model["convs"][ins[3]]
             v[out] = orc.qlinear_conv_int(v[ins[2]], c.x_scale, c.x_zp, c.wq, c.w_scale, c.w_zp, c.y_scale, c.y_zp,
                                           np.uint8, bias=c.bias_q, strides=(c.stride, c.stride), pads=(c.pad, c.pad),
-                                          bias_mode=orc.BIAS_ONNX_INT32)
+                                          group=c.group, bias_mode=orc.BIAS_ONNX_INT32)
         elif kind == "MaxPool":
             v[out] = orc.max_pool_q8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6])
         elif kind == "AddRelu":
             a = orc.dequantize_linear(v[ins[2]], *q[ins[2]])
             b = orc.dequantize_linear(v[ins[3]], *q[ins[3]])
             v[out] = orc.quantize_linear(orc.relu(orc.binary(orc.ADD, a, b)), q[out][0], q[out][1], np.uint8)
+        elif kind == "Add":
+            a = orc.dequantize_linear(v[ins[2]], *q[ins[2]])
+            b = orc.dequantize_linear(v[ins[3]], *q[ins[3]])
+            v[out] = orc.quantize_linear(orc.binary(orc.ADD, a, b), q[out][0], q[out][1], np.uint8)
         elif kind == "AveragePool":
             v[out] = orc.average_pool_q8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0),
                                          q[out][0], q[out][1], np.uint8)

@@ -229,3 +229,43 @@ def test_errors(g):
         g.ops.MatMulInteger(torch.zeros((2, 3), dtype=torch.uint8, device="cuda"),
                             torch.zeros((4, 5), dtype=torch.uint8, device="cuda"),
                             out=torch.zeros((2, 5), dtype=torch.int32, device="cuda"))
+
+
+@pytest.mark.parametrize("xdt", [np.uint8, np.int8])
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, stride, pad
+    (2, 32, 9, 10, 1, 1), (1, 96, 13, 12, 2, 1), (2, 16, 7, 7, 1, 0), (1, 144, 5, 6, 2, 0), (1, 48, 4, 4, 1, 1)])
+def test_depthwise_qlinear_conv(g, oracle, case, xdt):
+    """Depthwise 3x3 on channels-last operands (the paired-tap kernel), stateless call and plan,
+    both bias modes, fused Relu, ONNX rounding; NCHW operands take the generic kernel and must
+    give the same bytes."""
+    N, C, H, W, stride, pad = case
+    rng = np.random.default_rng(31)
+    x = rand_q(rng, (N, C, H, W), xdt)
+    w = rng.integers(-127, 128, size=(C, 1, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=C).astype(np.float32)
+    wz = np.zeros(C, np.int8)
+    bias = rng.integers(-300, 301, size=C).astype(np.int32)
+    xz = 117 if xdt == np.uint8 else -11
+    ys = np.float32(0.02 * 0.01 * 128 * 64 * 3 / 40)
+    kw = dict(strides=(stride, stride), pads=(pad, pad), group=C)
+    for bias_mode, flags in ((oracle.BIAS_ONNX_INT32, g.capi.BIAS_ONNX_INT32), (oracle.BIAS_REFERENCE_FLOAT, 0)):
+        want = oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, 120, np.uint8, bias=bias, bias_mode=bias_mode, **kw)
+        assert want.min() < want.max()
+        xd = g.to_channels_last(g.dev(x))
+        got = g.ops.QLinearConv(xd, 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, 120, g.dev(bias), flags=flags, **kw)
+        assert got.permute(0, 2, 3, 1).is_contiguous()
+        np.testing.assert_array_equal(g.host(got), want)
+        got_nchw = g.ops.QLinearConv(g.dev(x), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, 120, g.dev(bias), flags=flags, **kw)
+        np.testing.assert_array_equal(g.host(got_nchw), want)
+        plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), **kw)
+        for _ in range(2):
+            np.testing.assert_array_equal(g.host(plan.run(xd, 0.02, xz, ys, 120, flags=flags)), want)
+        plan.close()
+    # int8 output, fused Relu, ONNX rounding
+    fl = g.capi.BIAS_ONNX_INT32 | g.capi.FUSE_RELU | g.capi.ROUND_ONNX_RNE
+    want = np.maximum(oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, -5, np.int8, bias=bias, bias_mode=oracle.BIAS_ONNX_INT32,
+                                              round_mode=oracle.ROUND_ONNX_RNE, **kw), -5).astype(np.int8)
+    got = g.ops.QLinearConv(g.to_channels_last(g.dev(x)), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, -5, g.dev(bias),
+                            zero_point_dtype=torch.int8, flags=fl, **kw)
+    np.testing.assert_array_equal(g.host(got), want)

@@ -88,3 +88,22 @@ def test_hip_graph_replay_matches_eager(g, oracle):
         for ins in model["program"]:
             assert torch.equal(out[ins[1]], eager[ins[1]]), "replay %d: %s" % (i, ins[1])
     runner.close()
+
+
+def test_small_mobilenetv2_every_value(g, oracle):
+    """Reduced MobileNetV2: stem, inverted residual blocks with expansion, depthwise 3x3 at both
+    strides, linear projections, residual Adds, head, pool, classifier."""
+    blocks = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 2, 2), (6, 64, 2, 1))
+    model = g.pkg.workloads.build_mobilenetv2(batch=2, image=64, seed=7, blocks=blocks, stem=32, head=128, classes=10)
+    kinds = [ins[0] for ins in model["program"]]
+    assert "Add" in kinds and sum(c.group > 1 for c in model["convs"].values()) == 7
+    ref = check_model(g, oracle, model)
+    assert ref["logits_q"].min() < ref["logits_q"].max()
+
+
+def test_mobilenetv2_batch1(g, oracle):
+    """The real architecture (MobileNetV2-1.0, 224x224) on one image."""
+    model = g.pkg.workloads.build_mobilenetv2(batch=1, seed=4)
+    assert 2.9e8 < model["macs"] < 3.2e8          # ~300 MMAC per image
+    assert sum(c.group > 1 for c in model["convs"].values()) == 17
+    check_model(g, oracle, model)
