@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-inference path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|conv3x3|fusion|qdq]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|mobilenetv2|conv3x3|fusion|qdq]
 
 Default workload: ResNet-50 v1 int8 QDQ inference, batch 64, 224x224 (the configuration the
 headline metric is quoted on).  One step = one pass of the whole op program over one batch
@@ -32,7 +32,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "conv3x3", "fusion", "qdq"])
+    ap.add_argument("--workload", default="resnet50", choices=["resnet50", "mobilenetv2", "conv3x3", "fusion", "qdq"])
     ap.add_argument("--batch", type=int, default=0, help="override the batch size (changes the workload; for experiments)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every op from the host instead of replaying a HIP graph")
@@ -91,10 +91,11 @@ def cpu_info():
 
 # ------------------------------------------------------------------------------------------------
 
-def bench_resnet50(args, torch, pkg):
+def bench_resnet50(args, torch, pkg, mobilenet=False):
     wl = pkg.workloads
-    batch = args.batch or 64
-    model = wl.build_resnet50(batch=batch, seed=3)
+    batch = args.batch or (128 if mobilenet else 64)
+    build = (lambda **kw: wl.build_mobilenetv2(seed=4, **kw)) if mobilenet else (lambda **kw: wl.build_resnet50(seed=3, **kw))
+    model = build(batch=batch)
     runner = wl.DeviceRunner(model, pkg)
     x = torch.from_numpy(model["input"]).cuda()
     ops, capi = pkg.ops, pkg.capi
@@ -126,6 +127,8 @@ def bench_resnet50(args, torch, pkg):
         if ins[0] != "QLinearConv":
             continue
         c = model["convs"][ins[3]]
+        if mobilenet and c.group == 1:
+            continue  # MobileNetV2: the roofline figure is the depthwise kernel's
         fn = lambda: runner.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
                                               flags=capi.BIAS_ONNX_INT32, out=runner.bufs[ins[1]])
         torch.cuda._sleep(int(2.4e9 * 0.002))
@@ -143,28 +146,34 @@ def bench_resnet50(args, torch, pkg):
         ms = a.elapsed_time(b) / REP
         per_layer[name] = ms
         conv_ms_per_step += ms
-    achieved = conv_ops / (conv_ms_per_step * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % n_launch,
-                    achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
-                    ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
-    res = dict(metric="images/sec ResNet-50 int8 bs64 @1 GPU", value=batch / sec, unit="images/sec",
-               ms_per_step=sec * 1e3, dtype="int8",
-               config=dict(workload="resnet50_v1_int8_qdq", batch=batch, image=224, layout="channels_last",
-                           launch="host" if args.no_graph else "hip_graph_replay",
+    if mobilenet:
+        achieved = model["depthwise_bytes"] / (conv_ms_per_step * 1e-3) / 1e9
+        roofline = dict(bound="hbm", kernel="depthwise3x3_kernel (%d launches per step, summed)" % n_launch,
+                        achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
+                        bytes_per_step=model["depthwise_bytes"], kernel_ms_per_step=conv_ms_per_step)
+    else:
+        achieved = conv_ops / (conv_ms_per_step * 1e-3) / 1e12
+        roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % n_launch,
+                        achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
+                        ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
+    res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),
+               value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
+               config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,
+                           layout="channels_last", launch="host" if args.no_graph else "hip_graph_replay",
                            conv_gmac_per_image=model["macs"] / batch / 1e9))
 
     def cpu():
         from oracle import oracle as orc
         lit = _literal_executor(orc)
         cores = orc.max_threads()
-        one = wl.build_resnet50(batch=1, seed=3)
+        one = build(batch=1)
         orc.set_threads(1)
         t0 = time.perf_counter()
         wl.run_reference(one, lit, one["input"])
         dt1 = time.perf_counter() - t0
         # all cores, sized to roughly the requested budget
         nb = int(max(1, min(16, args.cpu_seconds / max(dt1 / cores * 1.5, 1e-3))))
-        many = wl.build_resnet50(batch=nb, seed=3)
+        many = build(batch=nb)
         orc.set_threads(cores)
         t0 = time.perf_counter()
         wl.run_reference(many, lit, many["input"])
@@ -316,8 +325,8 @@ def main():
     import __graft_entry__ as entry
     pkg = entry.load_package()
     pkg.capi.init(0)
-    if args.workload == "resnet50":
-        res, roofline, cpu, close = bench_resnet50(args, torch, pkg)
+    if args.workload in ("resnet50", "mobilenetv2"):
+        res, roofline, cpu, close = bench_resnet50(args, torch, pkg, mobilenet=args.workload == "mobilenetv2")
     elif args.workload == "conv3x3":
         res, roofline, cpu, close = bench_conv3x3(args, torch, pkg)
     else:

@@ -580,16 +580,12 @@ void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
     pw->wsum = nullptr;
 }
 
-// Depthwise 3x3 on int8 weights with zero weight zero points: paired weights and per-channel
-// sums, plus the per-run parameter vectors (they depend on the activation scale and zero point).
+// Depthwise 3x3 on int8 weights with zero weight zero points: paired weights and per-channel sums.
 struct DepthwiseState {
     int C = 0;
-    void* block = nullptr;  // one allocation: pairs | wsum | seed | scale | fbias
+    void* block = nullptr;  // one allocation: pairs | wsum
     int32_t* pairs = nullptr;
     int32_t* wsum = nullptr;
-    int32_t* seed = nullptr;
-    float* scale = nullptr;
-    float* fbias = nullptr;
 };
 
 bool weights_fit_depthwise(const chx_hip_tensor& w, int group) {
@@ -600,7 +596,7 @@ bool weights_fit_depthwise(const chx_hip_tensor& w, int group) {
 int make_depthwise(const chx_hip_tensor& w, bool persistent, hipStream_t s, DepthwiseState* st) {
     const int C = (int)w.shape[0];
     const size_t pairs_bytes = (size_t)(C / 16) * 5 * 16 * sizeof(int32_t);
-    const size_t total = pairs_bytes + (size_t)C * 16;
+    const size_t total = pairs_bytes + (size_t)C * 4;
     void* p = nullptr;
     if (persistent) CHX_HIP_CALL(hipMalloc(&p, total));
     else CHX_PROPAGATE(scratch_alloc(&p, total, s));
@@ -609,9 +605,6 @@ int make_depthwise(const chx_hip_tensor& w, bool persistent, hipStream_t s, Dept
     char* b = static_cast<char*>(p);
     st->pairs = reinterpret_cast<int32_t*>(b);
     st->wsum = reinterpret_cast<int32_t*>(b + pairs_bytes);
-    st->seed = st->wsum + C;
-    st->scale = reinterpret_cast<float*>(st->seed + C);
-    st->fbias = st->scale + C;
     return pack_depthwise(w, st->pairs, st->wsum, s);
 }
 
@@ -695,10 +688,10 @@ int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
     const chx_hip_tensor& y = *c.y;
     if (!is_depthwise_layout(x) || !is_depthwise_layout(y))
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel needs channels-last 8-bit operands with 16-byte aligned pixels");
+    if (x.strides[3] * x.shape[3] >= (int64_t(1) << 31))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: an input row spans 2 GiB or more");
     const bool xs = x.dtype == CHX_HIP_INT8;
     const int32_t zp_u = xs ? c.x_zp + 128 : c.x_zp;
-    CHX_PROPAGATE(launch_depthwise_params(st.C, st.wsum, zp_u, c.w_scale, c.w_scale_len, c.rq.x_scale, c.bias, c.rq.bias_mode,
-                                          st.seed, st.scale, st.fbias, s));
     DepthwiseArgs a;
     memset(&a, 0, sizeof(a));
     a.x = static_cast<const char*>(x.data);
@@ -714,9 +707,12 @@ int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
     a.x_signed = xs ? 1 : 0;
     a.x_zp_u = zp_u;
     a.pairs = st.pairs;
-    a.seed = st.seed;
-    a.scale = st.scale;
-    a.fbias = (c.bias && c.rq.bias_mode == kBiasReferenceFloat) ? st.fbias : nullptr;
+    a.wsum = st.wsum;
+    a.w_scale = c.w_scale;
+    a.w_scale_len = c.w_scale_len;
+    a.x_scale = c.rq.x_scale;
+    a.bias = c.rq.bias_mode == kBiasNone ? nullptr : c.bias;
+    a.float_bias = c.rq.bias_mode == kBiasReferenceFloat ? 1 : 0;
     a.q = c.rq.q;
     a.inv_y_scale = 1.0f / c.rq.q.scale;
     a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);

@@ -16,9 +16,12 @@ struct DepthwiseArgs {
     int32_t x_signed;       // int8 activations: codes and zero point are shifted by 128
     int32_t x_zp_u;         // zero point in the unsigned range (zp, or zp + 128 for int8)
     const int32_t* pairs;   // [C/16][5][16] paired weights (pack_depthwise)
-    const int32_t* seed;    // [C] accumulator start
-    const float* scale;     // [C] x_scale * w_scale[c]
-    const float* fbias;     // [C] or null: float bias added after the scale multiply (reference mode)
+    const int32_t* wsum;    // [C] sum of the nine weights of a channel
+    const float* w_scale;   // [w_scale_len]
+    int32_t w_scale_len;    // 1 or C
+    float x_scale;
+    const int32_t* bias;    // [C] or null
+    int32_t float_bias;     // bias is added as a float after the scale multiply (reference mode), else to the accumulator
     QuantParams q;
     float inv_y_scale;
     float lo_folded;
@@ -27,9 +30,6 @@ struct DepthwiseArgs {
 };
 
 int pack_depthwise(const chx_hip_tensor& w, int32_t* pairs, int32_t* wsum, hipStream_t s);
-int launch_depthwise_params(
-        int C, const int32_t* wsum, int32_t zp_u, const float* w_scale, int w_scale_len, float x_scale, const int32_t* bias,
-        int bias_mode, int32_t* seed, float* scale, float* fbias, hipStream_t s);
 int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s);
 
 }  // namespace chx

@@ -5,10 +5,11 @@
 // pre-paired weights with one v_dot2_i32_i16, so a 3x3 window costs five permutes and five dot
 // products instead of nine unpack-unpack-multiply-add sequences.
 //
-// A thread owns 16 consecutive channels (one 16-byte vector per pixel) and walks over
+// A thread owns kCh consecutive channels (one 8-byte vector per pixel) and walks over
 // kDwPixels output pixels of one output row; consecutive lanes own consecutive channel groups,
-// so every load and store of a wavefront covers whole pixels.  Weights (80 dwords), scales and
-// accumulator seeds stay in registers across the pixels.
+// so every load and store of a wavefront covers whole pixels.  Weights, scales and accumulator
+// seeds stay in registers across the pixels; the register footprint is kept small enough for
+// five or more waves per SIMD, which is what hides the load latency.
 //
 // Arithmetic: int8 activations are shifted to the unsigned range by flipping the top bit
 // (code + 128, zero point + 128); padding taps read the zero point, which makes them contribute
@@ -49,10 +50,14 @@ __global__ __launch_bounds__(256) void pack_depthwise_kernel(
     wsum[c] = sum;
 }
 
-template <bool kRne>
+constexpr int kCh = 8;           // channels per thread
+constexpr int kDw = kCh / 4;     // dwords per pixel vector
+typedef int vxi __attribute__((ext_vector_type(kDw)));
+
+template <bool kRne, bool kFloatBias, bool kXSigned>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int cgs = a.C / 16;
+    const int cgs = a.C / kCh;
     if (idx >= a.total) return;
     const int cg = (int)(idx % cgs);
     int64_t rest = idx / cgs;
@@ -60,55 +65,79 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
     rest /= a.ow_blocks;
     const int oh = (int)(rest % a.OH);
     const int n = (int)(rest / a.OH);
-    const int c0 = cg * 16;
+    const int c0 = cg * kCh;
 
-    int32_t wp[kPairs][16];
+    // pairs are stored per group of 16 channels: [c0 / 16][pair][c0 % 16 ...]
+    int32_t wp[kPairs][kCh];
+    const int32_t* pbase = a.pairs + (int64_t)(c0 / 16) * kPairs * 16 + (c0 % 16);
 #pragma unroll
     for (int p = 0; p < kPairs; ++p)
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const v4i v = *reinterpret_cast<const v4i*>(a.pairs + ((int64_t)cg * kPairs + p) * 16 + d * 4);
+        for (int d = 0; d < kDw; ++d) {
+            const v4i v = *reinterpret_cast<const v4i*>(pbase + p * 16 + d * 4);
 #pragma unroll
             for (int e = 0; e < 4; ++e) wp[p][d * 4 + e] = v[e];
         }
-    float sc[16];
-    int32_t seed[16];
+    // per channel: accumulator seed -zp * sum_t w (+ int32 bias, ONNX mode), scale x_scale * w_scale,
+    // float bias (reference mode)
+    float sc[kCh], fb[kCh];
+    int32_t seed[kCh];
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        const v4f s4 = *reinterpret_cast<const v4f*>(a.scale + c0 + d * 4);
-        const v4i a4 = *reinterpret_cast<const v4i*>(a.seed + c0 + d * 4);
+    for (int d = 0; d < kDw; ++d) {
+        const v4i ws4 = *reinterpret_cast<const v4i*>(a.wsum + c0 + d * 4);
+        v4i b4 = {0, 0, 0, 0};
+        if (a.bias) b4 = *reinterpret_cast<const v4i*>(a.bias + c0 + d * 4);
+        v4f s4;
+        if (a.w_scale_len > 1) s4 = *reinterpret_cast<const v4f*>(a.w_scale + c0 + d * 4);
+        else s4 = v4f{a.w_scale[0], a.w_scale[0], a.w_scale[0], a.w_scale[0]};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            sc[d * 4 + e] = s4[e];
-            seed[d * 4 + e] = a4[e];
+            seed[d * 4 + e] = -a.x_zp_u * ws4[e] + (kFloatBias ? 0 : b4[e]);
+            sc[d * 4 + e] = a.x_scale * s4[e];
+            fb[d * 4 + e] = kFloatBias ? (float)b4[e] : 0.f;
         }
     }
-    const int flip = a.x_signed ? (int)0x80808080 : 0;
-    const int fill = (int)(((uint32_t)(a.x_zp_u & 0xff)) * 0x01010101u);
+    const int fill = (int)(((uint32_t)(a.x_zp_u & 0xff)) * 0x01010101u);  // the zero point, already in the unsigned range
     const char* xn = a.x + (int64_t)n * a.x_n_stride + c0;
     char* yrow = a.y + (int64_t)n * a.y_n_stride + (int64_t)oh * a.y_h_stride + c0;
     const int ih0 = oh * a.sh - a.ph;
-    const bool float_bias = a.fbias != nullptr;
+    // the three input rows of this output row, clamped into the image so that every load is
+    // valid; what a tap outside the image contributes is replaced by the zero point afterwards
+    const char* rowp[3];
+    bool row_ok[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const int ih = ih0 + i;
+        row_ok[i] = (unsigned)ih < (unsigned)a.H;
+        rowp[i] = xn + (int64_t)min(max(ih, 0), a.H - 1) * a.x_h_stride;
+    }
+    const uint32_t wstride = (uint32_t)a.x_w_stride;  // the host checked that a row spans less than 2^31 bytes
 
     for (int p = 0; p < kDwPixels; ++p) {
         const int ow = owb * kDwPixels + p;
         if (ow >= a.OW) break;
         const int iw0 = ow * a.sw - a.pw;
-        v4i x[kTaps + 1];
+        vxi x[kTaps + 1];
 #pragma unroll
-        for (int t = 0; t < kTaps; ++t) {
-            const int ih = ih0 + t / 3, iw = iw0 + t % 3;
-            v4i v = {fill, fill, fill, fill};
-            if ((unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W) {
-                v = *reinterpret_cast<const v4i*>(xn + (int64_t)ih * a.x_h_stride + (int64_t)iw * a.x_w_stride);
-                v ^= flip;
+        for (int j = 0; j < 3; ++j) {
+            const int iw = iw0 + j;
+            const bool col_ok = (unsigned)iw < (unsigned)a.W;
+            const uint32_t off = (uint32_t)min(max(iw, 0), a.W - 1) * wstride;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                vxi v = *reinterpret_cast<const vxi*>(rowp[i] + off);
+                if (kXSigned) v ^= (int)0x80808080;
+                const bool ok = col_ok && row_ok[i];
+#pragma unroll
+                for (int d = 0; d < kDw; ++d) v[d] = ok ? v[d] : fill;
+                x[i * 3 + j] = v;
             }
-            x[t] = v;
         }
-        x[kTaps] = v4i{0, 0, 0, 0};
-        uint32_t out[4];
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
+        for (int d = 0; d < kDw; ++d) x[kTaps][d] = 0;
+        vxi o;
+#pragma unroll
+        for (int d = 0; d < kDw; ++d) {
             int32_t code[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -122,28 +151,13 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
                     acc = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, xp), __builtin_bit_cast(v2s, wp[q][ch]), acc, false);
                 }
                 float v = (float)acc * sc[ch];
-                if (float_bias) v = v + a.fbias[c0 + ch];
+                if (kFloatBias) v = v + fb[ch];
                 code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
             }
-            out[d] = pack4(code[0], code[1], code[2], code[3]);
+            o[d] = (int)pack4(code[0], code[1], code[2], code[3]);
         }
-        const v4i o = {(int)out[0], (int)out[1], (int)out[2], (int)out[3]};
-        *reinterpret_cast<v4i*>(yrow + (int64_t)ow * a.y_w_stride) = o;
+        *reinterpret_cast<vxi*>(yrow + (int64_t)ow * a.y_w_stride) = o;
     }
-}
-
-// seed[c] = -zp_u * wsum[c] (+ bias, ONNX mode); scale[c] = x_scale * w_scale[c]; fbias[c] = float(bias[c])
-__global__ __launch_bounds__(256) void depthwise_params_kernel(
-        int C, const int32_t* __restrict__ wsum, int32_t zp_u, const float* __restrict__ w_scale, int w_scale_len,
-        float x_scale, const int32_t* __restrict__ bias, int bias_mode, int32_t* __restrict__ seed,
-        float* __restrict__ scale, float* __restrict__ fbias) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
-    int32_t sd = -zp_u * wsum[c];
-    if (bias && bias_mode == kBiasOnnxInt32) sd += bias[c];
-    seed[c] = sd;
-    scale[c] = x_scale * (w_scale_len > 1 ? w_scale[c] : w_scale[0]);
-    fbias[c] = (bias && bias_mode == kBiasReferenceFloat) ? (float)bias[c] : 0.f;
 }
 
 }  // namespace
@@ -155,23 +169,22 @@ int pack_depthwise(const chx_hip_tensor& w, int32_t* pairs, int32_t* wsum, hipSt
     return launch_check("pack_depthwise_kernel");
 }
 
-int launch_depthwise_params(
-        int C, const int32_t* wsum, int32_t zp_u, const float* w_scale, int w_scale_len, float x_scale, const int32_t* bias,
-        int bias_mode, int32_t* seed, float* scale, float* fbias, hipStream_t s) {
-    depthwise_params_kernel<<<(C + 255) / 256, 256, 0, s>>>(C, wsum, zp_u, w_scale, w_scale_len, x_scale, bias, bias_mode, seed,
-                                                            scale, fbias);
-    return launch_check("depthwise_params_kernel");
-}
-
 int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
     a.ow_blocks = (a.OW + kDwPixels - 1) / kDwPixels;
-    a.total = (int64_t)a.N * a.OH * a.ow_blocks * (a.C / 16);
+    a.total = (int64_t)a.N * a.OH * a.ow_blocks * (a.C / kCh);
     if (a.total == 0) return CHX_HIP_OK;
     const unsigned blocks = (unsigned)((a.total + 255) / 256);
-    if (rne)
-        depthwise3x3_kernel<true><<<blocks, 256, 0, s>>>(a);
-    else
-        depthwise3x3_kernel<false><<<blocks, 256, 0, s>>>(a);
+    const bool fbias = a.bias != nullptr && a.float_bias != 0;
+    const bool xs = a.x_signed != 0;
+#define CHX_DW(RN, FB, XS) depthwise3x3_kernel<RN, FB, XS><<<blocks, 256, 0, s>>>(a)
+    if (rne) {
+        if (fbias) { if (xs) CHX_DW(true, true, true); else CHX_DW(true, true, false); }
+        else { if (xs) CHX_DW(true, false, true); else CHX_DW(true, false, false); }
+    } else {
+        if (fbias) { if (xs) CHX_DW(false, true, true); else CHX_DW(false, true, false); }
+        else { if (xs) CHX_DW(false, false, true); else CHX_DW(false, false, false); }
+    }
+#undef CHX_DW
     return launch_check("depthwise3x3_kernel");
 }
 
