@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every op from the host instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one plain copy kernel (fused Identity on float32) over this many MiB: the known traffic "
+                         "that hardware counters of a profiling run are scaled against")
     return ap.parse_args()
 
 
@@ -331,6 +334,12 @@ def main():
         res, roofline, cpu, close = bench_conv3x3(args, torch, pkg)
     else:
         res, roofline, cpu, close = bench_fusion(args, torch, pkg, qdq=args.workload == "qdq")
+    if args.copy_probe_mib:
+        n = args.copy_probe_mib * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda")
+        code = pkg.ops.fusion_program([("x", torch.float32)], [("y", "Identity", "x")], [("y", torch.float32)])
+        pkg.ops.ElementWiseNvrtc([src], 1, code, 9999)
+        torch.cuda.synchronize()
     out = dict(res)
     out.update(n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak", vs_baseline=None,
                data="synthetic", roofline=roofline)

@@ -175,6 +175,7 @@ struct PackedWeights {
     int8_t* wp = nullptr;
     int32_t* wsum = nullptr;
     int C64 = 0, OCpad = 0, KP = 0;
+    int BK = 64;         // K bytes per kernel step; the packed layout depends on it
     bool dense = false;  // taps packed densely; activations go through an explicit im2col
 };
 
@@ -193,6 +194,8 @@ size_t packed_bytes(int OC, int C, int KH, int KW, PackedWeights* pw) {
         pw->C64 = round_up(C, 64);
         pw->KP = KH * KW * pw->C64;
     }
+    // whole cache lines per pixel and step when the channels allow it
+    pw->BK = (!pw->dense && pw->C64 % 128 == 0) ? 128 : 64;
     return (size_t)pw->OCpad * pw->KP;
 }
 
@@ -470,7 +473,8 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.M = (int64_t)cs.N * cs.OH * cs.OW;
     a.OC = cs.OC;
     a.KP = pw.KP;
-    a.nk = pw.KP / 64;
+    a.bk = pw.BK;
+    a.nk = pw.KP / pw.BK;
     a.wp = pw.wp;
     a.wsum = pw.wsum;
     a.x_zp = c.x_zp;
@@ -564,8 +568,8 @@ int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedW
     }
     pw->wp = static_cast<int8_t*>(p0);
     pw->wsum = static_cast<int32_t*>(p1);
-    if (pw->dense) return pack_weights_dense(w, pw->KP, pw->OCpad, pw->wp, pw->wsum, s);
-    return pack_weights(w, pw->C64, pw->OCpad, pw->wp, pw->wsum, s);
+    if (pw->dense) return pack_weights_dense(w, pw->KP, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
+    return pack_weights(w, pw->C64, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
 }
 
 void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {

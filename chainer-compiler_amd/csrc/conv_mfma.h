@@ -16,9 +16,10 @@ struct ConvMfmaArgs {
     int32_t H, W, OH, OW, KH, KW, sh, sw, ph, pw;
     int64_t M;    // N * OH * OW
     int32_t OC;
-    int32_t nk;   // K steps: KH * KW * C64 / 64
+    int32_t bk;   // K bytes per step: 64, or 128 when C64 is a multiple of 128
+    int32_t nk;   // K steps: KP / bk
     int32_t KP;   // packed row length: KH * KW * C64
-    const int8_t* wp;     // [OCpad][KP]
+    const int8_t* wp;     // [OCpad / 64][nk][64][bk]
     const int32_t* wsum;  // [OCpad]
     int32_t x_zp;
     int32_t corr_mult;    // (128 - x_zp) for uint8 x, (-x_zp) for int8 x
@@ -55,9 +56,9 @@ inline void magic_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
     *shift = l;
 }
 
-int pack_weights_dense(const chx_hip_tensor& w, int Kd, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+int pack_weights_dense(const chx_hip_tensor& w, int Kd, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 int launch_im2col_dense(const Im2colArgs& a, hipStream_t s);
-int pack_weights(const chx_hip_tensor& w, int C64, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+int pack_weights(const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 // max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once)
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s);

@@ -38,17 +38,22 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kBK = 64;  // K bytes per step
+// Packed weights are stored in blocks that one K step of the kernel reads as whole cache
+// lines: Wp[oc / 64][k / BK][oc % 64][k % BK] with BK = 64 or 128 K-bytes per step, i.e. the 64
+// rows of a block are BK contiguous bytes each and a block is 64 * BK contiguous bytes.
+__host__ __device__ __forceinline__ int64_t packed_offset(int oc, int k, int KP, int BK) {
+    return ((int64_t)(oc >> 6) * (KP / BK) + k / BK) * (64 * BK) + (oc & 63) * BK + k % BK;
+}
 
 // ---------------------------------------------------------------------------------------------
-// Weight repacking: w [OC][C][KH][KW] (any strides) -> Wp [OCpad][KH*KW][C64] and
-// wsum[oc] = sum of the row.  One work-group per output channel.
+// Weight repacking: w [OC][C][KH][KW] (any strides) -> Wp, K index k = (kh*KW + kw)*C64 + c with
+// C64 = C rounded up to 64 (zero filled), and wsum[oc] = sum of the row.  One work-group per
+// output channel.
 __global__ __launch_bounds__(256) void pack_weights_kernel(
         const char* __restrict__ w, int64_t s_oc, int64_t s_c, int64_t s_kh, int64_t s_kw, int OC, int C, int KH, int KW,
-        int C64, int8_t* __restrict__ wp, int32_t* __restrict__ wsum) {
+        int C64, int BK, int8_t* __restrict__ wp, int32_t* __restrict__ wsum) {
     const int oc = blockIdx.x;
     const int KP = KH * KW * C64;
-    int8_t* dst = wp + (int64_t)oc * KP;
     int32_t local = 0;
     for (int k = threadIdx.x; k < KP; k += 256) {
         const int c = k % C64;
@@ -58,7 +63,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
             const int kh = pos / KW, kw = pos % KW;
             v = *reinterpret_cast<const int8_t*>(w + oc * s_oc + c * s_c + kh * s_kh + kw * s_kw);
         }
-        dst[k] = v;
+        wp[packed_offset(oc, k, KP, BK)] = v;
         local += v;
     }
     __shared__ int32_t red[256];
@@ -79,9 +84,8 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
 // holds anything (its weights are zero).
 __global__ __launch_bounds__(256) void pack_weights_dense_kernel(
         const char* __restrict__ w, int64_t s_oc, int64_t s_c, int64_t s_kh, int64_t s_kw, int OC, int C, int KH, int KW,
-        int Kd, int8_t* __restrict__ wp, int32_t* __restrict__ wsum) {
+        int Kd, int BK, int8_t* __restrict__ wp, int32_t* __restrict__ wsum) {
     const int oc = blockIdx.x;
-    int8_t* dst = wp + (int64_t)oc * Kd;
     const int K = KH * KW * C;
     int32_t local = 0;
     for (int k = threadIdx.x; k < Kd; k += 256) {
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(256) void pack_weights_dense_kernel(
             const int kh = pos / KW, kw = pos % KW;
             v = *reinterpret_cast<const int8_t*>(w + oc * s_oc + c * s_c + kh * s_kh + kw * s_kw);
         }
-        dst[k] = v;
+        wp[packed_offset(oc, k, Kd, BK)] = v;
         local += v;
     }
     __shared__ int32_t red[256];
@@ -214,8 +218,12 @@ __global__ __launch_bounds__(256) void im2col_dense_lds_kernel(Im2colArgs a, int
 }
 
 // ---------------------------------------------------------------------------------------------
+// Byte offset of K chunk kc (16 bytes) of a staged row.  The chunks of a row are XOR-swizzled
+// with row bits so that 128-bit fragment reads of consecutive rows fall on distinct banks:
+// rows of 64 bytes (4 chunks) with bits 2..3, rows of 128 bytes (8 chunks) with bits 1..3.
+template <int BK>
 __device__ __forceinline__ int lds_chunk_offset(int row, int kc) {
-    return row * kBK + ((kc ^ ((row >> 2) & 3)) << 4);
+    return BK == 64 ? row * 64 + ((kc ^ ((row >> 2) & 3)) << 4) : row * 128 + ((kc ^ ((row >> 1) & 7)) << 4);
 }
 
 // Row b (64 bytes) holds the byte b in every position.  A filter tap outside the image fetches
@@ -253,6 +261,29 @@ __device__ __forceinline__ void async_copy16(const void* src, uint32_t lds_addr)
             : "memory", "m0");
 }
 
+// 128-bit LDS read whose completion the caller waits for itself (wait_fragments): the compiler
+// would otherwise wait for every outstanding LDS operation at the first use, because it cannot
+// see through the inline assembly of the copies issued in between.
+__device__ __forceinline__ v4i lds_read16_nowait(uint32_t lds_addr) {
+    v4i v;
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(v) : "v"(lds_addr) : "memory");
+    return v;
+}
+
+// Wait until at most N LDS/scalar-memory operations of this wave are outstanding; the fragment
+// registers pass through so that their uses are ordered after the wait.
+template <int N, int FM, int FN>
+__device__ __forceinline__ void wait_fragments(v4i (&fa)[FM], v4i (&fb)[FN]) {
+    if constexpr (FM == 2 && FN == 2)
+        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]), "+v"(fb[1]) : "n"(N) : "memory");
+    else if constexpr (FM == 2 && FN == 1)
+        asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fb[0]) : "n"(N) : "memory");
+    else if constexpr (FM == 1 && FN == 2)
+        asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(fa[0]), "+v"(fb[0]), "+v"(fb[1]) : "n"(N) : "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fa[0]), "+v"(fb[0]) : "n"(N) : "memory");
+}
+
 // Wait until at most N of this wave's vector-memory operations are outstanding.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -266,32 +297,38 @@ __device__ __forceinline__ void wait_vmcnt() {
 // px_first, px_first + px_step, ...  The sequence of (pixel tile, K step) pairs is one flat
 // pipeline over a ring of NS LDS stages: the asynchronous copies run NS-1 steps ahead of the
 // MFMAs and cross tile boundaries, so the operands of the next tile are in flight while the
-// current tile is requantized and written out.  Per K step a wave issues FM + FN copy
-// instructions, reads its fragments back with 128-bit LDS loads, flips the sign bits of uint8
-// activations on the fragments, and feeds 2*FM*FN MFMAs; one barrier per step.
+// current tile is requantized and written out.  Per K step (BK = 64 or 128 K-bytes) a wave
+// issues (FM + FN) * BK/64 copy instructions, reads its fragments back with 128-bit LDS loads,
+// flips the sign bits of uint8 activations on the fragments, and feeds FM*FN*BK/32 MFMAs; one
+// barrier per step.
 //
-// LDS stage: rows of 64 K-bytes, weight rows first, then pixel rows.  A copy instruction fills
-// 1 KB = 16 consecutive rows; lane l lands in row l/4, slot l%4 and therefore fetches K chunk
-// (l%4) ^ ((l/16)%4) of that row, which is the XOR swizzle lds_chunk_offset() undoes on the
-// read side (bank-conflict-free 128-bit fragment reads).
+// LDS stage: rows of BK K-bytes, weight rows first, then pixel rows.  A copy instruction fills
+// 1 KB = 1024/BK consecutive rows; a lane lands in a fixed (row, slot) and fetches the K chunk
+// that the XOR swizzle of lds_chunk_offset() places there, so the 128-bit fragment reads are
+// free of bank conflicts.  BK = 128 is used when the channel count is a multiple of 128: then a
+// pixel's 128 K-bytes of one filter tap are one whole cache line, where two 64-byte steps
+// would each fetch the line and use half of it (the weight blocks are contiguous either way).
 //
 // kPad: some filter tap can fall outside the image, or the channel count is not a multiple
 // of 64.  Then each staged row carries a bit mask of its valid taps (computed once per pixel
 // tile) and an invalid chunk is fetched from a 64-byte row holding the zero point instead
 // (g_fill_rows), which makes it contribute (zp - zp) * w = 0.  Without kPad (1x1 and other
 // unpadded convolutions on 64-multiple channels, matrix products) every chunk is valid.
-template <int FM, int FN, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad>
+template <int FM, int FN, int BK, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv_mfma_kernel(ConvMfmaArgs a) {
     constexpr int T = 256;
     constexpr int TM = 64 * FM;  // output channels per tile
     constexpr int TN = 64 * FN;  // pixels per tile
-    constexpr int NS = 3;        // LDS stages
-    constexpr int STAGE_BYTES = (TM + TN) * kBK;
-    constexpr int COPIES = FM + FN;     // copy instructions per wave and stage
-    constexpr int OUT_PITCH = TM + 16;  // staging row pitch in bytes, keeps 16-byte alignment
-    constexpr int LDS_OUT = kOutInt32 ? 16 : TN * OUT_PITCH;
+    constexpr int STAGE_BYTES = (TM + TN) * BK;
+    constexpr int NS = 3 * STAGE_BYTES <= 80 * 1024 ? 3 : 2;  // LDS stages: two work-groups per compute unit
+    constexpr int CH = BK / 16;          // 16-byte chunks per staged row
+    constexpr int RPI = 64 / CH;         // rows one copy instruction fills
+    constexpr int CA = TM / RPI / 4;     // copy instructions per wave and stage, weight rows
+    constexpr int CB = TN / RPI / 4;     //   ... pixel rows
+    constexpr int COPIES = CA + CB;
+    constexpr int OUT_CHUNKS = TM / 16;  // 16-byte chunks per staged output row
+    static_assert(TN * TM <= STAGE_BYTES, "the output tile is staged in one ring slot");
     __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_out[LDS_OUT];
     __shared__ __attribute__((aligned(16))) float s_scale[TM];
     __shared__ __attribute__((aligned(16))) int32_t s_add[TM];
     __shared__ __attribute__((aligned(16))) float s_fbias[TM];
@@ -320,30 +357,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     const int total_stages = my_tiles * nk;
     if (total_stages == 0) return;
 
-    // rows this thread copies per stage: row0 + 64*j of the weight tile and of the pixel tile,
-    // K chunk kc of each
-    const int row0 = tid >> 2;
-    const int kc = (lane & 3) ^ ((lane >> 4) & 3);
-    const int8_t* wp_row[FM];
+    // rows this thread copies per stage: row0 + 4*RPI*j of the weight tile and of the pixel tile,
+    // K chunk kc of each (the chunk whose swizzled slot is lane % CH; it is the same for all j)
+    const int row0 = wave * RPI + lane / CH;
+    const int kc = BK == 64 ? (lane & 3) ^ ((lane >> 4) & 3) : (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+    const int8_t* wp_row[CA];
 #pragma unroll
-    for (int j = 0; j < FM; ++j) wp_row[j] = a.wp + (int64_t)(oc0 + row0 + 64 * j) * a.KP + kc * 16;
-    const char* fill_src = reinterpret_cast<const char*>(g_fill_rows) + (a.x_zp & 0xff) * 64 + kc * 16;
-    const uint32_t ring_addr = (uint32_t)(uintptr_t)ring + (uint32_t)wave * 1024u;  // LDS byte address
+    for (int j = 0; j < CA; ++j) wp_row[j] = a.wp + packed_offset(oc0 + row0 + 4 * RPI * j, kc * 16, a.KP, BK);
+    const char* fill_src = reinterpret_cast<const char*>(g_fill_rows) + (a.x_zp & 0xff) * 64 + (kc & 3) * 16;
+    const uint32_t ring_base = (uint32_t)(uintptr_t)ring;             // LDS byte address
+    const uint32_t ring_addr = ring_base + (uint32_t)wave * 1024u;
 
     // ---- copy side state: which (pixel tile, K step) the next stage fetches ----
-    const char* xb[FN];
+    const char* xb[CB];
     int ld_tile = px_first;
     int ld_k = 0, kh = 0, kw = 0, c0 = 0, kofs = 0;
     int64_t tap_off = 0;  // kh * x_h_stride + kw * x_w_stride
 
-    uint64_t tapmask[FN];  // kPad: bit (kh*KW + kw) set when that tap of the row's pixel is inside the image
+    uint64_t tapmask[CB];  // kPad: bit (kh*KW + kw) set when that tap of the row's pixel is inside the image
     int tap = 0;
 
     auto set_load_tile = [&]() {
         const int64_t mbase = (int64_t)ld_tile * TN + row0;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int64_t m = mbase + 64 * j;
+        for (int j = 0; j < CB; ++j) {
+            const int64_t m = mbase + 4 * RPI * j;
             const bool row_ok = m < a.M && ld_tile < px_hi;
             // rows past the end re-read the last pixel; they are never written back
             const uint32_t mm = m < a.M ? (uint32_t)m : (uint32_t)(a.M - 1);  // M fits 31 bits (checked on the host)
@@ -372,22 +410,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     // Every stage issues the same number of copies and none is conditional, so a fixed
     // vector-memory count identifies the stage about to be consumed.  Stages past the end of
     // this work-group's list re-read the last K step into a ring slot nobody reads again.
-    auto issue_stage = [&](int buf) {
+    // copy number q of the stage being fetched: the weight rows come first, then the pixel rows
+    auto issue_copy = [&](int buf, int q) {
         const uint32_t dst = ring_addr + (uint32_t)buf * STAGE_BYTES;
-#pragma unroll
-        for (int j = 0; j < FM; ++j) async_copy16(wp_row[j] + kofs, dst + j * 4096);
-        if (kPad) {
-            const bool c_ok = c0 + kc * 16 < a.C16;
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const bool ok = c_ok && ((tapmask[j] >> tap) & 1u);
-                async_copy16(ok ? xb[j] + tap_off + c0 : fill_src, dst + TM * kBK + j * 4096);
-            }
+        if (q < CA) {
+            async_copy16(wp_row[q] + kofs, dst + q * 4096);
         } else {
-#pragma unroll
-            for (int j = 0; j < FN; ++j) async_copy16(xb[j] + tap_off + c0, dst + TM * kBK + j * 4096);
+            const int j = q - CA;
+            bool ok = true;
+            if (kPad) ok = c0 + kc * 16 < a.C16 && ((tapmask[j] >> tap) & 1u);
+            async_copy16(ok ? xb[j] + tap_off + c0 : fill_src, dst + TM * BK + j * 4096);
         }
-        // advance to the next K step, or to the first K step of this work-group's next pixel tile
+    };
+    // advance to the next K step, or to the first K step of this work-group's next pixel tile
+    auto advance_stage = [&]() {
         if (++ld_k == nk) {
             if (ld_tile + px_step < px_hi) {
                 ld_k = 0; kh = 0; kw = 0; c0 = 0; kofs = 0; tap_off = 0; tap = 0;
@@ -397,8 +433,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                 --ld_k;  // nothing follows: keep fetching the last step
             }
         } else {
-            kofs += kBK;
-            c0 += kBK;
+            kofs += 64 * BK;  // next block of the packed weights
+            c0 += BK;
             if (c0 >= a.C64) {
                 c0 = 0;
                 ++tap;
@@ -414,7 +450,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 
     // the first NS-1 stages go out before anything else touches memory
 #pragma unroll
-    for (int d = 0; d < NS - 1; ++d) issue_stage(d);
+    for (int d = 0; d < NS - 1; ++d) {
+#pragma unroll
+        for (int q = 0; q < COPIES; ++q) issue_copy(d, q);
+        advance_stage();
+    }
 
     // per-channel epilogue constants; s_add seeds the accumulators
     for (int i = tid; i < TM; i += T) {
@@ -456,7 +496,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     seed_acc();
 
     // ---- epilogue of one finished pixel tile ----
-    auto epilogue = [&](int px_tile) {
+    // The 8-bit tile is transposed through the ring slot that was just consumed (the copies in
+    // flight target the other slots): rows of TM bytes per pixel, the 16-byte chunks of a row
+    // XOR-swizzled with bits 1.. of the pixel index so that neither the 4-byte writes of the
+    // accumulator layout nor the 16-byte reads of the store loop pile up on a bank.
+    auto staged = [&](char* slot, int pxl, int ocl) -> char* {
+        return slot + pxl * TM + ((((ocl >> 4) ^ (pxl >> 1)) & (OUT_CHUNKS - 1)) << 4) + (ocl & 15);
+    };
+    auto epilogue = [&](int px_tile, char* lds_out) {
         const int64_t m0 = (int64_t)px_tile * TN;
         if (kOutInt32) {
 #pragma unroll
@@ -505,26 +552,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                             if (kFloatBias) v = v + fb[e];  // reference mode: float bias after the scale multiply
                             code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
                         }
-                        *reinterpret_cast<uint32_t*>(lds_out + pxl * OUT_PITCH + ocl) = pack4(code[0], code[1], code[2], code[3]);
+                        *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
                     }
                 }
         };
+        __syncthreads();  // every wave is done reading the slot's operands
         if (a.rq.bias_mode == kBiasReferenceFloat) requantize_tile(std::true_type());
         else requantize_tile(std::false_type());
         __syncthreads();
-        constexpr int CHUNKS_PER_ROW = TM / 16;
-        for (int q = tid; q < TN * CHUNKS_PER_ROW; q += T) {
-            const int pxl = q / CHUNKS_PER_ROW;
-            const int ch = q % CHUNKS_PER_ROW;
+        for (int q = tid; q < TN * OUT_CHUNKS; q += T) {
+            const int pxl = q / OUT_CHUNKS;
+            const int ch = q % OUT_CHUNKS;
             const int64_t m = m0 + pxl;
             const int oc = oc0 + ch * 16;
             if (m >= a.M || oc >= a.OC) continue;
-            const v4i val = *reinterpret_cast<const v4i*>(lds_out + pxl * OUT_PITCH + ch * 16);
+            const char* src = staged(lds_out, pxl, ch * 16);
+            const v4i val = *reinterpret_cast<const v4i*>(src);
             char* dst = a.y + m * a.y_px_stride + oc;
             if (a.y_vec_ok && oc + 16 <= a.OC) {
                 *reinterpret_cast<v4i*>(dst) = val;
             } else {
-                const char* src = lds_out + pxl * OUT_PITCH + ch * 16;
 #pragma nounroll
                 for (int e = 0; e < 16 && oc + e < a.OC; ++e) dst[e] = src[e];
             }
@@ -543,36 +590,53 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         // everybody is done reading the slot the next copies overwrite
         wait_vmcnt<(NS - 2) * COPIES>();
         __syncthreads();
-        issue_stage(lbuf);
-        lbuf = lbuf + 1 == NS ? 0 : lbuf + 1;
 
-        const char* sa = ring + cbuf * STAGE_BYTES;
-        const char* sb = sa + TM * kBK;
+        char* slot = ring + cbuf * STAGE_BYTES;
+        const char* sa = slot;
+        const char* sb = sa + TM * BK;
         cbuf = cbuf + 1 == NS ? 0 : cbuf + 1;
-        v4i fa[2][FM], fb[2][FN];
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
+        // The copies of the stage NS-1 steps ahead are issued between the MFMA groups rather than
+        // in one burst: the copy unit takes a 1 KB instruction every 16 cycles or so, and a wave
+        // that issues them back to back sits in the queue instead of feeding the matrix cores.
+        constexpr int SUBS = BK / 32;  // MFMA K extents per stage
+        constexpr int PER_SUB = (COPIES + SUBS - 1) / SUBS;
+        v4i fa[SUBS][FM], fb[SUBS][FN];
+        const uint32_t sa_addr = ring_base + (uint32_t)(slot - ring);
+        auto read_fragments = [&](int sub) {
 #pragma unroll
             for (int i = 0; i < FM; ++i)
-                fa[sub][i] = *reinterpret_cast<const v4i*>(
-                        sa + lds_chunk_offset(wm * 32 * FM + i * 32 + frag_row, sub * 2 + frag_kc));
+                fa[sub][i] = lds_read16_nowait(sa_addr + lds_chunk_offset<BK>(wm * 32 * FM + i * 32 + frag_row, sub * 2 + frag_kc));
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                v4i v = *reinterpret_cast<const v4i*>(
-                        sb + lds_chunk_offset(wn * 32 * FN + j * 32 + frag_row, sub * 2 + frag_kc));
-                if (kXUnsigned) v ^= (int)0x80808080;  // uint8 code - 128 as int8
-                fb[sub][j] = v;
-            }
-        }
+            for (int j = 0; j < FN; ++j)
+                fb[sub][j] = lds_read16_nowait(sa_addr + TM * BK +
+                                               lds_chunk_offset<BK>(wn * 32 * FN + j * 32 + frag_row, sub * 2 + frag_kc));
+        };
+        // all reads of the stage go out at once; LDS reads complete in order, so extent sub is
+        // there when at most the reads of the later extents are outstanding
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub)
+        for (int sub = 0; sub < SUBS; ++sub) read_fragments(sub);
+#pragma unroll
+        for (int sub = 0; sub < SUBS; ++sub) {
+            if (sub == 0) wait_fragments<(SUBS - 1) * (FM + FN)>(fa[sub], fb[sub]);
+            else if (sub == 1) wait_fragments<(SUBS > 2 ? SUBS - 2 : 0) * (FM + FN)>(fa[sub], fb[sub]);
+            else if (sub == 2) wait_fragments<(SUBS > 3 ? SUBS - 3 : 0) * (FM + FN)>(fa[sub], fb[sub]);
+            else wait_fragments<0>(fa[sub], fb[sub]);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                if (kXUnsigned) fb[sub][j] ^= (int)0x80808080;  // uint8 code - 128 as int8
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[sub][i], fb[sub][j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int q = sub * PER_SUB; q < (sub + 1) * PER_SUB && q < COPIES; ++q) issue_copy(lbuf, q);
+            __builtin_amdgcn_sched_barrier(0);  // keep the read / MFMA / copy interleaving as written
+        }
+        advance_stage();
+        lbuf = lbuf + 1 == NS ? 0 : lbuf + 1;
         if (++ck == nk) {
-            epilogue(c_tile);
+            epilogue(c_tile, slot);
             seed_acc();
             ck = 0;
             c_tile += px_step;
@@ -581,7 +645,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     wait_vmcnt<0>();  // the copies past the end still target this work-group's LDS
 }
 
-template <int FM, int FN>
+template <int FM, int FN, int BK>
 int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool rne, int max_wgs_per_cu, hipStream_t s) {
     // persistent work-groups: as many as the device holds at once, a whole number per
     // output-channel tile
@@ -594,7 +658,7 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
         }
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, true, false, false, true>), 256, 0) !=
+                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, BK, true, false, false, true>), 256, 0) !=
                     hipSuccess ||
             per_cu < 1)
             per_cu = 2;
@@ -605,14 +669,14 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
     if (slots > cap) slots = cap;
     const unsigned grid = (unsigned)(8 * a.tiles_oc * slots);
     // padding-free variant: no tap can leave the image and channels fill whole 64-byte K steps
-    const bool pad = a.ph != 0 || a.pw != 0 || (a.C16 % 64) != 0 ||
+    const bool pad = a.ph != 0 || a.pw != 0 || (a.C16 % BK) != 0 ||
                      (int64_t)(a.OH - 1) * a.sh + a.KH > a.H || (int64_t)(a.OW - 1) * a.sw + a.KW > a.W;
 #define CHX_LAUNCH(XU, OI, RN)                                                           \
     do {                                                                                 \
         if (pad)                                                                         \
-            conv_mfma_kernel<FM, FN, XU, OI, RN, true><<<grid, 256, 0, s>>>(a);          \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, true><<<grid, 256, 0, s>>>(a);      \
         else                                                                             \
-            conv_mfma_kernel<FM, FN, XU, OI, RN, false><<<grid, 256, 0, s>>>(a);         \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, false><<<grid, 256, 0, s>>>(a);     \
     } while (0)
     if (out_int32) {
         if (x_unsigned) CHX_LAUNCH(true, true, false);
@@ -631,17 +695,17 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
 }  // namespace
 
 int pack_weights(
-        const chx_hip_tensor& w, int C64, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s) {
+        const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s) {
     pack_weights_kernel<<<OCpad, 256, 0, s>>>(
             static_cast<const char*>(w.data), w.strides[0], w.strides[1], w.strides[2], w.strides[3], (int)w.shape[0],
-            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, wp, wsum);
+            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, BK, wp, wsum);
     return launch_check("pack_weights_kernel");
 }
 
-int pack_weights_dense(const chx_hip_tensor& w, int Kd, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s) {
+int pack_weights_dense(const chx_hip_tensor& w, int Kd, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s) {
     pack_weights_dense_kernel<<<OCpad, 256, 0, s>>>(
             static_cast<const char*>(w.data), w.strides[0], w.strides[1], w.strides[2], w.strides[3], (int)w.shape[0],
-            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], Kd, wp, wsum);
+            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], Kd, BK, wp, wsum);
     return launch_check("pack_weights_dense_kernel");
 }
 
@@ -668,10 +732,14 @@ int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_c
     if (a.M == 0 || a.OC == 0) return CHX_HIP_OK;
     magic_divisor((uint32_t)a.OW, &a.ow_mul, &a.ow_shift);
     magic_divisor((uint32_t)a.OH, &a.oh_mul, &a.oh_shift);
-    if (tile_oc == 128 && tile_px == 128) return launch_config<2, 2>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
-    if (tile_oc == 64 && tile_px == 128) return launch_config<1, 2>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
-    if (tile_oc == 128 && tile_px == 64) return launch_config<2, 1>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
-    if (tile_oc == 64 && tile_px == 64) return launch_config<1, 1>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 128 && tile_px == 128) return a.bk == 128 ? launch_config<2, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
+                           : launch_config<2, 2, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 64 && tile_px == 128) return a.bk == 128 ? launch_config<1, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
+                           : launch_config<1, 2, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 128 && tile_px == 64) return a.bk == 128 ? launch_config<2, 1, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
+                           : launch_config<2, 1, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+    if (tile_oc == 64 && tile_px == 64) return a.bk == 128 ? launch_config<1, 1, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
+                           : launch_config<1, 1, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
     CHX_FAIL(CHX_HIP_EINVAL, "conv_mfma: no kernel for a %dx%d tile", tile_oc, tile_px);
 }
 
