@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every op from the host instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline")
+    ap.add_argument("--parts", type=int, default=1,
+                    help="run the batch as this many concurrent slices on separate streams (network workloads)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one plain copy kernel (fused Identity on float32) over this many MiB: the known traffic "
                          "that hardware counters of a profiling run are scaled against")
@@ -99,20 +101,27 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     batch = args.batch or (128 if mobilenet else 64)
     build = (lambda **kw: wl.build_mobilenetv2(seed=4, **kw)) if mobilenet else (lambda **kw: wl.build_resnet50(seed=3, **kw))
     model = build(batch=batch)
-    runner = wl.DeviceRunner(model, pkg)
     x = torch.from_numpy(model["input"]).cuda()
     ops, capi = pkg.ops, pkg.capi
     conv_ops = 2.0 * model["macs"]
 
+    # --parts N runs the batch as N concurrent slices on separate streams (the values are those of
+    # the whole-batch run; a single ResNet layer at batch 64 is too few work-groups to keep 256
+    # compute units busy through its ramp and tail, so slices fill each other's gaps).  The
+    # default is the plain whole-batch runner, whose launches are the ones the roofline figure
+    # below prices.
+    runner = wl.DeviceRunner(model, pkg) if args.parts <= 1 else None
+    timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts)
+
     def step(_timer):
-        runner.run(x)
+        timed_runner.run(x)
 
     # The timed region replays the whole program as one HIP graph (about 125 launches per step
     # would otherwise be bound by the host); --no-graph launches every op from the host instead.
     if args.no_graph:
         sec = timed_steps(torch, step, args.steps, args.warmup)
     else:
-        replay = runner.capture(x)
+        replay = timed_runner.capture(x)
         sec = timed_steps(torch, lambda _t: replay(), args.steps, args.warmup)
 
     # Launch duration of the dominant kernel: event pairs cannot be recorded inside a graph
@@ -122,32 +131,35 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # goes first so that the host is done submitting before the GPU starts.  The per-step
     # kernel time is the sum of the per-instruction averages.
     REP = 20
-    vals = runner.run(x)
-    torch.cuda.synchronize()
+    # the launches timed are those of the timed region: one slice's instructions, times the slices
+    slices = [(runner, x)] if args.parts <= 1 else [(r, x[lo:hi]) for (lo, hi), r in zip(timed_runner.slices, timed_runner.runners)]
     conv_ms_per_step, n_launch = 0.0, 0
     pairs = []
-    for ins in model["program"]:
-        if ins[0] != "QLinearConv":
-            continue
-        c = model["convs"][ins[3]]
-        if mobilenet and c.group == 1:
-            continue  # MobileNetV2: the roofline figure is the depthwise kernel's
-        fn = lambda: runner.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
-                                              flags=capi.BIAS_ONNX_INT32, out=runner.bufs[ins[1]])
-        torch.cuda._sleep(int(2.4e9 * 0.002))
-        a = torch.cuda.Event(enable_timing=True)
-        b = torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(REP):
-            fn()
-        b.record()
-        pairs.append((ins[3], a, b))
-        n_launch += 1
+    for rn, xs in slices:
+        vals = rn.run(xs)
+        torch.cuda.synchronize()
+        for ins in model["program"]:
+            if ins[0] != "QLinearConv":
+                continue
+            c = model["convs"][ins[3]]
+            if mobilenet and c.group == 1:
+                continue  # MobileNetV2: the roofline figure is the depthwise kernel's
+            fn = lambda: rn.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
+                                              flags=capi.BIAS_ONNX_INT32, out=rn.bufs[ins[1]])
+            torch.cuda._sleep(int(2.4e9 * 0.002))
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(REP):
+                fn()
+            b.record()
+            pairs.append((ins[3], a, b))
+            n_launch += 1
     torch.cuda.synchronize()
     per_layer = {}
     for name, a, b in pairs:
         ms = a.elapsed_time(b) / REP
-        per_layer[name] = ms
+        per_layer[name] = per_layer.get(name, 0.0) + ms
         conv_ms_per_step += ms
     if mobilenet:
         achieved = model["depthwise_bytes"] / (conv_ms_per_step * 1e-3) / 1e9
@@ -163,6 +175,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
                config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,
                            layout="channels_last", launch="host" if args.no_graph else "hip_graph_replay",
+                           concurrent_batch_slices=max(1, args.parts),
                            conv_gmac_per_image=model["macs"] / batch / 1e9))
 
     def cpu():
@@ -186,7 +199,8 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                     sample="%d images of the same network (batch %d), restated reference op sequence (fp32 dequantize, "
                            "im2col + sequential-k fp32 GEMM, quantize) with OpenMP over %d threads: %.1f s; one image "
                            "single-threaded, as ChainerX's native device runs: %.1f s" % (nb, nb, cores, dtn, dt1))
-    runner_close = runner.close
+    def runner_close():
+        timed_runner.close()
     return res, roofline, cpu, runner_close
 
 

@@ -364,6 +364,59 @@ class DeviceRunner(object):
             p.close()
 
 
+def slice_model(model, lo, hi):
+    """The same program on images lo..hi-1 of the batch (weights and quantization parameters are
+    shared; only the shapes and the input change)."""
+    sub = dict(model)
+    sub["shapes"] = {k: (hi - lo,) + tuple(v[1:]) for k, v in model["shapes"].items()}
+    sub["input"] = model["input"][lo:hi]
+    return sub
+
+
+class ConcurrentRunner(object):
+    """Runs the batch as `parts` independent slices, each on its own stream with its own plans and
+    buffers.  Inference is independent per image, so the values are those of the whole-batch
+    run; the point is occupancy: one ResNet layer at batch 64 is a few hundred work-groups, too
+    few to keep 256 compute units busy through its ramp and tail, and the slices' kernels fill
+    each other's gaps."""
+
+    def __init__(self, model, pkg, parts=2):
+        n = model["shapes"]["x"][0]
+        bounds = [n * i // parts for i in range(parts + 1)]
+        self.slices = [(bounds[i], bounds[i + 1]) for i in range(parts) if bounds[i + 1] > bounds[i]]
+        self.runners = [DeviceRunner(slice_model(model, lo, hi), pkg) for lo, hi in self.slices]
+        self.streams = [torch.cuda.Stream() for _ in self.runners]
+
+    def run(self, x):
+        cur = torch.cuda.current_stream()
+        outs = []
+        for (lo, hi), r, st in zip(self.slices, self.runners, self.streams):
+            st.wait_stream(cur)
+            with torch.cuda.stream(st):
+                outs.append(r.run(x[lo:hi]))
+        for st in self.streams:
+            cur.wait_stream(st)
+        return outs
+
+    def capture(self, x):
+        self.run(x)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            values = self.run(x)
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return values
+        return replay
+
+    def close(self):
+        self._graph = None
+        for r in self.runners:
+            r.close()
+
+
 def run_reference(model, orc, x, keep=None):
     """Executes the program with a CPU executor `orc` that offers the oracle's functions
     (quantize_linear, qlinear_conv_int, max_pool_q8, ...).  Test and benchmark code passes

@@ -107,3 +107,32 @@ def test_mobilenetv2_batch1(g, oracle):
     assert 2.9e8 < model["macs"] < 3.2e8          # ~300 MMAC per image
     assert sum(c.group > 1 for c in model["convs"].values()) == 17
     check_model(g, oracle, model)
+
+
+def test_concurrent_batch_slices_match_whole_batch(g, oracle):
+    """The batch run as concurrent slices on separate streams (eager and as a replayed HIP graph)
+    gives the bytes of the whole-batch run."""
+    wl = g.pkg.workloads
+    model = wl.build_resnet50(batch=5, image=64, seed=8, width=16, blocks=(1, 1, 1, 1), classes=10)
+    x = torch.from_numpy(model["input"]).cuda()
+    whole = wl.DeviceRunner(model, g.pkg)
+    want = {k: v.clone() for k, v in whole.run(x).items()}
+    torch.cuda.synchronize()
+    split = wl.ConcurrentRunner(model, g.pkg, parts=2)
+    assert [hi - lo for lo, hi in split.slices] == [2, 3]
+
+    def check(outs, tag):
+        torch.cuda.synchronize()
+        for ins in model["program"]:
+            got = torch.cat([o[ins[1]] for o in outs], dim=0)
+            assert torch.equal(got, want[ins[1]]), "%s: %s" % (tag, ins[1])
+    check(split.run(x), "eager")
+    replay = split.capture(x)
+    for i in range(3):
+        for r in split.runners:
+            for buf in r.bufs.values():
+                buf.zero_()
+        torch.cuda.synchronize()
+        check(replay(), "replay %d" % i)
+    whole.close()
+    split.close()
