@@ -1,0 +1,277 @@
+"""A small reader and writer of the ONNX protobuf messages that the test directories of
+chainer-compiler use: ModelProto / GraphProto / NodeProto / AttributeProto / TensorProto /
+ValueInfoProto, field numbers of onnx.proto (IR version 3 and later).  No onnx package is
+involved; only what the quantized-inference path needs is decoded (tensor element types
+float32, float64, uint8, int8, int32, int64, bool; attributes f, i, s, t, floats, ints).
+
+Test directory layout (scripts/runtests.py, tools/run_onnx_util.cc:87-162 of the
+chainer-compiler tree):  DIR/model.onnx, DIR/test_data_set_N/input_i.pb, .../output_i.pb,
+each .pb one serialized TensorProto.
+"""
+import struct
+
+import numpy as np
+
+# TensorProto.DataType
+FLOAT, UINT8, INT8, INT32, INT64, BOOL, DOUBLE = 1, 2, 3, 6, 7, 9, 11
+NP_OF = {FLOAT: np.float32, UINT8: np.uint8, INT8: np.int8, INT32: np.int32, INT64: np.int64, BOOL: np.bool_,
+         DOUBLE: np.float64}
+ONNX_OF = {np.dtype(v): k for k, v in NP_OF.items()}
+
+
+# ---- wire format ------------------------------------------------------------------------------
+
+def _read_varint(b, i):
+    v, shift = 0, 0
+    while True:
+        c = b[i]
+        i += 1
+        v |= (c & 0x7F) << shift
+        if not c & 0x80:
+            return v, i
+        shift += 7
+
+
+def fields(b):
+    """Yields (field number, wire type, value) of one message; length-delimited values as bytes."""
+    i, n = 0, len(b)
+    while i < n:
+        tag, i = _read_varint(b, i)
+        f, w = tag >> 3, tag & 7
+        if w == 0:
+            v, i = _read_varint(b, i)
+        elif w == 1:
+            v = b[i:i + 8]
+            i += 8
+        elif w == 2:
+            ln, i = _read_varint(b, i)
+            v = b[i:i + ln]
+            i += ln
+            if len(v) != ln:
+                raise ValueError("truncated ONNX message")
+        elif w == 5:
+            v = b[i:i + 4]
+            i += 4
+        else:
+            raise ValueError("unsupported wire type %d" % w)
+        yield f, w, v
+
+
+def _sint(v):
+    return v - (1 << 64) if v >= 1 << 63 else v
+
+
+def _varint(v):
+    v &= (1 << 64) - 1
+    out = bytearray()
+    while True:
+        c = v & 0x7F
+        v >>= 7
+        out.append(c | 0x80 if v else c)
+        if not v:
+            return bytes(out)
+
+
+def _key(f, w):
+    return _varint((f << 3) | w)
+
+
+def _ld(f, payload):
+    if isinstance(payload, str):
+        payload = payload.encode()
+    return _key(f, 2) + _varint(len(payload)) + payload
+
+
+def _vi(f, v):
+    return _key(f, 0) + _varint(v)
+
+
+def _packed_ints(b, w, out):
+    if w == 2:
+        i = 0
+        while i < len(b):
+            v, i = _read_varint(b, i)
+            out.append(_sint(v))
+    else:
+        out.append(_sint(b))
+
+
+# ---- TensorProto --------------------------------------------------------------------------------
+
+def parse_tensor(b):
+    """(name, numpy array) of a serialized TensorProto."""
+    dims, dtype, name, raw = [], FLOAT, "", None
+    f32, i32, i64, f64 = [], [], [], []
+    for f, w, v in fields(b):
+        if f == 1:
+            _packed_ints(v, w, dims)
+        elif f == 2:
+            dtype = v
+        elif f == 4:
+            f32 += list(struct.unpack("<%df" % (len(v) // 4), v)) if w == 2 else [struct.unpack("<f", v)[0]]
+        elif f == 5:
+            _packed_ints(v, w, i32)
+        elif f == 7:
+            _packed_ints(v, w, i64)
+        elif f == 8:
+            name = v.decode()
+        elif f == 9:
+            raw = bytes(v)
+        elif f == 10:
+            f64 += list(struct.unpack("<%dd" % (len(v) // 8), v)) if w == 2 else [struct.unpack("<d", v)[0]]
+    if dtype not in NP_OF:
+        raise ValueError("tensor '%s': element type %d is not supported" % (name, dtype))
+    dt = np.dtype(NP_OF[dtype])
+    if raw is not None:
+        a = np.frombuffer(raw, dtype=dt).copy()
+    elif dtype == FLOAT:
+        a = np.array(f32, dt)
+    elif dtype == DOUBLE:
+        a = np.array(f64, dt)
+    elif dtype == INT64:
+        a = np.array(i64, dt)
+    else:
+        a = np.array(i32).astype(dt)   # uint8 / int8 / int32 / bool travel in int32_data
+    return name, a.reshape(dims)
+
+
+def make_tensor(name, array):
+    a = np.asarray(array, order="C")   # keeps 0-d arrays 0-d
+    out = b"".join(_vi(1, d) for d in a.shape) + _vi(2, ONNX_OF[a.dtype])
+    if name:
+        out += _ld(8, name)
+    return out + _ld(9, a.tobytes())
+
+
+# ---- model --------------------------------------------------------------------------------------
+
+class Node(object):
+    def __init__(self, op_type, inputs, outputs, attrs=None, name="", domain=""):
+        self.op_type, self.inputs, self.outputs = op_type, list(inputs), list(outputs)
+        self.attrs, self.name, self.domain = dict(attrs or {}), name, domain
+
+
+class Graph(object):
+    def __init__(self):
+        self.name = ""
+        self.nodes, self.initializers = [], {}
+        self.inputs, self.outputs = [], []       # [(name, elem_type, shape)]
+
+
+def _parse_attr(b):
+    name, val, floats, ints = "", None, [], []
+    for f, w, v in fields(b):
+        if f == 1:
+            name = v.decode()
+        elif f == 2:
+            val = struct.unpack("<f", v)[0]
+        elif f == 3:
+            val = _sint(v)
+        elif f == 4:
+            val = v.decode()
+        elif f == 5:
+            val = parse_tensor(v)[1]
+        elif f == 7:
+            floats += list(struct.unpack("<%df" % (len(v) // 4), v)) if w == 2 else [struct.unpack("<f", v)[0]]
+        elif f == 8:
+            _packed_ints(v, w, ints)
+    if val is None:
+        val = ints if ints else floats
+    return name, val
+
+
+def _parse_value_info(b):
+    name, elem, shape = "", 0, []
+    for f, w, v in fields(b):
+        if f == 1:
+            name = v.decode()
+        elif f == 2:
+            for f2, _, v2 in fields(v):
+                if f2 == 1:                       # tensor_type
+                    for f3, _, v3 in fields(v2):
+                        if f3 == 1:
+                            elem = v3
+                        elif f3 == 2:             # shape
+                            for f4, _, v4 in fields(v3):
+                                if f4 == 1:       # dim
+                                    d = -1
+                                    for f5, _, v5 in fields(v4):
+                                        if f5 == 1:
+                                            d = _sint(v5)
+                                    shape.append(d)
+    return name, elem, shape
+
+
+def parse_model(b):
+    g = Graph()
+    graph_bytes = None
+    for f, w, v in fields(b):
+        if f == 7:
+            graph_bytes = v
+    if graph_bytes is None:
+        raise ValueError("ModelProto without a graph")
+    for f, w, v in fields(graph_bytes):
+        if f == 1:
+            ins, outs, attrs, op, name, domain = [], [], {}, "", "", ""
+            for f2, _, v2 in fields(v):
+                if f2 == 1:
+                    ins.append(v2.decode())
+                elif f2 == 2:
+                    outs.append(v2.decode())
+                elif f2 == 3:
+                    name = v2.decode()
+                elif f2 == 4:
+                    op = v2.decode()
+                elif f2 == 5:
+                    k, val = _parse_attr(v2)
+                    attrs[k] = val
+                elif f2 == 7:
+                    domain = v2.decode()
+            g.nodes.append(Node(op, ins, outs, attrs, name, domain))
+        elif f == 2:
+            g.name = v.decode()
+        elif f == 5:
+            name, a = parse_tensor(v)
+            g.initializers[name] = a
+        elif f == 11:
+            g.inputs.append(_parse_value_info(v))
+        elif f == 12:
+            g.outputs.append(_parse_value_info(v))
+    return g
+
+
+def _make_value_info(name, elem, shape):
+    dims = b"".join(_ld(1, _vi(1, d)) for d in shape)
+    tensor_type = _vi(1, elem) + _ld(2, dims)
+    return _ld(1, name) + _ld(2, _ld(1, tensor_type))
+
+
+def _make_attr(name, val):
+    out = _ld(1, name)
+    if isinstance(val, float):
+        return out + _key(2, 5) + struct.pack("<f", val) + _vi(20, 1)
+    if isinstance(val, (int, np.integer)):
+        return out + _vi(3, int(val)) + _vi(20, 2)
+    if isinstance(val, str):
+        return out + _ld(4, val) + _vi(20, 3)
+    if isinstance(val, np.ndarray):
+        return out + _ld(5, make_tensor("", val)) + _vi(20, 4)
+    vals = list(val)
+    if vals and isinstance(vals[0], float):
+        return out + b"".join(_key(7, 5) + struct.pack("<f", x) for x in vals) + _vi(20, 6)
+    return out + b"".join(_vi(8, int(x)) for x in vals) + _vi(20, 7)
+
+
+def make_model(graph, opset=10):
+    g = b""
+    for n in graph.nodes:
+        nb = b"".join(_ld(1, i) for i in n.inputs) + b"".join(_ld(2, o) for o in n.outputs)
+        if n.name:
+            nb += _ld(3, n.name)
+        nb += _ld(4, n.op_type) + b"".join(_ld(5, _make_attr(k, v)) for k, v in n.attrs.items())
+        g += _ld(1, nb)
+    g += _ld(2, graph.name or "graph")
+    g += b"".join(_ld(5, make_tensor(k, v)) for k, v in graph.initializers.items())
+    g += b"".join(_ld(11, _make_value_info(*vi)) for vi in graph.inputs)
+    g += b"".join(_ld(12, _make_value_info(*vi)) for vi in graph.outputs)
+    return _vi(1, 5) + _ld(2, "chainer-compiler_amd") + _ld(7, g) + _ld(8, _ld(1, "") + _vi(2, opset))

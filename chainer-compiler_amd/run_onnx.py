@@ -1,0 +1,112 @@
+"""run_onnx for the hip backend: runs the test case of one directory through the C++ ChxVM and
+checks the outputs the way tools/run_onnx.cc does.
+
+  python -m chainer_compiler_amd.run_onnx --test DIR [--rtol 1e-4] [--atol 1e-6] [--iterations N]
+         [--trace] [--backend hip]
+
+DIR/model.onnx is lowered by chxvm_emit; every DIR/test_data_set_N supplies input_i.pb and
+output_i.pb in graph order.  An output passes when dtype and shape are equal and every element
+has |a - b| <= atol + rtol * |b| (tools/util.cc:89-121; the defaults are run_onnx.cc:299-300).
+Exit status 0 when every data set passes.  (From a checkout, where the package directory is
+not importable by name, use `python chainer-compiler_amd/run_onnx.py ...`.)
+"""
+import argparse
+import glob
+import os
+import sys
+import time
+
+import numpy as np
+
+
+def _package():
+    here = os.path.dirname(os.path.abspath(__file__))
+    root = os.path.dirname(here)
+    if root not in sys.path:
+        sys.path.insert(0, root)
+    import __graft_entry__ as entry
+    return entry.load_package()
+
+
+def load_test_case(test_dir, onnx_lite):
+    graph = onnx_lite.parse_model(open(os.path.join(test_dir, "model.onnx"), "rb").read())
+    data_sets = []
+    for d in sorted(glob.glob(os.path.join(test_dir, "test_data_set_*"))):
+        def read(prefix):
+            out = []
+            i = 0
+            while os.path.exists(os.path.join(d, "%s_%d.pb" % (prefix, i))):
+                out.append(onnx_lite.parse_tensor(open(os.path.join(d, "%s_%d.pb" % (prefix, i)), "rb").read())[1])
+                i += 1
+            return out
+        data_sets.append((os.path.basename(d), read("input"), read("output")))
+    return graph, data_sets
+
+
+def mismatches(got, want, rtol, atol):
+    """Number of elements outside the tolerance; raises on a dtype or shape difference."""
+    if got.shape != want.shape:
+        raise ValueError("Cannot compare Arrays of different shapes: %s, %s" % (got.shape, want.shape))
+    if got.dtype != want.dtype:
+        raise ValueError("Cannot compare Arrays of different Dtypes: %s, %s" % (got.dtype, want.dtype))
+    a, b = got.astype(np.float64), want.astype(np.float64)
+    bad = np.isnan(a) | np.isnan(b) | (np.abs(a - b) > atol + rtol * np.abs(b))
+    return int(bad.sum())
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--test", required=True, help="test directory")
+    ap.add_argument("--backend", default="hip", choices=["hip"])
+    ap.add_argument("--rtol", type=float, default=1e-4)
+    ap.add_argument("--atol", type=float, default=1e-6)
+    ap.add_argument("--iterations", type=int, default=1)
+    ap.add_argument("--trace", action="store_true")
+    ap.add_argument("--verbose", action="store_true")
+    args = ap.parse_args(argv)
+
+    pkg = _package()
+    import importlib
+    import torch
+    onnx_lite = importlib.import_module(pkg.__name__ + ".onnx_lite")
+    emit = importlib.import_module(pkg.__name__ + ".chxvm_emit")
+    vm = importlib.import_module(pkg.__name__ + ".chxvm")
+    pkg.capi.init(0)
+
+    graph, data_sets = load_test_case(args.test, onnx_lite)
+    if not data_sets:
+        print("%s: no test_data_set_* directories" % args.test, file=sys.stderr)
+        return 2
+    serialized, input_names, output_names = emit.emit_program(graph)
+    program = vm.Program(serialized)
+    failed = 0
+    for name, inputs, wants in data_sets:
+        if len(inputs) != len(input_names) or len(wants) != len(output_names):
+            print("%s: %d inputs / %d outputs on disk, the graph has %d / %d" % (
+                name, len(inputs), len(wants), len(input_names), len(output_names)), file=sys.stderr)
+            return 2
+        feed = {n: torch.from_numpy(np.ascontiguousarray(a)).cuda() for n, a in zip(input_names, inputs)}
+        elapsed = []
+        for _ in range(max(1, args.iterations)):
+            t0 = time.perf_counter()
+            outs = program.run(feed, trace_level=1 if args.trace else 0)
+            elapsed.append(time.perf_counter() - t0)
+        for n, want in zip(output_names, wants):
+            bad = mismatches(outs[n], want, args.rtol, args.atol)
+            if bad:
+                failed += 1
+                print("FAIL %s/%s: %d of %d elements differ (rtol %g atol %g)" % (name, n, bad, want.size, args.rtol,
+                                                                                args.atol), file=sys.stderr)
+            elif args.verbose:
+                print("OK   %s/%s %s %s" % (name, n, want.dtype, want.shape))
+        if args.iterations > 1:
+            rest = elapsed[1:]   # the first run is discarded, as run_onnx.cc does
+            print("%s: average %.3f ms, best %.3f ms over %d runs" % (name, 1e3 * sum(rest) / len(rest), 1e3 * min(rest),
+                                                                    len(rest)))
+    program.close()
+    print("%s: %s" % (args.test, "FAILED" if failed else "OK"))
+    return 1 if failed else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,57 @@
+"""Test driver in the manner of scripts/runtests.py of the chainer-compiler tree: one run_onnx
+subprocess per test directory, a summary, and for every failure the captured output with the
+command line that reproduces it.  Every case here needs the GPU, so the cases run one after the
+other (the reference runs its CPU cases in parallel first and the GPU cases serially).
+
+  python chainer-compiler_amd/runtests.py DIR_OF_TEST_DIRS [-k FILTER] [--rtol R] [--atol A]
+"""
+import argparse
+import os
+import subprocess
+import sys
+import time
+
+# the quantized-path cases of the reference's node-test list (scripts/runtests.py:556-563)
+NODE_TESTS = ["test_quantizelinear", "test_dequantizelinear", "test_qlinearmatmul_2D", "test_qlinearmatmul_3D",
+              "test_qlinearconv", "test_convinteger_with_padding", "test_basic_convinteger", "test_matmulinteger"]
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("root", help="directory holding one sub-directory per test case")
+    ap.add_argument("-k", "--filter", default="")
+    ap.add_argument("--rtol", type=float, default=None)
+    ap.add_argument("--atol", type=float, default=None)
+    ap.add_argument("--timeout", type=float, default=120.0)
+    args = ap.parse_args(argv)
+    here = os.path.dirname(os.path.abspath(__file__))
+    cases = sorted(d for d in os.listdir(args.root)
+                   if os.path.exists(os.path.join(args.root, d, "model.onnx")) and args.filter in d)
+    if not cases:
+        print("no test cases under %s" % args.root, file=sys.stderr)
+        return 2
+    failures = []
+    t0 = time.time()
+    for i, case in enumerate(cases):
+        cmd = [sys.executable, os.path.join(here, "run_onnx.py"), "--test", os.path.join(args.root, case)]
+        if args.rtol is not None:
+            cmd += ["--rtol", str(args.rtol)]
+        if args.atol is not None:
+            cmd += ["--atol", str(args.atol)]
+        try:
+            p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=args.timeout)
+            ok, log = p.returncode == 0, p.stdout.decode("utf-8", "replace")
+        except subprocess.TimeoutExpired as e:
+            ok, log = False, (e.stdout or b"").decode("utf-8", "replace") + "\ntimed out"
+        print("[%d/%d] %s %s" % (i + 1, len(cases), "OK  " if ok else "FAIL", case))
+        sys.stdout.flush()
+        if not ok:
+            failures.append((case, cmd, log))
+    for case, cmd, log in failures:
+        print("=== %s ===\n%s\n$ %s" % (case, log, " ".join(cmd)))
+    print("%d/%d tests passed in %.1f s" % (len(cases) - len(failures), len(cases), time.time() - t0))
+    return 1 if failures else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

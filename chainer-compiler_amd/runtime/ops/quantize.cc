@@ -140,5 +140,14 @@ chainerx::Array ConvIntegerOp::RunImpl(
     return y;
 }
 
+// A float MatMul only exists on this backend between two DequantizeLinear and one
+// QuantizeLinear, the sequence ReplaceQLinearMatMul leaves (compiler/simplifier.cc:675-694);
+// ChxVM fuses that sequence into one quantized product when it loads the program (chxvm.cc).
+chainerx::Array MatMulOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
+    CHECK(false) << "float MatMul outside a DequantizeLinear, DequantizeLinear, MatMul, QuantizeLinear sequence "
+                    "is not part of the quantized-inference path of the hip runtime";
+    return chainerx::Array();
+}
+
 }  // namespace runtime
 }  // namespace chainer_compiler

@@ -1,0 +1,49 @@
+"""The reference's quantized-path node tests as ONNX test directories, run by the test driver
+(one run_onnx subprocess per directory) through the emitter and the C++ ChxVM on the MI355X."""
+import importlib
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_runtests_over_the_node_tests(onnx_vectors, tmp_path):
+    import gpu_util
+    import onnx_cases
+    ol = importlib.import_module(gpu_util.pkg.__name__ + ".onnx_lite")
+    driver = importlib.import_module(gpu_util.pkg.__name__ + ".runtests")
+    cases = onnx_cases.build_cases(ol, onnx_vectors)
+    assert sorted(cases) == sorted(driver.NODE_TESTS)
+    for name, case in cases.items():
+        onnx_cases.write_case(ol, str(tmp_path), name, case)
+    # one more directory whose expected output is wrong by one code: the driver must report it
+    g, ins, outs = cases["test_quantizelinear"]
+    wrong = outs[0].copy()
+    wrong[2] += 1
+    onnx_cases.write_case(ol, str(tmp_path), "zz_expected_failure", (g, ins, [wrong]))
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "chainer-compiler_amd", "runtests.py"), str(tmp_path)],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
+    log = p.stdout.decode()
+    print(log)
+    assert p.returncode == 1
+    for name in cases:
+        assert "OK   %s" % name in log
+    assert "FAIL zz_expected_failure" in log and "8/9 tests passed" in log
+    assert "1 of 6 elements differ" in log and "run_onnx.py --test" in log      # failure log + reproducing command
+
+
+def test_run_onnx_in_process_with_iterations(onnx_vectors, tmp_path, capsys):
+    import gpu_util
+    import onnx_cases
+    ol = importlib.import_module(gpu_util.pkg.__name__ + ".onnx_lite")
+    run_onnx = importlib.import_module(gpu_util.pkg.__name__ + ".run_onnx")
+    cases = onnx_cases.build_cases(ol, onnx_vectors)
+    d = onnx_cases.write_case(ol, str(tmp_path), "test_qlinearmatmul_3D", cases["test_qlinearmatmul_3D"])
+    assert run_onnx.main(["--test", d, "--iterations", "3", "--verbose"]) == 0
+    out = capsys.readouterr().out
+    assert "average" in out and "OK   test_data_set_0/y uint8 (2, 2, 3)" in out
