@@ -127,14 +127,14 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # Launch duration of the dominant kernel: event pairs cannot be recorded inside a graph
     # replay, and around single 15-60 us launches they mostly measure submission gaps.  So each
     # QLinearConv instruction of the program is launched REP times back to back between one
-    # event pair on the launch stream, on the buffers of the step just timed; a sleeping kernel
-    # goes first so that the host is done submitting before the GPU starts.  The per-step
+    # event pair on the launch stream, on the buffers of the step just timed.  The per-step
     # kernel time is the sum of the per-instruction averages.
     REP = 20
     # the launches timed are those of the timed region: one slice's instructions, times the slices
     slices = [(runner, x)] if args.parts <= 1 else [(r, x[lo:hi]) for (lo, hi), r in zip(timed_runner.slices, timed_runner.runners)]
     conv_ms_per_step, n_launch = 0.0, 0
     pairs = []
+    layer_graphs = []
     for rn, xs in slices:
         vals = rn.run(xs)
         torch.cuda.synchronize()
@@ -146,12 +146,19 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                 continue  # MobileNetV2: the roofline figure is the depthwise kernel's
             fn = lambda: rn.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
                                               flags=capi.BIAS_ONNX_INT32, out=rn.bufs[ins[1]])
-            torch.cuda._sleep(int(2.4e9 * 0.002))
+            # REP launches recorded into a graph of their own: replayed, they follow each other the way
+            # the instructions of the timed graph do, without host submission gaps between them
+            fn()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _ in range(REP):
+                    fn()
+            layer_graphs.append(g)
+            g.replay()
             a = torch.cuda.Event(enable_timing=True)
             b = torch.cuda.Event(enable_timing=True)
             a.record()
-            for _ in range(REP):
-                fn()
+            g.replay()
             b.record()
             pairs.append((ins[3], a, b))
             n_launch += 1
@@ -171,6 +178,15 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % n_launch,
                         achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
                         ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
+    if not mobilenet and batch == 64 and args.parts <= 1:
+        # HBM bytes of the same launches from hardware counters (FETCH_SIZE / WRITE_SIZE, scaled by a
+        # copy kernel of known size): measured in two separate profiling runs, kept with their commands
+        try:
+            t = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                                            "resnet50_bs64_conv_mfma_traffic.json")))
+            roofline["traffic"] = t["bytes_per_step"]
+        except (OSError, ValueError, KeyError):
+            pass
     res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),
                value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
                config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,
