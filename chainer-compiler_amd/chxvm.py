@@ -25,7 +25,7 @@ RUNTIME_EXPORTS = [
     "chxvm_last_error", "chxvm_num_ops", "chxvm_op_name", "chxvm_op_number", "chxvm_proto_roundtrip", "chxvm_free",
     "chxvm_program_create", "chxvm_program_destroy", "chxvm_program_num_instructions", "chxvm_program_num_inputs",
     "chxvm_program_input_name", "chxvm_program_run", "chxvm_outputs_count", "chxvm_outputs_name", "chxvm_outputs_get",
-    "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name",
+    "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name", "chxvm_set_option",
 ]
 
 # ChxVMValueProto.Type
@@ -77,6 +77,7 @@ def runtime():
         rt.chxvm_outputs_destroy.restype = None
         rt.chxvm_backend_config_has.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_char_p,
                                                 ctypes.POINTER(ctypes.c_int32)]
+        rt.chxvm_set_option.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
         rt.chxvm_backend_config_name.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
         _rt = rt
     return _rt
@@ -268,6 +269,14 @@ class ProgramBuilder:
             return None
         return outputs[0] if len(outputs) == 1 else tuple(outputs)
 
+    def add_raw(self, name, inputs, outputs, debug_info=""):
+        """An instruction of an op that has no signature in this runtime's table (it only exists
+        fused with its neighbours): `inputs` is a list of (value type name, value) in the operand
+        order of the reference's op table."""
+        number = self.index[name][0]
+        self.instructions.append(encode_instruction(number, inputs, outputs, debug_info=debug_info, id=self.next_id))
+        self.next_id += 1
+
     # conveniences -----------------------------------------------------------------------
     def input(self, name, dtype="float32", shape=()):
         self.input_names.append(name)
@@ -362,6 +371,11 @@ class Program:
             self.close()
         except Exception:
             pass
+
+
+def set_option(name, value):
+    """Runtime switches; "qlinearconv_bias" = "reference" (default) | "onnx_int32"."""
+    _check(runtime().chxvm_set_option(name.encode(), value.encode()))
 
 
 def proto_roundtrip(serialized):

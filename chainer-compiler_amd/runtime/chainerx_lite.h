@@ -329,6 +329,18 @@ inline Array EmptyChannelsLast(const Shape& nchw, Dtype dtype) {
     return nhwc.Transpose({0, 3, 1, 2});
 }
 
+// The same with the pixel pitch rounded up to 16 bytes (8-bit arrays): every pixel is then a whole
+// number of aligned 16-byte vectors, which the convolution kernels need, also for C = 24.
+inline Array EmptyChannelsLastPadded(const Shape& nchw, Dtype dtype) {
+    CHECK_EQ(4, nchw.size());
+    const int64_t es = GetItemSize(dtype);
+    const int64_t pitch = (nchw[1] * es + 15) / 16 * 16;
+    if (pitch == nchw[1] * es) return EmptyChannelsLast(nchw, dtype);
+    Array flat = Empty(Shape{nchw[0] * nchw[2] * nchw[3] * pitch}, Dtype::kUInt8);
+    std::shared_ptr<void> keep(flat.raw_data(), [flat](void*) {});  // shares the allocation
+    return Array::MakeOwned(keep, dtype, nchw, Strides{nchw[2] * nchw[3] * pitch, es, nchw[3] * pitch, pitch});
+}
+
 inline Array FromHost(const void* src, const Shape& shape, Dtype dtype) {
     Array a = Empty(shape, dtype);
     CHXVM_HIP_CALL(chx_hip_memcpy_h2d(a.raw_data(), src, static_cast<size_t>(a.GetNBytes()), nullptr));

@@ -45,6 +45,68 @@ private:
     int a_, a_scale_, a_zp_, b_, b_scale_, b_zp_, y_scale_, y_zp_, y_;
 };
 
+// DequantizeLinear, MaxPool | AveragePool, QuantizeLinear as one instruction on the 8-bit codes
+// (chx_hip_max_pool_q8 / chx_hip_average_pool_q8).  MaxPool operands: x, kernel_shape, strides,
+// pads, cover_all, auto_pad; AveragePool: x, kernel_shape, strides, pads, count_include_pad
+// (runtime/chxvm_defs.py:314-321 of the chainer-compiler tree).
+class FusedQuantizedPoolOp : public ChxVMOp {
+public:
+    FusedQuantizedPoolOp(const ChxVMInstructionProto& quantize, const ChxVMInstructionProto& pool,
+                         const ChxVMInstructionProto& dq, bool is_max)
+        : ChxVMOp(quantize), is_max_(is_max),
+          x_(dq.inputs[0].array), x_scale_(dq.inputs[1].scalar), x_zp_(dq.inputs[2].scalar),
+          y_scale_(quantize.inputs[1].scalar), y_zp_(quantize.inputs[2].scalar), y_(quantize.outputs[0]),
+          kernel_(pool.inputs[1].ints), strides_(pool.inputs[2].ints), pads_(pool.inputs[3].ints),
+          flag_(static_cast<int>(pool.inputs[4].i)) {
+        CHECK_EQ(2u, kernel_.size()) << "only 2-D pooling on the hip backend";
+        if (is_max) CHECK(pool.inputs[5].s.empty() || pool.inputs[5].s == "NOTSET") << "auto_pad is not supported for a quantized MaxPool";
+    }
+
+    void Run(ChxVMState* st) override {
+        if (st->trace_level()) std::cerr << (is_max_ ? "MaxPool" : "AveragePool") << "(quantized, fused) $" << x_ << " -> $" << y_ << std::endl;
+        const chainerx::Array x = st->GetArray(x_);
+        CHECK_EQ(4, x.ndim());
+        auto scalar_or_zero = [&](int slot) -> StrictScalar {
+            absl::optional<StrictScalar> z = st->GetOptionalScalar(slot);
+            return z.has_value() ? *z : StrictScalar(chainerx::Dtype::kUInt8, chainerx::Scalar(0u), false);
+        };
+        const float xs = static_cast<float>(st->GetScalar(x_scale_)), ys = static_cast<float>(st->GetScalar(y_scale_));
+        const StrictScalar xz = scalar_or_zero(x_zp_), yz = scalar_or_zero(y_zp_);
+        const int kh = static_cast<int>(kernel_[0]), kw = static_cast<int>(kernel_[1]);
+        const int sh = strides_.empty() ? 1 : static_cast<int>(strides_[0]), sw = strides_.empty() ? 1 : static_cast<int>(strides_[1]);
+        int pb[2] = {0, 0}, pe[2] = {0, 0};
+        if (pads_.size() == 2) { pb[0] = pe[0] = static_cast<int>(pads_[0]); pb[1] = pe[1] = static_cast<int>(pads_[1]); }
+        if (pads_.size() == 4) { pb[0] = static_cast<int>(pads_[0]); pb[1] = static_cast<int>(pads_[1]); pe[0] = static_cast<int>(pads_[2]); pe[1] = static_cast<int>(pads_[3]); }
+        auto out_dim = [&](int64_t in, int k, int s, int p0, int p1, bool cover_all) {
+            return cover_all ? (in + p0 + p1 - k + s - 1) / s + 1 : (in + p0 + p1 - k) / s + 1;
+        };
+        const bool cover_all = is_max_ && flag_ != 0;
+        const chainerx::Shape shape{x.shape()[0], x.shape()[1], out_dim(x.shape()[2], kh, sh, pb[0], pe[0], cover_all),
+                                    out_dim(x.shape()[3], kw, sw, pb[1], pe[1], cover_all)};
+        const bool channels_last = !x.IsContiguous() && x.strides()[1] == x.GetItemSize();
+        chainerx::Array y = channels_last ? chainerx::EmptyChannelsLastPadded(shape, yz.dtype()) : chainerx::Empty(shape, yz.dtype());
+        chx_hip_tensor xt = x.hip(), yt = y.hip();
+        if (is_max_) {
+            // the maximum of the codes is the quantized maximum only when both sides share the quantization
+            CHECK(xs == ys && static_cast<int64_t>(xz) == static_cast<int64_t>(yz) && xz.dtype() == yz.dtype())
+                    << "a quantized MaxPool needs the same scale and zero point before and after";
+            CHXVM_HIP_CALL(chx_hip_max_pool_q8(&xt, kh, kw, sh, sw, pb[0], pb[1], pe[0], pe[1], cover_all ? 1 : 0, &yt, nullptr));
+        } else {
+            CHECK(pb[0] == pe[0] && pb[1] == pe[1]) << "AveragePool pads must be symmetric";
+            CHXVM_HIP_CALL(chx_hip_average_pool_q8(&xt, xs, static_cast<int32_t>(static_cast<int64_t>(xz)), kh, kw, sh, sw, pb[0], pb[1],
+                                                   flag_, ys, static_cast<int32_t>(static_cast<int64_t>(yz)), CHX_HIP_ROUND_REFERENCE,
+                                                   &yt, nullptr));
+        }
+        st->SetArray(y_, y);
+    }
+
+private:
+    bool is_max_;
+    int x_, x_scale_, x_zp_, y_scale_, y_zp_, y_;
+    std::vector<int64_t> kernel_, strides_, pads_;
+    int flag_;
+};
+
 class NopOp : public ChxVMOp {
 public:
     explicit NopOp(const ChxVMInstructionProto& inst) : ChxVMOp(inst) {
@@ -82,12 +144,12 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
     // intermediate read exactly once apart from its Free.
     const int n = static_cast<int>(program.instructions.size());
     const int kDequantize = OpNumber("DequantizeLinear"), kMatMul = OpNumber("MatMul"), kQuantize = OpNumber("QuantizeLinear"),
-              kFree = OpNumber("Free");
+              kFree = OpNumber("Free"), kMaxPool = OpNumber("MaxPool"), kAveragePool = OpNumber("AveragePool");
     std::vector<int> producer(num_variables_ > 0 ? num_variables_ : 1, -1);
     for (int i = 0; i < n; ++i)
         for (int o : program.instructions[i].outputs)
             if (o >= 0) producer[o] = i;
-    std::vector<int> role(n, 0);  // 0 plain, 1 dropped, 2 fused (at the QuantizeLinear)
+    std::vector<int> role(n, 0);  // 0 plain, 1 dropped, 2 fused product, 3 fused pool (both at the QuantizeLinear)
     std::vector<std::pair<int, int>> fused_inputs(n);
     auto single_use = [&](int slot) {
         // one consumer plus at most one Free
@@ -100,6 +162,22 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         const ChxVMInstructionProto& qi = program.instructions[q];
         if (qi.op != kQuantize || qi.inputs.size() != 3 || qi.inputs[0].array < 0) continue;
         const int m = producer[qi.inputs[0].array];
+        if (m >= 0 && (program.instructions[m].op == kMaxPool || program.instructions[m].op == kAveragePool) &&
+            single_use(qi.inputs[0].array)) {
+            // DequantizeLinear -> pool -> QuantizeLinear; the pool's opaque context output must be unused
+            const ChxVMInstructionProto& pi = program.instructions[m];
+            const bool is_max = pi.op == kMaxPool;
+            const bool shape_ok = pi.inputs.size() == (is_max ? 6u : 5u) && pi.inputs[0].array >= 0 &&
+                                  (pi.outputs.size() < 2 || pi.outputs[1] < 0);
+            const int d = shape_ok ? producer[pi.inputs[0].array] : -1;
+            if (d >= 0 && program.instructions[d].op == kDequantize && program.instructions[d].inputs.size() == 3 &&
+                single_use(pi.inputs[0].array)) {
+                role[q] = 3;
+                fused_inputs[q] = std::make_pair(d, m);
+                role[m] = role[d] = 1;
+            }
+            continue;
+        }
         if (m < 0 || program.instructions[m].op != kMatMul || !single_use(qi.inputs[0].array)) continue;
         const ChxVMInstructionProto& mi = program.instructions[m];
         const int da = producer[mi.inputs[0].array], db = producer[mi.inputs[1].array];
@@ -121,6 +199,9 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         const bool frees_dead = inst.op == kFree && inst.inputs.size() == 1 && inst.inputs[0].array >= 0 && dead[inst.inputs[0].array];
         if (role[i] == 1 || frees_dead) {
             program_.emplace_back(new NopOp(inst));
+        } else if (role[i] == 3) {
+            const ChxVMInstructionProto& pool = program.instructions[fused_inputs[i].second];
+            program_.emplace_back(new FusedQuantizedPoolOp(inst, pool, program.instructions[fused_inputs[i].first], pool.op == kMaxPool));
         } else if (role[i] == 2) {
             program_.emplace_back(new FusedQLinearMatMulOp(inst, program.instructions[fused_inputs[i].first],
                                                            program.instructions[fused_inputs[i].second]));

@@ -11,6 +11,10 @@
 namespace chainer_compiler {
 namespace runtime {
 
+// QLinearConv bias: false (default) = the reference's unscaled float bias, true = the ONNX
+// operator's int32 bias added to the accumulator.
+void SetQLinearConvOnnxInt32Bias(bool on);
+
 class ChxVM {
 public:
     explicit ChxVM(const ChxVMProgramProto& program);

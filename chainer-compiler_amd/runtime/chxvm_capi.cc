@@ -148,6 +148,18 @@ void chxvm_outputs_destroy(chxvm_outputs* outputs) {
     delete outputs;
 }
 
+int32_t chxvm_set_option(const char* name, const char* value) {
+    return Guard([&] {
+        const std::string n = name, v = value;
+        if (n == "qlinearconv_bias") {
+            CHECK(v == "reference" || v == "onnx_int32") << "qlinearconv_bias is 'reference' or 'onnx_int32', got " << v;
+            SetQLinearConvOnnxInt32Bias(v == "onnx_int32");
+        } else {
+            CHECK(false) << "unknown option " << n;
+        }
+    });
+}
+
 int32_t chxvm_backend_config_has(const char* config, int32_t is_json, const char* section, const char* key, int32_t* out) {
     return Guard([&] {
         std::unique_ptr<BackendConfig> c = is_json ? BackendConfig::FromJSON(config) : BackendConfig::FromName(config);

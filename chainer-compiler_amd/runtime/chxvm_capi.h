@@ -51,6 +51,9 @@ const char* chxvm_outputs_name(const chxvm_outputs* outputs, int32_t i);
 int32_t chxvm_outputs_get(const chxvm_outputs* outputs, int32_t i, chx_hip_tensor* out);
 void chxvm_outputs_destroy(chxvm_outputs* outputs);
 
+/* name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32". */
+int32_t chxvm_set_option(const char* name, const char* value);
+
 /* BackendConfig queries.  `config` is a built-in name ("chxvm", "chxvm_test", "hip") or, with
  * is_json != 0, a JSON document.  section: "simplify_preproc", "simplify", "merge",
  * "expanding_functions" (membership) or "supported_ops" (HasOp).  *out = 0 or 1. */

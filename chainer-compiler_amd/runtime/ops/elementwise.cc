@@ -47,12 +47,30 @@ std::vector<chainerx::Array> ElementWiseNvrtcOp::RunImpl(ChxVMState* st, const s
     for (const chainerx::Array& input : orig_inputs)
         if (input.shape() == shape && (input.IsContiguous() || input.strides()[1] != input.GetItemSize())) channels_last = false;
 
+    // Activations whose pixel pitch is padded to 16 bytes (a convolution's output with C = 24, say):
+    // when every operand has that one layout and all values are 8-bit, the group runs over the padded
+    // pixels as they lie in memory, which is dense; the padding bytes compute garbage into padding.
+    bool padded = channels_last;
+    for (const chainerx::Array& input : orig_inputs)
+        padded = padded && input.shape() == shape && input.GetItemSize() == 1 && input.strides() == orig_inputs[0].strides() &&
+                 input.strides()[3] > shape[1] && input.strides()[2] == shape[3] * input.strides()[3] &&
+                 input.strides()[0] == shape[2] * input.strides()[2];
+    for (chainerx::Dtype dt : dtypes) padded = padded && chainerx::GetItemSize(dt) == 1;
+    const int64_t pitch = padded ? orig_inputs[0].strides()[3] : 0;
+    padded = padded && pitch == (shape[1] + 15) / 16 * 16;
+    auto widened = [&](chx_hip_tensor t) {
+        if (padded) t.shape[1] = pitch;
+        return t;
+    };
+
     std::vector<chainerx::Array> outputs;
     std::vector<chx_hip_tensor> in_desc, out_desc;
-    for (const chainerx::Array& input : orig_inputs) in_desc.push_back(input.hip());
+    for (const chainerx::Array& input : orig_inputs) in_desc.push_back(widened(input.hip()));
     for (int i = 0; i < num_outputs; ++i) {
-        outputs.push_back(channels_last ? chainerx::EmptyChannelsLast(shape, dtypes[i]) : chainerx::Empty(shape, dtypes[i]));
-        out_desc.push_back(outputs.back().hip());
+        outputs.push_back(padded          ? chainerx::EmptyChannelsLastPadded(shape, dtypes[i])
+                          : channels_last ? chainerx::EmptyChannelsLast(shape, dtypes[i])
+                                          : chainerx::Empty(shape, dtypes[i]));
+        out_desc.push_back(widened(outputs.back().hip()));
     }
     std::vector<const chx_hip_tensor*> in_ptr;
     std::vector<chx_hip_tensor*> out_ptr;

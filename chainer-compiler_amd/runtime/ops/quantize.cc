@@ -9,6 +9,8 @@ namespace runtime {
 
 namespace {
 
+bool g_onnx_int32_bias = false;
+
 StrictScalar DefaultZeroPoint() {
     // an absent zero point is uint8 0 (runtime/ops/quantize.cc:50-51,57-58)
     return StrictScalar(chainerx::Dtype::kUInt8, chainerx::Scalar(0u), false);
@@ -25,6 +27,13 @@ chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& sha
 }
 
 }  // namespace
+
+// The reference adds the bias of a QLinearConv as an unscaled float after the convolution
+// (runtime/ops/quantize.cc:93); networks quantized for the ONNX operator carry an int32 bias at
+// scale x_scale * w_scale[oc].  This switch selects which of the two the op computes.
+void SetQLinearConvOnnxInt32Bias(bool on) {
+    g_onnx_int32_bias = on;
+}
 
 chainerx::Array QuantizeLinearOp::RunImpl(
         ChxVMState* st, const chainerx::Array& x, const StrictScalar& y_scale, const absl::optional<StrictScalar>& y_zero_point_opt) {
@@ -94,13 +103,14 @@ chainerx::Array QLinearConvOp::RunImpl(
         impl_->params = p;
         impl_->w_data = q_w.raw_data();
     }
-    chainerx::Array y = EmptyLike4d(q_x, ConvOutputShape(q_x, q_w, p), y_zero_point.dtype());
+    // 8-bit activations leave a convolution channels-last, whatever layout came in
+    chainerx::Array y = chainerx::EmptyChannelsLastPadded(ConvOutputShape(q_x, q_w, p), y_zero_point.dtype());
     chx_hip_tensor xt = q_x.hip(), yt = y.hip();
     // the reference hands the raw bias to the fp32 convolution (quantize.cc:93)
     CHXVM_HIP_CALL(chx_hip_qconv_plan_run(
             impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
             static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)),
-            CHX_HIP_ROUND_REFERENCE | CHX_HIP_BIAS_REFERENCE_FLOAT, &yt, nullptr));
+            CHX_HIP_ROUND_REFERENCE | (g_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT), &yt, nullptr));
     return y;
 }
 

@@ -364,6 +364,65 @@ class DeviceRunner(object):
             p.close()
 
 
+def program_to_chxvm(model, vm, ops, keep=("logits",)):
+    """The op program as a serialized ChxVMProgramProto, in the form the reference's compiler gives
+    a QDQ graph: QuantizeLinear / QLinearConv / DequantizeLinear instructions with constant
+    operands, pools between a DequantizeLinear and a QuantizeLinear, residual sums as
+    ElementWiseNvrtc FusionGroups.  `vm` is the chxvm module, `ops` the ops module.
+    QLinearConv biases are int32 at scale x_scale * w_scale: run with the option
+    qlinearconv_bias = onnx_int32.  `keep` names the values that become program outputs."""
+    b = vm.ProgramBuilder()
+    q = model["qparams"]
+    slot = {}
+
+    def scalars(name):
+        return b.scalar(float(q[name][0]), "float32"), b.scalar(int(q[name][1]), "uint8")
+    for fid, ins in enumerate(model["program"]):
+        kind, out = ins[0], ins[1]
+        if kind == "QuantizeLinear":
+            slot[ins[2]] = b.input(ins[2], "float32", model["shapes"][ins[2]])
+            s, z = b.scalar(float(ins[3]), "float32"), b.scalar(int(ins[4]), "uint8")
+            slot[out] = b.QuantizeLinear(slot[ins[2]], s, z, debug_info=out)
+        elif kind == "QLinearConv":
+            c = model["convs"][ins[3]]
+            xs, xz = b.scalar(float(c.x_scale), "float32"), b.scalar(int(c.x_zp), "uint8")
+            ys, yz = b.scalar(float(c.y_scale), "float32"), b.scalar(int(c.y_zp), "uint8")
+            slot[out] = b.QLinearConv(slot[ins[2]], xs, xz, b.constant(c.wq), b.constant(c.w_scale), b.constant(c.w_zp), ys, yz,
+                                      b.constant(c.bias_q), [c.stride, c.stride], [c.pad, c.pad], c.group, "", debug_info=out)
+        elif kind in ("MaxPool", "AveragePool"):
+            s_in, z_in = scalars(ins[2])
+            f = b.DequantizeLinear(slot[ins[2]], s_in, z_in, debug_info=out)
+            g = b.new_slot()
+            if kind == "MaxPool":
+                k, st, pad, cover_all = ins[3], ins[4], ins[5], ins[6]
+                b.add_raw("MaxPool", [("ARRAY", f), ("INTS", [k, k]), ("INTS", [st, st]), ("INTS", [pad, pad]),
+                                      ("INT", 1 if cover_all else 0), ("STRING", "NOTSET")], [g, -1], debug_info=out)
+            else:
+                k = ins[3]
+                b.add_raw("AveragePool", [("ARRAY", f), ("INTS", [k, k]), ("INTS", [1, 1]), ("INTS", [0, 0]), ("INT", 0)],
+                          [g, -1], debug_info=out)
+            s_out, z_out = scalars(out)
+            slot[out] = b.QuantizeLinear(g, s_out, z_out, debug_info=out)
+            b.Free(f)
+            b.Free(g)
+        elif kind in ("AddRelu", "Add"):
+            make = add_relu_program if kind == "AddRelu" else add_program
+            code = make(ops, q[ins[2]], q[ins[3]], q[out])
+            slot[out] = b.ElementWiseNvrtc([slot[ins[2]], slot[ins[3]]], 1, code, fid, num_list_outputs=1, debug_info=out)[0]
+        elif kind == "DequantizeLinear":
+            s, z = b.scalar(float(ins[3]), "float32"), b.scalar(int(ins[4]), "uint8")
+            slot[out] = b.DequantizeLinear(slot[ins[2]], s, z, debug_info=out)
+        else:
+            raise ValueError(kind)
+        # the compiler frees a value after its last reader (compiler/scheduler.cc, compiler/chxvm/emitter.cc)
+        for name in ins[2:4]:
+            if isinstance(name, str) and name in slot and name not in keep and not _still_needed(model["program"], ins, name):
+                b.Free(slot[name])
+    for name in keep:
+        b.output(name, slot[name])
+    return b
+
+
 def slice_model(model, lo, hi):
     """The same program on images lo..hi-1 of the batch (weights and quantization parameters are
     shared; only the shapes and the input change)."""

@@ -339,3 +339,34 @@ def test_backend_config_from_json(chxvm):
         chxvm.BackendConfig.FromJSON('{"base": 3}')
     with pytest.raises(chxvm.ChxVMError):
         chxvm.BackendConfig.FromName("no_such_backend")
+
+
+def test_runtime_options(chxvm):
+    chxvm.set_option("qlinearconv_bias", "onnx_int32")
+    chxvm.set_option("qlinearconv_bias", "reference")
+    with pytest.raises(chxvm.ChxVMError, match="qlinearconv_bias"):
+        chxvm.set_option("qlinearconv_bias", "int64")
+    with pytest.raises(chxvm.ChxVMError, match="unknown option"):
+        chxvm.set_option("no_such_switch", "1")
+
+
+def test_whole_network_as_one_program(chxvm):
+    """A reduced ResNet converted to one ChxVMProgramProto survives the C++ reader and writer byte
+    for byte (loading it uploads its constants, so that part runs with the GPU tests); a pool
+    outside the DequantizeLinear -> pool -> QuantizeLinear pattern is refused at load."""
+    pkg = entry.load_package()
+    from importlib import import_module
+    wl = import_module(pkg.__name__ + ".workloads")
+    ops = import_module(pkg.__name__ + ".ops")
+    model = wl.build_resnet50(batch=1, image=32, seed=2, width=16, blocks=(1, 1, 1, 1), classes=4, device="cpu")
+    b = wl.program_to_chxvm(model, chxvm, ops)
+    data = b.serialize()
+    assert chxvm.proto_roundtrip(data) == data
+    assert len(b.instructions) > 3 * len(model["program"]) and b.input_names == ["x"]
+    lone = chxvm.ProgramBuilder()
+    x = lone.input("x", "float32", (1, 1, 4, 4))
+    y = lone.new_slot()
+    lone.add_raw("AveragePool", [("ARRAY", x), ("INTS", [2, 2]), ("INTS", [2, 2]), ("INTS", [0, 0]), ("INT", 0)], [y, -1])
+    lone.output("y", y)
+    with pytest.raises(chxvm.ChxVMError, match="AveragePool"):
+        chxvm.Program(lone.serialize())

@@ -200,3 +200,51 @@ def test_errors_name_the_instruction(g, vm):
     b.add("QuantizeLinear", x, s, -1, outputs=[q])
     with pytest.raises(vm.ChxVMError):
         vm.Program(b.serialize()).run({"x": g.dev(np.zeros(4, np.float32))})
+
+
+def _run_network_through_vm(g, vm, oracle, model, keep):
+    wl = g.pkg.workloads
+    serialized = wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize()
+    assert vm.proto_roundtrip(serialized) == serialized
+    vm.set_option("qlinearconv_bias", "onnx_int32")
+    try:
+        prog = vm.Program(serialized)
+        got = prog.run({"x": torch.from_numpy(model["input"]).cuda()})
+        prog.close()
+    finally:
+        vm.set_option("qlinearconv_bias", "reference")
+    oracle.set_threads(16)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"], keep=set(keep))
+    finally:
+        oracle.set_threads(1)
+    assert sorted(got) == sorted(keep)
+    for name in keep:
+        np.testing.assert_array_equal(got[name], ref[name], err_msg="value %s" % name)
+
+
+def test_small_resnet_as_one_program(g, vm, oracle):
+    """The reduced ResNet as one serialized program: QuantizeLinear, QLinearConv with constant
+    operands, DequantizeLinear -> MaxPool / AveragePool -> QuantizeLinear fused at load,
+    FusionGroups for the residual sums, Free after the last reader.  Every value, then only the logits."""
+    model = g.pkg.workloads.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]])
+    _run_network_through_vm(g, vm, oracle, model, ["logits"])
+
+
+def test_small_mobilenetv2_as_one_program(g, vm, oracle):
+    """Depthwise convolutions and 24-channel activations (pixel pitch padded to 16 bytes) in the VM."""
+    blocks = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 1, 2))
+    model = g.pkg.workloads.build_mobilenetv2(batch=2, image=64, seed=7, blocks=blocks, stem=32, head=128, classes=10)
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]])
+
+
+def test_unfused_pool_is_refused_at_load(g, vm):
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (1, 1, 4, 4))
+    y = b.new_slot()
+    b.add_raw("MaxPool", [("ARRAY", x), ("INTS", [2, 2]), ("INTS", [2, 2]), ("INTS", [0, 0]), ("INT", 0), ("STRING", "NOTSET")],
+              [y, -1])
+    b.output("y", y)
+    with pytest.raises(vm.ChxVMError, match="MaxPool"):
+        vm.Program(b.serialize())
