@@ -177,6 +177,7 @@ struct PackedWeights {
     int C64 = 0, OCpad = 0, KP = 0;
     int BK = 64;         // K bytes per kernel step; the packed layout depends on it
     bool dense = false;  // taps packed densely; activations go through an explicit im2col
+    int8_t* wd = nullptr;  // dense only: the same weights in the order of the planar-input kernel (inside wp's allocation)
 };
 
 // Dense packing pays when per-tap padding to 64 channels would at least double the K extent.
@@ -399,7 +400,14 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     memset(&a, 0, sizeof(a));
     int KH = cs.KH, KW = cs.KW, H = cs.H, W = cs.W, sh = c.p->stride_h, sw = c.p->stride_w, ph = c.p->pad_h_begin,
         pw_ = c.p->pad_w_begin, C16eff = C16;
-    if (pw.dense) {
+    // few channels read from planar rows: the direct kernel, no expanded matrix
+    const bool stem = pw.dense && pw.wd && !c.out_int32 && x.strides[3] == 1 &&
+                      stem_patch_fits(cs.C, cs.KH, cs.KW, sh, sw) && ph < 64 && pw_ < 64 &&
+                      (int64_t)cs.C * (x.strides[1] < 0 ? -x.strides[1] : x.strides[1]) < (int64_t(1) << 30) &&
+                      x.strides[2] > 0 && (int64_t)cs.H * x.strides[2] < (int64_t(1) << 30) && getenv("CHX_HIP_NO_STEM") == nullptr;
+    if (stem) {
+        // x is used in place
+    } else if (pw.dense) {
         // explicit im2col: [M][Kd] bytes, then a 1x1 convolution over Kd channels and M pixels in a row
         const int64_t M = (int64_t)cs.N * cs.OH * cs.OW;
         CHX_REQUIRE(M <= INT32_MAX, "QLinearConv: too many output pixels for the im2col path");
@@ -464,6 +472,32 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     }
     a.y_vec_ok = aligned(a.y, 16) && (a.y_px_stride % 16 == 0) ? 1 : 0;
     (void)es;
+    if (stem) {
+        ConvStemArgs sa;
+        memset(&sa, 0, sizeof(sa));
+        sa.x = static_cast<const char*>(x.data);
+        sa.x_n_stride = x.strides[0]; sa.x_c_stride = x.strides[1]; sa.x_h_stride = x.strides[2];
+        sa.N = cs.N; sa.C = cs.C; sa.H = cs.H; sa.W = cs.W; sa.OH = cs.OH; sa.OW = cs.OW; sa.KH = cs.KH; sa.KW = cs.KW;
+        sa.sh = sh; sa.sw = sw; sa.ph = ph; sa.pw = pw_;
+        sa.OC = cs.OC;
+        sa.wd = pw.wd;
+        sa.wsum = pw.wsum;
+        sa.x_zp = c.x_zp;
+        sa.x_unsigned = x.dtype == CHX_HIP_UINT8 ? 1 : 0;
+        sa.corr_mult = sa.x_unsigned ? 128 - c.x_zp : -c.x_zp;
+        sa.y = a.y; sa.y_px_stride = a.y_px_stride; sa.y_vec_ok = a.y_vec_ok;
+        sa.w_scale = c.w_scale; sa.w_scale_len = c.w_scale_len; sa.bias = c.bias;
+        sa.rq = c.rq;
+        sa.inv_y_scale = 1.0f / c.rq.q.scale;
+        sa.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
+        int rc = launch_conv_stem(sa, c.rne, s);
+        if (rc == CHX_HIP_OK && y_post) {
+            rc = launch_nhwc_to_nchw_u8(static_cast<const char*>(y_scratch), static_cast<char*>(y.data), cs.N, cs.OC,
+                                        (int64_t)cs.OH * cs.OW, (int)a.y_px_stride, s);
+        }
+        release_scratch(c.cache, y_scratch, s);
+        return rc;
+    }
     a.C16 = C16eff;
     a.C64 = pw.C64;
     a.H = H; a.W = W; a.KH = KH; a.KW = KW;
@@ -550,7 +584,11 @@ namespace {
 // Allocates and fills packed weights.  With `persistent` the buffers come from hipMalloc and
 // live until release_packed(); otherwise they are stream-ordered scratch.
 int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedWeights* pw) {
-    const size_t bytes = packed_bytes((int)w.shape[0], (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], pw);
+    const size_t mfma_bytes = packed_bytes((int)w.shape[0], (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], pw);
+    const bool stem = pw->dense && stem_shape_fits((int)w.shape[1], (int)w.shape[2], (int)w.shape[3]);
+    const size_t stem_bytes =
+            stem ? (size_t)(pw->OCpad / 64) * stem_k_blocks((int)w.shape[1], (int)w.shape[2], (int)w.shape[3]) * 2048 : 0;
+    const size_t bytes = mfma_bytes + stem_bytes;
     void* p0 = nullptr;
     void* p1 = nullptr;
     if (persistent) {
@@ -568,6 +606,8 @@ int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedW
     }
     pw->wp = static_cast<int8_t*>(p0);
     pw->wsum = static_cast<int32_t*>(p1);
+    pw->wd = stem ? pw->wp + mfma_bytes : nullptr;
+    if (stem) CHX_PROPAGATE(pack_weights_stem(w, pw->OCpad, pw->wd, s));
     if (pw->dense) return pack_weights_dense(w, pw->KP, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
     return pack_weights(w, pw->C64, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
 }
@@ -582,6 +622,7 @@ void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
     }
     pw->wp = nullptr;
     pw->wsum = nullptr;
+    pw->wd = nullptr;
 }
 
 // Depthwise 3x3 on int8 weights with zero weight zero points: paired weights and per-channel sums.

@@ -38,6 +38,33 @@ struct ConvMfmaArgs {
     uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
 };
 
+// Direct convolution over planar activations with few channels (conv_stem.hip).
+struct ConvStemArgs {
+    // activations, rows contiguous: element (n, c, ih, iw) at x + n*x_n_stride + c*x_c_stride + ih*x_h_stride + iw
+    const char* x;
+    int64_t x_n_stride, x_c_stride, x_h_stride;
+    int32_t N, C, H, W, OH, OW, KH, KW, sh, sw, ph, pw;
+    int32_t OC;
+    const int8_t* wd;     // pack_weights_stem
+    const int32_t* wsum;  // [OC padded]
+    int32_t x_zp;
+    int32_t x_unsigned;
+    int32_t corr_mult;    // (128 - x_zp) for uint8 x, (-x_zp) for int8 x
+    char* y;              // pixel-major, as for ConvMfmaArgs
+    int64_t y_px_stride;
+    int32_t y_vec_ok;
+    const float* w_scale;
+    int32_t w_scale_len;
+    const int32_t* bias;
+    RequantParams rq;
+    float inv_y_scale;
+    float lo_folded;
+    // filled by the launcher
+    int32_t KB, tiles_h, tiles_w, tiles;
+    uint32_t m_ppw, m_ph, m_kh;
+    uint32_t tpi_mul, tpi_shift, tw_mul, tw_shift;  // magic_divisor(tiles per image), magic_divisor(tiles_w)
+};
+
 struct Im2colArgs {
     const char* x;
     int64_t xs[4];  // byte strides of N, C, H, W
@@ -59,6 +86,12 @@ inline void magic_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
 int pack_weights_dense(const chx_hip_tensor& w, int Kd, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 int launch_im2col_dense(const Im2colArgs& a, hipStream_t s);
 int pack_weights(const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+// the stem kernel: weights [C][KH][KW] with C*KH <= 32 and KW <= 8; patch = LDS bytes of a tile's input rows
+bool stem_shape_fits(int C, int KH, int KW);
+bool stem_patch_fits(int C, int KH, int KW, int sh, int sw);
+int stem_k_blocks(int C, int KH, int KW);
+int pack_weights_stem(const chx_hip_tensor& w, int OCpad64, int8_t* wd, hipStream_t s);
+int launch_conv_stem(ConvStemArgs a, bool rne, hipStream_t s);
 // max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once)
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s);

@@ -284,10 +284,43 @@ __device__ __forceinline__ void wait_fragments(v4i (&fa)[FM], v4i (&fb)[FN]) {
         asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(fa[0]), "+v"(fb[0]) : "n"(N) : "memory");
 }
 
+// Touch every 64-byte line of the kernel arguments at once.  The argument block of a fresh launch
+// is not in any cache, and the compiler fetches the fields in several dependent batches that
+// each touch new lines: one round trip to memory per batch.  After this, one round trip.
+template <int BYTES>
+__device__ __forceinline__ void warm_kernel_arguments() {
+    const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
+    static_assert(BYTES <= 256, "four lines are touched");
+    int t0, t1, t2, t3;
+    asm volatile(
+            "s_load_dword %0, %4, 0x0\n\t"
+            "s_load_dword %1, %4, 0x40\n\t"
+            "s_load_dword %2, %4, 0x80\n\t"
+            "s_load_dword %3, %4, 0xc0\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3)
+            : "s"(ka)
+            : "memory");
+}
+
 // Wait until at most N of this wave's vector-memory operations are outstanding.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// LDS ring stages of a work-group: what fits the budget, between 2 and the cap.  The bytes in
+// flight towards a compute unit, (stages - 1) * stage bytes * resident work-groups, set the copy
+// rate that the memory latency allows.
+#ifndef CHX_CONV_LDS_BUDGET
+#define CHX_CONV_LDS_BUDGET (80 * 1024)
+#endif
+#ifndef CHX_CONV_NS_MAX
+#define CHX_CONV_NS_MAX 3
+#endif
+constexpr int ring_stages(int stage_bytes) {
+    const int fit = CHX_CONV_LDS_BUDGET / stage_bytes;
+    return fit < 2 ? 2 : fit > CHX_CONV_NS_MAX ? CHX_CONV_NS_MAX : fit;
 }
 
 // FM x FN MFMA tiles (32x32) per wavefront; four wavefronts in a 2x2 grid per work-group.
@@ -320,7 +353,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     constexpr int TM = 64 * FM;  // output channels per tile
     constexpr int TN = 64 * FN;  // pixels per tile
     constexpr int STAGE_BYTES = (TM + TN) * BK;
-    constexpr int NS = 3 * STAGE_BYTES <= 80 * 1024 ? 3 : 2;  // LDS stages: two work-groups per compute unit
+    constexpr int NS = ring_stages(STAGE_BYTES);
     constexpr int CH = BK / 16;          // 16-byte chunks per staged row
     constexpr int RPI = 64 / CH;         // rows one copy instruction fills
     constexpr int CA = TM / RPI / 4;     // copy instructions per wave and stage, weight rows
@@ -333,6 +366,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     __shared__ __attribute__((aligned(16))) int32_t s_add[TM];
     __shared__ __attribute__((aligned(16))) float s_fbias[TM];
 
+    warm_kernel_arguments<sizeof(ConvMfmaArgs)>();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -269,3 +269,56 @@ def test_depthwise_qlinear_conv(g, oracle, case, xdt):
     got = g.ops.QLinearConv(g.to_channels_last(g.dev(x)), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, -5, g.dev(bias),
                             zero_point_dtype=torch.int8, flags=fl, **kw)
     np.testing.assert_array_equal(g.host(got), want)
+
+
+@pytest.mark.parametrize("xdt", [np.uint8, np.int8])
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, OC, KH, KW, stride, pad
+    (2, 3, 37, 41, 64, 7, 7, 2, 3),     # ResNet stem geometry, ragged tiles
+    (1, 3, 33, 30, 32, 3, 3, 2, 1),     # MobileNetV2 stem geometry: 4-byte filter rows, half an output-channel block
+    (1, 1, 20, 20, 10, 5, 5, 1, 2),     # one channel, stride 1
+    (2, 4, 17, 19, 96, 3, 3, 1, 1),     # two output-channel blocks
+    (1, 3, 16, 50, 130, 7, 7, 2, 3),    # three blocks, the last with 2 channels
+    (1, 2, 9, 12, 7, 8, 8, 1, 0),       # filter rows of exactly 8 bytes
+    (1, 8, 12, 12, 16, 4, 4, 2, 1),     # C * KH = 32, the most K groups
+    (1, 3, 9, 9, 8, 3, 3, 3, 0),        # stride 3
+])
+def test_planar_input_qlinear_conv(g, oracle, case, xdt):
+    """Few input channels read from NCHW rows (the direct first-layer kernel): stateless call and
+    plan, NCHW and channels-last outputs, a strided view as input, both bias modes, fused Relu,
+    ONNX rounding."""
+    N, C, H, W, OC, KH, KW, stride, pad = case
+    rng = np.random.default_rng(51)
+    x = rand_q(rng, (N, C, H, W), xdt)
+    w = rng.integers(-127, 128, size=(OC, C, KH, KW)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-2000, 2001, size=OC).astype(np.int32)
+    xz = 103 if xdt == np.uint8 else -9
+    ys = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C * KH * KW) / 40)
+    kw = dict(strides=(stride, stride), pads=(pad, pad))
+    for bias_mode, flags in ((oracle.BIAS_ONNX_INT32, g.capi.BIAS_ONNX_INT32), (oracle.BIAS_REFERENCE_FLOAT, 0)):
+        want = oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, 121, np.uint8, bias=bias, bias_mode=bias_mode, **kw)
+        assert want.min() < want.max()
+        got = g.ops.QLinearConv(g.dev(x), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, 121, g.dev(bias), flags=flags, **kw)
+        np.testing.assert_array_equal(g.host(got), want)
+        plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), **kw)
+        out_cl = torch.empty((want.shape[0], want.shape[2], want.shape[3], want.shape[1]), dtype=torch.uint8,
+                             device="cuda").permute(0, 3, 1, 2)
+        out_nchw = torch.empty(want.shape, dtype=torch.uint8, device="cuda")
+        # a view into a larger tensor: channel and image strides that are not the dense ones
+        big = torch.zeros((N, C + 1, H + 2, W), dtype=g.dev(x).dtype, device="cuda")
+        big[:, :C, 1:H + 1, :] = g.dev(x)
+        view = big[:, :C, 1:H + 1, :]
+        for xin in (g.dev(x), view):
+            for out in (out_cl, out_nchw):
+                out.zero_()
+                plan.run(xin, 0.02, xz, ys, 121, flags=flags, out=out)
+                np.testing.assert_array_equal(g.host(out), want)
+        plan.close()
+    fl = g.capi.BIAS_ONNX_INT32 | g.capi.FUSE_RELU | g.capi.ROUND_ONNX_RNE
+    want = np.maximum(oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, -5, np.int8, bias=bias, bias_mode=oracle.BIAS_ONNX_INT32,
+                                              round_mode=oracle.ROUND_ONNX_RNE, **kw), -5).astype(np.int8)
+    got = g.ops.QLinearConv(g.dev(x), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, -5, g.dev(bias),
+                            zero_point_dtype=torch.int8, flags=fl, **kw)
+    np.testing.assert_array_equal(g.host(got), want)
