@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every op from the host instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline")
+    ap.add_argument("--no-fuse-residual", action="store_true",
+                    help="run the residual Add(+Relu) groups as kernels of their own instead of inside the convolution before them")
     ap.add_argument("--parts", type=int, default=1,
                     help="run the batch as this many concurrent slices on separate streams (network workloads)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
@@ -110,8 +112,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # compute units busy through its ramp and tail, so slices fill each other's gaps).  The
     # default is the plain whole-batch runner, whose launches are the ones the roofline figure
     # below prices.
-    runner = wl.DeviceRunner(model, pkg) if args.parts <= 1 else None
-    timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts)
+    fuse = not args.no_fuse_residual
+    runner = wl.DeviceRunner(model, pkg, fuse) if args.parts <= 1 else None
+    timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts, fuse)
 
     def step(_timer):
         timed_runner.run(x)
@@ -138,14 +141,14 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     for rn, xs in slices:
         vals = rn.run(xs)
         torch.cuda.synchronize()
-        for ins in model["program"]:
+        for fid, ins in enumerate(model["program"]):
             if ins[0] != "QLinearConv":
                 continue
             c = model["convs"][ins[3]]
             if mobilenet and c.group == 1:
                 continue  # MobileNetV2: the roofline figure is the depthwise kernel's
-            fn = lambda: rn.plans[ins[3]].run(vals[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
-                                              flags=capi.BIAS_ONNX_INT32, out=rn.bufs[ins[1]])
+            # the instruction as the timed step launches it (with its residual sum when that is fused in)
+            fn = lambda: rn.launch(fid, vals)
             # REP launches recorded into a graph of their own: replayed, they follow each other the way
             # the instructions of the timed graph do, without host submission gaps between them
             fn()
@@ -191,7 +194,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
                config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,
                            layout="channels_last", launch="host" if args.no_graph else "hip_graph_replay",
-                           concurrent_batch_slices=max(1, args.parts),
+                           concurrent_batch_slices=max(1, args.parts), residual_add="separate" if args.no_fuse_residual else "in_conv_epilogue",
                            conv_gmac_per_image=model["macs"] / batch / 1e9))
 
     def cpu():

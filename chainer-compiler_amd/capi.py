@@ -22,12 +22,13 @@ ROUND_ONNX_RNE = 1
 BIAS_REFERENCE_FLOAT = 0
 BIAS_ONNX_INT32 = 2
 FUSE_RELU = 4
+EINVAL, EUNSUPPORTED, ERUNTIME = 1, 2, 3
 
 EXPORTS = [
     "chx_hip_init", "chx_hip_last_error", "chx_hip_version", "chx_hip_get_device_props", "chx_hip_malloc",
     "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
-    "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
+    "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
     "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source",
     "chx_hip_max_pool_q8", "chx_hip_average_pool_q8",
 ]

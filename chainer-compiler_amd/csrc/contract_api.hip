@@ -364,6 +364,7 @@ struct ConvCall {
     int32_t w_scale_len;
     const int32_t* bias;
     RequantParams rq;
+    const ResidualAdd* res = nullptr;  // a residual sum fused behind the requantization
 };
 
 // Runs the MFMA kernel on packed weights.  x may be channels-last (used in place) or
@@ -405,6 +406,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
                       stem_patch_fits(cs.C, cs.KH, cs.KW, sh, sw) && ph < 64 && pw_ < 64 &&
                       (int64_t)cs.C * (x.strides[1] < 0 ? -x.strides[1] : x.strides[1]) < (int64_t(1) << 30) &&
                       x.strides[2] > 0 && (int64_t)cs.H * x.strides[2] < (int64_t(1) << 30) && getenv("CHX_HIP_NO_STEM") == nullptr;
+    if (stem && c.res) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "the planar-input kernel has no fused residual sum");
     if (stem) {
         // x is used in place
     } else if (pw.dense) {
@@ -456,7 +458,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     if (y_is_pixel_major(y, &y_px)) {
         a.y = static_cast<char*>(y.data);
         a.y_px_stride = y_px;
-    } else if (is_contiguous(y) && !c.out_int32) {
+    } else if (is_contiguous(y) && !c.out_int32 && !c.res) {
         const int64_t OHW = (int64_t)cs.OH * cs.OW;
         const int pitch = round_up(cs.OC, 16);
         if (acquire_scratch(c.cache, 1, (size_t)cs.N * OHW * pitch, s, &y_scratch) != CHX_HIP_OK) {
@@ -520,6 +522,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.rq = c.rq;
     a.inv_y_scale = c.out_int32 ? 0.f : 1.0f / c.rq.q.scale;
     a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
+    if (c.res) a.res = *c.res;
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64, cap = 0;
     pick_tile(cs.OC, a.M, &toc, &tpx);
@@ -893,6 +896,55 @@ extern "C" int chx_hip_qconv_plan_run(
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
     return launch_conv_direct(q.direct, rne, s);
+}
+
+extern "C" int chx_hip_qconv_plan_run_add(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
+        int32_t y_zero_point, int32_t y_dtype, uint32_t flags, const chx_hip_tensor* r, float r_scale, int32_t r_zero_point,
+        float out_scale, int32_t out_zero_point, int32_t relu, chx_hip_tensor* out, void* stream) {
+    CHX_REQUIRE(plan != nullptr, "QLinearConv+Add: null plan");
+    CHX_PROPAGATE(check_tensor(r, "QLinearConv+Add r"));
+    CHX_PROPAGATE(check_tensor(out, "QLinearConv+Add out"));
+    CHX_REQUIRE(is_q8(y_dtype) && is_q8(r->dtype) && is_q8(out->dtype), "QLinearConv+Add: y, r and out must be uint8 or int8");
+    CHX_REQUIRE(r->ndim == 4 && out->ndim == 4, "QLinearConv+Add: r and out must be 4-D");
+    for (int i = 0; i < 4; ++i)
+        CHX_REQUIRE(r->shape[i] == out->shape[i], "QLinearConv+Add: r and out differ in shape (no broadcasting)");
+    auto in_range = [](int32_t zp, int32_t dt) { return dt == CHX_HIP_INT8 ? zp >= -128 && zp <= 127 : zp >= 0 && zp <= 255; };
+    CHX_REQUIRE(in_range(r_zero_point, r->dtype) && in_range(out_zero_point, out->dtype),
+                "QLinearConv+Add: zero point out of the range of its type");
+    if (!(out_scale >= 0x1p-60f && out_scale <= 0x1p60f))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv+Add: out_scale outside [2^-60, 2^60]");
+    // the convolution's own result has the layout of `out` and the type y_dtype
+    chx_hip_tensor y = *out;
+    y.dtype = y_dtype;
+    QConvChecked q;
+    CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, &plan->w, &plan->w_scale, &plan->w_zero_point, y_scale,
+                              y_zero_point, plan->has_bias ? &plan->bias : nullptr, &plan->params, flags, &y, &q));
+    if (!plan->mfma) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv+Add: these weights do not run on the matrix-core kernel");
+    int64_t r_px = 0, o_px = 0;
+    if (!y_is_pixel_major(*r, &r_px) || !y_is_pixel_major(*out, &o_px))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv+Add: r and out must be channels-last");
+    ResidualAdd res;
+    memset(&res, 0, sizeof(res));
+    res.r = static_cast<const char*>(r->data);
+    res.r_px_stride = r_px;
+    res.r_vec_ok = aligned(r->data, 16) && r_px % 16 == 0 ? 1 : 0;
+    res.c_flip = y_dtype == CHX_HIP_INT8 ? 0x80808080u : 0u;
+    res.r_flip = r->dtype == CHX_HIP_INT8 ? 0x80808080u : 0u;
+    res.c_zpf = (float)(y_zero_point + (y_dtype == CHX_HIP_INT8 ? 128 : 0));
+    res.c_scale = y_scale;
+    res.r_zpf = (float)(r_zero_point + (r->dtype == CHX_HIP_INT8 ? 128 : 0));
+    res.r_scale = r_scale;
+    res.relu = relu ? 1 : 0;
+    res.out = make_quant_params(out_scale, out_zero_point, out->dtype == CHX_HIP_INT8);
+    res.inv_out_scale = 1.0f / out_scale;
+    res.big = 0x1p40f * out_scale;
+    hipStream_t s = as_stream(stream);
+    ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0);
+    call.cache = const_cast<ScratchCache*>(&plan->scratch);
+    call.tune = const_cast<TuneCache*>(&plan->tune);
+    call.res = &res;
+    return run_conv_mfma(call, plan->pw, s);
 }
 
 extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {

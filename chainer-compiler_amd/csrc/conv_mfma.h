@@ -7,6 +7,27 @@
 
 namespace chx {
 
+// A residual sum fused behind the requantization: the 8-bit code c of the convolution is not
+// written; the kernel writes  Q_out( act( DQ_y(c) + DQ_r(r) ) )  instead, which is what a
+// QLinearConv followed by the element-wise group {DequantizeLinear, DequantizeLinear, Add,
+// [Relu], QuantizeLinear} computes, operation by operation.  A signed code is read as
+// (byte ^ 0x80) - 128, so the flips and the "+128" below make one code path serve both types.
+struct ResidualAdd {
+    const char* r;         // pixel-major like y: element (m, oc) at r + m*r_px_stride + oc
+    int64_t r_px_stride;
+    int32_t r_vec_ok;      // 16-byte loads allowed
+    uint32_t c_flip;       // 0x80808080 when the convolution's code is int8
+    uint32_t r_flip;       // ... when r is int8
+    float c_zpf;           // y_zero_point (+128 for int8), as float
+    float c_scale;         // y_scale
+    float r_zpf;           // r's zero point (+128 for int8)
+    float r_scale;
+    int32_t relu;
+    QuantParams out;       // quantization of the sum
+    float inv_out_scale;
+    float big;             // 2^40 * out.scale: the dividend is limited to +-big (both sides saturate beyond)
+};
+
 struct ConvMfmaArgs {
     // activations, channels-last: element (n, c, ih, iw) at x + n*x_n_stride + ih*x_h_stride + iw*x_w_stride + c
     const char* x;
@@ -36,6 +57,7 @@ struct ConvMfmaArgs {
     float lo_folded;             // lower clamp bound with the fused Relu folded in (fold_relu_floor)
     int32_t tiles_oc, tiles_px;  // filled by the launcher
     uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
+    ResidualAdd res;             // res.r == nullptr: plain QLinearConv
 };
 
 // Direct convolution over planar activations with few channels (conv_stem.hip).

@@ -290,17 +290,45 @@ __device__ __forceinline__ void wait_fragments(v4i (&fa)[FM], v4i (&fb)[FN]) {
 template <int BYTES>
 __device__ __forceinline__ void warm_kernel_arguments() {
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
-    static_assert(BYTES <= 256, "four lines are touched");
-    int t0, t1, t2, t3;
+    constexpr int LINES = (BYTES + 63) / 64;
+    static_assert(LINES >= 4 && LINES <= 6, "between four and six lines are touched");
+    // offsets of the last lines, clamped into the block so that nothing outside it is read
+    constexpr int L4 = LINES > 4 ? 0x100 : 0xc0, L5 = LINES > 5 ? 0x140 : L4;
+    int t0, t1, t2, t3, t4, t5;
     asm volatile(
-            "s_load_dword %0, %4, 0x0\n\t"
-            "s_load_dword %1, %4, 0x40\n\t"
-            "s_load_dword %2, %4, 0x80\n\t"
-            "s_load_dword %3, %4, 0xc0\n\t"
+            "s_load_dword %0, %6, 0x0\n\t"
+            "s_load_dword %1, %6, 0x40\n\t"
+            "s_load_dword %2, %6, 0x80\n\t"
+            "s_load_dword %3, %6, 0xc0\n\t"
+            "s_load_dword %4, %6, %7\n\t"
+            "s_load_dword %5, %6, %8\n\t"
             "s_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3)
-            : "s"(ka)
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5)
+            : "s"(ka), "n"(L4), "n"(L5)
             : "memory");
+}
+
+// Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
+// (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
+// reference's order, one IEEE operation each.
+__device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
+        int32_t code[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
+            const float fb = ((float)((rw >> (8 * e)) & 0xffu) - p.r_zpf) * p.r_scale;
+            float sum = fa + fb;
+            if (p.relu) sum = __builtin_fmaxf(sum, 0.f);
+            sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
+            code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
+        }
+        out[w] = (int)pack4(code[0], code[1], code[2], code[3]);
+    }
+    return out;
 }
 
 // Wait until at most N of this wave's vector-memory operations are outstanding.
@@ -347,7 +375,7 @@ constexpr int ring_stages(int stage_bytes) {
 // tile) and an invalid chunk is fetched from a 64-byte row holding the zero point instead
 // (g_fill_rows), which makes it contribute (zp - zp) * w = 0.  Without kPad (1x1 and other
 // unpadded convolutions on 64-multiple channels, matrix products) every chunk is valid.
-template <int FM, int FN, int BK, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad>
+template <int FM, int FN, int BK, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad, bool kRes>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv_mfma_kernel(ConvMfmaArgs a) {
     constexpr int T = 256;
     constexpr int TM = 64 * FM;  // output channels per tile
@@ -600,10 +628,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             const int64_t m = m0 + pxl;
             const int oc = oc0 + ch * 16;
             if (m >= a.M || oc >= a.OC) continue;
-            const char* src = staged(lds_out, pxl, ch * 16);
-            const v4i val = *reinterpret_cast<const v4i*>(src);
+            char* src = staged(lds_out, pxl, ch * 16);
+            v4i val = *reinterpret_cast<const v4i*>(src);
+            const bool whole = oc + 16 <= a.OC;
+            if (kRes) {
+                const char* rsrc = a.res.r + m * a.res.r_px_stride + oc;
+                v4i rv = {0, 0, 0, 0};
+                if (a.res.r_vec_ok && whole) {
+                    rv = *reinterpret_cast<const v4i*>(rsrc);
+                } else {
+#pragma nounroll
+                    for (int w = 0; w < 4; ++w) {
+                        uint32_t word = 0;
+                        for (int e = 0; e < 4; ++e)
+                            if (oc + w * 4 + e < a.OC) word |= (uint32_t)(uint8_t)rsrc[w * 4 + e] << (8 * e);
+                        rv[w] = (int)word;
+                    }
+                }
+                val = add_residual16(val, rv, a.res);
+                if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
+            }
             char* dst = a.y + m * a.y_px_stride + oc;
-            if (a.y_vec_ok && oc + 16 <= a.OC) {
+            if (a.y_vec_ok && whole) {
                 *reinterpret_cast<v4i*>(dst) = val;
             } else {
 #pragma nounroll
@@ -692,7 +738,7 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
         }
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, BK, true, false, false, true>), 256, 0) !=
+                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, BK, true, false, false, true, false>), 256, 0) !=
                     hipSuccess ||
             per_cu < 1)
             per_cu = 2;
@@ -705,14 +751,20 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
     // padding-free variant: no tap can leave the image and channels fill whole 64-byte K steps
     const bool pad = a.ph != 0 || a.pw != 0 || (a.C16 % BK) != 0 ||
                      (int64_t)(a.OH - 1) * a.sh + a.KH > a.H || (int64_t)(a.OW - 1) * a.sw + a.KW > a.W;
-#define CHX_LAUNCH(XU, OI, RN)                                                           \
-    do {                                                                                 \
-        if (pad)                                                                         \
-            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, true><<<grid, 256, 0, s>>>(a);      \
-        else                                                                             \
-            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, false><<<grid, 256, 0, s>>>(a);     \
+#define CHX_LAUNCH_R(XU, OI, RN, RS)                                                       \
+    do {                                                                                   \
+        if (pad)                                                                           \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, true, RS><<<grid, 256, 0, s>>>(a);    \
+        else                                                                               \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, false, RS><<<grid, 256, 0, s>>>(a);   \
     } while (0)
-    if (out_int32) {
+#define CHX_LAUNCH(XU, OI, RN) CHX_LAUNCH_R(XU, OI, RN, false)
+    if (a.res.r) {
+        // the fused residual sum exists for 8-bit results in the reference's rounding
+        if (out_int32 || rne) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "conv_mfma: a fused residual sum needs an 8-bit result and the reference rounding");
+        if (x_unsigned) CHX_LAUNCH_R(true, false, false, true);
+        else CHX_LAUNCH_R(false, false, false, true);
+    } else if (out_int32) {
         if (x_unsigned) CHX_LAUNCH(true, true, false);
         else CHX_LAUNCH(false, true, false);
     } else if (rne) {
@@ -723,6 +775,7 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
         else CHX_LAUNCH(false, false, false);
     }
 #undef CHX_LAUNCH
+#undef CHX_LAUNCH_R
     return launch_check("conv_mfma_kernel");
 }
 

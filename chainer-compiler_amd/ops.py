@@ -217,6 +217,21 @@ class QLinearConvPlan(object):
             ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
         return out
 
+    def run_add(self, x, x_scale, x_zero_point, y_scale, y_zero_point, r, r_scale, r_zero_point, out_scale,
+                out_zero_point, relu, zero_point_dtype=torch.uint8, flags=0, out=None):
+        """QLinearConv followed by QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r))) as
+        one kernel (chx_hip_qconv_plan_run_add); `zero_point_dtype` is the type of the convolution's
+        own result y, which is not written.  Raises ChxHipError with code EUNSUPPORTED when the
+        weights or layouts do not fit; run the two ops separately then."""
+        handle, shape = self._plan_for(x)
+        if out is None:
+            out = _alloc_like_input_layout(r, shape, r.dtype)
+        capi.check(capi.lib().chx_hip_qconv_plan_run_add(
+            handle, capi.ref(x), _f(x_scale), _i(x_zero_point), _f(y_scale), _i(y_zero_point),
+            _i(capi._TORCH_TO_CHX[zero_point_dtype]), ctypes.c_uint32(flags), capi.ref(r), _f(r_scale), _i(r_zero_point),
+            _f(out_scale), _i(out_zero_point), _i(1 if relu else 0), capi.ref(out), capi.stream_ptr()))
+        return out
+
     def close(self):
         for handle in self._plans.values():
             capi.lib().chx_hip_qconv_plan_destroy(handle)

@@ -280,8 +280,19 @@ class DeviceRunner(object):
     """Runs a program on the MI355X: weights resident, one plan per QLinearConv, every
     activation channels-last, all intermediate buffers allocated once."""
 
-    def __init__(self, model, pkg):
+    def __init__(self, model, pkg, fuse_residual=False):
+        """fuse_residual: a QLinearConv whose only reader is the residual Add(+Relu) of its block runs
+        as one kernel with it; the convolution's own output is then not materialised."""
         self.m, self.ops, self.capi = model, pkg.ops, pkg.capi
+        self.fused_into = {}   # conv output name -> the Add instruction that absorbs it
+        if fuse_residual:
+            program = model["program"]
+            for i, ins in enumerate(program):
+                if ins[0] in ("AddRelu", "Add") and i > 0:
+                    prev = program[i - 1]
+                    readers = sum(1 for other in program if prev[1] in other[2:4] and other[0] != "QuantizeLinear")
+                    if prev[0] == "QLinearConv" and prev[1] in ins[2:4] and readers == 1 and model["convs"][prev[3]].group == 1:
+                        self.fused_into[prev[1]] = ins
         self.dev = {}
         self.plans = {}
         self.bufs = {}
@@ -316,30 +327,49 @@ class DeviceRunner(object):
             if ins[0] == "Add":
                 self.fusion[out] = add_program(self.ops, q[ins[2]], q[ins[3]], q[out])
 
-    def run(self, x):
+    def launch(self, fid, v):
+        """Launches instruction number `fid` of the program on the values `v` (name -> tensor)."""
         ops, q, m = self.ops, self.m["qparams"], self.m
+        ins = m["program"][fid]
+        kind, out = ins[0], ins[1]
+        buf = self.bufs[out]
+        if kind == "QuantizeLinear":
+            ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
+        elif kind == "QLinearConv" and out in self.fused_into:
+            add = self.fused_into[out]
+            other = add[3] if add[2] == out else add[2]
+            c = m["convs"][ins[3]]
+            # DequantizeLinear(a) + DequantizeLinear(b) is commutative bit for bit, so the
+            # convolution may be either operand of the Add
+            self.plans[ins[3]].run_add(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, v[other], q[other][0], q[other][1],
+                                       q[add[1]][0], q[add[1]][1], add[0] == "AddRelu", torch.uint8,
+                                       flags=self.capi.BIAS_ONNX_INT32, out=self.bufs[add[1]])
+            return None
+        elif kind in ("AddRelu", "Add") and (ins[2] in self.fused_into or ins[3] in self.fused_into):
+            pass   # written by the fused convolution
+        elif kind == "QLinearConv":
+            c = m["convs"][ins[3]]
+            self.plans[ins[3]].run(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
+                                   flags=self.capi.BIAS_ONNX_INT32, out=buf)
+        elif kind == "MaxPool":
+            ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
+        elif kind in ("AddRelu", "Add"):
+            ops.ElementWiseNvrtc([self.full[ins[2]], self.full[ins[3]]], 1, self.fusion[out], fid, outs=[self.full[out]])
+        elif kind == "AveragePool":
+            ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
+                              q[out][1], out=buf)
+        elif kind == "DequantizeLinear":
+            ops.DequantizeLinear(v[ins[2]], ins[3], ins[4], out=buf)
+        else:
+            raise ValueError(kind)
+        return buf
+
+    def run(self, x):
         v = {"x": x}
-        for fid, ins in enumerate(m["program"]):
-            kind, out = ins[0], ins[1]
-            buf = self.bufs[out]
-            if kind == "QuantizeLinear":
-                ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
-            elif kind == "QLinearConv":
-                c = m["convs"][ins[3]]
-                self.plans[ins[3]].run(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
-                                       flags=self.capi.BIAS_ONNX_INT32, out=buf)
-            elif kind == "MaxPool":
-                ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
-            elif kind in ("AddRelu", "Add"):
-                ops.ElementWiseNvrtc([self.full[ins[2]], self.full[ins[3]]], 1, self.fusion[out], fid, outs=[self.full[out]])
-            elif kind == "AveragePool":
-                ops.AveragePoolQ8(v[ins[2]], q[ins[2]][0], q[ins[2]][1], (ins[3], ins[3]), (1, 1), (0, 0), q[out][0],
-                                  q[out][1], out=buf)
-            elif kind == "DequantizeLinear":
-                ops.DequantizeLinear(v[ins[2]], ins[3], ins[4], out=buf)
-            else:
-                raise ValueError(kind)
-            v[out] = buf
+        for fid, ins in enumerate(self.m["program"]):
+            buf = self.launch(fid, v)
+            if buf is not None:
+                v[ins[1]] = buf
         return v
 
     def capture(self, x):
@@ -439,11 +469,11 @@ class ConcurrentRunner(object):
     few to keep 256 compute units busy through its ramp and tail, and the slices' kernels fill
     each other's gaps."""
 
-    def __init__(self, model, pkg, parts=2):
+    def __init__(self, model, pkg, parts=2, fuse_residual=False):
         n = model["shapes"]["x"][0]
         bounds = [n * i // parts for i in range(parts + 1)]
         self.slices = [(bounds[i], bounds[i + 1]) for i in range(parts) if bounds[i + 1] > bounds[i]]
-        self.runners = [DeviceRunner(slice_model(model, lo, hi), pkg) for lo, hi in self.slices]
+        self.runners = [DeviceRunner(slice_model(model, lo, hi), pkg, fuse_residual) for lo, hi in self.slices]
         self.streams = [torch.cuda.Stream() for _ in self.runners]
 
     def run(self, x):

@@ -164,6 +164,18 @@ int chx_hip_qconv_plan_create(
 int chx_hip_qconv_plan_run(
         const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
         int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
+/* A QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94) whose only reader is the
+ * element-wise group  QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r)))  of a
+ * residual block (ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161, act = Relu or
+ * nothing), run as one kernel: the convolution's 8-bit result y (type y_dtype, quantization
+ * y_scale / y_zero_point) is never written, `out` receives the group's result, computed operation
+ * by operation as the two ops would.  r and out: same shape as y, channels-last, uint8 or int8.
+ * CHX_HIP_EUNSUPPORTED when the plan's weights or the layouts do not fit the matrix-core kernel;
+ * the caller then runs the two ops separately. */
+int chx_hip_qconv_plan_run_add(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
+        int32_t y_zero_point, int32_t y_dtype, uint32_t flags, const chx_hip_tensor* r, float r_scale, int32_t r_zero_point,
+        float out_scale, int32_t out_zero_point, int32_t relu, chx_hip_tensor* out, void* stream);
 void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan);
 
 /* ---- integer contractions ------------------------------------------------------------- */

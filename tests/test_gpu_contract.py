@@ -322,3 +322,54 @@ def test_planar_input_qlinear_conv(g, oracle, case, xdt):
     got = g.ops.QLinearConv(g.dev(x), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, -5, g.dev(bias),
                             zero_point_dtype=torch.int8, flags=fl, **kw)
     np.testing.assert_array_equal(g.host(got), want)
+
+
+def _residual_sum(oracle, c, c_scale, c_zp, r, r_scale, r_zp, relu, out_scale, out_zp, out_dtype):
+    """QuantizeLinear(act(DequantizeLinear(c) + DequantizeLinear(r))), op by op on the CPU."""
+    s = oracle.binary(oracle.ADD, oracle.dequantize_linear(c, c_scale, c_zp), oracle.dequantize_linear(r, r_scale, r_zp))
+    if relu:
+        s = oracle.relu(s)
+    return oracle.quantize_linear(s, out_scale, out_zp, out_dtype)
+
+
+@pytest.mark.parametrize("ydt,rdt,odt", [(np.uint8, np.uint8, np.uint8), (np.int8, np.uint8, np.int8), (np.uint8, np.int8, np.uint8)])
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, OC, K, stride, pad
+    (2, 64, 9, 10, 256, 1, 1, 0), (1, 32, 7, 7, 24, 1, 1, 0), (2, 16, 8, 8, 70, 3, 1, 1), (1, 128, 6, 5, 128, 1, 2, 0)])
+def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
+    """chx_hip_qconv_plan_run_add against QLinearConv followed by the element-wise group, each on
+    the CPU oracle: with and without Relu, all type combinations, channel counts that leave partial
+    16-byte chunks, a residual with a padded pixel pitch."""
+    N, C, H, W, OC, K, stride, pad = case
+    rng = np.random.default_rng(61)
+    x = rand_q(rng, (N, C, H, W), np.uint8)
+    w = rng.integers(-127, 128, size=(OC, C, K, K)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-500, 501, size=OC).astype(np.int32)
+    ys = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C * K * K) / 40)
+    yz = 119 if ydt == np.uint8 else -7
+    kw = dict(strides=(stride, stride), pads=(pad, pad))
+    conv = oracle.qlinear_conv_int(x, 0.02, 101, w, ws, wz, ys, yz, ydt, bias=bias, bias_mode=oracle.BIAS_ONNX_INT32, **kw)
+    r = rand_q(rng, conv.shape, rdt)
+    rs, rz = np.float32(0.037), (131 if rdt == np.uint8 else 5)
+    os_, oz = np.float32(0.061), (99 if odt == np.uint8 else -20)
+    plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), **kw)
+    xd = g.to_channels_last(g.dev(x))
+    n, oc, oh, ow = conv.shape
+    pitch = (oc + 15) // 16 * 16
+    r_padded = torch.zeros((n, oh, ow, pitch), dtype=g.dev(r).dtype, device="cuda")[..., :oc].permute(0, 3, 1, 2)
+    r_padded.copy_(g.dev(r))
+    for relu in (False, True):
+        want = _residual_sum(oracle, conv, ys, yz, r, rs, rz, relu, os_, oz, odt)
+        assert want.min() < want.max()
+        for rd in (g.to_channels_last(g.dev(r)), r_padded):
+            got = plan.run_add(xd, 0.02, 101, ys, yz, rd, rs, rz, os_, oz, relu, zero_point_dtype=TDT[ydt],
+                               flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(rd, dtype=TDT[odt]))
+            np.testing.assert_array_equal(g.host(got), want)
+    # operands that are not channels-last are refused, not converted
+    with pytest.raises(g.capi.ChxHipError) as e:
+        plan.run_add(xd, 0.02, 101, ys, yz, g.dev(r), rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt],
+                     flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros(conv.shape, dtype=TDT[odt], device="cuda"))
+    assert e.value.code == g.capi.EUNSUPPORTED
+    plan.close()

@@ -17,19 +17,26 @@ def g():
 
 def check_model(g, oracle, model, threads=16):
     wl = g.pkg.workloads
-    runner = wl.DeviceRunner(model, g.pkg)
-    dev = runner.run(torch.from_numpy(model["input"]).cuda())
-    torch.cuda.synchronize()
     oracle.set_threads(threads)
     try:
         ref = wl.run_reference(model, oracle, model["input"])
     finally:
         oracle.set_threads(1)
-    for ins in model["program"]:
-        name = ins[1]
-        got = dev[name].cpu().numpy()
-        np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s" % (name, ins[0]))
-    runner.close()
+    # every op a kernel of its own, then with the residual sums inside the convolutions before them
+    # (those convolutions' own outputs are then not materialised)
+    for fuse in (False, True):
+        runner = wl.DeviceRunner(model, g.pkg, fuse_residual=fuse)
+        dev = runner.run(torch.from_numpy(model["input"]).cuda())
+        torch.cuda.synchronize()
+        assert bool(runner.fused_into) == (fuse and any(i[0] in ("Add", "AddRelu") for i in model["program"]))
+        for ins in model["program"]:
+            name = ins[1]
+            if name in runner.fused_into:
+                assert name not in dev
+                continue
+            got = dev[name].cpu().numpy()
+            np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s (fused residual: %s)" % (name, ins[0], fuse))
+        runner.close()
     return ref
 
 
