@@ -130,6 +130,67 @@ __global__ __launch_bounds__(kThreads) void average_pool_kernel(AvgArgs a) {
             (uint8_t)quantize_value<kRne>(mean, a.q);
 }
 
+// Channels-last operands, four channels per lane: one dword load per tap instead of four byte
+// loads, taps of a window row fetched together.  The sum runs over (kh, kw) in the same order as
+// above, per channel, so the result is the same bytes.
+template <bool kRne>
+__global__ __launch_bounds__(kThreads) void average_pool_cl4_kernel(AvgArgs a) {
+    const PoolArgs& p = a.p;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int C4 = p.C >> 2;
+    if (idx >= (p.total >> 2)) return;
+    const int c = (int)(idx % C4) * 4;
+    int64_t r = idx / C4;
+    const int ow = (int)(r % p.OW);
+    r /= p.OW;
+    const int oh = (int)(r % p.OH);
+    const int n = (int)(r / p.OH);
+    const uint32_t flip = p.is_signed ? 0x80808080u : 0u;   // int8 code = (byte ^ 0x80) - 128
+    const float zpf = a.x_zpf + (p.is_signed ? 128.f : 0.f);
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    int32_t cnt = 0;
+    const char* xn = p.x + n * p.xs[0] + c;
+    const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
+    // taps in (kh, kw) order, sixteen loads in flight at a time
+    const int taps = p.kh * p.kw;
+    int i = 0, j = 0;
+    for (int t0 = 0; t0 < taps; t0 += 16) {
+        uint32_t v[16];
+        uint32_t valid = 0;
+        int ii = i, jj = j;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int ih = ih0 + ii, iw = iw0 + jj;
+            // every load goes out, from a clamped address when the tap does not count: a branch around
+            // it would make the compiler wait for each load before the next
+            const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
+            v[t] = *reinterpret_cast<const uint32_t*>(xn + ihc * p.xs[2] + iwc * p.xs[3]) ^ flip;
+            valid |= (t0 + t < taps && ih == ihc && iw == iwc) ? 1u << t : 0u;
+            if (++jj == p.kw) {
+                jj = 0;
+                ++ii;
+            }
+        }
+        i = ii;
+        j = jj;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const bool on = (valid >> t) & 1u;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float term = ((float)((v[t] >> (8 * e)) & 0xffu) - zpf) * a.x_scale;
+                sum[e] = on ? sum[e] + term : sum[e];
+            }
+            cnt += on ? 1 : 0;
+        }
+    }
+    if (a.count_include_pad) cnt = p.kh * p.kw;
+    int32_t code[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) code[e] = quantize_value<kRne>(sum[e] / (float)cnt, a.q);
+    *reinterpret_cast<uint32_t*>(p.y + n * p.ys[0] + oh * p.ys[2] + ow * p.ys[3] + c) = pack4(code[0], code[1], code[2], code[3]);
+}
+
 int fill_pool_args(
         const chx_hip_tensor* x, chx_hip_tensor* y, int kh, int kw, int sh, int sw, int ph0, int pw0, int ph1, int pw1,
         int cover_all, const char* op, PoolArgs* a) {
@@ -205,6 +266,18 @@ extern "C" int chx_hip_average_pool_q8(
     a.count_include_pad = count_include_pad;
     a.q = make_quant_params(y_scale, y_zero_point, i8);
     hipStream_t s = as_stream(stream);
+    const bool cl4 = x->strides[1] == 1 && y->strides[1] == 1 && a.p.C % 4 == 0 && aligned(x->data, 4) && aligned(y->data, 4) &&
+                     x->strides[0] % 4 == 0 && x->strides[2] % 4 == 0 && x->strides[3] % 4 == 0 && y->strides[0] % 4 == 0 &&
+                     y->strides[2] % 4 == 0 && y->strides[3] % 4 == 0;
+    if (cl4) {
+        // small work-groups: a global pool has few outputs, and they should reach every compute unit
+        const unsigned blocks4 = (unsigned)((a.p.total / 4 + 63) / 64);
+        if (flags & CHX_HIP_ROUND_ONNX_RNE)
+            average_pool_cl4_kernel<true><<<blocks4, 64, 0, s>>>(a);
+        else
+            average_pool_cl4_kernel<false><<<blocks4, 64, 0, s>>>(a);
+        return launch_check("average_pool_cl4_kernel");
+    }
     const unsigned blocks = (unsigned)((a.p.total + kThreads - 1) / kThreads);
     if (flags & CHX_HIP_ROUND_ONNX_RNE)
         average_pool_kernel<true><<<blocks, kThreads, 0, s>>>(a);

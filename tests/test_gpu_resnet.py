@@ -61,6 +61,30 @@ def test_pooling_ops(g, oracle):
     np.testing.assert_array_equal(oracle.quantize_linear(pooled, 0.05, 30), oracle.max_pool_q8(x, (3, 3), (2, 2)))
 
 
+@pytest.mark.parametrize("xdt", [np.uint8, np.int8])
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, kernel, stride, pad, count_include_pad
+    (2, 32, 7, 7, 7, 1, 0, False), (1, 20, 9, 11, 3, 2, 1, False), (1, 8, 6, 6, 3, 1, 1, True), (1, 12, 10, 13, 9, 1, 0, False),
+    (2, 6, 5, 5, 2, 2, 0, False)])
+def test_average_pool_layouts(g, oracle, case, xdt):
+    """AveragePool between DequantizeLinear and QuantizeLinear: the four-channel channels-last
+    kernel (also windows wider than its eight-tap groups, padding, both count modes, int8) and the
+    generic one (NCHW operands, a channel count that is not a multiple of four) give the oracle's bytes."""
+    N, C, H, W, k, s, pad, cip = case
+    rng = np.random.default_rng(43)
+    lo, hi = (0, 256) if xdt == np.uint8 else (-128, 128)
+    x = rng.integers(lo, hi, size=(N, C, H, W)).astype(xdt)
+    xz = 77 if xdt == np.uint8 else -12
+    for ydt, yz, flags, rm in ((np.uint8, 9, 0, oracle.ROUND_REFERENCE), (np.int8, -30, g.capi.ROUND_ONNX_RNE, oracle.ROUND_ONNX_RNE)):
+        want = oracle.average_pool_q8(x, 0.05, xz, (k, k), (s, s), (pad, pad), 0.031, yz, ydt, count_include_pad=cip, round_mode=rm)
+        assert want.min() < want.max()
+        zdt = torch.uint8 if ydt == np.uint8 else torch.int8
+        for xd in (g.to_channels_last(g.dev(x)), g.dev(x)):
+            got = g.ops.AveragePoolQ8(xd, 0.05, xz, (k, k), (s, s), (pad, pad), 0.031, yz, count_include_pad=cip,
+                                      zero_point_dtype=zdt, flags=flags)
+            np.testing.assert_array_equal(g.host(got), want)
+
+
 def test_small_resnet_every_value(g, oracle):
     model = g.pkg.workloads.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
     ref = check_model(g, oracle, model)
