@@ -29,7 +29,7 @@ EXPORTS = [
     "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
-    "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source",
+    "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_match_residual_add",
     "chx_hip_max_pool_q8", "chx_hip_average_pool_q8",
 ]
 
@@ -143,3 +143,20 @@ def elementwise_source(code, fusion_id, in_descs, out_descs, compile=False):
     buf = ctypes.create_string_buffer(needed.value)
     check(lib().chx_hip_elementwise_source(*args, buf, ctypes.c_size_t(needed.value), None))
     return buf.value.decode()
+
+
+class ResidualGroup(ctypes.Structure):
+    _fields_ = [("in_scale", ctypes.c_float * 2), ("in_zero_point", ctypes.c_int32 * 2), ("in_dtype", ctypes.c_int32 * 2),
+                ("relu", ctypes.c_int32), ("out_scale", ctypes.c_float), ("out_zero_point", ctypes.c_int32),
+                ("out_dtype", ctypes.c_int32)]
+
+
+def match_residual_add(code):
+    """chx_hip_elementwise_match_residual_add: None, or a dict of the group's constants."""
+    matches = ctypes.c_int32()
+    grp = ResidualGroup()
+    check(lib().chx_hip_elementwise_match_residual_add(code.encode(), ctypes.byref(matches), ctypes.byref(grp)))
+    if not matches.value:
+        return None
+    return dict(in_scale=list(grp.in_scale), in_zero_point=list(grp.in_zero_point), in_dtype=list(grp.in_dtype), relu=bool(grp.relu),
+                out_scale=grp.out_scale, out_zero_point=grp.out_zero_point, out_dtype=grp.out_dtype)

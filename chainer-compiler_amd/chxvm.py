@@ -25,7 +25,7 @@ RUNTIME_EXPORTS = [
     "chxvm_last_error", "chxvm_num_ops", "chxvm_op_name", "chxvm_op_number", "chxvm_proto_roundtrip", "chxvm_free",
     "chxvm_program_create", "chxvm_program_destroy", "chxvm_program_num_instructions", "chxvm_program_num_inputs",
     "chxvm_program_input_name", "chxvm_program_run", "chxvm_outputs_count", "chxvm_outputs_name", "chxvm_outputs_get",
-    "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name", "chxvm_set_option",
+    "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name", "chxvm_set_option", "chxvm_counter",
 ]
 
 # ChxVMValueProto.Type
@@ -78,6 +78,8 @@ def runtime():
         rt.chxvm_backend_config_has.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_char_p,
                                                 ctypes.POINTER(ctypes.c_int32)]
         rt.chxvm_set_option.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
+        rt.chxvm_counter.argtypes = [ctypes.c_char_p]
+        rt.chxvm_counter.restype = ctypes.c_int64
         rt.chxvm_backend_config_name.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
         _rt = rt
     return _rt
@@ -374,8 +376,14 @@ class Program:
 
 
 def set_option(name, value):
-    """Runtime switches; "qlinearconv_bias" = "reference" (default) | "onnx_int32"."""
+    """Runtime switches: "qlinearconv_bias" = "reference" (default) | "onnx_int32";
+    "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards)."""
     _check(runtime().chxvm_set_option(name.encode(), value.encode()))
+
+
+def counter(name):
+    """Process-wide event counts of the runtime, e.g. "qlinearconv_residual_fusions"."""
+    return runtime().chxvm_counter(name.encode())
 
 
 def proto_roundtrip(serialized):

@@ -815,3 +815,54 @@ extern "C" int chx_hip_elementwise(
     }
     return CHX_HIP_OK;
 }
+
+extern "C" int chx_hip_elementwise_match_residual_add(const char* code, int32_t* matches, chx_hip_residual_group* group) {
+    using namespace chx;
+    CHX_REQUIRE(matches != nullptr && group != nullptr, "match_residual_add: null output");
+    *matches = 0;
+    memset(group, 0, sizeof(*group));
+    Program prog;
+    CHX_PROPAGATE(parse_program(code, &prog));
+    if (prog.inputs.size() != 2 || prog.outputs.size() != 1) return CHX_HIP_OK;
+    if (!is_q8(prog.inputs[0].dtype) || !is_q8(prog.inputs[1].dtype) || !is_q8(prog.outputs[0].dtype)) return CHX_HIP_OK;
+    if (prog.stmts.size() != 4 && prog.stmts.size() != 5) return CHX_HIP_OK;
+    const bool relu = prog.stmts.size() == 5;
+    std::string dq_name[2];
+    for (int i = 0; i < 2; ++i) {
+        // one DequantizeLinear per input, among the first two statements
+        const Stmt* found = nullptr;
+        for (int j = 0; j < 2; ++j)
+            if (prog.stmts[j].op == "DequantizeLinear" && prog.stmts[j].args.size() == 3 && prog.stmts[j].args[0] == prog.inputs[i].name)
+                found = found ? nullptr : &prog.stmts[j];
+        if (!found || prog.inputs[0].name == prog.inputs[1].name) return CHX_HIP_OK;
+        CHX_PROPAGATE(float_value(found->args[1], &group->in_scale[i]));
+        char* end = nullptr;
+        const long zp = strtol(found->args[2].c_str(), &end, 10);
+        if (!end || *end != 0) return CHX_HIP_OK;
+        group->in_zero_point[i] = (int32_t)zp;
+        group->in_dtype[i] = prog.inputs[i].dtype;
+        dq_name[i] = found->out;
+    }
+    const Stmt& add = prog.stmts[2];
+    if (add.op != "Add" || add.args.size() != 2) return CHX_HIP_OK;
+    if (!((add.args[0] == dq_name[0] && add.args[1] == dq_name[1]) || (add.args[0] == dq_name[1] && add.args[1] == dq_name[0])))
+        return CHX_HIP_OK;
+    std::string last = add.out;
+    if (relu) {
+        const Stmt& r = prog.stmts[3];
+        if (r.op != "Relu" || r.args.size() != 1 || r.args[0] != last) return CHX_HIP_OK;
+        last = r.out;
+    }
+    const Stmt& q = prog.stmts.back();
+    if (q.op != "QuantizeLinear" || q.args.size() != 4 || q.args[0] != last || q.out != prog.outputs[0].name) return CHX_HIP_OK;
+    CHX_PROPAGATE(float_value(q.args[1], &group->out_scale));
+    char* end = nullptr;
+    const long zp = strtol(q.args[2].c_str(), &end, 10);
+    int32_t qdt = 0;
+    if (!end || *end != 0 || !parse_dtype(q.args[3], &qdt) || qdt != prog.outputs[0].dtype) return CHX_HIP_OK;
+    group->out_zero_point = (int32_t)zp;
+    group->out_dtype = qdt;
+    group->relu = relu ? 1 : 0;
+    *matches = 1;
+    return CHX_HIP_OK;
+}

@@ -107,6 +107,78 @@ private:
     int flag_;
 };
 
+// A QLinearConv whose result is read only by a residual-sum FusionGroup (and that group): the
+// convolution gets the chance to compute the group inside its kernel.  When it does, the group's
+// result is stored in the group's output slot now and the group instruction later does nothing;
+// when it does not (other quantization constants at run time, operands the kernel does not take),
+// both instructions run as they are.
+bool g_fuse_residual = true;
+
+struct ResidualFusionState {
+    bool fused = false;  // of the current run
+};
+
+class QLinearConvWithResidualOp : public ChxVMOp {
+public:
+    QLinearConvWithResidualOp(const ChxVMInstructionProto& conv, const ChxVMInstructionProto& group, const chx_hip_residual_group& g,
+                              int conv_operand, std::shared_ptr<ResidualFusionState> state)
+        : ChxVMOp(conv), conv_(MakeChxVMOp(conv)), g_(g), k_(conv_operand), conv_out_(conv.outputs[0]),
+          other_(group.inputs[0].array_list[1 - conv_operand]), group_out_(group.outputs[0]), state_(std::move(state)) {
+    }
+    void InitImpl() override {
+        conv_->InitImpl();
+    }
+    void Run(ChxVMState* st) override {
+        QLinearConvResidualRequest req;
+        ChxVMVar* other = st->GetVar(other_);
+        if (!other->IsNull()) req.r = other->GetArray();
+        auto dt = [](int32_t d) { return static_cast<chainerx::Dtype>(d); };
+        req.y_scale = g_.in_scale[k_]; req.y_zero_point = g_.in_zero_point[k_]; req.y_dtype = dt(g_.in_dtype[k_]);
+        req.r_scale = g_.in_scale[1 - k_]; req.r_zero_point = g_.in_zero_point[1 - k_];
+        req.out_scale = g_.out_scale; req.out_zero_point = g_.out_zero_point; req.out_dtype = dt(g_.out_dtype);
+        req.relu = g_.relu != 0;
+        const bool r_fits = !req.r.IsNullHandle() && req.r.dtype() == dt(g_.in_dtype[1 - k_]);
+        SetQLinearConvResidualRequest(r_fits ? &req : nullptr);
+        try {
+            conv_->Run(st);
+        } catch (...) {
+            SetQLinearConvResidualRequest(nullptr);
+            throw;
+        }
+        SetQLinearConvResidualRequest(nullptr);
+        state_->fused = req.done;
+        if (req.done) {
+            if (st->trace_level()) std::cerr << "  (residual sum $" << group_out_ << " computed by the convolution)" << std::endl;
+            st->FreeVar(conv_out_);  // holds a null array: the convolution's own result was never written
+            st->SetArray(group_out_, req.out);
+        }
+    }
+
+private:
+    std::unique_ptr<ChxVMOp> conv_;
+    chx_hip_residual_group g_;
+    int k_, conv_out_, other_, group_out_;
+    std::shared_ptr<ResidualFusionState> state_;
+};
+
+class ResidualGroupOp : public ChxVMOp {
+public:
+    ResidualGroupOp(const ChxVMInstructionProto& group, std::shared_ptr<ResidualFusionState> state)
+        : ChxVMOp(group), group_(MakeChxVMOp(group)), state_(std::move(state)) {
+    }
+    void InitImpl() override {
+        group_->InitImpl();
+    }
+    void Run(ChxVMState* st) override {
+        if (state_->fused) return;
+        group_->Run(st);
+    }
+
+private:
+    std::unique_ptr<ChxVMOp> group_;
+    std::shared_ptr<ResidualFusionState> state_;
+};
+
 class NopOp : public ChxVMOp {
 public:
     explicit NopOp(const ChxVMInstructionProto& inst) : ChxVMOp(inst) {
@@ -189,6 +261,40 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         fused_inputs[q] = std::make_pair(da, db);
         role[m] = role[da] = role[db] = 1;
     }
+    // Residual sums: an ElementWiseNvrtc group of the form Q(act(DQ(a) + DQ(b))) one of whose operands
+    // is the result of a QLinearConv that nobody else reads, with the other operand produced
+    // before that convolution.  role 4 = the convolution, role 5 = the group.
+    const int kQLinearConv = OpNumber("QLinearConv"), kElementWise = OpNumber("ElementWiseNvrtc");
+    std::vector<int> partner(n, -1), conv_operand(n, 0);
+    std::vector<chx_hip_residual_group> groups(n);
+    for (int e = 0; e < n && g_fuse_residual; ++e) {
+        const ChxVMInstructionProto& ei = program.instructions[e];
+        if (ei.op != kElementWise || role[e] != 0 || ei.inputs.size() != 4 || ei.inputs[0].array_list.size() != 2 ||
+            ei.outputs.size() != 1)
+            continue;
+        int32_t matches = 0;
+        chx_hip_residual_group g;
+        if (chx_hip_elementwise_match_residual_add(ei.inputs[2].s.c_str(), &matches, &g) != 0 || !matches) continue;
+        for (int k = 1; k >= 0; --k) {
+            const int slot = ei.inputs[0].array_list[k], other = ei.inputs[0].array_list[1 - k];
+            if (slot < 0 || other < 0 || slot == other) continue;
+            const int c = producer[slot];
+            if (c < 0 || program.instructions[c].op != kQLinearConv || role[c] != 0 || !single_use(slot)) continue;
+            if (producer[other] >= c) continue;  // the other operand must exist when the convolution runs
+            bool other_alive = true;             // ... and still exist: no Free of it before the group
+            for (int i = c; i < e; ++i)
+                if (program.instructions[i].op == kFree && program.instructions[i].inputs[0].array == other) other_alive = false;
+            if (!other_alive) continue;
+            role[c] = 4;
+            role[e] = 5;
+            partner[c] = e;
+            partner[e] = c;
+            conv_operand[c] = k;
+            groups[c] = g;
+            break;
+        }
+    }
+    std::vector<std::shared_ptr<ResidualFusionState>> fusion_state(n);
     std::vector<bool> dead(num_variables_ > 0 ? num_variables_ : 1, false);
     for (int i = 0; i < n; ++i)
         if (role[i] == 1)
@@ -202,6 +308,12 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         } else if (role[i] == 3) {
             const ChxVMInstructionProto& pool = program.instructions[fused_inputs[i].second];
             program_.emplace_back(new FusedQuantizedPoolOp(inst, pool, program.instructions[fused_inputs[i].first], pool.op == kMaxPool));
+        } else if (role[i] == 4) {
+            fusion_state[i] = std::make_shared<ResidualFusionState>();
+            program_.emplace_back(new QLinearConvWithResidualOp(inst, program.instructions[partner[i]], groups[i], conv_operand[i],
+                                                                fusion_state[i]));
+        } else if (role[i] == 5) {
+            program_.emplace_back(new ResidualGroupOp(inst, fusion_state[partner[i]]));
         } else if (role[i] == 2) {
             program_.emplace_back(new FusedQLinearMatMulOp(inst, program.instructions[fused_inputs[i].first],
                                                            program.instructions[fused_inputs[i].second]));
@@ -213,6 +325,10 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
 }
 
 ChxVM::~ChxVM() = default;
+
+void SetFuseResidual(bool on) {
+    g_fuse_residual = on;
+}
 
 InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
     for (const std::string& name : input_names_)

@@ -15,6 +15,25 @@ namespace runtime {
 // operator's int32 bias added to the accumulator.
 void SetQLinearConvOnnxInt32Bias(bool on);
 
+// A residual sum that the next QLinearConvOp::RunImpl on this thread may compute inside its
+// kernel: out = QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r))) for its own result
+// y.  The op takes the request when y's quantization is the one the group dequantizes with and the
+// kernel accepts the operands; it then sets `done`, leaves the group's result in `out` and returns
+// a null array for y.  Otherwise it runs as usual and the caller runs the group afterwards.
+struct QLinearConvResidualRequest {
+    chainerx::Array r;
+    float y_scale = 0, r_scale = 0, out_scale = 0;
+    int32_t y_zero_point = 0, r_zero_point = 0, out_zero_point = 0;
+    chainerx::Dtype y_dtype = chainerx::Dtype::kUInt8, out_dtype = chainerx::Dtype::kUInt8;
+    bool relu = false;
+    chainerx::Array out;
+    bool done = false;
+};
+void SetQLinearConvResidualRequest(QLinearConvResidualRequest* request);  // null clears it
+int64_t QLinearConvResidualFusions();  // requests taken so far, process-wide
+// Whether programs loaded from now on pair such convolutions and groups at all (default: yes).
+void SetFuseResidual(bool on);
+
 class ChxVM {
 public:
     explicit ChxVM(const ChxVMProgramProto& program);

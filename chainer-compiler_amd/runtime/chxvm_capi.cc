@@ -154,10 +154,19 @@ int32_t chxvm_set_option(const char* name, const char* value) {
         if (n == "qlinearconv_bias") {
             CHECK(v == "reference" || v == "onnx_int32") << "qlinearconv_bias is 'reference' or 'onnx_int32', got " << v;
             SetQLinearConvOnnxInt32Bias(v == "onnx_int32");
+        } else if (n == "fuse_residual") {
+            CHECK(v == "on" || v == "off") << "fuse_residual is 'on' or 'off', got " << v;
+            SetFuseResidual(v == "on");
         } else {
             CHECK(false) << "unknown option " << n;
         }
     });
+}
+
+int64_t chxvm_counter(const char* name) {
+    const std::string n = name ? name : "";
+    if (n == "qlinearconv_residual_fusions") return QLinearConvResidualFusions();
+    return -1;
 }
 
 int32_t chxvm_backend_config_has(const char* config, int32_t is_json, const char* section, const char* key, int32_t* out) {

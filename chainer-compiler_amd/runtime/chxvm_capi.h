@@ -51,8 +51,13 @@ const char* chxvm_outputs_name(const chxvm_outputs* outputs, int32_t i);
 int32_t chxvm_outputs_get(const chxvm_outputs* outputs, int32_t i, chx_hip_tensor* out);
 void chxvm_outputs_destroy(chxvm_outputs* outputs);
 
-/* name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32". */
+/* name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32";
+ * name "fuse_residual": value "on" (default) or "off": whether a QLinearConv read only by a
+ * residual-sum group computes that group inside its kernel (decided when a program is loaded). */
 int32_t chxvm_set_option(const char* name, const char* value);
+/* Process-wide event counts.  name "qlinearconv_residual_fusions": runs of a QLinearConv that
+ * computed the residual-sum group behind it inside its kernel.  Unknown names give -1. */
+int64_t chxvm_counter(const char* name);
 
 /* BackendConfig queries.  `config` is a built-in name ("chxvm", "chxvm_test", "hip") or, with
  * is_json != 0, a JSON document.  section: "simplify_preproc", "simplify", "merge",

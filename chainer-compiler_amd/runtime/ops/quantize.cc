@@ -3,6 +3,9 @@
 // output allocation and one call into the C ABI (include/chx_hip.h).
 #include "../chainerx_util.h"
 #include "../gen/gen_chxvm_ops.h"
+#include "../chxvm.h"
+
+#include <atomic>
 
 namespace chainer_compiler {
 namespace runtime {
@@ -10,6 +13,8 @@ namespace runtime {
 namespace {
 
 bool g_onnx_int32_bias = false;
+thread_local QLinearConvResidualRequest* g_residual_request = nullptr;
+std::atomic<int64_t> g_residual_fusions{0};
 
 StrictScalar DefaultZeroPoint() {
     // an absent zero point is uint8 0 (runtime/ops/quantize.cc:50-51,57-58)
@@ -33,6 +38,14 @@ chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& sha
 // scale x_scale * w_scale[oc].  This switch selects which of the two the op computes.
 void SetQLinearConvOnnxInt32Bias(bool on) {
     g_onnx_int32_bias = on;
+}
+
+void SetQLinearConvResidualRequest(QLinearConvResidualRequest* request) {
+    g_residual_request = request;
+}
+
+int64_t QLinearConvResidualFusions() {
+    return g_residual_fusions.load();
 }
 
 chainerx::Array QuantizeLinearOp::RunImpl(
@@ -103,14 +116,34 @@ chainerx::Array QLinearConvOp::RunImpl(
         impl_->params = p;
         impl_->w_data = q_w.raw_data();
     }
+    const chainerx::Shape y_shape = ConvOutputShape(q_x, q_w, p);
+    const uint32_t flags = CHX_HIP_ROUND_REFERENCE | (g_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
+    if (QLinearConvResidualRequest* req = g_residual_request) {
+        const bool same_quantization = static_cast<float>(y_scale) == req->y_scale &&
+                                       static_cast<int64_t>(y_zero_point) == req->y_zero_point && y_zero_point.dtype() == req->y_dtype;
+        if (same_quantization && !req->r.IsNullHandle() && req->r.shape() == y_shape) {
+            chainerx::Array out = chainerx::EmptyChannelsLastPadded(y_shape, req->out_dtype);
+            chx_hip_tensor xt = q_x.hip(), rt = req->r.hip(), ot = out.hip();
+            const int rc = chx_hip_qconv_plan_run_add(
+                    impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
+                    req->y_scale, req->y_zero_point, static_cast<int32_t>(req->y_dtype), flags, &rt, req->r_scale, req->r_zero_point,
+                    req->out_scale, req->out_zero_point, req->relu ? 1 : 0, &ot, nullptr);
+            if (rc == CHX_HIP_OK) {
+                req->out = out;
+                req->done = true;
+                ++g_residual_fusions;
+                return chainerx::Array();
+            }
+            CHECK_EQ(CHX_HIP_EUNSUPPORTED, rc) << chx_hip_last_error();  // unsupported: run the ops one by one
+        }
+    }
     // 8-bit activations leave a convolution channels-last, whatever layout came in
-    chainerx::Array y = chainerx::EmptyChannelsLastPadded(ConvOutputShape(q_x, q_w, p), y_zero_point.dtype());
+    chainerx::Array y = chainerx::EmptyChannelsLastPadded(y_shape, y_zero_point.dtype());
     chx_hip_tensor xt = q_x.hip(), yt = y.hip();
     // the reference hands the raw bias to the fp32 convolution (quantize.cc:93)
     CHXVM_HIP_CALL(chx_hip_qconv_plan_run(
             impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
-            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)),
-            CHX_HIP_ROUND_REFERENCE | (g_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT), &yt, nullptr));
+            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, nullptr));
     return y;
 }
 

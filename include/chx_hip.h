@@ -249,6 +249,24 @@ int chx_hip_elementwise_source(
         chx_hip_tensor* const* outputs, int32_t n_outputs, int32_t compile, char* buffer, size_t buffer_size,
         size_t* needed);
 
+/* Says whether a fusion program (the `code` of an ElementWiseNvrtc instruction, emitted per
+ * FusionGroup by compiler/chxvm/emitter.cc:621-729) is exactly the residual sum of a quantized
+ * network,  out = QuantizeLinear(act(DequantizeLinear(in0) + DequantizeLinear(in1)))  with
+ * act = Relu or nothing, and if so with which constants: the form chx_hip_qconv_plan_run_add
+ * computes inside the convolution that produces one of the operands.  Host-only (no GPU work).
+ * A program that does not parse is an error; one that parses but has another form sets
+ * *matches = 0. */
+typedef struct chx_hip_residual_group {
+    float in_scale[2];          /* DequantizeLinear constants of input 0 and input 1 */
+    int32_t in_zero_point[2];
+    int32_t in_dtype[2];
+    int32_t relu;
+    float out_scale;
+    int32_t out_zero_point;
+    int32_t out_dtype;
+} chx_hip_residual_group;
+int chx_hip_elementwise_match_residual_add(const char* code, int32_t* matches, chx_hip_residual_group* group);
+
 #ifdef __cplusplus
 }
 #endif

@@ -348,6 +348,9 @@ def test_runtime_options(chxvm):
         chxvm.set_option("qlinearconv_bias", "int64")
     with pytest.raises(chxvm.ChxVMError, match="unknown option"):
         chxvm.set_option("no_such_switch", "1")
+    chxvm.set_option("fuse_residual", "off")
+    chxvm.set_option("fuse_residual", "on")
+    assert chxvm.counter("qlinearconv_residual_fusions") >= 0 and chxvm.counter("no_such_counter") == -1
 
 
 def test_whole_network_as_one_program(chxvm):

@@ -90,3 +90,35 @@ def test_operand_errors():
     with pytest.raises(capi.ChxHipError, match="is uint8, program says float32"):
         capi.elementwise_source(CHAIN, 0, [fake((4, 5), dtype=capi.UINT8), fake(()), fake(()), fake((4, 5))],
                                 [fake((4, 5))])
+
+
+def test_residual_sum_groups_are_recognised():
+    """The one group shape a convolution can absorb: Q(act(DQ(in0) + DQ(in1))), operands of the Add in
+    either order, Relu optional; anything else is left to the element-wise kernel."""
+    import numpy as np
+    u8, i8 = torch.uint8, torch.int8
+
+    def group(relu=True, swap=False, tail=(), out_dtype="uint8", rne=False, second="b"):
+        st = [("fa", "DequantizeLinear", "a", 0.05, 128), ("fb", "DequantizeLinear", second, "0x3ca3d70a", -3)]
+        st.append(("s", "Add", "fb", "fa") if swap else ("s", "Add", "fa", "fb"))
+        last = "s"
+        if relu:
+            st.append(("r", "Relu", "s"))
+            last = "r"
+        st.extend(tail)
+        q = ("q", "QuantizeLinear", tail[-1][0] if tail else last, 0.06, 7, out_dtype) + (("rne",) if rne else ())
+        return ops.fusion_program([("a", u8), ("b", i8)], st + [q], [("q", u8 if out_dtype == "uint8" else i8)])
+    for relu in (True, False):
+        for swap in (True, False):
+            m = capi.match_residual_add(group(relu, swap))
+            assert m is not None and m["relu"] == relu
+            assert m["in_scale"] == [np.float32(0.05), np.float32(0.02)] and m["in_zero_point"] == [128, -3]
+            assert m["in_dtype"] == [capi.UINT8, capi.INT8]
+            assert (m["out_scale"], m["out_zero_point"], m["out_dtype"]) == (np.float32(0.06), 7, capi.UINT8)
+    assert capi.match_residual_add(group(out_dtype="int8"))["out_dtype"] == capi.INT8
+    assert capi.match_residual_add(group(rne=True)) is None                       # another rounding
+    assert capi.match_residual_add(group(tail=(("t", "Tanh", "r"),))) is None     # another activation
+    assert capi.match_residual_add(group(second="a")) is None                     # the same operand twice
+    assert capi.match_residual_add(CHAIN) is None                                 # float chain
+    with pytest.raises(capi.ChxHipError):
+        capi.match_residual_add("not a program")

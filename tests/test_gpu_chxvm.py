@@ -202,8 +202,9 @@ def test_errors_name_the_instruction(g, vm):
         vm.Program(b.serialize()).run({"x": g.dev(np.zeros(4, np.float32))})
 
 
-def _run_network_through_vm(g, vm, oracle, model, keep):
+def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None):
     wl = g.pkg.workloads
+    before = vm.counter("qlinearconv_residual_fusions")
     serialized = wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize()
     assert vm.proto_roundtrip(serialized) == serialized
     vm.set_option("qlinearconv_bias", "onnx_int32")
@@ -221,6 +222,8 @@ def _run_network_through_vm(g, vm, oracle, model, keep):
     assert sorted(got) == sorted(keep)
     for name in keep:
         np.testing.assert_array_equal(got[name], ref[name], err_msg="value %s" % name)
+    if fused_residuals is not None:
+        assert vm.counter("qlinearconv_residual_fusions") - before == fused_residuals
 
 
 def test_small_resnet_as_one_program(g, vm, oracle):
@@ -228,15 +231,65 @@ def test_small_resnet_as_one_program(g, vm, oracle):
     operands, DequantizeLinear -> MaxPool / AveragePool -> QuantizeLinear fused at load,
     FusionGroups for the residual sums, Free after the last reader.  Every value, then only the logits."""
     model = g.pkg.workloads.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
-    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]])
-    _run_network_through_vm(g, vm, oracle, model, ["logits"])
+    # every value is a program output: nothing may be absorbed into another instruction
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0)
+    # only the logits: each of the five residual sums is computed by the convolution before it
+    blocks = sum(1 for ins in model["program"] if ins[0] == "AddRelu")
+    assert blocks == 5
+    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks)
+    # the block outputs too: the sums are still absorbed (their convolutions' results are not outputs)
+    keep = ["logits"] + [ins[1] for ins in model["program"] if ins[0] == "AddRelu"]
+    _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=blocks)
+    vm.set_option("fuse_residual", "off")
+    try:
+        _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=0)
+    finally:
+        vm.set_option("fuse_residual", "on")
 
 
 def test_small_mobilenetv2_as_one_program(g, vm, oracle):
     """Depthwise convolutions and 24-channel activations (pixel pitch padded to 16 bytes) in the VM."""
     blocks = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 1, 2))
     model = g.pkg.workloads.build_mobilenetv2(batch=2, image=64, seed=7, blocks=blocks, stem=32, head=128, classes=10)
-    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]])
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0)
+    adds = [ins[1] for ins in model["program"] if ins[0] == "Add"]
+    assert len(adds) >= 1
+    _run_network_through_vm(g, vm, oracle, model, ["logits"] + adds, fused_residuals=len(adds))
+
+
+def test_residual_group_with_other_constants_runs_unfused(g, vm, oracle):
+    """A group whose DequantizeLinear constants are not the convolution's output quantization is not
+    the convolution's to compute: both instructions run as they are, and the result is the oracle's."""
+    rng = np.random.default_rng(77)
+    x = rand_q(rng, (1, 16, 6, 6), np.uint8)
+    w = rng.integers(-127, 128, size=(32, 16, 1, 1)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=32).astype(np.float32)
+    r = rand_q(rng, (1, 32, 6, 6), np.uint8)
+    u8 = torch.uint8
+
+    def scale_bits(v):
+        return "0x%08x" % np.float32(v).view(np.uint32)
+    for group_scale, expect in ((0.25, 1), (0.26, 0)):
+        code = g.ops.fusion_program(
+            [("a", u8), ("b", u8)],
+            [("fa", "DequantizeLinear", "a", scale_bits(group_scale), 120), ("fb", "DequantizeLinear", "b", scale_bits(0.1), 3),
+             ("s", "Add", "fb", "fa"), ("q", "QuantizeLinear", "s", scale_bits(0.3), 100, "uint8")], [("q", u8)])
+        b = vm.ProgramBuilder()
+        xs = b.input("x", "uint8", x.shape)
+        rs = b.input("r", "uint8", r.shape)
+        y = b.QLinearConv(xs, b.scalar(0.02, "float32"), b.scalar(128, "uint8"), b.constant(w), b.constant(ws),
+                          b.constant(np.zeros(32, np.int8)), b.scalar(0.25, "float32"), b.scalar(120, "uint8"), None, [1, 1], [0, 0], 1, "")
+        out = b.ElementWiseNvrtc([y, rs], 1, code, 7, num_list_outputs=1)[0]
+        b.Free(y)
+        b.output("out", out)
+        before = vm.counter("qlinearconv_residual_fusions")
+        prog = vm.Program(b.serialize())
+        got = prog.run({"x": g.to_channels_last(g.dev(x)), "r": g.to_channels_last(g.dev(r))})["out"]
+        prog.close()
+        assert vm.counter("qlinearconv_residual_fusions") - before == expect
+        conv = oracle.qlinear_conv_int(x, 0.02, 128, w, ws, np.zeros(32, np.int8), np.float32(0.25), 120, np.uint8)
+        s_ = oracle.binary(oracle.ADD, oracle.dequantize_linear(r, 0.1, 3), oracle.dequantize_linear(conv, group_scale, 120))
+        np.testing.assert_array_equal(got, oracle.quantize_linear(s_, 0.3, 100, np.uint8))
 
 
 def test_unfused_pool_is_refused_at_load(g, vm):
