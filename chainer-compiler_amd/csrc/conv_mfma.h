@@ -57,6 +57,7 @@ struct ConvMfmaArgs {
     float lo_folded;             // lower clamp bound with the fused Relu folded in (fold_relu_floor)
     int32_t tiles_oc, tiles_px;  // filled by the launcher
     uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
+    uint32_t row_unit;           // bit i*KW set for every filter row i (when KH*KW <= 32), filled by the launcher
     ResidualAdd res;             // res.r == nullptr: plain QLinearConv
 };
 

@@ -458,11 +458,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                 // taps (i, jj) inside the image: i in [r_lo, r_hi), jj in [c_lo, c_hi)
                 const int c_lo = min(max(-iw0, 0), a.KW), c_hi = min(max(a.W - iw0, 0), a.KW);
                 const int r_lo = min(max(-ih0, 0), a.KH), r_hi = min(max(a.H - ih0, 0), a.KH);
-                const uint64_t below_hi = c_hi >= 64 ? ~(uint64_t)0 : ((uint64_t)1 << c_hi) - 1;  // a 1x64 filter fills the mask
-                const uint64_t cols = c_hi > c_lo ? below_hi & ~(((uint64_t)1 << c_lo) - 1) : 0;
                 uint64_t mask = 0;
-                for (int i = 0; i < a.KH; ++i)
-                    if (i >= r_lo && i < r_hi) mask |= cols << (i * a.KW);
+                if (a.KH * a.KW <= 32) {
+                    // up to 32 taps (3x3, 5x5): the column bits repeated in every filter row by one
+                    // multiplication with the bits KW apart, then the rows outside the image cut off
+                    const uint32_t cols = c_hi > c_lo ? ((1u << c_hi) - 1u) & ~((1u << c_lo) - 1u) : 0u;
+                    const uint32_t lo_bit = (uint32_t)(r_lo * a.KW), hi_bit = (uint32_t)(r_hi * a.KW);
+                    const uint32_t below_hi = hi_bit >= 32 ? ~0u : (1u << hi_bit) - 1u;
+                    const uint32_t rows = r_hi > r_lo ? below_hi & ~((1u << lo_bit) - 1u) : 0u;
+                    mask = (cols * a.row_unit) & rows;
+                } else {
+                    const uint64_t below_hi = c_hi >= 64 ? ~(uint64_t)0 : ((uint64_t)1 << c_hi) - 1;  // a 1x64 filter fills the mask
+                    const uint64_t cols = c_hi > c_lo ? below_hi & ~(((uint64_t)1 << c_lo) - 1) : 0;
+                    for (int i = 0; i < a.KH; ++i)
+                        if (i >= r_lo && i < r_hi) mask |= cols << (i * a.KW);
+                }
                 tapmask[j] = row_ok ? mask : 0;
             }
         }
@@ -819,6 +829,9 @@ int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_c
     if (a.M == 0 || a.OC == 0) return CHX_HIP_OK;
     magic_divisor((uint32_t)a.OW, &a.ow_mul, &a.ow_shift);
     magic_divisor((uint32_t)a.OH, &a.oh_mul, &a.oh_shift);
+    a.row_unit = 0;
+    if (a.KH * a.KW <= 32)
+        for (int i = 0; i < a.KH; ++i) a.row_unit |= 1u << (i * a.KW);
     if (tile_oc == 128 && tile_px == 128) return a.bk == 128 ? launch_config<2, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
                            : launch_config<2, 2, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
     if (tile_oc == 64 && tile_px == 128) return a.bk == 128 ? launch_config<1, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
