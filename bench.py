@@ -178,7 +178,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                         bytes_per_step=model["depthwise_bytes"], kernel_ms_per_step=conv_ms_per_step)
     else:
         achieved = conv_ops / (conv_ms_per_step * 1e-3) / 1e12
-        roofline = dict(bound="mfma", kernel="conv_mfma_kernel (%d launches per step, summed)" % n_launch,
+        roofline = dict(bound="mfma", kernel="QLinearConv launches of one step, summed (%d: conv_mfma_kernel, the first layer conv_stem_kernel)" % n_launch,
                         achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
                         ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
     if not mobilenet and batch == 64 and args.parts <= 1:

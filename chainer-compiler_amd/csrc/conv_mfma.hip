@@ -311,12 +311,14 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 // Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
 // (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
 // reference's order, one IEEE operation each.
+template <bool kU8>
 __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
     v4i out;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
         const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
         int32_t code[4];
+        float pre[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
@@ -324,9 +326,10 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
             float sum = fa + fb;
             if (p.relu) sum = __builtin_fmaxf(sum, 0.f);
             sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
-            code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
+            if (kU8) pre[e] = quantize_prefloor_u8<false>(sum, p.out, p.inv_out_scale, 0.f);
+            else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
         }
-        out[w] = (int)pack4(code[0], code[1], code[2], code[3]);
+        out[w] = kU8 ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
     }
     return out;
 }
@@ -603,9 +606,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                 }
             return;
         }
-        // requantize: one instance of the element loop per bias mode (the branch is uniform)
-        auto requantize_tile = [&](auto float_bias_tag) {
+        // requantize: one instance of the element loop per bias mode and per conversion path (the
+        // branches are uniform).  kPath 0: any 8-bit type and rounding; 1: uint8 in the reference's
+        // rounding through floor_sat_u8x4/8; 2: the same with a lower bound above 0 (a folded Relu).
+        auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
+            constexpr int kPath = decltype(path_tag)::value;
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -614,25 +620,78 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                     const v4f sc = *reinterpret_cast<const v4f*>(&s_scale[ocl]);
                     v4f fb = {0.f, 0.f, 0.f, 0.f};
                     if (kFloatBias) fb = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
+                    if (kPath == 0) {
 #pragma unroll
-                    for (int j = 0; j < FN; ++j) {
-                        const int pxl = wn * 32 * FN + j * 32 + (lane & 31);
-                        int32_t code[4];
+                        for (int j = 0; j < FN; ++j) {
+                            const int pxl = wn * 32 * FN + j * 32 + (lane & 31);
+                            int32_t code[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            float v = (float)acc[i][j][g * 4 + e] * sc[e];
-                            if (kFloatBias) v = v + fb[e];  // reference mode: float bias after the scale multiply
-                            code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                            for (int e = 0; e < 4; ++e) {
+                                float v = (float)acc[i][j][g * 4 + e] * sc[e];
+                                if (kFloatBias) v = v + fb[e];  // reference mode: float bias after the scale multiply
+                                code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                            }
+                            *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
                         }
-                        *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
+                    } else {
+                        float pre[FN * 4];
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                float v = (float)acc[i][j][g * 4 + e] * sc[e];
+                                if (kFloatBias) v = v + fb[e];
+                                pre[j * 4 + e] = quantize_prefloor_u8<kPath == 2>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                            }
+                        uint32_t word[FN];
+                        if constexpr (FN == 2) {
+                            floor_sat_u8x8(pre, &word[0], &word[1]);
+                        } else {
+                            word[0] = floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]);
+                        }
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+                            *reinterpret_cast<uint32_t*>(staged(lds_out, wn * 32 * FN + j * 32 + (lane & 31), ocl)) = word[j];
                     }
                 }
         };
+        // The residual chunks this thread will add are requested now: their latency runs under the
+        // requantization instead of in front of every store.
+        constexpr int ITER = TN * OUT_CHUNKS / T;
+        v4i rres[ITER];
+        if (kRes) {
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int q = tid + it * T;
+                const int64_t m = m0 + q / OUT_CHUNKS;
+                const int oc = oc0 + (q % OUT_CHUNKS) * 16;
+                rres[it] = v4i{0, 0, 0, 0};
+                if (m < a.M && oc + 16 <= a.OC && a.res.r_vec_ok)
+                    rres[it] = *reinterpret_cast<const v4i*>(a.res.r + m * a.res.r_px_stride + oc);
+            }
+        }
         __syncthreads();  // every wave is done reading the slot's operands
-        if (a.rq.bias_mode == kBiasReferenceFloat) requantize_tile(std::true_type());
-        else requantize_tile(std::false_type());
+        {
+            using P0 = std::integral_constant<int, 0>;
+            using P1 = std::integral_constant<int, 1>;
+            using P2 = std::integral_constant<int, 2>;
+            const bool u8_reference = !kRne && a.rq.q.lo == 0.f && a.rq.q.hi == 255.f;
+            const bool float_bias = a.rq.bias_mode == kBiasReferenceFloat;
+            if (!u8_reference) {
+                if (float_bias) requantize_tile(std::true_type(), P0());
+                else requantize_tile(std::false_type(), P0());
+            } else if (a.lo_folded > 0.f) {
+                if (float_bias) requantize_tile(std::true_type(), P2());
+                else requantize_tile(std::false_type(), P2());
+            } else {
+                if (float_bias) requantize_tile(std::true_type(), P1());
+                else requantize_tile(std::false_type(), P1());
+            }
+        }
         __syncthreads();
-        for (int q = tid; q < TN * OUT_CHUNKS; q += T) {
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int q = tid + it * T;
             const int pxl = q / OUT_CHUNKS;
             const int ch = q % OUT_CHUNKS;
             const int64_t m = m0 + pxl;
@@ -642,11 +701,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             v4i val = *reinterpret_cast<const v4i*>(src);
             const bool whole = oc + 16 <= a.OC;
             if (kRes) {
-                const char* rsrc = a.res.r + m * a.res.r_px_stride + oc;
-                v4i rv = {0, 0, 0, 0};
-                if (a.res.r_vec_ok && whole) {
-                    rv = *reinterpret_cast<const v4i*>(rsrc);
-                } else {
+                v4i rv = rres[it];
+                if (!(a.res.r_vec_ok && whole)) {
+                    const char* rsrc = a.res.r + m * a.res.r_px_stride + oc;
 #pragma nounroll
                     for (int w = 0; w < 4; ++w) {
                         uint32_t word = 0;
@@ -655,7 +712,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                         rv[w] = (int)word;
                     }
                 }
-                val = add_residual16(val, rv, a.res);
+                val = a.res.out.lo == 0.f ? add_residual16<true>(val, rv, a.res) : add_residual16<false>(val, rv, a.res);
                 if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
             }
             char* dst = a.y + m * a.y_px_stride + oc;

@@ -242,8 +242,11 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
         }
 
         // requantize into the wave's staging rows
-        auto requantize_tile = [&](auto float_bias_tag) {
+        // kPath 0: any 8-bit type and rounding; 1: uint8 in the reference's rounding through
+        // floor_sat_u8x4; 2: the same with a lower bound above 0 (a folded Relu)
+        auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
+            constexpr int kPath = decltype(path_tag)::value;
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 if (oc0 + i * 32 >= a.OC) break;
@@ -254,18 +257,36 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
                     v4f fbs = {0.f, 0.f, 0.f, 0.f};
                     if (kFloatBias) fbs = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
                     int32_t code[4];
+                    float pre[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         float v = (float)acc[i][g * 4 + e] * sc[e];
                         if (kFloatBias) v = v + fbs[e];
-                        code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                        if (kPath == 0) code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                        else pre[e] = quantize_prefloor_u8<kPath == 2>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
                     }
-                    *reinterpret_cast<uint32_t*>(staged(p, ocl)) = pack4(code[0], code[1], code[2], code[3]);
+                    *reinterpret_cast<uint32_t*>(staged(p, ocl)) =
+                            kPath == 0 ? pack4(code[0], code[1], code[2], code[3]) : floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]);
                 }
             }
         };
-        if (a.rq.bias_mode == kBiasReferenceFloat) requantize_tile(std::true_type());
-        else requantize_tile(std::false_type());
+        {
+            using P0 = std::integral_constant<int, 0>;
+            using P1 = std::integral_constant<int, 1>;
+            using P2 = std::integral_constant<int, 2>;
+            const bool u8_reference = !kRne && a.rq.q.lo == 0.f && a.rq.q.hi == 255.f;
+            const bool float_bias = a.rq.bias_mode == kBiasReferenceFloat;
+            if (!u8_reference) {
+                if (float_bias) requantize_tile(std::true_type(), P0());
+                else requantize_tile(std::false_type(), P0());
+            } else if (a.lo_folded > 0.f) {
+                if (float_bias) requantize_tile(std::true_type(), P2());
+                else requantize_tile(std::false_type(), P2());
+            } else {
+                if (float_bias) requantize_tile(std::true_type(), P1());
+                else requantize_tile(std::false_type(), P1());
+            }
+        }
         // the staging rows are private to the wave: its own LDS operations complete in order
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {

@@ -97,6 +97,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
             fb[d * 4 + e] = kFloatBias ? (float)b4[e] : 0.f;
         }
     }
+    const bool u8_reference = !kRne && a.q.lo == 0.f && a.q.hi == 255.f, lower_bound = a.lo_folded > 0.f;  // uniform
     const int fill = (int)(((uint32_t)(a.x_zp_u & 0xff)) * 0x01010101u);  // the zero point, already in the unsigned range
     const char* xn = a.x + (int64_t)n * a.x_n_stride + c0;
     char* yrow = a.y + (int64_t)n * a.y_n_stride + (int64_t)oh * a.y_h_stride + c0;
@@ -139,6 +140,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
 #pragma unroll
         for (int d = 0; d < kDw; ++d) {
             int32_t code[4];
+            float pre[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int ch = d * 4 + e;
@@ -152,9 +154,12 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
                 }
                 float v = (float)acc * sc[ch];
                 if (kFloatBias) v = v + fb[ch];
-                code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
+                // uint8 in the reference's rounding: clamp, conversion and packing in floor_sat_u8x4
+                if (u8_reference) pre[e] = lower_bound ? quantize_prefloor_u8<true>(v, a.q, a.inv_y_scale, a.lo_folded)
+                                                        : quantize_prefloor_u8<false>(v, a.q, a.inv_y_scale, 0.f);
+                else code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
             }
-            o[d] = (int)pack4(code[0], code[1], code[2], code[3]);
+            o[d] = u8_reference ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
         }
         *reinterpret_cast<vxi*>(yrow + (int64_t)ow * a.y_w_stride) = o;
     }

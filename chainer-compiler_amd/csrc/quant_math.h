@@ -106,6 +106,60 @@ __device__ __forceinline__ int32_t quantize_value_folded(float v, const QuantPar
     return (int32_t)s;
 }
 
+// uint8 results in the reference's rounding without the clamp, the conversion and the byte
+// packing as separate instructions.  v_cvt_pk_u8_f32 converts with the current fp32 rounding
+// mode, saturates to [0, 255] and drops the byte into place; under round-toward-minus-infinity it
+// is clamp(floor(x), 0, 255) for every finite x (checked on gfx950 over all 2^32 inputs).  With
+// x = t + 0.5f computed beforehand in the default rounding, that is the reference's
+// AsType(Maximum(0, Minimum(t, 255)) + 0.5f): inside the range the two are the same operations,
+// below it both give 0 (t + 0.5f <= 0.5 there), above it both give 255.  The rounding mode of the
+// wave is switched and restored inside one asm statement, so no other instruction can end up
+// between the two switches.  A lower bound above 0 (a folded Relu) is applied to t by the caller.
+__device__ __forceinline__ uint32_t floor_sat_u8x4(float a, float b, float c, float d) {
+    uint32_t r;
+    asm volatile(
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2\n\t"
+            "v_cvt_pk_u8_f32 %0, %1, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %0, %2, 1, %0\n\t"
+            "v_cvt_pk_u8_f32 %0, %3, 2, %0\n\t"
+            "v_cvt_pk_u8_f32 %0, %4, 3, %0\n\t"
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+            : "=&v"(r)
+            : "v"(a), "v"(b), "v"(c), "v"(d));
+    return r;
+}
+
+__device__ __forceinline__ void floor_sat_u8x8(const float (&x)[8], uint32_t* lo, uint32_t* hi) {
+    uint32_t r0, r1;
+    asm volatile(
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2\n\t"
+            "v_cvt_pk_u8_f32 %0, %2, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %1, %6, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %0, %3, 1, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %7, 1, %1\n\t"
+            "v_cvt_pk_u8_f32 %0, %4, 2, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %8, 2, %1\n\t"
+            "v_cvt_pk_u8_f32 %0, %5, 3, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %9, 3, %1\n\t"
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+            : "=&v"(r0), "=&v"(r1)
+            : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]));
+    *lo = r0;
+    *hi = r1;
+}
+
+// The value handed to floor_sat_u8x4/8 for one element: quantize_value_folded up to and including
+// the + 0.5f, with only the lower bound applied (and only when it is above 0).
+template <bool kLowerBound>
+__device__ __forceinline__ float quantize_prefloor_u8(float v, const QuantParams& q, float inv_scale, float lo_folded) {
+    const float q0 = v * inv_scale;
+    const float r = __builtin_fmaf(-q0, q.scale, v);
+    float s = __builtin_fmaf(r, inv_scale, q0);
+    s = s + q.zpf;
+    if (kLowerBound) s = __builtin_fmaxf(s, lo_folded);
+    return s + 0.5f;
+}
+
 // dequantize_array, runtime/ops/quantize.cc:37-44: (float(x) - zp) * scale.
 // Subtracting 0.0f is exact, so the "skip when zero" needs no branch either.
 __device__ __forceinline__ float dequantize_value(int32_t q, float zpf, float scale) {
