@@ -128,49 +128,42 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         sec = timed_steps(torch, lambda _t: replay(), args.steps, args.warmup)
 
     # Launch duration of the dominant kernel: event pairs cannot be recorded inside a graph
-    # replay, and around single 15-60 us launches they mostly measure submission gaps.  So each
-    # QLinearConv instruction of the program is launched REP times back to back between one
-    # event pair on the launch stream, on the buffers of the step just timed.  The per-step
-    # kernel time is the sum of the per-instruction averages.
-    REP = 20
+    # replay, and around single 10-60 us launches they mostly measure submission gaps.  So the
+    # QLinearConv instructions of the program (for MobileNetV2: the depthwise ones) are recorded,
+    # in program order and on the buffers of the step just timed, into a graph of their own;
+    # that graph is replayed REP times between one event pair on the launch stream.  Every layer
+    # then finds its input where the timed step leaves it (written many launches earlier, not
+    # just re-read), and launches follow each other without host submission gaps.
+    REP = 10
     # the launches timed are those of the timed region: one slice's instructions, times the slices
     slices = [(runner, x)] if args.parts <= 1 else [(r, x[lo:hi]) for (lo, hi), r in zip(timed_runner.slices, timed_runner.runners)]
     conv_ms_per_step, n_launch = 0.0, 0
-    pairs = []
     layer_graphs = []
     for rn, xs in slices:
         vals = rn.run(xs)
         torch.cuda.synchronize()
+        fids = []
         for fid, ins in enumerate(model["program"]):
             if ins[0] != "QLinearConv":
                 continue
-            c = model["convs"][ins[3]]
-            if mobilenet and c.group == 1:
+            if mobilenet and model["convs"][ins[3]].group == 1:
                 continue  # MobileNetV2: the roofline figure is the depthwise kernel's
-            # the instruction as the timed step launches it (with its residual sum when that is fused in)
-            fn = lambda: rn.launch(fid, vals)
-            # REP launches recorded into a graph of their own: replayed, they follow each other the way
-            # the instructions of the timed graph do, without host submission gaps between them
-            fn()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for _ in range(REP):
-                    fn()
-            layer_graphs.append(g)
+            fids.append(fid)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for fid in fids:
+                rn.launch(fid, vals)   # as the timed step launches it (with its residual sum when that is fused in)
+        layer_graphs.append(g)
+        g.replay()
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(REP):
             g.replay()
-            a = torch.cuda.Event(enable_timing=True)
-            b = torch.cuda.Event(enable_timing=True)
-            a.record()
-            g.replay()
-            b.record()
-            pairs.append((ins[3], a, b))
-            n_launch += 1
-    torch.cuda.synchronize()
-    per_layer = {}
-    for name, a, b in pairs:
-        ms = a.elapsed_time(b) / REP
-        per_layer[name] = per_layer.get(name, 0.0) + ms
-        conv_ms_per_step += ms
+        b.record()
+        torch.cuda.synchronize()
+        conv_ms_per_step += a.elapsed_time(b) / REP
+        n_launch += len(fids)
     if mobilenet:
         achieved = model["depthwise_bytes"] / (conv_ms_per_step * 1e-3) / 1e9
         roofline = dict(bound="hbm", kernel="depthwise3x3_kernel (%d launches per step, summed)" % n_launch,
