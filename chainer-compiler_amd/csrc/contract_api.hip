@@ -939,6 +939,9 @@ extern "C" int chx_hip_qconv_plan_run_add(
     res.out = make_quant_params(out_scale, out_zero_point, out->dtype == CHX_HIP_INT8);
     res.inv_out_scale = 1.0f / out_scale;
     res.big = 0x1p40f * out_scale;
+    // |DQ(y) + DQ(r)| <= 511 * (|y_scale| + |r_scale|): when that is far below `big`, limiting is the identity
+    const double reach = 511.0 * (fabs((double)y_scale) + fabs((double)r_scale));
+    res.guard = (reach == reach && reach < 0.25 * (double)res.big) ? 0 : 1;
     hipStream_t s = as_stream(stream);
     ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0);
     call.cache = const_cast<ScratchCache*>(&plan->scratch);

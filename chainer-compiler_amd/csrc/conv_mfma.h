@@ -26,6 +26,7 @@ struct ResidualAdd {
     QuantParams out;       // quantization of the sum
     float inv_out_scale;
     float big;             // 2^40 * out.scale: the dividend is limited to +-big (both sides saturate beyond)
+    int32_t guard;         // 0 when the operand scales already keep every sum far inside +-big
 };
 
 struct ConvMfmaArgs {

@@ -311,7 +311,7 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 // Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
 // (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
 // reference's order, one IEEE operation each.
-template <bool kU8>
+template <bool kU8, bool kGuard>
 __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
     v4i out;
 #pragma unroll
@@ -325,7 +325,7 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
             const float fb = ((float)((rw >> (8 * e)) & 0xffu) - p.r_zpf) * p.r_scale;
             float sum = fa + fb;
             if (p.relu) sum = __builtin_fmaxf(sum, 0.f);
-            sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
+            if (kGuard) sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
             if (kU8) pre[e] = quantize_prefloor_u8<false>(sum, p.out, p.inv_out_scale, 0.f);
             else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
         }
@@ -712,7 +712,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                         rv[w] = (int)word;
                     }
                 }
-                val = a.res.out.lo == 0.f ? add_residual16<true>(val, rv, a.res) : add_residual16<false>(val, rv, a.res);
+                if (a.res.guard)
+                    val = a.res.out.lo == 0.f ? add_residual16<true, true>(val, rv, a.res) : add_residual16<false, true>(val, rv, a.res);
+                else
+                    val = a.res.out.lo == 0.f ? add_residual16<true, false>(val, rv, a.res) : add_residual16<false, false>(val, rv, a.res);
                 if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
             }
             char* dst = a.y + m * a.y_px_stride + oc;
