@@ -26,6 +26,7 @@ RUNTIME_EXPORTS = [
     "chxvm_program_create", "chxvm_program_destroy", "chxvm_program_num_instructions", "chxvm_program_num_inputs",
     "chxvm_program_input_name", "chxvm_program_run", "chxvm_outputs_count", "chxvm_outputs_name", "chxvm_outputs_get",
     "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name", "chxvm_set_option", "chxvm_counter",
+    "chxc_compile", "chxc_transform", "chxc_fusion_program", "chxc_quantize_data", "chxc_free",
 ]
 
 # ChxVMValueProto.Type
@@ -78,6 +79,8 @@ def runtime():
         rt.chxvm_backend_config_has.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_char_p,
                                                 ctypes.POINTER(ctypes.c_int32)]
         rt.chxvm_set_option.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
+        rt.chxc_free.argtypes = [ctypes.c_void_p]
+        rt.chxc_free.restype = None
         rt.chxvm_counter.argtypes = [ctypes.c_char_p]
         rt.chxvm_counter.restype = ctypes.c_int64
         rt.chxvm_backend_config_name.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
@@ -379,6 +382,62 @@ def set_option(name, value):
     """Runtime switches: "qlinearconv_bias" = "reference" (default) | "onnx_int32";
     "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards)."""
     _check(runtime().chxvm_set_option(name.encode(), value.encode()))
+
+
+# ---------------------------------------------------------------------------------------------
+# compiler side (compiler/compiler_capi.h)
+# ---------------------------------------------------------------------------------------------
+
+def _options(options):
+    import json
+    return json.dumps(options or {}).encode()
+
+
+def compile_onnx(model_bytes, options=None):
+    """ONNX ModelProto bytes -> serialized ChxVMProgramProto, through the quantizer and fusion passes
+    that `options` selects (see compiler_capi.h)."""
+    rt = runtime()
+    out, n = ctypes.c_void_p(), ctypes.c_size_t()
+    _check(rt.chxc_compile(bytes(model_bytes), len(model_bytes), _options(options), ctypes.byref(out), ctypes.byref(n)))
+    try:
+        return ctypes.string_at(out, n.value)
+    finally:
+        rt.chxc_free(out)
+
+
+def transform_onnx(model_bytes, options=None):
+    """Runs the passes only: (ONNX ModelProto bytes of the rewritten graph, one-line-per-node description)."""
+    rt = runtime()
+    out, n, desc = ctypes.c_void_p(), ctypes.c_size_t(), ctypes.c_void_p()
+    _check(rt.chxc_transform(bytes(model_bytes), len(model_bytes), _options(options), ctypes.byref(out), ctypes.byref(n),
+                             ctypes.byref(desc)))
+    try:
+        return ctypes.string_at(out, n.value), ctypes.string_at(desc).decode()
+    finally:
+        rt.chxc_free(out)
+        rt.chxc_free(desc)
+
+
+def fusion_program(model_bytes, group, options=None):
+    """Program text of fusion group number `group` (1-based) after the passes."""
+    rt = runtime()
+    text = ctypes.c_void_p()
+    _check(rt.chxc_fusion_program(bytes(model_bytes), len(model_bytes), _options(options), int(group), ctypes.byref(text)))
+    try:
+        return ctypes.string_at(text).decode()
+    finally:
+        rt.chxc_free(text)
+
+
+def quantize_data(data, dtype):
+    """The weight quantization of the quantizer pass on one float32 array: (codes, scale, zero_point)."""
+    a = np.ascontiguousarray(data, dtype=np.float32).ravel()
+    codes = np.empty(a.size, np.int32)
+    scale, zp = ctypes.c_float(), ctypes.c_int64()
+    dt = np.dtype(dtype)
+    _check(runtime().chxc_quantize_data(a.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(a.size), DTYPE[str(dt)], ctypes.byref(scale),
+                                        ctypes.byref(zp), codes.ctypes.data_as(ctypes.c_void_p)))
+    return codes.reshape(np.shape(data)).astype(dt), np.float32(scale.value), zp.value
 
 
 def counter(name):

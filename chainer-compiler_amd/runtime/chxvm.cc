@@ -1,5 +1,7 @@
 #include "chxvm.h"
 
+#include <set>
+
 #include <iostream>
 
 namespace chainer_compiler {
@@ -179,6 +181,23 @@ private:
     std::shared_ptr<ResidualFusionState> state_;
 };
 
+// A fused op followed by the Free instructions of its operands that the program had placed
+// between the instructions it replaces.
+class SequenceOp : public ChxVMOp {
+public:
+    SequenceOp(const ChxVMInstructionProto& inst, std::vector<std::unique_ptr<ChxVMOp>> ops) : ChxVMOp(inst), ops_(std::move(ops)) {
+    }
+    void InitImpl() override {
+        for (auto& op : ops_) op->InitImpl();
+    }
+    void Run(ChxVMState* st) override {
+        for (auto& op : ops_) op->Run(st);
+    }
+
+private:
+    std::vector<std::unique_ptr<ChxVMOp>> ops_;
+};
+
 class NopOp : public ChxVMOp {
 public:
     explicit NopOp(const ChxVMInstructionProto& inst) : ChxVMOp(inst) {
@@ -294,6 +313,32 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
             break;
         }
     }
+    // A fused op runs where its last instruction stood but reads the operands of the earlier ones: a
+    // Free of such an operand between the two (the compiler frees a value right after its last
+    // reader) moves behind the fused op.
+    std::vector<std::vector<int>> deferred_frees(n);
+    std::vector<bool> deferred(n, false);
+    for (int q = 0; q < n; ++q) {
+        if (role[q] != 2 && role[q] != 3) continue;
+        std::vector<int> dropped = {fused_inputs[q].first, fused_inputs[q].second};
+        if (role[q] == 2) dropped.push_back(producer[program.instructions[q].inputs[0].array]);
+        std::set<int> operands;
+        int first = q;
+        for (int d : dropped) {
+            first = d < first ? d : first;
+            for (const ChxVMValueProto& v : program.instructions[d].inputs) {
+                if (v.type == ChxVMValueProto::ARRAY || v.type == ChxVMValueProto::OPTIONAL_ARRAY) operands.insert(v.array);
+                if (v.type == ChxVMValueProto::SCALAR || v.type == ChxVMValueProto::OPTIONAL_SCALAR) operands.insert(v.scalar);
+            }
+        }
+        for (int i = first; i < q; ++i) {
+            const ChxVMInstructionProto& fi = program.instructions[i];
+            if (fi.op == kFree && fi.inputs.size() == 1 && fi.inputs[0].array >= 0 && operands.count(fi.inputs[0].array)) {
+                deferred[i] = true;
+                deferred_frees[q].push_back(i);
+            }
+        }
+    }
     std::vector<std::shared_ptr<ResidualFusionState>> fusion_state(n);
     std::vector<bool> dead(num_variables_ > 0 ? num_variables_ : 1, false);
     for (int i = 0; i < n; ++i)
@@ -303,7 +348,7 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
     for (int i = 0; i < n; ++i) {
         const ChxVMInstructionProto& inst = program.instructions[i];
         const bool frees_dead = inst.op == kFree && inst.inputs.size() == 1 && inst.inputs[0].array >= 0 && dead[inst.inputs[0].array];
-        if (role[i] == 1 || frees_dead) {
+        if (role[i] == 1 || frees_dead || deferred[i]) {
             program_.emplace_back(new NopOp(inst));
         } else if (role[i] == 3) {
             const ChxVMInstructionProto& pool = program.instructions[fused_inputs[i].second];
@@ -319,6 +364,12 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
                                                            program.instructions[fused_inputs[i].second]));
         } else {
             program_.emplace_back(MakeChxVMOp(inst));
+        }
+        if (!deferred_frees[i].empty()) {
+            std::vector<std::unique_ptr<ChxVMOp>> seq;
+            seq.push_back(std::move(program_.back()));
+            for (int f : deferred_frees[i]) seq.emplace_back(MakeChxVMOp(program.instructions[f]));
+            program_.back().reset(new SequenceOp(inst, std::move(seq)));
         }
         program_.back()->InitImpl();
     }

@@ -27,6 +27,15 @@ int32_t Guard(Fn fn) {
 
 }  // namespace
 
+namespace chainer_compiler {
+namespace runtime {
+// for the other C faces of this library (compiler/compiler_capi.cc)
+void SetLastError(const std::string& message) {
+    g_last_error = message;
+}
+}  // namespace runtime
+}  // namespace chainer_compiler
+
 struct chxvm_program {
     std::unique_ptr<ChxVM> vm;
 };

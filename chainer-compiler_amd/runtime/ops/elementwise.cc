@@ -81,5 +81,64 @@ std::vector<chainerx::Array> ElementWiseNvrtcOp::RunImpl(ChxVMState* st, const s
     return outputs;
 }
 
+// The float element-wise ops that stay single instructions when no fusion group takes them
+// (runtime/ops/math.cc:31-41,105, activation.cc:20-22,55-61 of the chainer-compiler tree): each runs
+// as a one-statement program through the same generator, so a value computed by a lone op and the
+// same value computed inside a group are the same bits.
+namespace {
+
+chainerx::Array RunFloatOp(const char* op, const std::vector<chainerx::Array>& inputs) {
+    static const char* names[] = {"a", "b"};
+    chainerx::Shape shape = inputs[0].shape();
+    std::string code = "chxhip-fusion 1\nin";
+    for (size_t i = 0; i < inputs.size(); ++i) {
+        CHECK(inputs[i].dtype() == chainerx::Dtype::kFloat32) << op << " runs on float32 arrays on the hip backend, got " << inputs[i].dtype();
+        shape = chainerx::internal::BroadcastShapes(shape, inputs[i].shape());
+        code += std::string(" ") + names[i] + ":float32";
+    }
+    code += std::string("\ny = ") + op;
+    for (size_t i = 0; i < inputs.size(); ++i) code += std::string(" ") + names[i];
+    code += "\nout y:float32\n";
+    chainerx::Array y = chainerx::Empty(shape, chainerx::Dtype::kFloat32);
+    std::vector<chx_hip_tensor> in_desc;
+    for (const chainerx::Array& a : inputs) in_desc.push_back(a.hip());
+    chx_hip_tensor out_desc = y.hip();
+    std::vector<const chx_hip_tensor*> in_ptr;
+    for (chx_hip_tensor& t : in_desc) in_ptr.push_back(&t);
+    chx_hip_tensor* out_ptr = &out_desc;
+    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, in_ptr.data(), static_cast<int32_t>(in_ptr.size()), &out_ptr, 1, nullptr));
+    return y;
+}
+
+}  // namespace
+
+chainerx::Array AddOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
+    return RunFloatOp("Add", {a, b});
+}
+chainerx::Array SubOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
+    return RunFloatOp("Sub", {a, b});
+}
+chainerx::Array MulOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
+    return RunFloatOp("Mul", {a, b});
+}
+chainerx::Array DivOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
+    return RunFloatOp("Div", {a, b});
+}
+chainerx::Array NegOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Neg", {x});
+}
+chainerx::Array ExpOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Exp", {x});
+}
+chainerx::Array TanhOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Tanh", {x});
+}
+chainerx::Array SigmoidOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Sigmoid", {x});
+}
+chainerx::Array ReluOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Relu", {x});
+}
+
 }  // namespace runtime
 }  // namespace chainer_compiler

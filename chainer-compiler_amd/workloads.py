@@ -453,6 +453,69 @@ def program_to_chxvm(model, vm, ops, keep=("logits",)):
     return b
 
 
+def program_to_onnx(model, onnx_lite, keep=("logits",)):
+    """The op program as an ONNX QDQ graph (serialized ModelProto): QuantizeLinear / QLinearConv /
+    DequantizeLinear nodes with initializers, pools between a DequantizeLinear and a QuantizeLinear,
+    residual sums as DequantizeLinear, DequantizeLinear, Add, [Relu], QuantizeLinear -- what a
+    quantization tool leaves and the compiler side here takes (fusion pass, emitter)."""
+    g = onnx_lite.Graph()
+    g.name = "network"
+    q = model["qparams"]
+    inits = {}
+
+    def const(name, value):
+        inits[name] = np.asarray(value)
+        return name
+
+    def qp(name):
+        return [const(name + "_scale", np.float32(q[name][0])), const(name + "_zp", np.uint8(q[name][1]))]
+    nodes = []
+    for ins in model["program"]:
+        kind, out = ins[0], ins[1]
+        if kind == "QuantizeLinear":
+            g.inputs.append((ins[2], onnx_lite.FLOAT, list(model["shapes"][ins[2]])))
+            nodes.append(onnx_lite.Node("QuantizeLinear", [ins[2], const(out + "_scale", np.float32(ins[3])), const(out + "_zp", np.uint8(ins[4]))],
+                                        [out]))
+        elif kind == "QLinearConv":
+            c = model["convs"][ins[3]]
+            n = ins[3]
+            operands = [ins[2], const(n + "_xs", np.float32(c.x_scale)), const(n + "_xz", np.uint8(c.x_zp)), const(n + "_w", c.wq),
+                        const(n + "_ws", c.w_scale), const(n + "_wz", c.w_zp), const(n + "_ys", np.float32(c.y_scale)),
+                        const(n + "_yz", np.uint8(c.y_zp)), const(n + "_b", c.bias_q)]
+            k = c.wq.shape[2]
+            nodes.append(onnx_lite.Node("QLinearConv", operands, [out],
+                                        {"strides": [c.stride, c.stride], "pads": [c.pad] * 4, "group": c.group, "kernel_shape": [k, k]}, name=n))
+        elif kind in ("MaxPool", "AveragePool"):
+            nodes.append(onnx_lite.Node("DequantizeLinear", [ins[2]] + qp(ins[2]), [out + "__f"]))
+            if kind == "MaxPool":
+                attrs = {"kernel_shape": [ins[3]] * 2, "strides": [ins[4]] * 2, "pads": [ins[5]] * 4, "chainer_cover_all": 1 if ins[6] else 0}
+            else:
+                attrs = {"kernel_shape": [ins[3]] * 2, "strides": [1, 1], "pads": [0] * 4}
+            nodes.append(onnx_lite.Node(kind, [out + "__f"], [out + "__p"], attrs))
+            nodes.append(onnx_lite.Node("QuantizeLinear", [out + "__p"] + qp(out), [out]))
+        elif kind in ("AddRelu", "Add"):
+            nodes.append(onnx_lite.Node("DequantizeLinear", [ins[2]] + qp(ins[2]), [out + "__fa"]))
+            nodes.append(onnx_lite.Node("DequantizeLinear", [ins[3]] + qp(ins[3]), [out + "__fb"]))
+            nodes.append(onnx_lite.Node("Add", [out + "__fa", out + "__fb"], [out + "__s"]))
+            last = out + "__s"
+            if kind == "AddRelu":
+                nodes.append(onnx_lite.Node("Relu", [last], [out + "__r"]))
+                last = out + "__r"
+            nodes.append(onnx_lite.Node("QuantizeLinear", [last] + qp(out), [out]))
+        elif kind == "DequantizeLinear":
+            nodes.append(onnx_lite.Node("DequantizeLinear", [ins[2], const(out + "_scale", np.float32(ins[3])), const(out + "_zp", np.uint8(ins[4]))],
+                                        [out]))
+        else:
+            raise ValueError(kind)
+    g.nodes = nodes
+    g.initializers = inits
+    g.inputs += [(k, onnx_lite.ONNX_OF[v.dtype], list(v.shape)) for k, v in inits.items()]
+    for name in keep:
+        elem = onnx_lite.FLOAT if name == "logits" else onnx_lite.UINT8
+        g.outputs.append((name, elem, list(model["shapes"][name])))
+    return onnx_lite.make_model(g)
+
+
 def slice_model(model, lo, hi):
     """The same program on images lo..hi-1 of the batch (weights and quantization parameters are
     shared; only the shapes and the input change)."""

@@ -1,0 +1,333 @@
+"""The compiler side without a GPU: ONNX reader/writer, graph IR, fusion-group formation, the hip
+program builder, the quantizer pass and the emitter -- against the reference's own fusion test
+(compiler/fusion_test.cc: Tanh -> Sigmoid becomes one group of two), against independent numpy
+restatements of the weight quantization formulas (compiler/quantize.cc:68-89), and against the
+rewrites that pass documents (node sequences, operand order, copied attributes)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+import __graft_entry__ as entry  # noqa: E402
+
+pkg = entry.load_package()
+from importlib import import_module  # noqa: E402
+
+onnx_lite = import_module(pkg.__name__ + ".onnx_lite")
+F = onnx_lite.FLOAT
+
+
+@pytest.fixture(scope="module")
+def vm():
+    mod = import_module(pkg.__name__ + ".chxvm")
+    if not os.path.exists(mod.RUNTIME_LIB):
+        entry.build()
+    mod.runtime()
+    return mod
+
+
+def model(nodes, inputs, outputs, initializers=None):
+    g = onnx_lite.Graph()
+    g.name = "test"
+    g.nodes = [onnx_lite.Node(*n) if not isinstance(n, onnx_lite.Node) else n for n in nodes]
+    g.inputs = [(n, F, list(s)) for n, s in inputs]
+    g.outputs = [(n, F, list(s)) for n, s in outputs]
+    g.initializers = dict(initializers or {})
+    for name, a in g.initializers.items():
+        g.inputs.append((name, onnx_lite.ONNX_OF[a.dtype], list(a.shape)))
+    return onnx_lite.make_model(g)
+
+
+def lines(desc):
+    return [l for l in desc.splitlines() if l]
+
+
+def ops_of(desc):
+    return [l.split("(")[0] for l in lines(desc)]
+
+
+def test_fusion_basic_tanh_sigmoid(vm):
+    """compiler/fusion_test.cc:11-30."""
+    m = model([("Tanh", ["input"], ["tmp"]), ("Sigmoid", ["tmp"], ["output"])], [("input", ())], [("output", ())])
+    for kind in ("nvrtc", "hip"):
+        _, desc = vm.transform_onnx(m, {"fuse": kind})
+        assert len(lines(desc)) == 1
+        assert lines(desc)[0].startswith("ChainerFusionGroup(input) -> (output)")
+        assert lines(desc)[0].endswith("[%s #1: Tanh Sigmoid]" % kind)
+    _, desc = vm.transform_onnx(m, {"fuse": "none"})
+    assert ops_of(desc) == ["Tanh", "Sigmoid"]
+
+
+def test_fusable_sets_and_minimum_size(vm):
+    chain = [("Mul", ["x", "a"], ["t0"]), ("Add", ["t0", "b"], ["t1"]), ("Tanh", ["t1"], ["t2"]), ("Sigmoid", ["c"], ["t3"]),
+             ("Mul", ["t2", "t3"], ["t4"]), ("Add", ["t4", "x"], ["t5"]), ("Relu", ["t5"], ["y"])]
+    m = model(chain, [("x", (4, 8)), ("a", (8,)), ("b", (8,)), ("c", (4, 8))], [("y", (4, 8))])
+    # the reference's set has no Relu: it stays outside the group
+    _, desc = vm.transform_onnx(m, {"fuse": "nvrtc"})
+    assert ops_of(desc) == ["ChainerFusionGroup", "Relu"]
+    assert "Mul Add Tanh Sigmoid Mul Add" in desc or sorted(lines(desc)[0].split(": ")[1].rstrip("]").split()) == \
+        sorted("Mul Add Tanh Sigmoid Mul Add".split())
+    # the hip set takes the whole chain; inputs in name order
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    assert ops_of(desc) == ["ChainerFusionGroup"]
+    assert lines(desc)[0].startswith("ChainerFusionGroup(a, b, c, x) -> (y)")
+    # one calculation is not a group (min_fuse_ops = 2); Identity and Constant do not count
+    m1 = model([("Add", ["x", "x"], ["t"]), ("Identity", ["t"], ["y"])], [("x", (3,))], [("y", (3,))])
+    _, desc = vm.transform_onnx(m1, {"fuse": "hip"})
+    assert ops_of(desc) == ["Add", "Identity"]
+
+
+def test_fusion_rejects_cycles_and_unused_constants(vm):
+    # s = Tanh(x); m = Softmax(s) (not fusable); y = Add(s, m): fusing Tanh and Add would put the
+    # group both before and after Softmax
+    m = model([("Tanh", ["x"], ["s"]), ("Softmax", ["s"], ["m"]), ("Add", ["s", "m"], ["y"])], [("x", (2, 3))], [("y", (2, 3))])
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    assert ops_of(desc) == ["Tanh", "Softmax", "Add"]
+    # with a second fusable node before the fork the front part still fuses
+    m = model([("Exp", ["x"], ["e"]), ("Tanh", ["e"], ["s"]), ("Softmax", ["s"], ["m"]), ("Add", ["s", "m"], ["y"])],
+              [("x", (2, 3))], [("y", (2, 3))])
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    assert ops_of(desc) == ["ChainerFusionGroup", "Softmax", "Add"]
+    # a one-element float constant joins the group that reads it; one that only outside nodes read does not
+    k = onnx_lite.Node("Constant", [], ["k"], {"value": np.array(2.0, np.float32)})
+    k2 = onnx_lite.Node("Constant", [], ["k2"], {"value": np.array(3.0, np.float32)})
+    m = model([k, k2, ("Mul", ["x", "k"], ["t"]), ("Tanh", ["t"], ["u"]), ("Softmax", ["u"], ["v"]), ("Pow", ["v", "k2"], ["y"])],
+              [("x", (2, 3))], [("y", (2, 3))])
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    assert ops_of(desc) == ["Constant", "ChainerFusionGroup", "Softmax", "Pow"]
+    assert "Constant Mul Tanh" in desc or "[hip #1: Constant Mul Tanh]" in desc
+
+
+def test_hip_program_text_compiles(vm):
+    capi = pkg.capi
+    k = onnx_lite.Node("Constant", [], ["half"], {"value": np.array(0.5, np.float32)})
+    clip = onnx_lite.Node("Clip", ["t1"], ["t2"], {"min": 0.0, "max": 6.0})
+    m = model([k, ("Mul", ["x", "half"], ["t0"]), ("Add", ["t0", "b"], ["t1"]), clip, ("Neg", ["t2"], ["y"])],
+              [("x", (4, 8)), ("b", (8,))], [("y", (4, 8))])
+    text = vm.fusion_program(m, 1, {"fuse": "hip"})
+    st = [l for l in text.splitlines()]
+    assert st[0] == "chxhip-fusion 1" and st[1] == "in v_fi000_b:float32 v_fi001_x:float32"
+    assert st[2].endswith("= Const 0x3f000000")
+    assert [l.split(" = ")[1].split()[0] for l in st[2:-1]] == ["Const", "Mul", "Add", "Clip", "Neg"]
+    assert "0x00000000 0x40c00000" in st[5] and st[-1].startswith("out ") and st[-1].endswith(":float32")
+    # the generator accepts it and hiprtc compiles the kernel for gfx950 (host only)
+    full = capi.make_desc(0x10000000, capi.FLOAT32, (4, 8), (32, 4))
+    vec = capi.make_desc(0x20000000, capi.FLOAT32, (8,), (4,))
+    src = capi.elementwise_source(text, 1, [vec, full], [full], compile=True)
+    assert "fusion1_" in src
+
+
+def test_quantize_dequantize_parameters_are_written_into_the_group(vm):
+    """QuantizeLinear / DequantizeLinear with constant parameters fuse (hip set only); the scale and
+    zero point are no operands of the kernel."""
+    inits = {"s1": np.array(0.05, np.float32), "z1": np.array(128, np.uint8), "s2": np.array(0.02, np.float32),
+             "z2": np.array(3, np.int8), "s3": np.array(0.06, np.float32), "z3": np.array(7, np.uint8)}
+    g = onnx_lite.Graph()
+    g.nodes = [onnx_lite.Node("DequantizeLinear", ["a", "s1", "z1"], ["fa"]), onnx_lite.Node("DequantizeLinear", ["b", "s2", "z2"], ["fb"]),
+               onnx_lite.Node("Add", ["fa", "fb"], ["s"]), onnx_lite.Node("Relu", ["s"], ["r"]),
+               onnx_lite.Node("QuantizeLinear", ["r", "s3", "z3"], ["q"])]
+    g.inputs = [("a", onnx_lite.UINT8, [2, 16, 4, 4]), ("b", onnx_lite.INT8, [2, 16, 4, 4])]
+    g.inputs += [(k, onnx_lite.ONNX_OF[v.dtype], []) for k, v in inits.items()]
+    g.outputs = [("q", onnx_lite.UINT8, [2, 16, 4, 4])]
+    g.initializers = inits
+    m = onnx_lite.make_model(g)
+    _, desc = vm.transform_onnx(m, {"fuse": "nvrtc"})
+    assert ops_of(desc) == ["DequantizeLinear", "DequantizeLinear", "Add", "Relu", "QuantizeLinear"]   # Add alone is no group
+    text = vm.fusion_program(m, 1, {"fuse": "hip"})
+    st = text.splitlines()
+    assert st[1].split()[1:] == ["v_fi000_a:uint8", "v_fi001_b:int8"]
+    assert "DequantizeLinear v_fi000_a 0x3d4ccccd 128" in text and "DequantizeLinear v_fi001_b 0x3ca3d70a 3" in text
+    assert st[-2].endswith("0x3d75c28f 7 uint8") and st[-1].endswith(":uint8")
+    # this is exactly the residual-sum group a convolution can absorb
+    got = pkg.capi.match_residual_add(text)
+    assert got is not None and got["relu"] and got["in_zero_point"] == [128, 3] and got["out_zero_point"] == 7
+    # and the emitted instruction takes only the two tensors
+    prog = vm.compile_onnx(m, {"fuse": "hip"})
+    insts = decode_program(vm, prog)
+    assert [i[0] for i in insts] == ["In", "In", "ElementWiseNvrtc", "Free", "Free", "Out"]
+    assert insts[2][1][0] == ("ARRAY_LIST", [1, 2])
+
+
+def decode_program(vm, data):
+    """[(op name, [(value type name, value)], outputs)] of a serialized program."""
+    names = {v: k for k, v in vm.VALUE_TYPE.items()}
+    out = []
+    for f, w, v in onnx_lite.fields(data):
+        if f != 1:
+            continue
+        op, ins, outs = None, [], []
+        for f2, w2, v2 in onnx_lite.fields(v):
+            if f2 == 1:
+                op = vm.op_name(v2)
+            elif f2 == 2:
+                typ, val, lst = None, None, []
+                for f3, w3, v3 in onnx_lite.fields(v2):
+                    if f3 == 1:
+                        typ = names[v3]
+                    elif f3 in (2, 3, 8, 11, 12, 13):
+                        val = v3 - (1 << 64) if v3 >= 1 << 63 else v3
+                    elif f3 == 4:
+                        val = np.frombuffer(v3, "<f8")[0]
+                    elif f3 == 6:
+                        val = bytes(v3).decode()
+                    elif f3 in (5, 7):
+                        lst.append(v3 - (1 << 64) if v3 >= 1 << 63 else v3)
+                    elif f3 == 10:
+                        lst.append(float(np.frombuffer(v3, "<f8")[0]))
+                ins.append((typ, lst if typ in ("INTS", "INT_VALUES", "ARRAY_LIST", "DOUBLES") else val))
+            elif f2 == 3:
+                outs.append(v2 - (1 << 64) if v2 >= 1 << 63 else v2)
+        out.append((op, ins, outs))
+    return out
+
+
+def numpy_quantize(data, dtype):
+    """compiler/quantize.cc:68-89, spelled with numpy float32 operations."""
+    d = np.asarray(data, np.float32)
+    rmin, rmax = np.float32(min(d.min(), 0)), np.float32(max(d.max(), 0))
+    if dtype == np.int8:
+        scale = np.float32(np.float32(max(abs(rmin), abs(rmax)) * np.float32(2)) / np.float32(254))
+        return np.rint((d / scale).astype(np.float64)).astype(np.float32).astype(np.int8), scale, 0
+    scale = np.float32((rmax - rmin) / np.float32(255)) if rmin != rmax else np.float32(1)
+    zp = int(np.rint(np.float32(np.float32(0) - rmin) / scale))
+    return (np.rint((d / scale).astype(np.float64)).astype(np.float32) + np.float32(zp)).astype(np.uint8), scale, zp
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int8])
+def test_weight_quantization_formulas(vm, dtype):
+    rng = np.random.default_rng(5)
+    for case in range(6):
+        w = (rng.standard_normal((7, 5, 3)) * (0.01 + case)).astype(np.float32)
+        if case == 1:
+            w = np.abs(w)            # all positive: the range is widened to contain 0
+        if case == 2:
+            w = -np.abs(w)
+        codes, scale, zp = vm.quantize_data(w, dtype)
+        want, wscale, wzp = numpy_quantize(w, dtype)
+        assert scale == wscale and zp == wzp
+        np.testing.assert_array_equal(codes, want)
+        # reconstruction error within half a step (one step at the clamped end of uint8)
+        recon = (codes.astype(np.float32) - zp) * scale
+        assert np.abs(recon - w).max() <= scale * 0.5001 + 1e-7
+    codes, scale, zp = vm.quantize_data(np.zeros(4, np.float32), np.uint8)
+    assert scale == 1 and zp == 0 and not codes.any()
+
+
+CONV_ATTRS = {"strides": [2, 2], "pads": [1, 1, 1, 1], "kernel_shape": [3, 3], "group": 1, "dilations": [1, 1]}
+
+
+def conv_model(rng, with_bias=False):
+    w = (rng.standard_normal((6, 4, 3, 3)) * 0.2).astype(np.float32)
+    inits = {"w": w}
+    ins = ["x", "w"]
+    if with_bias:
+        inits["bias"] = np.zeros(6, np.float32)
+        ins.append("bias")
+    m = model([onnx_lite.Node("Conv", ins, ["y"], dict(CONV_ATTRS))], [("x", (1, 4, 8, 8))], [("y", (1, 6, 4, 4))], inits)
+    return m, w
+
+
+def test_quantizer_static_qlinear_rewrite(vm):
+    rng = np.random.default_rng(6)
+    m, w = conv_model(rng)
+    opts = {"fuse": "none", "quantize": {"mode": "QLinearOps", "static": True, "asymmetric_input_types": True, "per_channel": True,
+                                         "inputs": {"x": {"scale": 0.02, "zero_point": 121}},
+                                         "outputs": {"y": {"scale": 0.05, "zero_point": 7, "dtype": "uint8"}}}}
+    out, desc = vm.transform_onnx(m, opts)
+    g = onnx_lite.parse_model(out)
+    kinds = [n.op_type for n in g.nodes]
+    assert sorted(kinds) == sorted(["Constant"] * 7 + ["QuantizeLinear", "QLinearConv", "DequantizeLinear"])
+    const = {n.outputs[0]: n.attrs["value"] for n in g.nodes if n.op_type == "Constant"}
+    q = next(n for n in g.nodes if n.op_type == "QuantizeLinear")
+    conv = next(n for n in g.nodes if n.op_type == "QLinearConv")
+    dq = next(n for n in g.nodes if n.op_type == "DequantizeLinear")
+    # x -> QuantizeLinear(x, 0.02, uint8 121) -> QLinearConv(..) -> DequantizeLinear(.., 0.05, 7) -> y
+    assert q.inputs[0] == "x" and const[q.inputs[1]] == np.float32(0.02) and const[q.inputs[2]] == 121 and const[q.inputs[2]].dtype == np.uint8
+    assert conv.inputs[0] == q.outputs[0] and conv.inputs[1:3] == q.inputs[1:3]
+    assert dq.inputs[0] == conv.outputs[0] and dq.outputs == ["y"] and dq.inputs[1:] == conv.inputs[6:8]
+    assert const[conv.inputs[6]] == np.float32(0.05) and const[conv.inputs[7]] == 7
+    for k, v in CONV_ATTRS.items():
+        assert conv.attrs[k] == v
+    # per-channel int8 weights: every output channel on its own scale
+    wq, ws, wz = const[conv.inputs[3]], const[conv.inputs[4]], const[conv.inputs[5]]
+    assert wq.dtype == np.int8 and wq.shape == w.shape and ws.shape == (6,) and wz.shape == (6,) and wz.dtype == np.int8 and not wz.any()
+    for c in range(6):
+        want, scale, _ = numpy_quantize(w[c], np.int8)
+        np.testing.assert_array_equal(wq[c], want)
+        assert ws[c] == scale
+    # per tensor, uint8 weights (the reference's default input types)
+    opts["quantize"].update(per_channel=False, asymmetric_input_types=False)
+    g = onnx_lite.parse_model(vm.transform_onnx(m, opts)[0])
+    const = {n.outputs[0]: n.attrs["value"] for n in g.nodes if n.op_type == "Constant"}
+    conv = next(n for n in g.nodes if n.op_type == "QLinearConv")
+    want, scale, zp = numpy_quantize(w, np.uint8)
+    np.testing.assert_array_equal(const[conv.inputs[3]], want)
+    assert const[conv.inputs[4]].shape == () and const[conv.inputs[4]] == scale and const[conv.inputs[5]] == zp
+    # missing parameters are an error that names the value
+    bad = {"fuse": "none", "quantize": {"mode": "QLinearOps", "static": True, "inputs": {"x": {"scale": 0.02, "zero_point": 1}}}}
+    with pytest.raises(vm.ChxVMError, match="output 'y'"):
+        vm.transform_onnx(m, bad)
+
+
+def test_quantizer_dynamic_integer_rewrite(vm):
+    """The default mode (compiler/passes.cc:121-125): parameters computed at run time, integer
+    contraction, scale back in float."""
+    rng = np.random.default_rng(7)
+    m, w = conv_model(rng)
+    out, desc = vm.transform_onnx(m, {"fuse": "none", "quantize": {"per_channel": True}})
+    g = onnx_lite.parse_model(out)
+    kinds = [n.op_type for n in g.nodes]
+    for op, count in (("ReduceMin", 1), ("ReduceMax", 1), ("Sub", 2), ("Div", 2), ("Floor", 1), ("Cast", 2), ("QuantizeLinear", 1),
+                      ("ConvInteger", 1), ("Mul", 2), ("Reshape", 1)):
+        assert kinds.count(op) == count, (op, kinds)
+    conv = next(n for n in g.nodes if n.op_type == "ConvInteger")
+    for k, v in CONV_ATTRS.items():
+        assert conv.attrs[k] == v
+    const = {n.outputs[0]: n.attrs["value"] for n in g.nodes if n.op_type == "Constant"}
+    want, scale, zp = numpy_quantize(w[0], np.uint8)
+    np.testing.assert_array_equal(const[conv.inputs[1]][0], want)            # uint8 weights per channel
+    reshape = next(n for n in g.nodes if n.op_type == "Reshape")
+    assert const[reshape.inputs[1]].tolist() == [6, 1, 1]
+    last = g.nodes[-1]
+    assert last.op_type == "Mul" and last.outputs == ["y"]
+    casts = [n for n in g.nodes if n.op_type == "Cast"]
+    assert sorted(c.attrs["to"] for c in casts) == [onnx_lite.FLOAT, onnx_lite.UINT8]
+    # int8 activations would use the symmetric formula; MatMul takes the same route, per tensor
+    mm = model([("MatMul", ["a", "b"], ["y"])], [("a", (3, 5))], [("y", (3, 2))], {"b": rng.standard_normal((5, 2)).astype(np.float32)})
+    g = onnx_lite.parse_model(vm.transform_onnx(mm, {"fuse": "none", "quantize": {}})[0])
+    assert [n.op_type for n in g.nodes].count("MatMulInteger") == 1 and "Reshape" not in [n.op_type for n in g.nodes]
+    # a convolution with a bias is left alone (compiler/quantize.cc:383-387)
+    mb, _ = conv_model(rng, with_bias=True)
+    g = onnx_lite.parse_model(vm.transform_onnx(mb, {"fuse": "none", "quantize": {}})[0])
+    assert [n.op_type for n in g.nodes] == ["Conv"]
+
+
+def test_emitted_program_for_a_quantized_convolution(vm):
+    rng = np.random.default_rng(8)
+    m, w = conv_model(rng)
+    opts = {"quantize": {"mode": "QLinearOps", "static": True, "asymmetric_input_types": True, "per_channel": True,
+                         "inputs": {"x": {"scale": 0.02, "zero_point": 121}}, "outputs": {"y": {"scale": 0.05, "zero_point": 7}}}}
+    insts = decode_program(vm, vm.compile_onnx(m, opts))
+    names = [i[0] for i in insts]
+    assert names[0] == "In" and names[-1] == "Out"
+    assert names.count("QuantizeLinear") == 1 and names.count("QLinearConv") == 1 and names.count("DequantizeLinear") == 1
+    conv = next(i for i in insts if i[0] == "QLinearConv")
+    kinds = [t for t, _ in conv[1]]
+    assert kinds == ["ARRAY", "SCALAR", "SCALAR", "ARRAY", "ARRAY", "ARRAY", "SCALAR", "SCALAR", "ARRAY", "INTS", "INTS", "INT", "STRING"]
+    assert conv[1][8][1] == -1 and conv[1][9][1] == [2, 2] and conv[1][10][1] == [1, 1] and conv[1][11][1] == 1 and conv[1][12][1] == ""
+    # scales and zero points of the activations are scalar constants, the per-channel weight parameters arrays
+    assert names.count("FloatScalarConstant") == 2 and names.count("IntScalarConstant") == 2
+    assert names.count("IntConstant") == 2 and names.count("FloatConstant") == 1
+    # every temporary is freed after its last reader; the program survives the C++ reader and writer
+    assert names.count("Free") >= 3
+    data = vm.compile_onnx(m, opts)
+    assert vm.proto_roundtrip(data) == data
+    # node types outside the path are refused by the emitter, by name
+    sm = model([("Softmax", ["x"], ["y"])], [("x", (2, 3))], [("y", (2, 3))])
+    with pytest.raises(vm.ChxVMError, match="Softmax"):
+        vm.compile_onnx(sm)
+    with pytest.raises(vm.ChxVMError, match="unknown option"):
+        vm.compile_onnx(sm, {"fuze": "hip"})

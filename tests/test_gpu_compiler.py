@@ -1,0 +1,108 @@
+"""ONNX graphs through the compiler side (quantizer, fusion, emitter) and the C++ VM on the MI355X,
+compared with the CPU oracle: bit-exact for the 8-bit results and for the fused fp32 chain."""
+import numpy as np
+import pytest
+import torch
+
+import test_compiler_cpu as cc
+
+pytestmark = pytest.mark.gpu
+onnx_lite = cc.onnx_lite
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+@pytest.fixture(scope="module")
+def vm(g):
+    from importlib import import_module
+    return import_module(g.pkg.__name__ + ".chxvm")
+
+
+CHAIN = [("Mul", ["x", "a"], ["t0"]), ("Add", ["t0", "b"], ["t1"]), ("Tanh", ["t1"], ["t2"]), ("Sigmoid", ["c"], ["t3"]),
+         ("Mul", ["t2", "t3"], ["t4"]), ("Add", ["t4", "x"], ["t5"]), ("Relu", ["t5"], ["y"])]
+ORACLE_CHAIN = [("t0", "Mul", "x", "a"), ("t1", "Add", "t0", "b"), ("t2", "Tanh", "t1"), ("t3", "Sigmoid", "c"),
+                ("t4", "Mul", "t2", "t3"), ("t5", "Add", "t4", "x"), ("y", "Relu", "t5")]
+
+
+def test_float_chain_fused_and_op_by_op(g, vm, oracle):
+    """relu(tanh(x*a+b)*sigmoid(c)+x): as one hip group, as the reference's group plus a lone Relu,
+    and as seven single instructions -- the same bits each time, the oracle's."""
+    rng = np.random.default_rng(11)
+    shape = (6, 50, 128)
+    x, c = rng.standard_normal(shape).astype(np.float32), rng.standard_normal(shape).astype(np.float32)
+    a, b = rng.standard_normal(128).astype(np.float32), rng.standard_normal(128).astype(np.float32)
+    want = oracle.run_chain(ORACLE_CHAIN, dict(x=x, a=a, b=b, c=c))["y"]
+    m = cc.model(CHAIN, [("x", shape), ("a", (128,)), ("b", (128,)), ("c", shape)], [("y", shape)])
+    counts = {}
+    for fuse in ("hip", "nvrtc", "none"):
+        data = vm.compile_onnx(m, {"fuse": fuse})
+        names = [i[0] for i in cc.decode_program(vm, data)]
+        counts[fuse] = (names.count("ElementWiseNvrtc"), names.count("Relu"), names.count("Mul"))
+        prog = vm.Program(data)
+        got = prog.run({k: torch.from_numpy(v).cuda() for k, v in dict(x=x, a=a, b=b, c=c).items()})["y"]
+        prog.close()
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32), err_msg=fuse)
+    assert counts == {"hip": (1, 0, 0), "nvrtc": (1, 1, 0), "none": (0, 1, 2)}
+
+
+@pytest.mark.parametrize("per_channel,int8_weights", [(True, True), (False, True), (False, False), (True, False)])
+def test_quantized_convolution_from_a_float_graph(g, vm, oracle, per_channel, int8_weights):
+    """Conv -> (quantizer, static QLinearOps) -> QuantizeLinear, QLinearConv, DequantizeLinear, run on
+    the device: equal to the oracle's ops applied to weights quantized by the numpy restatement."""
+    rng = np.random.default_rng(12)
+    m, w = cc.conv_model(rng)
+    x = rng.standard_normal((1, 4, 8, 8)).astype(np.float32)
+    opts = {"quantize": {"mode": "QLinearOps", "static": True, "asymmetric_input_types": int8_weights, "per_channel": per_channel,
+                         "inputs": {"x": {"scale": 0.03, "zero_point": 121}}, "outputs": {"y": {"scale": 0.11, "zero_point": 90}}}}
+    prog = vm.Program(vm.compile_onnx(m, opts))
+    got = prog.run({"x": torch.from_numpy(x).cuda()})["y"]
+    prog.close()
+    wdt = np.int8 if int8_weights else np.uint8
+    if per_channel:
+        parts = [cc.numpy_quantize(w[c], wdt) for c in range(w.shape[0])]
+        wq = np.stack([p[0] for p in parts])
+        ws, wz = np.array([p[1] for p in parts], np.float32), np.array([p[2] for p in parts]).astype(wdt)
+    else:
+        wq, s, z = cc.numpy_quantize(w, wdt)
+        ws, wz = np.float32(s), np.array(z).astype(wdt)
+    xq = oracle.quantize_linear(x, 0.03, 121, np.uint8)
+    yq = oracle.qlinear_conv_int(xq, 0.03, 121, wq, ws, wz, np.float32(0.11), 90, np.uint8, strides=(2, 2), pads=(1, 1))
+    want = oracle.dequantize_linear(yq, 0.11, 90)
+    assert len(np.unique(yq)) > 8
+    np.testing.assert_array_equal(got, want)
+
+
+def test_network_from_an_onnx_qdq_graph(g, vm, oracle):
+    """The reduced ResNet written as an ONNX QDQ graph: the fusion pass turns every
+    DequantizeLinear, DequantizeLinear, Add, Relu, QuantizeLinear run into one hip group, the emitter
+    writes their parameters into the program text, and the VM computes each group inside the
+    convolution before it; the logits are the oracle's."""
+    wl = g.pkg.workloads
+    model = wl.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
+    m = wl.program_to_onnx(model, onnx_lite)
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    groups = [l for l in desc.splitlines() if l.startswith("ChainerFusionGroup")]
+    assert len(groups) == 5 and all(l.endswith(": DequantizeLinear DequantizeLinear Add Relu QuantizeLinear]") or
+                                    sorted(l.split(": ")[1].rstrip("]").split()) ==
+                                    sorted("DequantizeLinear DequantizeLinear Add Relu QuantizeLinear".split()) for l in groups)
+    data = vm.compile_onnx(m, {"fuse": "hip"})
+    before = vm.counter("qlinearconv_residual_fusions")
+    vm.set_option("qlinearconv_bias", "onnx_int32")
+    try:
+        prog = vm.Program(data)
+        got = prog.run({"x": torch.from_numpy(model["input"]).cuda()})["logits"]
+        prog.close()
+    finally:
+        vm.set_option("qlinearconv_bias", "reference")
+    assert vm.counter("qlinearconv_residual_fusions") - before == 5
+    oracle.set_threads(16)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"], keep={"logits"})
+    finally:
+        oracle.set_threads(1)
+    np.testing.assert_array_equal(got, ref["logits"])
