@@ -2,10 +2,11 @@
 checks the outputs the way tools/run_onnx.cc does.
 
   python -m chainer_compiler_amd.run_onnx --test DIR [--rtol 1e-4] [--atol 1e-6] [--iterations N]
-         [--trace] [--backend hip]
+         [--trace] [--backend hip] [--quantize] [--no_fuse_operations] [--dump_onnx FILE]
 
-DIR/model.onnx is lowered by chxvm_emit; every DIR/test_data_set_N supplies input_i.pb and
-output_i.pb in graph order.  An output passes when dtype and shape are equal and every element
+DIR/model.onnx goes through the compiler side of the runtime library (quantizer when --quantize is
+given, fusion-group formation, ChxVM emitter: chxvm.compile_onnx); every DIR/test_data_set_N
+supplies input_i.pb and output_i.pb in graph order.  An output passes when dtype and shape are equal and every element
 has |a - b| <= atol + rtol * |b| (tools/util.cc:89-121; the defaults are run_onnx.cc:299-300).
 Exit status 0 when every data set passes.  (From a checkout, where the package directory is
 not importable by name, use `python chainer-compiler_amd/run_onnx.py ...`.)
@@ -62,6 +63,10 @@ def main(argv=None):
     ap.add_argument("--atol", type=float, default=1e-6)
     ap.add_argument("--iterations", type=int, default=1)
     ap.add_argument("--trace", action="store_true")
+    ap.add_argument("--quantize", action="store_true",
+                    help="run the quantizer pass in its default mode (dynamic parameters, integer ops), as the reference's flag does")
+    ap.add_argument("--no_fuse_operations", action="store_true", help="no fusion groups: every node an instruction of its own")
+    ap.add_argument("--dump_onnx", default="", help="write the graph after the passes to this file")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args(argv)
 
@@ -69,7 +74,6 @@ def main(argv=None):
     import importlib
     import torch
     onnx_lite = importlib.import_module(pkg.__name__ + ".onnx_lite")
-    emit = importlib.import_module(pkg.__name__ + ".chxvm_emit")
     vm = importlib.import_module(pkg.__name__ + ".chxvm")
     pkg.capi.init(0)
 
@@ -77,8 +81,15 @@ def main(argv=None):
     if not data_sets:
         print("%s: no test_data_set_* directories" % args.test, file=sys.stderr)
         return 2
-    serialized, input_names, output_names = emit.emit_program(graph)
-    program = vm.Program(serialized)
+    model_bytes = open(os.path.join(args.test, "model.onnx"), "rb").read()
+    options = {"fuse": "none" if args.no_fuse_operations else "hip"}
+    if args.quantize:
+        options["quantize"] = {}
+    if args.dump_onnx:
+        open(args.dump_onnx, "wb").write(vm.transform_onnx(model_bytes, options)[0])
+    input_names = [name for name, _, _ in graph.inputs if name not in graph.initializers]
+    output_names = [name for name, _, _ in graph.outputs]
+    program = vm.Program(vm.compile_onnx(model_bytes, options))
     failed = 0
     for name, inputs, wants in data_sets:
         if len(inputs) != len(input_names) or len(wants) != len(output_names):

