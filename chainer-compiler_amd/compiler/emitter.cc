@@ -42,6 +42,12 @@ ChxVMValueProto ScalarIn(int id, bool optional = false) {
     v.set_scalar(id);
     return v;
 }
+ChxVMValueProto ShapeIn(int id) {
+    ChxVMValueProto v;
+    v.type = ChxVMValueProto::SHAPE;
+    v.set_shape(id);
+    return v;
+}
 ChxVMValueProto IntIn(int64_t i) {
     ChxVMValueProto v;
     v.type = ChxVMValueProto::INT;
@@ -172,8 +178,7 @@ private:
             c->outputs.push_back(IdOf(v));
             return;
         }
-        CHECK(!(scalar_uses_.count(v) && array_uses_.count(v) && t.NumElements() == 1))
-                << "constant '" << v->name() << "' is read both as a scalar and as an array";
+        // read both ways: an array constant, which the scalar readers convert (runtime/chxvm_var.cc:70-76)
         ChxVMInstructionProto* c = Add(is_float ? "FloatConstant" : "IntConstant");
         if (is_float) {
             std::vector<double> values(t.NumElements());
@@ -291,7 +296,20 @@ private:
                                    IntIn(n.GetInt("count_include_pad", 0))});
             }
             inst->outputs.push_back(-1);  // the backward context is not kept
-        } else if (op == "Identity" || op == "Neg" || op == "Exp" || op == "Tanh" || op == "Sigmoid" || op == "Relu") {
+        } else if (op == "Max" || op == "Min") {
+            std::vector<int> ins;
+            for (size_t i = 0; i < nin; ++i) ins.push_back(Operand(n, i));
+            simple(op, {ArrayListIn(ins)});
+        } else if ((op == "ReduceMax" || op == "ReduceMin") && nin == 1) {
+            simple(op, {ArrayIn(Operand(n, 0)), IntsIn(n.GetInts("axes")), IntIn(n.GetInt("keepdims", 1))});
+        } else if (op == "Reshape" && nin == 2) {
+            simple(op, {ArrayIn(Operand(n, 0)), ShapeIn(Operand(n, 1))});
+        } else if (op == "Cast" && nin == 1) {
+            const CDtype to = DtypeFromOnnx(static_cast<int>(n.GetInt("to", 0)));
+            CHECK(to != kUnknown) << n.ToString() << ": unsupported target type " << n.GetInt("to", 0);
+            simple(op, {ArrayIn(Operand(n, 0)), IntIn(to)});
+        } else if (op == "Identity" || op == "Neg" || op == "Exp" || op == "Tanh" || op == "Sigmoid" || op == "Relu" || op == "Abs" ||
+                   op == "Floor") {
             CHECK_EQ(1UL, nin) << n.ToString();
             simple(op, {ArrayIn(Operand(n, 0))});
         } else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div") {

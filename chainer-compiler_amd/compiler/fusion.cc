@@ -164,7 +164,7 @@ int FuseElementwiseOperations(Graph* graph) {
 }
 
 int FuseHipOperations(Graph* graph) {
-    static const std::set<std::string> float_ops = {"Identity", "Add", "Sub", "Mul", "Div", "Neg", "Tanh", "Sigmoid", "Exp", "Relu"};
+    static const std::set<std::string> float_ops = {"Identity", "Add", "Sub", "Mul", "Div", "Neg", "Tanh", "Sigmoid", "Exp", "Relu", "Abs", "Floor"};
     auto constant_operands = [](const Node& node, size_t first) {
         for (size_t i = first; i < node.inputs().size(); ++i) {
             if (node.input(i)->IsNull()) continue;
@@ -203,8 +203,16 @@ int FuseHipOperations(Graph* graph) {
     // A QuantizeLinear closes an element-wise computation and a DequantizeLinear opens the next one:
     // the 8-bit tensor between them is an activation of the network (other nodes read it, the
     // runtime keeps it channels-last), so groups do not grow across that edge.
+    // One kernel writes every output of a group in one shape (the broadcast of its operands,
+    // runtime/ops/nvrtc.cc:100-104), so two nodes whose results are known to differ in shape (a 0-d
+    // scale and the [OC] vector it is multiplied into) do not share a group.
     auto can_cross = [](const Node& producer, const Node& user) {
-        return !(producer.op_type() == "QuantizeLinear" && user.op_type() == "DequantizeLinear");
+        if (producer.op_type() == "QuantizeLinear" && user.op_type() == "DequantizeLinear") return false;
+        if (producer.op_type() == "Constant") return true;  // read in place by the kernel, no output of its own
+        const Type& a = producer.output(0)->type();
+        const Type& b = user.output(0)->type();
+        if (a.has_dims && b.has_dims && a.dims != b.dims) return false;
+        return true;
     };
     return FuseAllConnectedNodes("hip", graph, 2, false, is_fusable, can_cross);
 }
@@ -297,7 +305,8 @@ std::string BuildHipProgram(const Node& group, std::vector<int>* used_inputs) {
         const std::string out = CleanseIdent(node->output(0)->name());
         const std::string& op = node->op_type();
         CDtype out_dtype = kFloat32;
-        if (op == "Identity" || op == "Neg" || op == "Tanh" || op == "Sigmoid" || op == "Exp" || op == "Relu") {
+        if (op == "Identity" || op == "Neg" || op == "Tanh" || op == "Sigmoid" || op == "Exp" || op == "Relu" || op == "Abs" ||
+            op == "Floor") {
             os << out << " = " << op << " " << ins[0] << "\n";
         } else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div" || op == "Max" || op == "Min") {
             CHECK_EQ(2UL, ins.size()) << node->ToString();

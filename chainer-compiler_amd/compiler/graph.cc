@@ -529,11 +529,57 @@ void InferDtypes(Graph* graph) {
         } else if (!n->inputs().empty() && !n->input(0)->IsNull()) {
             dt = dtype_of(n->input(0));
         }
-        if (dt == kUnknown) continue;
+        // shapes, where they follow from the operands alone: a reduction over everything gives a 0-d
+        // value, element-wise ops broadcast, the quantizing ops keep the shape of their first operand
+        auto dims_of = [](const Value* v, std::vector<int64_t>* dims) {
+            if (v->type().has_dims) {
+                for (int64_t d : v->type().dims)
+                    if (d < 0) return false;
+                *dims = v->type().dims;
+                return true;
+            }
+            if (v->initializer()) {
+                *dims = v->initializer()->dims();
+                return true;
+            }
+            return false;
+        };
+        static const std::set<std::string> unary = {"Identity", "Neg", "Abs", "Floor", "Exp", "Tanh", "Sigmoid", "Relu", "Cast", "Clip",
+                                                    "QuantizeLinear", "DequantizeLinear"};
+        static const std::set<std::string> binary = {"Add", "Sub", "Mul", "Div", "Max", "Min"};
+        std::vector<int64_t> dims;
+        bool has_dims = false;
+        if (op == "Constant") {
+            if (std::unique_ptr<Tensor> t = n->tensor_value()) {
+                dims = t->dims();
+                has_dims = true;
+            }
+        } else if ((op == "ReduceMin" || op == "ReduceMax") && n->GetInts("axes").empty() && n->GetInt("keepdims", 1) == 0) {
+            has_dims = true;
+        } else if (unary.count(op) && !n->inputs().empty() && !n->input(0)->IsNull()) {
+            has_dims = dims_of(n->input(0), &dims);
+        } else if (binary.count(op) && n->inputs().size() == 2) {
+            std::vector<int64_t> a, b;
+            if (dims_of(n->input(0), &a) && dims_of(n->input(1), &b)) {
+                has_dims = true;
+                const size_t rank = std::max(a.size(), b.size());
+                dims.assign(rank, 1);
+                for (size_t i = 0; i < rank && has_dims; ++i) {
+                    const int64_t da = i < rank - a.size() ? 1 : a[i - (rank - a.size())];
+                    const int64_t db = i < rank - b.size() ? 1 : b[i - (rank - b.size())];
+                    if (da != db && da != 1 && db != 1) has_dims = false;
+                    dims[i] = da == 1 ? db : da;
+                }
+            }
+        }
         for (Value* o : n->outputs()) {
-            if (o->IsNull() || o->type().dtype != kUnknown) continue;
+            if (o->IsNull()) continue;
             Type t = o->type();
-            t.dtype = dt;
+            if (t.dtype == kUnknown) t.dtype = dt;
+            if (!t.has_dims && has_dims) {
+                t.dims = dims;
+                t.has_dims = true;
+            }
             o->set_type(t);
         }
     }

@@ -195,8 +195,9 @@ private:
 // Element types of the values no ValueInfo speaks of, for the node types of this path: the 8-bit
 // type of a quantizing op is that of its zero-point operand (uint8 without one), DequantizeLinear
 // gives float32, the integer contractions int32, Cast its `to`, everything else its first operand's
-// type (the part of the reference's type inference, compiler/type_inference.cc, that the fusion
-// rule and the program builder depend on).
+// type; shapes where they follow from the operands alone (constants, reductions over everything,
+// element-wise broadcasting).  The part of the reference's type inference
+// (compiler/type_inference.cc) that the fusion rule and the program builder depend on.
 void InferDtypes(Graph* graph);
 
 // compiler/topology.cc:15-59

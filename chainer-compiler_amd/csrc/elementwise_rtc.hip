@@ -21,7 +21,7 @@
 //   in  <name>:<dtype> ...            dtype: float32 | uint8 | int8
 //   <name> = <Op> <operand> ...       operands are earlier names or, where noted, literals
 //   out <name>:<dtype> ...
-// Ops: Identity a | Neg a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
+// Ops: Identity a | Neg a | Abs a | Floor a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
 //      Tanh a | Sigmoid a | Exp a | Relu a | Clip a <lo> <hi> | Const <value>
 //      QuantizeLinear a <scale> <zero_point> <uint8|int8> [rne]   (float -> 8-bit code)
 //      DequantizeLinear q <scale> <zero_point>                    (8-bit code -> float)
@@ -218,6 +218,14 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
             os << "  const float " << o << " = -" << a << ";\n";
+        } else if (s.op == "Abs") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = __builtin_fabsf(" << a << ");\n";
+        } else if (s.op == "Floor") {
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = __builtin_floorf(" << a << ");\n";
         } else if (s.op == "Tanh") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));

@@ -1,0 +1,139 @@
+// The small float ops that the dynamic quantization rewrite puts around the quantized ones
+// (compiler/quantize.cc:165-196,230-243 of the chainer-compiler tree): the minimum / maximum of a
+// whole float32 tensor (ReduceMin / ReduceMax without axes, keepdims = 0) and element type
+// conversions (Cast: int32 -> float32 for the scale-back, float32 -> uint8 / int8 for a computed
+// zero point).  Both take any strides; neither is on the timed path of a statically quantized
+// network.
+#include "chx_internal.h"
+
+namespace chx {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ int64_t strided_offset(int64_t flat, const StridedDesc& d) {
+    int64_t off = 0;
+    for (int a = d.ndim - 1; a >= 0; --a) {
+        const int64_t q = flat / d.shape[a];
+        off += (flat - q * d.shape[a]) * d.strides[a];
+        flat = q;
+    }
+    return off;
+}
+
+StridedDesc make_desc(const chx_hip_tensor& t) {
+    StridedDesc d;
+    d.ndim = t.ndim;
+    for (int i = 0; i < t.ndim; ++i) {
+        d.shape[i] = t.shape[i];
+        d.strides[i] = t.strides[i];
+    }
+    return d;
+}
+
+// min and max are exact and order-independent (a NaN anywhere gives NaN, as the comparison-based
+// reduction of the CPU path does not guarantee either way; NaN inputs are outside the tested domain)
+template <bool kMax>
+__device__ __forceinline__ float pick(float a, float b) {
+    return kMax ? (a > b ? a : b) : (a < b ? a : b);
+}
+
+template <bool kMax>
+__device__ float block_reduce(float v) {
+    __shared__ float red[kThreads];
+    red[threadIdx.x] = v;
+    __syncthreads();
+    for (int s = kThreads / 2; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] = pick<kMax>(red[threadIdx.x], red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    return red[0];
+}
+
+template <bool kMax>
+__global__ __launch_bounds__(kThreads) void reduce_partial_kernel(const char* __restrict__ x, StridedDesc xd, int64_t n, float* __restrict__ partial) {
+    float v = *reinterpret_cast<const float*>(x);  // element 0 exists: n > 0
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads)
+        v = pick<kMax>(v, *reinterpret_cast<const float*>(x + strided_offset(i, xd)));
+    v = block_reduce<kMax>(v);
+    if (threadIdx.x == 0) partial[blockIdx.x] = v;
+}
+
+template <bool kMax>
+__global__ __launch_bounds__(kThreads) void reduce_final_kernel(const float* __restrict__ partial, int count, float* __restrict__ y) {
+    float v = partial[0];
+    for (int i = threadIdx.x; i < count; i += kThreads) v = pick<kMax>(v, partial[i]);
+    v = block_reduce<kMax>(v);
+    if (threadIdx.x == 0) *y = v;
+}
+
+// AsType: float -> integer truncates toward zero; integer -> float rounds to nearest
+template <class From, class To>
+__global__ __launch_bounds__(kThreads) void cast_kernel(const char* __restrict__ x, StridedDesc xd, char* __restrict__ y, StridedDesc yd, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    *reinterpret_cast<To*>(y + strided_offset(i, yd)) = static_cast<To>(*reinterpret_cast<const From*>(x + strided_offset(i, xd)));
+}
+
+template <class From>
+int cast_from(const chx_hip_tensor& x, chx_hip_tensor& y, int64_t n, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads);
+    const StridedDesc xd = make_desc(x), yd = make_desc(y);
+    const char* xp = static_cast<const char*>(x.data);
+    char* yp = static_cast<char*>(y.data);
+    switch (y.dtype) {
+        case CHX_HIP_FLOAT32: cast_kernel<From, float><<<blocks, kThreads, 0, s>>>(xp, xd, yp, yd, n); break;
+        case CHX_HIP_INT32: cast_kernel<From, int32_t><<<blocks, kThreads, 0, s>>>(xp, xd, yp, yd, n); break;
+        case CHX_HIP_UINT8: cast_kernel<From, uint8_t><<<blocks, kThreads, 0, s>>>(xp, xd, yp, yd, n); break;
+        case CHX_HIP_INT8: cast_kernel<From, int8_t><<<blocks, kThreads, 0, s>>>(xp, xd, yp, yd, n); break;
+        default: CHX_FAIL(CHX_HIP_EUNSUPPORTED, "Cast: no conversion to %s on the device", dtype_name(y.dtype));
+    }
+    return launch_check("cast_kernel");
+}
+
+}  // namespace
+}  // namespace chx
+
+using namespace chx;
+
+extern "C" int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "ReduceMin/ReduceMax x"));
+    CHX_PROPAGATE(check_tensor(y, "ReduceMin/ReduceMax y"));
+    CHX_REQUIRE(x->dtype == CHX_HIP_FLOAT32 && y->dtype == CHX_HIP_FLOAT32, "ReduceMin/ReduceMax: float32 only");
+    CHX_REQUIRE(numel(*y) == 1, "ReduceMin/ReduceMax: y must hold one element (all axes reduced)");
+    const int64_t n = numel(*x);
+    CHX_REQUIRE(n > 0, "ReduceMin/ReduceMax of an empty tensor");
+    hipStream_t s = as_stream(stream);
+    int blocks = (int)((n + kThreads * 8 - 1) / (kThreads * 8));
+    blocks = blocks < 1 ? 1 : blocks > 1024 ? 1024 : blocks;
+    void* partial = nullptr;
+    CHX_PROPAGATE(scratch_alloc(&partial, sizeof(float) * blocks, s));
+    const StridedDesc xd = make_desc(*x);
+    if (is_max) {
+        reduce_partial_kernel<true><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, static_cast<float*>(partial));
+        reduce_final_kernel<true><<<1, kThreads, 0, s>>>(static_cast<const float*>(partial), blocks, static_cast<float*>(y->data));
+    } else {
+        reduce_partial_kernel<false><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, static_cast<float*>(partial));
+        reduce_final_kernel<false><<<1, kThreads, 0, s>>>(static_cast<const float*>(partial), blocks, static_cast<float*>(y->data));
+    }
+    const int rc = launch_check("reduce_min_max");
+    scratch_free(partial, s);
+    return rc;
+}
+
+extern "C" int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "Cast x"));
+    CHX_PROPAGATE(check_tensor(y, "Cast y"));
+    CHX_REQUIRE(x->ndim == y->ndim, "Cast: x and y differ in rank");
+    for (int i = 0; i < x->ndim; ++i) CHX_REQUIRE(x->shape[i] == y->shape[i], "Cast: x and y differ in shape");
+    const int64_t n = numel(*x);
+    if (n == 0) return CHX_HIP_OK;
+    hipStream_t s = as_stream(stream);
+    switch (x->dtype) {
+        case CHX_HIP_FLOAT32: return cast_from<float>(*x, *y, n, s);
+        case CHX_HIP_INT32: return cast_from<int32_t>(*x, *y, n, s);
+        case CHX_HIP_UINT8: return cast_from<uint8_t>(*x, *y, n, s);
+        case CHX_HIP_INT8: return cast_from<int8_t>(*x, *y, n, s);
+        default: CHX_FAIL(CHX_HIP_EUNSUPPORTED, "Cast: no conversion from %s on the device", dtype_name(x->dtype));
+    }
+}

@@ -264,6 +264,9 @@ public:
         return r;
     }
 
+    // A view of a contiguous array with another shape of the same size.
+    Array Reshape(const Shape& to) const;
+
     // chx_hip_tensor of this array (ChainerX strides are bytes already).
     chx_hip_tensor hip() const {
         chx_hip_tensor t;
@@ -348,6 +351,15 @@ inline Array FromHost(const void* src, const Shape& shape, Dtype dtype) {
 }
 
 // Synchronizing read of a contiguous array.
+inline Array Array::Reshape(const Shape& to) const {
+    CHECK(IsContiguous());
+    Array r;
+    r.body_ = std::make_shared<Body>(*body_);
+    r.body_->shape = to;
+    r.body_->strides = ContiguousStrides(to, GetItemSize());
+    return r;
+}
+
 inline void ToHost(const Array& a, void* dst) {
     CHECK(a.IsContiguous()) << "ToHost needs a contiguous array";
     CHXVM_HIP_CALL(chx_hip_memcpy_d2h(dst, static_cast<char*>(a.raw_data()) + a.offset(), static_cast<size_t>(a.GetNBytes()), nullptr));

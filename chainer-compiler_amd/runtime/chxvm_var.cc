@@ -57,6 +57,20 @@ const StrictScalar& ChxVMVar::GetScalar() const {
 }
 
 const chainerx::Shape& ChxVMVar::GetShape() const {
+    if (kind() == Kind::kArray) {
+        // a 1-D integer array read back as a shape (runtime/chxvm_var.cc:78-83, ArrayToShape)
+        if (!array_as_shape_) {
+            const chainerx::Array& a = std::get<chainerx::Array>(val_);
+            CHECK_GE(1, a.ndim()) << "a shape operand must be a vector";
+            CHECK(a.dtype() == chainerx::Dtype::kInt64 && a.IsContiguous()) << "a shape operand must be a contiguous int64 vector";
+            std::vector<int64_t> host(a.GetTotalSize());
+            if (!host.empty()) chainerx::ToHost(a, host.data());
+            chainerx::Shape shape;
+            for (int64_t d : host) shape.push_back(d);
+            array_as_shape_ = std::make_shared<chainerx::Shape>(shape);
+        }
+        return *array_as_shape_;
+    }
     CHECK_EQ(static_cast<int>(Kind::kShape), static_cast<int>(kind()));
     return std::get<chainerx::Shape>(val_);
 }

@@ -69,6 +69,7 @@ private:
     mutable VarInternalType val_;
     mutable std::shared_ptr<chainerx::Array> scalar_as_array_;
     mutable std::shared_ptr<StrictScalar> array_as_scalar_;
+    mutable std::shared_ptr<chainerx::Shape> array_as_shape_;
 };
 
 }  // namespace runtime

@@ -139,6 +139,81 @@ chainerx::Array SigmoidOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
 chainerx::Array ReluOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
     return RunFloatOp("Relu", {x});
 }
+chainerx::Array AbsOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Abs", {x});
+}
+chainerx::Array FloorOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Floor", {x});
+}
+
+// Maximum / Minimum folded over the operands (runtime/ops/math.cc:179-195)
+chainerx::Array MaxOp::RunImpl(ChxVMState* st, const std::vector<chainerx::Array>& inputs) {
+    CHECK_LT(0UL, inputs.size());
+    chainerx::Array result = inputs[0];
+    for (size_t i = 1; i < inputs.size(); ++i) result = RunFloatOp("Max", {result, inputs[i]});
+    return result;
+}
+chainerx::Array MinOp::RunImpl(ChxVMState* st, const std::vector<chainerx::Array>& inputs) {
+    CHECK_LT(0UL, inputs.size());
+    chainerx::Array result = inputs[0];
+    for (size_t i = 1; i < inputs.size(); ++i) result = RunFloatOp("Min", {result, inputs[i]});
+    return result;
+}
+
+namespace {
+
+// every axis reduced and dropped: the form the quantizer emits (compiler/quantize.cc:171-174)
+chainerx::Array ReduceAll(const chainerx::Array& x, const chainerx::StackVector<int64_t, chainerx::kMaxNdim>& axes, int keepdims, bool is_max) {
+    CHECK(axes.empty() || static_cast<int>(axes.size()) == x.ndim()) << "only the reduction over all axes runs on the hip backend";
+    CHECK_EQ(0, keepdims) << "keepdims is not supported on the hip backend";
+    CHECK(x.dtype() == chainerx::Dtype::kFloat32) << "ReduceMin / ReduceMax run on float32 arrays on the hip backend";
+    chainerx::Array y = chainerx::Empty(chainerx::Shape{}, chainerx::Dtype::kFloat32);
+    chx_hip_tensor xt = x.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_reduce_min_max(&xt, is_max ? 1 : 0, &yt, nullptr));
+    return y;
+}
+
+}  // namespace
+
+chainerx::Array ReduceMaxOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return ReduceAll(x, axes, keepdims, true);
+}
+chainerx::Array ReduceMinOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return ReduceAll(x, axes, keepdims, false);
+}
+
+// x.AsType(to) (runtime/ops/manipulation.cc:157-159)
+chainerx::Array CastOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
+    const chainerx::Dtype dt = static_cast<chainerx::Dtype>(to);
+    if (dt == input.dtype()) return input;
+    chainerx::Array y = chainerx::Empty(input.shape(), dt);
+    chx_hip_tensor xt = input.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, nullptr));
+    return y;
+}
+
+// a view of the same memory (runtime/ops/manipulation.cc:20-22); -1 and 0 entries as ONNX defines them
+chainerx::Array ReshapeOp::RunImpl(ChxVMState* st, const chainerx::Array& data, const chainerx::Shape& shape) {
+    CHECK(data.IsContiguous()) << "Reshape of a non-contiguous array is not supported on the hip backend";
+    chainerx::Shape to = shape;
+    int64_t known = 1;
+    int wildcard = -1;
+    for (int i = 0; i < static_cast<int>(to.size()); ++i) {
+        if (to[i] == 0) {
+            CHECK_LT(i, data.ndim());
+            to[i] = data.shape()[i];
+        }
+        if (to[i] == -1) {
+            CHECK_EQ(-1, wildcard) << "more than one -1 in a Reshape";
+            wildcard = i;
+        } else {
+            known *= to[i];
+        }
+    }
+    if (wildcard >= 0) to[wildcard] = known ? data.GetTotalSize() / known : 0;
+    CHECK_EQ(data.GetTotalSize(), to.GetTotalSize()) << "Reshape changes the number of elements";
+    return data.Reshape(to);
+}
 
 }  // namespace runtime
 }  // namespace chainer_compiler

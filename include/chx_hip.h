@@ -249,6 +249,15 @@ int chx_hip_elementwise_source(
         chx_hip_tensor* const* outputs, int32_t n_outputs, int32_t compile, char* buffer, size_t buffer_size,
         size_t* needed);
 
+/* ReduceMaxOp / ReduceMinOp::RunImpl (runtime/ops/statistics.cc:13-19, chainerx::AMax / AMin) for the only form
+ * the quantizer emits (compiler/quantize.cc:171-174): every axis reduced, keepdims = 0.  x float32,
+ * any strides; y float32 with one element. */
+int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream);
+
+/* CastOp::RunImpl (runtime/ops/manipulation.cc:157-159, CastTo): element types float32,
+ * int32, uint8, int8 on either side; float -> integer truncates toward zero. */
+int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream);
+
 /* Says whether a fusion program (the `code` of an ElementWiseNvrtc instruction, emitted per
  * FusionGroup by compiler/chxvm/emitter.cc:621-729) is exactly the residual sum of a quantized
  * network,  out = QuantizeLinear(act(DequantizeLinear(in0) + DequantizeLinear(in1)))  with

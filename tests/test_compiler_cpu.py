@@ -101,6 +101,26 @@ def test_fusion_rejects_cycles_and_unused_constants(vm):
     assert "Constant Mul Tanh" in desc or "[hip #1: Constant Mul Tanh]" in desc
 
 
+def test_groups_keep_to_one_result_shape(vm):
+    # ReduceMax over everything gives a 0-d value; its product with a [6] constant has six elements.
+    # One kernel writes every output of a group in the broadcast shape, so the two do not share a group.
+    k = onnx_lite.Node("Constant", [], ["half"], {"value": np.array(0.5, np.float32)})
+    w = onnx_lite.Node("Constant", [], ["w"], {"value": np.arange(6, dtype=np.float32)})
+    red = onnx_lite.Node("ReduceMax", ["x"], ["m"], {"keepdims": 0})
+    m = model([k, w, red, ("Mul", ["m", "half"], ["s"]), ("Abs", ["s"], ["t"]), ("Mul", ["t", "w"], ["u"]), ("Neg", ["u"], ["y"])],
+              [("x", (4, 8))], [("y", (6,)), ("t", ())])
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    groups = [l for l in lines(desc) if l.startswith("ChainerFusionGroup")]
+    assert len(groups) == 2
+    assert any("Mul Abs" in g and "-> (t)" in g for g in groups)
+    assert any("Mul Neg" in g and "-> (y)" in g for g in groups)
+    # operands of one shape: the chain stays whole
+    m = model([("Mul", ["a", "b"], ["s"]), ("Abs", ["s"], ["t"]), ("Mul", ["t", "c"], ["u"]), ("Neg", ["u"], ["y"])],
+              [("a", (4,)), ("b", (4,)), ("c", (4,))], [("y", (4,))])
+    _, desc = vm.transform_onnx(m, {"fuse": "hip"})
+    assert ops_of(desc) == ["ChainerFusionGroup"]
+
+
 def test_hip_program_text_compiles(vm):
     capi = pkg.capi
     k = onnx_lite.Node("Constant", [], ["half"], {"value": np.array(0.5, np.float32)})

@@ -106,3 +106,52 @@ def test_network_from_an_onnx_qdq_graph(g, vm, oracle):
     finally:
         oracle.set_threads(1)
     np.testing.assert_array_equal(got, ref["logits"])
+
+
+def _dynamic_uint8_params(x):
+    """The run-time parameter graph of the quantizer for a uint8 operand (compiler/quantize.cc:165-196),
+    in float32 numpy operations: the range is NOT widened to contain 0 here."""
+    rmin, rmax = np.float32(x.min()), np.float32(x.max())
+    scale = np.float32(np.float32(rmax - rmin) / np.float32(255))
+    zp = np.uint8(np.floor(np.float32(np.float32(0) - rmin) / scale))
+    return scale, zp
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_dynamic_integer_quantization_runs_end_to_end(g, vm, oracle, per_channel):
+    """The reference's --quantize path (dynamic parameters, integer ops): ReduceMin/ReduceMax, the scalar
+    arithmetic, QuantizeLinear, ConvInteger / MatMulInteger, Cast and the scale-back Mul all run on
+    the device; the result equals the same sequence spelled with numpy and the oracle."""
+    rng = np.random.default_rng(13)
+    m, w = cc.conv_model(rng)
+    x = (rng.standard_normal((1, 4, 8, 8)) * 2 + 0.3).astype(np.float32)
+    prog = vm.Program(vm.compile_onnx(m, {"quantize": {"per_channel": per_channel}}))
+    got = prog.run({"x": torch.from_numpy(x).cuda()})["y"]
+    prog.close()
+    scale, zp = _dynamic_uint8_params(x)
+    xq = oracle.quantize_linear(x, scale, int(zp), np.uint8)
+    if per_channel:
+        parts = [cc.numpy_quantize(w[c], np.uint8) for c in range(w.shape[0])]
+        wq = np.stack([p[0] for p in parts])
+        ws, wz = np.array([p[1] for p in parts], np.float32), np.array([p[2] for p in parts], np.uint8)
+    else:
+        wq, s, z = cc.numpy_quantize(w, np.uint8)
+        ws, wz = np.float32(s), np.array(z, np.uint8)
+    acc = oracle.conv_integer(xq, wq, int(zp), wz, strides=(2, 2), pads=(1, 1), group=1, auto_pad="")
+    scales = (scale * ws).astype(np.float32)
+    want = acc.astype(np.float32) * (scales.reshape(-1, 1, 1) if per_channel else scales)
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+    # the quantized result tracks the float convolution
+    ref = torch.nn.functional.conv2d(torch.from_numpy(x), torch.from_numpy(w), stride=2, padding=1).numpy()
+    assert np.abs(got - ref).max() < 0.05 * np.abs(ref).max() + 0.05
+    # MatMul the same way
+    b = rng.standard_normal((5, 3)).astype(np.float32)
+    a = rng.standard_normal((4, 5)).astype(np.float32)
+    mm = cc.model([("MatMul", ["a", "b"], ["y"])], [("a", (4, 5))], [("y", (4, 3))], {"b": b})
+    prog = vm.Program(vm.compile_onnx(mm, {"quantize": {}}))
+    got = prog.run({"a": torch.from_numpy(a).cuda()})["y"]
+    prog.close()
+    sa, za = _dynamic_uint8_params(a)
+    bq, sb, zb = cc.numpy_quantize(b, np.uint8)
+    acc = oracle.matmul_integer(oracle.quantize_linear(a, sa, int(za), np.uint8), bq, np.array(za, np.uint8), np.array(zb, np.uint8))
+    np.testing.assert_array_equal(got, acc.astype(np.float32) * np.float32(sa * sb))
