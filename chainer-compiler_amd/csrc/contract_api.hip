@@ -239,6 +239,7 @@ struct TunedConfig {
     int64_t M;
     int32_t H, W, OH, OW;
     int tile_oc, tile_px, max_wgs_per_cu;
+    bool with_res;  // measured with a fused residual sum (an entry of its own: the epilogue differs)
 };
 struct TuneCache {
     std::vector<TunedConfig> entries;
@@ -530,9 +531,9 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     const TunedConfig* tuned = nullptr;
     if (c.tune) {
         for (const TunedConfig& t : c.tune->entries)
-            if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW) tuned = &t;
+            if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW && t.with_res == (c.res != nullptr)) tuned = &t;
         if (!tuned && autotune_enabled() && !stream_is_capturing(s)) {
-            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0};
+            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, c.res != nullptr};
             rc = tune_conv_mfma(a, xu, c.out_int32, c.rne, s, &best);
             if (rc == CHX_HIP_OK) {
                 c.tune->entries.push_back(best);
