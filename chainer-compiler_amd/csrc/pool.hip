@@ -36,8 +36,24 @@ __device__ __forceinline__ uint32_t max4_u8(uint32_t a, uint32_t b) {
     return r;
 }
 
+// Byte-wise maximum of two dwords kept as two dwords of 16-bit lanes (even bytes, odd bytes): the
+// packed 16-bit maximum then does two bytes per instruction.
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+struct SplitBytes {
+    uint32_t even, odd;
+};
+__device__ __forceinline__ SplitBytes split_bytes(uint32_t x) {
+    return SplitBytes{x & 0x00ff00ffu, (x >> 8) & 0x00ff00ffu};
+}
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2us, a), __builtin_bit_cast(v2us, b)));
+}
+
 // channels-last, C % 16 == 0: one lane = 16 channels of one output pixel.  int8 codes are
-// compared as unsigned after flipping the sign bit.
+// compared as unsigned after flipping the sign bit.  The taps go out in groups of nine
+// unconditional loads: a tap outside the image reads the nearest pixel inside instead, which
+// belongs to the same window whenever the window touches the image at all, so it does not change
+// the maximum (a branch around the load would make every load wait for the one before).
 __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
     const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= a.total) return;
@@ -49,22 +65,37 @@ __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
     const int oh = (int)(r % a.OH);
     const int n = (int)(r / a.OH);
     const uint32_t flip = a.is_signed ? 0x80808080u : 0u;
-    v4u m = {0, 0, 0, 0};
-    for (int i = 0; i < a.kh; ++i) {
-        const int ih = oh * a.sh - a.ph + i;
-        if ((unsigned)ih >= (unsigned)a.H) continue;
-        for (int j = 0; j < a.kw; ++j) {
-            const int iw = ow * a.sw - a.pw + j;
-            if ((unsigned)iw >= (unsigned)a.W) continue;
-            v4u v = *reinterpret_cast<const v4u*>(a.x + n * a.xs[0] + ih * a.xs[2] + iw * a.xs[3] + cg * 16);
-            m[0] = max4_u8(m[0], v[0] ^ flip);
-            m[1] = max4_u8(m[1], v[1] ^ flip);
-            m[2] = max4_u8(m[2], v[2] ^ flip);
-            m[3] = max4_u8(m[3], v[3] ^ flip);
+    const int ih0 = oh * a.sh - a.ph, iw0 = ow * a.sw - a.pw;
+    const bool touches = ih0 < a.H && ih0 + a.kh > 0 && iw0 < a.W && iw0 + a.kw > 0;
+    const char* xn = a.x + n * a.xs[0] + cg * 16;
+    SplitBytes m[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+    const int taps = a.kh * a.kw;
+    int i = 0, j = 0;
+    for (int t0 = 0; t0 < taps; t0 += 9) {
+        v4u v[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int ih = min(max(ih0 + i, 0), a.H - 1), iw = min(max(iw0 + j, 0), a.W - 1);
+            v[t] = *reinterpret_cast<const v4u*>(xn + ih * a.xs[2] + iw * a.xs[3]);
+            // past the last tap: stay on it
+            if (t0 + t + 1 < taps && ++j == a.kw) {
+                j = 0;
+                ++i;
+            }
         }
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const SplitBytes x = split_bytes(v[t][d] ^ flip);
+                m[d].even = pk_max_u16(m[d].even, x.even);
+                m[d].odd = pk_max_u16(m[d].odd, x.odd);
+            }
     }
-    m[0] ^= flip; m[1] ^= flip; m[2] ^= flip; m[3] ^= flip;
-    *reinterpret_cast<v4u*>(a.y + n * a.ys[0] + oh * a.ys[2] + ow * a.ys[3] + cg * 16) = m;
+    v4u out;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) out[d] = touches ? (m[d].even | (m[d].odd << 8)) ^ flip : flip;
+    *reinterpret_cast<v4u*>(a.y + n * a.ys[0] + oh * a.ys[2] + ow * a.ys[3] + cg * 16) = out;
 }
 
 // any strides: one lane = one output element, channel index fastest
@@ -135,6 +166,7 @@ __global__ __launch_bounds__(kThreads) void average_pool_kernel(AvgArgs a) {
 // above, per channel, so the result is the same bytes.
 template <bool kRne>
 __global__ __launch_bounds__(kThreads) void average_pool_cl4_kernel(AvgArgs a) {
+    constexpr int kBatch = 16;  // loads in flight at a time
     const PoolArgs& p = a.p;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int C4 = p.C >> 2;
@@ -151,21 +183,21 @@ __global__ __launch_bounds__(kThreads) void average_pool_cl4_kernel(AvgArgs a) {
     int32_t cnt = 0;
     const char* xn = p.x + n * p.xs[0] + c;
     const int ih0 = oh * p.sh - p.ph, iw0 = ow * p.sw - p.pw;
-    // taps in (kh, kw) order, sixteen loads in flight at a time
+    // taps in (kh, kw) order
     const int taps = p.kh * p.kw;
     int i = 0, j = 0;
-    for (int t0 = 0; t0 < taps; t0 += 16) {
-        uint32_t v[16];
-        uint32_t valid = 0;
+    for (int t0 = 0; t0 < taps; t0 += kBatch) {
+        uint32_t v[kBatch];
+        uint64_t valid = 0;
         int ii = i, jj = j;
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
+        for (int t = 0; t < kBatch; ++t) {
             const int ih = ih0 + ii, iw = iw0 + jj;
             // every load goes out, from a clamped address when the tap does not count: a branch around
             // it would make the compiler wait for each load before the next
             const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
             v[t] = *reinterpret_cast<const uint32_t*>(xn + ihc * p.xs[2] + iwc * p.xs[3]) ^ flip;
-            valid |= (t0 + t < taps && ih == ihc && iw == iwc) ? 1u << t : 0u;
+            valid |= (t0 + t < taps && ih == ihc && iw == iwc) ? uint64_t(1) << t : uint64_t(0);
             if (++jj == p.kw) {
                 jj = 0;
                 ++ii;
@@ -174,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void average_pool_cl4_kernel(AvgArgs a) {
         i = ii;
         j = jj;
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
+        for (int t = 0; t < kBatch; ++t) {
             const bool on = (valid >> t) & 1u;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -189,6 +221,41 @@ __global__ __launch_bounds__(kThreads) void average_pool_cl4_kernel(AvgArgs a) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) code[e] = quantize_value<kRne>(sum[e] / (float)cnt, a.q);
     *reinterpret_cast<uint32_t*>(p.y + n * p.ys[0] + oh * p.ys[2] + ow * p.ys[3] + c) = pack4(code[0], code[1], code[2], code[3]);
+}
+
+// The window is the whole image (global pooling) and the pixels of an image are one dense run:
+// tap t of channel group c is at x + n*xs[0] + t*xs[3] + c, every tap counts, and all loads go out
+// before the first sum.  The sum runs over the pixels in storage order = (kh, kw) order, so the
+// result is the bytes of the kernels above.
+constexpr int kGlobalPoolTaps = 64;
+template <bool kRne>
+__global__ __launch_bounds__(kThreads) void global_average_pool_cl4_kernel(AvgArgs a) {
+    const PoolArgs& p = a.p;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int C4 = p.C >> 2;
+    if (idx >= (p.total >> 2)) return;
+    const int c = (int)(idx % C4) * 4;
+    const int64_t n = idx / C4;
+    const uint32_t flip = p.is_signed ? 0x80808080u : 0u;
+    const float zpf = a.x_zpf + (p.is_signed ? 128.f : 0.f);
+    const int taps = p.H * p.W;
+    const char* xn = p.x + n * p.xs[0] + c;
+    const uint32_t pitch = (uint32_t)p.xs[3];
+    uint32_t v[kGlobalPoolTaps];
+#pragma unroll
+    for (int t = 0; t < kGlobalPoolTaps; ++t) v[t] = *reinterpret_cast<const uint32_t*>(xn + (uint32_t)min(t, taps - 1) * pitch) ^ flip;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < kGlobalPoolTaps; ++t) {
+        if (t < taps) {  // uniform
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = sum[e] + ((float)((v[t] >> (8 * e)) & 0xffu) - zpf) * a.x_scale;
+        }
+    }
+    int32_t code[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) code[e] = quantize_value<kRne>(sum[e] / (float)taps, a.q);
+    *reinterpret_cast<uint32_t*>(p.y + n * p.ys[0] + c) = pack4(code[0], code[1], code[2], code[3]);
 }
 
 int fill_pool_args(
@@ -272,10 +339,18 @@ extern "C" int chx_hip_average_pool_q8(
     if (cl4) {
         // small work-groups: a global pool has few outputs, and they should reach every compute unit
         const unsigned blocks4 = (unsigned)((a.p.total / 4 + 63) / 64);
-        if (flags & CHX_HIP_ROUND_ONNX_RNE)
-            average_pool_cl4_kernel<true><<<blocks4, 64, 0, s>>>(a);
-        else
-            average_pool_cl4_kernel<false><<<blocks4, 64, 0, s>>>(a);
+        const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
+        const PoolArgs& p = a.p;
+        // the window is the whole image, stored as one dense run of pixels
+        const bool whole_image = p.OH == 1 && p.OW == 1 && p.ph == 0 && p.pw == 0 && p.kh == p.H && p.kw == p.W &&
+                                 (p.H == 1 || p.xs[2] == p.W * p.xs[3]) && p.H * p.W <= kGlobalPoolTaps;
+        if (whole_image) {
+            if (rne) global_average_pool_cl4_kernel<true><<<blocks4, 64, 0, s>>>(a);
+            else global_average_pool_cl4_kernel<false><<<blocks4, 64, 0, s>>>(a);
+            return launch_check("global_average_pool_cl4_kernel");
+        }
+        if (rne) average_pool_cl4_kernel<true><<<blocks4, 64, 0, s>>>(a);
+        else average_pool_cl4_kernel<false><<<blocks4, 64, 0, s>>>(a);
         return launch_check("average_pool_cl4_kernel");
     }
     const unsigned blocks = (unsigned)((a.p.total + kThreads - 1) / kThreads);

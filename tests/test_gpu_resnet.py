@@ -50,6 +50,10 @@ def test_pooling_ops(g, oracle):
     xi = rng.integers(-128, 128, size=(1, 16, 9, 9)).astype(np.int8)
     np.testing.assert_array_equal(g.host(g.ops.MaxPoolQ8(g.to_channels_last(g.dev(xi)), (2, 2), (2, 2), (1, 1))),
                                   oracle.max_pool_q8(xi, (2, 2), (2, 2), (1, 1)))
+    # windows of more than nine taps (the kernel's load groups), one tap, padded on every side
+    for k, st, pad in (((4, 5), (2, 3), (1, 2)), ((1, 1), (2, 2), (0, 0)), ((5, 5), (1, 1), (2, 2))):
+        np.testing.assert_array_equal(g.host(g.ops.MaxPoolQ8(g.to_channels_last(g.dev(xi)), k, st, pad)),
+                                      oracle.max_pool_q8(xi, k, st, pad), err_msg=str((k, st, pad)))
     want = oracle.average_pool_q8(x, 0.05, 30, (7, 7), (1, 1), (0, 0), 0.02, 7)
     np.testing.assert_array_equal(g.host(g.ops.AveragePoolQ8(g.to_channels_last(g.dev(x)), 0.05, 30, (7, 7), (1, 1), (0, 0),
                                                              0.02, 7)), want)
@@ -65,7 +69,9 @@ def test_pooling_ops(g, oracle):
 @pytest.mark.parametrize("case", [
     # N, C, H, W, kernel, stride, pad, count_include_pad
     (2, 32, 7, 7, 7, 1, 0, False), (1, 20, 9, 11, 3, 2, 1, False), (1, 8, 6, 6, 3, 1, 1, True), (1, 12, 10, 13, 9, 1, 0, False),
-    (2, 6, 5, 5, 2, 2, 0, False)])
+    (2, 6, 5, 5, 2, 2, 0, False),
+    # whole-image windows: 64 taps is the most the global-pool kernel takes, 81 goes the general way
+    (1, 8, 8, 8, 8, 1, 0, False), (1, 8, 9, 9, 9, 1, 0, False), (3, 4, 1, 1, 1, 1, 0, False)])
 def test_average_pool_layouts(g, oracle, case, xdt):
     """AveragePool between DequantizeLinear and QuantizeLinear: the four-channel channels-last
     kernel (also windows wider than its eight-tap groups, padding, both count modes, int8) and the
