@@ -629,11 +629,11 @@ void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
     pw->wd = nullptr;
 }
 
-// Depthwise 3x3 on int8 weights with zero weight zero points: paired weights and per-channel sums.
+// Depthwise 3x3 on int8 weights with zero weight zero points: packed filter rows and per-channel sums.
 struct DepthwiseState {
     int C = 0;
-    void* block = nullptr;  // one allocation: pairs | wsum
-    int32_t* pairs = nullptr;
+    void* block = nullptr;  // one allocation: rows | wsum
+    int32_t* rows = nullptr;
     int32_t* wsum = nullptr;
 };
 
@@ -644,17 +644,17 @@ bool weights_fit_depthwise(const chx_hip_tensor& w, int group) {
 
 int make_depthwise(const chx_hip_tensor& w, bool persistent, hipStream_t s, DepthwiseState* st) {
     const int C = (int)w.shape[0];
-    const size_t pairs_bytes = (size_t)(C / 16) * 5 * 16 * sizeof(int32_t);
-    const size_t total = pairs_bytes + (size_t)C * 4;
+    const size_t rows_bytes = (size_t)(C / 4) * 12 * sizeof(int32_t);
+    const size_t total = rows_bytes + (size_t)C * 4;
     void* p = nullptr;
     if (persistent) CHX_HIP_CALL(hipMalloc(&p, total));
     else CHX_PROPAGATE(scratch_alloc(&p, total, s));
     st->C = C;
     st->block = p;
     char* b = static_cast<char*>(p);
-    st->pairs = reinterpret_cast<int32_t*>(b);
-    st->wsum = reinterpret_cast<int32_t*>(b + pairs_bytes);
-    return pack_depthwise(w, st->pairs, st->wsum, s);
+    st->rows = reinterpret_cast<int32_t*>(b);
+    st->wsum = reinterpret_cast<int32_t*>(b + rows_bytes);
+    return pack_depthwise(w, st->rows, st->wsum, s);
 }
 
 void release_depthwise(DepthwiseState* st, bool persistent, hipStream_t s) {
@@ -737,8 +737,8 @@ int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
     const chx_hip_tensor& y = *c.y;
     if (!is_depthwise_layout(x) || !is_depthwise_layout(y))
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel needs channels-last 8-bit operands with 16-byte aligned pixels");
-    if (x.strides[3] * x.shape[3] >= (int64_t(1) << 31))
-        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: an input row spans 2 GiB or more");
+    if (x.strides[3] * x.shape[3] >= (int64_t(1) << 31) || y.strides[3] * y.shape[3] >= (int64_t(1) << 31))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: an input or output row spans 2 GiB or more");
     const bool xs = x.dtype == CHX_HIP_INT8;
     const int32_t zp_u = xs ? c.x_zp + 128 : c.x_zp;
     DepthwiseArgs a;
@@ -755,7 +755,7 @@ int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
     a.sh = c.p->stride_h; a.sw = c.p->stride_w; a.ph = c.p->pad_h_begin; a.pw = c.p->pad_w_begin;
     a.x_signed = xs ? 1 : 0;
     a.x_zp_u = zp_u;
-    a.pairs = st.pairs;
+    a.rows = st.rows;
     a.wsum = st.wsum;
     a.w_scale = c.w_scale;
     a.w_scale_len = c.w_scale_len;

@@ -15,7 +15,7 @@ struct DepthwiseArgs {
     int32_t N, C, H, W, OH, OW, sh, sw, ph, pw;
     int32_t x_signed;       // int8 activations: codes and zero point are shifted by 128
     int32_t x_zp_u;         // zero point in the unsigned range (zp, or zp + 128 for int8)
-    const int32_t* pairs;   // [C/16][5][16] paired weights (pack_depthwise)
+    const int32_t* rows;    // [C/4][3][4] filter rows as byte triples (pack_depthwise)
     const int32_t* wsum;    // [C] sum of the nine weights of a channel
     const float* w_scale;   // [w_scale_len]
     int32_t w_scale_len;    // 1 or C
@@ -25,11 +25,11 @@ struct DepthwiseArgs {
     QuantParams q;
     float inv_y_scale;
     float lo_folded;
-    int32_t ow_blocks;      // filled by the launcher
+    int32_t oh_blocks;      // filled by the launcher
     int64_t total;          // filled by the launcher
 };
 
-int pack_depthwise(const chx_hip_tensor& w, int32_t* pairs, int32_t* wsum, hipStream_t s);
+int pack_depthwise(const chx_hip_tensor& w, int32_t* rows, int32_t* wsum, hipStream_t s);
 int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s);
 
 }  // namespace chx

@@ -1,20 +1,22 @@
 // Depthwise 3x3 QLinearConv (group == C == OC, one filter per channel) on channels-last 8-bit
-// tensors.  Nine multiply-accumulates per output byte make this a memory-bound op; the work per
-// element is kept low by pairing filter taps: for each channel, the codes of taps (2p, 2p+1) are
-// gathered into one dword of two 16-bit lanes with a byte permute and multiplied against the
-// pre-paired weights with one v_dot2_i32_i16, so a 3x3 window costs five permutes and five dot
-// products instead of nine unpack-unpack-multiply-add sequences.
+// tensors.  Nine multiply-accumulates per output byte make this a memory-bound op, so the work per
+// byte has to be small:
+//   * a thread owns four consecutive channels (one dword per pixel) of one output column and walks
+//     down kRows output rows.  Consecutive lanes own consecutive channel groups, then consecutive
+//     pixels of the row: every load and store of a wavefront is one dense run of bytes, whatever
+//     the channel count.
+//   * per input row the thread loads the three dwords under the filter row and repacks them, per
+//     channel, into one dword [x(i,0), x(i,1), x(i,2), 0] with two byte permutes; one
+//     v_dot4_i32_i8 against [w(i,0), w(i,1), w(i,2), 0] is then a whole filter row.  The packed
+//     rows stay in registers while the window moves down: with stride 1 an output row costs one
+//     new input row (3 loads, 8 permutes, 12 dot products for its four bytes) instead of nine
+//     loads and nine unpack-multiply-add sequences per byte.
 //
-// A thread owns kCh consecutive channels (one 8-byte vector per pixel) and walks over
-// kDwPixels output pixels of one output row; consecutive lanes own consecutive channel groups,
-// so every load and store of a wavefront covers whole pixels.  Weights, scales and accumulator
-// seeds stay in registers across the pixels; the register footprint is kept small enough for
-// five or more waves per SIMD, which is what hides the load latency.
-//
-// Arithmetic: int8 activations are shifted to the unsigned range by flipping the top bit
-// (code + 128, zero point + 128); padding taps read the zero point, which makes them contribute
-// (zp - zp) * w = 0; the accumulator starts at  -zp * sum_t w[c][t] (+ bias in ONNX mode), so the
-// int32 sum is exactly  sum_t (x - zp) * w  and the epilogue is the shared requantization.
+// Arithmetic: the codes are brought to the signed range (uint8: flip the top bit = code - 128;
+// int8: as stored), the zero point likewise; padding taps read the zero point, which makes them
+// contribute (zp - zp) * w = 0; the accumulator starts at  -zp_signed * sum_t w[c][t]  (+ bias in
+// ONNX mode), so the int32 sum is exactly  sum_t (x - zp) * w  and the epilogue is the shared
+// requantization.
 #include <type_traits>
 
 #include "contract.h"
@@ -25,171 +27,221 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef short v2s __attribute__((ext_vector_type(2)));
 
-constexpr int kDwPixels = 4;
-constexpr int kTaps = 9;
-constexpr int kPairs = 5;
 
-// w [C][1][3][3] (any strides) -> pairs [C/16][kPairs][16] dwords (lo16 = tap 2p, hi16 = tap 2p+1 or 0)
-// and wsum[c].  One thread per channel.
+// w [C][1][3][3] (any strides) -> rows [C/4][3][4] dwords, dword (i, e) of a channel group =
+// bytes [w(i,0), w(i,1), w(i,2), 0] of channel 4*group + e, and wsum[c].  One thread per channel.
 __global__ __launch_bounds__(256) void pack_depthwise_kernel(
-        const char* __restrict__ w, int64_t s_oc, int64_t s_kh, int64_t s_kw, int C, int32_t* __restrict__ pairs,
+        const char* __restrict__ w, int64_t s_oc, int64_t s_kh, int64_t s_kw, int C, int32_t* __restrict__ rows,
         int32_t* __restrict__ wsum) {
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    int32_t t[kTaps + 1];
     int32_t sum = 0;
-    for (int i = 0; i < kTaps; ++i) {
-        t[i] = *reinterpret_cast<const int8_t*>(w + c * s_oc + (i / 3) * s_kh + (i % 3) * s_kw);
-        sum += t[i];
+    for (int i = 0; i < 3; ++i) {
+        uint32_t word = 0;
+        for (int j = 0; j < 3; ++j) {
+            const int32_t t = *reinterpret_cast<const int8_t*>(w + c * s_oc + i * s_kh + j * s_kw);
+            sum += t;
+            word |= ((uint32_t)t & 0xffu) << (8 * j);
+        }
+        rows[(c / 4) * 12 + i * 4 + (c % 4)] = (int32_t)word;
     }
-    t[kTaps] = 0;
-    for (int p = 0; p < kPairs; ++p)
-        pairs[((c / 16) * kPairs + p) * 16 + (c % 16)] = (t[2 * p] & 0xffff) | (t[2 * p + 1] << 16);
     wsum[c] = sum;
 }
 
-constexpr int kCh = 8;           // channels per thread
-constexpr int kDw = kCh / 4;     // dwords per pixel vector
-typedef int vxi __attribute__((ext_vector_type(kDw)));
+// kStep: vertical stride 1 or 2 (the packed input rows shared between neighbouring output rows
+// are kept), 0: any stride (every output row loads its three input rows).
+// kPath: 0 any 8-bit type and rounding; 1 uint8 in the reference's rounding (floor_sat_u8x4);
+// 2 the same with a lower bound above 0 (a folded Relu).  Chosen by the launcher, so that the
+// row loop has no branches and the loads of a whole strip are in flight together.
+// Output rows per thread.  More rows spread the per-thread set-up (index arithmetic, masks, filter
+// rows and constants) and the two halo rows over more outputs, at the price of registers for the
+// loads in flight: stride 1 takes 14 rows when the output height is a multiple of 14 (224 / 2^k
+// images), otherwise 8.
+constexpr int rows_per_thread(int step, bool tall) { return step == 1 ? (tall ? 14 : 8) : step == 2 ? 4 : 1; }
+constexpr int kDwThreads = 64;  // small groups: (output columns x channel groups) of a row is rarely a multiple of 256
+template <bool kRne, bool kFloatBias, int kStep, int kPath, bool kTall>
+__global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs a) {
+    constexpr int kRows = rows_per_thread(kStep, kTall);
+    constexpr int kInRows = kStep == 1 ? kRows + 2 : kStep == 2 ? 2 * kRows + 1 : 3;
+    // grid: x over (output column, channel group) of one strip of output rows, y the strip, z the image
+    const uint32_t idx = blockIdx.x * kDwThreads + threadIdx.x;
+    const uint32_t cgs = (uint32_t)a.C >> 2;
+    if (idx >= (uint32_t)a.OW * cgs) return;
+    const int ow = (int)(idx / cgs);
+    const int cg = (int)(idx - (uint32_t)ow * cgs);
+    const int ohb = blockIdx.y;
+    const int n = blockIdx.z;
+    const int c0 = cg * 4;
 
-template <bool kRne, bool kFloatBias, bool kXSigned>
-__global__ __launch_bounds__(256) void depthwise3x3_kernel(DepthwiseArgs a) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int cgs = a.C / kCh;
-    if (idx >= a.total) return;
-    const int cg = (int)(idx % cgs);
-    int64_t rest = idx / cgs;
-    const int owb = (int)(rest % a.ow_blocks);
-    rest /= a.ow_blocks;
-    const int oh = (int)(rest % a.OH);
-    const int n = (int)(rest / a.OH);
-    const int c0 = cg * kCh;
-
-    // pairs are stored per group of 16 channels: [c0 / 16][pair][c0 % 16 ...]
-    int32_t wp[kPairs][kCh];
-    const int32_t* pbase = a.pairs + (int64_t)(c0 / 16) * kPairs * 16 + (c0 % 16);
-#pragma unroll
-    for (int p = 0; p < kPairs; ++p)
-#pragma unroll
-        for (int d = 0; d < kDw; ++d) {
-            const v4i v = *reinterpret_cast<const v4i*>(pbase + p * 16 + d * 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) wp[p][d * 4 + e] = v[e];
-        }
-    // per channel: accumulator seed -zp * sum_t w (+ int32 bias, ONNX mode), scale x_scale * w_scale,
-    // float bias (reference mode)
-    float sc[kCh], fb[kCh];
-    int32_t seed[kCh];
-#pragma unroll
-    for (int d = 0; d < kDw; ++d) {
-        const v4i ws4 = *reinterpret_cast<const v4i*>(a.wsum + c0 + d * 4);
-        v4i b4 = {0, 0, 0, 0};
-        if (a.bias) b4 = *reinterpret_cast<const v4i*>(a.bias + c0 + d * 4);
-        v4f s4;
-        if (a.w_scale_len > 1) s4 = *reinterpret_cast<const v4f*>(a.w_scale + c0 + d * 4);
-        else s4 = v4f{a.w_scale[0], a.w_scale[0], a.w_scale[0], a.w_scale[0]};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            seed[d * 4 + e] = -a.x_zp_u * ws4[e] + (kFloatBias ? 0 : b4[e]);
-            sc[d * 4 + e] = a.x_scale * s4[e];
-            fb[d * 4 + e] = kFloatBias ? (float)b4[e] : 0.f;
-        }
-    }
-    const bool u8_reference = !kRne && a.q.lo == 0.f && a.q.hi == 255.f, lower_bound = a.lo_folded > 0.f;  // uniform
-    const int fill = (int)(((uint32_t)(a.x_zp_u & 0xff)) * 0x01010101u);  // the zero point, already in the unsigned range
-    const char* xn = a.x + (int64_t)n * a.x_n_stride + c0;
-    char* yrow = a.y + (int64_t)n * a.y_n_stride + (int64_t)oh * a.y_h_stride + c0;
-    const int ih0 = oh * a.sh - a.ph;
-    // the three input rows of this output row, clamped into the image so that every load is
+    v4i wq[3];
+    float sc[4], fb[4];
+    int32_t seed[4];
+    const uint32_t flip = a.x_signed ? 0u : 0x80808080u;                        // stored code -> signed range
+    const uint32_t fill = (uint32_t)((a.x_zp_u ^ 0x80) & 0xff) * 0x01010101u;   // the zero point in the signed range
+    // addresses = a base that is the same for the whole work-group (image, row: scalar registers)
+    // + a 32-bit offset per lane (column, channel group)
+    const char* xn = a.x + (int64_t)n * a.x_n_stride;
+    char* yn = a.y + (int64_t)n * a.y_n_stride;
+    const uint32_t y_off = (uint32_t)ow * (uint32_t)a.y_w_stride + (uint32_t)c0;  // the host checked that a row spans less than 2^31 bytes
+    // the three input columns of this output column, clamped into the image so that every load is
     // valid; what a tap outside the image contributes is replaced by the zero point afterwards
-    const char* rowp[3];
-    bool row_ok[3];
+    const int iw0 = ow * a.sw - a.pw;
+    uint32_t coff[3], col_mask[3];
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
-        const int ih = ih0 + i;
-        row_ok[i] = (unsigned)ih < (unsigned)a.H;
-        rowp[i] = xn + (int64_t)min(max(ih, 0), a.H - 1) * a.x_h_stride;
+    for (int j = 0; j < 3; ++j) {
+        const int iw = iw0 + j;
+        col_mask[j] = (unsigned)iw < (unsigned)a.W ? ~0u : 0u;
+        coff[j] = (uint32_t)min(max(iw, 0), a.W - 1) * (uint32_t)a.x_w_stride + (uint32_t)c0;
     }
-    const uint32_t wstride = (uint32_t)a.x_w_stride;  // the host checked that a row spans less than 2^31 bytes
-
-    for (int p = 0; p < kDwPixels; ++p) {
-        const int ow = owb * kDwPixels + p;
-        if (ow >= a.OW) break;
-        const int iw0 = ow * a.sw - a.pw;
-        vxi x[kTaps + 1];
+    // the three dwords of input row ih under the filter, in the signed range, taps outside the image
+    // replaced by the zero point
+    auto load_row = [&](int ih, uint32_t (&v)[3]) {
+        const uint32_t row_mask = (unsigned)ih < (unsigned)a.H ? ~0u : 0u;
+        const char* rowp = xn + (int64_t)min(max(ih, 0), a.H - 1) * a.x_h_stride;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            const int iw = iw0 + j;
-            const bool col_ok = (unsigned)iw < (unsigned)a.W;
-            const uint32_t off = (uint32_t)min(max(iw, 0), a.W - 1) * wstride;
-#pragma unroll
-            for (int i = 0; i < 3; ++i) {
-                vxi v = *reinterpret_cast<const vxi*>(rowp[i] + off);
-                if (kXSigned) v ^= (int)0x80808080;
-                const bool ok = col_ok && row_ok[i];
-#pragma unroll
-                for (int d = 0; d < kDw; ++d) v[d] = ok ? v[d] : fill;
-                x[i * 3 + j] = v;
-            }
+            // bit arithmetic, not a conditional: as a select of the loaded value the compiler
+            // turns it into a branch around the load, and every load then waits for the one before
+            const uint32_t m = row_mask & col_mask[j];
+            v[j] = ((*reinterpret_cast<const uint32_t*>(rowp + coff[j]) ^ flip) & m) | (fill & ~m);
         }
+    };
+    // ... as four dwords, one per channel: bytes [x(ih, iw0), x(ih, iw0+1), x(ih, iw0+2), 0]
+    auto pack_row = [&](const uint32_t (&v)[3], uint32_t (&rp)[4]) {
 #pragma unroll
-        for (int d = 0; d < kDw; ++d) x[kTaps][d] = 0;
-        vxi o;
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t t = __builtin_amdgcn_perm(v[1], v[0], 0x0c0c0000u | ((4u + e) << 8) | (uint32_t)e);  // [v0.e, v1.e, 0, 0]
+            rp[e] = __builtin_amdgcn_perm(v[2], t, 0x0c000100u | ((4u + e) << 16));                               // [v0.e, v1.e, v2.e, 0]
+        }
+    };
+    auto finish = [&](int oh, const uint32_t (&r0)[4], const uint32_t (&r1)[4], const uint32_t (&r2)[4]) {
+        int32_t code[4];
+        float pre[4];
 #pragma unroll
-        for (int d = 0; d < kDw; ++d) {
-            int32_t code[4];
-            float pre[4];
+        for (int e = 0; e < 4; ++e) {
+            // the three-operand form: no copy of the seed into the accumulator first
+            int32_t acc;
+            asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(acc) : "v"(r0[e]), "v"(wq[0][e]), "v"(seed[e]));
+            acc = __builtin_amdgcn_sdot4((int)r1[e], wq[1][e], acc, false);
+            acc = __builtin_amdgcn_sdot4((int)r2[e], wq[2][e], acc, false);
+            float v = (float)acc * sc[e];
+            if (kFloatBias) v = v + fb[e];
+            // uint8 in the reference's rounding: clamp, conversion and packing in floor_sat_u8x4
+            if (kPath == 2) pre[e] = quantize_prefloor_u8<true>(v, a.q, a.inv_y_scale, a.lo_folded);
+            else if (kPath == 1) pre[e] = quantize_prefloor_u8<false>(v, a.q, a.inv_y_scale, 0.f);
+            else code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
+        }
+        const uint32_t o = kPath ? floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : pack4(code[0], code[1], code[2], code[3]);
+        if (oh < a.OH) *reinterpret_cast<uint32_t*>(yn + (int64_t)oh * a.y_h_stride + y_off) = o;
+    };
+
+    // filter rows and per-channel constants; requested after the strip's input rows so that all of it is in flight together
+    auto load_constants = [&]() {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) wq[i] = *reinterpret_cast<const v4i*>(a.rows + (int64_t)cg * 12 + i * 4);
+        // per channel: accumulator seed -zp * sum_t w (+ int32 bias, ONNX mode), scale x_scale * w_scale,
+        // float bias (reference mode)
+        {
+            const v4i ws4 = *reinterpret_cast<const v4i*>(a.wsum + c0);
+            v4i b4 = {0, 0, 0, 0};
+            if (a.bias) b4 = *reinterpret_cast<const v4i*>(a.bias + c0);
+            v4f s4;
+            if (a.w_scale_len > 1) s4 = *reinterpret_cast<const v4f*>(a.w_scale + c0);
+            else s4 = v4f{a.w_scale[0], a.w_scale[0], a.w_scale[0], a.w_scale[0]};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int ch = d * 4 + e;
-                int32_t acc = seed[ch];
-#pragma unroll
-                for (int q = 0; q < kPairs; ++q) {
-                    // bytes: [x(2q).b_e, 0, x(2q+1).b_e, 0]
-                    const uint32_t sel = 0x0c000c00u | (uint32_t)e | ((uint32_t)(4 + e) << 16);
-                    const uint32_t xp = __builtin_amdgcn_perm((uint32_t)x[2 * q + 1][d], (uint32_t)x[2 * q][d], sel);
-                    acc = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, xp), __builtin_bit_cast(v2s, wp[q][ch]), acc, false);
-                }
-                float v = (float)acc * sc[ch];
-                if (kFloatBias) v = v + fb[ch];
-                // uint8 in the reference's rounding: clamp, conversion and packing in floor_sat_u8x4
-                if (u8_reference) pre[e] = lower_bound ? quantize_prefloor_u8<true>(v, a.q, a.inv_y_scale, a.lo_folded)
-                                                        : quantize_prefloor_u8<false>(v, a.q, a.inv_y_scale, 0.f);
-                else code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
+                seed[e] = (128 - a.x_zp_u) * ws4[e] + (kFloatBias ? 0 : b4[e]);
+                sc[e] = a.x_scale * s4[e];
+                fb[e] = kFloatBias ? (float)b4[e] : 0.f;
             }
-            o[d] = u8_reference ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
         }
-        *reinterpret_cast<vxi*>(yrow + (int64_t)ow * a.y_w_stride) = o;
+    };
+    const int oh0 = ohb * kRows;
+    uint32_t raw[kInRows][3], rp[3][4];
+    if constexpr (kStep == 1) {
+        // output row oh0 + p reads input rows ih0 + p .. ih0 + p + 2: two of them are already packed
+        const int ih0 = oh0 - a.ph;
+#pragma unroll
+        for (int r = 0; r < kInRows; ++r) load_row(ih0 + r, raw[r]);
+        load_constants();
+        pack_row(raw[0], rp[0]);
+        pack_row(raw[1], rp[1]);
+#pragma unroll
+        for (int p = 0; p < kRows; ++p) {
+            pack_row(raw[p + 2], rp[(p + 2) % 3]);
+            finish(oh0 + p, rp[p % 3], rp[(p + 1) % 3], rp[(p + 2) % 3]);
+        }
+    } else if constexpr (kStep == 2) {
+        // output row oh0 + p reads input rows ih0 + 2p .. ih0 + 2p + 2: the last one is the next row's first
+        const int ih0 = oh0 * 2 - a.ph;
+#pragma unroll
+        for (int r = 0; r < kInRows; ++r) load_row(ih0 + r, raw[r]);
+        load_constants();
+        pack_row(raw[0], rp[0]);
+#pragma unroll
+        for (int p = 0; p < kRows; ++p) {
+            const int first = (p & 1) ? 2 : 0, last = 2 - first;
+            pack_row(raw[2 * p + 1], rp[1]);
+            pack_row(raw[2 * p + 2], rp[last]);
+            finish(oh0 + p, rp[first], rp[1], rp[last]);
+        }
+    } else {
+        const int ih0 = oh0 * a.sh - a.ph;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) load_row(ih0 + r, raw[r]);
+        load_constants();
+#pragma unroll
+        for (int r = 0; r < 3; ++r) pack_row(raw[r], rp[r]);
+        finish(oh0, rp[0], rp[1], rp[2]);
     }
 }
 
 }  // namespace
 
-int pack_depthwise(const chx_hip_tensor& w, int32_t* pairs, int32_t* wsum, hipStream_t s) {
+int pack_depthwise(const chx_hip_tensor& w, int32_t* rows, int32_t* wsum, hipStream_t s) {
     const int C = (int)w.shape[0];
     pack_depthwise_kernel<<<(C + 255) / 256, 256, 0, s>>>(
-            static_cast<const char*>(w.data), w.strides[0], w.strides[2], w.strides[3], C, pairs, wsum);
+            static_cast<const char*>(w.data), w.strides[0], w.strides[2], w.strides[3], C, rows, wsum);
     return launch_check("pack_depthwise_kernel");
 }
 
 int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
-    a.ow_blocks = (a.OW + kDwPixels - 1) / kDwPixels;
-    a.total = (int64_t)a.N * a.OH * a.ow_blocks * (a.C / kCh);
+    const int step = a.sh == 1 ? 1 : a.sh == 2 ? 2 : 0;
+    const bool tall = step == 1 && a.OH % 14 == 0;
+    const int rows = rows_per_thread(step, tall);
+    a.oh_blocks = (a.OH + rows - 1) / rows;
+    a.total = (int64_t)a.N * a.oh_blocks * a.OW * (a.C / 4);
     if (a.total == 0) return CHX_HIP_OK;
-    const unsigned blocks = (unsigned)((a.total + 255) / 256);
+    if (a.oh_blocks > 65535 || a.N > 65535 || (int64_t)a.OW * (a.C / 4) >= (int64_t(1) << 31))
+        CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: more than 65535 images or row strips, or a row of 2^31 channel groups");
+    const dim3 blocks((unsigned)(((int64_t)a.OW * (a.C / 4) + kDwThreads - 1) / kDwThreads), (unsigned)a.oh_blocks, (unsigned)a.N);
     const bool fbias = a.bias != nullptr && a.float_bias != 0;
-    const bool xs = a.x_signed != 0;
-#define CHX_DW(RN, FB, XS) depthwise3x3_kernel<RN, FB, XS><<<blocks, 256, 0, s>>>(a)
+    const bool u8_reference = !rne && a.q.lo == 0.f && a.q.hi == 255.f;
+    const int path = !u8_reference ? 0 : a.lo_folded > 0.f ? 2 : 1;
+#define CHX_DW_P(RN, FB, ST, TL)                                                                    \
+    do {                                                                                            \
+        if (path == 0) depthwise3x3_kernel<RN, FB, ST, 0, TL><<<blocks, kDwThreads, 0, s>>>(a);     \
+        else if (RN) CHX_FAIL(CHX_HIP_ERUNTIME, "depthwise: conversion path");                      \
+        else if (path == 1) depthwise3x3_kernel<false, FB, ST, 1, TL><<<blocks, kDwThreads, 0, s>>>(a); \
+        else depthwise3x3_kernel<false, FB, ST, 2, TL><<<blocks, kDwThreads, 0, s>>>(a);            \
+    } while (0)
+#define CHX_DW_S(RN, FB)                               \
+    do {                                               \
+        if (tall) CHX_DW_P(RN, FB, 1, true);           \
+        else if (step == 1) CHX_DW_P(RN, FB, 1, false); \
+        else if (step == 2) CHX_DW_P(RN, FB, 2, false); \
+        else CHX_DW_P(RN, FB, 0, false);               \
+    } while (0)
     if (rne) {
-        if (fbias) { if (xs) CHX_DW(true, true, true); else CHX_DW(true, true, false); }
-        else { if (xs) CHX_DW(true, false, true); else CHX_DW(true, false, false); }
+        if (fbias) CHX_DW_S(true, true);
+        else CHX_DW_S(true, false);
     } else {
-        if (fbias) { if (xs) CHX_DW(false, true, true); else CHX_DW(false, true, false); }
-        else { if (xs) CHX_DW(false, false, true); else CHX_DW(false, false, false); }
+        if (fbias) CHX_DW_S(false, true);
+        else CHX_DW_S(false, false);
     }
-#undef CHX_DW
+#undef CHX_DW_S
+#undef CHX_DW_P
     return launch_check("depthwise3x3_kernel");
 }
 

@@ -234,12 +234,15 @@ def test_errors(g):
 @pytest.mark.parametrize("xdt", [np.uint8, np.int8])
 @pytest.mark.parametrize("case", [
     # N, C, H, W, stride, pad
-    (2, 32, 9, 10, 1, 1), (1, 96, 13, 12, 2, 1), (2, 16, 7, 7, 1, 0), (1, 144, 5, 6, 2, 0), (1, 48, 4, 4, 1, 1)])
+    (2, 32, 9, 10, 1, 1), (1, 96, 13, 12, 2, 1), (2, 16, 7, 7, 1, 0), (1, 144, 5, 6, 2, 0), (1, 48, 4, 4, 1, 1),
+    # 14 and 28 output rows (the 14-row strips), a stride the row reuse does not cover, strides that differ
+    (1, 16, 14, 5, 1, 1), (1, 16, 30, 3, 1, 0), (1, 32, 11, 10, 3, 1), (1, 16, 12, 9, (2, 1), 1), (1, 16, 9, 12, (1, 3), 1)])
 def test_depthwise_qlinear_conv(g, oracle, case, xdt):
-    """Depthwise 3x3 on channels-last operands (the paired-tap kernel), stateless call and plan,
-    both bias modes, fused Relu, ONNX rounding; NCHW operands take the generic kernel and must
+    """Depthwise 3x3 on channels-last operands (the row-packing kernel), stateless call and plan,
+    both bias modes, fused Relu in both roundings; NCHW operands take the generic kernel and must
     give the same bytes."""
     N, C, H, W, stride, pad = case
+    stride = stride if isinstance(stride, tuple) else (stride, stride)
     rng = np.random.default_rng(31)
     x = rand_q(rng, (N, C, H, W), xdt)
     w = rng.integers(-127, 128, size=(C, 1, 3, 3)).astype(np.int8)
@@ -248,7 +251,7 @@ def test_depthwise_qlinear_conv(g, oracle, case, xdt):
     bias = rng.integers(-300, 301, size=C).astype(np.int32)
     xz = 117 if xdt == np.uint8 else -11
     ys = np.float32(0.02 * 0.01 * 128 * 64 * 3 / 40)
-    kw = dict(strides=(stride, stride), pads=(pad, pad), group=C)
+    kw = dict(strides=stride, pads=(pad, pad), group=C)
     for bias_mode, flags in ((oracle.BIAS_ONNX_INT32, g.capi.BIAS_ONNX_INT32), (oracle.BIAS_REFERENCE_FLOAT, 0)):
         want = oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, 120, np.uint8, bias=bias, bias_mode=bias_mode, **kw)
         assert want.min() < want.max()
@@ -269,6 +272,13 @@ def test_depthwise_qlinear_conv(g, oracle, case, xdt):
     got = g.ops.QLinearConv(g.to_channels_last(g.dev(x)), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, -5, g.dev(bias),
                             zero_point_dtype=torch.int8, flags=fl, **kw)
     np.testing.assert_array_equal(g.host(got), want)
+    # uint8 output in the reference's rounding with the Relu folded into the lower bound
+    want = np.maximum(oracle.qlinear_conv_int(x, 0.02, xz, w, ws, wz, ys, 120, np.uint8, bias=bias, bias_mode=oracle.BIAS_REFERENCE_FLOAT, **kw),
+                      120).astype(np.uint8)
+    got = g.ops.QLinearConv(g.to_channels_last(g.dev(x)), 0.02, xz, g.dev(w), g.dev(ws), g.dev(wz), ys, 120, g.dev(bias),
+                            flags=g.capi.FUSE_RELU, **kw)
+    np.testing.assert_array_equal(g.host(got), want)
+    assert (want > 120).any() and (want == 120).any()
 
 
 @pytest.mark.parametrize("xdt", [np.uint8, np.int8])
