@@ -328,7 +328,7 @@ def _to_numpy(desc):
                                                  ctypes.c_size_t(span), None))
     view = np.lib.stride_tricks.as_strided(buf[:dt.itemsize].view(dt), shape=shape, strides=strides) if span else \
         np.empty(shape, dt)
-    return np.ascontiguousarray(view)
+    return np.array(view, order="C")  # a copy that keeps 0-d arrays 0-d (ascontiguousarray would make them 1-d)
 
 
 class Program:

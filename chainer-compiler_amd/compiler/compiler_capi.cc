@@ -93,6 +93,7 @@ std::unique_ptr<Graph> Transform(const void* model, size_t size, const char* opt
     *xmodel = ParseOnnxModel(std::string(static_cast<const char*>(model), size));
     std::unique_ptr<Graph> graph = Graph::FromOnnx(xmodel->graph);
     const Options o = ParseOptions(options);
+    ExpandDynamicQuantizeLinear(graph.get());
     if (o.quantize) Quantize(o.q, graph.get());
     InferDtypes(graph.get());
     if (o.fuse == "hip") FuseHipOperations(graph.get());

@@ -296,6 +296,14 @@ private:
                                    IntIn(n.GetInt("count_include_pad", 0))});
             }
             inst->outputs.push_back(-1);  // the backward context is not kept
+        } else if (op == "Clip" && nin >= 1 && nin <= 3) {
+            // compiler/chxvm/simple_node_emitter.cc:506-512: bounds as attributes or as operands
+            if (nin == 1) {
+                simple("StaticClip", {ArrayIn(Operand(n, 0)), FloatIn(n.GetFloat("max", 3.4028234663852886e38f)),
+                                      FloatIn(n.GetFloat("min", -3.4028234663852886e38f))});
+            } else {
+                simple(op, {ArrayIn(Operand(n, 0)), ScalarIn(Operand(n, 1, true), true), ScalarIn(Operand(n, 2, true), true)});
+            }
         } else if (op == "Max" || op == "Min") {
             std::vector<int> ins;
             for (size_t i = 0; i < nin; ++i) ins.push_back(Operand(n, i));
@@ -309,7 +317,7 @@ private:
             CHECK(to != kUnknown) << n.ToString() << ": unsupported target type " << n.GetInt("to", 0);
             simple(op, {ArrayIn(Operand(n, 0)), IntIn(to)});
         } else if (op == "Identity" || op == "Neg" || op == "Exp" || op == "Tanh" || op == "Sigmoid" || op == "Relu" || op == "Abs" ||
-                   op == "Floor") {
+                   op == "Floor" || op == "Round") {
             CHECK_EQ(1UL, nin) << n.ToString();
             simple(op, {ArrayIn(Operand(n, 0))});
         } else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div") {

@@ -164,7 +164,7 @@ int FuseElementwiseOperations(Graph* graph) {
 }
 
 int FuseHipOperations(Graph* graph) {
-    static const std::set<std::string> float_ops = {"Identity", "Add", "Sub", "Mul", "Div", "Neg", "Tanh", "Sigmoid", "Exp", "Relu", "Abs", "Floor"};
+    static const std::set<std::string> float_ops = {"Identity", "Add", "Sub", "Mul", "Div", "Neg", "Tanh", "Sigmoid", "Exp", "Relu", "Abs", "Floor", "Round"};
     auto constant_operands = [](const Node& node, size_t first) {
         for (size_t i = first; i < node.inputs().size(); ++i) {
             if (node.input(i)->IsNull()) continue;
@@ -306,7 +306,7 @@ std::string BuildHipProgram(const Node& group, std::vector<int>* used_inputs) {
         const std::string& op = node->op_type();
         CDtype out_dtype = kFloat32;
         if (op == "Identity" || op == "Neg" || op == "Tanh" || op == "Sigmoid" || op == "Exp" || op == "Relu" || op == "Abs" ||
-            op == "Floor") {
+            op == "Floor" || op == "Round") {
             os << out << " = " << op << " " << ins[0] << "\n";
         } else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div" || op == "Max" || op == "Min") {
             CHECK_EQ(2UL, ins.size()) << node->ToString();

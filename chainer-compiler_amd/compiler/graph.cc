@@ -544,7 +544,7 @@ void InferDtypes(Graph* graph) {
             }
             return false;
         };
-        static const std::set<std::string> unary = {"Identity", "Neg", "Abs", "Floor", "Exp", "Tanh", "Sigmoid", "Relu", "Cast", "Clip",
+        static const std::set<std::string> unary = {"Identity", "Neg", "Abs", "Floor", "Round", "Exp", "Tanh", "Sigmoid", "Relu", "Cast", "Clip",
                                                     "QuantizeLinear", "DequantizeLinear"};
         static const std::set<std::string> binary = {"Add", "Sub", "Mul", "Div", "Max", "Min"};
         std::vector<int64_t> dims;

@@ -230,4 +230,40 @@ bool Quantize(const QuantizationOptions& opts, Graph* graph) {
     return result;
 }
 
+int ExpandDynamicQuantizeLinear(Graph* graph) {
+    int replaced = 0;
+    for (Node* node : graph->GetLiveNodes()) {
+        if (node->op_type() != "DynamicQuantizeLinear") continue;
+        CHECK_EQ(1UL, node->inputs().size()) << node->ToString();
+        CHECK_EQ(3UL, node->outputs().size()) << node->ToString();
+        Value* x = node->input(0);
+        Value* const y = node->output(0);
+        Value* const y_scale = node->output(1);
+        Value* const y_zero_point = node->output(2);
+        GraphBuilder gb(graph, "ExpandDynamicQuantizeLinear", y);
+        graph->DetachNode(node);  // its outputs get new producers below
+        auto reduce = [&](const char* op) {
+            Value* v = gb.Op(op, {x});
+            v->producer()->SetInt("keepdims", 0);
+            return v;
+        };
+        Value* q_min = gb.Const(ScalarTensor(0.f));
+        Value* q_max = gb.Const(ScalarTensor(255.f));
+        Value* x_min_adjusted = gb.Op("Min", {reduce("ReduceMin"), q_min});
+        Value* x_max_adjusted = gb.Op("Max", {reduce("ReduceMax"), q_min});
+        Value* scale = gb.Op("Div", {gb.Op("Sub", {x_max_adjusted, x_min_adjusted}), q_max});
+        Value* initial_zero_point = gb.Op("Sub", {q_min, gb.Op("Div", {x_min_adjusted, scale})});
+        Value* rounded = gb.Op("Round", {gb.Op("Clip", {initial_zero_point, q_min, q_max})});
+        Value* zero_point = gb.Op("Cast", {rounded});
+        zero_point->producer()->SetInt("to", DtypeToOnnx(kUInt8));
+        zero_point->set_type(Type(kUInt8, {}));
+        scale->set_type(Type(kFloat32, {}));
+        gb.Op("Identity", {scale}, y_scale);
+        gb.Op("Identity", {zero_point}, y_zero_point);
+        gb.Op("QuantizeLinear", {x, scale, zero_point}, y);
+        ++replaced;
+    }
+    return replaced;
+}
+
 }  // namespace chainer_compiler

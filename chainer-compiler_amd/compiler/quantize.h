@@ -35,6 +35,13 @@ struct QuantizationOptions {
 // Returns whether anything was rewritten.
 bool Quantize(const QuantizationOptions& opts, Graph* graph);
 
+// Replaces every DynamicQuantizeLinear node by the body of the ONNX function of that name
+// (what the FunctionExpander of compiler/simplifier.cc:825-888 does with the schema's function,
+// enabled by configs/chxvm.json:55-57): ReduceMin/ReduceMax, the range widened to contain 0,
+// scale = range / 255, zero point = Cast(Round(Clip(0 - min / scale, 0, 255))), QuantizeLinear.
+// Returns the number of nodes replaced.
+int ExpandDynamicQuantizeLinear(Graph* graph);
+
 // One tensor quantized the way the pass quantizes weights (compiler/quantize.cc:68-89), exposed for tests.
 struct QuantizedData {
     float rmin, rmax, scale;

@@ -21,7 +21,7 @@
 //   in  <name>:<dtype> ...            dtype: float32 | uint8 | int8
 //   <name> = <Op> <operand> ...       operands are earlier names or, where noted, literals
 //   out <name>:<dtype> ...
-// Ops: Identity a | Neg a | Abs a | Floor a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
+// Ops: Identity a | Neg a | Abs a | Floor a | Round a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
 //      Tanh a | Sigmoid a | Exp a | Relu a | Clip a <lo> <hi> | Const <value>
 //      QuantizeLinear a <scale> <zero_point> <uint8|int8> [rne]   (float -> 8-bit code)
 //      DequantizeLinear q <scale> <zero_point>                    (8-bit code -> float)
@@ -226,6 +226,11 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
             os << "  const float " << o << " = __builtin_floorf(" << a << ");\n";
+        } else if (s.op == "Round") {
+            // to the nearest integer, ties to even (RoundOp, runtime/ops/quantize.cc:148-151)
+            CHX_PROPAGATE(need(1));
+            CHX_PROPAGATE(val(0, 'f', &a));
+            os << "  const float " << o << " = __builtin_rintf(" << a << ");\n";
         } else if (s.op == "Tanh") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));

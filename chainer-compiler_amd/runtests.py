@@ -11,9 +11,12 @@ import subprocess
 import sys
 import time
 
-# the quantized-path cases of the reference's node-test list (scripts/runtests.py:556-563)
+# the quantized-path cases of the reference's node-test list (scripts/runtests.py:556-564,577-582)
 NODE_TESTS = ["test_quantizelinear", "test_dequantizelinear", "test_qlinearmatmul_2D", "test_qlinearmatmul_3D",
-              "test_qlinearconv", "test_convinteger_with_padding", "test_basic_convinteger", "test_matmulinteger"]
+              "test_qlinearconv", "test_convinteger_with_padding", "test_basic_convinteger", "test_matmulinteger",
+              "test_round", "test_dynamicquantizelinear", "test_dynamicquantizelinear_max_adjusted", "test_dynamicquantizelinear_min_adjusted",
+              "test_dynamicquantizelinear_expanded", "test_dynamicquantizelinear_max_adjusted_expanded",
+              "test_dynamicquantizelinear_min_adjusted_expanded"]
 
 
 def main(argv=None):

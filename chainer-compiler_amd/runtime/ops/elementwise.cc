@@ -2,6 +2,8 @@
 // chainer-compiler tree): result shape = broadcast of the inputs, outputs allocated here, the
 // kernel generated, compiled, cached and launched behind chx_hip_elementwise.  The inputs are
 // handed over as they are; nothing is broadcast or copied first.
+#include <cstdio>
+#include <cstring>
 #include <sstream>
 
 #include "../gen/gen_chxvm_ops.h"
@@ -144,6 +146,44 @@ chainerx::Array AbsOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
 }
 chainerx::Array FloorOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
     return RunFloatOp("Floor", {x});
+}
+// ties to even (runtime/ops/quantize.cc:148-151, SlowRound)
+chainerx::Array RoundOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return RunFloatOp("Round", {x});
+}
+
+namespace {
+
+// Minimum(Maximum(x, lo), hi) with the bounds written into the program (runtime/ops/math.cc:140-154);
+// a missing bound is the end of the float range, which changes no finite value
+chainerx::Array ClipTo(const chainerx::Array& x, float lo, float hi) {
+    CHECK(x.dtype() == chainerx::Dtype::kFloat32) << "Clip runs on float32 arrays on the hip backend, got " << x.dtype();
+    uint32_t lo_bits, hi_bits;
+    std::memcpy(&lo_bits, &lo, 4);
+    std::memcpy(&hi_bits, &hi, 4);
+    char line[96];
+    std::snprintf(line, sizeof(line), "y = Clip a 0x%08x 0x%08x\n", lo_bits, hi_bits);
+    const std::string code = std::string("chxhip-fusion 1\nin a:float32\n") + line + "out y:float32\n";
+    chainerx::Array y = chainerx::Empty(x.shape(), chainerx::Dtype::kFloat32);
+    chx_hip_tensor in_desc = x.hip(), out_desc = y.hip();
+    const chx_hip_tensor* in_ptr = &in_desc;
+    chx_hip_tensor* out_ptr = &out_desc;
+    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, &in_ptr, 1, &out_ptr, 1, nullptr));
+    return y;
+}
+
+constexpr float kFloatMax = 3.4028234663852886e38f;
+
+}  // namespace
+
+chainerx::Array StaticClipOp::RunImpl(ChxVMState* st, const chainerx::Array& x) {
+    return ClipTo(x, min, max);
+}
+// the operands arrive as (x, min, max): the emitter passes the node's inputs in their order
+// (compiler/chxvm/simple_node_emitter.cc:511, runtime/ops/math.cc:144-154)
+chainerx::Array ClipOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& x, const absl::optional<StrictScalar>& min, const absl::optional<StrictScalar>& max) {
+    return ClipTo(x, min.has_value() ? static_cast<float>(*min) : -kFloatMax, max.has_value() ? static_cast<float>(*max) : kFloatMax);
 }
 
 // Maximum / Minimum folded over the operands (runtime/ops/math.cc:179-195)

@@ -1,6 +1,7 @@
 """Writes tests/golden/onnx_node_vectors.json.
 
-The reference pins its quantized ops with eight ONNX backend node tests
+The reference pins its quantized ops with eight ONNX backend node tests and the three
+DynamicQuantizeLinear ones
 (scripts/runtests.py:556-563,577-582 in the chainer-compiler tree); their data
 files live in an ONNX checkout that is not part of that tree.  The inputs and
 expected outputs below are the ONNX operator-specification examples those node
@@ -71,6 +72,24 @@ V["test_convinteger_with_padding"] = dict(
     w=[1, 1, 1, 1], w_shape=[1, 1, 2, 2], pads=[1, 1],
     y=[1, 3, 5, 3, 5, 12, 16, 9, 11, 24, 28, 15, 7, 15, 17, 9], y_shape=[1, 1, 4, 4])
 
+# DynamicQuantizeLinear: y_scale and y_zero_point are outputs of the node
+V["test_dynamicquantizelinear"] = dict(
+    x=[0, 2, -3, -2.5, 1.34, 0.5], x_shape=[6],
+    y=[153, 255, 0, 26, 221, 179], y_scale=0.0196078438, y_zero_point=153)
+
+V["test_dynamicquantizelinear_max_adjusted"] = dict(
+    x=[-1.0, -2.1, -1.3, -2.5, -3.34, -4.0], x_shape=[6],
+    y=[191, 121, 172, 96, 42, 0], y_scale=0.0156862754, y_zero_point=255)
+
+V["test_dynamicquantizelinear_min_adjusted"] = dict(
+    x=[1, 2.1, 1.3, 2.5, 3.34, 4.0, 1.5, 2.6, 3.9, 4.0, 3.0, 2.345], x_shape=[3, 4],
+    y=[64, 134, 83, 159, 213, 255, 96, 166, 249, 255, 191, 149], y_scale=0.0156862754, y_zero_point=0)
+
+# Round (ties to even), which the DynamicQuantizeLinear body uses and the reference also runs on its own
+V["test_round"] = dict(
+    x=[0.1, 0.5, 0.9, 1.2, 1.5, 1.8, 2.3, 2.5, 2.7, -1.1, -1.5, -1.9, -2.2, -2.5, -2.8],
+    y=[0.0, 0.0, 1.0, 1.0, 2.0, 2.0, 2.0, 2.0, 3.0, -1.0, -2.0, -2.0, -2.0, -2.0, -3.0])
+
 
 def rne_sat(v, lo=0, hi=255):
     return np.clip(np.rint(v), lo, hi).astype(np.int64)
@@ -112,6 +131,20 @@ def check():
         got = [[int(xp[i:i + 2, j:j + 2].sum()) for j in range(oh)] for i in range(oh)]
         assert np.array(got).reshape(-1).tolist() == t["y"], (name, got)
 
+    # DynamicQuantizeLinear, from the operator definition in float32 as the node test generator
+    # evaluates it: range widened to contain 0, scale = range / 255, zero point = clip(round(0 - min /
+    # scale)), y = clip(round(x / scale) + zero point)
+    for name in ("test_dynamicquantizelinear", "test_dynamicquantizelinear_max_adjusted", "test_dynamicquantizelinear_min_adjusted"):
+        t = V[name]
+        x = np.array(t["x"], dtype=np.float32)
+        x_min, x_max = np.minimum(np.float32(0), x.min()), np.maximum(np.float32(0), x.max())
+        scale = np.float32((x_max - x_min) / np.float32(255))
+        zp = np.clip(np.rint((np.float32(0) - x_min) / scale), 0, 255).astype(np.uint8)
+        y = np.clip(np.rint(x / scale) + zp, 0, 255).astype(np.uint8)
+        assert y.tolist() == t["y"] and int(zp) == t["y_zero_point"], (name, y, zp)
+        assert np.float32(t["y_scale"]) == scale, (name, scale)
+    t = V["test_round"]
+    assert np.rint(np.array(t["x"], dtype=np.float32)).tolist() == t["y"]
 
 if __name__ == "__main__":
     check()

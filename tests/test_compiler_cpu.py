@@ -121,6 +121,28 @@ def test_groups_keep_to_one_result_shape(vm):
     assert ops_of(desc) == ["ChainerFusionGroup"]
 
 
+def test_dynamic_quantize_linear_is_expanded(vm):
+    """DynamicQuantizeLinear becomes the body of its ONNX function (compiler/simplifier.cc:825-888 with
+    the schema of ONNX 1.5): same node types, in that order, and the three outputs keep their names."""
+    g = onnx_lite.Graph()
+    g.name = "dql"
+    g.nodes = [onnx_lite.Node("DynamicQuantizeLinear", ["x"], ["y", "s", "z"])]
+    g.inputs = [("x", F, [3, 4])]
+    g.outputs = [("y", onnx_lite.ONNX_OF[np.dtype(np.uint8)], [3, 4]), ("s", F, []), ("z", onnx_lite.ONNX_OF[np.dtype(np.uint8)], [])]
+    _, desc = vm.transform_onnx(onnx_lite.make_model(g), {"fuse": "none"})
+    assert sorted(ops_of(desc)) == sorted(["Constant", "Constant", "ReduceMin", "Min", "ReduceMax", "Max", "Sub", "Div", "Div", "Sub",
+                                           "Clip", "Round", "Cast", "Identity", "Identity", "QuantizeLinear"])
+    by_out = {l.split("-> (")[1].split(")")[0]: l for l in lines(desc)}
+    assert by_out["y"].startswith("QuantizeLinear(x, ") and by_out["s"].startswith("Identity(") and by_out["z"].startswith("Identity(")
+    # with the hip rule the 0-d arithmetic between the reductions and the Cast is one group
+    _, desc = vm.transform_onnx(onnx_lite.make_model(g), {"fuse": "hip"})
+    groups = [l for l in lines(desc) if l.startswith("ChainerFusionGroup")]
+    assert len(groups) == 1 and "Clip" in groups[0] and "Round" in groups[0]
+    insts = decode_program(vm, vm.compile_onnx(onnx_lite.make_model(g), {"fuse": "none"}))
+    names = [i[0] for i in insts]
+    assert "Clip" in names and "Round" in names and names.count("Out") == 3
+
+
 def test_hip_program_text_compiles(vm):
     capi = pkg.capi
     k = onnx_lite.Node("Constant", [], ["half"], {"value": np.array(0.5, np.float32)})
