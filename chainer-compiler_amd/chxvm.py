@@ -380,7 +380,10 @@ class Program:
 
 def set_option(name, value):
     """Runtime switches: "qlinearconv_bias" = "reference" (default) | "onnx_int32";
-    "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards)."""
+    "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards);
+    "chrome_tracing" = file that every later run writes its per-instruction timeline to, "" = off;
+    "dump_outputs_dir" = directory that every later run writes the instructions' named array
+    outputs to as .npy files, "" = off."""
     _check(runtime().chxvm_set_option(name.encode(), value.encode()))
 
 

@@ -244,7 +244,10 @@ private:
             inst->inputs.push_back(IntIn(static_cast<int64_t>(n.outputs().size())));
             inst->inputs.push_back(StringIn(code));
             inst->inputs.push_back(IntIn(n.chainer_fusion_group()));
-            for (Value* o : n.outputs()) inst->outputs.push_back(IdOf(o));
+            for (Value* o : n.outputs()) {
+                inst->outputs.push_back(IdOf(o));
+                inst->output_names.push_back(o->name());
+            }
             return;
         }
         CHECK_EQ(1UL, n.outputs().size()) << n.ToString();
@@ -253,6 +256,7 @@ private:
             ChxVMInstructionProto* inst = Add(name, dbg);
             inst->inputs = std::move(inputs);
             inst->outputs.push_back(IdOf(out));
+            inst->output_names.push_back(out->name());  // names the per-op output dumps (compiler/chxvm/emitter.cc:72-77)
             return inst;
         };
         if ((op == "QuantizeLinear" || op == "DequantizeLinear") && nin >= 2 && nin <= 3) {

@@ -67,6 +67,9 @@ def main(argv=None):
                     help="run the quantizer pass in its default mode (dynamic parameters, integer ops), as the reference's flag does")
     ap.add_argument("--no_fuse_operations", action="store_true", help="no fusion groups: every node an instruction of its own")
     ap.add_argument("--dump_onnx", default="", help="write the graph after the passes to this file")
+    ap.add_argument("--chrome_tracing", default="", help="write a per-instruction timeline (Chrome tracing format) of the last run")
+    ap.add_argument("--dump_outputs_dir", default="", help="write every named array output of every instruction there as .npy")
+    ap.add_argument("--report_json", default="", help="write {\"elapsed_times\": [msec, ...]} (the first of several runs dropped)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args(argv)
 
@@ -90,13 +93,18 @@ def main(argv=None):
     input_names = [name for name, _, _ in graph.inputs if name not in graph.initializers]
     output_names = [name for name, _, _ in graph.outputs]
     program = vm.Program(vm.compile_onnx(model_bytes, options))
+    if args.dump_outputs_dir:
+        os.makedirs(args.dump_outputs_dir, exist_ok=True)
+    vm.set_option("chrome_tracing", args.chrome_tracing)
+    vm.set_option("dump_outputs_dir", args.dump_outputs_dir)
     failed = 0
+    elapsed_times = []
     for name, inputs, wants in data_sets:
         if len(inputs) != len(input_names) or len(wants) != len(output_names):
             print("%s: %d inputs / %d outputs on disk, the graph has %d / %d" % (
                 name, len(inputs), len(wants), len(input_names), len(output_names)), file=sys.stderr)
             return 2
-        feed = {n: torch.from_numpy(np.ascontiguousarray(a)).cuda() for n, a in zip(input_names, inputs)}
+        feed = {n: torch.from_numpy(np.array(a, order="C")).cuda() for n, a in zip(input_names, inputs)}
         elapsed = []
         for _ in range(max(1, args.iterations)):
             t0 = time.perf_counter()
@@ -110,11 +118,18 @@ def main(argv=None):
                                                                                 args.atol), file=sys.stderr)
             elif args.verbose:
                 print("OK   %s/%s %s %s" % (name, n, want.dtype, want.shape))
+        elapsed_times += [1e3 * t for t in (elapsed[1:] if len(elapsed) > 1 else elapsed)]
         if args.iterations > 1:
             rest = elapsed[1:]   # the first run is discarded, as run_onnx.cc does
             print("%s: average %.3f ms, best %.3f ms over %d runs" % (name, 1e3 * sum(rest) / len(rest), 1e3 * min(rest),
                                                                     len(rest)))
     program.close()
+    vm.set_option("chrome_tracing", "")
+    vm.set_option("dump_outputs_dir", "")
+    if args.report_json:
+        import json
+        with open(args.report_json, "w") as f:   # tools/run_onnx.cc:493-498
+            json.dump({"elapsed_times": elapsed_times}, f)
     print("%s: %s" % (args.test, "FAILED" if failed else "OK"))
     return 1 if failed else 0
 

@@ -1,8 +1,16 @@
 #include "chxvm.h"
 
+#include <cstring>
+#include <fstream>
+#include <iomanip>
+#include <map>
+#include <sstream>
+
 #include <set>
 
 #include <iostream>
+
+#include "chrome_tracing.h"
 
 namespace chainer_compiler {
 namespace runtime {
@@ -381,6 +389,74 @@ void SetFuseResidual(bool on) {
     g_fuse_residual = on;
 }
 
+namespace {
+
+// .npy (format 1.0) with the elements in logical (row-major) order, whatever the strides on the device
+void SaveNpy(const chainerx::Array& a, const std::string& filename) {
+    static const std::map<chainerx::Dtype, const char*> descr = {
+            {chainerx::Dtype::kBool, "|b1"},   {chainerx::Dtype::kInt8, "|i1"},     {chainerx::Dtype::kInt16, "<i2"},
+            {chainerx::Dtype::kInt32, "<i4"},  {chainerx::Dtype::kInt64, "<i8"},    {chainerx::Dtype::kUInt8, "|u1"},
+            {chainerx::Dtype::kFloat16, "<f2"}, {chainerx::Dtype::kFloat32, "<f4"}, {chainerx::Dtype::kFloat64, "<f8"}};
+    auto it = descr.find(a.dtype());
+    CHECK(it != descr.end()) << "no .npy type for " << a.dtype();
+    const int64_t item = a.GetItemSize(), total = a.GetTotalSize();
+    // the bytes the array spans on the device, then a gather by strides on the host
+    int64_t span = total ? item : 0;
+    for (int i = 0; i < a.ndim() && total; ++i) {
+        CHECK_LE(0, a.strides()[i]) << "negative strides in an output dump";
+        span += (a.shape()[i] - 1) * a.strides()[i];
+    }
+    std::vector<char> raw(static_cast<size_t>(span)), packed(static_cast<size_t>(total * item));
+    if (span) {
+        const chx_hip_tensor t = a.hip();
+        CHXVM_HIP_CALL(chx_hip_memcpy_d2h(raw.data(), t.data, static_cast<size_t>(span), nullptr));
+    }
+    std::vector<int64_t> index(static_cast<size_t>(a.ndim()), 0);
+    for (int64_t flat = 0; flat < total; ++flat) {
+        int64_t off = 0;
+        for (int i = 0; i < a.ndim(); ++i) off += index[i] * a.strides()[i];
+        std::memcpy(&packed[static_cast<size_t>(flat * item)], &raw[static_cast<size_t>(off)], static_cast<size_t>(item));
+        for (int i = a.ndim() - 1; i >= 0; --i) {
+            if (++index[i] < a.shape()[i]) break;
+            index[i] = 0;
+        }
+    }
+    std::ostringstream header;
+    header << "{'descr': '" << it->second << "', 'fortran_order': False, 'shape': (";
+    for (int i = 0; i < a.ndim(); ++i) header << a.shape()[i] << (a.ndim() == 1 || i + 1 < a.ndim() ? "," : "") << (i + 1 < a.ndim() ? " " : "");
+    header << "), }";
+    std::string h = header.str();
+    while ((10 + h.size() + 1) % 64 != 0) h += ' ';
+    h += '\n';
+    std::ofstream ofs(filename, std::ios::binary);
+    CHECK(ofs) << "cannot write " << filename;
+    const unsigned char magic[10] = {0x93, 'N', 'U', 'M', 'P', 'Y', 1, 0, static_cast<unsigned char>(h.size() & 0xff),
+                                     static_cast<unsigned char>(h.size() >> 8)};
+    ofs.write(reinterpret_cast<const char*>(magic), 10);
+    ofs.write(h.data(), static_cast<std::streamsize>(h.size()));
+    ofs.write(packed.data(), static_cast<std::streamsize>(packed.size()));
+}
+
+// runtime/chxvm.cc:70-92
+void DumpOutput(ChxVMState* st, const ChxVMOp* op, const std::string& output_dir) {
+    const ChxVMInstructionProto& inst = op->instruction();
+    for (size_t i = 0; i < inst.outputs.size() && i < inst.output_names.size(); ++i) {
+        const int id = inst.outputs[i];
+        const std::string& name = inst.output_names[i];
+        if (id <= 0 || name.empty()) continue;
+        ChxVMVar* var = st->GetVar(id);
+        if (!var || !var->IsArray()) continue;
+        std::string clean = name;
+        for (char& c : clean)
+            if (c == '/') c = '_';
+        std::ostringstream oss;
+        oss << output_dir << '/' << std::setfill('0') << std::setw(5) << inst.id << '_' << clean << ".npy";
+        SaveNpy(var->GetArray(), oss.str());
+    }
+}
+
+}  // namespace
+
 InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
     for (const std::string& name : input_names_)
         CHECK(program_inputs.count(name)) << "Input '" << name << "' not found";  // runtime/chxvm.cc:142-143
@@ -388,13 +464,20 @@ InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
     while (state.pc() < static_cast<int>(program_.size())) {
         const int pc = state.pc();
         ChxVMOp* op = program_[pc].get();
+        size_t event = 0;
+        if (options.chrome_tracing) event = options.chrome_tracing->Begin("ChxVM", op->name(), pc, op->instruction().flops);
         try {
             op->Run(&state);
         } catch (...) {
             std::cerr << "Exception in " << op->name() << " (pc " << pc << ") " << op->debug_info() << std::endl;
             throw;
         }
+        if (options.chrome_tracing) {
+            CHXVM_HIP_CALL(chx_hip_stream_synchronize(nullptr));
+            options.chrome_tracing->End(event);
+        }
         state.set_pc(state.pc() + 1);  // jumps set pc - 1 themselves (runtime/ops/controlflow.cc:7-21)
+        if (!options.dump_outputs_dir.empty()) DumpOutput(&state, op, options.dump_outputs_dir);
     }
     return state.GetOutputs();
 }

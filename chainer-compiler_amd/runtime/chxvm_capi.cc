@@ -4,6 +4,7 @@
 #include <cstring>
 #include <string>
 
+#include "chrome_tracing.h"
 #include "chxvm.h"
 #include "configs/backend_config.h"
 
@@ -13,6 +14,8 @@ using namespace chainer_compiler::runtime;
 namespace {
 
 thread_local std::string g_last_error;
+// run options of chxvm_set_option, applied by every later chxvm_program_run
+std::string g_chrome_tracing_path, g_dump_outputs_dir;
 
 template <class Fn>
 int32_t Guard(Fn fn) {
@@ -126,7 +129,14 @@ int32_t chxvm_program_run(
         }
         ChxVMOptions options;
         options.trace_level = trace_level;
+        options.dump_outputs_dir = g_dump_outputs_dir;
+        std::unique_ptr<ChromeTracingEmitter> tracing;
+        if (!g_chrome_tracing_path.empty()) {
+            tracing.reset(new ChromeTracingEmitter());
+            options.chrome_tracing = tracing.get();
+        }
         InOuts result = program->vm->Run(in, options);
+        if (tracing) tracing->Emit(g_chrome_tracing_path);
         std::unique_ptr<chxvm_outputs> o(new chxvm_outputs());
         for (const auto& p : result) {
             o->names.push_back(p.first);
@@ -166,6 +176,10 @@ int32_t chxvm_set_option(const char* name, const char* value) {
         } else if (n == "fuse_residual") {
             CHECK(v == "on" || v == "off") << "fuse_residual is 'on' or 'off', got " << v;
             SetFuseResidual(v == "on");
+        } else if (n == "chrome_tracing") {
+            g_chrome_tracing_path = v;
+        } else if (n == "dump_outputs_dir") {
+            g_dump_outputs_dir = v;
         } else {
             CHECK(false) << "unknown option " << n;
         }

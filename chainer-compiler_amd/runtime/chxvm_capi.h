@@ -53,7 +53,12 @@ void chxvm_outputs_destroy(chxvm_outputs* outputs);
 
 /* name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32";
  * name "fuse_residual": value "on" (default) or "off": whether a QLinearConv read only by a
- * residual-sum group computes that group inside its kernel (decided when a program is loaded). */
+ * residual-sum group computes that group inside its kernel (decided when a program is loaded);
+ * name "chrome_tracing": value a file name; every later chxvm_program_run writes its
+ * per-instruction timeline there in the Chrome tracing format (the device is synchronized after
+ * each instruction while this is on), "" switches it off;
+ * name "dump_outputs_dir": value a directory; every later run writes each named array output of
+ * each instruction there as <5-digit instruction id>_<name>.npy, "" switches it off. */
 int32_t chxvm_set_option(const char* name, const char* value);
 /* Process-wide event counts.  name "qlinearconv_residual_fusions": runs of a QLinearConv that
  * computed the residual-sum group behind it inside its kernel.  Unknown names give -1. */

@@ -14,11 +14,19 @@ namespace runtime {
 
 typedef std::map<std::string, std::shared_ptr<ChxVMVar>> InOuts;
 
+class ChromeTracingEmitter;
+
 struct ChxVMOptions {
     int trace_level = 0;
     bool is_training = false;
     bool check_nans = false;
     bool check_infs = false;
+    // an event per executed instruction; the device is synchronized after each one so that an
+    // event spans the instruction's kernels (runtime/chxvm.cc:180 times the host side only)
+    ChromeTracingEmitter* chrome_tracing = nullptr;
+    // every named array output of every instruction as <dir>/<5-digit instruction id>_<name>.npy
+    // (runtime/chxvm.cc:70-92)
+    std::string dump_outputs_dir;
 };
 
 class ChxVMState {

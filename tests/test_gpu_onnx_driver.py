@@ -47,3 +47,41 @@ def test_run_onnx_in_process_with_iterations(onnx_vectors, tmp_path, capsys):
     assert run_onnx.main(["--test", d, "--iterations", "3", "--verbose"]) == 0
     out = capsys.readouterr().out
     assert "average" in out and "OK   test_data_set_0/y uint8 (2, 2, 3)" in out
+
+
+def test_run_onnx_parity_tooling(onnx_vectors, tmp_path):
+    """--chrome_tracing, --dump_outputs_dir and --report_json of the reference's run_onnx
+    (tools/run_onnx.cc:147-149,208-209,493-498): one trace event per executed instruction, every
+    named array output as a .npy that numpy reads back, the elapsed times with the warm-up run dropped."""
+    import json
+    import gpu_util
+    import onnx_cases
+    ol = importlib.import_module(gpu_util.pkg.__name__ + ".onnx_lite")
+    run_onnx = importlib.import_module(gpu_util.pkg.__name__ + ".run_onnx")
+    vm = importlib.import_module(gpu_util.pkg.__name__ + ".chxvm")
+    cases = onnx_cases.build_cases(ol, onnx_vectors)
+    name = "test_dynamicquantizelinear_min_adjusted_expanded"
+    d = onnx_cases.write_case(ol, str(tmp_path), name, cases[name])
+    trace, dumps, report = str(tmp_path / "trace.json"), str(tmp_path / "dumps"), str(tmp_path / "report.json")
+    assert run_onnx.main(["--test", d, "--no_fuse_operations", "--iterations", "3", "--chrome_tracing", trace,
+                          "--dump_outputs_dir", dumps, "--report_json", report]) == 0
+    events = json.load(open(trace))
+    program = vm.compile_onnx(open(os.path.join(d, "model.onnx"), "rb").read(), {"fuse": "none"})
+    loaded = vm.Program(program)
+    assert len(events) == loaded.num_instructions
+    loaded.close()
+    names = [e["name"] for e in events]
+    assert all(e["ph"] == "X" and e["cat"] == "ChxVM" and e["dur"] >= 0 for e in events)
+    assert [e["args"]["pc"] for e in events] == list(range(len(events)))
+    for op in ("ReduceMin", "ReduceMax", "Clip", "Round", "Cast", "QuantizeLinear", "In", "Out", "Free"):
+        assert op in names
+    files = sorted(os.listdir(dumps))
+    by_name = {f.split("_", 1)[1][:-4]: np.load(os.path.join(dumps, f)) for f in files}
+    graph, inputs, outs = cases[name]
+    np.testing.assert_array_equal(by_name["y"], outs[0])
+    assert by_name["y"].shape == (3, 4) and by_name["y"].dtype == np.uint8
+    assert by_name["Scale"].shape == () and by_name["Scale"] == outs[1]
+    assert by_name["Zeropoint"] == outs[2] and by_name["Rounded_ZeroPoint_FP"] == np.float32(0)
+    assert all(f[:5].isdigit() for f in files)
+    times = json.load(open(report))["elapsed_times"]
+    assert len(times) == 2 and all(t > 0 for t in times)
