@@ -742,8 +742,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         __syncthreads();
 
         char* slot = ring + cbuf * STAGE_BYTES;
-        const char* sa = slot;
-        const char* sb = sa + TM * BK;
         cbuf = cbuf + 1 == NS ? 0 : cbuf + 1;
         // The copies of the stage NS-1 steps ahead are issued between the MFMA groups rather than
         // in one burst: the copy unit takes a 1 KB instruction every 16 cycles or so, and a wave
