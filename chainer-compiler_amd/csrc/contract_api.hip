@@ -943,6 +943,7 @@ extern "C" int chx_hip_qconv_plan_run_add(
     // |DQ(y) + DQ(r)| <= 511 * (|y_scale| + |r_scale|): when that is far below `big`, limiting is the identity
     const double reach = 511.0 * (fabs((double)y_scale) + fabs((double)r_scale));
     res.guard = (reach == reach && reach < 0.25 * (double)res.big) ? 0 : 1;
+    res.lean = out->dtype == CHX_HIP_UINT8 && r->dtype == CHX_HIP_UINT8 && r_zero_point == 0 && out_zero_point == 0 ? 1 : 0;
     hipStream_t s = as_stream(stream);
     ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0);
     call.cache = const_cast<ScratchCache*>(&plan->scratch);

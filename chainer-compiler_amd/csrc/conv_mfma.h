@@ -27,6 +27,7 @@ struct ResidualAdd {
     float inv_out_scale;
     float big;             // 2^40 * out.scale: the dividend is limited to +-big (both sides saturate beyond)
     int32_t guard;         // 0 when the operand scales already keep every sum far inside +-big
+    int32_t lean;          // uint8 result with zero point 0 and r with zero point 0: see add_residual16
 };
 
 struct ConvMfmaArgs {

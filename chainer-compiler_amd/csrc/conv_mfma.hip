@@ -311,8 +311,13 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 // Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
 // (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
 // reference's order, one IEEE operation each.
-template <bool kU8, bool kGuard>
+// kLean (uint8 result, zero points of r and of the result both 0, as between the Relu outputs of a
+// residual network): the two "- 0.0f" / "+ 0.0f" change no value and are left out, and so is the
+// Relu, because QuantizeLinear is monotone, Q(max(s, 0)) = max(Q(s), Q(0)) = max(Q(s), 0), and the
+// saturating conversion already stops at 0.
+template <bool kU8, bool kGuard, bool kLean = false>
 __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
+    static_assert(kU8 || !kLean, "the lean variant is for uint8 results");
     v4i out;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -322,11 +327,12 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
-            const float fb = ((float)((rw >> (8 * e)) & 0xffu) - p.r_zpf) * p.r_scale;
+            const float rb = (float)((rw >> (8 * e)) & 0xffu);
+            const float fb = kLean ? rb * p.r_scale : (rb - p.r_zpf) * p.r_scale;
             float sum = fa + fb;
-            if (p.relu) sum = __builtin_fmaxf(sum, 0.f);
+            if (!kLean && p.relu) sum = __builtin_fmaxf(sum, 0.f);
             if (kGuard) sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
-            if (kU8) pre[e] = quantize_prefloor_u8<false>(sum, p.out, p.inv_out_scale, 0.f);
+            if (kU8) pre[e] = quantize_prefloor_u8<false, !kLean>(sum, p.out, p.inv_out_scale, 0.f);
             else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
         }
         out[w] = kU8 ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
@@ -334,7 +340,6 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
     return out;
 }
 
-// Wait until at most N of this wave's vector-memory operations are outstanding.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -608,7 +613,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         }
         // requantize: one instance of the element loop per bias mode and per conversion path (the
         // branches are uniform).  kPath 0: any 8-bit type and rounding; 1: uint8 in the reference's
-        // rounding through floor_sat_u8x4/8; 2: the same with a lower bound above 0 (a folded Relu).
+        // rounding through floor_sat_u8x4/8; 2: the same with a lower bound above 0 (a folded Relu);
+        // 3: as 1 with a zero point of 0.
         auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
             constexpr int kPath = decltype(path_tag)::value;
@@ -641,7 +647,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                             for (int e = 0; e < 4; ++e) {
                                 float v = (float)acc[i][j][g * 4 + e] * sc[e];
                                 if (kFloatBias) v = v + fb[e];
-                                pre[j * 4 + e] = quantize_prefloor_u8<kPath == 2>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                                pre[j * 4 + e] = quantize_prefloor_u8<kPath == 2, kPath != 3>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
                             }
                         uint32_t word[FN];
                         if constexpr (FN == 2) {
@@ -675,6 +681,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             using P0 = std::integral_constant<int, 0>;
             using P1 = std::integral_constant<int, 1>;
             using P2 = std::integral_constant<int, 2>;
+            using P3 = std::integral_constant<int, 3>;
             const bool u8_reference = !kRne && a.rq.q.lo == 0.f && a.rq.q.hi == 255.f;
             const bool float_bias = a.rq.bias_mode == kBiasReferenceFloat;
             if (!u8_reference) {
@@ -683,6 +690,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             } else if (a.lo_folded > 0.f) {
                 if (float_bias) requantize_tile(std::true_type(), P2());
                 else requantize_tile(std::false_type(), P2());
+            } else if (a.rq.q.zpf == 0.f) {
+                if (float_bias) requantize_tile(std::true_type(), P3());
+                else requantize_tile(std::false_type(), P3());
             } else {
                 if (float_bias) requantize_tile(std::true_type(), P1());
                 else requantize_tile(std::false_type(), P1());
@@ -712,7 +722,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                         rv[w] = (int)word;
                     }
                 }
-                if (a.res.guard)
+                if (a.res.lean)
+                    val = a.res.guard ? add_residual16<true, true, true>(val, rv, a.res) : add_residual16<true, false, true>(val, rv, a.res);
+                else if (a.res.guard)
                     val = a.res.out.lo == 0.f ? add_residual16<true, true>(val, rv, a.res) : add_residual16<false, true>(val, rv, a.res);
                 else
                     val = a.res.out.lo == 0.f ? add_residual16<true, false>(val, rv, a.res) : add_residual16<false, false>(val, rv, a.res);

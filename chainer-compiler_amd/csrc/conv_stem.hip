@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
                         float v = (float)acc[i][g * 4 + e] * sc[e];
                         if (kFloatBias) v = v + fbs[e];
                         if (kPath == 0) code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
-                        else pre[e] = quantize_prefloor_u8<kPath == 2>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                        else pre[e] = quantize_prefloor_u8<kPath == 2, kPath != 3>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
                     }
                     *reinterpret_cast<uint32_t*>(staged(p, ocl)) =
                             kPath == 0 ? pack4(code[0], code[1], code[2], code[3]) : floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]);
@@ -274,6 +274,7 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
             using P0 = std::integral_constant<int, 0>;
             using P1 = std::integral_constant<int, 1>;
             using P2 = std::integral_constant<int, 2>;
+            using P3 = std::integral_constant<int, 3>;  // as 1 with a zero point of 0
             const bool u8_reference = !kRne && a.rq.q.lo == 0.f && a.rq.q.hi == 255.f;
             const bool float_bias = a.rq.bias_mode == kBiasReferenceFloat;
             if (!u8_reference) {
@@ -282,6 +283,9 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
             } else if (a.lo_folded > 0.f) {
                 if (float_bias) requantize_tile(std::true_type(), P2());
                 else requantize_tile(std::false_type(), P2());
+            } else if (a.rq.q.zpf == 0.f) {
+                if (float_bias) requantize_tile(std::true_type(), P3());
+                else requantize_tile(std::false_type(), P3());
             } else {
                 if (float_bias) requantize_tile(std::true_type(), P1());
                 else requantize_tile(std::false_type(), P1());

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void pack_depthwise_kernel(
 // kStep: vertical stride 1 or 2 (the packed input rows shared between neighbouring output rows
 // are kept), 0: any stride (every output row loads its three input rows).
 // kPath: 0 any 8-bit type and rounding; 1 uint8 in the reference's rounding (floor_sat_u8x4);
-// 2 the same with a lower bound above 0 (a folded Relu).  Chosen by the launcher, so that the
+// 2 the same with a lower bound above 0 (a folded Relu); 3 as 1 with a zero point of 0.  Chosen by the launcher, so that the
 // row loop has no branches and the loads of a whole strip are in flight together.
 // Output rows per thread.  More rows spread the per-thread set-up (index arithmetic, masks, filter
 // rows and constants) and the two halo rows over more outputs, at the price of registers for the
@@ -130,6 +130,7 @@ __global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs 
             // uint8 in the reference's rounding: clamp, conversion and packing in floor_sat_u8x4
             if (kPath == 2) pre[e] = quantize_prefloor_u8<true>(v, a.q, a.inv_y_scale, a.lo_folded);
             else if (kPath == 1) pre[e] = quantize_prefloor_u8<false>(v, a.q, a.inv_y_scale, 0.f);
+            else if (kPath == 3) pre[e] = quantize_prefloor_u8<false, false>(v, a.q, a.inv_y_scale, 0.f);
             else code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
         }
         const uint32_t o = kPath ? floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : pack4(code[0], code[1], code[2], code[3]);
@@ -218,12 +219,13 @@ int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
     const dim3 blocks((unsigned)(((int64_t)a.OW * (a.C / 4) + kDwThreads - 1) / kDwThreads), (unsigned)a.oh_blocks, (unsigned)a.N);
     const bool fbias = a.bias != nullptr && a.float_bias != 0;
     const bool u8_reference = !rne && a.q.lo == 0.f && a.q.hi == 255.f;
-    const int path = !u8_reference ? 0 : a.lo_folded > 0.f ? 2 : 1;
+    const int path = !u8_reference ? 0 : a.lo_folded > 0.f ? 2 : a.q.zpf == 0.f ? 3 : 1;
 #define CHX_DW_P(RN, FB, ST, TL)                                                                    \
     do {                                                                                            \
         if (path == 0) depthwise3x3_kernel<RN, FB, ST, 0, TL><<<blocks, kDwThreads, 0, s>>>(a);     \
         else if (RN) CHX_FAIL(CHX_HIP_ERUNTIME, "depthwise: conversion path");                      \
         else if (path == 1) depthwise3x3_kernel<false, FB, ST, 1, TL><<<blocks, kDwThreads, 0, s>>>(a); \
+        else if (path == 3) depthwise3x3_kernel<false, FB, ST, 3, TL><<<blocks, kDwThreads, 0, s>>>(a); \
         else depthwise3x3_kernel<false, FB, ST, 2, TL><<<blocks, kDwThreads, 0, s>>>(a);            \
     } while (0)
 #define CHX_DW_S(RN, FB)                               \

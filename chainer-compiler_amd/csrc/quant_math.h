@@ -150,12 +150,14 @@ __device__ __forceinline__ void floor_sat_u8x8(const float (&x)[8], uint32_t* lo
 
 // The value handed to floor_sat_u8x4/8 for one element: quantize_value_folded up to and including
 // the + 0.5f, with only the lower bound applied (and only when it is above 0).
-template <bool kLowerBound>
+// kZeroPoint = false is for a zero point of 0: adding 0.0f changes no value (-0 becomes +0, which the
+// next addition would do as well), so the instruction is left out.
+template <bool kLowerBound, bool kZeroPoint = true>
 __device__ __forceinline__ float quantize_prefloor_u8(float v, const QuantParams& q, float inv_scale, float lo_folded) {
     const float q0 = v * inv_scale;
     const float r = __builtin_fmaf(-q0, q.scale, v);
     float s = __builtin_fmaf(r, inv_scale, q0);
-    s = s + q.zpf;
+    if (kZeroPoint) s = s + q.zpf;
     if (kLowerBound) s = __builtin_fmaxf(s, lo_folded);
     return s + 0.5f;
 }

@@ -334,6 +334,30 @@ def test_planar_input_qlinear_conv(g, oracle, case, xdt):
     np.testing.assert_array_equal(g.host(got), want)
 
 
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, OC, K, stride, pad, group: the matrix-core kernel, the first-layer kernel, the depthwise kernel
+    (2, 64, 9, 10, 96, 1, 1, 0, 1), (1, 32, 8, 8, 40, 3, 1, 1, 1), (2, 3, 20, 22, 32, 3, 2, 1, 1), (1, 48, 14, 6, 48, 3, 1, 1, 48)])
+def test_qlinear_conv_with_output_zero_point_zero(g, oracle, case):
+    """uint8 results with y_zero_point = 0 (every activation behind a Relu): the kernels leave the
+    addition of the zero point out; negative values must saturate to 0 as the reference's clip does."""
+    N, C, H, W, OC, K, stride, pad, group = case
+    rng = np.random.default_rng(71)
+    x = rand_q(rng, (N, C, H, W), np.uint8)
+    w = rng.integers(-127, 128, size=(OC, C // group, K, K)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-300, 301, size=OC).astype(np.int32)
+    ys = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C // group * K * K) / 60)
+    kw = dict(strides=(stride, stride), pads=(pad, pad), group=group)
+    for bias_mode, flags in ((oracle.BIAS_ONNX_INT32, g.capi.BIAS_ONNX_INT32), (oracle.BIAS_REFERENCE_FLOAT, 0)):
+        want = oracle.qlinear_conv_int(x, 0.02, 101, w, ws, wz, ys, 0, np.uint8, bias=bias, bias_mode=bias_mode, **kw)
+        assert (want == 0).mean() > 0.2 and want.max() > 100
+        for xd in ((g.dev(x),) if C == 3 else (g.to_channels_last(g.dev(x)),)):
+            for fl in (flags, flags | g.capi.FUSE_RELU):   # with a zero point of 0 the Relu changes nothing
+                got = g.ops.QLinearConv(xd, 0.02, 101, g.dev(w), g.dev(ws), g.dev(wz), ys, 0, g.dev(bias), flags=fl, **kw)
+                np.testing.assert_array_equal(g.host(got), want)
+
+
 def _residual_sum(oracle, c, c_scale, c_zp, r, r_scale, r_zp, relu, out_scale, out_zp, out_dtype):
     """QuantizeLinear(act(DequantizeLinear(c) + DequantizeLinear(r))), op by op on the CPU."""
     s = oracle.binary(oracle.ADD, oracle.dequantize_linear(c, c_scale, c_zp), oracle.dequantize_linear(r, r_scale, r_zp))
@@ -377,6 +401,16 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
             got = plan.run_add(xd, 0.02, 101, ys, yz, rd, rs, rz, os_, oz, relu, zero_point_dtype=TDT[ydt],
                                flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(rd, dtype=TDT[odt]))
             np.testing.assert_array_equal(g.host(got), want)
+    # zero points of 0 on the residual and on the result (what lies between the Relu outputs of a
+    # residual network): the kernel leaves out the two additions of 0 and, for uint8, the Relu,
+    # which the saturation at 0 already is; negative sums must still come out as 0
+    if rdt == np.uint8:
+        for relu in (False, True):
+            want = _residual_sum(oracle, conv, ys, yz, r, rs, 0, relu, os_, 0, odt)
+            got = plan.run_add(xd, 0.02, 101, ys, yz, g.to_channels_last(g.dev(r)), rs, 0, os_, 0, relu, zero_point_dtype=TDT[ydt],
+                               flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(g.to_channels_last(g.dev(r)), dtype=TDT[odt]))
+            np.testing.assert_array_equal(g.host(got), want)
+            assert want.min() < want.max()
     # operands that are not channels-last are refused, not converted
     with pytest.raises(g.capi.ChxHipError) as e:
         plan.run_add(xd, 0.02, 101, ys, yz, g.dev(r), rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt],
