@@ -120,9 +120,10 @@ __global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs 
         float pre[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            // the three-operand form: no copy of the seed into the accumulator first
-            int32_t acc;
-            asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(acc) : "v"(r0[e]), "v"(wq[0][e]), "v"(seed[e]));
+            // (all three through the builtin: the compiler then knows they are dot products and keeps the
+            // wait states that gfx950 wants between a dot product and a different instruction reading its result)
+            int32_t acc = seed[e];
+            acc = __builtin_amdgcn_sdot4((int)r0[e], wq[0][e], acc, false);
             acc = __builtin_amdgcn_sdot4((int)r1[e], wq[1][e], acc, false);
             acc = __builtin_amdgcn_sdot4((int)r2[e], wq[2][e], acc, false);
             float v = (float)acc * sc[e];
