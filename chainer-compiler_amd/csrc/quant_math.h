@@ -114,10 +114,13 @@ __device__ __forceinline__ int32_t quantize_value_folded(float v, const QuantPar
 // AsType(Maximum(0, Minimum(t, 255)) + 0.5f): inside the range the two are the same operations,
 // below it both give 0 (t + 0.5f <= 0.5 there), above it both give 255.  The rounding mode of the
 // wave is switched and restored inside one asm statement, so no other instruction can end up
-// between the two switches.  A lower bound above 0 (a folded Relu) is applied to t by the caller.
+// between the two switches; the s_nop in front keeps two wait states between the restoring write of
+// one statement and the switching write of the next, which the compiler cannot see (two writes of
+// the same hardware register want that distance).  A lower bound above 0 (a folded Relu) is applied to t by the caller.
 __device__ __forceinline__ uint32_t floor_sat_u8x4(float a, float b, float c, float d) {
     uint32_t r;
     asm volatile(
+            "s_nop 1\n\t"
             "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2\n\t"
             "v_cvt_pk_u8_f32 %0, %1, 0, 0\n\t"
             "v_cvt_pk_u8_f32 %0, %2, 1, %0\n\t"
@@ -132,6 +135,7 @@ __device__ __forceinline__ uint32_t floor_sat_u8x4(float a, float b, float c, fl
 __device__ __forceinline__ void floor_sat_u8x8(const float (&x)[8], uint32_t* lo, uint32_t* hi) {
     uint32_t r0, r1;
     asm volatile(
+            "s_nop 1\n\t"
             "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2\n\t"
             "v_cvt_pk_u8_f32 %0, %2, 0, 0\n\t"
             "v_cvt_pk_u8_f32 %1, %6, 0, 0\n\t"
