@@ -83,7 +83,7 @@ ChxVMValueProto StringIn(const std::string& s) {
 const std::map<std::string, std::set<int>>& ScalarOperands() {
     static const std::map<std::string, std::set<int>> m = {
             {"QuantizeLinear", {1, 2}}, {"DequantizeLinear", {1, 2}}, {"QLinearConv", {1, 2, 6, 7}},
-            {"QLinearMatMul", {1, 2, 4, 5, 6, 7}}, {"ConvInteger", {2}}};
+            {"QLinearMatMul", {1, 2, 4, 5, 6, 7}}, {"ConvInteger", {2}}, {"Clip", {1, 2}}};
     return m;
 }
 

@@ -259,7 +259,7 @@ std::string BuildHipProgram(const Node& group, std::vector<int>* used_inputs) {
     // point, bound) is a constant of the outer graph: it is written into the statement and is no
     // operand of the kernel.
     std::map<const Value*, std::unique_ptr<Tensor>> constants;
-    std::set<const Value*> data_inputs;
+    std::set<const Value*> data_inputs, absent;
     for (Node* node : body.GetLiveNodes()) {
         const std::string& op = node->op_type();
         const size_t first_param = (op == "QuantizeLinear" || op == "DequantizeLinear" || op == "Clip") ? 1 : node->inputs().size();
@@ -270,6 +270,10 @@ std::string BuildHipProgram(const Node& group, std::vector<int>* used_inputs) {
     for (size_t i = 0; i < body.input_values().size(); ++i) {
         Value* v = body.input_values()[i];
         if (!data_inputs.count(v)) {
+            if (group.input(static_cast<int>(i))->IsNull()) {  // an absent bound of a Clip
+                absent.insert(v);
+                continue;
+            }
             constants[v] = OneElementConstant(group.input(static_cast<int>(i)));
             CHECK(constants[v]) << "parameter '" << group.input(static_cast<int>(i))->name() << "' of the group is not a one-element constant";
             continue;
@@ -313,8 +317,9 @@ std::string BuildHipProgram(const Node& group, std::vector<int>* used_inputs) {
             os << out << " = " << op << " " << ins[0] << " " << ins[1] << "\n";
         } else if (op == "Clip") {
             double lo = node->GetFloat("min", -3.4028234663852886e38f), hi = node->GetFloat("max", 3.4028234663852886e38f);
-            if (node->inputs().size() > 1 && !node->input(1)->IsNull()) lo = constant_of(node->input(1))->GetAsDouble(0);
-            if (node->inputs().size() > 2 && !node->input(2)->IsNull()) hi = constant_of(node->input(2))->GetAsDouble(0);
+            auto given = [&](size_t i) { return node->inputs().size() > i && !node->input(i)->IsNull() && !absent.count(node->input(i)); };
+            if (given(1)) lo = constant_of(node->input(1))->GetAsDouble(0);
+            if (given(2)) hi = constant_of(node->input(2))->GetAsDouble(0);
             os << out << " = Clip " << ins[0] << " " << FloatBits(lo) << " " << FloatBits(hi) << "\n";
         } else if (op == "QuantizeLinear" || op == "DequantizeLinear") {
             const double scale = constant_of(node->input(1))->GetAsDouble(0);

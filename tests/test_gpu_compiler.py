@@ -155,3 +155,37 @@ def test_dynamic_integer_quantization_runs_end_to_end(g, vm, oracle, per_channel
     bq, sb, zb = cc.numpy_quantize(b, np.uint8)
     acc = oracle.matmul_integer(oracle.quantize_linear(a, sa, int(za), np.uint8), bq, np.array(za, np.uint8), np.array(zb, np.uint8))
     np.testing.assert_array_equal(got, acc.astype(np.float32) * np.float32(sa * sb))
+
+
+def test_clip_round_and_friends_as_single_instructions(g, vm):
+    """Clip with attribute bounds (StaticClip), Clip with operand bounds, one bound missing, Round
+    (ties to even), Abs, Floor, Max and Min as instructions of their own and inside one hip group:
+    the bytes numpy gives for the same float32 operations."""
+    rng = np.random.default_rng(14)
+    x = np.concatenate([rng.uniform(-9, 9, 500).astype(np.float32),
+                        np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 6.0, -3.0, 0.0], np.float32)]).reshape(1, 509)
+    f32 = np.float32
+    lo = onnx_lite.Node("Constant", [], ["lo"], {"value": np.array(-2.25, f32)})
+    hi = onnx_lite.Node("Constant", [], ["hi"], {"value": np.array(5.5, f32)})
+    nodes = [lo, hi,
+             onnx_lite.Node("Clip", ["x"], ["a"], {"min": -3.0, "max": 6.0}),       # bounds as attributes
+             onnx_lite.Node("Clip", ["x", "lo", "hi"], ["b"]),                       # bounds as operands
+             onnx_lite.Node("Clip", ["x", "", "hi"], ["c"]),                         # no lower bound
+             ("Round", ["x"], ["d"]), ("Abs", ["x"], ["e"]), ("Floor", ["x"], ["f"]),
+             ("Max", ["a", "d"], ["m"]), ("Min", ["b", "f"], ["n"])]
+    outs = ["a", "b", "c", "d", "e", "f", "m", "n"]
+    m = cc.model(nodes, [("x", x.shape)], [(o, x.shape) for o in outs])
+    a, b, c = np.clip(x, f32(-3), f32(6)), np.clip(x, f32(-2.25), f32(5.5)), np.minimum(x, f32(5.5))
+    d, e, f = np.rint(x), np.abs(x), np.floor(x)
+    want = dict(a=a, b=b, c=c, d=d, e=e, f=f, m=np.maximum(a, d), n=np.minimum(b, f))
+    assert d[0, -9:].tolist() == [0.0, 2.0, 2.0, -0.0, -2.0, -2.0, 6.0, -3.0, 0.0]
+    for fuse in ("none", "hip"):
+        data = vm.compile_onnx(m, {"fuse": fuse})
+        names = [i[0] for i in cc.decode_program(vm, data)]
+        if fuse == "none":
+            assert names.count("StaticClip") == 1 and names.count("Clip") == 2 and "Round" in names
+        prog = vm.Program(data)
+        got = prog.run({"x": torch.from_numpy(x).cuda()})
+        prog.close()
+        for o in outs:
+            np.testing.assert_array_equal(got[o].view(np.uint32), want[o].view(np.uint32), err_msg="%s (%s)" % (o, fuse))
