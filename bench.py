@@ -9,8 +9,10 @@ that is already resident in HBM (fp32 NCHW input; QuantizeLinear is part of the 
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the int8 MFMA implicit-GEMM
 convolution for resnet50 / conv3x3, the fused element-wise kernel for fusion / qdq), timed
 live with events on the launch stream: around every launch of the timed region for the
-single-kernel workloads, and for resnet50 (whose timed region is a HIP graph replay) around
-back-to-back repeats of each convolution launch right after it.  `cpu_baseline` times the
+single-kernel workloads; for the networks (whose timed region is a HIP graph replay, where
+no events can be placed) the convolution launches of the step are recorded in program order
+into a graph of their own, which is replayed ten times between one event pair right after
+the timed region.  `cpu_baseline` times the
 restated reference CPU op sequence (the oracle's literal fp32 path) on the host cores for a
 bounded sample of the same workload.
 """

@@ -210,13 +210,16 @@ bool weights_fit_mfma(const chx_hip_tensor& w, int group) {
 }
 
 // Tile shape: the largest tile that still gives every compute unit a work-group.
-void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px) {
-    // CHX_HIP_TILE=<oc>,<px> forces a tile shape (tuning aid)
+void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px, int* max_wgs_per_cu) {
+    // CHX_HIP_TILE=<oc>,<px>[,<work-groups per compute unit>] forces a launch configuration (read on
+    // every call: a tuning aid, and how the tests reach every configuration the tuner may choose)
     if (const char* env = getenv("CHX_HIP_TILE")) {
-        int toc = 0, tpx = 0;
-        if (sscanf(env, "%d,%d", &toc, &tpx) == 2 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128)) {
+        int toc = 0, tpx = 0, cap = 0;
+        const int got = sscanf(env, "%d,%d,%d", &toc, &tpx, &cap);
+        if (got >= 2 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128) && cap >= 0) {
             *tile_oc = toc;
             *tile_px = tpx;
+            *max_wgs_per_cu = got == 3 ? cap : 0;
             return;
         }
     }
@@ -246,11 +249,8 @@ struct TuneCache {
 };
 
 bool autotune_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("CHX_HIP_AUTOTUNE");  // CHX_HIP_AUTOTUNE=0 keeps the heuristic
-        return !(e && e[0] == '0') && !getenv("CHX_HIP_TILE");
-    }();
-    return on;
+    const char* e = getenv("CHX_HIP_AUTOTUNE");  // CHX_HIP_AUTOTUNE=0 keeps the heuristic
+    return !(e && e[0] == '0') && !getenv("CHX_HIP_TILE");
 }
 
 bool stream_is_capturing(hipStream_t s) {
@@ -526,7 +526,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     if (c.res) a.res = *c.res;
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64, cap = 0;
-    pick_tile(cs.OC, a.M, &toc, &tpx);
+    pick_tile(cs.OC, a.M, &toc, &tpx, &cap);
     int rc = CHX_HIP_OK;
     const TunedConfig* tuned = nullptr;
     if (c.tune) {

@@ -417,3 +417,57 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
                      flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros(conv.shape, dtype=TDT[odt], device="cuda"))
     assert e.value.code == g.capi.EUNSUPPORTED
     plan.close()
+
+
+@pytest.mark.parametrize("tile", [(128, 128), (64, 128), (128, 64), (64, 64)])
+def test_every_launch_configuration_of_the_matrix_core_kernel(g, oracle, tile):
+    """The tuner picks one of 4 tile shapes x 3 occupancy caps per layer shape by timing, so a test
+    that leaves the choice to it covers one configuration per case.  CHX_HIP_TILE forces each in
+    turn: ragged pixel and channel tiles, 64- and 128-byte K steps, padded and padding-free taps,
+    channel counts that do not fill a K step, int32 results, the fused residual sum, work-groups
+    that walk over several pixel tiles."""
+    import os
+    rng = np.random.default_rng(83)
+
+    def qconv_case(N, C, H, W, OC, K, stride, pad):
+        x = rand_q(rng, (N, C, H, W), np.uint8)
+        w = rng.integers(-127, 128, size=(OC, C, K, K)).astype(np.int8)
+        ws = rng.uniform(0.002, 0.02, size=OC).astype(np.float32)
+        bias = rng.integers(-500, 501, size=OC).astype(np.int32)
+        ys = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C * K * K) / 40)
+        kw = dict(strides=(stride, stride), pads=(pad, pad))
+        want = oracle.qlinear_conv_int(x, 0.02, 101, w, ws, np.zeros(OC, np.int8), ys, 119, np.uint8, bias=bias,
+                                       bias_mode=oracle.BIAS_ONNX_INT32, **kw)
+        return x, w, ws, bias, ys, kw, want
+
+    # the last case has more pixel tiles than resident work-groups: each work-group walks over several
+    convs = [qconv_case(3, 64, 13, 11, 200, 3, 1, 1), qconv_case(2, 256, 9, 7, 136, 1, 1, 0), qconv_case(2, 24, 11, 10, 72, 3, 2, 1),
+             qconv_case(16, 64, 80, 79, 64, 1, 1, 0)]
+    xi = rand_q(rng, (2, 128, 9, 9), np.uint8)
+    wi = rand_q(rng, (80, 128, 3, 3), np.int8)
+    want_int = oracle.conv_integer(xi, wi, 77, None, strides=(1, 1), pads=(0, 0), group=1, auto_pad="")
+    # residual sum behind the second case
+    x1, w1, ws1, bias1, ys1, kw1, conv1 = convs[1]
+    r = rand_q(rng, conv1.shape, np.uint8)
+    want_sum = _residual_sum(oracle, conv1, ys1, 119, r, np.float32(0.037), 131, True, np.float32(0.061), 99, np.uint8)
+    before = os.environ.get("CHX_HIP_TILE")
+    try:
+        for cap in (0, 2, 1):
+            os.environ["CHX_HIP_TILE"] = "%d,%d,%d" % (tile[0], tile[1], cap)
+            for x, w, ws, bias, ys, kw, want in convs:
+                plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(np.zeros(len(ws), np.int8)), g.dev(bias), **kw)
+                got = plan.run(g.to_channels_last(g.dev(x)), 0.02, 101, ys, 119, torch.uint8, flags=g.capi.BIAS_ONNX_INT32)
+                np.testing.assert_array_equal(g.host(got), want, err_msg="tile %s cap %d conv %s" % (tile, cap, x.shape))
+                if x is x1:
+                    rd = g.to_channels_last(g.dev(r))
+                    got = plan.run_add(g.to_channels_last(g.dev(x)), 0.02, 101, ys, 119, rd, 0.037, 131, 0.061, 99, True,
+                                       zero_point_dtype=torch.uint8, flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(rd))
+                    np.testing.assert_array_equal(g.host(got), want_sum, err_msg="tile %s cap %d residual sum" % (tile, cap))
+                plan.close()
+            got = g.ops.ConvInteger(g.to_channels_last(g.dev(xi)), g.dev(wi), 77, None)
+            np.testing.assert_array_equal(g.host(got), want_int, err_msg="tile %s cap %d ConvInteger" % (tile, cap))
+    finally:
+        if before is None:
+            os.environ.pop("CHX_HIP_TILE", None)
+        else:
+            os.environ["CHX_HIP_TILE"] = before
