@@ -202,8 +202,8 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         wl.run_reference(one, lit, one["input"])
         dt1 = time.perf_counter() - t0
         # all cores, sized to roughly the requested budget
-        nb = int(max(1, min(16, args.cpu_seconds / max(dt1 / cores * 1.5, 1e-3))))
-        many = build(batch=nb)
+        nb = int(max(1, min(batch, args.cpu_seconds / max(dt1 / cores * 1.5, 1e-3))))
+        many = model if nb == batch else build(batch=nb)
         orc.set_threads(cores)
         t0 = time.perf_counter()
         wl.run_reference(many, lit, many["input"])
