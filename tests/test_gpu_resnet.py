@@ -173,3 +173,40 @@ def test_concurrent_batch_slices_match_whole_batch(g, oracle):
         check(replay(), "replay %d" % i)
     whole.close()
     split.close()
+
+
+@pytest.mark.parametrize("net,batch,seed", [("resnet50", 64, 3), ("mobilenetv2", 128, 4)])
+def test_benchmark_configuration_at_full_size(g, oracle, net, batch, seed):
+    """The timed configuration itself: the full batch, residual sums inside the convolutions, the tuned
+    launch configurations, one HIP graph replay.  Three images of the batch are followed through the
+    oracle tensor by tensor; all of them through a property that needs no oracle: every op on the
+    path is independent per image, so a permuted batch must give the permuted results."""
+    wl = g.pkg.workloads
+    model = (wl.build_resnet50 if net == "resnet50" else wl.build_mobilenetv2)(batch=batch, seed=seed)
+    runner = wl.DeviceRunner(model, g.pkg, fuse_residual=True)
+    assert runner.fused_into
+    x = torch.from_numpy(model["input"]).cuda()
+    runner.run(x)                      # eager first: the plans time their launch configurations here
+    torch.cuda.synchronize()
+    replay = runner.capture(x)
+    out = {k: v.clone() for k, v in replay().items()}
+    torch.cuda.synchronize()
+    picks = [0, batch // 2 + 5, batch - 1]
+    oracle.set_threads(16)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"][picks])
+    finally:
+        oracle.set_threads(1)
+    for ins in model["program"]:
+        name = ins[1]
+        if name in runner.fused_into:
+            continue
+        np.testing.assert_array_equal(out[name][picks].cpu().numpy(), ref[name], err_msg="%s after %s" % (name, ins[0]))
+    perm = torch.randperm(batch, generator=torch.Generator().manual_seed(seed)).cuda()
+    x.copy_(x[perm])
+    again = replay()
+    torch.cuda.synchronize()
+    for name in ("logits_q", "logits"):
+        assert torch.equal(again[name], out[name][perm]), name
+    assert out["logits_q"].min() < out["logits_q"].max()
+    runner.close()
