@@ -30,7 +30,7 @@ EXPORTS = [
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
     "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_match_residual_add",
-    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_cast",
+    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_cast", "chx_hip_count_nonfinite",
 ]
 
 

@@ -383,7 +383,9 @@ def set_option(name, value):
     "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards);
     "chrome_tracing" = file that every later run writes its per-instruction timeline to, "" = off;
     "dump_outputs_dir" = directory that every later run writes the instructions' named array
-    outputs to as .npy files, "" = off."""
+    outputs to as .npy files, "" = off;
+    "check_nans" / "check_infs" = "on" | "off" (default): every later run scans the results of each
+    instruction and fails, naming the instruction's operands and results, at the first NaN / Inf."""
     _check(runtime().chxvm_set_option(name.encode(), value.encode()))
 
 

@@ -4,6 +4,8 @@
 // conversions (Cast: int32 -> float32 for the scale-back, float32 -> uint8 / int8 for a computed
 // zero point).  Both take any strides; neither is on the timed path of a statically quantized
 // network.
+#include <vector>
+
 #include "chx_internal.h"
 
 namespace chx {
@@ -75,6 +77,25 @@ __global__ __launch_bounds__(kThreads) void cast_kernel(const char* __restrict__
     *reinterpret_cast<To*>(y + strided_offset(i, yd)) = static_cast<To>(*reinterpret_cast<const From*>(x + strided_offset(i, xd)));
 }
 
+// NaN: the only value that differs from itself; Inf: |x| equal to the largest exponent with a zero
+// mantissa (chainerx::IsNan / IsInf of the reference's scans)
+template <bool kInf>
+__global__ __launch_bounds__(kThreads) void count_nonfinite_kernel(const char* __restrict__ x, StridedDesc xd, int64_t n, uint32_t* __restrict__ partial) {
+    __shared__ uint32_t red[kThreads];
+    uint32_t found = 0;  // a block looks at fewer than 2^32 elements
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+        const uint32_t bits = *reinterpret_cast<const uint32_t*>(x + strided_offset(i, xd)) & 0x7fffffffu;
+        found += kInf ? (bits == 0x7f800000u) : (bits > 0x7f800000u);
+    }
+    red[threadIdx.x] = found;
+    __syncthreads();
+    for (int s = kThreads / 2; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) partial[blockIdx.x] = red[0];
+}
+
 template <class From>
 int cast_from(const chx_hip_tensor& x, chx_hip_tensor& y, int64_t n, hipStream_t s) {
     const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads);
@@ -136,4 +157,36 @@ extern "C" int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* st
         case CHX_HIP_INT8: return cast_from<int8_t>(*x, *y, n, s);
         default: CHX_FAIL(CHX_HIP_EUNSUPPORTED, "Cast: no conversion from %s on the device", dtype_name(x->dtype));
     }
+}
+
+extern "C" int chx_hip_count_nonfinite(const chx_hip_tensor* x, int32_t infinities, int64_t* count, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "non-finite scan x"));
+    CHX_REQUIRE(count != nullptr, "non-finite scan: count is null");
+    *count = 0;
+    if (x->dtype != CHX_HIP_FLOAT32) return CHX_HIP_OK;  // integers hold neither
+    const int64_t n = numel(*x);
+    if (n == 0) return CHX_HIP_OK;
+    hipStream_t s = as_stream(stream);
+    int blocks = (int)((n + kThreads * 8 - 1) / (kThreads * 8));
+    blocks = blocks < 1 ? 1 : blocks > 2048 ? 2048 : blocks;
+    CHX_REQUIRE(n / blocks < (int64_t(1) << 32) - kThreads, "non-finite scan: array too large");
+    void* dev = nullptr;
+    CHX_PROPAGATE(scratch_alloc(&dev, sizeof(uint32_t) * blocks, s));
+    const StridedDesc xd = make_desc(*x);
+    // every block writes its own count: nothing to clear beforehand, no atomics
+    if (infinities) count_nonfinite_kernel<true><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, static_cast<uint32_t*>(dev));
+    else count_nonfinite_kernel<false><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, static_cast<uint32_t*>(dev));
+    int rc = launch_check("count_nonfinite_kernel");
+    std::vector<uint32_t> partial((size_t)blocks);
+    if (rc == CHX_HIP_OK && (hipMemcpyAsync(partial.data(), dev, sizeof(uint32_t) * blocks, hipMemcpyDeviceToHost, s) != hipSuccess ||
+                             hipStreamSynchronize(s) != hipSuccess)) {
+        (void)hipGetLastError();
+        rc = CHX_HIP_ERUNTIME;
+    }
+    scratch_free(dev, s);
+    if (rc != CHX_HIP_OK) CHX_FAIL(rc, "non-finite scan: reading the counts back failed");
+    int64_t host = 0;
+    for (uint32_t c : partial) host += c;
+    *count = host;
+    return CHX_HIP_OK;
 }

@@ -69,6 +69,8 @@ def main(argv=None):
     ap.add_argument("--dump_onnx", default="", help="write the graph after the passes to this file")
     ap.add_argument("--chrome_tracing", default="", help="write a per-instruction timeline (Chrome tracing format) of the last run")
     ap.add_argument("--dump_outputs_dir", default="", help="write every named array output of every instruction there as .npy")
+    ap.add_argument("--check_nans", action="store_true", help="check for NaNs after each operation")
+    ap.add_argument("--check_infs", action="store_true", help="check for infinities after each operation")
     ap.add_argument("--report_json", default="", help="write {\"elapsed_times\": [msec, ...]} (the first of several runs dropped)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args(argv)
@@ -97,6 +99,8 @@ def main(argv=None):
         os.makedirs(args.dump_outputs_dir, exist_ok=True)
     vm.set_option("chrome_tracing", args.chrome_tracing)
     vm.set_option("dump_outputs_dir", args.dump_outputs_dir)
+    vm.set_option("check_nans", "on" if args.check_nans else "off")
+    vm.set_option("check_infs", "on" if args.check_infs else "off")
     failed = 0
     elapsed_times = []
     for name, inputs, wants in data_sets:
@@ -126,6 +130,8 @@ def main(argv=None):
     program.close()
     vm.set_option("chrome_tracing", "")
     vm.set_option("dump_outputs_dir", "")
+    vm.set_option("check_nans", "off")
+    vm.set_option("check_infs", "off")
     if args.report_json:
         import json
         with open(args.report_json, "w") as f:   # tools/run_onnx.cc:493-498

@@ -16,6 +16,7 @@ namespace {
 thread_local std::string g_last_error;
 // run options of chxvm_set_option, applied by every later chxvm_program_run
 std::string g_chrome_tracing_path, g_dump_outputs_dir;
+bool g_check_nans = false, g_check_infs = false;
 
 template <class Fn>
 int32_t Guard(Fn fn) {
@@ -130,6 +131,8 @@ int32_t chxvm_program_run(
         ChxVMOptions options;
         options.trace_level = trace_level;
         options.dump_outputs_dir = g_dump_outputs_dir;
+        options.check_nans = g_check_nans;
+        options.check_infs = g_check_infs;
         std::unique_ptr<ChromeTracingEmitter> tracing;
         if (!g_chrome_tracing_path.empty()) {
             tracing.reset(new ChromeTracingEmitter());
@@ -180,6 +183,9 @@ int32_t chxvm_set_option(const char* name, const char* value) {
             g_chrome_tracing_path = v;
         } else if (n == "dump_outputs_dir") {
             g_dump_outputs_dir = v;
+        } else if (n == "check_nans" || n == "check_infs") {  // --check_nans / --check_infs of tools/run_onnx.cc
+            CHECK(v == "on" || v == "off") << n << " is 'on' or 'off', got " << v;
+            (n == "check_nans" ? g_check_nans : g_check_infs) = v == "on";
         } else {
             CHECK(false) << "unknown option " << n;
         }

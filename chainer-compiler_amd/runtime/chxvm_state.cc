@@ -1,5 +1,6 @@
 #include "chxvm_state.h"
 
+#include <iostream>
 #include <sstream>
 
 namespace chainer_compiler {
@@ -81,9 +82,46 @@ std::string ChxVMState::GetVarString(int index) {
 }
 
 std::string ChxVMState::GetVarListString(const std::vector<int>& indices) {
-    std::ostringstream oss;
-    for (int i : indices) oss << " $" << i << "=" << GetVarString(i);
+    std::ostringstream oss;  // "[a, b]" as runtime/chxvm_state.cc:147-167 prints a list
+    oss << '[';
+    for (size_t i = 0; i < indices.size(); ++i) oss << (i ? ", " : "") << GetVarString(indices[i]);
+    oss << ']';
     return oss.str();
+}
+
+namespace {
+
+bool HasNonFinite(const ChxVMVar& var, bool infinities) {
+    if (var.kind() != ChxVMVar::Kind::kArray) return false;  // scalars live on the host and are what the program says
+    const chainerx::Array& a = var.GetArray();
+    if (a.dtype() != chainerx::Dtype::kFloat32 || a.GetTotalSize() == 0) return false;
+    chx_hip_tensor t = a.hip();
+    int64_t count = 0;
+    CHXVM_HIP_CALL(chx_hip_count_nonfinite(&t, infinities ? 1 : 0, &count, nullptr));
+    return count != 0;
+}
+
+}  // namespace
+
+void ChxVMState::CheckNonFinite(const std::vector<int>& inputs, const std::vector<int>& outputs, bool infinities) {
+    for (int output : outputs) {
+        if (output < 0) continue;
+        if (!HasNonFinite(*GetVar(output), infinities)) continue;
+        std::ostringstream oss;
+        oss << (infinities ? "Inf" : "NaN") << " detected!\n";
+        for (size_t i = 0; i < inputs.size(); ++i) oss << "input #" << i << ": " << GetVarString(inputs[i]) << "\n";
+        for (size_t i = 0; i < outputs.size(); ++i) oss << "output #" << i << ": " << GetVarString(outputs[i]) << "\n";
+        std::cerr << oss.str();
+        CHECK(false) << oss.str();
+    }
+}
+
+void ChxVMState::CheckNans(const std::vector<int>& inputs, const std::vector<int>& outputs) {
+    CheckNonFinite(inputs, outputs, false);
+}
+
+void ChxVMState::CheckInfs(const std::vector<int>& inputs, const std::vector<int>& outputs) {
+    CheckNonFinite(inputs, outputs, true);
 }
 
 void ChxVMState::Input(const std::string& name, int index) {

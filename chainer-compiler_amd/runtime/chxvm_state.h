@@ -68,12 +68,11 @@ public:
         return outputs_;
     }
 
-    // NaN/Inf scans of the reference (runtime/chxvm_state.cc:245-263) are float-only debugging
-    // aids; the quantized path keeps the switches but has nothing to scan.
-    void CheckNans(const std::vector<int>&, const std::vector<int>&) {
-    }
-    void CheckInfs(const std::vector<int>&, const std::vector<int>&) {
-    }
+    // Scans of an instruction's outputs for NaN / Inf elements (runtime/chxvm_state.cc:202-263): a hit
+    // prints every operand and result of the instruction and fails the run.  float32 arrays are
+    // scanned on the device; the 8-bit and int32 arrays of the quantized path hold neither.
+    void CheckNans(const std::vector<int>& inputs, const std::vector<int>& outputs);
+    void CheckInfs(const std::vector<int>& inputs, const std::vector<int>& outputs);
 
     int trace_level() const {
         return options_.trace_level;
@@ -89,6 +88,8 @@ public:
     }
 
 private:
+    void CheckNonFinite(const std::vector<int>& inputs, const std::vector<int>& outputs, bool infinities);
+
     int pc_ = 0;
     std::vector<std::unique_ptr<ChxVMVar>> variables_;
     InOuts inputs_;

@@ -254,6 +254,13 @@ int chx_hip_elementwise_source(
  * any strides; y float32 with one element. */
 int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream);
 
+/* The scan behind ChxVMState::CheckNans / CheckInfs (runtime/chxvm_state.cc:215-263: chainerx::IsNan / IsInf,
+ * Sum, AsScalar): *count receives the number of NaN elements of x (infinities = 0) or of +-Inf elements
+ * (infinities != 0).  float32 arrays with any strides are scanned, other element types hold neither and
+ * give 0.  Synchronizes the stream (the caller acts on the count), so it is a debugging aid and stays out
+ * of captured graphs. */
+int chx_hip_count_nonfinite(const chx_hip_tensor* x, int32_t infinities, int64_t* count, void* stream);
+
 /* CastOp::RunImpl (runtime/ops/manipulation.cc:157-159, CastTo): element types float32,
  * int32, uint8, int8 on either side; float -> integer truncates toward zero. */
 int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream);

@@ -128,6 +128,14 @@ def test_generated_run_glue_has_null_skip_and_trace(generated):
     assert "st->SetArray(y, RunImpl(st, st->GetArray(x), st->GetScalar(y_scale), st->GetOptionalScalar(y_zero_point)))" in \
         body.replace("\n", " ").replace("  ", " ") or "RunImpl(st, st->GetArray(x)" in body
     assert "MakeChxVMOp" in src and "case 139:" in src or "QuantizeLinearOp(inst)" in src
+    # the trace lines of runtime/gen_chxvm.py:190-236,309-318 and the scans of :321-328, after the call
+    flat = body.replace("\n", " ")
+    assert '"$" << y << " = " << "QuantizeLinear("' in flat and 'st->GetVarString(x) << " ->"' in flat
+    call = flat.index("RunImpl(")
+    assert flat.index('st->GetVarString(y) << std::endl', call) < flat.index("st->check_infs()", call) < flat.index("st->check_nans()", call)
+    assert "st->CheckInfs({x}, {y});" in flat and "st->CheckNans({x}, {y});" in flat
+    lst = re.search(r"void ElementWiseNvrtcOp::Run\(ChxVMState\* st\) \{(.*?)\n\}\n", src, flags=re.S).group(1)
+    assert "st->CheckNans({}, outputs);" in lst and "ArrayListToString(inputs)" in lst
 
 
 # ---- wire format ------------------------------------------------------------------------------

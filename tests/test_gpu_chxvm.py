@@ -301,3 +301,59 @@ def test_unfused_pool_is_refused_at_load(g, vm):
     b.output("y", y)
     with pytest.raises(vm.ChxVMError, match="MaxPool"):
         vm.Program(b.serialize())
+
+
+def test_nan_and_inf_scans(g, vm, capsys):
+    """check_nans / check_infs (runtime/chxvm_state.cc:202-263): off by default; when on, the first
+    instruction whose result holds a NaN / an Inf fails the run and names its operands."""
+    b = vm.ProgramBuilder()
+    x = b.input("x", "uint8", (4, 6))
+    d = b.DequantizeLinear(x, b.scalar(float("inf"), "float32"), b.scalar(3, "uint8"))   # (x - 3) * inf
+    b.output("d", d)
+    prog = vm.Program(b.serialize())
+    xv = np.full((4, 6), 9, np.uint8)
+    xv[2, 5] = 3                                            # 0 * inf = NaN
+    try:
+        out = prog.run({"x": g.dev(xv)})["d"]
+        assert np.isnan(out[2, 5]) and np.isinf(out).sum() == 23
+        vm.set_option("check_infs", "on")
+        with pytest.raises(vm.ChxVMError, match=r"Inf detected!(.|\n)*input #0: uint8\(4, 6\)(.|\n)*output #0: float32\(4, 6\)"):
+            prog.run({"x": g.dev(xv)})
+        vm.set_option("check_infs", "off")
+        vm.set_option("check_nans", "on")
+        with pytest.raises(vm.ChxVMError, match="NaN detected!"):
+            prog.run({"x": g.dev(xv)})
+        xv[2, 5] = 4                                        # no NaN left: the NaN scan passes, Inf is not its business
+        assert np.isinf(prog.run({"x": g.dev(xv)})["d"]).all()
+        with pytest.raises(vm.ChxVMError, match="'on' or 'off'"):
+            vm.set_option("check_nans", "1")
+    finally:
+        vm.set_option("check_nans", "off")
+        vm.set_option("check_infs", "off")
+        prog.close()
+
+
+def test_count_nonfinite_entry_point(g):
+    """chx_hip_count_nonfinite on dense and strided float32 arrays; other element types count 0."""
+    import ctypes
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((37, 2, 129)).astype(np.float32)
+    a[3, 1, 7] = np.nan
+    a[36, 0, 128] = -np.nan
+    a[0, 0, 0] = np.inf
+    a[5, 1, 100] = -np.inf
+    a[6, 1, 101] = np.inf
+    a[7, 0, 1] = np.float32(3.4028235e38)                    # largest finite value: neither
+    t = g.dev(a)
+
+    def count(tensor, infinities):
+        n = ctypes.c_int64(-1)
+        g.capi.check(g.capi.lib().chx_hip_count_nonfinite(g.capi.ref(tensor), ctypes.c_int32(infinities), ctypes.byref(n), g.capi.stream_ptr()))
+        return n.value
+    assert (count(t, 0), count(t, 1)) == (2, 3)
+    view = t[:, 1, ::2]                                      # strided: row 1 of every pair, even columns
+    assert (count(view, 0), count(view, 1)) == (int(np.isnan(a[:, 1, ::2]).sum()), int(np.isinf(a[:, 1, ::2]).sum())) == (0, 1)
+    assert count(g.dev(np.arange(12, dtype=np.int32)), 0) == 0 and count(t[:0], 1) == 0
+    big = torch.zeros(3_000_001, device="cuda")
+    big[::1000] = float("inf")
+    assert count(big, 1) == 3001 and count(big, 0) == 0
