@@ -239,7 +239,9 @@ class ProgramBuilder:
             raise AttributeError(name)
         return lambda *args, **kw: self.add(name, *args, **kw)
 
-    def add(self, name, *args, outputs=None, debug_info="", num_list_outputs=None):
+    def add(self, name, *args, outputs=None, debug_info="", num_list_outputs=None, output_types=(), output_names=()):
+        """output_types: (dtype number, shape) per output, output_names: their names; what a compiler
+        declares for the run-time type check and the output dumps."""
         number, ins, outs = self.index[name]
         if ins is None:
             raise ChxVMError("op %s has no signature in the op table of this runtime" % name)
@@ -268,7 +270,8 @@ class ProgramBuilder:
         flat = []
         for o in outputs:
             flat.extend(o if isinstance(o, (list, tuple)) else [o])
-        self.instructions.append(encode_instruction(number, enc, flat, debug_info=debug_info, id=self.next_id))
+        self.instructions.append(encode_instruction(number, enc, flat, debug_info=debug_info, id=self.next_id,
+                                                    output_types=output_types, output_names=output_names))
         self.next_id += 1
         if not outputs:
             return None
@@ -385,7 +388,11 @@ def set_option(name, value):
     "dump_outputs_dir" = directory that every later run writes the instructions' named array
     outputs to as .npy files, "" = off;
     "check_nans" / "check_infs" = "on" | "off" (default): every later run scans the results of each
-    instruction and fails, naming the instruction's operands and results, at the first NaN / Inf."""
+    instruction and fails, naming the instruction's operands and results, at the first NaN / Inf;
+    "check_types" = "on" | "off" (default): the inputs are checked against the program's input types
+    and every typed result against the dtype and shape its instruction declares;
+    "dump_memory_usage" = "0" (default) | "1" (bytes per variable slot and the peak, after the run) |
+    "2" (also the bytes held after every instruction)."""
     _check(runtime().chxvm_set_option(name.encode(), value.encode()))
 
 

@@ -221,6 +221,20 @@ private:
         inst->inputs.push_back(StringIn(auto_pad));
     }
 
+    // The type a result is declared with, for the run-time check of every typed result
+    // (compiler/chxvm/chxvm_value.cc:22-33): dtype and shape when both are known, else untyped.
+    static ChxVMTypeProto TypeOf(const Value* v) {
+        ChxVMTypeProto type;
+        const Type& t = v->type();
+        bool known = t.dtype != kUnknown && t.has_dims;
+        for (int64_t d : t.dims) known = known && d > 0;  // 0 and -1 stand for an unknown extent
+        if (known) {
+            type.set_dtype(t.dtype);
+            for (int64_t d : t.dims) type.shape.push_back(static_cast<int32_t>(d));
+        }
+        return type;
+    }
+
     void EmitNode(const Node& n) {
         const std::string& op = n.op_type();
         const size_t nin = n.inputs().size();
@@ -246,6 +260,7 @@ private:
             inst->inputs.push_back(IntIn(n.chainer_fusion_group()));
             for (Value* o : n.outputs()) {
                 inst->outputs.push_back(IdOf(o));
+                inst->output_types.push_back(TypeOf(o));
                 inst->output_names.push_back(o->name());
             }
             return;
@@ -256,6 +271,7 @@ private:
             ChxVMInstructionProto* inst = Add(name, dbg);
             inst->inputs = std::move(inputs);
             inst->outputs.push_back(IdOf(out));
+            inst->output_types.push_back(TypeOf(out));
             inst->output_names.push_back(out->name());  // names the per-op output dumps (compiler/chxvm/emitter.cc:72-77)
             return inst;
         };

@@ -69,6 +69,8 @@ def main(argv=None):
     ap.add_argument("--dump_onnx", default="", help="write the graph after the passes to this file")
     ap.add_argument("--chrome_tracing", default="", help="write a per-instruction timeline (Chrome tracing format) of the last run")
     ap.add_argument("--dump_outputs_dir", default="", help="write every named array output of every instruction there as .npy")
+    ap.add_argument("--check_types", action="store_true", help="check dtype and shape of the inputs and of every typed result")
+    ap.add_argument("--dump_memory_usage", type=int, default=0, choices=[0, 1, 2], help="1: peak memory held by the variables, 2: after every instruction too")
     ap.add_argument("--check_nans", action="store_true", help="check for NaNs after each operation")
     ap.add_argument("--check_infs", action="store_true", help="check for infinities after each operation")
     ap.add_argument("--report_json", default="", help="write {\"elapsed_times\": [msec, ...]} (the first of several runs dropped)")
@@ -100,6 +102,8 @@ def main(argv=None):
     vm.set_option("chrome_tracing", args.chrome_tracing)
     vm.set_option("dump_outputs_dir", args.dump_outputs_dir)
     vm.set_option("check_nans", "on" if args.check_nans else "off")
+    vm.set_option("check_types", "on" if args.check_types else "off")
+    vm.set_option("dump_memory_usage", str(args.dump_memory_usage))
     vm.set_option("check_infs", "on" if args.check_infs else "off")
     failed = 0
     elapsed_times = []
@@ -132,6 +136,8 @@ def main(argv=None):
     vm.set_option("dump_outputs_dir", "")
     vm.set_option("check_nans", "off")
     vm.set_option("check_infs", "off")
+    vm.set_option("check_types", "off")
+    vm.set_option("dump_memory_usage", "0")
     if args.report_json:
         import json
         with open(args.report_json, "w") as f:   # tools/run_onnx.cc:493-498

@@ -228,7 +228,7 @@ int CountUses(const ChxVMProgramProto& program, int slot) {
 
 }  // namespace
 
-ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_names) {
+ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_names), input_types_(program.input_types) {
     // number of variable slots = highest id mentioned + 1 (runtime/chxvm.cc:104-140)
     int max_id = -1;
     for (const ChxVMInstructionProto& inst : program.instructions) {
@@ -455,12 +455,54 @@ void DumpOutput(ChxVMState* st, const ChxVMOp* op, const std::string& output_dir
     }
 }
 
+chainerx::Shape ShapeOf(const ChxVMTypeProto& type) {
+    return chainerx::Shape(type.shape.begin(), type.shape.end());
+}
+
+// runtime/chxvm.cc:38-64: an instruction that names its outputs also types them; dtype 0 = untyped
+void CheckType(ChxVMState* st, const ChxVMOp* op) {
+    const ChxVMInstructionProto& inst = op->instruction();
+    if (inst.output_names.empty()) return;
+    CHECK_EQ(inst.outputs.size(), inst.output_types.size()) << op->name() << ": " << op->debug_info();
+    for (size_t i = 0; i < inst.outputs.size(); ++i) {
+        const ChxVMTypeProto& type = inst.output_types[i];
+        if (type.dtype == 0) continue;
+        const int id = inst.outputs[i];
+        CHECK_LT(0, id);
+        ChxVMVar* var = st->GetVar(id);
+        if (var->IsNull()) continue;
+        const chainerx::Array& a = st->GetArray(id);
+        CHECK_EQ(static_cast<chainerx::Dtype>(type.dtype), a.dtype()) << "Dtype check failed in output #" << i << ": " << op->debug_info();
+        CHECK_EQ(ShapeOf(type), a.shape()) << "Shape check failed in output #" << i << ": " << op->debug_info();
+    }
+}
+
+int64_t InMbs(int64_t bytes) {
+    return bytes / 1000 / 1000;
+}
+
 }  // namespace
 
 InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
-    for (const std::string& name : input_names_)
-        CHECK(program_inputs.count(name)) << "Input '" << name << "' not found";  // runtime/chxvm.cc:142-143
+    CHECK_EQ(input_names_.size(), input_types_.size());
+    for (size_t i = 0; i < input_names_.size(); ++i) {
+        const std::string& name = input_names_[i];
+        auto found = program_inputs.find(name);
+        CHECK(found != program_inputs.end()) << "Input '" << name << "' not found";  // runtime/chxvm.cc:142-143
+        if (!options.check_types) continue;
+        const ChxVMTypeProto& type = input_types_[i];
+        const ChxVMVar& var = *found->second;
+        if (var.IsArray()) {
+            if (type.dtype == 0) continue;
+            const chainerx::Array& a = var.GetArray();
+            CHECK_EQ(static_cast<chainerx::Dtype>(type.dtype), a.dtype()) << "Input '" << name << "' has an unexpected dtype";
+            CHECK_EQ(ShapeOf(type), a.shape()) << "Input '" << name << "' has an unexpected shape";
+        } else {
+            CHECK_EQ(0, type.dtype) << "Input '" << name << "' must be a tensor";
+        }
+    }
     ChxVMState state(options, num_variables_, program_inputs);
+    int64_t peak_used_mbs = 0;
     while (state.pc() < static_cast<int>(program_.size())) {
         const int pc = state.pc();
         ChxVMOp* op = program_[pc].get();
@@ -477,7 +519,17 @@ InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
             options.chrome_tracing->End(event);
         }
         state.set_pc(state.pc() + 1);  // jumps set pc - 1 themselves (runtime/ops/controlflow.cc:7-21)
+        if (options.check_types) CheckType(&state, op);
         if (!options.dump_outputs_dir.empty()) DumpOutput(&state, op, options.dump_outputs_dir);
+        if (options.dump_memory_usage >= 1) {
+            const int64_t used_mbs = InMbs(state.GetTotalVariableSize());
+            peak_used_mbs = std::max(peak_used_mbs, used_mbs);
+            if (options.dump_memory_usage >= 2) std::cerr << " Memory usage=" << used_mbs << "MB" << std::endl;
+        }
+    }
+    if (options.dump_memory_usage >= 1) {
+        state.ShowVariableStatus();
+        std::cerr << "Peak memory usage=" << peak_used_mbs << "MB" << std::endl;
     }
     return state.GetOutputs();
 }

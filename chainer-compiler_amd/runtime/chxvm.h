@@ -55,6 +55,7 @@ public:
 private:
     std::vector<std::unique_ptr<ChxVMOp>> program_;
     std::vector<std::string> input_names_;
+    std::vector<ChxVMTypeProto> input_types_;
     int num_variables_ = 0;
 };
 

@@ -16,7 +16,8 @@ namespace {
 thread_local std::string g_last_error;
 // run options of chxvm_set_option, applied by every later chxvm_program_run
 std::string g_chrome_tracing_path, g_dump_outputs_dir;
-bool g_check_nans = false, g_check_infs = false;
+bool g_check_nans = false, g_check_infs = false, g_check_types = false;
+int g_dump_memory_usage = 0;
 
 template <class Fn>
 int32_t Guard(Fn fn) {
@@ -133,6 +134,8 @@ int32_t chxvm_program_run(
         options.dump_outputs_dir = g_dump_outputs_dir;
         options.check_nans = g_check_nans;
         options.check_infs = g_check_infs;
+        options.check_types = g_check_types;
+        options.dump_memory_usage = g_dump_memory_usage;
         std::unique_ptr<ChromeTracingEmitter> tracing;
         if (!g_chrome_tracing_path.empty()) {
             tracing.reset(new ChromeTracingEmitter());
@@ -183,9 +186,12 @@ int32_t chxvm_set_option(const char* name, const char* value) {
             g_chrome_tracing_path = v;
         } else if (n == "dump_outputs_dir") {
             g_dump_outputs_dir = v;
-        } else if (n == "check_nans" || n == "check_infs") {  // --check_nans / --check_infs of tools/run_onnx.cc
+        } else if (n == "check_nans" || n == "check_infs" || n == "check_types") {  // the flags of the same names of tools/run_onnx.cc
             CHECK(v == "on" || v == "off") << n << " is 'on' or 'off', got " << v;
-            (n == "check_nans" ? g_check_nans : g_check_infs) = v == "on";
+            (n == "check_nans" ? g_check_nans : n == "check_infs" ? g_check_infs : g_check_types) = v == "on";
+        } else if (n == "dump_memory_usage") {
+            CHECK(v == "0" || v == "1" || v == "2") << "dump_memory_usage is 0, 1 or 2, got " << v;
+            g_dump_memory_usage = v[0] - '0';
         } else {
             CHECK(false) << "unknown option " << n;
         }

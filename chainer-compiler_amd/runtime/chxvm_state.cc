@@ -1,6 +1,8 @@
 #include "chxvm_state.h"
 
+#include <algorithm>
 #include <iostream>
+#include <map>
 #include <sstream>
 
 namespace chainer_compiler {
@@ -122,6 +124,27 @@ void ChxVMState::CheckNans(const std::vector<int>& inputs, const std::vector<int
 
 void ChxVMState::CheckInfs(const std::vector<int>& inputs, const std::vector<int>& outputs) {
     CheckNonFinite(inputs, outputs, true);
+}
+
+int64_t ChxVMState::GetTotalVariableSize() const {
+    std::map<const void*, int64_t> sizes;
+    for (const auto& v : variables_) {
+        if (!v || !v->IsArray()) continue;
+        const chainerx::Array& a = v->GetArray();
+        if (a.IsNullHandle()) continue;
+        int64_t& bytes = sizes[a.raw_data()];
+        bytes = std::max(bytes, a.GetNBytes());
+    }
+    int64_t total = 0;
+    for (const auto& p : sizes) total += p.second;
+    return total;
+}
+
+void ChxVMState::ShowVariableStatus() const {
+    for (size_t i = 0; i < variables_.size(); ++i) {
+        if (!variables_[i]) continue;
+        std::cerr << "$" << i << ": " << variables_[i]->GetNBytes() << std::endl;
+    }
 }
 
 void ChxVMState::Input(const std::string& name, int index) {

@@ -19,8 +19,14 @@ class ChromeTracingEmitter;
 struct ChxVMOptions {
     int trace_level = 0;
     bool is_training = false;
+    // inputs against the program's input_types before the run, every typed result against the
+    // instruction's output_types after it (runtime/chxvm.cc:38-64,140-158)
+    bool check_types = false;
     bool check_nans = false;
     bool check_infs = false;
+    // 1: bytes held by the variable slots at their peak, printed after the run; 2: also after every
+    // instruction (runtime/chxvm.cc:208-237; the allocator hooks of the reference have no counterpart)
+    int dump_memory_usage = 0;
     // an event per executed instruction; the device is synchronized after each one so that an
     // event spans the instruction's kernels (runtime/chxvm.cc:180 times the host side only)
     ChromeTracingEmitter* chrome_tracing = nullptr;
@@ -63,6 +69,11 @@ public:
 
     void Input(const std::string& name, int index);
     void Output(const std::string& name, int index);
+
+    // bytes of device memory the variable slots keep alive, shared buffers counted once
+    // (runtime/chxvm_state.cc:274-290), and the per-slot list of runtime/chxvm_state.cc:265-272
+    int64_t GetTotalVariableSize() const;
+    void ShowVariableStatus() const;
 
     const InOuts& GetOutputs() const {
         return outputs_;

@@ -85,3 +85,43 @@ def test_run_onnx_parity_tooling(onnx_vectors, tmp_path):
     assert all(f[:5].isdigit() for f in files)
     times = json.load(open(report))["elapsed_times"]
     assert len(times) == 2 and all(t > 0 for t in times)
+
+
+def test_type_checks_and_memory_report(onnx_vectors, tmp_path, capfd):
+    """--check_types (runtime/chxvm.cc:38-64,140-158) and --dump_memory_usage (:208-237): every node
+    test passes with the checks on (the emitter declares each result's dtype and shape where the
+    graph knows them); an input of another shape, or a result that contradicts its declaration, fails."""
+    import gpu_util
+    import onnx_cases
+    ol = importlib.import_module(gpu_util.pkg.__name__ + ".onnx_lite")
+    run_onnx = importlib.import_module(gpu_util.pkg.__name__ + ".run_onnx")
+    vm = importlib.import_module(gpu_util.pkg.__name__ + ".chxvm")
+    cases = onnx_cases.build_cases(ol, onnx_vectors)
+    for name in ("test_qlinearconv", "test_dynamicquantizelinear_expanded", "test_qlinearmatmul_3D", "test_convinteger_with_padding"):
+        d = onnx_cases.write_case(ol, str(tmp_path), name, cases[name])
+        capfd.readouterr()
+        assert run_onnx.main(["--test", d, "--check_types", "--check_nans", "--check_infs", "--dump_memory_usage", "2"]) == 0, name
+        err = capfd.readouterr().err
+        import re
+        assert "Peak memory usage=" in err and " Memory usage=" in err and re.search(r"^\$\d+: \d+$", err, flags=re.M)   # slots alive at the end
+    # a program whose declarations are wrong
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (3, 5))
+    q = b.QuantizeLinear(x, b.scalar(0.5, "float32"), b.scalar(3, "uint8"), output_types=[(vm.DTYPE["uint8"], [3, 5])], output_names=["q"])
+    d = b.DequantizeLinear(q, b.scalar(0.5, "float32"), b.scalar(3, "uint8"), output_types=[(vm.DTYPE["float32"], [5, 3])],
+                           output_names=["d"], debug_info="the badly declared one")
+    b.output("q", q)
+    prog = vm.Program(b.serialize())
+    xv = np.zeros((3, 5), np.float32)
+    try:
+        vm.set_option("check_types", "on")
+        with pytest.raises(vm.ChxVMError, match="Shape check failed in output #0: the badly declared one"):
+            prog.run({"x": gpu_util.dev(xv)})
+        with pytest.raises(vm.ChxVMError, match="Input 'x' has an unexpected shape"):
+            prog.run({"x": gpu_util.dev(np.zeros((5, 3), np.float32))})
+        with pytest.raises(vm.ChxVMError, match="Input 'x' has an unexpected dtype"):
+            prog.run({"x": gpu_util.dev(np.zeros((3, 5), np.uint8))})
+    finally:
+        vm.set_option("check_types", "off")
+    assert prog.run({"x": gpu_util.dev(np.zeros((5, 3), np.float32))})["q"].shape == (5, 3)   # unchecked by default, as in the reference
+    prog.close()
