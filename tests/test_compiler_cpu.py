@@ -195,35 +195,7 @@ def test_quantize_dequantize_parameters_are_written_into_the_group(vm):
 
 def decode_program(vm, data):
     """[(op name, [(value type name, value)], outputs)] of a serialized program."""
-    names = {v: k for k, v in vm.VALUE_TYPE.items()}
-    out = []
-    for f, w, v in onnx_lite.fields(data):
-        if f != 1:
-            continue
-        op, ins, outs = None, [], []
-        for f2, w2, v2 in onnx_lite.fields(v):
-            if f2 == 1:
-                op = vm.op_name(v2)
-            elif f2 == 2:
-                typ, val, lst = None, None, []
-                for f3, w3, v3 in onnx_lite.fields(v2):
-                    if f3 == 1:
-                        typ = names[v3]
-                    elif f3 in (2, 3, 8, 11, 12, 13):
-                        val = v3 - (1 << 64) if v3 >= 1 << 63 else v3
-                    elif f3 == 4:
-                        val = np.frombuffer(v3, "<f8")[0]
-                    elif f3 == 6:
-                        val = bytes(v3).decode()
-                    elif f3 in (5, 7):
-                        lst.append(v3 - (1 << 64) if v3 >= 1 << 63 else v3)
-                    elif f3 == 10:
-                        lst.append(float(np.frombuffer(v3, "<f8")[0]))
-                ins.append((typ, lst if typ in ("INTS", "INT_VALUES", "ARRAY_LIST", "DOUBLES") else val))
-            elif f2 == 3:
-                outs.append(v2 - (1 << 64) if v2 >= 1 << 63 else v2)
-        out.append((op, ins, outs))
-    return out
+    return vm.decode_program(data)
 
 
 def numpy_quantize(data, dtype):

@@ -100,7 +100,7 @@ def test_type_checks_and_memory_report(onnx_vectors, tmp_path, capfd):
     for name in ("test_qlinearconv", "test_dynamicquantizelinear_expanded", "test_qlinearmatmul_3D", "test_convinteger_with_padding"):
         d = onnx_cases.write_case(ol, str(tmp_path), name, cases[name])
         capfd.readouterr()
-        assert run_onnx.main(["--test", d, "--check_types", "--check_nans", "--check_infs", "--dump_memory_usage", "2"]) == 0, name
+        assert run_onnx.main(["--test", d, "--check_nans", "--check_infs", "--dump_memory_usage", "2"]) == 0, name   # types: checked by default
         err = capfd.readouterr().err
         import re
         assert "Peak memory usage=" in err and " Memory usage=" in err and re.search(r"^\$\d+: \d+$", err, flags=re.M)   # slots alive at the end
@@ -125,3 +125,33 @@ def test_type_checks_and_memory_report(onnx_vectors, tmp_path, capfd):
         vm.set_option("check_types", "off")
     assert prog.run({"x": gpu_util.dev(np.zeros((5, 3), np.float32))})["q"].shape == (5, 3)   # unchecked by default, as in the reference
     prog.close()
+
+
+def test_run_onnx_compile_flags(onnx_vectors, tmp_path, capsys):
+    """--compile_only, --out_chxvm, --dump_chxvm, --out_onnx, --no_check_values, --skip_runtime_type_check
+    (tools/run_onnx.cc:294-310)."""
+    import gpu_util
+    import onnx_cases
+    ol = importlib.import_module(gpu_util.pkg.__name__ + ".onnx_lite")
+    run_onnx = importlib.import_module(gpu_util.pkg.__name__ + ".run_onnx")
+    vm = importlib.import_module(gpu_util.pkg.__name__ + ".chxvm")
+    cases = onnx_cases.build_cases(ol, onnx_vectors)
+    graph, inputs, outputs = cases["test_quantizelinear"]
+    d = onnx_cases.write_case(ol, str(tmp_path), "test_quantizelinear", cases["test_quantizelinear"])
+    prog_file, onnx_file = str(tmp_path / "p.chxvm"), str(tmp_path / "o.onnx")
+    capsys.readouterr()
+    assert run_onnx.main(["--test", d, "--compile_only", "--out_chxvm", prog_file, "--dump_chxvm", "--out_onnx", onnx_file]) == 0
+    listing = capsys.readouterr().out
+    assert "QuantizeLinear(" in listing and "-> $" in listing and "Out(" in listing
+    loaded = vm.Program(open(prog_file, "rb").read())            # the file is the program
+    out = loaded.run({n: gpu_util.dev(np.array(a, order="C")) for (n, _, _), a in zip(graph.inputs, inputs)})
+    np.testing.assert_array_equal(out[graph.outputs[0][0]], outputs[0])
+    loaded.close()
+    assert [n.op_type for n in ol.parse_model(open(onnx_file, "rb").read()).nodes] == ["QuantizeLinear"]
+    # wrong expectations on disk: fails, passes with --no_check_values
+    bad = (graph, inputs, [np.array(outputs[0]) ^ 1])
+    d2 = onnx_cases.write_case(ol, str(tmp_path / "bad"), "test_quantizelinear", bad)
+    assert run_onnx.main(["--test", d2]) == 1
+    assert run_onnx.main(["--test", d2, "--no_check_values", "--skip_runtime_type_check"]) == 0
+    assert run_onnx.mismatches(np.array([np.nan, 1.0], np.float32), np.array([np.nan, 1.0], np.float32), 1e-4, 1e-6, equal_nan=True) == 0
+    assert run_onnx.mismatches(np.array([np.nan, 1.0], np.float32), np.array([2.0, 1.0], np.float32), 1e-4, 1e-6, equal_nan=True) == 1
