@@ -55,12 +55,37 @@ Options ParseOptions(const char* text) {
     if (!text || !*text) return o;
     const Json j = Json::Parse(text);
     CHECK(j.is_object()) << "options must be a JSON object";
-    for (const auto& kv : j.items()) CHECK(kv.first == "quantize" || kv.first == "fuse") << "unknown option '" << kv.first << "'";
+    // Besides "fuse" and the "quantize" object, the compiler flags of the reference that concern this
+    // path are accepted under their own names (scripts/generate_flags_code.py:4-173; use_hip is the
+    // flag a hip back-end adds next to use_nvrtc): fuse_operations, use_hip, use_nvrtc, backend_name,
+    // quantize as a bool (its default mode, compiler/passes.cc:121-125), disable_per_channel_quantize.
+    static const char* const kKnown[] = {"quantize", "fuse", "fuse_operations", "use_hip", "use_nvrtc", "backend_name",
+                                         "disable_per_channel_quantize"};
+    for (const auto& kv : j.items()) {
+        bool known = false;
+        for (const char* k : kKnown) known = known || kv.first == k;
+        CHECK(known) << "unknown option '" << kv.first << "'";
+    }
+    if (const Json* b = j.find("backend_name")) CHECK(b->is_string() && b->string() == "hip") << "backend_name is 'hip' here";
     if (const Json* f = j.find("fuse")) {
         CHECK(f->is_string() && (f->string() == "hip" || f->string() == "nvrtc" || f->string() == "none")) << "fuse is 'hip', 'nvrtc' or 'none'";
         o.fuse = f->string();
+    } else if (j.find("fuse_operations") || j.find("use_hip") || j.find("use_nvrtc")) {
+        auto flag = [&](const char* name) {
+            const Json* v = j.find(name);
+            return v && v->boolean();
+        };
+        // groups are formed when fuse_operations is on; which generator they are built for follows
+        // the use_* flag (compiler/passes.cc:56-60, compiler/chxvm/emitter.cc:697-700)
+        o.fuse = !flag("fuse_operations") ? "none" : flag("use_nvrtc") && !flag("use_hip") ? "nvrtc" : "hip";
     }
-    if (const Json* q = j.find("quantize")) {
+    const Json* quantize = j.find("quantize");
+    if (quantize && !quantize->is_object()) {
+        o.quantize = quantize->boolean();
+        quantize = nullptr;
+    }
+    if (const Json* d = j.find("disable_per_channel_quantize")) o.q.per_channel = !d->boolean();
+    if (const Json* q = quantize) {
         CHECK(q->is_object()) << "quantize must be an object";
         o.quantize = true;
         for (const auto& kv : q->items()) {

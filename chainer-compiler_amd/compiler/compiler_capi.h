@@ -5,10 +5,13 @@
  *
  * options: a JSON document (// comments allowed), every member optional:
  *   {"quantize": {"mode": "IntegerOps" | "QLinearOps",      // default IntegerOps (compiler/passes.cc:121-125)
- *                 "per_channel": false, "static": false, "asymmetric_input_types": false,
+ *                 "per_channel": true, "static": false, "asymmetric_input_types": false,   // defaults of compiler/quantize.h:30-40
  *                 "inputs":  {"<value name>": {"scale": 0.02, "zero_point": 128}},
  *                 "outputs": {"<value name>": {"scale": 0.05, "zero_point": 128, "dtype": "uint8" | "int8"}}},
  *    "fuse": "hip" | "nvrtc" | "none"}                      // default "hip"; "nvrtc" = the reference's fusable set
+ * The reference's own flag names (scripts/generate_flags_code.py:4-173) are accepted as members too:
+ *   "quantize": true (the default mode), "disable_per_channel_quantize": bool, "backend_name": "hip", and, when
+ *   "fuse" is absent, "fuse_operations" with "use_hip" / "use_nvrtc" (no groups unless fuse_operations is true).
  */
 #pragma once
 

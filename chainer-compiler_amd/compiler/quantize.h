@@ -24,7 +24,7 @@ struct QuantizationParams {
 
 struct QuantizationOptions {
     int nbits = 8;
-    bool per_channel = false;
+    bool per_channel = true;  // compiler/quantize.h:34; --disable_per_channel_quantize clears it (compiler/passes.cc:123)
     bool is_static = false;
     bool asymmertic_input_types = false;  // (spelled as in the reference) int8 weights instead of uint8
     QuantizationMode mode = QuantizationMode::IntegerOps;

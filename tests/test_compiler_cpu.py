@@ -345,3 +345,34 @@ def test_emitted_program_for_a_quantized_convolution(vm):
         vm.compile_onnx(sm)
     with pytest.raises(vm.ChxVMError, match="unknown option"):
         vm.compile_onnx(sm, {"fuze": "hip"})
+
+
+def test_reference_flag_names_as_options(vm):
+    """The compiler flags of the reference that concern this path are accepted under their own names
+    (scripts/generate_flags_code.py:4-173; use_hip beside use_nvrtc): quantize as a bool selects the
+    default mode with per-channel weights (compiler/passes.cc:121-125, compiler/quantize.h:34),
+    disable_per_channel_quantize clears that; fuse_operations + use_hip / use_nvrtc choose the groups."""
+    rng = np.random.default_rng(9)
+    m, w = conv_model(rng)
+
+    def kinds(options):
+        return [n.op_type for n in onnx_lite.parse_model(vm.transform_onnx(m, options)[0]).nodes]
+    per_channel = kinds({"fuse_operations": False, "quantize": True})
+    assert per_channel == kinds({"fuse": "none", "quantize": {"per_channel": True}}) == kinds({"fuse": "none", "quantize": {}})
+    assert "Reshape" in per_channel and "ConvInteger" in per_channel               # [OC] scales reshaped to [OC, 1, 1]
+    per_tensor = kinds({"fuse_operations": False, "quantize": True, "disable_per_channel_quantize": True})
+    assert per_tensor == kinds({"fuse": "none", "quantize": {"per_channel": False}}) and "Reshape" not in per_tensor
+    assert kinds({"quantize": False, "fuse_operations": False}) == ["Conv"]
+    chain = model([("Tanh", ["x"], ["t"]), ("Sigmoid", ["t"], ["s"]), ("Relu", ["s"], ["y"])], [("x", (4, 5))], [("y", (4, 5))])
+
+    def groups(options):
+        return lines(vm.transform_onnx(chain, options)[1])
+    assert groups({"fuse_operations": True, "use_hip": True, "backend_name": "hip"}) == groups({"fuse": "hip"})
+    assert groups({"fuse_operations": True, "use_nvrtc": True}) == groups({"fuse": "nvrtc"})
+    assert groups({"fuse_operations": False, "use_hip": True}) == groups({"fuse": "none"})
+    assert [l.split("(")[0] for l in groups({"fuse": "none"})] == ["Tanh", "Sigmoid", "Relu"]
+    assert groups({"fuse": "hip"}) != groups({"fuse": "nvrtc"})                     # Relu is fusable for hip only
+    with pytest.raises(vm.ChxVMError, match="backend_name"):
+        vm.transform_onnx(chain, {"backend_name": "chxvm"})
+    with pytest.raises(vm.ChxVMError, match="unknown option 'use_tvm'"):
+        vm.transform_onnx(chain, {"use_tvm": True})
