@@ -35,6 +35,17 @@ def test_runtests_over_the_node_tests(onnx_vectors, tmp_path):
         assert "OK   %s" % name in log
     assert "FAIL zz_expected_failure" in log and "%d/%d tests passed" % (len(cases), len(cases) + 1) in log
     assert "1 of 6 elements differ" in log and "run_onnx.py --test" in log      # failure log + reproducing command
+    # the failure log names the failed case with its command and output; --failed reruns only what it lists
+    flog = open(os.path.join(str(tmp_path), "failed_tests.log")).read()
+    assert flog.startswith("=== zz_expected_failure ===\n$ ") and "1 of 6 elements differ" in flog and "see %s" % os.path.join(str(tmp_path), "failed_tests.log") in log
+    again = subprocess.run([sys.executable, os.path.join(ROOT, "chainer-compiler_amd", "runtests.py"), str(tmp_path), "--failed"],
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=300)
+    assert again.returncode == 1 and "[1/1] FAIL zz_expected_failure" in again.stdout.decode()
+    ok = subprocess.run([sys.executable, os.path.join(ROOT, "chainer-compiler_amd", "runtests.py"), str(tmp_path), "-k", "^test_(round|matmul)",
+                         "--show_log", "--verbose", "--no_fuse_operations"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=300)
+    text = ok.stdout.decode()
+    assert ok.returncode == 0 and "2/2 tests passed" in text and "OK   test_data_set_0/" in text
+    assert not os.path.exists(os.path.join(str(tmp_path), "failed_tests.log"))          # a clean run removes the stale list
 
 
 def test_run_onnx_in_process_with_iterations(onnx_vectors, tmp_path, capsys):
