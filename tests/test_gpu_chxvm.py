@@ -357,3 +357,26 @@ def test_count_nonfinite_entry_point(g):
     big = torch.zeros(3_000_001, device="cuda")
     big[::1000] = float("inf")
     assert count(big, 1) == 3001 and count(big, 0) == 0
+
+
+def test_trace_lines(g, vm, capfd):
+    """trace_level 1 prints, per instruction, the lines of the reference's generated glue
+    (runtime/gen_chxvm.py:190-236,309-318): "$out = Op($in, ...)", the array operands' dtype and shape,
+    " ->", the results' dtype and shape."""
+    import re
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (3, 5))
+    q = b.QuantizeLinear(x, b.scalar(0.5, "float32"), None, debug_info="the quantization")
+    b.output("q", q)
+    prog = vm.Program(b.serialize())
+    capfd.readouterr()
+    prog.run({"x": g.dev(np.ones((3, 5), np.float32))}, trace_level=1)
+    err = capfd.readouterr().err
+    prog.close()
+    assert re.search(r"^# the quantization\n\$%d = QuantizeLinear\(\$%d, \$\d+, \$-1\)\n \$%d=float32\(3, 5\) -> \$%d=uint8\(3, 5\)$" % (q, x, x, q),
+                     err, flags=re.M), err
+    assert re.search(r'^\$%d = In\("?name"?\)\n' % x, err, flags=re.M) and re.search(r"^Out\(.*\$%d\)$" % q, err, flags=re.M), err
+    prog = vm.Program(b.serialize())
+    prog.run({"x": g.dev(np.ones((3, 5), np.float32))})          # silent by default
+    assert capfd.readouterr().err == ""
+    prog.close()
