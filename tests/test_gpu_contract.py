@@ -471,3 +471,69 @@ def test_every_launch_configuration_of_the_matrix_core_kernel(g, oracle, tile):
             os.environ.pop("CHX_HIP_TILE", None)
         else:
             os.environ["CHX_HIP_TILE"] = before
+
+
+def test_random_convolution_sweep(g, oracle):
+    """Seeded random QLinearConv / ConvInteger configurations across every dispatch path (matrix-core
+    tiles, first-layer kernel, depthwise kernel, generic kernel): shapes, kernel sizes, strides, pads,
+    groups, element types, layouts, bias modes, per-tensor and per-channel scales; bit-exact."""
+    rng = np.random.default_rng(2024)
+    seen = 0
+    for trial in range(70):
+        kh, kw = (int(rng.choice([1, 2, 3, 5, 7])) for _ in range(2))
+        kind = trial % 5
+        if kind == 0:        # depthwise 3x3 and its neighbours
+            C = int(rng.integers(1, 80))
+            group, OC = C, C * int(rng.choice([1, 1, 1, 2]))
+            kh = kw = int(rng.choice([3, 3, 1, 5]))
+            if trial % 10 == 0:      # every other one in the form the depthwise kernel takes: channels in sixteens, 3x3
+                C = group = OC = 16 * int(rng.integers(1, 7))
+                kh = kw = 3
+        elif kind == 1:      # grouped
+            group = int(rng.choice([2, 3, 4]))
+            C, OC = group * int(rng.integers(1, 20)), group * int(rng.integers(1, 20))
+        elif kind == 2:      # few planar channels (first layer)
+            group, C, OC = 1, int(rng.integers(1, 5)), int(rng.integers(1, 70))
+        else:                # dense
+            group, C, OC = 1, int(rng.choice([8, 16, 24, 32, 48, 64, 72, 128, 160, 256, int(rng.integers(1, 200))])), int(rng.integers(1, 200))
+        H, W = int(rng.integers(1, 22)), int(rng.integers(1, 22))
+        sh, sw = int(rng.choice([1, 1, 2, 3])), int(rng.choice([1, 1, 2, 3]))
+        ph, pw = int(rng.integers(0, kh // 2 + 2)), int(rng.integers(0, kw // 2 + 2))
+        if H + 2 * ph < kh or W + 2 * pw < kw:
+            continue
+        N = int(rng.integers(1, 4))
+        xdt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        wdt = [np.int8, np.int8, np.uint8][int(rng.integers(0, 3))]
+        if kind == 0 and trial % 10 == 0:
+            wdt = np.int8
+        ydt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        x = rand_q(rng, (N, C, H, W), xdt)
+        w = rand_q(rng, (OC, C // group, kh, kw), wdt)
+        per_channel = bool(rng.integers(0, 2))
+        ws = rng.uniform(0.002, 0.02, size=OC if per_channel else 1).astype(np.float32)
+        wz = rand_q(rng, (OC if per_channel else 1,), wdt) if rng.integers(0, 3) == 0 else np.zeros(OC if per_channel else 1, wdt)
+        xz = int(rand_q(rng, (1,), xdt)[0])
+        yz = int(rand_q(rng, (1,), ydt)[0]) if rng.integers(0, 4) else 0
+        K = (C // group) * kh * kw
+        ys = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(K) / float(rng.choice([20, 60, 200])))
+        bias_mode = int(rng.integers(0, 3))
+        bias = rng.integers(-400, 401, size=OC).astype(np.int32)
+        kw_ = dict(strides=(sh, sw), pads=(ph, pw), group=group)
+        okw, flags, b = dict(kw_), 0, None
+        if bias_mode == 1:
+            b, okw["bias"], okw["bias_mode"] = bias, bias, oracle.BIAS_REFERENCE_FLOAT
+        elif bias_mode == 2:
+            b, okw["bias"], okw["bias_mode"], flags = bias, bias, oracle.BIAS_ONNX_INT32, g.capi.BIAS_ONNX_INT32
+        tag = "trial %d: x%s %s w%s %s strides %s pads %s group %d per_channel %s bias %d y %s" % (
+            trial, x.shape, xdt.__name__, w.shape, wdt.__name__, (sh, sw), (ph, pw), group, per_channel, bias_mode, ydt.__name__)
+        xd = g.dev(x) if rng.integers(0, 2) and not (kind == 0 and trial % 10 == 0) else g.to_channels_last(g.dev(x))
+        wsd, wzd = (g.dev(ws), g.dev(wz)) if per_channel else (g.dev(ws.reshape(())), g.dev(wz.reshape(())))
+        want = oracle.qlinear_conv_int(x, 0.02, xz, w, ws if per_channel else ws[:1], wz if per_channel else wz[:1], ys, yz, ydt, **okw)
+        got = g.ops.QLinearConv(xd, 0.02, xz, g.dev(w), wsd, wzd, ys, yz, None if b is None else g.dev(b),
+                                zero_point_dtype=TDT[ydt], flags=flags, **kw_)
+        np.testing.assert_array_equal(g.host(got), want, err_msg=tag)
+        want_i = oracle.conv_integer(x, w, xz, wz if per_channel else wz[:1], auto_pad="", **kw_)
+        got_i = g.ops.ConvInteger(xd, g.dev(w), xz, wzd if per_channel else g.dev(wz[:1].reshape(())), **kw_)
+        np.testing.assert_array_equal(g.host(got_i), want_i, err_msg=tag)
+        seen += 1
+    assert seen >= 55
