@@ -159,3 +159,63 @@ def test_kernel_cache_and_errors(g):
         g.ops.ElementWiseNvrtc([x, torch.randn(7, device="cuda")], 1,
                                g.ops.fusion_program([("x", F32), ("z", F32)], [("y", "Add", "x", "z")], [("y", F32)]),
                                outs=[torch.empty(1000, device="cuda")])
+
+
+def test_random_programs(g, oracle):
+    """Seeded random element-wise programs (every op of the generator, constants, operands that
+    broadcast on inner and outer axes, one to three results) against the op-by-op CPU evaluation;
+    bit-exact.  Exp only sees bounded values and divisors are positive, so no NaN arises whose
+    ordering in Max / Min would be a matter of definition."""
+    rng = np.random.default_rng(77)
+    exact = {"Neg": np.negative, "Abs": np.abs, "Floor": np.floor, "Round": np.rint, "Max": np.maximum, "Min": np.minimum}
+    shapes = [((4, 5, 33), (5, 1)), ((2, 3, 4, 129), (1, 129)), ((7, 64), (7, 1)), ((1000,), ()), ((3, 1, 17), (1, 6, 1)), ((2, 2, 2, 2, 5), (2, 1, 5))]
+    for trial in range(24):
+        shape, kshape = shapes[trial % len(shapes)]
+        inputs = dict(x=(rng.standard_normal(shape) * 2).astype(np.float32), k=rng.standard_normal(kshape).astype(np.float32),
+                      c=rng.standard_normal(shape).astype(np.float32))
+        full_shape = np.broadcast_shapes(shape, kshape)
+        stmts, pool, bounded = [], ["x", "k", "c"], set()
+        shape_of = {n: v.shape for n, v in inputs.items()}
+
+        def emit(op, *args):
+            name = "v%d" % len(stmts)
+            stmts.append((name, op) + args)
+            pool.append(name)
+            shape_of[name] = np.broadcast_shapes(*[shape_of[a] for a in args if isinstance(a, str)]) if op != "Const" else ()
+            return name
+        for _ in range(int(rng.integers(3, 14))):
+            op = str(rng.choice(["Add", "Sub", "Mul", "Div", "Max", "Min", "Neg", "Abs", "Floor", "Round", "Relu", "Identity", "Tanh",
+                                 "Sigmoid", "Exp", "Clip", "Const"]))
+            a, b = (str(v) for v in rng.choice(pool, 2))
+            if op == "Const":
+                emit("Const", float(np.float32(rng.standard_normal())))
+            elif op == "Clip":
+                lo = float(np.float32(rng.uniform(-2, 0)))
+                bounded.add(emit("Clip", a, lo, float(np.float32(lo + rng.uniform(0.1, 3)))))
+            elif op in ("Tanh", "Sigmoid"):
+                bounded.add(emit(op, a))
+            elif op == "Exp":
+                bounded.add(emit("Exp", a if a in bounded else emit("Tanh", a)))
+            elif op == "Div":
+                emit("Div", a, emit("Exp", emit("Tanh", b)))
+            elif op in ("Add", "Sub", "Mul", "Max", "Min"):
+                emit(op, a, b)
+            else:
+                emit(op, a)
+        # results have the shape all operands broadcast to (runtime/ops/nvrtc.cc:100-113)
+        candidates = [n for n in pool[3:] if tuple(shape_of[n]) == tuple(full_shape)]
+        if not candidates:
+            candidates = [emit("Add", emit("Add", pool[-1], "x"), "k")]
+        outs = [str(n) for n in rng.choice(candidates, size=min(len(candidates), int(rng.integers(1, 4))), replace=False)]
+        env = dict(inputs)
+        for stmt in stmts:
+            if stmt[1] in exact:
+                env[stmt[0]] = exact[stmt[1]](*[env[a] for a in stmt[2:]]).astype(np.float32)
+            else:
+                env = oracle.run_chain([stmt], env)
+        prog = g.ops.fusion_program([("x", F32), ("k", F32), ("c", F32)], stmts, [(o, F32) for o in outs])
+        got = g.ops.ElementWiseNvrtc([g.dev(inputs[n]) for n in ("x", "k", "c")], len(outs), prog, 1000 + trial)
+        for o, t in zip(outs, got):
+            want = np.broadcast_to(env[o], full_shape)
+            assert not np.isnan(want).any()
+            np.testing.assert_array_equal(g.host(t), want, err_msg="trial %d, %s of %s" % (trial, o, stmts))
