@@ -537,3 +537,28 @@ def test_random_convolution_sweep(g, oracle):
         np.testing.assert_array_equal(g.host(got_i), want_i, err_msg=tag)
         seen += 1
     assert seen >= 55
+
+
+def test_random_matmul_sweep(g, oracle):
+    """Seeded random MatMulInteger / QLinearMatMul shapes (2-D, batched N-D, K and N that leave
+    partial tiles, every element-type pairing, zero points, strided operands); bit-exact."""
+    rng = np.random.default_rng(4242)
+    for trial in range(40):
+        M, K, N = (int(rng.choice([1, 2, 7, 16, 33, 64, 100, 129, int(rng.integers(1, 300))])) for _ in range(3))
+        batch = [(), (), (3,), (2, 2)][int(rng.integers(0, 4))]
+        adt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        bdt = [np.int8, np.uint8][int(rng.integers(0, 2))]
+        a, b = rand_q(rng, batch + (M, K), adt), rand_q(rng, batch + (K, N), bdt)
+        az = rand_q(rng, (1,), adt) if rng.integers(0, 2) else None
+        bz = rand_q(rng, (N,) if rng.integers(0, 2) else (1,), bdt) if rng.integers(0, 2) else None
+        tag = "trial %d: a%s %s b%s %s" % (trial, a.shape, adt.__name__, b.shape, bdt.__name__)
+        bd = g.dev(b) if rng.integers(0, 2) else g.dev(np.ascontiguousarray(np.swapaxes(b, -1, -2))).transpose(-1, -2)
+        got = g.ops.MatMulInteger(g.dev(a), bd, None if az is None else g.dev(az), None if bz is None else g.dev(bz))
+        np.testing.assert_array_equal(g.host(got), oracle.matmul_integer(a, b, az, bz), err_msg=tag)
+        ydt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        a_zp, b_zp, y_zp = int(rand_q(rng, (1,), adt)[0]), int(rand_q(rng, (1,), bdt)[0]), int(rand_q(rng, (1,), ydt)[0])
+        b_scale = np.float32(rng.uniform(0.002, 0.02))
+        y_scale = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(K) / float(rng.choice([20, 60, 200])))
+        want = oracle.qlinear_matmul_int(a, 0.02, a_zp, b, b_scale, b_zp, y_scale, y_zp, ydt)
+        got = g.ops.QLinearMatMul(g.dev(a), 0.02, a_zp, bd, b_scale, b_zp, y_scale, y_zp, zero_point_dtype=TDT[ydt])
+        np.testing.assert_array_equal(g.host(got), want, err_msg=tag + " QLinearMatMul -> " + ydt.__name__)
