@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kThreads) void max_pool_generic_kernel(PoolArgs a) 
     r /= a.OW;
     const int oh = (int)(r % a.OH);
     const int n = (int)(r / a.OH);
-    int32_t m = -1000;
+    int32_t m = a.is_signed ? -128 : 0;  // a window in the padding altogether: the lowest code, as Q(lowest float) is
     for (int i = 0; i < a.kh; ++i) {
         const int ih = oh * a.sh - a.ph + i;
         if ((unsigned)ih >= (unsigned)a.H) continue;

@@ -526,8 +526,9 @@ void orc_round_f32(const float* x, int64_t n, float* y) {
  * and zero point on both sides equals the maximum of the codes, because the
  * dequantization map is increasing and Q(DQ(q)) == q for uint8 (checked exhaustively
  * in the tests).  Out-of-image taps never win (ChainerX pads max-pooling with the
- * lowest value); cover_all makes the last window start inside the image even when
- * it overhangs: out = ceil((in + p0 + p1 - k) / s) + 1 instead of floor.
+ * lowest value); cover_all adds a last window for what floor would leave uncovered
+ * (out = ceil((in + p0 + p1 - k) / s) + 1 instead of floor), which with pads can lie in the
+ * padding altogether.
  *
  * orc_average_pool_q8: y = Q( (sum over the window of DQ(x)) / count ), the sum taken
  * in fp32 in (kh, kw) order starting from 0.  PARITY UNPINNED for that order and for
@@ -550,7 +551,9 @@ void orc_max_pool_q8(
     for (int64_t nc = 0; nc < N * C; ++nc) {
         for (int64_t oh = 0; oh < OH; ++oh)
             for (int64_t ow = 0; ow < OW; ++ow) {
-                int32_t m = -1000;
+                /* a window that lies in the padding altogether (possible with cover_all and pads) has the
+                 * lowest float as its maximum, which QuantizeLinear clamps to the lowest code */
+                int32_t m = x_is_int8 ? -128 : 0;
                 for (int64_t i = 0; i < kh; ++i)
                     for (int64_t j = 0; j < kw; ++j) {
                         const int64_t ih = oh * sh - ph0 + i, iw = ow * sw - pw0 + j;

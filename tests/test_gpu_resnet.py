@@ -210,3 +210,40 @@ def test_benchmark_configuration_at_full_size(g, oracle, net, batch, seed):
         assert torch.equal(again[name], out[name][perm]), name
     assert out["logits_q"].min() < out["logits_q"].max()
     runner.close()
+
+
+def test_random_pool_sweep(g, oracle):
+    """Seeded random MaxPool / AveragePool windows on quantized tensors: kernel, stride, pads,
+    cover_all / count_include_pad, channel counts on and off the vector widths of the channels-last
+    kernels, both layouts, both element types; bit-exact."""
+    rng = np.random.default_rng(909)
+    done = 0
+    for trial in range(60):
+        N, C = int(rng.integers(1, 4)), int(rng.choice([1, 3, 4, 8, 12, 16, 20, 32, 48, 64, int(rng.integers(1, 90))]))
+        H, W = int(rng.integers(1, 20)), int(rng.integers(1, 20))
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        if trial % 6 == 0:
+            kh, kw = H, W                                   # the window is the whole image
+        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        ph, pw = int(rng.integers(0, kh // 2 + 1)), int(rng.integers(0, kw // 2 + 1))
+        if H + 2 * ph < kh or W + 2 * pw < kw:
+            continue
+        xdt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        lo, hi = (0, 256) if xdt == np.uint8 else (-128, 128)
+        x = rng.integers(lo, hi, size=(N, C, H, W)).astype(xdt)
+        xd = g.dev(x) if rng.integers(0, 3) == 0 else g.to_channels_last(g.dev(x))
+        tag = "trial %d: x%s %s kernel %s strides %s pads %s" % (trial, x.shape, xdt.__name__, (kh, kw), (sh, sw), (ph, pw))
+        cover_all = bool(rng.integers(0, 2))
+        np.testing.assert_array_equal(g.host(g.ops.MaxPoolQ8(xd, (kh, kw), (sh, sw), (ph, pw), cover_all)),
+                                      oracle.max_pool_q8(x, (kh, kw), (sh, sw), (ph, pw), cover_all), err_msg=tag + " max, cover_all %s" % cover_all)
+        cip = bool(rng.integers(0, 2))
+        xz = int(rng.integers(lo, hi))
+        ydt = [np.uint8, np.int8][int(rng.integers(0, 2))]
+        yz = int(rng.integers(0, 256) if ydt == np.uint8 else rng.integers(-128, 128))
+        ys = np.float32(rng.uniform(0.02, 0.08))
+        want = oracle.average_pool_q8(x, 0.05, xz, (kh, kw), (sh, sw), (ph, pw), ys, yz, ydt, count_include_pad=cip)
+        got = g.ops.AveragePoolQ8(xd, 0.05, xz, (kh, kw), (sh, sw), (ph, pw), ys, yz, count_include_pad=cip,
+                                  zero_point_dtype=torch.uint8 if ydt == np.uint8 else torch.int8)
+        np.testing.assert_array_equal(g.host(got), want, err_msg=tag + " average, count_include_pad %s -> %s" % (cip, ydt.__name__))
+        done += 1
+    assert done >= 50

@@ -241,3 +241,28 @@ def test_chain_matches_stepwise_numpy(oracle):
     np.testing.assert_array_equal(env["t1"], t1)
     want = np.maximum(oracle.tanh(t1) * oracle.sigmoid(c) + x, 0)
     np.testing.assert_array_equal(env["y"], want)
+
+
+def test_max_pool_window_in_the_padding_gives_the_lowest_code(oracle):
+    """cover_all with pads can add a window that lies in the padding altogether.  Spelled out in
+    float (ChainerX pads max-pooling with the lowest value): DequantizeLinear, maximum over a window
+    padded with -inf, QuantizeLinear -> the clamp's lower end, i.e. the lowest code of the type."""
+    rng = np.random.default_rng(17)
+    for dt, lowest in ((np.uint8, 0), (np.int8, -128)):
+        x = rng.integers(30, 100, size=(1, 2, 11, 16)).astype(dt)
+        got = oracle.max_pool_q8(x, (2, 3), (2, 2), (1, 1), True)
+        assert got.shape == (1, 2, 7, 9)                      # rows start at -1, 1, ..., 11: the last one is past the image
+        dq = oracle.dequantize_linear(x, np.float32(0.05), 30 if dt == np.uint8 else -30)
+        padded = np.full((1, 2, 11 + 1 + 3, 16 + 1 + 3), -np.inf, np.float32)
+        padded[:, :, 1:12, 1:17] = dq
+        want = np.empty((1, 2, 7, 9), np.float32)
+        for oh in range(7):
+            for ow in range(9):
+                want[:, :, oh, ow] = padded[:, :, 2 * oh:2 * oh + 2, 2 * ow:2 * ow + 3].max(axis=(2, 3))
+        assert np.isinf(want[:, :, 6, :]).all() and np.isfinite(want[:, :, :6, :]).all()
+        assert (got[:, :, 6, :] == lowest).all()
+        if dt == np.uint8:
+            # the three float ops give the same bytes; for int8 they do not (the reference's QuantizeLinear turns a negative
+            # code q into q + 1), which is why only uint8 pools are computed on codes inside a program
+            with np.errstate(all="ignore"):
+                np.testing.assert_array_equal(got, oracle.quantize_linear(want, np.float32(0.05), 30, dt))
