@@ -380,3 +380,28 @@ def test_trace_lines(g, vm, capfd):
     prog.run({"x": g.dev(np.ones((3, 5), np.float32))})          # silent by default
     assert capfd.readouterr().err == ""
     prog.close()
+
+
+def test_max_pool_on_codes_is_for_uint8_only(g, vm, oracle):
+    """DequantizeLinear -> MaxPool -> QuantizeLinear with one scale and zero point runs as the maximum
+    of the codes for uint8 (Q(DQ(q)) == q); with int8 codes the reference's truncating QuantizeLinear
+    gives q + 1 for a negative q, so the VM refuses instead of returning other bytes."""
+    def pool_program(zp, zdt):
+        b = vm.ProgramBuilder()
+        x = b.input("x", zdt, (1, 16, 6, 6))
+        s, z = b.scalar(0.05, "float32"), b.scalar(zp, zdt)
+        d = b.DequantizeLinear(x, s, z)
+        p = b.new_slot()
+        b.add_raw("MaxPool", [("ARRAY", d), ("INTS", [2, 2]), ("INTS", [2, 2]), ("INTS", [0, 0]), ("INT", 0), ("STRING", "NOTSET")], [p, -1])
+        q = b.QuantizeLinear(p, s, z)
+        b.output("q", q)
+        return b.serialize()
+    rng = np.random.default_rng(8)
+    xu = rng.integers(0, 256, size=(1, 16, 6, 6)).astype(np.uint8)
+    prog = vm.Program(pool_program(30, "uint8"))
+    np.testing.assert_array_equal(prog.run({"x": g.dev(xu)})["q"], oracle.max_pool_q8(xu, (2, 2), (2, 2)))
+    prog.close()
+    xi = rng.integers(-128, 128, size=(1, 16, 6, 6)).astype(np.int8)
+    with pytest.raises(vm.ChxVMError, match="int8"):
+        prog = vm.Program(pool_program(-3, "int8"))
+        prog.run({"x": g.dev(xi)})
