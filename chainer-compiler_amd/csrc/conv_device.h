@@ -1,0 +1,88 @@
+// Device-side pieces shared by the matrix-core convolution kernels (conv_mfma.hip, conv_bs.hip).
+// Everything here has internal linkage: each translation unit gets its own copy.
+#pragma once
+
+#include "conv_mfma.h"
+
+namespace chx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Row b (64 bytes) holds the byte b in every position.  A filter tap outside the image fetches
+// the row of the activation zero point, so padding needs no data-dependent fix-up.
+#define CHX_B16(v) v, v, v, v, v, v, v, v, v, v, v, v, v, v, v, v
+#define CHX_ROW(v) CHX_B16(v), CHX_B16(v), CHX_B16(v), CHX_B16(v)
+#define CHX_ROWS16(h)                                                                                     \
+    CHX_ROW((h) * 16 + 0), CHX_ROW((h) * 16 + 1), CHX_ROW((h) * 16 + 2), CHX_ROW((h) * 16 + 3),           \
+    CHX_ROW((h) * 16 + 4), CHX_ROW((h) * 16 + 5), CHX_ROW((h) * 16 + 6), CHX_ROW((h) * 16 + 7),           \
+    CHX_ROW((h) * 16 + 8), CHX_ROW((h) * 16 + 9), CHX_ROW((h) * 16 + 10), CHX_ROW((h) * 16 + 11),         \
+    CHX_ROW((h) * 16 + 12), CHX_ROW((h) * 16 + 13), CHX_ROW((h) * 16 + 14), CHX_ROW((h) * 16 + 15)
+__device__ __attribute__((aligned(64))) const unsigned char g_fill_rows[256 * 64] = {
+        CHX_ROWS16(0), CHX_ROWS16(1), CHX_ROWS16(2),  CHX_ROWS16(3),  CHX_ROWS16(4),  CHX_ROWS16(5),  CHX_ROWS16(6),  CHX_ROWS16(7),
+        CHX_ROWS16(8), CHX_ROWS16(9), CHX_ROWS16(10), CHX_ROWS16(11), CHX_ROWS16(12), CHX_ROWS16(13), CHX_ROWS16(14), CHX_ROWS16(15)};
+#undef CHX_ROWS16
+#undef CHX_ROW
+#undef CHX_B16
+
+// n / d for n < 2^31 with the multiplier and shift of magic_divisor() (conv_mfma.h).
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t mul, uint32_t shift) {
+    return (__umulhi(n, mul) + n) >> shift;
+}
+
+// Asynchronous copy of 16 bytes per lane from global memory straight into LDS: lane i of the
+// wavefront writes LDS bytes [lds_addr + 16*i, lds_addr + 16*i + 16).  lds_addr must be the
+// same for all lanes (it travels in M0).  Completion is tracked by the wave's vector-memory
+// counter like any load; nothing passes through registers.
+__device__ __forceinline__ void async_copy16(const void* src, uint32_t lds_addr) {
+    asm volatile(
+            "s_mov_b32 m0, %1\n\t"
+            "s_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, off"
+            :
+            : "v"(src), "s"(lds_addr)
+            : "memory", "m0");
+}
+
+// Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
+// (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
+// reference's order, one IEEE operation each.
+// kLean (uint8 result, zero points of r and of the result both 0, as between the Relu outputs of a
+// residual network): the two "- 0.0f" / "+ 0.0f" change no value and are left out, and so is the
+// Relu, because QuantizeLinear is monotone, Q(max(s, 0)) = max(Q(s), Q(0)) = max(Q(s), 0), and the
+// saturating conversion already stops at 0.
+template <bool kU8, bool kGuard, bool kLean = false>
+__device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
+    static_assert(kU8 || !kLean, "the lean variant is for uint8 results");
+    v4i out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
+        int32_t code[4];
+        float pre[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
+            const float rb = (float)((rw >> (8 * e)) & 0xffu);
+            const float fb = kLean ? rb * p.r_scale : (rb - p.r_zpf) * p.r_scale;
+            float sum = fa + fb;
+            if (!kLean && p.relu) sum = __builtin_fmaxf(sum, 0.f);
+            if (kGuard) sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
+            if (kU8) pre[e] = quantize_prefloor_u8<false, !kLean>(sum, p.out, p.inv_out_scale, 0.f);
+            else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
+        }
+        out[w] = kU8 ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
+    }
+    return out;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+
+}  // namespace
+}  // namespace chx

@@ -9,34 +9,32 @@
 //     (kh, kw) the 64 channels of a K slice are 64 contiguous bytes of x, or the
 //     padding value when the tap falls outside the image;
 //   - uint8 activations are turned into int8 by flipping the top bit (x - 128) on the
-//     way into LDS; the exact result is restored per output channel in the epilogue:
+//     fragments read back from LDS; the exact result is restored by the accumulator seed:
 //         sum (x - zp) w = sum (x - 128) w + (128 - zp) * sum_k w[oc, k]
 //     Out-of-image taps are filled with the zero point itself, which makes them
 //     contribute (zp - zp) * w = 0, the reference's zero padding of the already
 //     zero-point-subtracted tensor (runtime/chainerx_util.cc:232-274, 313-340).
 //
 // Work-group: four wavefronts in a 2x2 grid over a tile of (64*FM) output channels x
-// (64*FN) pixels, 64 K-bytes per step; each wavefront owns FM x FN MFMA tiles of 32x32.
-// Global memory latency is covered by keeping three K steps in flight in registers
-// ahead of the double-buffered LDS stage that is being consumed.  The 16-byte chunks of
-// an LDS row are XOR-swizzled with bits 2..3 of the row index so that the 128-bit LDS
-// reads of a wavefront's 16-lane groups fall on distinct banks.
+// (64*FN) pixels; each wavefront owns FM x FN MFMA tiles of 32x32.  Both operands reach LDS by
+// asynchronous global->LDS copies (nothing passes through registers) into a ring of two or
+// three stages of 64 or 128 K-bytes; the copies run ahead of the MFMAs across tile boundaries.
+// The 16-byte chunks of a staged row are XOR-swizzled with row bits so that the 128-bit
+// fragment reads of a wavefront fall on distinct banks (lds_chunk_offset).
 //
 // Epilogue: the requantization of quant_math.h per element, codes packed four output
-// channels at a time, transposed through LDS into [pixel][oc] rows and written as
-// 128-bit stores to the channels-last output.  With an int32 output (ConvInteger,
-// MatMulInteger) the accumulators are stored directly.
+// channels at a time, transposed through the ring slot just consumed into [pixel][oc] rows
+// and written as 128-bit stores to the channels-last output; optionally the residual sum of
+// the element-wise group behind the convolution (ResidualAdd).  With an int32 output
+// (ConvInteger, MatMulInteger) the accumulators are stored directly.
 #include <type_traits>
 
 #include "contract.h"
 #include "conv_mfma.h"
+#include "conv_device.h"
 
 namespace chx {
 namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Packed weights are stored in blocks that one K step of the kernel reads as whole cache
 // lines: Wp[oc / 64][k / BK][oc % 64][k % BK] with BK = 64 or 128 K-bytes per step, i.e. the 64
@@ -226,41 +224,6 @@ __device__ __forceinline__ int lds_chunk_offset(int row, int kc) {
     return BK == 64 ? row * 64 + ((kc ^ ((row >> 2) & 3)) << 4) : row * 128 + ((kc ^ ((row >> 1) & 7)) << 4);
 }
 
-// Row b (64 bytes) holds the byte b in every position.  A filter tap outside the image fetches
-// the row of the activation zero point, so padding needs no data-dependent fix-up.
-#define CHX_B16(v) v, v, v, v, v, v, v, v, v, v, v, v, v, v, v, v
-#define CHX_ROW(v) CHX_B16(v), CHX_B16(v), CHX_B16(v), CHX_B16(v)
-#define CHX_ROWS16(h)                                                                                     \
-    CHX_ROW((h) * 16 + 0), CHX_ROW((h) * 16 + 1), CHX_ROW((h) * 16 + 2), CHX_ROW((h) * 16 + 3),           \
-    CHX_ROW((h) * 16 + 4), CHX_ROW((h) * 16 + 5), CHX_ROW((h) * 16 + 6), CHX_ROW((h) * 16 + 7),           \
-    CHX_ROW((h) * 16 + 8), CHX_ROW((h) * 16 + 9), CHX_ROW((h) * 16 + 10), CHX_ROW((h) * 16 + 11),         \
-    CHX_ROW((h) * 16 + 12), CHX_ROW((h) * 16 + 13), CHX_ROW((h) * 16 + 14), CHX_ROW((h) * 16 + 15)
-__device__ __attribute__((aligned(64))) const unsigned char g_fill_rows[256 * 64] = {
-        CHX_ROWS16(0), CHX_ROWS16(1), CHX_ROWS16(2),  CHX_ROWS16(3),  CHX_ROWS16(4),  CHX_ROWS16(5),  CHX_ROWS16(6),  CHX_ROWS16(7),
-        CHX_ROWS16(8), CHX_ROWS16(9), CHX_ROWS16(10), CHX_ROWS16(11), CHX_ROWS16(12), CHX_ROWS16(13), CHX_ROWS16(14), CHX_ROWS16(15)};
-#undef CHX_ROWS16
-#undef CHX_ROW
-#undef CHX_B16
-
-// n / d for n < 2^31 with the multiplier and shift of magic_divisor() (conv_mfma.h).
-__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t mul, uint32_t shift) {
-    return (__umulhi(n, mul) + n) >> shift;
-}
-
-// Asynchronous copy of 16 bytes per lane from global memory straight into LDS: lane i of the
-// wavefront writes LDS bytes [lds_addr + 16*i, lds_addr + 16*i + 16).  lds_addr must be the
-// same for all lanes (it travels in M0).  Completion is tracked by the wave's vector-memory
-// counter like any load; nothing passes through registers.
-__device__ __forceinline__ void async_copy16(const void* src, uint32_t lds_addr) {
-    asm volatile(
-            "s_mov_b32 m0, %1\n\t"
-            "s_nop 0\n\t"
-            "global_load_lds_dwordx4 %0, off"
-            :
-            : "v"(src), "s"(lds_addr)
-            : "memory", "m0");
-}
-
 // 128-bit LDS read whose completion the caller waits for itself (wait_fragments): the compiler
 // would otherwise wait for every outstanding LDS operation at the first use, because it cannot
 // see through the inline assembly of the copies issued in between.
@@ -306,43 +269,6 @@ __device__ __forceinline__ void warm_kernel_arguments() {
             : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5)
             : "s"(ka), "n"(L4), "n"(L5)
             : "memory");
-}
-
-// Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
-// (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
-// reference's order, one IEEE operation each.
-// kLean (uint8 result, zero points of r and of the result both 0, as between the Relu outputs of a
-// residual network): the two "- 0.0f" / "+ 0.0f" change no value and are left out, and so is the
-// Relu, because QuantizeLinear is monotone, Q(max(s, 0)) = max(Q(s), Q(0)) = max(Q(s), 0), and the
-// saturating conversion already stops at 0.
-template <bool kU8, bool kGuard, bool kLean = false>
-__device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
-    static_assert(kU8 || !kLean, "the lean variant is for uint8 results");
-    v4i out;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
-        int32_t code[4];
-        float pre[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
-            const float rb = (float)((rw >> (8 * e)) & 0xffu);
-            const float fb = kLean ? rb * p.r_scale : (rb - p.r_zpf) * p.r_scale;
-            float sum = fa + fb;
-            if (!kLean && p.relu) sum = __builtin_fmaxf(sum, 0.f);
-            if (kGuard) sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
-            if (kU8) pre[e] = quantize_prefloor_u8<false, !kLean>(sum, p.out, p.inv_out_scale, 0.f);
-            else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
-        }
-        out[w] = kU8 ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
-    }
-    return out;
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
 // LDS ring stages of a work-group: what fits the budget, between 2 and the cap.  The bytes in

@@ -32,6 +32,21 @@
  *                            ChainerX's Sigmoid routine is not in the tree.
  *   orc_tanh_f32/orc_exp_f32 call the host libm, as std::tanh/std::exp do in
  *                            ChainerX's native kernels.
+ *   orc_max_pool_q8          pinned: numpy restatement over an explicitly padded
+ *                            array (both types, cover_all, pads, whole-image
+ *                            window), and the three float ops spelled out
+ *                            (DequantizeLinear, maximum over a -inf padded
+ *                            tensor, QuantizeLinear) for uint8.
+ *   orc_average_pool_q8      pinned: numpy restatement (tap-major loop over a
+ *                            zero-padded float tensor, both pad-count modes,
+ *                            both roundings, all four type pairs), the exact
+ *                            family (power-of-two scales: integer arithmetic
+ *                            fixes the mean), constant images, and the
+ *                            whole-image window against a sequential float32
+ *                            running sum.  What stays PARITY UNPINNED is only
+ *                            that ChainerX's kernel sums in (kh, kw) order and
+ *                            divides by the count (its source is not in the
+ *                            tree); the tests show the order matters.
  */
 #include <math.h>
 #include <stdint.h>
@@ -531,9 +546,9 @@ void orc_round_f32(const float* x, int64_t n, float* y) {
  * padding altogether.
  *
  * orc_average_pool_q8: y = Q( (sum over the window of DQ(x)) / count ), the sum taken
- * in fp32 in (kh, kw) order starting from 0.  PARITY UNPINNED for that order and for
- * "divide by count" (ChainerX's AveragePool kernel is not in the tree); padding taps
- * add 0 and count toward `count` when count_include_pad. */
+ * in fp32 in (kh, kw) order starting from 0; padding taps add 0 and count toward
+ * `count` when count_include_pad.  (That ChainerX's AveragePool kernel, which is not
+ * in the tree, uses this order and divides by the count is recalled, not verified.) */
 static int64_t pool_out_dim(int64_t in, int64_t p0, int64_t p1, int64_t k, int64_t s, int cover_all) {
     if (cover_all) return (in + p0 + p1 - k + s - 1) / s + 1;
     return (in + p0 + p1 - k) / s + 1;

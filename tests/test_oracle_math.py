@@ -266,3 +266,172 @@ def test_max_pool_window_in_the_padding_gives_the_lowest_code(oracle):
             # code q into q + 1), which is why only uint8 pools are computed on codes inside a program
             with np.errstate(all="ignore"):
                 np.testing.assert_array_equal(got, oracle.quantize_linear(want, np.float32(0.05), 30, dt))
+
+
+# --- pools between a DequantizeLinear and a QuantizeLinear (runtime/ops/pooling.cc:47-75) -------------
+# Independent restatements: the oracle walks output pixels and gathers taps; these build an explicitly
+# padded array and walk the taps, whole output planes at a time.
+
+def np_dequantize(q, scale, zp):
+    return (q.astype(np.float32) - np.float32(zp)) * np.float32(scale)
+
+
+def np_average_pool_q8(x, x_scale, x_zp, kernel, strides, pads, y_scale, y_zp, y_dtype, count_include_pad, rne=False):
+    N, C, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = kernel, strides, pads
+    OH, OW = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    val = np.zeros((N, C, H + 2 * ph, W + 2 * pw), np.float32)       # zero padding of the float tensor
+    val[:, :, ph:ph + H, pw:pw + W] = np_dequantize(x, x_scale, x_zp)
+    inside = np.zeros((H + 2 * ph, W + 2 * pw), np.int64)
+    inside[ph:ph + H, pw:pw + W] = 1
+    total = np.zeros((N, C, OH, OW), np.float32)
+    count = np.zeros((OH, OW), np.int64)
+    for i in range(kh):                                               # taps in (kh, kw) order, one fp32 addition each
+        for j in range(kw):
+            total = total + val[:, :, i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw]
+            count += inside[i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw]
+    if count_include_pad:
+        count[:] = kh * kw
+    mean = total / count.astype(np.float32)
+    lo, hi = (0, 255) if y_dtype == np.uint8 else (-128, 127)
+    if rne:
+        s = mean / np.float32(y_scale)
+        return np.clip(np.rint(s) + y_zp, lo, hi).astype(y_dtype)
+    return np_quantize(mean, y_scale, y_zp, lo, hi).astype(y_dtype)
+
+
+POOL_CASES = [  # kernel, strides, pads, H, W
+    ((3, 3), (1, 1), (1, 1), 9, 11), ((2, 2), (2, 2), (0, 0), 8, 10), ((3, 2), (2, 1), (1, 0), 7, 9),
+    ((5, 5), (3, 2), (2, 2), 13, 12), ((7, 7), (1, 1), (0, 0), 7, 7), ((1, 1), (1, 1), (0, 0), 4, 5),
+    ((3, 3), (2, 2), (1, 1), 14, 14), ((2, 3), (1, 2), (1, 1), 5, 6)]
+
+
+@pytest.mark.parametrize("x_dt,y_dt", [(np.uint8, np.uint8), (np.int8, np.int8), (np.uint8, np.int8), (np.int8, np.uint8)])
+@pytest.mark.parametrize("include_pad", [False, True])
+def test_average_pool_vs_numpy(oracle, x_dt, y_dt, include_pad):
+    rng = np.random.default_rng(31)
+    for kernel, strides, pads, H, W in POOL_CASES:
+        lo, hi = (0, 256) if x_dt == np.uint8 else (-128, 128)
+        x = rng.integers(lo, hi, size=(2, 3, H, W)).astype(x_dt)
+        x_zp = int(rng.integers(lo, hi))
+        y_zp = int(rng.integers(0, 256)) if y_dt == np.uint8 else int(rng.integers(-128, 128))
+        x_scale, y_scale = np.float32(rng.uniform(0.01, 0.1)), np.float32(rng.uniform(0.01, 0.1))
+        for rne in (False, True):
+            got = oracle.average_pool_q8(x, x_scale, x_zp, kernel, strides, pads, y_scale, y_zp, y_dt, include_pad,
+                                         oracle.ROUND_ONNX_RNE if rne else oracle.ROUND_REFERENCE)
+            want = np_average_pool_q8(x, x_scale, x_zp, kernel, strides, pads, y_scale, y_zp, y_dt, include_pad, rne)
+            np.testing.assert_array_equal(got, want, err_msg=str((kernel, strides, pads, rne)))
+
+
+def test_average_pool_exact_family(oracle):
+    """Power-of-two scales and small windows: every partial sum of the window is a small integer times
+    the scale, exact in fp32 in any order, so the mean is fixed by integer arithmetic alone."""
+    rng = np.random.default_rng(32)
+    for kernel, strides, pads, H, W in POOL_CASES:
+        for x_dt in (np.uint8, np.int8):
+            lo, hi = (0, 256) if x_dt == np.uint8 else (-128, 128)
+            x = rng.integers(lo, hi, size=(1, 2, H, W)).astype(x_dt)
+            x_zp = int(rng.integers(lo, hi))
+            for include_pad in (False, True):
+                got = oracle.average_pool_q8(x, 0.125, x_zp, kernel, strides, pads, 0.25, 3, np.uint8, include_pad)
+                OH, OW = got.shape[2:]
+                want = np.empty_like(got)
+                for c in range(2):
+                    for oh in range(OH):
+                        for ow in range(OW):
+                            r0, c0 = oh * strides[0] - pads[0], ow * strides[1] - pads[1]
+                            rows = range(max(r0, 0), min(r0 + kernel[0], H))
+                            cols = range(max(c0, 0), min(c0 + kernel[1], W))
+                            isum = sum(int(x[0, c, r, q]) - x_zp for r in rows for q in cols)   # exact integer
+                            n = kernel[0] * kernel[1] if include_pad else len(rows) * len(cols)
+                            mean = np.float32(isum * 0.125) / np.float32(n)                      # one rounding: the division
+                            want[0, c, oh, ow] = np_quantize(np.array([mean], np.float32), 0.25, 3, 0, 255)[0]
+                np.testing.assert_array_equal(got, want)
+
+
+def test_average_pool_of_a_constant_image_is_the_constant(oracle):
+    """x == c everywhere, window inside the image, one power-of-two scale on both sides: the sum of n equal
+    values v is n*v exactly, the mean is v, and Q(DQ(c)) == c."""
+    for c in (0, 1, 77, 128, 254, 255):
+        x = np.full((1, 2, 8, 8), c, np.uint8)
+        for kernel in ((2, 2), (3, 3), (8, 8), (5, 7)):
+            got = oracle.average_pool_q8(x, 0.0625, 128, kernel, (1, 1), (0, 0), 0.0625, 128, np.uint8)
+            assert (got == c).all()
+    # with zero padding counted in, a corner window of a 3x3/pad 1 pool sees 4 of 9 taps
+    x = np.full((1, 1, 6, 6), 200, np.uint8)
+    got = oracle.average_pool_q8(x, 0.5, 128, (3, 3), (1, 1), (1, 1), 0.5, 128, np.uint8, True)
+    corner = np_quantize(np.array([np.float32(4 * 36.0) / np.float32(9)], np.float32), 0.5, 128, 0, 255)[0]
+    assert got[0, 0, 0, 0] == corner and got[0, 0, 2, 2] == 200
+    got = oracle.average_pool_q8(x, 0.5, 128, (3, 3), (1, 1), (1, 1), 0.5, 128, np.uint8, False)
+    assert (got == 200).all()
+
+
+def test_global_average_pool_is_a_sequential_row_major_sum(oracle):
+    """kernel = whole image: the (kh, kw) order is the image's row-major order, so the sum is the last
+    entry of a float32 running sum (np.cumsum accumulates sequentially in the array's type)."""
+    rng = np.random.default_rng(33)
+    for H, W in ((7, 7), (4, 9), (14, 14)):
+        x = rng.integers(0, 256, size=(3, 5, H, W)).astype(np.uint8)
+        x_scale, y_scale = np.float32(0.0371), np.float32(0.0193)
+        got = oracle.average_pool_q8(x, x_scale, 11, (H, W), (1, 1), (0, 0), y_scale, 4, np.uint8)
+        run = np.cumsum(np_dequantize(x, x_scale, 11).reshape(3, 5, H * W), axis=2, dtype=np.float32)[:, :, -1]
+        mean = run / np.float32(H * W)
+        np.testing.assert_array_equal(got.reshape(3, 5), np_quantize(mean, y_scale, 4, 0, 255).astype(np.uint8))
+        # the order matters for this input (otherwise the test above would pin nothing about it)
+    x = rng.integers(0, 256, size=(64, 64, 7, 7)).astype(np.uint8)
+    fwd = np.cumsum(np_dequantize(x, 0.0371, 11).reshape(64, 64, 49), axis=2, dtype=np.float32)[:, :, -1]
+    rev = np.cumsum(np_dequantize(x, 0.0371, 11).reshape(64, 64, 49)[:, :, ::-1], axis=2, dtype=np.float32)[:, :, -1]
+    assert (fwd != rev).any()
+
+
+def np_max_pool_q8(x, kernel, strides, pads, cover_all):
+    N, C, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = kernel, strides, pads
+    if cover_all:
+        OH, OW = -((H + 2 * ph - kh) // -sh) + 1, -((W + 2 * pw - kw) // -sw) + 1
+    else:
+        OH, OW = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    lowest = np.iinfo(x.dtype).min
+    # room for the windows that cover_all adds past the symmetric padding
+    PH, PW = (OH - 1) * sh + kh, (OW - 1) * sw + kw
+    pad = np.full((N, C, max(PH, H + 2 * ph), max(PW, W + 2 * pw)), lowest, np.int64)
+    pad[:, :, ph:ph + H, pw:pw + W] = x
+    out = np.full((N, C, OH, OW), lowest, np.int64)
+    for i in range(kh):
+        for j in range(kw):
+            out = np.maximum(out, pad[:, :, i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw])
+    return out.astype(x.dtype)
+
+
+@pytest.mark.parametrize("dt", [np.uint8, np.int8])
+@pytest.mark.parametrize("cover_all", [False, True])
+def test_max_pool_vs_numpy(oracle, dt, cover_all):
+    rng = np.random.default_rng(34)
+    info = np.iinfo(dt)
+    for kernel, strides, pads, H, W in POOL_CASES + [((3, 3), (2, 2), (0, 0), 112, 112)]:
+        x = rng.integers(info.min, info.max + 1, size=(2, 3, H, W)).astype(dt)
+        got = oracle.max_pool_q8(x, kernel, strides, pads, cover_all)
+        np.testing.assert_array_equal(got, np_max_pool_q8(x, kernel, strides, pads, cover_all), err_msg=str((kernel, strides, pads)))
+    # kernel = whole image: the maximum of each plane
+    x = rng.integers(info.min, info.max + 1, size=(2, 3, 6, 5)).astype(dt)
+    np.testing.assert_array_equal(oracle.max_pool_q8(x, (6, 5), (1, 1), (0, 0), cover_all).reshape(2, 3), x.max(axis=(2, 3)))
+
+
+def test_max_pool_on_codes_equals_the_three_float_ops_for_uint8(oracle):
+    """DequantizeLinear -> MaxPool over a -inf padded float tensor -> QuantizeLinear, spelled out, gives the maximum
+    of the codes for uint8 (increasing dequantization, Q(DQ(q)) == q), for any zero point and window."""
+    rng = np.random.default_rng(35)
+    for kernel, strides, pads, H, W in POOL_CASES:
+        x = rng.integers(0, 256, size=(1, 2, H, W)).astype(np.uint8)
+        zp = int(rng.integers(0, 256))
+        scale = np.float32(rng.uniform(0.01, 0.2))
+        got = oracle.max_pool_q8(x, kernel, strides, pads, False)
+        OH, OW = got.shape[2:]
+        val = np.full((1, 2, H + 2 * pads[0], W + 2 * pads[1]), -np.inf, np.float32)
+        val[:, :, pads[0]:pads[0] + H, pads[1]:pads[1] + W] = np_dequantize(x, scale, zp)
+        want = np.full((1, 2, OH, OW), -np.inf, np.float32)
+        for i in range(kernel[0]):
+            for j in range(kernel[1]):
+                want = np.maximum(want, val[:, :, i:i + (OH - 1) * strides[0] + 1:strides[0], j:j + (OW - 1) * strides[1] + 1:strides[1]])
+        with np.errstate(all="ignore"):
+            np.testing.assert_array_equal(got, np_quantize(want, scale, zp, 0, 255).astype(np.uint8))
