@@ -43,6 +43,10 @@ def parse():
                     help="run the residual Add(+Relu) groups as kernels of their own instead of inside the convolution before them")
     ap.add_argument("--parts", type=int, default=1,
                     help="run the batch as this many concurrent slices on separate streams (network workloads)")
+    ap.add_argument("--runner", default="chxvm", choices=["chxvm", "python"],
+                    help="network workloads: chxvm = the serialized ChxVMProgramProto through the C++ VM of the runtime library "
+                         "(libchxvm_hip_runtime.so), its run recorded into a device graph and replayed; python = the op program "
+                         "driven from Python through the C ABI (ops.py), also replayed as a graph")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one plain copy kernel (fused Identity on float32) over this many MiB: the known traffic "
                          "that hardware counters of a profiling run are scaled against")
@@ -115,7 +119,8 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # default is the plain whole-batch runner, whose launches are the ones the roofline figure
     # below prices.
     fuse = not args.no_fuse_residual
-    runner = wl.DeviceRunner(model, pkg, fuse) if args.parts <= 1 else None
+    # values share memory once their last reader has run, as in the VM (whose allocator reuses freed slots)
+    runner = wl.DeviceRunner(model, pkg, fuse, reuse_buffers=True) if args.parts <= 1 else None
     timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts, fuse)
 
     def step(_timer):
@@ -123,7 +128,23 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
 
     # The timed region replays the whole program as one HIP graph (about 125 launches per step
     # would otherwise be bound by the host); --no-graph launches every op from the host instead.
-    if args.no_graph:
+    vm_prog = vm_replay = None
+    use_vm = args.runner == "chxvm" and args.parts <= 1 and fuse
+    if use_vm:
+        # the drop-in itself: the network as one serialized program in the C++ VM
+        import importlib
+        vm = importlib.import_module(pkg.__name__ + ".chxvm")
+        vm_prog = vm.Program(wl.program_to_chxvm(model, vm, ops, keep=("logits",)).serialize())
+        vm_prog.set_option("qlinearconv_bias", "onnx_int32")
+        if args.no_graph:
+            def step(_timer):  # noqa: F811  (the host walks the instructions; results are copied back, as run_onnx does)
+                vm_prog.run({"x": x})
+            sec = timed_steps(torch, step, args.steps, args.warmup)
+        else:
+            vm_replay = vm_prog.capture({"x": x})
+            stream = capi.stream_ptr()
+            sec = timed_steps(torch, lambda _t: vm_replay.launch(stream), args.steps, args.warmup)
+    elif args.no_graph:
         sec = timed_steps(torch, step, args.steps, args.warmup)
     else:
         replay = timed_runner.capture(x)
@@ -142,8 +163,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     conv_ms_per_step, n_launch = 0.0, 0
     layer_graphs = []
     for rn, xs in slices:
-        vals = rn.run(xs)
+        rn.run(xs)
         torch.cuda.synchronize()
+        vals = dict(rn.bufs, x=xs)   # every value's buffer (with reuse_buffers several share memory, as in the timed step)
         fids = []
         for fid, ins in enumerate(model["program"]):
             if ins[0] != "QLinearConv":
@@ -178,17 +200,30 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                         ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
     if not mobilenet and batch == 64 and args.parts <= 1:
         # HBM bytes of the same launches from hardware counters (FETCH_SIZE / WRITE_SIZE, scaled by a
-        # copy kernel of known size): measured in two separate profiling runs, kept with their commands
+        # copy kernel of known size): NOT measured in this run but taken from two separate profiling runs,
+        # kept with their commands; traffic_source says which file, so a reader can see how old it is
         try:
             t = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
                                             "resnet50_bs64_conv_mfma_traffic.json")))
             roofline["traffic"] = t["bytes_per_step"]
+            roofline["traffic_source"] = "profiles/resnet50_bs64_conv_mfma_traffic.json (%s)" % t.get("measured_at", "separate rocprofv3 --pmc runs")
         except (OSError, ValueError, KeyError):
             pass
+    # the launch configurations the plans measured for these launches: tile (output channels x pixels) and
+    # work-groups per compute unit -> number of layers
+    hist = {}
+    for rn, _xs in slices:
+        for plan in rn.plans.values():
+            for line in plan.describe():
+                f = dict(kv.split("=") for kv in line.split() if "=" in kv)
+                key = "%s/%s%s" % (f.get("tile"), f.get("wgs_per_cu"), "+res" if f.get("res") == "1" else "")
+                hist[key] = hist.get(key, 0) + 1
+    roofline["configs"] = hist
     res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),
                value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
                config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,
                            layout="channels_last", launch="host" if args.no_graph else "hip_graph_replay",
+                           runner="chxvm (serialized ChxVMProgramProto in libchxvm_hip_runtime.so)" if use_vm else "python (ops.py over the C ABI)",
                            concurrent_batch_slices=max(1, args.parts), residual_add="separate" if args.no_fuse_residual else "in_conv_epilogue",
                            conv_gmac_per_image=model["macs"] / batch / 1e9))
 
@@ -214,6 +249,10 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                            "im2col + sequential-k fp32 GEMM, quantize) with OpenMP over %d threads: %.1f s; one image "
                            "single-threaded, as ChainerX's native device runs: %.1f s" % (nb, nb, cores, dtn, dt1))
     def runner_close():
+        if vm_replay is not None:
+            vm_replay.close()
+        if vm_prog is not None:
+            vm_prog.close()
         timed_runner.close()
     return res, roofline, cpu, runner_close
 

@@ -26,6 +26,8 @@ RUNTIME_EXPORTS = [
     "chxvm_program_create", "chxvm_program_destroy", "chxvm_program_num_instructions", "chxvm_program_num_inputs",
     "chxvm_program_input_name", "chxvm_program_run", "chxvm_outputs_count", "chxvm_outputs_name", "chxvm_outputs_get",
     "chxvm_outputs_destroy", "chxvm_backend_config_has", "chxvm_backend_config_name", "chxvm_set_option", "chxvm_counter",
+    "chxvm_program_set_option", "chxvm_program_counter", "chxvm_program_capture", "chxvm_replay_launch", "chxvm_replay_synchronize",
+    "chxvm_replay_outputs", "chxvm_replay_info", "chxvm_replay_destroy",
     "chxc_compile", "chxc_transform", "chxc_fusion_program", "chxc_quantize_data", "chxc_free",
 ]
 
@@ -83,6 +85,17 @@ def runtime():
         rt.chxc_free.restype = None
         rt.chxvm_counter.argtypes = [ctypes.c_char_p]
         rt.chxvm_counter.restype = ctypes.c_int64
+        rt.chxvm_program_set_option.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_char_p]
+        rt.chxvm_program_counter.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        rt.chxvm_program_counter.restype = ctypes.c_int64
+        rt.chxvm_replay_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        rt.chxvm_replay_synchronize.argtypes = [ctypes.c_void_p]
+        rt.chxvm_replay_outputs.argtypes = [ctypes.c_void_p]
+        rt.chxvm_replay_outputs.restype = ctypes.c_void_p
+        rt.chxvm_replay_info.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        rt.chxvm_replay_info.restype = ctypes.c_int64
+        rt.chxvm_replay_destroy.argtypes = [ctypes.c_void_p]
+        rt.chxvm_replay_destroy.restype = None
         rt.chxvm_backend_config_name.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
         _rt = rt
     return _rt
@@ -369,9 +382,71 @@ class Program:
         finally:
             rt.chxvm_outputs_destroy(out)
 
+    def capture(self, inputs):
+        """Records one run on the device buffers of `inputs` ({name: torch device tensor}; keep them alive,
+        refill them before a launch) and returns the Replay."""
+        rt = runtime()
+        names = list(inputs)
+        c_names = (ctypes.c_char_p * len(names))(*[n.encode() for n in names])
+        descs = (capi.Tensor * len(names))(*[capi.desc(inputs[n]) for n in names])
+        out = ctypes.c_void_p()
+        _check(rt.chxvm_program_capture(self._h, c_names, descs, len(names), ctypes.byref(out)))
+        return Replay(out, dict(inputs))
+
+    def set_option(self, name, value):
+        """Options of this program, overriding the process-wide ones of set_option():
+        "qlinearconv_bias" = "reference" | "onnx_int32" | "default"."""
+        _check(runtime().chxvm_program_set_option(self._h, name.encode(), value.encode()))
+
+    def counter(self, name):
+        """Event counts of this program over all its runs, e.g. "qlinearconv_residual_fusions"."""
+        return runtime().chxvm_program_counter(self._h, name.encode())
+
     def close(self):
         if self._h:
             runtime().chxvm_program_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Replay:
+    """A recorded run of a Program (chxvm_program_capture): launch() replays it on a stream."""
+
+    def __init__(self, handle, inputs):
+        self._h = handle
+        self.inputs = inputs  # keeps the input buffers alive
+
+    def launch(self, stream=None):
+        """Enqueues the recorded run; stream: a raw stream pointer (e.g. capi.stream_ptr()), None = the replay's own."""
+        _check(runtime().chxvm_replay_launch(self._h, stream))
+
+    def synchronize(self):
+        """Waits for launches on the replay's own stream."""
+        _check(runtime().chxvm_replay_synchronize(self._h))
+
+    def outputs(self):
+        """{name: numpy array} of the last launch; the device must be done with it (synchronize())."""
+        rt = runtime()
+        out = rt.chxvm_replay_outputs(self._h)
+        result = {}
+        for i in range(rt.chxvm_outputs_count(out)):
+            d = capi.Tensor()
+            _check(rt.chxvm_outputs_get(out, i, ctypes.byref(d)))
+            result[rt.chxvm_outputs_name(out, i).decode()] = _to_numpy(d)
+        return result
+
+    def info(self, name):
+        """"pool_bytes", "pool_blocks", "warm_runs"."""
+        return runtime().chxvm_replay_info(self._h, name.encode())
+
+    def close(self):
+        if self._h:
+            runtime().chxvm_replay_destroy(self._h)
             self._h = ctypes.c_void_p()
 
     def __del__(self):

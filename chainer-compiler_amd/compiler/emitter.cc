@@ -316,6 +316,12 @@ private:
                                    IntIn(n.GetInt("count_include_pad", 0))});
             }
             inst->outputs.push_back(-1);  // the backward context is not kept
+            // an instruction that names its outputs names and types all of them (the run-time type check
+            // compares the counts, runtime/chxvm.cc:38-64): the dropped context is nameless and untyped
+            if (!inst->output_names.empty()) {
+                inst->output_names.push_back("");
+                inst->output_types.push_back(ChxVMTypeProto());
+            }
         } else if (op == "Clip" && nin >= 1 && nin <= 3) {
             // compiler/chxvm/simple_node_emitter.cc:506-512: bounds as attributes or as operands
             if (nin == 1) {

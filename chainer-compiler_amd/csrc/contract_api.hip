@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <string>
 #include <vector>
 
 #include "contract.h"
@@ -342,6 +343,27 @@ bool y_is_pixel_major(const chx_hip_tensor& y, int64_t* px_stride) {
     if (stride < y.shape[1] * es) return false;
     *px_stride = stride;
     return true;
+}
+
+// [lowest, highest + 1) byte address any element of t occupies
+void byte_range(const chx_hip_tensor& t, uintptr_t* lo, uintptr_t* hi) {
+    int64_t below = 0, above = dtype_size(t.dtype);
+    for (int i = 0; i < t.ndim; ++i) {
+        if (t.shape[i] <= 1) continue;
+        const int64_t span = (t.shape[i] - 1) * t.strides[i];
+        if (span < 0) below += span;
+        else above += span;
+    }
+    *lo = reinterpret_cast<uintptr_t>(t.data) + below;
+    *hi = reinterpret_cast<uintptr_t>(t.data) + above;
+}
+
+bool byte_ranges_overlap(const chx_hip_tensor& a, const chx_hip_tensor& b) {
+    if (numel(a) == 0 || numel(b) == 0) return false;
+    uintptr_t alo, ahi, blo, bhi;
+    byte_range(a, &alo, &ahi);
+    byte_range(b, &blo, &bhi);
+    return alo < bhi && blo < ahi;
 }
 
 // Scratch buffers that outlive a call: a plan keeps its transposition / im2col space so that
@@ -915,6 +937,10 @@ extern "C" int chx_hip_qconv_plan_run_add(
                 "QLinearConv+Add: zero point out of the range of its type");
     if (!(out_scale >= 0x1p-60f && out_scale <= 0x1p60f))
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv+Add: out_scale outside [2^-60, 2^60]");
+    // `out` is written while x and r are still being read (and, when the launch configurations are timed,
+    // several times over)
+    CHX_PROPAGATE(check_tensor(x, "QLinearConv+Add x"));
+    CHX_REQUIRE(!byte_ranges_overlap(*out, *x) && !byte_ranges_overlap(*out, *r), "QLinearConv+Add: out overlaps x or r in memory");
     // the convolution's own result has the layout of `out` and the type y_dtype
     chx_hip_tensor y = *out;
     y.dtype = y_dtype;
@@ -950,6 +976,20 @@ extern "C" int chx_hip_qconv_plan_run_add(
     call.tune = const_cast<TuneCache*>(&plan->tune);
     call.res = &res;
     return run_conv_mfma(call, plan->pw, s);
+}
+
+extern "C" int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_t buf_size) {
+    CHX_REQUIRE(plan != nullptr && buf != nullptr && buf_size > 0, "QLinearConv plan: null argument");
+    std::string text;
+    for (const TunedConfig& t : plan->tune.entries) {
+        char line[160];
+        snprintf(line, sizeof(line), "M=%lld %dx%d res=%d tile=%dx%d wgs_per_cu=%d\n", (long long)t.M, t.OH, t.OW, t.with_res ? 1 : 0,
+                 t.tile_oc, t.tile_px, t.max_wgs_per_cu);
+        text += line;
+    }
+    strncpy(buf, text.c_str(), buf_size - 1);
+    buf[buf_size - 1] = 0;
+    return CHX_HIP_OK;
 }
 
 extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {

@@ -78,6 +78,10 @@ void scratch_free(void* p, hipStream_t s) {
 
 using namespace chx;
 
+struct chx_hip_graph {
+    hipGraphExec_t exec;
+};
+
 extern "C" {
 
 const char* chx_hip_last_error(void) {
@@ -156,6 +160,68 @@ int chx_hip_memset(void* dst, int value, size_t bytes, void* stream) {
 int chx_hip_stream_synchronize(void* stream) {
     CHX_HIP_CALL(hipStreamSynchronize(as_stream(stream)));
     return CHX_HIP_OK;
+}
+
+int chx_hip_stream_create(void** stream) {
+    CHX_REQUIRE(stream != nullptr, "null output");
+    hipStream_t s = nullptr;
+    CHX_HIP_CALL(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return CHX_HIP_OK;
+}
+
+int chx_hip_stream_destroy(void* stream) {
+    if (stream) CHX_HIP_CALL(hipStreamDestroy(as_stream(stream)));
+    return CHX_HIP_OK;
+}
+
+int chx_hip_capture_begin(void* stream) {
+    CHX_REQUIRE(stream != nullptr, "the null stream cannot be captured");
+    // thread-local mode: calls of other threads (another program running eagerly) are not affected
+    CHX_HIP_CALL(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return CHX_HIP_OK;
+}
+
+int chx_hip_capture_end(void* stream, chx_hip_graph** graph) {
+    CHX_REQUIRE(stream != nullptr && graph != nullptr, "null argument");
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &g);
+    if (e != hipSuccess || g == nullptr) {
+        (void)hipGetLastError();
+        if (g) (void)hipGraphDestroy(g);
+        CHX_FAIL(CHX_HIP_ERUNTIME, "the capture did not give a graph: %s", hipGetErrorString(e));
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) CHX_FAIL(CHX_HIP_ERUNTIME, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    chx_hip_graph* out = new chx_hip_graph();
+    out->exec = exec;
+    *graph = out;
+    return CHX_HIP_OK;
+}
+
+int chx_hip_stream_is_capturing(void* stream) {
+    if (!stream) return 0;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return st != hipStreamCaptureStatusNone ? 1 : 0;
+}
+
+int chx_hip_graph_launch(const chx_hip_graph* graph, void* stream) {
+    CHX_REQUIRE(graph != nullptr, "null graph");
+    CHX_HIP_CALL(hipGraphLaunch(graph->exec, as_stream(stream)));
+    return CHX_HIP_OK;
+}
+
+void chx_hip_graph_destroy(chx_hip_graph* graph) {
+    if (!graph) return;
+    (void)hipGraphExecDestroy(graph->exec);
+    delete graph;
 }
 
 }  // extern "C"

@@ -232,6 +232,15 @@ class QLinearConvPlan(object):
             _f(out_scale), _i(out_zero_point), _i(1 if relu else 0), capi.ref(out), capi.stream_ptr()))
         return out
 
+    def describe(self):
+        """The launch configurations measured so far (chx_hip_qconv_plan_describe), one per line."""
+        lines = []
+        for handle in self._plans.values():
+            buf = ctypes.create_string_buffer(4096)
+            capi.check(capi.lib().chx_hip_qconv_plan_describe(handle, buf, ctypes.c_size_t(len(buf))))
+            lines += [l for l in buf.value.decode().splitlines() if l]
+        return lines
+
     def close(self):
         for handle in self._plans.values():
             capi.lib().chx_hip_qconv_plan_destroy(handle)

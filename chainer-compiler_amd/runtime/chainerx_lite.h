@@ -291,10 +291,23 @@ public:
         return a;
     }
 
+    // An array over memory that the caller of the runtime keeps alive and may rewrite or release between
+    // runs.  Views of it (Transpose, Reshape) are borrowed as well.  Anything derived from its contents and
+    // kept beyond the instruction that reads it would go stale.
+    static Array MakeBorrowed(void* data, Dtype dtype, const Shape& shape, const Strides& strides) {
+        Array a = MakeOwned(std::shared_ptr<void>(data, [](void*) {}), dtype, shape, strides);
+        a.body_->borrowed = true;
+        return a;
+    }
+    bool IsBorrowed() const {
+        return body_->borrowed;
+    }
+
 private:
     struct Body {
         std::shared_ptr<void> data;
         int64_t offset = 0;
+        bool borrowed = false;
         Dtype dtype = Dtype::kFloat32;
         Shape shape;
         Strides strides;
@@ -315,12 +328,60 @@ inline Strides ContiguousStrides(const Shape& shape, int64_t item_size) {
     return s;
 }
 
+// Where the arrays of the calling thread come from and which stream its kernels go to.  The default is the
+// device runtime's allocator and the null stream, the counterpart of ChainerX's default device.  A run that is
+// to be captured into a graph installs a pool of its own (no allocation by the device runtime may happen while
+// a stream records) and the stream that records.
+class DeviceAllocator {
+public:
+    virtual ~DeviceAllocator() = default;
+    // memory of at least `bytes` bytes that stays valid until the returned handle is released
+    virtual std::shared_ptr<void> Allocate(size_t bytes) = 0;
+};
+
+struct DeviceContext {
+    void* stream = nullptr;
+    DeviceAllocator* allocator = nullptr;
+};
+
+inline DeviceContext& CurrentDeviceContext() {
+    thread_local DeviceContext context;
+    return context;
+}
+
+inline void* CurrentStream() {
+    return CurrentDeviceContext().stream;
+}
+
+// Installs a context for the lifetime of the object (one run of a program).
+class DeviceContextScope {
+public:
+    DeviceContextScope(void* stream, DeviceAllocator* allocator) : saved_(CurrentDeviceContext()) {
+        CurrentDeviceContext().stream = stream;
+        CurrentDeviceContext().allocator = allocator;
+    }
+    ~DeviceContextScope() {
+        CurrentDeviceContext() = saved_;
+    }
+    DeviceContextScope(const DeviceContextScope&) = delete;
+    DeviceContextScope& operator=(const DeviceContextScope&) = delete;
+
+private:
+    DeviceContext saved_;
+};
+
 // chainerx::Empty on the HIP device: C-contiguous.
 inline Array Empty(const Shape& shape, Dtype dtype) {
     const int64_t bytes = shape.GetTotalSize() * GetItemSize(dtype);
-    void* p = nullptr;
-    CHXVM_HIP_CALL(chx_hip_malloc(&p, static_cast<size_t>(bytes > 0 ? bytes : 1)));
-    std::shared_ptr<void> data(p, [](void* q) { (void)chx_hip_free(q); });
+    const size_t want = static_cast<size_t>(bytes > 0 ? bytes : 1);
+    std::shared_ptr<void> data;
+    if (DeviceAllocator* allocator = CurrentDeviceContext().allocator) {
+        data = allocator->Allocate(want);
+    } else {
+        void* p = nullptr;
+        CHXVM_HIP_CALL(chx_hip_malloc(&p, want));
+        data = std::shared_ptr<void>(p, [](void* q) { (void)chx_hip_free(q); });
+    }
     return Array::MakeOwned(std::move(data), dtype, shape, ContiguousStrides(shape, GetItemSize(dtype)));
 }
 
@@ -346,7 +407,7 @@ inline Array EmptyChannelsLastPadded(const Shape& nchw, Dtype dtype) {
 
 inline Array FromHost(const void* src, const Shape& shape, Dtype dtype) {
     Array a = Empty(shape, dtype);
-    CHXVM_HIP_CALL(chx_hip_memcpy_h2d(a.raw_data(), src, static_cast<size_t>(a.GetNBytes()), nullptr));
+    CHXVM_HIP_CALL(chx_hip_memcpy_h2d(a.raw_data(), src, static_cast<size_t>(a.GetNBytes()), chainerx::CurrentStream()));
     return a;
 }
 
@@ -362,7 +423,7 @@ inline Array Array::Reshape(const Shape& to) const {
 
 inline void ToHost(const Array& a, void* dst) {
     CHECK(a.IsContiguous()) << "ToHost needs a contiguous array";
-    CHXVM_HIP_CALL(chx_hip_memcpy_d2h(dst, static_cast<char*>(a.raw_data()) + a.offset(), static_cast<size_t>(a.GetNBytes()), nullptr));
+    CHXVM_HIP_CALL(chx_hip_memcpy_d2h(dst, static_cast<char*>(a.raw_data()) + a.offset(), static_cast<size_t>(a.GetNBytes()), chainerx::CurrentStream()));
 }
 
 // chainerx::AsScalar: the single element of an array, read back to the host (a stream
@@ -370,7 +431,7 @@ inline void ToHost(const Array& a, void* dst) {
 inline Scalar AsScalar(const Array& a) {
     CHECK_EQ(1, a.GetTotalSize()) << "AsScalar needs exactly one element";
     unsigned char buf[8] = {0};
-    CHXVM_HIP_CALL(chx_hip_memcpy_d2h(buf, static_cast<char*>(a.raw_data()) + a.offset(), static_cast<size_t>(a.GetItemSize()), nullptr));
+    CHXVM_HIP_CALL(chx_hip_memcpy_d2h(buf, static_cast<char*>(a.raw_data()) + a.offset(), static_cast<size_t>(a.GetItemSize()), chainerx::CurrentStream()));
     switch (a.dtype()) {
         case Dtype::kBool: return Scalar(buf[0] != 0);
         case Dtype::kInt8: return Scalar(int64_t(*reinterpret_cast<int8_t*>(buf)));

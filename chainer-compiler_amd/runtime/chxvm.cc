@@ -47,7 +47,7 @@ public:
                 &at, static_cast<float>(st->GetScalar(a_scale_)), static_cast<int32_t>(static_cast<int64_t>(az)), &bt,
                 static_cast<float>(st->GetScalar(b_scale_)), static_cast<int32_t>(static_cast<int64_t>(bz)),
                 static_cast<float>(st->GetScalar(y_scale_)), static_cast<int32_t>(static_cast<int64_t>(yz)),
-                nullptr, CHX_HIP_ROUND_REFERENCE, &yt, nullptr));
+                nullptr, CHX_HIP_ROUND_REFERENCE, &yt, chainerx::CurrentStream()));
         st->SetArray(y_, y);
     }
 
@@ -103,12 +103,12 @@ public:
             // Q(DQ(q)) == q holds for uint8 only: the reference's QuantizeLinear truncates after adding 0.5, so a
             // negative int8 code q comes back as q + 1, and the maximum of the codes is not what the three ops give
             CHECK(xz.dtype() == chainerx::Dtype::kUInt8) << "a quantized MaxPool of int8 codes is not computed on the hip backend";
-            CHXVM_HIP_CALL(chx_hip_max_pool_q8(&xt, kh, kw, sh, sw, pb[0], pb[1], pe[0], pe[1], cover_all ? 1 : 0, &yt, nullptr));
+            CHXVM_HIP_CALL(chx_hip_max_pool_q8(&xt, kh, kw, sh, sw, pb[0], pb[1], pe[0], pe[1], cover_all ? 1 : 0, &yt, chainerx::CurrentStream()));
         } else {
             CHECK(pb[0] == pe[0] && pb[1] == pe[1]) << "AveragePool pads must be symmetric";
             CHXVM_HIP_CALL(chx_hip_average_pool_q8(&xt, xs, static_cast<int32_t>(static_cast<int64_t>(xz)), kh, kw, sh, sw, pb[0], pb[1],
                                                    flag_, ys, static_cast<int32_t>(static_cast<int64_t>(yz)), CHX_HIP_ROUND_REFERENCE,
-                                                   &yt, nullptr));
+                                                   &yt, chainerx::CurrentStream()));
         }
         st->SetArray(y_, y);
     }
@@ -151,14 +151,14 @@ public:
         req.out_scale = g_.out_scale; req.out_zero_point = g_.out_zero_point; req.out_dtype = dt(g_.out_dtype);
         req.relu = g_.relu != 0;
         const bool r_fits = !req.r.IsNullHandle() && req.r.dtype() == dt(g_.in_dtype[1 - k_]);
-        SetQLinearConvResidualRequest(r_fits ? &req : nullptr);
+        st->set_residual_request(r_fits ? &req : nullptr);
         try {
             conv_->Run(st);
         } catch (...) {
-            SetQLinearConvResidualRequest(nullptr);
+            st->set_residual_request(nullptr);
             throw;
         }
-        SetQLinearConvResidualRequest(nullptr);
+        st->set_residual_request(nullptr);
         state_->fused = req.done;
         if (req.done) {
             if (st->trace_level()) std::cerr << "  (residual sum $" << group_out_ << " computed by the convolution)" << std::endl;
@@ -412,7 +412,7 @@ void SaveNpy(const chainerx::Array& a, const std::string& filename) {
     std::vector<char> raw(static_cast<size_t>(span)), packed(static_cast<size_t>(total * item));
     if (span) {
         const chx_hip_tensor t = a.hip();
-        CHXVM_HIP_CALL(chx_hip_memcpy_d2h(raw.data(), t.data, static_cast<size_t>(span), nullptr));
+        CHXVM_HIP_CALL(chx_hip_memcpy_d2h(raw.data(), t.data, static_cast<size_t>(span), chainerx::CurrentStream()));
     }
     std::vector<int64_t> index(static_cast<size_t>(a.ndim()), 0);
     for (int64_t flat = 0; flat < total; ++flat) {
@@ -447,7 +447,8 @@ void DumpOutput(ChxVMState* st, const ChxVMOp* op, const std::string& output_dir
         const int id = inst.outputs[i];
         const std::string& name = inst.output_names[i];
         if (id <= 0 || name.empty()) continue;
-        ChxVMVar* var = st->GetVar(id);
+        // an instruction fused away when the program was loaded leaves its named outputs unset
+        ChxVMVar* var = st->PeekVar(id);
         if (!var || !var->IsArray()) continue;
         std::string clean = name;
         for (char& c : clean)
@@ -472,8 +473,9 @@ void CheckType(ChxVMState* st, const ChxVMOp* op) {
         if (type.dtype == 0) continue;
         const int id = inst.outputs[i];
         CHECK_LT(0, id);
-        ChxVMVar* var = st->GetVar(id);
-        if (var->IsNull()) continue;
+        // unset: the instruction was fused into a neighbour when the program was loaded (or its result freed already)
+        ChxVMVar* var = st->PeekVar(id);
+        if (!var || var->IsNull() || !var->IsArray()) continue;
         const chainerx::Array& a = st->GetArray(id);
         CHECK_EQ(static_cast<chainerx::Dtype>(type.dtype), a.dtype()) << "Dtype check failed in output #" << i << ": " << op->debug_info();
         CHECK_EQ(ShapeOf(type), a.shape()) << "Shape check failed in output #" << i << ": " << op->debug_info();
@@ -518,7 +520,7 @@ InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
             throw;
         }
         if (options.chrome_tracing) {
-            CHXVM_HIP_CALL(chx_hip_stream_synchronize(nullptr));
+            CHXVM_HIP_CALL(chx_hip_stream_synchronize(chainerx::CurrentStream()));
             options.chrome_tracing->End(event);
         }
         state.set_pc(state.pc() + 1);  // jumps set pc - 1 themselves (runtime/ops/controlflow.cc:7-21)
@@ -534,6 +536,7 @@ InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
         state.ShowVariableStatus();
         std::cerr << "Peak memory usage=" << peak_used_mbs << "MB" << std::endl;
     }
+    residual_fusions_ += state.residual_fusions();
     return state.GetOutputs();
 }
 

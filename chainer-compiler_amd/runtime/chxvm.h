@@ -11,12 +11,8 @@
 namespace chainer_compiler {
 namespace runtime {
 
-// QLinearConv bias: false (default) = the reference's unscaled float bias, true = the ONNX
-// operator's int32 bias added to the accumulator.
-void SetQLinearConvOnnxInt32Bias(bool on);
-
-// A residual sum that the next QLinearConvOp::RunImpl on this thread may compute inside its
-// kernel: out = QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r))) for its own result
+// A residual sum that the next QLinearConvOp::RunImpl of a run (ChxVMState::set_residual_request) may
+// compute inside its kernel: out = QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r))) for its own result
 // y.  The op takes the request when y's quantization is the one the group dequantizes with and the
 // kernel accepts the operands; it then sets `done`, leaves the group's result in `out` and returns
 // a null array for y.  Otherwise it runs as usual and the caller runs the group afterwards.
@@ -29,8 +25,7 @@ struct QLinearConvResidualRequest {
     chainerx::Array out;
     bool done = false;
 };
-void SetQLinearConvResidualRequest(QLinearConvResidualRequest* request);  // null clears it
-int64_t QLinearConvResidualFusions();  // requests taken so far, process-wide
+int64_t QLinearConvResidualFusions();  // requests taken so far, process-wide (a statistic; the runs count their own)
 // Whether programs loaded from now on pair such convolutions and groups at all (default: yes).
 void SetFuseResidual(bool on);
 
@@ -41,6 +36,10 @@ public:
 
     // Runs the whole program; returns the values named by its Out instructions.
     InOuts Run(const InOuts& program_inputs, const ChxVMOptions& options);
+    // residual sums that convolutions of this program computed inside their kernels, over all runs
+    int64_t residual_fusions() const {
+        return residual_fusions_;
+    }
 
     int num_variables() const {
         return num_variables_;
@@ -57,6 +56,7 @@ private:
     std::vector<std::string> input_names_;
     std::vector<ChxVMTypeProto> input_types_;
     int num_variables_ = 0;
+    int64_t residual_fusions_ = 0;
 };
 
 }  // namespace runtime

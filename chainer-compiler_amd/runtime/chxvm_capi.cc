@@ -7,6 +7,7 @@
 #include "chrome_tracing.h"
 #include "chxvm.h"
 #include "configs/backend_config.h"
+#include "replay.h"
 
 using chainer_compiler::BackendConfig;
 using namespace chainer_compiler::runtime;
@@ -17,6 +18,7 @@ thread_local std::string g_last_error;
 // run options of chxvm_set_option, applied by every later chxvm_program_run
 std::string g_chrome_tracing_path, g_dump_outputs_dir;
 bool g_check_nans = false, g_check_infs = false, g_check_types = false;
+bool g_onnx_int32_bias = false;  // the default of programs that have not been given their own (chxvm_program_set_option)
 int g_dump_memory_usage = 0;
 
 template <class Fn>
@@ -43,6 +45,7 @@ void SetLastError(const std::string& message) {
 
 struct chxvm_program {
     std::unique_ptr<ChxVM> vm;
+    int onnx_int32_bias = -1;  // -1: the process default at the time of a run
 };
 
 struct chxvm_outputs {
@@ -50,6 +53,41 @@ struct chxvm_outputs {
     std::vector<chainerx::Array> arrays;
     InOuts keep_inputs;
 };
+
+struct chxvm_replay {
+    std::shared_ptr<PoolAllocator> pool;
+    void* stream = nullptr;
+    chx_hip_graph* graph = nullptr;
+    chxvm_outputs outputs;
+    int32_t warm_runs = 0;
+
+    ~chxvm_replay() {
+        chx_hip_graph_destroy(graph);
+        outputs.arrays.clear();
+        outputs.keep_inputs.clear();
+        if (stream) (void)chx_hip_stream_destroy(stream);
+    }
+};
+
+namespace {
+
+InOuts BorrowInputs(const char* const* input_names, const chx_hip_tensor* inputs, int32_t num_inputs) {
+    InOuts in;
+    for (int32_t i = 0; i < num_inputs; ++i) {
+        const chx_hip_tensor& t = inputs[i];
+        chainerx::Shape shape;
+        chainerx::Strides strides;
+        for (int d = 0; d < t.ndim; ++d) {
+            shape.push_back(t.shape[d]);
+            strides.push_back(t.strides[d]);
+        }
+        chainerx::Array a = chainerx::Array::MakeBorrowed(t.data, static_cast<chainerx::Dtype>(t.dtype), shape, strides);
+        CHECK(in.emplace(input_names[i], std::make_shared<ChxVMVar>(a)).second) << "duplicate input " << input_names[i];
+    }
+    return in;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -116,19 +154,7 @@ int32_t chxvm_program_run(
         int32_t trace_level,
         chxvm_outputs** out) {
     return Guard([&] {
-        InOuts in;
-        for (int32_t i = 0; i < num_inputs; ++i) {
-            const chx_hip_tensor& t = inputs[i];
-            chainerx::Shape shape;
-            chainerx::Strides strides;
-            for (int d = 0; d < t.ndim; ++d) {
-                shape.push_back(t.shape[d]);
-                strides.push_back(t.strides[d]);
-            }
-            std::shared_ptr<void> borrowed(t.data, [](void*) {});
-            chainerx::Array a = chainerx::Array::MakeOwned(borrowed, static_cast<chainerx::Dtype>(t.dtype), shape, strides);
-            CHECK(in.emplace(input_names[i], std::make_shared<ChxVMVar>(a)).second) << "duplicate input " << input_names[i];
-        }
+        InOuts in = BorrowInputs(input_names, inputs, num_inputs);
         ChxVMOptions options;
         options.trace_level = trace_level;
         options.dump_outputs_dir = g_dump_outputs_dir;
@@ -136,6 +162,7 @@ int32_t chxvm_program_run(
         options.check_infs = g_check_infs;
         options.check_types = g_check_types;
         options.dump_memory_usage = g_dump_memory_usage;
+        options.qlinearconv_onnx_int32_bias = program->onnx_int32_bias >= 0 ? program->onnx_int32_bias != 0 : g_onnx_int32_bias;
         std::unique_ptr<ChromeTracingEmitter> tracing;
         if (!g_chrome_tracing_path.empty()) {
             tracing.reset(new ChromeTracingEmitter());
@@ -152,6 +179,84 @@ int32_t chxvm_program_run(
         CHXVM_HIP_CALL(chx_hip_stream_synchronize(nullptr));  // device sync at the end of a run (tools/run_onnx.cc:462)
         *out = o.release();
     });
+}
+
+int32_t chxvm_program_capture(
+        chxvm_program* program, const char* const* input_names, const chx_hip_tensor* inputs, int32_t num_inputs, chxvm_replay** out) {
+    return Guard([&] {
+        CHECK(program != nullptr && out != nullptr) << "null argument";
+        *out = nullptr;
+        InOuts in = BorrowInputs(input_names, inputs, num_inputs);
+        ChxVMOptions options;  // no tracing, checking or dumping: all of them read results back
+        options.qlinearconv_onnx_int32_bias = program->onnx_int32_bias >= 0 ? program->onnx_int32_bias != 0 : g_onnx_int32_bias;
+        std::unique_ptr<chxvm_replay> r(new chxvm_replay());
+        r->pool = std::make_shared<PoolAllocator>();
+        CHXVM_HIP_CALL(chx_hip_stream_create(&r->stream));
+        // Eager runs on the stream until one of them finds every block it asks for in the pool: plans are
+        // built, launch configurations measured, fused kernels compiled, and the pool reaches the state that
+        // the recorded run starts from.
+        for (;;) {
+            const int64_t before = r->pool->blocks_created();
+            {
+                chainerx::DeviceContextScope scope(r->stream, r->pool.get());
+                (void)program->vm->Run(in, options);
+            }
+            CHXVM_HIP_CALL(chx_hip_stream_synchronize(r->stream));
+            ++r->warm_runs;
+            if (r->pool->blocks_created() == before) break;
+            CHECK_LT(r->warm_runs, 8) << "the runs of this program keep allocating new blocks";
+        }
+        r->pool->set_frozen(true);
+        CHXVM_HIP_CALL(chx_hip_capture_begin(r->stream));
+        InOuts result;
+        try {
+            chainerx::DeviceContextScope scope(r->stream, r->pool.get());
+            result = program->vm->Run(in, options);
+        } catch (...) {
+            chx_hip_graph* dropped = nullptr;
+            (void)chx_hip_capture_end(r->stream, &dropped);
+            chx_hip_graph_destroy(dropped);
+            throw;
+        }
+        CHXVM_HIP_CALL(chx_hip_capture_end(r->stream, &r->graph));
+        for (const auto& p : result) {
+            r->outputs.names.push_back(p.first);
+            r->outputs.arrays.push_back(p.second->GetArray());
+        }
+        r->outputs.keep_inputs = in;
+        *out = r.release();
+    });
+}
+
+int32_t chxvm_replay_launch(chxvm_replay* replay, void* stream) {
+    return Guard([&] {
+        CHECK(replay != nullptr && replay->graph != nullptr) << "null replay";
+        CHXVM_HIP_CALL(chx_hip_graph_launch(replay->graph, stream ? stream : replay->stream));
+    });
+}
+
+int32_t chxvm_replay_synchronize(chxvm_replay* replay) {
+    return Guard([&] {
+        CHECK(replay != nullptr) << "null replay";
+        CHXVM_HIP_CALL(chx_hip_stream_synchronize(replay->stream));
+    });
+}
+
+const chxvm_outputs* chxvm_replay_outputs(const chxvm_replay* replay) {
+    return replay ? &replay->outputs : nullptr;
+}
+
+int64_t chxvm_replay_info(const chxvm_replay* replay, const char* name) {
+    const std::string n = name ? name : "";
+    if (!replay) return -1;
+    if (n == "pool_bytes") return replay->pool->bytes_reserved();
+    if (n == "pool_blocks") return replay->pool->blocks_created();
+    if (n == "warm_runs") return replay->warm_runs;
+    return -1;
+}
+
+void chxvm_replay_destroy(chxvm_replay* replay) {
+    delete replay;
 }
 
 int32_t chxvm_outputs_count(const chxvm_outputs* outputs) {
@@ -178,7 +283,7 @@ int32_t chxvm_set_option(const char* name, const char* value) {
         const std::string n = name, v = value;
         if (n == "qlinearconv_bias") {
             CHECK(v == "reference" || v == "onnx_int32") << "qlinearconv_bias is 'reference' or 'onnx_int32', got " << v;
-            SetQLinearConvOnnxInt32Bias(v == "onnx_int32");
+            g_onnx_int32_bias = v == "onnx_int32";
         } else if (n == "fuse_residual") {
             CHECK(v == "on" || v == "off") << "fuse_residual is 'on' or 'off', got " << v;
             SetFuseResidual(v == "on");
@@ -196,6 +301,25 @@ int32_t chxvm_set_option(const char* name, const char* value) {
             CHECK(false) << "unknown option " << n;
         }
     });
+}
+
+int32_t chxvm_program_set_option(chxvm_program* program, const char* name, const char* value) {
+    return Guard([&] {
+        CHECK(program != nullptr) << "null program";
+        const std::string n = name, v = value;
+        if (n == "qlinearconv_bias") {
+            CHECK(v == "reference" || v == "onnx_int32" || v == "default") << "qlinearconv_bias is 'reference', 'onnx_int32' or 'default', got " << v;
+            program->onnx_int32_bias = v == "default" ? -1 : v == "onnx_int32" ? 1 : 0;
+        } else {
+            CHECK(false) << "unknown program option " << n;
+        }
+    });
+}
+
+int64_t chxvm_program_counter(const chxvm_program* program, const char* name) {
+    const std::string n = name ? name : "";
+    if (program && n == "qlinearconv_residual_fusions") return program->vm->residual_fusions();
+    return -1;
 }
 
 int64_t chxvm_counter(const char* name) {

@@ -51,7 +51,37 @@ const char* chxvm_outputs_name(const chxvm_outputs* outputs, int32_t i);
 int32_t chxvm_outputs_get(const chxvm_outputs* outputs, int32_t i, chx_hip_tensor* out);
 void chxvm_outputs_destroy(chxvm_outputs* outputs);
 
-/* name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32";
+/* One run of the program recorded into a device graph.  A program of the quantized-inference path does the
+ * same work on every run, so the run is recorded once and replayed without the host walking the
+ * instructions (the reference's interpreter launches every kernel from the host, runtime/chxvm.cc:168-236).
+ * capture() runs the program eagerly until its device memory comes out of a pool of the replay's own without
+ * growing it (plans are built and launch configurations measured on the way), then records one more run.
+ * The inputs are the device buffers of the descriptors: the caller keeps them alive and refills them before a
+ * launch.  A program whose run reads results back to the host (data-dependent scalars, as in a dynamically
+ * quantized graph; the debugging options) cannot be recorded: capture() fails with the reason, nothing is left
+ * recording.  launch() enqueues the recorded run on `stream`, or on the replay's own stream when that is
+ * null (synchronize() waits for it); the outputs (same names and shapes on every launch) are device memory of
+ * the replay, valid until destroy, rewritten by every launch.  One replay must not be launched concurrently
+ * with itself. */
+typedef struct chxvm_replay chxvm_replay;
+int32_t chxvm_program_capture(
+        chxvm_program* program, const char* const* input_names, const chx_hip_tensor* inputs, int32_t num_inputs, chxvm_replay** out);
+int32_t chxvm_replay_launch(chxvm_replay* replay, void* stream);
+int32_t chxvm_replay_synchronize(chxvm_replay* replay);
+const chxvm_outputs* chxvm_replay_outputs(const chxvm_replay* replay);  /* owned by the replay: do not destroy */
+/* name "pool_bytes" / "pool_blocks": device memory the replay holds; "warm_runs": eager runs before the recorded one */
+int64_t chxvm_replay_info(const chxvm_replay* replay, const char* name);
+void chxvm_replay_destroy(chxvm_replay* replay);
+
+/* Options of one program, which override the process-wide ones below.  name "qlinearconv_bias": value
+ * "reference", "onnx_int32", or "default" (follow chxvm_set_option again).  Programs with different
+ * settings may run in one process, also concurrently. */
+int32_t chxvm_program_set_option(chxvm_program* program, const char* name, const char* value);
+/* Event counts of one program over all its runs; names as for chxvm_counter. */
+int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
+
+/* Process-wide defaults, read when a run starts.
+ * name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32";
  * name "fuse_residual": value "on" (default) or "off": whether a QLinearConv read only by a
  * residual-sum group computes that group inside its kernel (decided when a program is loaded);
  * name "chrome_tracing": value a file name; every later chxvm_program_run writes its

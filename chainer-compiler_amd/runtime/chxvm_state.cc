@@ -19,6 +19,11 @@ ChxVMVar* ChxVMState::GetVar(int index) {
     return variables_[index].get();
 }
 
+ChxVMVar* ChxVMState::PeekVar(int index) {
+    if (index < 0 || index >= static_cast<int>(variables_.size())) return nullptr;
+    return variables_[index].get();
+}
+
 void ChxVMState::SetVar(int index, const ChxVMVar& var) {
     CHECK_LE(0, index);
     CHECK_GT(static_cast<int>(variables_.size()), index);
@@ -99,7 +104,7 @@ bool HasNonFinite(const ChxVMVar& var, bool infinities) {
     if (a.dtype() != chainerx::Dtype::kFloat32 || a.GetTotalSize() == 0) return false;
     chx_hip_tensor t = a.hip();
     int64_t count = 0;
-    CHXVM_HIP_CALL(chx_hip_count_nonfinite(&t, infinities ? 1 : 0, &count, nullptr));
+    CHXVM_HIP_CALL(chx_hip_count_nonfinite(&t, infinities ? 1 : 0, &count, chainerx::CurrentStream()));
     return count != 0;
 }
 

@@ -15,6 +15,7 @@ namespace runtime {
 typedef std::map<std::string, std::shared_ptr<ChxVMVar>> InOuts;
 
 class ChromeTracingEmitter;
+struct QLinearConvResidualRequest;
 
 struct ChxVMOptions {
     int trace_level = 0;
@@ -33,6 +34,9 @@ struct ChxVMOptions {
     // every named array output of every instruction as <dir>/<5-digit instruction id>_<name>.npy
     // (runtime/chxvm.cc:70-92)
     std::string dump_outputs_dir;
+    // QLinearConv bias: false = the reference's unscaled float bias added after the convolution
+    // (runtime/ops/quantize.cc:93), true = the ONNX operator's int32 bias added to the accumulator
+    bool qlinearconv_onnx_int32_bias = false;
 };
 
 class ChxVMState {
@@ -55,6 +59,8 @@ public:
     void SetArrayList(const std::vector<int>& index, const std::vector<chainerx::Array>& vars);
 
     ChxVMVar* GetVar(int index);
+    // the same without the check that the slot is set: null for a slot that holds nothing (never written, or freed)
+    ChxVMVar* PeekVar(int index);
     void SetVar(int index, const ChxVMVar& var);
 
     const chainerx::Shape& GetShape(int index);
@@ -97,6 +103,25 @@ public:
     bool check_infs() const {
         return options_.check_infs;
     }
+    const ChxVMOptions& options() const {
+        return options_;
+    }
+
+    // A residual sum that the next QLinearConvOp::RunImpl of this run may compute inside its kernel
+    // (see QLinearConvResidualRequest in chxvm.h); null when none is pending.
+    QLinearConvResidualRequest* residual_request() const {
+        return residual_request_;
+    }
+    void set_residual_request(QLinearConvResidualRequest* request) {
+        residual_request_ = request;
+    }
+    // residual sums computed inside a convolution during this run
+    int64_t residual_fusions() const {
+        return residual_fusions_;
+    }
+    void count_residual_fusion() {
+        ++residual_fusions_;
+    }
 
 private:
     void CheckNonFinite(const std::vector<int>& inputs, const std::vector<int>& outputs, bool infinities);
@@ -106,6 +131,8 @@ private:
     InOuts inputs_;
     InOuts outputs_;
     ChxVMOptions options_;
+    QLinearConvResidualRequest* residual_request_ = nullptr;
+    int64_t residual_fusions_ = 0;
 };
 
 }  // namespace runtime

@@ -79,7 +79,7 @@ std::vector<chainerx::Array> ElementWiseNvrtcOp::RunImpl(ChxVMState* st, const s
     for (chx_hip_tensor& t : in_desc) in_ptr.push_back(&t);
     for (chx_hip_tensor& t : out_desc) out_ptr.push_back(&t);
     CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), fusion_id, in_ptr.data(), static_cast<int32_t>(in_ptr.size()), out_ptr.data(),
-                                       static_cast<int32_t>(out_ptr.size()), nullptr));
+                                       static_cast<int32_t>(out_ptr.size()), chainerx::CurrentStream()));
     return outputs;
 }
 
@@ -108,7 +108,7 @@ chainerx::Array RunFloatOp(const char* op, const std::vector<chainerx::Array>& i
     std::vector<const chx_hip_tensor*> in_ptr;
     for (chx_hip_tensor& t : in_desc) in_ptr.push_back(&t);
     chx_hip_tensor* out_ptr = &out_desc;
-    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, in_ptr.data(), static_cast<int32_t>(in_ptr.size()), &out_ptr, 1, nullptr));
+    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, in_ptr.data(), static_cast<int32_t>(in_ptr.size()), &out_ptr, 1, chainerx::CurrentStream()));
     return y;
 }
 
@@ -168,7 +168,7 @@ chainerx::Array ClipTo(const chainerx::Array& x, float lo, float hi) {
     chx_hip_tensor in_desc = x.hip(), out_desc = y.hip();
     const chx_hip_tensor* in_ptr = &in_desc;
     chx_hip_tensor* out_ptr = &out_desc;
-    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, &in_ptr, 1, &out_ptr, 1, nullptr));
+    CHXVM_HIP_CALL(chx_hip_elementwise(code.c_str(), 0, &in_ptr, 1, &out_ptr, 1, chainerx::CurrentStream()));
     return y;
 }
 
@@ -209,7 +209,7 @@ chainerx::Array ReduceAll(const chainerx::Array& x, const chainerx::StackVector<
     CHECK(x.dtype() == chainerx::Dtype::kFloat32) << "ReduceMin / ReduceMax run on float32 arrays on the hip backend";
     chainerx::Array y = chainerx::Empty(chainerx::Shape{}, chainerx::Dtype::kFloat32);
     chx_hip_tensor xt = x.hip(), yt = y.hip();
-    CHXVM_HIP_CALL(chx_hip_reduce_min_max(&xt, is_max ? 1 : 0, &yt, nullptr));
+    CHXVM_HIP_CALL(chx_hip_reduce_min_max(&xt, is_max ? 1 : 0, &yt, chainerx::CurrentStream()));
     return y;
 }
 
@@ -228,7 +228,7 @@ chainerx::Array CastOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
     if (dt == input.dtype()) return input;
     chainerx::Array y = chainerx::Empty(input.shape(), dt);
     chx_hip_tensor xt = input.hip(), yt = y.hip();
-    CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, nullptr));
+    CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, chainerx::CurrentStream()));
     return y;
 }
 

@@ -12,8 +12,6 @@ namespace runtime {
 
 namespace {
 
-bool g_onnx_int32_bias = false;
-thread_local QLinearConvResidualRequest* g_residual_request = nullptr;
 std::atomic<int64_t> g_residual_fusions{0};
 
 StrictScalar DefaultZeroPoint() {
@@ -33,17 +31,6 @@ chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& sha
 
 }  // namespace
 
-// The reference adds the bias of a QLinearConv as an unscaled float after the convolution
-// (runtime/ops/quantize.cc:93); networks quantized for the ONNX operator carry an int32 bias at
-// scale x_scale * w_scale[oc].  This switch selects which of the two the op computes.
-void SetQLinearConvOnnxInt32Bias(bool on) {
-    g_onnx_int32_bias = on;
-}
-
-void SetQLinearConvResidualRequest(QLinearConvResidualRequest* request) {
-    g_residual_request = request;
-}
-
 int64_t QLinearConvResidualFusions() {
     return g_residual_fusions.load();
 }
@@ -55,7 +42,7 @@ chainerx::Array QuantizeLinearOp::RunImpl(
     chainerx::Array y = EmptyLike4d(x, x.shape(), y_zero_point.dtype());
     chx_hip_tensor xt = x.hip(), yt = y.hip();
     CHXVM_HIP_CALL(chx_hip_quantize_linear(&xt, static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)),
-                                           CHX_HIP_ROUND_REFERENCE, &yt, nullptr));
+                                           CHX_HIP_ROUND_REFERENCE, &yt, chainerx::CurrentStream()));
     return y;
 }
 
@@ -65,18 +52,40 @@ chainerx::Array DequantizeLinearOp::RunImpl(
     chainerx::Array y = EmptyLike4d(x, x.shape(), chainerx::Dtype::kFloat32);
     chx_hip_tensor xt = x.hip(), yt = y.hip();
     CHXVM_HIP_CALL(chx_hip_dequantize_linear(&xt, static_cast<float>(x_scale),
-                                             static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &yt, nullptr));
+                                             static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &yt, chainerx::CurrentStream()));
     return y;
 }
 
-// Per-instruction state: the plan holds the weights repacked for the MFMA kernel.  The
-// reference re-dequantizes the weights on every call (quantize.cc:76-88); an op object lives as
-// long as the program, so the repacking is done once.
+// Per-instruction state: the plan holds the weights repacked for the MFMA kernel (and the device addresses
+// of the scales, zero points and bias).  The reference re-dequantizes the weights on every call
+// (quantize.cc:76-88); an op object lives as long as the program, so for operands that are constants of
+// the program the repacking is done once.  The plan is tied to the four operand arrays it was built
+// from: the op keeps a reference to each (their memory cannot be released and handed out again while the
+// plan lives) and rebuilds the plan when a run brings other ones.  Operands that come from the caller
+// of the runtime (program inputs: memory that may be rewritten or released between runs) get no plan;
+// such a convolution goes through the one-shot entry point, which repacks per call.
 class QLinearConvOp::QLinearConvImpl {
 public:
     chx_hip_qconv_plan* plan = nullptr;
     chx_hip_conv_params params;
-    void* w_data = nullptr;
+    chainerx::Array w, w_scale, w_zero_point, bias;  // what the plan was built from
+
+    bool Matches(const chainerx::Array& q_w, const chainerx::Array& s, const chainerx::Array& z, const absl::optional<chainerx::Array>& b,
+                 const chx_hip_conv_params& p) const {
+        auto same = [](const chainerx::Array& kept, const chainerx::Array& now) {
+            return !kept.IsNullHandle() && kept.raw_data() == now.raw_data() && kept.offset() == now.offset() &&
+                   kept.shape() == now.shape() && kept.strides() == now.strides() && kept.dtype() == now.dtype();
+        };
+        if (!same(w, q_w) || !same(w_scale, s) || !same(w_zero_point, z)) return false;
+        if (b.has_value() != !bias.IsNullHandle()) return false;
+        if (b.has_value() && !same(bias, *b)) return false;
+        return memcmp(&params, &p, sizeof(p)) == 0;
+    }
+    void Drop() {
+        chx_hip_qconv_plan_destroy(plan);
+        plan = nullptr;
+        w = w_scale = w_zero_point = bias = chainerx::Array();
+    }
 };
 
 void QLinearConvOp::InitImpl() {
@@ -103,22 +112,36 @@ chainerx::Array QLinearConvOp::RunImpl(
     CHECK_EQ(w_scale.shape().size(), w_zero_point.shape().size());
     CheckQuantizedDtype(y_zero_point.dtype(), "QLinearConv y_zero_point");
     const chx_hip_conv_params p = MakeConvParams(q_x, q_w, strides, pads, group, auto_pad);
-    // the plan is keyed on the weight array and the completed attributes; both are constants
-    // of the instruction in every program the compiler emits
-    if (impl_->plan && (impl_->w_data != q_w.raw_data() || memcmp(&impl_->params, &p, sizeof(p)) != 0)) {
-        chx_hip_qconv_plan_destroy(impl_->plan);
-        impl_->plan = nullptr;
+    const chainerx::Shape y_shape = ConvOutputShape(q_x, q_w, p);
+    // The reference adds the bias as an unscaled float after the convolution (runtime/ops/quantize.cc:93);
+    // networks quantized for the ONNX operator carry an int32 bias at scale x_scale * w_scale[oc].  The
+    // options of the run say which of the two this program means.
+    const uint32_t flags =
+            CHX_HIP_ROUND_REFERENCE | (st->options().qlinearconv_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
+    const bool constants = !q_w.IsBorrowed() && !w_scale.IsBorrowed() && !w_zero_point.IsBorrowed() && !(b.has_value() && b->IsBorrowed());
+    if (!constants) {
+        if (impl_->plan) impl_->Drop();
+        chainerx::Array y = chainerx::EmptyChannelsLastPadded(y_shape, y_zero_point.dtype());
+        chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), yt = y.hip(), bt;
+        if (b.has_value()) bt = b->hip();
+        CHXVM_HIP_CALL(chx_hip_qlinear_conv(
+                &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &wt, &st2, &zt,
+                static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), b.has_value() ? &bt : nullptr, &p,
+                flags, &yt, chainerx::CurrentStream()));
+        return y;
     }
+    if (impl_->plan && !impl_->Matches(q_w, w_scale, w_zero_point, b, p)) impl_->Drop();
     if (!impl_->plan) {
         chx_hip_tensor wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), bt;
         if (b.has_value()) bt = b->hip();
         CHXVM_HIP_CALL(chx_hip_qconv_plan_create(&wt, &st2, &zt, b.has_value() ? &bt : nullptr, &p, nullptr, &impl_->plan));
         impl_->params = p;
-        impl_->w_data = q_w.raw_data();
+        impl_->w = q_w;
+        impl_->w_scale = w_scale;
+        impl_->w_zero_point = w_zero_point;
+        impl_->bias = b.has_value() ? *b : chainerx::Array();
     }
-    const chainerx::Shape y_shape = ConvOutputShape(q_x, q_w, p);
-    const uint32_t flags = CHX_HIP_ROUND_REFERENCE | (g_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
-    if (QLinearConvResidualRequest* req = g_residual_request) {
+    if (QLinearConvResidualRequest* req = st->residual_request()) {
         const bool same_quantization = static_cast<float>(y_scale) == req->y_scale &&
                                        static_cast<int64_t>(y_zero_point) == req->y_zero_point && y_zero_point.dtype() == req->y_dtype;
         if (same_quantization && !req->r.IsNullHandle() && req->r.shape() == y_shape) {
@@ -127,11 +150,12 @@ chainerx::Array QLinearConvOp::RunImpl(
             const int rc = chx_hip_qconv_plan_run_add(
                     impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
                     req->y_scale, req->y_zero_point, static_cast<int32_t>(req->y_dtype), flags, &rt, req->r_scale, req->r_zero_point,
-                    req->out_scale, req->out_zero_point, req->relu ? 1 : 0, &ot, nullptr);
+                    req->out_scale, req->out_zero_point, req->relu ? 1 : 0, &ot, chainerx::CurrentStream());
             if (rc == CHX_HIP_OK) {
                 req->out = out;
                 req->done = true;
                 ++g_residual_fusions;
+                st->count_residual_fusion();
                 return chainerx::Array();
             }
             CHECK_EQ(CHX_HIP_EUNSUPPORTED, rc) << chx_hip_last_error();  // unsupported: run the ops one by one
@@ -140,10 +164,9 @@ chainerx::Array QLinearConvOp::RunImpl(
     // 8-bit activations leave a convolution channels-last, whatever layout came in
     chainerx::Array y = chainerx::EmptyChannelsLastPadded(y_shape, y_zero_point.dtype());
     chx_hip_tensor xt = q_x.hip(), yt = y.hip();
-    // the reference hands the raw bias to the fp32 convolution (quantize.cc:93)
     CHXVM_HIP_CALL(chx_hip_qconv_plan_run(
             impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
-            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, nullptr));
+            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, chainerx::CurrentStream()));
     return y;
 }
 

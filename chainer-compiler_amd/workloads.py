@@ -280,13 +280,17 @@ class DeviceRunner(object):
     """Runs a program on the MI355X: weights resident, one plan per QLinearConv, every
     activation channels-last, all intermediate buffers allocated once."""
 
-    def __init__(self, model, pkg, fuse_residual=False):
+    def __init__(self, model, pkg, fuse_residual=False, reuse_buffers=False):
         """fuse_residual: a QLinearConv whose only reader is the residual Add(+Relu) of its block runs
-        as one kernel with it; the convolution's own output is then not materialised."""
+        as one kernel with it; the convolution's own output is then not materialised.
+        reuse_buffers: a value's memory goes back to a pool after its last reader and is handed to later
+        values (as the VM's allocator does when the program frees a slot): the working set of a step is
+        then a few tensors instead of every tensor of the network, and run() returns only values that are
+        still live at the end (the program's last result is)."""
         self.m, self.ops, self.capi = model, pkg.ops, pkg.capi
         self.fused_into = {}   # conv output name -> the Add instruction that absorbs it
+        program = model["program"]
         if fuse_residual:
-            program = model["program"]
             for i, ins in enumerate(program):
                 if ins[0] in ("AddRelu", "Add") and i > 0:
                     prev = program[i - 1]
@@ -298,41 +302,75 @@ class DeviceRunner(object):
         self.bufs = {}
         self.fusion = {}
         self.full = {}
+        self.reuse_buffers = reuse_buffers
         for name, c in model["convs"].items():
             t = [torch.from_numpy(a).cuda() for a in (c.wq, c.w_scale, c.w_zp, c.bias_q)]
             self.dev[name] = t
             self.plans[name] = self.ops.QLinearConvPlan(t[0], t[1], t[2], t[3], strides=(c.stride, c.stride),
                                                         pads=(c.pad, c.pad), group=c.group)
-        for ins in model["program"]:
-            out = ins[1]
+        # raw byte blocks: fresh per value, or from the pool of released ones (the smallest that fits)
+        free_blocks = []
+
+        def take(nbytes):
+            fits = [i for i, b in enumerate(free_blocks) if b.numel() >= nbytes]
+            if reuse_buffers and fits:
+                best = free_blocks.pop(min(fits, key=lambda i: free_blocks[i].numel()))
+                best[:nbytes].zero_()
+                return best
+            return torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        last_use = {}
+        for i, ins in enumerate(program):
+            for name in ins[2:4]:
+                if isinstance(name, str):
+                    last_use[name] = i
+        block_of = {}
+
+        def make(out, kind):
             shp = model["shapes"][out]
-            if ins[0] == "DequantizeLinear":
-                self.bufs[out] = torch.empty(shp, dtype=torch.float32, device="cuda")
-            elif ins[0] == "QuantizeLinear":
+            if kind == "DequantizeLinear":
+                n = int(np.prod(shp)) * 4
+                block_of[out] = take(n)
+                self.bufs[out] = block_of[out][:n].view(torch.float32).view(shp)
+            elif kind == "QuantizeLinear":
                 # the network input stays NCHW like the fp32 tensor it is quantized from (one flat,
                 # fully coalesced pass); the 3-channel stem reads it through its im2col step
-                self.bufs[out] = torch.empty(shp, dtype=torch.uint8, device="cuda")
+                n = int(np.prod(shp))
+                block_of[out] = take(n)
+                self.bufs[out] = block_of[out][:n].view(shp)
             else:
                 # channels-last with the pixel pitch rounded up to 16 bytes, so that every pixel is a
                 # whole number of aligned 16-byte vectors also for channel counts like 24
                 n, c, h, w = shp
                 pitch = (c + 15) // 16 * 16
-                full = torch.zeros((n, h, w, pitch), dtype=torch.uint8, device="cuda")
+                block_of[out] = take(n * h * w * pitch)
+                full = block_of[out][:n * h * w * pitch].view(n, h, w, pitch)
                 self.bufs[out] = full[..., :c].permute(0, 3, 1, 2)
                 # element-wise groups run over the padded pixels as they lie in memory (dense)
                 self.full[out] = full.permute(0, 3, 1, 2)
+        for i, ins in enumerate(program):
+            kind, out = ins[0], ins[1]
+            if kind == "QLinearConv" and out in self.fused_into:
+                add = self.fused_into[out]
+                make(add[1], add[0])     # the fused convolution writes the sum here, one instruction early
+            elif out not in self.bufs:
+                make(out, kind)
             q = model["qparams"]
-            if ins[0] == "AddRelu":
+            if kind == "AddRelu":
                 self.fusion[out] = add_relu_program(self.ops, q[ins[2]], q[ins[3]], q[out])
-            if ins[0] == "Add":
+            if kind == "Add":
                 self.fusion[out] = add_program(self.ops, q[ins[2]], q[ins[3]], q[out])
+            if reuse_buffers:
+                for name in set(n for n in ins[2:4] if isinstance(n, str)):
+                    if last_use.get(name) == i and name in block_of:
+                        free_blocks.append(block_of.pop(name))
+        self.live_at_end = set(block_of)
 
     def launch(self, fid, v):
         """Launches instruction number `fid` of the program on the values `v` (name -> tensor)."""
         ops, q, m = self.ops, self.m["qparams"], self.m
         ins = m["program"][fid]
         kind, out = ins[0], ins[1]
-        buf = self.bufs[out]
+        buf = self.bufs.get(out)   # none for a convolution whose result only exists inside the fused residual sum
         if kind == "QuantizeLinear":
             ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
         elif kind == "QLinearConv" and out in self.fused_into:
@@ -370,6 +408,8 @@ class DeviceRunner(object):
             buf = self.launch(fid, v)
             if buf is not None:
                 v[ins[1]] = buf
+        if self.reuse_buffers:
+            return {k: t for k, t in v.items() if k == "x" or k in self.live_at_end}
         return v
 
     def capture(self, x):

@@ -118,6 +118,23 @@ int chx_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream); 
 int chx_hip_memset(void* dst, int value, size_t bytes, void* stream);
 int chx_hip_stream_synchronize(void* stream);
 
+/* Streams and captured graphs, for hosts that replay a fixed instruction sequence (the ChxVM runtime
+ * mirror captures one run of a program and replays it; nothing in the reference corresponds: its
+ * interpreter launches every kernel from the host on the default stream, runtime/chxvm.cc:168-236).
+ * A stream from chx_hip_stream_create has the default priority and does not synchronize with the
+ * null stream.  Between capture_begin and capture_end the calls of this library on that stream are
+ * recorded instead of run; calls that must synchronize, allocate with the device runtime or time
+ * kernels are refused by the device runtime, capture_end then fails and leaves no graph. */
+int chx_hip_stream_create(void** stream);
+int chx_hip_stream_destroy(void* stream);
+typedef struct chx_hip_graph chx_hip_graph;
+int chx_hip_capture_begin(void* stream);
+int chx_hip_capture_end(void* stream, chx_hip_graph** graph);
+/* 1 while `stream` records (a null stream never does) */
+int chx_hip_stream_is_capturing(void* stream);
+int chx_hip_graph_launch(const chx_hip_graph* graph, void* stream);
+void chx_hip_graph_destroy(chx_hip_graph* graph);
+
 /* ---- QuantizeLinear / DequantizeLinear ------------------------------------------------ */
 
 /* QuantizeLinearOp::RunImpl -> quantize_array, runtime/ops/quantize.cc:16-35,48-53.
@@ -164,12 +181,19 @@ int chx_hip_qconv_plan_create(
 int chx_hip_qconv_plan_run(
         const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
         int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
+/* The launch configurations the plan has measured so far, as text into buf (truncated to buf_size - 1
+ * characters): one "M=<output pixels> <OH>x<OW> res=<0|1> tile=<oc>x<px> wgs_per_cu=<n, 0 = as many as fit>"
+ * per line; empty for a plan that does not run on the matrix-core kernel or has not run eagerly yet.  No
+ * counterpart in the reference; benchmarks report it next to their timings. */
+int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_t buf_size);
 /* A QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94) whose only reader is the
  * element-wise group  QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r)))  of a
  * residual block (ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161, act = Relu or
  * nothing), run as one kernel: the convolution's 8-bit result y (type y_dtype, quantization
  * y_scale / y_zero_point) is never written, `out` receives the group's result, computed operation
  * by operation as the two ops would.  r and out: same shape as y, channels-last, uint8 or int8.
+ * `out` must not overlap x or r in memory (the first call on a new shape may run the kernel several
+ * times on the call's operands to pick a launch configuration): CHX_HIP_EINVAL when it does.
  * CHX_HIP_EUNSUPPORTED when the plan's weights or the layouts do not fit the matrix-core kernel;
  * the caller then runs the two ops separately. */
 int chx_hip_qconv_plan_run_add(

@@ -405,3 +405,221 @@ def test_max_pool_on_codes_is_for_uint8_only(g, vm, oracle):
     with pytest.raises(vm.ChxVMError, match="int8"):
         prog = vm.Program(pool_program(-3, "int8"))
         prog.run({"x": g.dev(xi)})
+
+
+def _conv_program(vm, shape, w, ws, wz, bias, xq, yq, weights_as_inputs=False):
+    """QuantizeLinear -> QLinearConv -> Out; the four weight-side operands constants or program inputs."""
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", shape)
+    s_x, z_x = b.scalar(float(xq[0]), "float32"), b.scalar(int(xq[1]), "uint8")
+    q = b.QuantizeLinear(x, s_x, z_x)
+    if weights_as_inputs:
+        ops = [b.input("w", "int8", w.shape), b.input("w_scale", "float32", ws.shape), b.input("w_zero_point", "int8", wz.shape),
+               b.input("bias", "int32", bias.shape)]
+    else:
+        ops = [b.constant(w), b.constant(ws), b.constant(wz), b.constant(bias)]
+    y = b.QLinearConv(q, s_x, z_x, ops[0], ops[1], ops[2], b.scalar(float(yq[0]), "float32"), b.scalar(int(yq[1]), "uint8"), ops[3],
+                      [1, 1], [1, 1], 1, "")
+    b.Free(q)
+    b.output("y", y)
+    return vm.Program(b.serialize())
+
+
+def test_two_programs_keep_their_own_bias_mode(g, vm, oracle):
+    """The bias mode of a QLinearConv is an option of the run, not of the process: two programs with
+    different settings, run alternately, each give the result of their own mode."""
+    rng = np.random.default_rng(21)
+    N, C, H, W, OC = 2, 32, 8, 9, 64
+    w = rng.integers(-127, 128, size=(OC, C, 3, 3)).astype(np.int8)
+    ws = rng.uniform(0.001, 0.01, size=OC).astype(np.float32)
+    wz = np.zeros(OC, np.int8)
+    bias = rng.integers(-3000, 3000, size=OC).astype(np.int32)
+    xq, yq = (np.float32(0.02), 128), (np.float32(0.2), 100)
+    p_ref = _conv_program(vm, (N, C, H, W), w, ws, wz, bias, xq, yq)
+    p_onnx = _conv_program(vm, (N, C, H, W), w, ws, wz, bias, xq, yq)
+    p_onnx.set_option("qlinearconv_bias", "onnx_int32")
+    p_ref.set_option("qlinearconv_bias", "reference")
+    xv = rng.uniform(-2.5, 2.5, size=(N, C, H, W)).astype(np.float32)
+    qx = oracle.quantize_linear(xv, xq[0], xq[1], np.uint8)
+    want = {mode: oracle.qlinear_conv_int(qx, xq[0], xq[1], w, ws, wz, yq[0], yq[1], np.uint8, bias=bias, bias_mode=mode,
+                                          strides=(1, 1), pads=(1, 1)) for mode in (oracle.BIAS_REFERENCE_FLOAT, oracle.BIAS_ONNX_INT32)}
+    assert (want[oracle.BIAS_REFERENCE_FLOAT] != want[oracle.BIAS_ONNX_INT32]).any()
+    for _ in range(2):
+        np.testing.assert_array_equal(p_ref.run({"x": g.dev(xv)})["y"], want[oracle.BIAS_REFERENCE_FLOAT])
+        np.testing.assert_array_equal(p_onnx.run({"x": g.dev(xv)})["y"], want[oracle.BIAS_ONNX_INT32])
+    # "default" follows the process-wide switch again
+    p_onnx.set_option("qlinearconv_bias", "default")
+    np.testing.assert_array_equal(p_onnx.run({"x": g.dev(xv)})["y"], want[oracle.BIAS_REFERENCE_FLOAT])
+    with pytest.raises(vm.ChxVMError, match="unknown program option"):
+        p_ref.set_option("no_such_option", "on")
+
+
+def test_weights_that_are_program_inputs_are_read_on_every_run(g, vm, oracle):
+    """Weight-side operands that come from the caller get no cached plan: a second run with other weights at
+    the same device addresses (rewritten in place) computes with the new ones."""
+    rng = np.random.default_rng(22)
+    N, C, H, W, OC = 1, 64, 7, 7, 64
+    xq, yq = (np.float32(0.02), 128), (np.float32(0.15), 128)
+    xv = rng.uniform(-2.5, 2.5, size=(N, C, H, W)).astype(np.float32)
+    qx = oracle.quantize_linear(xv, xq[0], xq[1], np.uint8)
+    shapes = ((OC, C, 3, 3), (OC,), (OC,), (OC,))
+    prog = _conv_program(vm, (N, C, H, W), np.zeros(shapes[0], np.int8), np.zeros(OC, np.float32), np.zeros(OC, np.int8),
+                         np.zeros(OC, np.int32), xq, yq, weights_as_inputs=True)
+    dev = {"w": torch.zeros(shapes[0], dtype=torch.int8, device="cuda"), "w_scale": torch.zeros(OC, dtype=torch.float32, device="cuda"),
+           "w_zero_point": torch.zeros(OC, dtype=torch.int8, device="cuda"), "bias": torch.zeros(OC, dtype=torch.int32, device="cuda")}
+    seen = []
+    for seed in (1, 2, 3):
+        r = np.random.default_rng(seed)
+        w = r.integers(-127, 128, size=shapes[0]).astype(np.int8)
+        ws = r.uniform(0.001, 0.01, size=OC).astype(np.float32)
+        bias = r.integers(-5, 6, size=OC).astype(np.int32)
+        dev["w"].copy_(torch.from_numpy(w))           # the same device memory, new contents
+        dev["w_scale"].copy_(torch.from_numpy(ws))
+        dev["bias"].copy_(torch.from_numpy(bias))
+        torch.cuda.synchronize()
+        got = prog.run(dict(dev, x=g.dev(xv)))["y"]
+        want = oracle.qlinear_conv_int(qx, xq[0], xq[1], w, ws, np.zeros(OC, np.int8), yq[0], yq[1], np.uint8, bias=bias,
+                                       bias_mode=oracle.BIAS_REFERENCE_FLOAT, strides=(1, 1), pads=(1, 1))
+        np.testing.assert_array_equal(got, want)
+        seen.append(got)
+    assert (seen[0] != seen[1]).any() and (seen[1] != seen[2]).any()
+
+
+def test_type_checks_and_dumps_of_a_program_with_fused_instructions(g, vm, oracle, tmp_path):
+    """A compiled network: pools (two outputs, the second the dropped context), QLinearConv with the residual
+    group behind it computed inside, DequantizeLinear absorbed into pools.  With the run-time type check on
+    and every named output dumped, the instructions that were fused away (their named outputs stay unset)
+    are skipped, everything else is checked and written."""
+    from importlib import import_module
+    onnx_lite = import_module(g.pkg.__name__ + ".onnx_lite")
+    wl = g.pkg.workloads
+    model = wl.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(1, 1, 1, 1), classes=10)
+    data = vm.compile_onnx(wl.program_to_onnx(model, onnx_lite), {"fuse": "hip"})
+    prog = vm.Program(data)
+    prog.set_option("qlinearconv_bias", "onnx_int32")
+    before = prog.counter("qlinearconv_residual_fusions")
+    vm.set_option("check_types", "on")
+    vm.set_option("dump_outputs_dir", str(tmp_path))
+    try:
+        got = prog.run({"x": torch.from_numpy(model["input"]).cuda()})["logits"]
+    finally:
+        vm.set_option("check_types", "off")
+        vm.set_option("dump_outputs_dir", "")
+    assert prog.counter("qlinearconv_residual_fusions") - before == 4
+    oracle.set_threads(16)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"], keep={"logits"})
+    finally:
+        oracle.set_threads(1)
+    np.testing.assert_array_equal(got, ref["logits"])
+    dumped = sorted(p.name for p in tmp_path.iterdir())
+    assert len(dumped) > 10 and any(name.endswith("logits.npy") for name in dumped)
+    last = [p for p in tmp_path.iterdir() if p.name.endswith("logits.npy")][0]
+    np.testing.assert_array_equal(np.load(last), ref["logits"])
+
+
+def test_recorded_run_replays_with_new_inputs(g, vm, oracle):
+    """A program recorded into a device graph: every replay (with eager work and synchronizations of the
+    program's own in between) gives the oracle's values for what the input buffer holds at that time."""
+    wl = g.pkg.workloads
+    for model in (wl.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10),
+                  wl.build_mobilenetv2(batch=2, image=64, seed=7, blocks=((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 1, 2)), stem=32,
+                                       head=128, classes=10)):
+        keep = ["logits"] + [ins[1] for ins in model["program"] if ins[0] in ("AddRelu", "Add")]
+        prog = vm.Program(wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize())
+        prog.set_option("qlinearconv_bias", "onnx_int32")
+        x = torch.from_numpy(model["input"]).cuda()
+        replay = prog.capture({"x": x})
+        assert replay.info("warm_runs") >= 2 and replay.info("pool_bytes") > 0
+        rng = np.random.default_rng(9)
+        oracle.set_threads(16)
+        try:
+            for i in range(4):
+                xv = model["input"] if i == 0 else (model["input"] * np.float32(0.5 + 0.25 * i) +
+                                                    rng.standard_normal(model["input"].shape).astype(np.float32) * np.float32(0.3))
+                x.copy_(torch.from_numpy(xv))
+                torch.cuda.synchronize()
+                replay.launch()
+                replay.synchronize()
+                got = replay.outputs()
+                ref = wl.run_reference(model, oracle, xv, keep=set(keep))
+                for name in keep:
+                    np.testing.assert_array_equal(got[name], ref[name], err_msg="replay %d value %s" % (i, name))
+                # eager work of the same program between the replays (its plans and kernels are shared)
+                eager = prog.run({"x": x})
+                np.testing.assert_array_equal(eager["logits"], ref["logits"])
+        finally:
+            oracle.set_threads(1)
+        # launched on the caller's stream as well
+        replay.launch(g.capi.stream_ptr())
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(replay.outputs()["logits"], ref["logits"])
+        replay.close()
+        prog.close()
+
+
+def test_a_program_that_reads_results_back_cannot_be_recorded(g, vm):
+    """A dynamically quantized graph computes its scales on the device and reads them back as scalars: the
+    capture fails with the reason, and the program still runs eagerly afterwards."""
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", (4, 64))
+    lo = b.ReduceMin(x, [], 0)
+    s = b.new_slot()
+    b.add_raw("Identity", [("ARRAY", lo)], [s])
+    q = b.QuantizeLinear(x, b.scalar(0.05, "float32"), b.scalar(3, "uint8"))
+    b.output("q", q)
+    b.output("lo", lo)
+    prog = vm.Program(b.serialize())
+    xv = np.random.default_rng(3).standard_normal((4, 64)).astype(np.float32)
+    xd = g.dev(xv)
+    try:
+        replay = prog.capture({"x": xd})
+    except vm.ChxVMError as e:
+        assert "capture" in str(e) or "captur" in str(e) or "graph" in str(e)
+    else:
+        # the reduction itself needs no read-back in this build: then the replay must be right
+        replay.launch()
+        replay.synchronize()
+        assert np.float32(replay.outputs()["lo"]) == xv.min()
+        replay.close()
+    out = prog.run({"x": xd})
+    assert np.float32(out["lo"]) == xv.min()
+
+
+@pytest.mark.parametrize("net,batch,seed", [("resnet50", 64, 3), ("mobilenetv2", 128, 4)])
+def test_benchmark_networks_at_full_size_through_the_vm(g, vm, oracle, net, batch, seed):
+    """What bench.py times by default: the whole network at its benchmark batch as one serialized program in the
+    C++ VM, its run recorded and replayed.  Three images of the batch are compared with the oracle on the
+    logits and on every block output; all images through the property that needs no oracle (every op of the
+    path is independent per image, so a permuted batch gives the permuted results)."""
+    wl = g.pkg.workloads
+    model = (wl.build_resnet50 if net == "resnet50" else wl.build_mobilenetv2)(batch=batch, seed=seed)
+    keep = ["logits"] + [ins[1] for ins in model["program"] if ins[0] in ("AddRelu", "Add")]
+    prog = vm.Program(wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize())
+    prog.set_option("qlinearconv_bias", "onnx_int32")
+    x = torch.from_numpy(model["input"]).cuda()
+    replay = prog.capture({"x": x})
+    fused = prog.counter("qlinearconv_residual_fusions")
+    assert fused >= len(keep) - 1          # every residual sum was computed inside its convolution, in every run
+    replay.launch()
+    replay.synchronize()
+    out = replay.outputs()
+    picks = [0, batch // 2 + 5, batch - 1]
+    oracle.set_threads(16)
+    try:
+        ref = wl.run_reference(model, oracle, model["input"][picks], keep=set(keep))
+    finally:
+        oracle.set_threads(1)
+    for name in keep:
+        np.testing.assert_array_equal(out[name][picks], ref[name], err_msg=name)
+    assert out["logits"].min() < out["logits"].max()
+    perm = torch.randperm(batch, generator=torch.Generator().manual_seed(seed))
+    x.copy_(x[perm.cuda()])
+    torch.cuda.synchronize()
+    replay.launch(g.capi.stream_ptr())
+    torch.cuda.synchronize()
+    again = replay.outputs()
+    for name in keep:
+        np.testing.assert_array_equal(again[name], out[name][perm.numpy()], err_msg=name)
+    replay.close()
+    prog.close()

@@ -416,6 +416,12 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
         plan.run_add(xd, 0.02, 101, ys, yz, g.dev(r), rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt],
                      flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros(conv.shape, dtype=TDT[odt], device="cuda"))
     assert e.value.code == g.capi.EUNSUPPORTED
+    # the sum written over its own residual operand (same type) is refused: the kernel may run more than once
+    if rdt == odt:
+        rd = g.to_channels_last(g.dev(r))
+        with pytest.raises(g.capi.ChxHipError) as e:
+            plan.run_add(xd, 0.02, 101, ys, yz, rd, rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt], flags=g.capi.BIAS_ONNX_INT32, out=rd)
+        assert e.value.code == g.capi.EINVAL and "overlaps" in str(e.value)
     plan.close()
 
 
