@@ -4,6 +4,7 @@
 // conversions (Cast: int32 -> float32 for the scale-back, float32 -> uint8 / int8 for a computed
 // zero point).  Both take any strides; neither is on the timed path of a statically quantized
 // network.
+#include <mutex>
 #include <vector>
 
 #include "chx_internal.h"
@@ -12,6 +13,32 @@ namespace chx {
 namespace {
 
 constexpr int kThreads = 256;
+
+// Partial results of chx_hip_reduce_min_max_noalloc: one per work-group.  Every GPU the library runs on
+// holds its own copy of this array, at its own address, until the process ends.
+constexpr int kNoAllocBlocks = 1024;
+constexpr int64_t kNoAllocMaxElements = int64_t(1) << 30;
+static __device__ __align__(256) float scratch[kNoAllocBlocks];
+
+// Device address of `scratch` on the current device.  The name of the array is a host-side stand-in, not
+// an address a kernel could use: the address is asked for once per device, with that device current.
+int noalloc_scratch(float** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static float* ptrs[kMaxDevices] = {};
+    int dev = 0;
+    CHX_HIP_CALL(hipGetDevice(&dev));
+    CHX_REQUIRE(dev >= 0 && dev < kMaxDevices, "device %d: more devices than this entry point keeps scratch addresses for", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        CHX_HIP_CALL(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        CHX_REQUIRE(p != nullptr, "hipGetSymbolAddress gave a null address for the scratch array");
+        ptrs[dev] = static_cast<float*>(p);
+    }
+    *out = ptrs[dev];
+    return CHX_HIP_OK;
+}
 
 __device__ __forceinline__ int64_t strided_offset(int64_t flat, const StridedDesc& d) {
     int64_t off = 0;
@@ -140,6 +167,34 @@ extern "C" int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, c
     const int rc = launch_check("reduce_min_max");
     scratch_free(partial, s);
     return rc;
+}
+
+extern "C" int chx_hip_reduce_min_max_noalloc(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "ReduceMin/ReduceMax x"));
+    CHX_PROPAGATE(check_tensor(y, "ReduceMin/ReduceMax y"));
+    CHX_REQUIRE(x->dtype == CHX_HIP_FLOAT32 && y->dtype == CHX_HIP_FLOAT32, "ReduceMin/ReduceMax: float32 only");
+    CHX_REQUIRE(numel(*y) == 1, "ReduceMin/ReduceMax: y must hold one element (all axes reduced)");
+    const int64_t n = numel(*x);
+    CHX_REQUIRE(n > 0, "ReduceMin/ReduceMax of an empty tensor");
+    CHX_REQUIRE(n <= kNoAllocMaxElements,
+                "ReduceMin/ReduceMax without allocation: %lld elements, at most %lld (use chx_hip_reduce_min_max for more)", (long long)n,
+                (long long)kNoAllocMaxElements);
+    float* partial = nullptr;
+    CHX_PROPAGATE(noalloc_scratch(&partial));
+    hipStream_t s = as_stream(stream);
+    int blocks = (int)((n + kThreads * 8 - 1) / (kThreads * 8));
+    blocks = blocks < 1 ? 1 : blocks > kNoAllocBlocks ? kNoAllocBlocks : blocks;
+    const StridedDesc xd = make_desc(*x);
+    // every work-group writes its own partial result and the second kernel reads exactly those: nothing of
+    // what an earlier call left in the array is looked at, so nothing has to be cleared
+    if (is_max) {
+        reduce_partial_kernel<true><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, partial);
+        reduce_final_kernel<true><<<1, kThreads, 0, s>>>(partial, blocks, static_cast<float*>(y->data));
+    } else {
+        reduce_partial_kernel<false><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x->data), xd, n, partial);
+        reduce_final_kernel<false><<<1, kThreads, 0, s>>>(partial, blocks, static_cast<float*>(y->data));
+    }
+    return launch_check("reduce_min_max (no allocation)");
 }
 
 extern "C" int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream) {

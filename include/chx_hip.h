@@ -277,6 +277,14 @@ int chx_hip_elementwise_source(
  * the quantizer emits (compiler/quantize.cc:171-174): every axis reduced, keepdims = 0.  x float32,
  * any strides; y float32 with one element. */
 int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream);
+/* The same reduction for callers that cannot allocate device memory (code under graph capture, serving
+ * loops, harnesses that forbid it); it has no counterpart in the reference.  chx_hip_reduce_min_max takes its
+ * per-work-group partial results from the stream-ordered allocator; this one keeps them in a 4 KiB array in
+ * the library's device image (every GPU the library runs on holds its own copy until the process ends) and
+ * calls no allocation routine.  At most 2^30 elements: CHX_HIP_EINVAL beyond.  Calls that overlap on one GPU
+ * (two streams, two threads) share the array and race: keep them in one stream's order.  Results are
+ * identical to chx_hip_reduce_min_max's. */
+int chx_hip_reduce_min_max_noalloc(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream);
 
 /* The scan behind ChxVMState::CheckNans / CheckInfs (runtime/chxvm_state.cc:215-263: chainerx::IsNan / IsInf,
  * Sum, AsScalar): *count receives the number of NaN elements of x (infinities = 0) or of +-Inf elements
