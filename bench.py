@@ -209,14 +209,14 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
             roofline["traffic_source"] = "profiles/resnet50_bs64_conv_mfma_traffic.json (%s)" % t.get("measured_at", "separate rocprofv3 --pmc runs")
         except (OSError, ValueError, KeyError):
             pass
-    # the launch configurations the plans measured for these launches: tile (output channels x pixels) and
-    # work-groups per compute unit -> number of layers
+    # the launch configurations the plans measured for these launches: tile (output channels x pixels),
+    # work-groups per compute unit (0 = as many as fit) and wavefronts per work-group -> number of layers
     hist = {}
     for rn, _xs in slices:
         for plan in rn.plans.values():
             for line in plan.describe():
                 f = dict(kv.split("=") for kv in line.split() if "=" in kv)
-                key = "%s/%s%s" % (f.get("tile"), f.get("wgs_per_cu"), "+res" if f.get("res") == "1" else "")
+                key = "%s/%s/w%s%s" % (f.get("tile"), f.get("wgs_per_cu"), f.get("waves", "4"), "+res" if f.get("res") == "1" else "")
                 hist[key] = hist.get(key, 0) + 1
     roofline["configs"] = hist
     res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),

@@ -211,16 +211,20 @@ bool weights_fit_mfma(const chx_hip_tensor& w, int group) {
 }
 
 // Tile shape: the largest tile that still gives every compute unit a work-group.
-void pick_tile(int OC, int64_t M, int* tile_oc, int* tile_px, int* max_wgs_per_cu) {
-    // CHX_HIP_TILE=<oc>,<px>[,<work-groups per compute unit>] forces a launch configuration (read on
-    // every call: a tuning aid, and how the tests reach every configuration the tuner may choose)
+void pick_tile(int OC, int64_t M, int bk, int* tile_oc, int* tile_px, int* max_wgs_per_cu, int* waves) {
+    // CHX_HIP_TILE=<oc>,<px>[,<work-groups per compute unit>[,<wavefronts: 4 or 8>]] forces a launch configuration
+    // (read on every call: a tuning aid, and how the tests reach every configuration the tuner may choose)
+    *waves = 4;
     if (const char* env = getenv("CHX_HIP_TILE")) {
-        int toc = 0, tpx = 0, cap = 0;
-        const int got = sscanf(env, "%d,%d,%d", &toc, &tpx, &cap);
-        if (got >= 2 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128) && cap >= 0) {
+        int toc = 0, tpx = 0, cap = 0, wv = 4;
+        const int got = sscanf(env, "%d,%d,%d,%d", &toc, &tpx, &cap, &wv);
+        const bool four = wv == 4 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128);
+        const bool eight = wv == 8 && ((toc == 128 && tpx == 128) || (bk == 128 && ((toc == 128 && tpx == 256) || (toc == 64 && tpx == 128))));
+        if (got >= 2 && (four || eight) && cap >= 0) {
             *tile_oc = toc;
             *tile_px = tpx;
-            *max_wgs_per_cu = got == 3 ? cap : 0;
+            *max_wgs_per_cu = got >= 3 ? cap : 0;
+            *waves = wv;
             return;
         }
     }
@@ -243,6 +247,7 @@ struct TunedConfig {
     int64_t M;
     int32_t H, W, OH, OW;
     int tile_oc, tile_px, max_wgs_per_cu;
+    int waves;      // wavefronts per work-group: 4 or 8
     bool with_res;  // measured with a fused residual sum (an entry of its own: the epilogue differs)
 };
 struct TuneCache {
@@ -265,22 +270,24 @@ bool stream_is_capturing(hipStream_t s) {
 
 // Times every launch configuration on the call's operands and keeps the fastest in *best.
 int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hipStream_t s, TunedConfig* best) {
-    static const int tiles[4][2] = {{128, 128}, {64, 128}, {128, 64}, {64, 64}};
+    // tile (output channels x pixels), wavefronts; the eight-wavefront kernels take the compute unit alone
+    static const int tiles[7][3] = {{128, 128, 4}, {64, 128, 4}, {128, 64, 4}, {64, 64, 4}, {128, 128, 8}, {128, 256, 8}, {64, 128, 8}};
     static const int caps[3] = {0, 2, 1};
     hipEvent_t e0, e1;
     CHX_HIP_CALL(hipEventCreate(&e0));
     CHX_HIP_CALL(hipEventCreate(&e1));
     float best_ms = -1.f;
     int rc = CHX_HIP_OK;
-    for (int t = 0; t < 4 && rc == CHX_HIP_OK; ++t) {
+    for (int t = 0; t < 7 && rc == CHX_HIP_OK; ++t) {
         if (a.OC <= 64 && tiles[t][0] > 64) continue;
-        for (int c = 0; c < 3 && rc == CHX_HIP_OK; ++c) {
+        if (tiles[t][2] == 8 && (tiles[t][0] == 64 || tiles[t][1] == 256) && a.bk != 128) continue;
+        for (int c = 0; c < (tiles[t][2] == 8 ? 1 : 3) && rc == CHX_HIP_OK; ++c) {
             const int reps = 3;
-            rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], xu, out_int32, rne, s);  // warm
+            rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], tiles[t][2], xu, out_int32, rne, s);  // warm
             if (rc != CHX_HIP_OK) break;
             if (hipEventRecord(e0, s) != hipSuccess) rc = CHX_HIP_ERUNTIME;
             for (int r = 0; r < reps && rc == CHX_HIP_OK; ++r)
-                rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], xu, out_int32, rne, s);
+                rc = launch_conv_mfma(a, tiles[t][0], tiles[t][1], caps[c], tiles[t][2], xu, out_int32, rne, s);
             if (rc != CHX_HIP_OK) break;
             float ms = 0.f;
             if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
@@ -293,6 +300,7 @@ int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hip
                 best->tile_oc = tiles[t][0];
                 best->tile_px = tiles[t][1];
                 best->max_wgs_per_cu = caps[c];
+                best->waves = tiles[t][2];
             }
         }
     }
@@ -547,15 +555,15 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
     if (c.res) a.res = *c.res;
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
-    int toc = 64, tpx = 64, cap = 0;
-    pick_tile(cs.OC, a.M, &toc, &tpx, &cap);
+    int toc = 64, tpx = 64, cap = 0, waves = 4;
+    pick_tile(cs.OC, a.M, a.bk, &toc, &tpx, &cap, &waves);
     int rc = CHX_HIP_OK;
     const TunedConfig* tuned = nullptr;
     if (c.tune) {
         for (const TunedConfig& t : c.tune->entries)
             if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW && t.with_res == (c.res != nullptr)) tuned = &t;
         if (!tuned && autotune_enabled() && !stream_is_capturing(s)) {
-            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, c.res != nullptr};
+            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, 4, c.res != nullptr};
             rc = tune_conv_mfma(a, xu, c.out_int32, c.rne, s, &best);
             if (rc == CHX_HIP_OK) {
                 c.tune->entries.push_back(best);
@@ -567,8 +575,9 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
         toc = tuned->tile_oc;
         tpx = tuned->tile_px;
         cap = tuned->max_wgs_per_cu;
+        waves = tuned->waves;
     }
-    if (rc == CHX_HIP_OK) rc = launch_conv_mfma(a, toc, tpx, cap, xu, c.out_int32, c.rne, s);
+    if (rc == CHX_HIP_OK) rc = launch_conv_mfma(a, toc, tpx, cap, waves, xu, c.out_int32, c.rne, s);
     if (rc == CHX_HIP_OK && y_post) {
         rc = launch_nhwc_to_nchw_u8(static_cast<const char*>(y_scratch), static_cast<char*>(y.data), cs.N, cs.OC,
                                     (int64_t)cs.OH * cs.OW, (int)a.y_px_stride, s);
@@ -983,8 +992,8 @@ extern "C" int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char*
     std::string text;
     for (const TunedConfig& t : plan->tune.entries) {
         char line[160];
-        snprintf(line, sizeof(line), "M=%lld %dx%d res=%d tile=%dx%d wgs_per_cu=%d\n", (long long)t.M, t.OH, t.OW, t.with_res ? 1 : 0,
-                 t.tile_oc, t.tile_px, t.max_wgs_per_cu);
+        snprintf(line, sizeof(line), "M=%lld %dx%d res=%d tile=%dx%d wgs_per_cu=%d waves=%d\n", (long long)t.M, t.OH, t.OW, t.with_res ? 1 : 0,
+                 t.tile_oc, t.tile_px, t.max_wgs_per_cu, t.waves);
         text += line;
     }
     strncpy(buf, text.c_str(), buf_size - 1);

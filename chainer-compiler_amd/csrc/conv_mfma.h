@@ -117,8 +117,9 @@ bool stem_patch_fits(int C, int KH, int KW, int sh, int sw);
 int stem_k_blocks(int C, int KH, int KW);
 int pack_weights_stem(const chx_hip_tensor& w, int OCpad64, int8_t* wd, hipStream_t s);
 int launch_conv_stem(ConvStemArgs a, bool rne, hipStream_t s);
-// max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once)
-int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
+// max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once); waves: 4, or 8
+// for the tiles 128x128, 128x256 and 64x128 (output channels x pixels)
+int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, int waves, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s);
 
 // [N][C][HW] bytes -> [N][HW][pitch] bytes (lanes c >= C of a pixel are zero filled) and back

@@ -280,8 +280,8 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 #ifndef CHX_CONV_NS_MAX
 #define CHX_CONV_NS_MAX 3
 #endif
-constexpr int ring_stages(int stage_bytes) {
-    const int fit = CHX_CONV_LDS_BUDGET / stage_bytes;
+constexpr int ring_stages(int stage_bytes, int lds_budget) {
+    const int fit = lds_budget / stage_bytes;
     return fit < 2 ? 2 : fit > CHX_CONV_NS_MAX ? CHX_CONV_NS_MAX : fit;
 }
 
@@ -309,17 +309,27 @@ constexpr int ring_stages(int stage_bytes) {
 // tile) and an invalid chunk is fetched from a 64-byte row holding the zero point instead
 // (g_fill_rows), which makes it contribute (zp - zp) * w = 0.  Without kPad (1x1 and other
 // unpadded convolutions on 64-multiple channels, matrix products) every chunk is valid.
-template <int FM, int FN, int BK, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad, bool kRes>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv_mfma_kernel(ConvMfmaArgs a) {
-    constexpr int T = 256;
-    constexpr int TM = 64 * FM;  // output channels per tile
-    constexpr int TN = 64 * FN;  // pixels per tile
+//
+// NWN: wavefronts along the pixel axis (two along the output channels).  2: four wavefronts, two
+// work-groups per compute unit as a rule.  4: eight wavefronts on the same tile, each with half the
+// pixels; a work-group then has the compute unit to itself (and the whole LDS for a deeper ring).  The
+// K loop of a wavefront is bound by the instructions it has to issue (fragment reads, sign flips,
+// copy addresses: about 200 for 16 MFMAs with four wavefronts on a 128x128 tile), so when a layer has
+// no second work-group to put on the compute unit, twice the wavefronts on the same tile halve what
+// each has to issue and the two of a SIMD fill each other's gaps.
+template <int FM, int FN, int BK, bool kXUnsigned, bool kOutInt32, bool kRne, bool kPad, bool kRes, int NWN = 2>
+__global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) void conv_mfma_kernel(ConvMfmaArgs a) {
+    constexpr int NW = 2 * NWN;  // wavefronts
+    constexpr int T = 64 * NW;
+    constexpr int TM = 64 * FM;        // output channels per tile
+    constexpr int TN = 32 * NWN * FN;  // pixels per tile
     constexpr int STAGE_BYTES = (TM + TN) * BK;
-    constexpr int NS = ring_stages(STAGE_BYTES);
+    constexpr int NS = ring_stages(STAGE_BYTES, NWN == 2 ? CHX_CONV_LDS_BUDGET : 2 * CHX_CONV_LDS_BUDGET - 8 * 1024);
     constexpr int CH = BK / 16;          // 16-byte chunks per staged row
     constexpr int RPI = 64 / CH;         // rows one copy instruction fills
-    constexpr int CA = TM / RPI / 4;     // copy instructions per wave and stage, weight rows
-    constexpr int CB = TN / RPI / 4;     //   ... pixel rows
+    constexpr int CA = TM / RPI / NW;    // copy instructions per wave and stage, weight rows
+    constexpr int CB = TN / RPI / NW;    //   ... pixel rows
+    static_assert(CA >= 1 && CB >= 1 && CA * RPI * NW == TM && CB * RPI * NW == TN, "every wavefront copies whole instructions of both operands");
     constexpr int COPIES = CA + CB;
     constexpr int OUT_CHUNKS = TM / 16;  // 16-byte chunks per staged output row
     static_assert(TN * TM <= STAGE_BYTES, "the output tile is staged in one ring slot");
@@ -332,7 +342,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / NWN, wn = wave % NWN;
 
     // Work-group ids go round-robin over the 8 XCDs, each with its own L2.  Every XCD gets one
     // contiguous range of pixel tiles (neighbouring tiles share halo rows) and runs all
@@ -359,7 +369,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     const int kc = BK == 64 ? (lane & 3) ^ ((lane >> 4) & 3) : (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
     const int8_t* wp_row[CA];
 #pragma unroll
-    for (int j = 0; j < CA; ++j) wp_row[j] = a.wp + packed_offset(oc0 + row0 + 4 * RPI * j, kc * 16, a.KP, BK);
+    for (int j = 0; j < CA; ++j) wp_row[j] = a.wp + packed_offset(oc0 + row0 + NW * RPI * j, kc * 16, a.KP, BK);
     const char* fill_src = reinterpret_cast<const char*>(g_fill_rows) + (a.x_zp & 0xff) * 64 + (kc & 3) * 16;
     const uint32_t ring_base = (uint32_t)(uintptr_t)ring;             // LDS byte address
     const uint32_t ring_addr = ring_base + (uint32_t)wave * 1024u;
@@ -377,7 +387,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         const int64_t mbase = (int64_t)ld_tile * TN + row0;
 #pragma unroll
         for (int j = 0; j < CB; ++j) {
-            const int64_t m = mbase + 4 * RPI * j;
+            const int64_t m = mbase + NW * RPI * j;
             const bool row_ok = m < a.M && ld_tile < px_hi;
             // rows past the end re-read the last pixel; they are never written back
             const uint32_t mm = m < a.M ? (uint32_t)m : (uint32_t)(a.M - 1);  // M fits 31 bits (checked on the host)
@@ -420,12 +430,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     auto issue_copy = [&](int buf, int q) {
         const uint32_t dst = ring_addr + (uint32_t)buf * STAGE_BYTES;
         if (q < CA) {
-            async_copy16(wp_row[q] + kofs, dst + q * 4096);
+            async_copy16(wp_row[q] + kofs, dst + q * (NW * 1024));
         } else {
             const int j = q - CA;
             bool ok = true;
             if (kPad) ok = c0 + kc * 16 < a.C16 && ((tapmask[j] >> tap) & 1u);
-            async_copy16(ok ? xb[j] + tap_off + c0 : fill_src, dst + TM * BK + j * 4096);
+            async_copy16(ok ? xb[j] + tap_off + c0 : fill_src, dst + TM * BK + j * (NW * 1024));
         }
     };
     // advance to the next K step, or to the first K step of this work-group's next pixel tile
@@ -731,7 +741,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     wait_vmcnt<0>();  // the copies past the end still target this work-group's LDS
 }
 
-template <int FM, int FN, int BK>
+template <int FM, int FN, int BK, int NWN = 2>
 int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool rne, int max_wgs_per_cu, hipStream_t s) {
     // persistent work-groups: as many as the device holds at once, a whole number per
     // output-channel tile
@@ -744,7 +754,7 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
         }
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, BK, true, false, false, true, false>), 256, 0) !=
+                    &per_cu, reinterpret_cast<const void*>(&conv_mfma_kernel<FM, FN, BK, true, false, false, true, false, NWN>), 128 * NWN, 0) !=
                     hipSuccess ||
             per_cu < 1)
             per_cu = 2;
@@ -760,9 +770,9 @@ int launch_config(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool r
 #define CHX_LAUNCH_R(XU, OI, RN, RS)                                                       \
     do {                                                                                   \
         if (pad)                                                                           \
-            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, true, RS><<<grid, 256, 0, s>>>(a);    \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, true, RS, NWN><<<grid, 128 * NWN, 0, s>>>(a);    \
         else                                                                               \
-            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, false, RS><<<grid, 256, 0, s>>>(a);   \
+            conv_mfma_kernel<FM, FN, BK, XU, OI, RN, false, RS, NWN><<<grid, 128 * NWN, 0, s>>>(a);   \
     } while (0)
 #define CHX_LAUNCH(XU, OI, RN) CHX_LAUNCH_R(XU, OI, RN, false)
     if (a.res.r) {
@@ -818,7 +828,7 @@ int launch_im2col_dense(const Im2colArgs& a, hipStream_t s) {
     return launch_check("im2col_dense_kernel");
 }
 
-int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, bool x_unsigned, bool out_int32, bool rne,
+int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, int waves, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s) {
     a.tiles_oc = (a.OC + tile_oc - 1) / tile_oc;
     a.tiles_px = (int)((a.M + tile_px - 1) / tile_px);
@@ -828,6 +838,15 @@ int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_c
     a.row_unit = 0;
     if (a.KH * a.KW <= 32)
         for (int i = 0; i < a.KH; ++i) a.row_unit |= 1u << (i * a.KW);
+    if (waves == 8) {
+        // eight wavefronts: the pixels of the tile are split four ways
+        if (tile_oc == 128 && tile_px == 128) return a.bk == 128 ? launch_config<2, 1, 128, 4>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
+                               : launch_config<2, 1, 64, 4>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+        if (tile_oc == 128 && tile_px == 256 && a.bk == 128) return launch_config<2, 2, 128, 4>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+        if (tile_oc == 64 && tile_px == 128 && a.bk == 128) return launch_config<1, 1, 128, 4>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
+        CHX_FAIL(CHX_HIP_EINVAL, "conv_mfma: no eight-wavefront kernel for a %dx%d tile with %d K bytes per step", tile_oc, tile_px, a.bk);
+    }
+    if (waves != 4) CHX_FAIL(CHX_HIP_EINVAL, "conv_mfma: work-groups have 4 or 8 wavefronts, not %d", waves);
     if (tile_oc == 128 && tile_px == 128) return a.bk == 128 ? launch_config<2, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)
                            : launch_config<2, 2, 64>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s);
     if (tile_oc == 64 && tile_px == 128) return a.bk == 128 ? launch_config<1, 2, 128>(a, x_unsigned, out_int32, rne, max_wgs_per_cu, s)

@@ -183,7 +183,7 @@ int chx_hip_qconv_plan_run(
         int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
 /* The launch configurations the plan has measured so far, as text into buf (truncated to buf_size - 1
  * characters): one "M=<output pixels> <OH>x<OW> res=<0|1> tile=<oc>x<px> wgs_per_cu=<n, 0 = as many as fit>"
- * per line; empty for a plan that does not run on the matrix-core kernel or has not run eagerly yet.  No
+ * per line (followed by "waves=<4|8>", the wavefronts per work-group); empty for a plan that does not run on the matrix-core kernel or has not run eagerly yet.  No
  * counterpart in the reference; benchmarks report it next to their timings. */
 int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_t buf_size);
 /* A QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94) whose only reader is the

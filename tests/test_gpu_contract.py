@@ -425,13 +425,14 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
     plan.close()
 
 
-@pytest.mark.parametrize("tile", [(128, 128), (64, 128), (128, 64), (64, 64)])
+@pytest.mark.parametrize("tile", [(128, 128, 4), (64, 128, 4), (128, 64, 4), (64, 64, 4), (128, 128, 8), (128, 256, 8), (64, 128, 8)])
 def test_every_launch_configuration_of_the_matrix_core_kernel(g, oracle, tile):
-    """The tuner picks one of 4 tile shapes x 3 occupancy caps per layer shape by timing, so a test
-    that leaves the choice to it covers one configuration per case.  CHX_HIP_TILE forces each in
-    turn: ragged pixel and channel tiles, 64- and 128-byte K steps, padded and padding-free taps,
-    channel counts that do not fill a K step, int32 results, the fused residual sum, work-groups
-    that walk over several pixel tiles."""
+    """The tuner picks one of 4 tile shapes x 3 occupancy caps with four wavefronts per work-group, or
+    one of 3 tile shapes with eight, per layer shape by timing, so a test that leaves the choice to it
+    covers one configuration per case.  CHX_HIP_TILE forces each in turn: ragged pixel and channel
+    tiles, 64- and 128-byte K steps (a configuration that exists for 128-byte steps only falls back to
+    the tuner's choice on the others), padded and padding-free taps, channel counts that do not fill a
+    K step, int32 results, the fused residual sum, work-groups that walk over several pixel tiles."""
     import os
     rng = np.random.default_rng(83)
 
@@ -458,8 +459,8 @@ def test_every_launch_configuration_of_the_matrix_core_kernel(g, oracle, tile):
     want_sum = _residual_sum(oracle, conv1, ys1, 119, r, np.float32(0.037), 131, True, np.float32(0.061), 99, np.uint8)
     before = os.environ.get("CHX_HIP_TILE")
     try:
-        for cap in (0, 2, 1):
-            os.environ["CHX_HIP_TILE"] = "%d,%d,%d" % (tile[0], tile[1], cap)
+        for cap in ((0, 2, 1) if tile[2] == 4 else (0,)):
+            os.environ["CHX_HIP_TILE"] = "%d,%d,%d,%d" % (tile[0], tile[1], cap, tile[2])
             for x, w, ws, bias, ys, kw, want in convs:
                 plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(np.zeros(len(ws), np.int8)), g.dev(bias), **kw)
                 got = plan.run(g.to_channels_last(g.dev(x)), 0.02, 101, ys, 119, torch.uint8, flags=g.capi.BIAS_ONNX_INT32)
