@@ -57,11 +57,11 @@ template <bool kU8, bool kGuard, bool kLean = false>
 __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p) {
     static_assert(kU8 || !kLean, "the lean variant is for uint8 results");
     v4i out;
+    float pre[16];
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
         const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
         int32_t code[4];
-        float pre[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float fa = ((float)((cw >> (8 * e)) & 0xffu) - p.c_zpf) * p.c_scale;
@@ -70,10 +70,17 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
             float sum = fa + fb;
             if (!kLean && p.relu) sum = __builtin_fmaxf(sum, 0.f);
             if (kGuard) sum = __builtin_amdgcn_fmed3f(sum, -p.big, p.big);
-            if (kU8) pre[e] = quantize_prefloor_u8<false, !kLean>(sum, p.out, p.inv_out_scale, 0.f);
+            if (kU8) pre[w * 4 + e] = quantize_prefloor_u8<false, !kLean>(sum, p.out, p.inv_out_scale, 0.f);
             else code[e] = quantize_value_folded<false>(sum, p.out, p.inv_out_scale, p.out.lo);
         }
-        out[w] = kU8 ? (int)floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : (int)pack4(code[0], code[1], code[2], code[3]);
+        if (!kU8) out[w] = (int)pack4(code[0], code[1], code[2], code[3]);
+    }
+    if (kU8) {
+        // all sixteen conversions under one switch of the rounding mode
+        uint32_t words[4];
+        floor_sat_u8x16(pre, words);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) out[w] = (int)words[w];
     }
     return out;
 }

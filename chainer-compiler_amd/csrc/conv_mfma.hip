@@ -549,20 +549,20 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         }
         // requantize: one instance of the element loop per bias mode and per conversion path (the
         // branches are uniform).  kPath 0: any 8-bit type and rounding; 1: uint8 in the reference's
-        // rounding through floor_sat_u8x4/8; 2: the same with a lower bound above 0 (a folded Relu);
+        // rounding through floor_sat_u8x16; 2: the same with a lower bound above 0 (a folded Relu);
         // 3: as 1 with a zero point of 0.
         auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
             constexpr int kPath = decltype(path_tag)::value;
+            if constexpr (kPath == 0) {
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+                for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
-                    const v4f sc = *reinterpret_cast<const v4f*>(&s_scale[ocl]);
-                    v4f fb = {0.f, 0.f, 0.f, 0.f};
-                    if (kFloatBias) fb = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
-                    if (kPath == 0) {
+                    for (int g = 0; g < 4; ++g) {
+                        const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
+                        const v4f sc = *reinterpret_cast<const v4f*>(&s_scale[ocl]);
+                        v4f fb = {0.f, 0.f, 0.f, 0.f};
+                        if (kFloatBias) fb = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
 #pragma unroll
                         for (int j = 0; j < FN; ++j) {
                             const int pxl = wn * 32 * FN + j * 32 + (lane & 31);
@@ -575,27 +575,43 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                             }
                             *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
                         }
-                    } else {
-                        float pre[FN * 4];
-#pragma unroll
-                        for (int j = 0; j < FN; ++j)
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                float v = (float)acc[i][j][g * 4 + e] * sc[e];
-                                if (kFloatBias) v = v + fb[e];
-                                pre[j * 4 + e] = quantize_prefloor_u8<kPath == 2, kPath != 3>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
-                            }
-                        uint32_t word[FN];
-                        if constexpr (FN == 2) {
-                            floor_sat_u8x8(pre, &word[0], &word[1]);
-                        } else {
-                            word[0] = floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]);
-                        }
-#pragma unroll
-                        for (int j = 0; j < FN; ++j)
-                            *reinterpret_cast<uint32_t*>(staged(lds_out, wn * 32 * FN + j * 32 + (lane & 31), ocl)) = word[j];
                     }
-                }
+            } else {
+                // sixteen values (4 / FN row groups of the accumulator) per switch of the rounding mode
+                constexpr int G = 4 / FN;
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int gb = 0; gb < 4; gb += G) {
+                        float pre[16];
+#pragma unroll
+                        for (int gl = 0; gl < G; ++gl) {
+                            const int g = gb + gl;
+                            const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
+                            const v4f sc = *reinterpret_cast<const v4f*>(&s_scale[ocl]);
+                            v4f fb = {0.f, 0.f, 0.f, 0.f};
+                            if (kFloatBias) fb = *reinterpret_cast<const v4f*>(&s_fbias[ocl]);
+#pragma unroll
+                            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    float v = (float)acc[i][j][g * 4 + e] * sc[e];
+                                    if (kFloatBias) v = v + fb[e];
+                                    pre[(gl * FN + j) * 4 + e] =
+                                            quantize_prefloor_u8<kPath == 2, kPath != 3>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                                }
+                        }
+                        uint32_t word[4];
+                        floor_sat_u8x16(pre, word);
+#pragma unroll
+                        for (int gl = 0; gl < G; ++gl) {
+                            const int ocl = wm * 32 * FM + i * 32 + (gb + gl) * 8 + (lane >> 5) * 4;
+#pragma unroll
+                            for (int j = 0; j < FN; ++j)
+                                *reinterpret_cast<uint32_t*>(staged(lds_out, wn * 32 * FN + j * 32 + (lane & 31), ocl)) = word[gl * FN + j];
+                        }
+                    }
+            }
         };
         // The residual chunks this thread will add are requested now: their latency runs under the
         // requantization instead of in front of every store.

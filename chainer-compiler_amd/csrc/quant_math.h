@@ -152,6 +152,38 @@ __device__ __forceinline__ void floor_sat_u8x8(const float (&x)[8], uint32_t* lo
     *hi = r1;
 }
 
+// Sixteen values under one switch of the rounding mode: word w holds x[4w .. 4w+3].
+__device__ __forceinline__ void floor_sat_u8x16(const float (&x)[16], uint32_t (&out)[4]) {
+    uint32_t r0, r1, r2, r3;
+    asm volatile(
+            "s_nop 1\n\t"
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2\n\t"
+            "v_cvt_pk_u8_f32 %0, %4, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %1, %8, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %2, %12, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %3, %16, 0, 0\n\t"
+            "v_cvt_pk_u8_f32 %0, %5, 1, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %9, 1, %1\n\t"
+            "v_cvt_pk_u8_f32 %2, %13, 1, %2\n\t"
+            "v_cvt_pk_u8_f32 %3, %17, 1, %3\n\t"
+            "v_cvt_pk_u8_f32 %0, %6, 2, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %10, 2, %1\n\t"
+            "v_cvt_pk_u8_f32 %2, %14, 2, %2\n\t"
+            "v_cvt_pk_u8_f32 %3, %18, 2, %3\n\t"
+            "v_cvt_pk_u8_f32 %0, %7, 3, %0\n\t"
+            "v_cvt_pk_u8_f32 %1, %11, 3, %1\n\t"
+            "v_cvt_pk_u8_f32 %2, %15, 3, %2\n\t"
+            "v_cvt_pk_u8_f32 %3, %19, 3, %3\n\t"
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0"
+            : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+            : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]), "v"(x[8]), "v"(x[9]), "v"(x[10]),
+              "v"(x[11]), "v"(x[12]), "v"(x[13]), "v"(x[14]), "v"(x[15]));
+    out[0] = r0;
+    out[1] = r1;
+    out[2] = r2;
+    out[3] = r3;
+}
+
 // The value handed to floor_sat_u8x4/8 for one element: quantize_value_folded up to and including
 // the + 0.5f, with only the lower bound applied (and only when it is above 0).
 // kZeroPoint = false is for a zero point of 0: adding 0.0f changes no value (-0 becomes +0, which the
