@@ -336,6 +336,15 @@ private:
             simple(op, {ArrayListIn(ins)});
         } else if ((op == "ReduceMax" || op == "ReduceMin") && nin == 1) {
             simple(op, {ArrayIn(Operand(n, 0)), IntsIn(n.GetInts("axes")), IntIn(n.GetInt("keepdims", 1))});
+        } else if (op == "MatMul" && nin == 2) {
+            simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1))});
+        } else if (op == "Gemm" && (nin == 2 || nin == 3)) {
+            // compiler/chxvm/simple_node_emitter.cc:316-318; attribute defaults of compiler/gen_node.py
+            simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true)), FloatIn(n.GetFloat("alpha", 1.f)),
+                        FloatIn(n.GetFloat("beta", 1.f)), IntIn(n.GetInt("transA", 0)), IntIn(n.GetInt("transB", 0))});
+        } else if (op == "Flatten" && nin == 1) {
+            // compiler/chxvm/simple_node_emitter.cc:698-701
+            simple(op, {ArrayIn(Operand(n, 0)), IntIn(n.GetInt("axis", 1))});
         } else if (op == "Reshape" && nin == 2) {
             simple(op, {ArrayIn(Operand(n, 0)), ShapeIn(Operand(n, 1))});
         } else if (op == "Cast" && nin == 1) {

@@ -2,8 +2,9 @@
 // leaving the 8-bit domain.  In a ChxVM program these appear as
 //   DequantizeLinear -> MaxPool / AveragePool (runtime/ops/pooling.cc:47-75) -> QuantizeLinear;
 // the hip backend lowers each such triple to one of these kernels.
-//   max:     with the same scale and zero point on both sides the triple equals the
-//            maximum of the codes (dequantization is increasing, Q(DQ(q)) == q).
+//   max:     with the same scale and zero point on both sides the triple is a function of the
+//            maximum of the codes (dequantization is increasing): uint8 Q(DQ(q)) == q; int8
+//            Q(DQ(q)) == q + (q < 0), because QuantizeLinear adds 0.5 and the cast truncates toward zero.
 //   average: y = Q( (sum of DQ(x) over the window, fp32, in (kh, kw) order) / count ).
 // Both are bandwidth-bound; channels-last tensors move 16 channels per lane.
 #include <cstring>
@@ -92,9 +93,16 @@ __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
                 m[d].odd = pk_max_u16(m[d].odd, x.odd);
             }
     }
+    // int8: the QuantizeLinear behind the pool adds 0.5 and truncates toward zero, so a negative code
+    // comes back one higher (q + 0.5 truncates to q + 1 for q < 0, to q for q >= 0).  In the flipped
+    // domain a negative code is a byte below 128: add one to exactly those (no carry can leave the byte).
     v4u out;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) out[d] = touches ? (m[d].even | (m[d].odd << 8)) ^ flip : flip;
+    for (int d = 0; d < 4; ++d) {
+        uint32_t u = touches ? m[d].even | (m[d].odd << 8) : 0u;
+        if (a.is_signed) u += (~u >> 7) & 0x01010101u;
+        out[d] = u ^ flip;
+    }
     *reinterpret_cast<v4u*>(a.y + n * a.ys[0] + oh * a.ys[2] + ow * a.ys[3] + cg * 16) = out;
 }
 
@@ -120,6 +128,7 @@ __global__ __launch_bounds__(kThreads) void max_pool_generic_kernel(PoolArgs a) 
             m = v > m ? v : m;
         }
     }
+    if (m < 0) ++m;  // int8 only: Q adds 0.5 and truncates toward zero
     *reinterpret_cast<uint8_t*>(a.y + n * a.ys[0] + c * a.ys[1] + oh * a.ys[2] + ow * a.ys[3]) = (uint8_t)m;
 }
 

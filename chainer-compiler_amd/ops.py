@@ -187,6 +187,43 @@ def QLinearMatMul(a, a_scale, a_zero_point, b, b_scale, b_zero_point, y_scale, y
     return out
 
 
+def Gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=0, trans_b=0, out=None):
+    """GemmOp::RunImpl, runtime/ops/math.cc:160-177, on float32 matrices."""
+    if out is None:
+        m = a.shape[1] if trans_a else a.shape[0]
+        n = b.shape[0] if trans_b else b.shape[1]
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    capi.check(capi.lib().chx_hip_gemm_f32(capi.ref(a), capi.ref(b), capi.ref(c), _f(alpha), _f(beta), ctypes.c_int32(int(trans_a)),
+                                           ctypes.c_int32(int(trans_b)), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
+def Linear(x, w, b=None, n_batch_axes=1, out=None):
+    """LinearOp::RunImpl, runtime/ops/connection.cc:12-15 (chainerx::Linear): x . w^T + b over the
+    first n_batch_axes axes of x."""
+    if out is None:
+        out = torch.empty(tuple(x.shape[:n_batch_axes]) + (w.shape[0],), dtype=torch.float32, device=x.device)
+    capi.check(capi.lib().chx_hip_linear_f32(capi.ref(x), capi.ref(w), capi.ref(b), ctypes.c_int32(int(n_batch_axes)), capi.ref(out),
+                                             capi.stream_ptr()))
+    return out
+
+
+def Flatten(x, axis=1):
+    """FlattenOp::RunImpl, runtime/ops/manipulation.cc:20-28: [d0 * ... * d(axis-1), the rest], the
+    elements in their logical (row-major) order: a view when x is contiguous, else a device copy."""
+    ax = axis + x.dim() if axis < 0 else axis
+    if not 0 <= ax < x.dim():
+        raise ValueError("Flatten: axis %d is outside [0, %d)" % (axis, x.dim()))
+    d0 = 1
+    for d in x.shape[:ax]:
+        d0 *= int(d)
+    if not x.is_contiguous():
+        dense = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
+        capi.check(capi.lib().chx_hip_cast(capi.ref(x), capi.ref(dense), capi.stream_ptr()))  # same type: a strided copy
+        x = dense
+    return x.view(d0, -1)
+
+
 class QLinearConvPlan(object):
     """Weight-side state of one QLinearConv instruction (chx_hip_qconv_plan): repacked
     weights and per-channel sums, built once and reused by every run."""
@@ -261,7 +298,8 @@ def _pool_out(in_dim, p0, p1, k, s, cover_all):
 
 def MaxPoolQ8(x, kernel_shape, strides=(), pads=(), cover_all=False, out=None):
     """DequantizeLinear -> MaxPool (runtime/ops/pooling.cc:47-61) -> QuantizeLinear with equal
-    quantization parameters, on the 8-bit codes."""
+    quantization parameters, on the 8-bit codes: their maximum m for uint8, m + (m < 0) for int8 (the
+    QuantizeLinear adds 0.5 and truncates toward zero)."""
     strides = _complement(strides, 2, 1)
     pads = _complement(pads, 2, 0)
     if out is None:

@@ -1,0 +1,72 @@
+// The float layers around a quantized network on the hip backend: GemmOp and MatMulOp
+// (runtime/ops/math.cc:156-177 of the chainer-compiler tree), LinearOp (runtime/ops/connection.cc:12-15),
+// FlattenOp (runtime/ops/manipulation.cc:20-28).  The products run in chx_hip_gemm_f32 /
+// chx_hip_linear_f32; Flatten is a view, after a device copy when the array is not dense.
+#include "../gen/gen_chxvm_ops.h"
+
+namespace chainer_compiler {
+namespace runtime {
+
+namespace {
+
+void CheckFloat32(const chainerx::Array& a, const char* op, const char* name) {
+    CHECK(a.dtype() == chainerx::Dtype::kFloat32) << op << ": " << name << " must be float32 on the hip backend, not " << a.dtype();
+}
+
+}  // namespace
+
+// A dense copy in logical (row-major) order; the array itself when it already is dense.
+chainerx::Array AsContiguous(const chainerx::Array& a) {
+    if (a.IsContiguous()) return a;
+    chainerx::Array dense = chainerx::Empty(a.shape(), a.dtype());
+    chx_hip_tensor xt = a.hip(), yt = dense.hip();
+    CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, chainerx::CurrentStream()));  // same element type on both sides: a strided copy
+    return dense;
+}
+
+chainerx::Array GemmOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b, const absl::optional<chainerx::Array>& c) {
+    CheckFloat32(a, "Gemm", "a");
+    CheckFloat32(b, "Gemm", "b");
+    CHECK_EQ(2, a.ndim()) << "Gemm: a must be a matrix";
+    CHECK_EQ(2, b.ndim()) << "Gemm: b must be a matrix";
+    if (c.has_value()) CheckFloat32(*c, "Gemm", "c");
+    const int64_t m = a.shape()[trans_a ? 1 : 0], n = b.shape()[trans_b ? 0 : 1];
+    chainerx::Array y = chainerx::Empty(chainerx::Shape{m, n}, chainerx::Dtype::kFloat32);
+    chx_hip_tensor at = a.hip(), bt = b.hip(), yt = y.hip(), ct;
+    if (c.has_value()) ct = c->hip();
+    CHXVM_HIP_CALL(chx_hip_gemm_f32(&at, &bt, c.has_value() ? &ct : nullptr, static_cast<float>(alpha), static_cast<float>(beta),
+                                    trans_a ? 1 : 0, trans_b ? 1 : 0, &yt, chainerx::CurrentStream()));
+    return y;
+}
+
+chainerx::Array LinearOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& x, const chainerx::Array& w, const absl::optional<chainerx::Array>& b) {
+    CheckFloat32(x, "Linear", "x");
+    CheckFloat32(w, "Linear", "w");
+    if (b.has_value()) CheckFloat32(*b, "Linear", "b");
+    CHECK_EQ(2, w.ndim()) << "Linear: w must be [out, in]";
+    CHECK(n_batch_axes >= 1 && n_batch_axes < x.ndim()) << "Linear: n_batch_axes " << n_batch_axes << " for an x of rank " << x.ndim();
+    const chainerx::Array xd = AsContiguous(x);
+    chainerx::Shape shape;
+    for (int i = 0; i < n_batch_axes; ++i) shape.push_back(x.shape()[i]);
+    shape.push_back(w.shape()[0]);
+    chainerx::Array y = chainerx::Empty(shape, chainerx::Dtype::kFloat32);
+    chx_hip_tensor xt = xd.hip(), wt = w.hip(), yt = y.hip(), bt;
+    if (b.has_value()) bt = b->hip();
+    CHXVM_HIP_CALL(chx_hip_linear_f32(&xt, &wt, b.has_value() ? &bt : nullptr, static_cast<int32_t>(n_batch_axes), &yt,
+                                      chainerx::CurrentStream()));
+    return y;
+}
+
+chainerx::Array FlattenOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
+    const int ax = axis < 0 ? static_cast<int>(axis) + input.ndim() : static_cast<int>(axis);  // ResolveAxis, chainerx_util.cc:417-422
+    CHECK_GE(ax, 0);
+    CHECK_LT(ax, input.ndim());
+    int64_t d0 = 1, d1 = 1;
+    for (int i = 0; i < input.ndim(); ++i) (i < ax ? d0 : d1) *= input.shape()[i];
+    return AsContiguous(input).Reshape(chainerx::Shape{d0, d1});
+}
+
+}  // namespace runtime
+}  // namespace chainer_compiler

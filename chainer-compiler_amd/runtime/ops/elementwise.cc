@@ -11,6 +11,8 @@
 namespace chainer_compiler {
 namespace runtime {
 
+chainerx::Array AsContiguous(const chainerx::Array& a);  // ops/connection.cc
+
 namespace {
 
 // dtypes of the outputs, from the program's `out name:dtype ...` line
@@ -232,9 +234,9 @@ chainerx::Array CastOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
     return y;
 }
 
-// a view of the same memory (runtime/ops/manipulation.cc:20-22); -1 and 0 entries as ONNX defines them
+// a view of the same memory, after a dense copy where the array is not dense (runtime/ops/manipulation.cc:30-53);
+// -1 and 0 entries as ONNX defines them
 chainerx::Array ReshapeOp::RunImpl(ChxVMState* st, const chainerx::Array& data, const chainerx::Shape& shape) {
-    CHECK(data.IsContiguous()) << "Reshape of a non-contiguous array is not supported on the hip backend";
     chainerx::Shape to = shape;
     int64_t known = 1;
     int wildcard = -1;
@@ -252,7 +254,7 @@ chainerx::Array ReshapeOp::RunImpl(ChxVMState* st, const chainerx::Array& data, 
     }
     if (wildcard >= 0) to[wildcard] = known ? data.GetTotalSize() / known : 0;
     CHECK_EQ(data.GetTotalSize(), to.GetTotalSize()) << "Reshape changes the number of elements";
-    return data.Reshape(to);
+    return AsContiguous(data).Reshape(to);  // chainerx::Reshape copies likewise when the strides do not allow a view
 }
 
 }  // namespace runtime

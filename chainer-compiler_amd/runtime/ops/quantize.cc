@@ -206,13 +206,17 @@ chainerx::Array ConvIntegerOp::RunImpl(
     return y;
 }
 
-// A float MatMul only exists on this backend between two DequantizeLinear and one
-// QuantizeLinear, the sequence ReplaceQLinearMatMul leaves (compiler/simplifier.cc:675-694);
-// ChxVM fuses that sequence into one quantized product when it loads the program (chxvm.cc).
+// MatMulOp::RunImpl, runtime/ops/math.cc:156-158 (NumpyMatMul, runtime/chainerx_util.cc:210-230) for
+// matrices.  Between two DequantizeLinear and one QuantizeLinear (the sequence ReplaceQLinearMatMul
+// leaves, compiler/simplifier.cc:675-694) ChxVM fuses the product into one quantized kernel when it
+// loads the program (chxvm.cc) and this op does not run; anywhere else it is a float32 product.
 chainerx::Array MatMulOp::RunImpl(ChxVMState* st, const chainerx::Array& a, const chainerx::Array& b) {
-    CHECK(false) << "float MatMul outside a DequantizeLinear, DequantizeLinear, MatMul, QuantizeLinear sequence "
-                    "is not part of the quantized-inference path of the hip runtime";
-    return chainerx::Array();
+    CHECK(a.ndim() == 2 && b.ndim() == 2) << "float MatMul of operands that are not matrices is not computed on the hip backend";
+    CHECK(a.dtype() == chainerx::Dtype::kFloat32 && b.dtype() == chainerx::Dtype::kFloat32) << "float MatMul: float32 operands only";
+    chainerx::Array y = chainerx::Empty(chainerx::Shape{a.shape()[0], b.shape()[1]}, chainerx::Dtype::kFloat32);
+    chx_hip_tensor at = a.hip(), bt = b.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_gemm_f32(&at, &bt, nullptr, 1.f, 1.f, 0, 0, &yt, chainerx::CurrentStream()));
+    return y;
 }
 
 }  // namespace runtime

@@ -228,12 +228,37 @@ int chx_hip_qlinear_matmul(
         int32_t b_zero_point, float y_scale, int32_t y_zero_point, const chx_hip_tensor* bias, uint32_t flags,
         chx_hip_tensor* y, void* stream);
 
+/* ---- float32 layers around a quantized network ------------------------------------------ */
+
+/* GemmOp::RunImpl, runtime/ops/math.cc:160-177:  r = op(a) . op(b);  r *= alpha when alpha != 1;
+ * y = r when c is NULL or beta == 0, else r + (beta != 1 ? c * beta : c), c broadcast over
+ * [M, N] as numpy does (a vector is a row).  All float32, any strides; trans_a / trans_b
+ * transpose the matrix operands.  The dot product is summed in float32 in ascending k from 0,
+ * one rounding per multiplication and per addition (the order of ChainerX's Dot is not in the
+ * reference tree; results are compared with the reference's own tolerance). */
+int chx_hip_gemm_f32(
+        const chx_hip_tensor* a, const chx_hip_tensor* b, const chx_hip_tensor* c, float alpha, float beta, int32_t trans_a,
+        int32_t trans_b, chx_hip_tensor* y, void* stream);
+
+/* LinearOp::RunImpl, runtime/ops/connection.cc:12-15 (chainerx::Linear): x is taken as a matrix
+ * [product of its first n_batch_axes extents, product of the rest], y = x . w^T + b with
+ * w [out, in] and b [out] or NULL; y has the batch extents of x and one axis of `out`.  The axes
+ * of x (and of y) on each side of n_batch_axes must be contiguous with each other.  The same
+ * arithmetic as chx_hip_gemm_f32 with trans_b, alpha = beta = 1 (GemmOp takes this route then,
+ * math.cc:162-164). */
+int chx_hip_linear_f32(
+        const chx_hip_tensor* x, const chx_hip_tensor* w, const chx_hip_tensor* b, int32_t n_batch_axes, chx_hip_tensor* y,
+        void* stream);
+
 /* ---- pooling on quantized tensors ------------------------------------------------------ */
 
 /* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized
  * network: DequantizeLinear -> MaxPool -> QuantizeLinear with one scale and zero
- * point on both sides, which equals the maximum of the 8-bit codes.  x, y uint8 or
- * int8 (same dtype), [N,C,H,W].  cover_all as in ChainerX: the output extent is
+ * point on both sides.  For uint8 that is the maximum m of the 8-bit codes; for int8
+ * it is m + (m < 0), because quantize_array (runtime/ops/quantize.cc:16-35) adds 0.5
+ * and casts with truncation toward zero, which moves a negative code up by one (a
+ * window in the padding altogether gives -127).  x, y uint8 or int8 (same dtype),
+ * [N,C,H,W].  cover_all as in ChainerX: the output extent is
  * ceil((in + pads - k) / s) + 1 and overhanging windows see only the image. */
 int chx_hip_max_pool_q8(
         const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,

@@ -32,11 +32,18 @@
  *                            ChainerX's Sigmoid routine is not in the tree.
  *   orc_tanh_f32/orc_exp_f32 call the host libm, as std::tanh/std::exp do in
  *                            ChainerX's native kernels.
+ *   orc_gemm_f32             pinned for everything but the order of the fp32 sum:
+ *                            float64 numpy within a bound from the row norms,
+ *                            bit-equal on integer-valued operands (every sum
+ *                            exact), the alpha/beta/c branches one by one, a
+ *                            row against a sequential float32 running sum.
+ *                            PARITY UNPINNED for the order (ascending k):
+ *                            ChainerX's Dot is not in the tree.
  *   orc_max_pool_q8          pinned: numpy restatement over an explicitly padded
  *                            array (both types, cover_all, pads, whole-image
  *                            window), and the three float ops spelled out
  *                            (DequantizeLinear, maximum over a -inf padded
- *                            tensor, QuantizeLinear) for uint8.
+ *                            tensor, QuantizeLinear) for uint8 and int8.
  *   orc_average_pool_q8      pinned: numpy restatement (tap-major loop over a
  *                            zero-padded float tensor, both pad-count modes,
  *                            both roundings, all four type pairs), the exact
@@ -196,6 +203,41 @@ void orc_matmul_integer(
                     out[j] += av * bv;
                 }
             }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* GemmOp::RunImpl, runtime/ops/math.cc:160-177 (and through it LinearOp::RunImpl,
+ * runtime/ops/connection.cc:12-15, which is the case trans_b, alpha = beta = 1 with a
+ * vector c).  a is [M,K] (or [K,M] when trans_a), b [K,N] (or [N,K] when trans_b), both
+ * dense row-major; c is dense [c_rows, c_cols] with each extent 1 or the full one (numpy
+ * broadcasting), c == NULL for none.
+ *   r = Dot(op(a), op(b));  if (alpha != 1) r *= alpha;  if (beta == 0 || !c) return r;
+ *   xc = beta != 1 ? c * beta : c;  return r + xc
+ * Dot is a float32 sum in ascending k from 0, one rounding per operation (this file is
+ * compiled with -ffp-contract=off). */
+void orc_gemm_f32(
+        const float* a, const float* b, const float* c, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha,
+        float beta, int64_t c_rows, int64_t c_cols, float* y) {
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t i = 0; i < M; ++i) {
+        for (int64_t j = 0; j < N; ++j) {
+            float acc = 0.f;
+            for (int64_t k = 0; k < K; ++k) {
+                const float av = trans_a ? a[k * M + i] : a[i * K + k];
+                const float bv = trans_b ? b[j * K + k] : b[k * N + j];
+                const float p = av * bv;
+                acc = acc + p;
+            }
+            float r = acc;
+            if (alpha != 1.f) r = r * alpha;
+            if (c != NULL && beta != 0.f) {
+                float xc = c[(c_rows == 1 ? 0 : i) * c_cols + (c_cols == 1 ? 0 : j)];
+                if (beta != 1.f) xc = xc * beta;
+                r = r + xc;
+            }
+            y[i * N + j] = r;
         }
     }
 }
@@ -538,9 +580,9 @@ void orc_round_f32(const float* x, int64_t n, float* y) {
  * runs it (MaxPoolOp / AveragePoolOp::RunImpl, runtime/ops/pooling.cc:47-75).
  *
  * orc_max_pool_q8: DequantizeLinear -> MaxPool -> QuantizeLinear with the same scale
- * and zero point on both sides equals the maximum of the codes, because the
- * dequantization map is increasing and Q(DQ(q)) == q for uint8 (checked exhaustively
- * in the tests).  Out-of-image taps never win (ChainerX pads max-pooling with the
+ * and zero point on both sides is a function of the maximum m of the codes, because the
+ * dequantization map is increasing: Q(DQ(m)) == m for uint8 and m + (m < 0) for int8
+ * (both checked exhaustively in the tests against the three float operations).  Out-of-image taps never win (ChainerX pads max-pooling with the
  * lowest value); cover_all adds a last window for what floor would leave uncovered
  * (out = ceil((in + p0 + p1 - k) / s) + 1 instead of floor), which with pads can lie in the
  * padding altogether.
@@ -576,8 +618,11 @@ void orc_max_pool_q8(
                         const int32_t v = load_q(x, x_is_int8, (nc * H + ih) * W + iw);
                         if (v > m) m = v;
                     }
+                /* int8: QuantizeLinear adds 0.5 and the cast truncates toward zero (quantize.cc:16-35), so a
+                 * negative code q comes back as q + 1: q + 0.5 (give or take the rounding of DQ and the
+                 * division, far below 0.5) truncates to q + 1 for q < 0 and to q for q >= 0 */
                 if (x_is_int8)
-                    ((int8_t*)y)[(nc * OH + oh) * OW + ow] = (int8_t)m;
+                    ((int8_t*)y)[(nc * OH + oh) * OW + ow] = (int8_t)(m < 0 ? m + 1 : m);
                 else
                     ((uint8_t*)y)[(nc * OH + oh) * OW + ow] = (uint8_t)m;
             }

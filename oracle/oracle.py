@@ -113,6 +113,42 @@ def _zp_arr(zp):
     return np.ascontiguousarray(z), z.size
 
 
+def gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=False, trans_b=False):
+    """GemmOp::RunImpl, runtime/ops/math.cc:160-177."""
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    K2, N = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    assert K == K2 and a.ndim == 2 and b.ndim == 2
+    y = np.empty((M, N), dtype=np.float32)
+    cp, c_rows, c_cols = None, 0, 0
+    if c is not None:
+        c = _c(c, np.float32)
+        c2 = c.reshape((1,) * (2 - c.ndim) + c.shape)
+        c_rows, c_cols = c2.shape
+        assert c_rows in (1, M) and c_cols in (1, N)
+        cp = _p(c)
+    lib().orc_gemm_f32(_p(a), _p(b), cp, ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K), ctypes.c_int(int(trans_a)),
+                       ctypes.c_int(int(trans_b)), _f(alpha), _f(beta), ctypes.c_int64(c_rows), ctypes.c_int64(c_cols), _p(y))
+    return y
+
+
+def linear(x, w, b=None, n_batch_axes=1):
+    """LinearOp::RunImpl, runtime/ops/connection.cc:12-15 (chainerx::Linear)."""
+    x = _c(x, np.float32)
+    rows = int(np.prod(x.shape[:n_batch_axes]))
+    y = gemm(x.reshape(rows, -1), w, b, trans_b=True)
+    return y.reshape(x.shape[:n_batch_axes] + (w.shape[0],))
+
+
+def flatten(x, axis=1):
+    """FlattenOp::RunImpl, runtime/ops/manipulation.cc:20-28."""
+    x = np.asarray(x)
+    ax = axis + x.ndim if axis < 0 else axis
+    assert 0 <= ax < x.ndim
+    return np.ascontiguousarray(x).reshape(int(np.prod(x.shape[:ax], dtype=np.int64)), int(np.prod(x.shape[ax:], dtype=np.int64)))
+
+
 def matmul_integer(a, b, a_zero_point=None, b_zero_point=None):
     a = _c(a)
     b = _c(b)

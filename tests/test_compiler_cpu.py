@@ -376,3 +376,22 @@ def test_reference_flag_names_as_options(vm):
         vm.transform_onnx(chain, {"backend_name": "chxvm"})
     with pytest.raises(vm.ChxVMError, match="unknown option 'use_tvm'"):
         vm.transform_onnx(chain, {"use_tvm": True})
+
+
+def test_float_head_nodes_are_emitted_with_the_reference_operand_lists(vm):
+    """Flatten, Gemm, MatMul (compiler/chxvm/simple_node_emitter.cc:312-318, 698-701): operands in the order of
+    runtime/chxvm_defs.py, attribute defaults of the ONNX nodes (alpha = beta = 1, no transposition, axis 1)."""
+    N = onnx_lite.Node
+    w, b, w2 = np.zeros((9, 32), np.float32), np.zeros(9, np.float32), np.zeros((9, 4), np.float32)
+    m = model([N("Flatten", ["x"], ["f"], {}), N("Gemm", ["f", "w", "b"], ["h"], {"transB": 1, "alpha": 0.5}), N("Gemm", ["h", "w2"], ["h2"], {}),
+               N("MatMul", ["h2", "w3"], ["y"], {})],
+              [("x", (3, 2, 4, 4))], [("y", (3, 4))], {"w": w, "b": b, "w2": w2, "w3": np.zeros((4, 4), np.float32)})
+    insts = decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))
+    flat = next(i for i in insts if i[0] == "Flatten")
+    assert [t for t, _ in flat[1]] == ["ARRAY", "INT"] and flat[1][1][1] == 1
+    g1, g2 = [i for i in insts if i[0] == "Gemm"]
+    assert [t for t, _ in g1[1]] == ["ARRAY", "ARRAY", "ARRAY", "FLOAT", "FLOAT", "INT", "INT"]
+    assert [v for _, v in g1[1][3:]] == [0.5, 1.0, 0, 1] and g1[1][2][1] > 0
+    assert [v for _, v in g2[1][2:]] == [-1, 1.0, 1.0, 0, 0]          # no c: the optional operand is -1
+    mm = next(i for i in insts if i[0] == "MatMul")
+    assert [t for t, _ in mm[1]] == ["ARRAY", "ARRAY"]

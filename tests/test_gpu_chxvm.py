@@ -382,10 +382,10 @@ def test_trace_lines(g, vm, capfd):
     prog.close()
 
 
-def test_max_pool_on_codes_is_for_uint8_only(g, vm, oracle):
-    """DequantizeLinear -> MaxPool -> QuantizeLinear with one scale and zero point runs as the maximum
-    of the codes for uint8 (Q(DQ(q)) == q); with int8 codes the reference's truncating QuantizeLinear
-    gives q + 1 for a negative q, so the VM refuses instead of returning other bytes."""
+def test_max_pool_on_codes_for_both_8_bit_types(g, vm, oracle):
+    """DequantizeLinear -> MaxPool -> QuantizeLinear with one scale and zero point runs as one kernel on the
+    codes: the maximum for uint8 (Q(DQ(q)) == q); for int8 the reference's truncating QuantizeLinear gives
+    q + 1 for a negative q, and so does the kernel.  Checked against the three float ops of the oracle."""
     def pool_program(zp, zdt):
         b = vm.ProgramBuilder()
         x = b.input("x", zdt, (1, 16, 6, 6))
@@ -397,14 +397,19 @@ def test_max_pool_on_codes_is_for_uint8_only(g, vm, oracle):
         b.output("q", q)
         return b.serialize()
     rng = np.random.default_rng(8)
-    xu = rng.integers(0, 256, size=(1, 16, 6, 6)).astype(np.uint8)
-    prog = vm.Program(pool_program(30, "uint8"))
-    np.testing.assert_array_equal(prog.run({"x": g.dev(xu)})["q"], oracle.max_pool_q8(xu, (2, 2), (2, 2)))
-    prog.close()
-    xi = rng.integers(-128, 128, size=(1, 16, 6, 6)).astype(np.int8)
-    with pytest.raises(vm.ChxVMError, match="int8"):
-        prog = vm.Program(pool_program(-3, "int8"))
-        prog.run({"x": g.dev(xi)})
+    for dt, zp in ((np.uint8, 30), (np.int8, -3)):
+        info = np.iinfo(dt)
+        x = rng.integers(info.min, info.max + 1, size=(1, 16, 6, 6)).astype(dt)
+        prog = vm.Program(pool_program(zp, np.dtype(dt).name))
+        got = prog.run({"x": g.dev(x)})["q"]
+        prog.close()
+        np.testing.assert_array_equal(got, oracle.max_pool_q8(x, (2, 2), (2, 2)))
+        pooled = oracle.dequantize_linear(x, np.float32(0.05), zp).reshape(1, 16, 3, 2, 3, 2).max(axis=(3, 5))
+        np.testing.assert_array_equal(got, oracle.quantize_linear(pooled, np.float32(0.05), zp, dt))
+        if dt == np.int8:
+            m = x.reshape(1, 16, 3, 2, 3, 2).max(axis=(3, 5)).astype(np.int64)
+            assert (m < 0).any()
+            np.testing.assert_array_equal(got, m + (m < 0))
 
 
 def _conv_program(vm, shape, w, ws, wz, bias, xq, yq, weights_as_inputs=False):

@@ -1,0 +1,163 @@
+"""The float32 layers around a quantized network: Gemm, Linear, MatMul, Flatten (runtime/ops/math.cc:156-177,
+runtime/ops/connection.cc:12-15, runtime/ops/manipulation.cc:20-28 of the chainer-compiler tree), through
+the C ABI and as instructions of a serialized program.  The device sums in the oracle's order (ascending
+k, one rounding per operation), so results are compared bit for bit; against a float64 product the bar
+is the bound of a float32 sum of K terms."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.capi.init(0)
+    return gpu_util
+
+
+@pytest.fixture(scope="module")
+def vm(g):
+    from importlib import import_module
+    return import_module(g.pkg.__name__ + ".chxvm")
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.int32)
+
+
+GEMM_CASES = [
+    # M, N, K, trans_a, trans_b, c shape (None: no c), alpha, beta
+    (32, 100, 784, False, False, None, 1.0, 1.0),          # the MLP of the reference's quantization test, first layer
+    (32, 10, 100, False, True, (10,), 1.0, 1.0),           # the Linear route of GemmOp
+    (64, 1000, 2048, False, True, (1000,), 1.0, 1.0),      # ResNet-50 classifier at batch 64
+    (7, 5, 3, True, False, (7, 1), 0.5, 2.0),
+    (65, 129, 17, True, True, (65, 129), 1.0, -1.0),
+    (1, 1, 1, False, False, (1, 1), 3.0, 1.0),
+    (130, 66, 300, False, False, (1, 66), 1.0, 0.0),       # beta == 0: c is not read
+    (3, 4, 0, False, False, (4,), 1.0, 1.0),               # an empty sum is 0
+]
+
+
+@pytest.mark.parametrize("case", GEMM_CASES, ids=lambda c: "M%d_N%d_K%d_%s%s" % (c[0], c[1], c[2], "T" if c[3] else "N", "T" if c[4] else "N"))
+def test_gemm_through_the_c_abi(g, oracle, case):
+    M, N, K, ta, tb, cshape, alpha, beta = case
+    rng = np.random.default_rng(M * 1000 + N)
+    a = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    b = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    c = None if cshape is None else rng.standard_normal(cshape).astype(np.float32)
+    if beta == 0.0 and c is not None:
+        c[...] = np.nan
+    want = oracle.gemm(a, b, c, alpha, beta, ta, tb)
+    got = g.host(g.ops.Gemm(g.dev(a), g.dev(b), None if c is None else g.dev(c), alpha, beta, int(ta), int(tb)))
+    assert got.shape == (M, N) and got.dtype == np.float32
+    np.testing.assert_array_equal(bits(got), bits(want))
+    if K:
+        A, B = (a.T if ta else a).astype(np.float64), (b.T if tb else b).astype(np.float64)
+        exact = alpha * (A @ B) + (0 if c is None or beta == 0.0 else beta * c.astype(np.float64))
+        bound = (K + 3) * 2.0 ** -24 * (abs(alpha) * (np.abs(A) @ np.abs(B)) + (0 if c is None or beta == 0.0 else np.abs(beta * c)))
+        assert (np.abs(got - exact) <= bound + 1e-30).all()
+
+
+def test_gemm_reads_operands_through_their_strides(g, oracle):
+    rng = np.random.default_rng(7)
+    big_a = rng.standard_normal((40, 90)).astype(np.float32)
+    big_b = rng.standard_normal((90, 50)).astype(np.float32)
+    a, b = big_a[3:33:2, 5:65:3], big_b[10:30, ::5]      # 15 x 20 and 20 x 10 views
+    da, db = g.dev(big_a)[3:33:2, 5:65:3], g.dev(big_b)[10:30, ::5]
+    out = torch.zeros((15, 30), dtype=torch.float32, device="cuda")[:, ::3]
+    g.ops.Gemm(da, db, out=out)
+    np.testing.assert_array_equal(bits(g.host(out)), bits(oracle.gemm(np.ascontiguousarray(a), np.ascontiguousarray(b))))
+    # a transposed view is the transposed operand
+    np.testing.assert_array_equal(bits(g.host(g.ops.Gemm(da.t(), db.t(), trans_a=1, trans_b=1))),
+                                  bits(oracle.gemm(np.ascontiguousarray(a), np.ascontiguousarray(b))))
+
+
+def test_gemm_refuses_what_it_cannot_compute(g):
+    a, b = g.dev(np.zeros((3, 4), np.float32)), g.dev(np.zeros((5, 6), np.float32))
+    with pytest.raises(g.capi.ChxHipError, match="inner extents"):
+        g.ops.Gemm(a, b)
+    with pytest.raises(g.capi.ChxHipError, match="float32"):
+        g.ops.Gemm(a, g.dev(np.zeros((4, 6), np.int32)))
+    with pytest.raises(g.capi.ChxHipError, match="broadcast"):
+        g.ops.Gemm(a, g.dev(np.zeros((4, 6), np.float32)), g.dev(np.zeros((5,), np.float32)))
+
+
+def test_linear_over_batch_axes(g, oracle):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    for nb, k in ((1, 60), (2, 20), (3, 5)):
+        w = rng.standard_normal((7, k)).astype(np.float32)
+        bias = rng.standard_normal((7,)).astype(np.float32)
+        got = g.host(g.ops.Linear(g.dev(x), g.dev(w), g.dev(bias), nb))
+        assert got.shape == x.shape[:nb] + (7,)
+        np.testing.assert_array_equal(bits(got), bits(oracle.linear(x, w, bias, nb)))
+        np.testing.assert_array_equal(bits(g.host(g.ops.Linear(g.dev(x), g.dev(w), None, nb))), bits(oracle.linear(x, w, None, nb)))
+    with pytest.raises(g.capi.ChxHipError, match="n_batch_axes"):
+        g.ops.Linear(g.dev(x), g.dev(np.zeros((7, 5), np.float32)), None, 4)
+
+
+def test_flatten(g, oracle):
+    x = np.arange(2 * 3 * 4 * 5).reshape(2, 3, 4, 5).astype(np.float32)
+    for axis in (0, 1, 2, 3, -1, -3):
+        np.testing.assert_array_equal(g.host(g.ops.Flatten(g.dev(x), axis)), oracle.flatten(x, axis))
+    # a channels-last tensor flattens in its logical (NCHW) order
+    np.testing.assert_array_equal(g.host(g.ops.Flatten(g.to_channels_last(g.dev(x)), 1)), x.reshape(2, 60))
+    q = np.arange(2 * 16 * 3 * 3).reshape(2, 16, 3, 3).astype(np.uint8)
+    np.testing.assert_array_equal(g.host(g.ops.Flatten(g.to_channels_last(g.dev(q)), 1)), q.reshape(2, 144))
+    with pytest.raises(ValueError):
+        g.ops.Flatten(g.dev(x), 4)
+
+
+def test_float_layers_as_program_instructions(g, vm, oracle):
+    """Flatten -> Gemm (Linear route) -> Relu -> MatMul -> Linear in one serialized program, against the
+    oracle op by op."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((4, 8, 3, 3)).astype(np.float32)
+    w1 = rng.standard_normal((20, 72)).astype(np.float32)
+    b1 = rng.standard_normal((20,)).astype(np.float32)
+    w2 = rng.standard_normal((20, 6)).astype(np.float32)
+    w3 = rng.standard_normal((5, 6)).astype(np.float32)
+    b = vm.ProgramBuilder()
+    xs = b.input("x", "float32", x.shape)
+    f = b.Flatten(xs, 1)
+    h = b.Gemm(f, b.constant(w1), b.constant(b1), 1.0, 1.0, 0, 1)
+    r = b.Relu(h)
+    m = b.MatMul(r, b.constant(w2))
+    y = b.Linear(m, b.constant(w3), None, 1)
+    g2 = b.Gemm(r, b.constant(w2), None, 0.25, 1.0, 0, 0)
+    for name, slot in (("f", f), ("h", h), ("m", m), ("y", y), ("g2", g2)):
+        b.output(name, slot)
+    prog = vm.Program(b.serialize())
+    want_f = oracle.flatten(x, 1)
+    want_h = oracle.gemm(want_f, w1, b1, trans_b=True)
+    want_r = np.maximum(want_h, np.float32(0))
+    want_m = oracle.gemm(want_r, w2)
+    want_y = oracle.linear(want_m, w3)
+    for xd in (g.dev(x), g.to_channels_last(g.dev(x))):     # a channels-last input is copied dense by Flatten
+        out = prog.run({"x": xd})
+        np.testing.assert_array_equal(out["f"], want_f)
+        np.testing.assert_array_equal(bits(out["h"]), bits(want_h))
+        np.testing.assert_array_equal(bits(out["m"]), bits(want_m))
+        np.testing.assert_array_equal(bits(out["y"]), bits(want_y))
+        np.testing.assert_array_equal(bits(out["g2"]), bits(oracle.gemm(want_r, w2, alpha=0.25)))
+    prog.close()
+
+
+def test_float_layers_from_an_onnx_graph(g, vm, oracle):
+    """Flatten, Gemm and MatMul nodes of an ONNX graph reach the VM through the compiler's emitter."""
+    import test_compiler_cpu as cc
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((3, 2, 4, 4)).astype(np.float32)
+    w = rng.standard_normal((9, 32)).astype(np.float32)
+    bias = rng.standard_normal((9,)).astype(np.float32)
+    w2 = rng.standard_normal((9, 4)).astype(np.float32)
+    N = cc.onnx_lite.Node
+    m = cc.model([N("Flatten", ["x"], ["f"], {"axis": 1}), N("Gemm", ["f", "w", "b"], ["h"], {"transB": 1}), N("MatMul", ["h", "w2"], ["y"], {})],
+                 [("x", x.shape)], [("y", (3, 4))], {"w": w, "b": bias, "w2": w2})
+    prog = vm.Program(vm.compile_onnx(m, {"fuse": "none"}))
+    got = prog.run({"x": g.dev(x)})
+    prog.close()
+    want = oracle.gemm(oracle.gemm(oracle.flatten(x, 1), w, bias, trans_b=True), w2)
+    np.testing.assert_array_equal(bits(got["y"]), bits(want))

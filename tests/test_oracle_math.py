@@ -243,16 +243,19 @@ def test_chain_matches_stepwise_numpy(oracle):
     np.testing.assert_array_equal(env["y"], want)
 
 
-def test_max_pool_window_in_the_padding_gives_the_lowest_code(oracle):
+def test_max_pool_window_in_the_padding_gives_what_quantizing_the_lowest_float_gives(oracle):
     """cover_all with pads can add a window that lies in the padding altogether.  Spelled out in
     float (ChainerX pads max-pooling with the lowest value): DequantizeLinear, maximum over a window
-    padded with -inf, QuantizeLinear -> the clamp's lower end, i.e. the lowest code of the type."""
+    padded with -inf, QuantizeLinear -> the clamp's lower end plus 0.5, truncated: 0 for uint8, -127 for int8."""
     rng = np.random.default_rng(17)
-    for dt, lowest in ((np.uint8, 0), (np.int8, -128)):
+    for dt, lowest in ((np.uint8, 0), (np.int8, -127)):
         x = rng.integers(30, 100, size=(1, 2, 11, 16)).astype(dt)
+        if dt == np.int8:
+            x[0, 0, ::2] -= 110                               # negative codes as well
         got = oracle.max_pool_q8(x, (2, 3), (2, 2), (1, 1), True)
         assert got.shape == (1, 2, 7, 9)                      # rows start at -1, 1, ..., 11: the last one is past the image
-        dq = oracle.dequantize_linear(x, np.float32(0.05), 30 if dt == np.uint8 else -30)
+        zp = 30 if dt == np.uint8 else -30
+        dq = oracle.dequantize_linear(x, np.float32(0.05), zp)
         padded = np.full((1, 2, 11 + 1 + 3, 16 + 1 + 3), -np.inf, np.float32)
         padded[:, :, 1:12, 1:17] = dq
         want = np.empty((1, 2, 7, 9), np.float32)
@@ -261,11 +264,9 @@ def test_max_pool_window_in_the_padding_gives_the_lowest_code(oracle):
                 want[:, :, oh, ow] = padded[:, :, 2 * oh:2 * oh + 2, 2 * ow:2 * ow + 3].max(axis=(2, 3))
         assert np.isinf(want[:, :, 6, :]).all() and np.isfinite(want[:, :, :6, :]).all()
         assert (got[:, :, 6, :] == lowest).all()
-        if dt == np.uint8:
-            # the three float ops give the same bytes; for int8 they do not (the reference's QuantizeLinear turns a negative
-            # code q into q + 1), which is why only uint8 pools are computed on codes inside a program
-            with np.errstate(all="ignore"):
-                np.testing.assert_array_equal(got, oracle.quantize_linear(want, np.float32(0.05), 30, dt))
+        # the three float ops give the same bytes
+        with np.errstate(all="ignore"):
+            np.testing.assert_array_equal(got, oracle.quantize_linear(want, np.float32(0.05), zp, dt))
 
 
 # --- pools between a DequantizeLinear and a QuantizeLinear (runtime/ops/pooling.cc:47-75) -------------
@@ -400,7 +401,22 @@ def np_max_pool_q8(x, kernel, strides, pads, cover_all):
     for i in range(kh):
         for j in range(kw):
             out = np.maximum(out, pad[:, :, i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw])
+    if x.dtype == np.int8:
+        out = out + (out < 0)   # the QuantizeLinear behind the pool: q + 0.5 truncates toward zero
     return out.astype(x.dtype)
+
+
+def test_quantize_of_dequantize_is_the_code_for_uint8_and_one_more_for_negative_int8_codes():
+    """Q(DQ(q)) over every code, a spread of scales and every zero point: q for uint8; q + (q < 0) for int8, where
+    q + 0.5 is truncated toward zero by the cast (quantize.cc:16-35)."""
+    rng = np.random.default_rng(36)
+    scales = np.concatenate([rng.uniform(1e-4, 10.0, 40), 2.0 ** np.arange(-8, 4)]).astype(np.float32)
+    for dt, lo, hi in ((np.uint8, 0, 255), (np.int8, -128, 127)):
+        q = np.arange(lo, hi + 1).astype(dt)
+        want = q.astype(np.int64) + ((q.astype(np.int64) < 0) if dt == np.int8 else 0)
+        for scale in scales:
+            for zp in range(lo, hi + 1, 5):
+                np.testing.assert_array_equal(np_quantize(np_dequantize(q, scale, zp), scale, zp, lo, hi), want, err_msg=str((dt, scale, zp)))
 
 
 @pytest.mark.parametrize("dt", [np.uint8, np.int8])
@@ -414,16 +430,20 @@ def test_max_pool_vs_numpy(oracle, dt, cover_all):
         np.testing.assert_array_equal(got, np_max_pool_q8(x, kernel, strides, pads, cover_all), err_msg=str((kernel, strides, pads)))
     # kernel = whole image: the maximum of each plane
     x = rng.integers(info.min, info.max + 1, size=(2, 3, 6, 5)).astype(dt)
-    np.testing.assert_array_equal(oracle.max_pool_q8(x, (6, 5), (1, 1), (0, 0), cover_all).reshape(2, 3), x.max(axis=(2, 3)))
+    m = x.max(axis=(2, 3)).astype(np.int64)
+    np.testing.assert_array_equal(oracle.max_pool_q8(x, (6, 5), (1, 1), (0, 0), cover_all).reshape(2, 3), m + ((m < 0) if dt == np.int8 else 0))
 
 
-def test_max_pool_on_codes_equals_the_three_float_ops_for_uint8(oracle):
-    """DequantizeLinear -> MaxPool over a -inf padded float tensor -> QuantizeLinear, spelled out, gives the maximum
-    of the codes for uint8 (increasing dequantization, Q(DQ(q)) == q), for any zero point and window."""
+@pytest.mark.parametrize("dt", [np.uint8, np.int8])
+def test_max_pool_on_codes_equals_the_three_float_ops(oracle, dt):
+    """DequantizeLinear -> MaxPool over a -inf padded float tensor -> QuantizeLinear, spelled out, for any zero point
+    and window: the maximum of the codes for uint8 (increasing dequantization, Q(DQ(q)) == q), one more for a negative
+    maximum for int8."""
     rng = np.random.default_rng(35)
+    info = np.iinfo(dt)
     for kernel, strides, pads, H, W in POOL_CASES:
-        x = rng.integers(0, 256, size=(1, 2, H, W)).astype(np.uint8)
-        zp = int(rng.integers(0, 256))
+        x = rng.integers(info.min, info.max + 1, size=(1, 2, H, W)).astype(dt)
+        zp = int(rng.integers(info.min, info.max + 1))
         scale = np.float32(rng.uniform(0.01, 0.2))
         got = oracle.max_pool_q8(x, kernel, strides, pads, False)
         OH, OW = got.shape[2:]
@@ -434,4 +454,89 @@ def test_max_pool_on_codes_equals_the_three_float_ops_for_uint8(oracle):
             for j in range(kernel[1]):
                 want = np.maximum(want, val[:, :, i:i + (OH - 1) * strides[0] + 1:strides[0], j:j + (OW - 1) * strides[1] + 1:strides[1]])
         with np.errstate(all="ignore"):
-            np.testing.assert_array_equal(got, np_quantize(want, scale, zp, 0, 255).astype(np.uint8))
+            np.testing.assert_array_equal(got, np_quantize(want, scale, zp, info.min, info.max).astype(dt))
+
+
+# --- Gemm / Linear / Flatten (runtime/ops/math.cc:160-177, connection.cc:12-15, manipulation.cc:20-28) ---
+# What numpy fixes: the value up to the rounding of a float32 sum (float64 product, bound from the row
+# norms), every bit on integer-valued operands (each partial sum is exact, so no order can differ), the
+# alpha / beta / c branches, and the order on one row (a sequential float32 running sum).
+
+def test_gemm_against_float64_within_the_float32_sum_bound(oracle):
+    rng = np.random.default_rng(51)
+    for M, N, K, ta, tb in ((5, 7, 33, False, False), (16, 3, 100, True, False), (3, 9, 64, False, True), (8, 8, 17, True, True)):
+        a = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+        b = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+        got = oracle.gemm(a, b, trans_a=ta, trans_b=tb)
+        A = (a.T if ta else a).astype(np.float64)
+        B = (b.T if tb else b).astype(np.float64)
+        exact = A @ B
+        bound = (K + 1) * 2.0 ** -24 * (np.abs(A) @ np.abs(B))   # a float32 sum of K products
+        assert got.dtype == np.float32 and got.shape == (M, N)
+        assert (np.abs(got - exact) <= bound + 1e-30).all()
+        # a transposed operand is the product of the transposed matrix, bit for bit
+        np.testing.assert_array_equal(got, oracle.gemm(np.ascontiguousarray(A.astype(np.float32)), np.ascontiguousarray(B.astype(np.float32))))
+
+
+def test_gemm_is_exact_on_integer_valued_operands(oracle):
+    """Every product and partial sum is an integer below 2^24: float32 holds them exactly, so any order of
+    summation gives numpy's int64 result, and a dropped term or a wrong index does not."""
+    rng = np.random.default_rng(52)
+    a = rng.integers(-30, 31, size=(9, 40)).astype(np.float32)
+    b = rng.integers(-30, 31, size=(40, 11)).astype(np.float32)
+    c = rng.integers(-100, 101, size=(11,)).astype(np.float32)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    np.testing.assert_array_equal(oracle.gemm(a, b), want.astype(np.float32))
+    np.testing.assert_array_equal(oracle.gemm(a.T.copy(), b.T.copy(), trans_a=True, trans_b=True), want.astype(np.float32))
+    np.testing.assert_array_equal(oracle.gemm(a, b, c), (want + c.astype(np.int64)).astype(np.float32))
+    np.testing.assert_array_equal(oracle.gemm(a, b, c, alpha=2.0, beta=3.0), (2 * want + 3 * c.astype(np.int64)).astype(np.float32))
+    # c broadcasts as numpy does: a column, a full matrix, a single element
+    col = rng.integers(-9, 10, size=(9, 1)).astype(np.float32)
+    full = rng.integers(-9, 10, size=(9, 11)).astype(np.float32)
+    np.testing.assert_array_equal(oracle.gemm(a, b, col), (want + col.astype(np.int64)).astype(np.float32))
+    np.testing.assert_array_equal(oracle.gemm(a, b, full), (want + full.astype(np.int64)).astype(np.float32))
+    np.testing.assert_array_equal(oracle.gemm(a, b, np.float32([[5]])), (want + 5).astype(np.float32))
+    # beta == 0 leaves c out altogether, even a c of NaNs
+    np.testing.assert_array_equal(oracle.gemm(a, b, np.full(11, np.nan, np.float32), beta=0.0), want.astype(np.float32))
+    # Linear = x . w^T + b over the flattened batch axes
+    x = rng.integers(-5, 6, size=(2, 3, 4, 5)).astype(np.float32)
+    w = rng.integers(-5, 6, size=(6, 20)).astype(np.float32)
+    bias = rng.integers(-5, 6, size=(6,)).astype(np.float32)
+    np.testing.assert_array_equal(oracle.linear(x, w, bias, n_batch_axes=2),
+                                  (x.reshape(6, 20).astype(np.int64) @ w.T.astype(np.int64) + bias.astype(np.int64)).reshape(2, 3, 6).astype(np.float32))
+    np.testing.assert_array_equal(oracle.linear(x.reshape(2, 60), rng.integers(-2, 3, size=(4, 60)).astype(np.float32) * 0 + 1),
+                                  np.repeat(x.reshape(2, 60).sum(axis=1, keepdims=True), 4, axis=1))
+
+
+def test_gemm_rounds_once_per_operation_in_the_order_of_math_cc(oracle):
+    """r = Dot; r *= alpha; xc = c * beta; r + xc: each step rounds to float32 on its own (no fused
+    multiply-add), and the dot product of a row is the sequential float32 running sum."""
+    rng = np.random.default_rng(53)
+    a = rng.standard_normal((4, 300)).astype(np.float32)
+    b = rng.standard_normal((300, 5)).astype(np.float32)
+    c = rng.standard_normal((5,)).astype(np.float32)
+    alpha, beta = np.float32(0.7), np.float32(-1.3)
+    prods = a[:, :, None] * b[None, :, :]                       # float32 products
+    dot = np.zeros((4, 5), np.float32)
+    for k in range(300):
+        dot = dot + prods[:, k, :]                              # one float32 addition each, ascending k
+    np.testing.assert_array_equal(oracle.gemm(a, b), dot)
+    np.testing.assert_array_equal(oracle.gemm(a, b, c, alpha=alpha, beta=beta), dot * alpha + c * beta)
+    np.testing.assert_array_equal(oracle.gemm(a, b, c, alpha=alpha), dot * alpha + c)
+    np.testing.assert_array_equal(oracle.gemm(a, b, c, beta=beta), dot + c * beta)
+    # the order matters on this data: the same terms added in descending k give other bits somewhere
+    back = np.zeros((4, 5), np.float32)
+    for k in reversed(range(300)):
+        back = back + prods[:, k, :]
+    assert (back != dot).any()
+
+
+def test_flatten(oracle):
+    x = np.arange(2 * 3 * 4 * 5).reshape(2, 3, 4, 5).astype(np.float32)
+    for axis, shape in ((0, (1, 120)), (1, (2, 60)), (2, (6, 20)), (3, (24, 5)), (-1, (24, 5)), (-3, (2, 60))):
+        got = oracle.flatten(x, axis)
+        assert got.shape == shape
+        np.testing.assert_array_equal(got.ravel(), x.ravel())
+    # a channels-last view flattens in its logical (NCHW) order
+    nhwc = np.ascontiguousarray(x.transpose(0, 2, 3, 1)).transpose(0, 3, 1, 2)
+    np.testing.assert_array_equal(oracle.flatten(nhwc, 1), x.reshape(2, 60))
