@@ -353,6 +353,7 @@ int generate_source(
     os << "#pragma clang fp contract(off)\n";
     os << "#define FM_FN __device__ __forceinline__\n";
     os << "#define FM_TABLE_QUALIFIER static __device__ const\n";
+    os << "#define FM_DEVICE_DIV 1\n";
     std::ostringstream body;
     bool uses_table = false;
     CHX_PROPAGATE(emit_elem(prog, use_fma, body, &uses_table));

@@ -63,6 +63,26 @@ fm_u64 kExp2fTab[32] = {
         0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
 };
 
+// n / d for the three divisions of tanhf and the sigmoid below.  On the device (FM_DEVICE_DIV) it is the
+// reciprocal instruction, one multiplication and two fused multiply-adds: q = n * rcp(d), then one correction
+// by the exact remainder, q + (n - d*q) * rcp(d).  That is 4 instructions where the compiler's IEEE division
+// takes 11 (operand scaling, a refined reciprocal, two corrections, special-case fix-up).  It is not a correctly
+// rounded quotient for every pair of floats, and it has no range handling (d must be normal and finite, the
+// quotient and n * rcp(d) neither overflowing nor denormal); it is used only where the callers' operands stay
+// in range, and what makes it valid there is the test that compares tanhf and the sigmoid built on it with the
+// C library over every one of the 2^32 arguments on the device (tests/test_gpu_elementwise.py).  The host build
+// divides.
+FM_FN float div_in_range(float n, float d) {
+#ifdef FM_DEVICE_DIV
+    const float r = __builtin_amdgcn_rcpf(d);
+    const float q = n * r;
+    const float rem = __builtin_fmaf(-d, q, n);
+    return __builtin_fmaf(rem, r, q);
+#else
+    return n / d;
+#endif
+}
+
 // expf.  kUseFma selects the operation grouping of the C library build that is
 // dispatched on x86-64 CPUs with FMA3: there the compiler contracted the reduction
 // r = InvLn2N*x - kd into one fused multiply-add (and the cubic's multiply-adds,
@@ -234,7 +254,9 @@ FM_FN float tanhf_faithful(float x) {
     const float hxs = xr * hfx;
     const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
     const float t3 = 3.0f - r1 * hfx;
-    const float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+    // 6 - xr*t3 is within a few percent of 6 and r1 - t3 of -2 for every finite argument (xr is the reduced
+    // argument, |xr| <= 0.35); a non-finite argument is replaced by its case's constant at the end
+    const float e = hxs * div_in_range(r1 - t3, 6.0f - xr * t3);
     const float y_k0 = xr - (xr * e - hxs);
     float e2 = (xr * (e - c) - c);
     e2 -= hxs;
@@ -260,7 +282,10 @@ FM_FN float tanhf_faithful(float x) {
     t = k == 0 ? y_k0 : t;
     t = hx < 0x33000000u ? arg : t;  // |arg| < 2^-25: expm1f returns its argument
 
-    const float q = (big ? two : t) / (t + two);
+    // |x| >= 1: 2 / (t + 2) with t = expm1(2|x|) in [6.3, 1.3e19] while |x| < 22 (beyond, z is the constant
+    // below and what this division gives is not used); |x| < 1: t / (t + 2) with t in (-0.87, 0] and
+    // t + 2 in (1.13, 2], the quotient at least 2^-55 in magnitude where it is used
+    const float q = div_in_range(big ? two : t, t + two);
     float z = big ? one - q : -q;
     z = ix >= 0x41b00000u ? one : z;           // |x| >= 22 (and +-inf): one - tiny
     float r = (jx >> 31) == 0 ? z : -z;
@@ -275,7 +300,9 @@ template <bool kUseFma>
 FM_FN float sigmoid_faithful(float x) {
     const float e = expf_faithful<kUseFma>(-x);
     const float d = 1.0f + e;
-    return 1.0f / d;
+    // d >= 1; beyond 2^125 (x < -86.6) the reciprocal approaches the denormal range and the plain division takes over
+    if (d > 0x1p125f) return 1.0f / d;
+    return div_in_range(1.0f, d);
 }
 
 }  // namespace chx_fm

@@ -47,22 +47,41 @@ def unary_program(ops, op):
 
 
 @pytest.mark.parametrize("op", ["Tanh", "Exp", "Sigmoid"])
-def test_transcendentals_bit_exact_over_strided_float_space(g, oracle, op):
-    # every 251st fp32 bit pattern (17.1 M inputs) plus the neighbourhoods where the
-    # algorithms switch branches
-    bits = np.arange(0, 1 << 32, 251, dtype=np.uint64).astype(np.uint32)
+def test_transcendentals_bit_exact_over_every_float(g, oracle, op):
+    """Every fp32 bit pattern, all 2^32 of them, against the host C library (in chunks of 2^26; about 15 s per
+    function with the host side on all cores).  The device code of tanhf and of the sigmoid divides with a short
+    sequence that is valid because this test says so (div_in_range in csrc/faithful_math.h), hence no sampling.
+    CHX_FM_DEVICE_STRIDE=n in the environment takes every n-th pattern plus the neighbourhoods where the
+    algorithms switch branches."""
+    import os
+    stride = int(os.environ.get("CHX_FM_DEVICE_STRIDE", "1"))
     edges = np.array([0x3f800000, 0x41b00000, 0x24000000, 0x3eb17218, 0x3F851592, 0x33000000, 0x4195b844,
-                      0x42b17218, 0x42b00000, 0x42cff1b5, 0x4202422f, 0xc27c65d9, 0x7f800000, 0x00800000],
+                      0x42b17218, 0x42b00000, 0x42cff1b5, 0x4202422f, 0xc27c65d9, 0x7f800000, 0x00800000,
+                      0x7e800000, 0x7e000000, 0xc2ad0000, 0xc2ae0000],
                      dtype=np.uint32)
     near = (edges[:, None].astype(np.int64) + np.arange(-64, 65)[None, :]).astype(np.uint32).reshape(-1)
-    bits = np.concatenate([bits, near, near | np.uint32(0x80000000)])
-    x = bits.view(np.float32)
-    want = {"Tanh": oracle.tanh, "Exp": oracle.exp, "Sigmoid": oracle.sigmoid}[op](x)
-    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, unary_program(g.ops, op))[0])
-    nan = np.isnan(want)
-    assert np.array_equal(np.isnan(got), nan)
-    mism = (got.view(np.uint32) != want.view(np.uint32)) & ~nan
-    assert mism.sum() == 0, "%d of %d differ, first x=%r" % (mism.sum(), x.size, x[mism][:4])
+    fn = {"Tanh": oracle.tanh, "Exp": oracle.exp, "Sigmoid": oracle.sigmoid}[op]
+    prog = unary_program(g.ops, op)
+    threads = oracle.max_threads() if stride < 16 else 1
+    oracle.set_threads(threads)
+    try:
+        chunk = (1 << 26) * stride
+        total = 0
+        for lo in range(0, 1 << 32, chunk):
+            bits = np.arange(lo, min(lo + chunk, 1 << 32), stride, dtype=np.uint64).astype(np.uint32)
+            if lo == 0:
+                bits = np.concatenate([bits, near, near | np.uint32(0x80000000)])
+            x = bits.view(np.float32)
+            want = fn(x)
+            got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, prog)[0])
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan)
+            mism = (got.view(np.uint32) != want.view(np.uint32)) & ~nan
+            assert mism.sum() == 0, "%d of %d differ, first x=%r" % (mism.sum(), x.size, x[mism][:4])
+            total += x.size
+        assert total >= (1 << 32) // stride
+    finally:
+        oracle.set_threads(1)
 
 
 @pytest.mark.parametrize("shape,vec_shape", [((8, 64, 256), (256,)), ((3, 5, 7), (7,)), ((2, 1000), (1000,)),
