@@ -211,14 +211,21 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
             pass
     # the launch configurations the plans measured for these launches: tile (output channels x pixels),
     # work-groups per compute unit (0 = as many as fit) and wavefronts per work-group -> number of layers
-    hist = {}
+    hist, forms = {}, {}
     for rn, _xs in slices:
         for plan in rn.plans.values():
             for line in plan.describe():
                 f = dict(kv.split("=") for kv in line.split() if "=" in kv)
+                if "residual" in f:
+                    # the fused residual sum of this layer: two multiply-adds with constants that the plan's search
+                    # found exact on all code pairs ("affine"), or the operation-by-operation arithmetic ("exact")
+                    forms[f["residual"]] = forms.get(f["residual"], 0) + 1
+                    continue
                 key = "%s/%s/w%s%s" % (f.get("tile"), f.get("wgs_per_cu"), f.get("waves", "4"), "+res" if f.get("res") == "1" else "")
                 hist[key] = hist.get(key, 0) + 1
     roofline["configs"] = hist
+    if forms:
+        roofline["residual_sums"] = forms
     res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),
                value=batch / sec, unit="images/sec", ms_per_step=sec * 1e3, dtype="int8",
                config=dict(workload="mobilenetv2_int8_qdq" if mobilenet else "resnet50_v1_int8_qdq", batch=batch, image=224,

@@ -812,6 +812,10 @@ struct chx_hip_qconv_plan {
     chx::PackedWeights pw;
     chx::ScratchCache scratch;  // makes run() unsafe to call concurrently on one plan
     chx::TuneCache tune;
+    // the residual sum last fused behind this convolution (run_add): its parameters, and whether constants were found
+    // with which its two-multiply-add form is exact (find_affine_residual); kept so that the search runs once
+    bool res_known = false;
+    chx::ResidualAdd res_key, res_found;
 };
 
 extern "C" int chx_hip_qlinear_conv(
@@ -980,6 +984,43 @@ extern "C" int chx_hip_qconv_plan_run_add(
     res.guard = (reach == reach && reach < 0.25 * (double)res.big) ? 0 : 1;
     res.lean = out->dtype == CHX_HIP_UINT8 && r->dtype == CHX_HIP_UINT8 && r_zero_point == 0 && out_zero_point == 0 ? 1 : 0;
     hipStream_t s = as_stream(stream);
+    // The cheaper form of the sum, where the search over its constants has shown it exact for these parameters.  The
+    // search runs on the first call with new parameters (it synchronizes the stream and allocates, so not while the
+    // stream is being captured: such a call computes the sum operation by operation).  CHX_HIP_AFFINE_RESIDUAL=0
+    // keeps the operation-by-operation arithmetic everywhere.
+    {
+        chx_hip_qconv_plan* mp = const_cast<chx_hip_qconv_plan*>(plan);
+        ResidualAdd key;
+        memcpy(&key, &res, sizeof(key));  // byte copies: the comparison below is one of bytes, padding included
+        key.r = nullptr;
+        key.r_px_stride = 0;
+        key.r_vec_ok = 0;
+        const char* env = getenv("CHX_HIP_AFFINE_RESIDUAL");
+        const bool wanted = !(env && env[0] == '0');
+        if (wanted && mp->res_known && memcmp(&key, &mp->res_key, sizeof(key)) == 0) {
+            res.affine = mp->res_found.affine;
+            res.kc = mp->res_found.kc;
+            res.kr = mp->res_found.kr;
+            res.k0 = mp->res_found.k0;
+            res.floor_pre = mp->res_found.floor_pre;
+        } else if (wanted && !stream_is_capturing(s)) {
+            int32_t* counts = nullptr;
+            CHX_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&counts), kAffineCandidates * sizeof(int32_t)));
+            ResidualAdd found;
+            memcpy(&found, &key, sizeof(found));
+            const int rc = find_affine_residual(&found, counts, s);
+            (void)hipFree(counts);
+            CHX_PROPAGATE(rc);
+            memcpy(&mp->res_key, &key, sizeof(key));
+            memcpy(&mp->res_found, &found, sizeof(found));
+            mp->res_known = true;
+            res.affine = found.affine;
+            res.kc = found.kc;
+            res.kr = found.kr;
+            res.k0 = found.k0;
+            res.floor_pre = found.floor_pre;
+        }
+    }
     ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0);
     call.cache = const_cast<ScratchCache*>(&plan->scratch);
     call.tune = const_cast<TuneCache*>(&plan->tune);
@@ -996,6 +1037,7 @@ extern "C" int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char*
                  t.tile_oc, t.tile_px, t.max_wgs_per_cu, t.waves);
         text += line;
     }
+    if (plan->res_known) text += plan->res_found.affine ? "residual=affine\n" : "residual=exact\n";
     strncpy(buf, text.c_str(), buf_size - 1);
     buf[buf_size - 1] = 0;
     return CHX_HIP_OK;

@@ -85,6 +85,40 @@ __device__ __forceinline__ v4i add_residual16(v4i c, v4i r, const ResidualAdd& p
     return out;
 }
 
+// add_residual16 in the variant the parameters call for (the branches are uniform).
+__device__ __forceinline__ v4i add_residual16_any(v4i val, v4i rv, const ResidualAdd& p) {
+    if (p.lean) return p.guard ? add_residual16<true, true, true>(val, rv, p) : add_residual16<true, false, true>(val, rv, p);
+    if (p.guard) return p.out.lo == 0.f ? add_residual16<true, true>(val, rv, p) : add_residual16<false, true>(val, rv, p);
+    return p.out.lo == 0.f ? add_residual16<true, false>(val, rv, p) : add_residual16<false, false>(val, rv, p);
+}
+
+// The same sixteen codes from two fused multiply-adds per element (ResidualAdd::affine): with per-tensor scales
+// the group Q(act(DQ(c) + DQ(r))) is, in real arithmetic, floor(c*kc + r*kr + k0) saturated; in float32 the two
+// forms can differ where a sum falls within rounding distance of a code boundary, so this one is used only with
+// constants for which find_affine_residual has compared it with add_residual16 on every pair of codes.  Five
+// vector instructions per element instead of twelve.  kFloor: a Relu with a non-zero zero point of the sum (the
+// saturation at 0 is the Relu otherwise).
+template <bool kFloor>
+__device__ __forceinline__ v4i affine_residual16(v4i c, v4i r, const ResidualAdd& p) {
+    float pre[16];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t cw = (uint32_t)c[w] ^ p.c_flip, rw = (uint32_t)r[w] ^ p.r_flip;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float cf = (float)((cw >> (8 * e)) & 0xffu);
+            const float rf = (float)((rw >> (8 * e)) & 0xffu);
+            float t = __builtin_fmaf(rf, p.kr, p.k0);
+            t = __builtin_fmaf(cf, p.kc, t);
+            if (kFloor) t = __builtin_fmaxf(t, p.floor_pre);
+            pre[w * 4 + e] = t;
+        }
+    }
+    uint32_t words[4];
+    floor_sat_u8x16(pre, words);
+    return v4i{(int)words[0], (int)words[1], (int)words[2], (int)words[3]};
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");

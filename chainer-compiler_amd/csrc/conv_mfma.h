@@ -28,7 +28,15 @@ struct ResidualAdd {
     float big;             // 2^40 * out.scale: the dividend is limited to +-big (both sides saturate beyond)
     int32_t guard;         // 0 when the operand scales already keep every sum far inside +-big
     int32_t lean;          // uint8 result with zero point 0 and r with zero point 0: see add_residual16
+    // The sum as two fused multiply-adds, floor((c * kc + (r * kr + k0))) saturated to [0, 255] (and not below
+    // floor_pre when a Relu is part of the group): set only after find_affine_residual has found constants for which
+    // this gives the byte of the operation-by-operation arithmetic for every one of the 65536 pairs of codes.
+    int32_t affine;
+    float kc, kr, k0, floor_pre;
 };
+
+// Number of constant triples find_affine_residual tries: the float32 neighbours of the real-valued constants.
+constexpr int kAffineCandidates = 5 * 5 * 13;
 
 struct ConvMfmaArgs {
     // activations, channels-last: element (n, c, ih, iw) at x + n*x_n_stride + ih*x_h_stride + iw*x_w_stride + c
@@ -119,6 +127,13 @@ int pack_weights_stem(const chx_hip_tensor& w, int OCpad64, int8_t* wd, hipStrea
 int launch_conv_stem(ConvStemArgs a, bool rne, hipStream_t s);
 // max_wgs_per_cu caps the persistent grid (0: as many work-groups as the device holds at once); waves: 4, or 8
 // for the tiles 128x128, 128x256 and 64x128 (output channels x pixels)
+// Looks for constants (kc, kr, k0) with which the two-multiply-add form of the residual sum equals the
+// operation-by-operation one on all 65536 code pairs: every candidate is checked on the device against
+// add_residual16, the mismatch counts come back to the host (synchronizes the stream).  Returns CHX_HIP_OK and sets
+// p->affine (1 when a candidate without mismatch exists; then kc, kr, k0, floor_pre are filled in).  Only for uint8
+// sums without the range guard; otherwise p->affine stays 0.  `scratch` holds kAffineCandidates int32 on the device.
+int find_affine_residual(ResidualAdd* p, int32_t* scratch, hipStream_t s);
+
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, int waves, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s);
 

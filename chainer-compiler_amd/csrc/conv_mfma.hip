@@ -27,7 +27,9 @@
 // and written as 128-bit stores to the channels-last output; optionally the residual sum of
 // the element-wise group behind the convolution (ResidualAdd).  With an int32 output
 // (ConvInteger, MatMulInteger) the accumulators are stored directly.
+#include <cmath>
 #include <type_traits>
+#include <vector>
 
 #include "contract.h"
 #include "conv_mfma.h"
@@ -674,12 +676,9 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                         rv[w] = (int)word;
                     }
                 }
-                if (a.res.lean)
-                    val = a.res.guard ? add_residual16<true, true, true>(val, rv, a.res) : add_residual16<true, false, true>(val, rv, a.res);
-                else if (a.res.guard)
-                    val = a.res.out.lo == 0.f ? add_residual16<true, true>(val, rv, a.res) : add_residual16<false, true>(val, rv, a.res);
-                else
-                    val = a.res.out.lo == 0.f ? add_residual16<true, false>(val, rv, a.res) : add_residual16<false, false>(val, rv, a.res);
+                if (a.res.affine == 1) val = affine_residual16<false>(val, rv, a.res);
+                else if (a.res.affine == 2) val = affine_residual16<true>(val, rv, a.res);
+                else val = add_residual16_any(val, rv, a.res);
                 if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
             }
             char* dst = a.y + m * a.y_px_stride + oc;
@@ -842,6 +841,95 @@ int launch_im2col_dense(const Im2colArgs& a, hipStream_t s) {
     }
     im2col_dense_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a);
     return launch_check("im2col_dense_kernel");
+}
+
+namespace {
+
+// One work-group per candidate, one thread per residual code r, all 256 convolution codes c in turn (sixteen at a
+// time, as the epilogue processes them): counts the pairs on which the two forms differ.
+__global__ __launch_bounds__(256) void affine_residual_search_kernel(ResidualAdd exact, const float* __restrict__ cand, int32_t* __restrict__ mismatches) {
+    ResidualAdd p = exact;
+    p.kc = cand[blockIdx.x * 3 + 0];
+    p.kr = cand[blockIdx.x * 3 + 1];
+    p.k0 = cand[blockIdx.x * 3 + 2];
+    const uint32_t r = threadIdx.x;
+    const v4i rw = {(int)(r * 0x01010101u), (int)(r * 0x01010101u), (int)(r * 0x01010101u), (int)(r * 0x01010101u)};
+    int bad = 0;
+    for (uint32_t c0 = 0; c0 < 256; c0 += 16) {
+        v4i cw;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t b = c0 + 4 * w;
+            cw[w] = (int)(b | ((b + 1) << 8) | ((b + 2) << 16) | ((b + 3) << 24));
+        }
+        const v4i want = add_residual16_any(cw, rw, exact);
+        const v4i got = exact.affine == 2 ? affine_residual16<true>(cw, rw, p) : affine_residual16<false>(cw, rw, p);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) bad |= want[w] != got[w] ? 1 : 0;
+    }
+    const int total = __syncthreads_count(bad);  // threads (residual codes) with a difference anywhere
+    if (threadIdx.x == 0) mismatches[blockIdx.x] = total;
+}
+
+}  // namespace
+
+int find_affine_residual(ResidualAdd* p, int32_t* scratch, hipStream_t s) {
+    p->affine = 0;
+    // uint8 sums only (the floor-mode conversion saturates to [0, 255]); with the range guard active the scales are
+    // extreme and the sum stays with the guarded arithmetic
+    if (p->out.lo != 0.f || p->guard) return CHX_HIP_OK;
+    const double so = (double)p->out.scale;
+    const double kc = (double)p->c_scale / so, kr = (double)p->r_scale / so;
+    const double k0 = -(double)p->c_zpf * kc - (double)p->r_zpf * kr + (double)p->out.zpf + 0.5;
+    if (!(fabs(kc) < 1e6 && fabs(kr) < 1e6 && fabs(k0) < 1e6)) return CHX_HIP_OK;
+    const int mode = (p->relu && p->out.zpf != 0.f) ? 2 : 1;
+    std::vector<float> cand((size_t)kAffineCandidates * 3);
+    auto step = [](float x, int n) {
+        for (int i = 0; i < (n < 0 ? -n : n); ++i) x = nextafterf(x, n > 0 ? INFINITY : -INFINITY);
+        return x;
+    };
+    int idx = 0;
+    // nearest neighbours first: the order of preference
+    static const int order5[5] = {0, -1, 1, -2, 2};
+    static const int order13[13] = {0, -1, 1, -2, 2, -3, 3, -4, 4, -5, 5, -6, 6};
+    for (int a = 0; a < 5; ++a)
+        for (int b = 0; b < 5; ++b)
+            for (int c = 0; c < 13; ++c) {
+                cand[idx * 3 + 0] = step((float)kc, order5[a]);
+                cand[idx * 3 + 1] = step((float)kr, order5[b]);
+                cand[idx * 3 + 2] = step((float)k0, order13[c]);
+                ++idx;
+            }
+    float* dcand = nullptr;
+    CHX_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&dcand), cand.size() * sizeof(float)));
+    ResidualAdd probe = *p;
+    probe.affine = mode;
+    probe.floor_pre = p->out.zpf + 0.5f;
+    int rc = CHX_HIP_OK;
+    std::vector<int32_t> bad((size_t)kAffineCandidates, 1);
+    if (hipMemcpyAsync(dcand, cand.data(), cand.size() * sizeof(float), hipMemcpyHostToDevice, s) != hipSuccess) rc = CHX_HIP_ERUNTIME;
+    if (rc == CHX_HIP_OK) {
+        affine_residual_search_kernel<<<kAffineCandidates, 256, 0, s>>>(probe, dcand, scratch);
+        rc = launch_check("affine_residual_search_kernel");
+    }
+    if (rc == CHX_HIP_OK && (hipMemcpyAsync(bad.data(), scratch, bad.size() * sizeof(int32_t), hipMemcpyDeviceToHost, s) != hipSuccess ||
+                             hipStreamSynchronize(s) != hipSuccess))
+        rc = CHX_HIP_ERUNTIME;
+    (void)hipFree(dcand);
+    if (rc != CHX_HIP_OK) {
+        (void)hipGetLastError();
+        CHX_FAIL(rc, "checking the two-multiply-add form of a residual sum failed");
+    }
+    for (int i = 0; i < kAffineCandidates; ++i)
+        if (bad[i] == 0) {
+            p->affine = mode;
+            p->kc = cand[i * 3 + 0];
+            p->kr = cand[i * 3 + 1];
+            p->k0 = cand[i * 3 + 2];
+            p->floor_pre = probe.floor_pre;
+            break;
+        }
+    return CHX_HIP_OK;
 }
 
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, int waves, bool x_unsigned, bool out_int32, bool rne,

@@ -183,15 +183,22 @@ int chx_hip_qconv_plan_run(
         int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream);
 /* The launch configurations the plan has measured so far, as text into buf (truncated to buf_size - 1
  * characters): one "M=<output pixels> <OH>x<OW> res=<0|1> tile=<oc>x<px> wgs_per_cu=<n, 0 = as many as fit>"
- * per line (followed by "waves=<4|8>", the wavefronts per work-group); empty for a plan that does not run on the matrix-core kernel or has not run eagerly yet.  No
- * counterpart in the reference; benchmarks report it next to their timings. */
+ * per line (followed by "waves=<4|8>", the wavefronts per work-group), and after a chx_hip_qconv_plan_run_add a line
+ * "residual=affine" or "residual=exact" (which arithmetic the fused sum uses, see there); empty for a plan that
+ * does not run on the matrix-core kernel or has not run eagerly yet.  No counterpart in the reference; benchmarks
+ * report it next to their timings. */
 int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_t buf_size);
 /* A QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94) whose only reader is the
  * element-wise group  QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r)))  of a
  * residual block (ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161, act = Relu or
  * nothing), run as one kernel: the convolution's 8-bit result y (type y_dtype, quantization
- * y_scale / y_zero_point) is never written, `out` receives the group's result, computed operation
- * by operation as the two ops would.  r and out: same shape as y, channels-last, uint8 or int8.
+ * y_scale / y_zero_point) is never written, `out` receives the group's result, the bytes the two ops
+ * give.  The sum is computed operation by operation as the ops would; for a uint8 result the first
+ * call with new parameters (outside stream capture; it synchronizes the stream) also looks for
+ * constants with which floor(y*kc + (r*kr + k0)), two fused multiply-adds, gives the same byte as that
+ * arithmetic on every one of the 65536 pairs of codes, checks each candidate on the device against
+ * the arithmetic itself, and uses the short form from then on if one passes (CHX_HIP_AFFINE_RESIDUAL=0
+ * in the environment keeps the long one).  r and out: same shape as y, channels-last, uint8 or int8.
  * `out` must not overlap x or r in memory (the first call on a new shape may run the kernel several
  * times on the call's operands to pick a launch configuration): CHX_HIP_EINVAL when it does.
  * CHX_HIP_EUNSUPPORTED when the plan's weights or the layouts do not fit the matrix-core kernel;

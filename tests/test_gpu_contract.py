@@ -370,10 +370,15 @@ def _residual_sum(oracle, c, c_scale, c_zp, r, r_scale, r_zp, relu, out_scale, o
 @pytest.mark.parametrize("case", [
     # N, C, H, W, OC, K, stride, pad
     (2, 64, 9, 10, 256, 1, 1, 0), (1, 32, 7, 7, 24, 1, 1, 0), (2, 16, 8, 8, 70, 3, 1, 1), (1, 128, 6, 5, 128, 1, 2, 0)])
-def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
+@pytest.mark.parametrize("form", ["searched", "exact"])
+def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt, form, monkeypatch):
     """chx_hip_qconv_plan_run_add against QLinearConv followed by the element-wise group, each on
     the CPU oracle: with and without Relu, all type combinations, channel counts that leave partial
-    16-byte chunks, a residual with a padded pixel pitch."""
+    16-byte chunks, a residual with a padded pixel pitch.  Once as the library runs it by default (a
+    uint8 sum in its two-multiply-add form wherever the plan's search finds constants that make it exact)
+    and once with the operation-by-operation arithmetic forced."""
+    if form == "exact":
+        monkeypatch.setenv("CHX_HIP_AFFINE_RESIDUAL", "0")
     N, C, H, W, OC, K, stride, pad = case
     rng = np.random.default_rng(61)
     x = rand_q(rng, (N, C, H, W), np.uint8)
@@ -411,6 +416,14 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
                                flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(g.to_channels_last(g.dev(r)), dtype=TDT[odt]))
             np.testing.assert_array_equal(g.host(got), want)
             assert want.min() < want.max()
+    # which arithmetic the last sum used is on record; an int8 sum always keeps the long form
+    forms = [l for l in plan.describe() if l.startswith("residual=")]
+    if form == "exact":
+        assert forms == []                    # no search was made
+    else:
+        assert forms and forms[-1] in ("residual=affine", "residual=exact")
+        if odt == np.int8:
+            assert forms[-1] == "residual=exact"
     # operands that are not channels-last are refused, not converted
     with pytest.raises(g.capi.ChxHipError) as e:
         plan.run_add(xd, 0.02, 101, ys, yz, g.dev(r), rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt],
@@ -423,6 +436,42 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt):
             plan.run_add(xd, 0.02, 101, ys, yz, rd, rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt], flags=g.capi.BIAS_ONNX_INT32, out=rd)
         assert e.value.code == g.capi.EINVAL and "overlaps" in str(e.value)
     plan.close()
+
+
+def test_residual_sum_in_two_multiply_adds_over_all_code_pairs(g, oracle):
+    """The short form of the fused sum, for the quantization parameters of the sixteen residual blocks of the
+    ResNet-50 benchmark network (as calibrated: scales from 0.13 to 750, convolution zero points around 130) and a
+    few others: a 1x1 convolution with identity weights passes every code c through, so one call per parameter set
+    puts all 65536 (c, r) pairs through the kernel's epilogue, compared with the oracle's three ops.  The plan must
+    find constants for most of them (the search is exhaustive over the pairs, so a found form is exact by
+    construction; this test checks that through the kernel, and that the search is not vacuous)."""
+    params = [(0.21131895, 122, 0.1626821, 130, 0.12926471, 0), (0.3873351, 147, 0.12926471, 0, 0.18676299, 0),
+              (0.8456785, 137, 0.754098, 123, 0.51624763, 0), (1.5676626, 134, 0.51624763, 0, 1.0724535, 0),
+              (14.470264, 128, 4.5852566, 0, 7.2227073, 0), (272.5226, 138, 273.2742, 117, 164.99017, 0),
+              (746.74634, 141, 256.19128, 0, 383.77518, 0), (0.05, 120, 0.03, 7, 0.04, 33), (0.011, 0, 0.5, 255, 0.07, 250),
+              (1.0, 128, 1.0, 128, 1.0, 0), (0.3, 3, 0.3, 3, 0.1, 0)]
+    # x: 256 pixels x 256 channels, pixel p holds code p in every channel... the convolution must reproduce c exactly:
+    # identity weights with scale 1, x_scale = y_scale, equal zero points -> y code == x code
+    C = 64
+    w = np.zeros((C, C, 1, 1), np.int8)
+    w[np.arange(C), np.arange(C), 0, 0] = 1
+    ws, wz = np.ones(C, np.float32), np.zeros(C, np.int8)
+    codes = np.arange(256, dtype=np.uint8)
+    x = np.broadcast_to(codes.reshape(1, 1, 256, 1), (1, C, 256, 256 // 1)).copy()      # c varies along H
+    r = np.broadcast_to(codes.reshape(1, 1, 1, 256), (1, C, 256, 256)).copy()           # r varies along W
+    found = 0
+    for cs, cz, rs, rz, os_, oz in params:
+        for relu in (True, False):
+            plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), None)
+            xd, rd = g.to_channels_last(g.dev(x)), g.to_channels_last(g.dev(r))
+            conv = oracle.qlinear_conv_int(x, np.float32(cs), cz, w, ws, wz, np.float32(cs), cz, np.uint8)
+            np.testing.assert_array_equal(conv, x)
+            want = _residual_sum(oracle, conv, np.float32(cs), cz, r, np.float32(rs), rz, relu, np.float32(os_), oz, np.uint8)
+            got = plan.run_add(xd, cs, cz, cs, cz, rd, rs, rz, os_, oz, relu, zero_point_dtype=torch.uint8, out=torch.zeros_like(rd))
+            np.testing.assert_array_equal(g.host(got), want, err_msg=str((cs, cz, rs, rz, os_, oz, relu)))
+            found += "residual=affine" in plan.describe()
+            plan.close()
+    assert found >= len(params)       # of 2 * len(params) sums
 
 
 @pytest.mark.parametrize("tile", [(128, 128, 4), (64, 128, 4), (128, 64, 4), (64, 64, 4), (128, 128, 8), (128, 256, 8), (64, 128, 8)])
