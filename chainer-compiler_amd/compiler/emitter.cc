@@ -322,6 +322,26 @@ private:
                 inst->output_names.push_back("");
                 inst->output_types.push_back(ChxVMTypeProto());
             }
+        } else if ((op == "GlobalMaxPool" || op == "GlobalAveragePool") && nin == 1) {
+            // ReplaceGlobalPool, compiler/simplifier.cc:272-290: the pool whose window is the input's spatial extent
+            const Type& t = n.input(0)->type();
+            bool known = t.has_dims;
+            for (int64_t d : t.dims) known = known && d > 0;
+            CHECK(known) << "The input shape of " << op << " must be known";
+            CHECK_LT(2u, t.dims.size()) << "The input of " << op << " must have at least 3 dimensions";
+            const std::vector<int64_t> kernel(t.dims.begin() + 2, t.dims.end());
+            const std::vector<int64_t> ones(kernel.size(), 1), zeros(kernel.size(), 0);
+            ChxVMInstructionProto* inst;
+            if (op == "GlobalMaxPool") {
+                inst = simple("MaxPool", {ArrayIn(Operand(n, 0)), IntsIn(kernel), IntsIn(ones), IntsIn(zeros), IntIn(0), StringIn("NOTSET")});
+            } else {
+                inst = simple("AveragePool", {ArrayIn(Operand(n, 0)), IntsIn(kernel), IntsIn(ones), IntsIn(zeros), IntIn(0)});
+            }
+            inst->outputs.push_back(-1);
+            if (!inst->output_names.empty()) {
+                inst->output_names.push_back("");
+                inst->output_types.push_back(ChxVMTypeProto());
+            }
         } else if (op == "Clip" && nin >= 1 && nin <= 3) {
             // compiler/chxvm/simple_node_emitter.cc:506-512: bounds as attributes or as operands
             if (nin == 1) {

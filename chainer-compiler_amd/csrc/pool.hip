@@ -267,13 +267,58 @@ __global__ __launch_bounds__(kThreads) void global_average_pool_cl4_kernel(AvgAr
     *reinterpret_cast<uint32_t*>(p.y + n * p.ys[0] + c) = pack4(code[0], code[1], code[2], code[3]);
 }
 
+// The float32 pools of MaxPoolOp / AveragePoolOp::RunImpl (runtime/ops/pooling.cc:47-75), for the float layers
+// that stay around a quantized network: one lane = one output element, any strides, the taps in (kh, kw)
+// order.  max: padding never wins, a window in the padding altogether gives the lowest finite float.  average:
+// one float32 addition per tap that lies in the image, starting from 0, divided by the taps that count.
+template <bool kMax>
+__global__ __launch_bounds__(kThreads) void pool_f32_kernel(PoolArgs a, int count_include_pad) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= a.total) return;
+    // the unit-stride axis of y fastest, so that neighbouring lanes write neighbouring floats
+    const bool channels_fastest = a.ys[1] == 4;
+    int c, ow, oh, n;
+    int64_t r = idx;
+    if (channels_fastest) {
+        c = (int)(r % a.C); r /= a.C;
+        ow = (int)(r % a.OW); r /= a.OW;
+        oh = (int)(r % a.OH);
+        n = (int)(r / a.OH);
+    } else {
+        ow = (int)(r % a.OW); r /= a.OW;
+        oh = (int)(r % a.OH); r /= a.OH;
+        c = (int)(r % a.C);
+        n = (int)(r / a.C);
+    }
+    float acc = kMax ? -3.402823466e+38f : 0.f;
+    int cnt = 0;
+    for (int i = 0; i < a.kh; ++i) {
+        const int ih = oh * a.sh - a.ph + i;
+        if ((unsigned)ih >= (unsigned)a.H) continue;
+        for (int j = 0; j < a.kw; ++j) {
+            const int iw = ow * a.sw - a.pw + j;
+            if ((unsigned)iw >= (unsigned)a.W) continue;
+            const float v = *reinterpret_cast<const float*>(a.x + n * a.xs[0] + c * a.xs[1] + ih * a.xs[2] + iw * a.xs[3]);
+            if (kMax) acc = v > acc ? v : acc;
+            else acc = acc + v;
+            ++cnt;
+        }
+    }
+    if (!kMax) {
+        if (count_include_pad) cnt = a.kh * a.kw;
+        acc = acc / (float)cnt;
+    }
+    *reinterpret_cast<float*>(a.y + n * a.ys[0] + c * a.ys[1] + oh * a.ys[2] + ow * a.ys[3]) = acc;
+}
+
 int fill_pool_args(
         const chx_hip_tensor* x, chx_hip_tensor* y, int kh, int kw, int sh, int sw, int ph0, int pw0, int ph1, int pw1,
-        int cover_all, const char* op, PoolArgs* a) {
+        int cover_all, const char* op, PoolArgs* a, bool float32 = false) {
     CHX_PROPAGATE(check_tensor(x, op));
     CHX_PROPAGATE(check_tensor(y, op));
     CHX_REQUIRE(x->ndim == 4 && y->ndim == 4, "%s: x and y must be 4-D", op);
-    CHX_REQUIRE(is_q8(x->dtype) && is_q8(y->dtype), "%s: x and y must be uint8 or int8", op);
+    if (float32) CHX_REQUIRE(x->dtype == CHX_HIP_FLOAT32 && y->dtype == CHX_HIP_FLOAT32, "%s: x and y must be float32", op);
+    else CHX_REQUIRE(is_q8(x->dtype) && is_q8(y->dtype), "%s: x and y must be uint8 or int8", op);
     CHX_REQUIRE(kh >= 1 && kw >= 1 && sh >= 1 && sw >= 1 && ph0 >= 0 && pw0 >= 0 && ph1 >= 0 && pw1 >= 0,
                 "%s: bad kernel, stride or padding", op);
     const int64_t H = x->shape[2], W = x->shape[3];
@@ -368,4 +413,26 @@ extern "C" int chx_hip_average_pool_q8(
     else
         average_pool_kernel<false><<<blocks, kThreads, 0, s>>>(a);
     return launch_check("average_pool_kernel");
+}
+
+extern "C" int chx_hip_max_pool_f32(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+        int32_t pad_h_begin, int32_t pad_w_begin, int32_t pad_h_end, int32_t pad_w_end, int32_t cover_all,
+        chx_hip_tensor* y, void* stream) {
+    PoolArgs a;
+    CHX_PROPAGATE(fill_pool_args(x, y, kernel_h, kernel_w, stride_h, stride_w, pad_h_begin, pad_w_begin, pad_h_end,
+                                 pad_w_end, cover_all, "MaxPool", &a, true));
+    if (a.total == 0) return CHX_HIP_OK;
+    pool_f32_kernel<true><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, as_stream(stream)>>>(a, 0);
+    return launch_check("pool_f32_kernel");
+}
+
+extern "C" int chx_hip_average_pool_f32(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w, int32_t pad_h,
+        int32_t pad_w, int32_t count_include_pad, chx_hip_tensor* y, void* stream) {
+    PoolArgs a;
+    CHX_PROPAGATE(fill_pool_args(x, y, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, 0, "AveragePool", &a, true));
+    if (a.total == 0) return CHX_HIP_OK;
+    pool_f32_kernel<false><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, as_stream(stream)>>>(a, count_include_pad ? 1 : 0);
+    return launch_check("pool_f32_kernel");
 }

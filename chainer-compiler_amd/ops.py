@@ -296,6 +296,35 @@ def _pool_out(in_dim, p0, p1, k, s, cover_all):
     return (in_dim + p0 + p1 - k) // s + 1
 
 
+def MaxPool(x, kernel_shape, strides=(), pads=(), cover_all=False, out=None):
+    """MaxPoolOp::RunImpl on a float32 array, runtime/ops/pooling.cc:47-61 (the result; the op's second output,
+    the context for a backward pass, has no use in inference)."""
+    strides = _complement(strides, 2, 1)
+    pads = _complement(pads, 2, 0)
+    if out is None:
+        shape = (x.shape[0], x.shape[1], _pool_out(x.shape[2], pads[0], pads[0], kernel_shape[0], strides[0], cover_all),
+                 _pool_out(x.shape[3], pads[1], pads[1], kernel_shape[1], strides[1], cover_all))
+        out = _alloc_like_input_layout(x, shape, torch.float32)
+    capi.check(capi.lib().chx_hip_max_pool_f32(
+        capi.ref(x), _i(kernel_shape[0]), _i(kernel_shape[1]), _i(strides[0]), _i(strides[1]), _i(pads[0]), _i(pads[1]),
+        _i(pads[0]), _i(pads[1]), _i(1 if cover_all else 0), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
+def AveragePool(x, kernel_shape, strides=(), pads=(), count_include_pad=False, out=None):
+    """AveragePoolOp::RunImpl on a float32 array, runtime/ops/pooling.cc:63-75."""
+    strides = _complement(strides, 2, 1)
+    pads = _complement(pads, 2, 0)
+    if out is None:
+        shape = (x.shape[0], x.shape[1], _pool_out(x.shape[2], pads[0], pads[0], kernel_shape[0], strides[0], False),
+                 _pool_out(x.shape[3], pads[1], pads[1], kernel_shape[1], strides[1], False))
+        out = _alloc_like_input_layout(x, shape, torch.float32)
+    capi.check(capi.lib().chx_hip_average_pool_f32(
+        capi.ref(x), _i(kernel_shape[0]), _i(kernel_shape[1]), _i(strides[0]), _i(strides[1]), _i(pads[0]), _i(pads[1]),
+        _i(1 if count_include_pad else 0), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
 def MaxPoolQ8(x, kernel_shape, strides=(), pads=(), cover_all=False, out=None):
     """DequantizeLinear -> MaxPool (runtime/ops/pooling.cc:47-61) -> QuantizeLinear with equal
     quantization parameters, on the 8-bit codes: their maximum m for uint8, m + (m < 0) for int8 (the

@@ -119,6 +119,49 @@ private:
     int flag_;
 };
 
+// MaxPoolOp / AveragePoolOp::RunImpl on a float32 array (runtime/ops/pooling.cc:47-75) that is not between a
+// DequantizeLinear and a QuantizeLinear: operands as above.  The second output of the reference's ops, the opaque
+// context of a backward pass, is not produced; a program that reads it is refused when it is loaded.
+class FloatPoolOp : public ChxVMOp {
+public:
+    FloatPoolOp(const ChxVMInstructionProto& pool, bool is_max)
+        : ChxVMOp(pool), is_max_(is_max), x_(pool.inputs[0].array), y_(pool.outputs[0]), kernel_(pool.inputs[1].ints),
+          strides_(pool.inputs[2].ints), pads_(pool.inputs[3].ints), flag_(static_cast<int>(pool.inputs[4].i)) {
+        CHECK_EQ(2u, kernel_.size()) << "only 2-D pooling on the hip backend";
+        CHECK(pool.outputs.size() < 2 || pool.outputs[1] < 0) << "the backward context of a pool is not produced on the hip backend";
+        if (is_max) CHECK(pool.inputs[5].s.empty() || pool.inputs[5].s == "NOTSET") << "auto_pad is not supported for MaxPool on the hip backend";
+    }
+
+    void Run(ChxVMState* st) override {
+        if (st->trace_level()) std::cerr << (is_max_ ? "MaxPool" : "AveragePool") << "($" << x_ << ") -> $" << y_ << std::endl;
+        const chainerx::Array x = st->GetArray(x_);
+        CHECK_EQ(4, x.ndim());
+        CHECK(x.dtype() == chainerx::Dtype::kFloat32) << "a pool outside a DequantizeLinear / QuantizeLinear pair takes float32, not " << x.dtype();
+        const int kh = static_cast<int>(kernel_[0]), kw = static_cast<int>(kernel_[1]);
+        const int sh = strides_.empty() ? 1 : static_cast<int>(strides_[0]), sw = strides_.empty() ? 1 : static_cast<int>(strides_[1]);
+        int ph = 0, pw = 0;
+        if (pads_.size() >= 2) { ph = static_cast<int>(pads_[0]); pw = static_cast<int>(pads_[1]); }
+        if (pads_.size() == 4) CHECK(pads_[0] == pads_[2] && pads_[1] == pads_[3]) << "paddings for beginning and end must be the same";
+        const bool cover_all = is_max_ && flag_ != 0;
+        auto out_dim = [&](int64_t in, int k, int s, int p) { return cover_all ? (in + 2 * p - k + s - 1) / s + 1 : (in + 2 * p - k) / s + 1; };
+        const chainerx::Shape shape{x.shape()[0], x.shape()[1], out_dim(x.shape()[2], kh, sh, ph), out_dim(x.shape()[3], kw, sw, pw)};
+        chainerx::Array y = chainerx::Empty(shape, chainerx::Dtype::kFloat32);
+        chx_hip_tensor xt = x.hip(), yt = y.hip();
+        if (is_max_) {
+            CHXVM_HIP_CALL(chx_hip_max_pool_f32(&xt, kh, kw, sh, sw, ph, pw, ph, pw, cover_all ? 1 : 0, &yt, chainerx::CurrentStream()));
+        } else {
+            CHXVM_HIP_CALL(chx_hip_average_pool_f32(&xt, kh, kw, sh, sw, ph, pw, flag_, &yt, chainerx::CurrentStream()));
+        }
+        st->SetArray(y_, y);
+    }
+
+private:
+    bool is_max_;
+    int x_, y_;
+    std::vector<int64_t> kernel_, strides_, pads_;
+    int flag_;
+};
+
 // A QLinearConv whose result is read only by a residual-sum FusionGroup (and that group): the
 // convolution gets the chance to compute the group inside its kernel.  When it does, the group's
 // result is stored in the group's output slot now and the group instruction later does nothing;
@@ -372,6 +415,9 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         } else if (role[i] == 2) {
             program_.emplace_back(new FusedQLinearMatMulOp(inst, program.instructions[fused_inputs[i].first],
                                                            program.instructions[fused_inputs[i].second]));
+        } else if ((inst.op == kMaxPool || inst.op == kAveragePool) && inst.inputs.size() == (inst.op == kMaxPool ? 6u : 5u) &&
+                   inst.inputs[0].array >= 0 && !inst.outputs.empty()) {
+            program_.emplace_back(new FloatPoolOp(inst, inst.op == kMaxPool));
         } else {
             program_.emplace_back(MakeChxVMOp(inst));
         }

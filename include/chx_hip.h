@@ -257,6 +257,20 @@ int chx_hip_linear_f32(
         const chx_hip_tensor* x, const chx_hip_tensor* w, const chx_hip_tensor* b, int32_t n_batch_axes, chx_hip_tensor* y,
         void* stream);
 
+/* MaxPoolOp / AveragePoolOp::RunImpl on float32 arrays, runtime/ops/pooling.cc:47-75: [N,C,H,W] with any
+ * strides.  max: out extent with cover_all as in ChainerX (ceil instead of floor, plus one), taps in the
+ * padding never win, a window in the padding altogether gives the lowest finite float.  average: symmetric
+ * pads, the window's taps added in (kh, kw) order in float32 from 0, divided by kernel_h * kernel_w when
+ * count_include_pad and by the number of taps inside the image otherwise.  (The sum order and the padding value
+ * of ChainerX's own kernels are not in the reference tree.) */
+int chx_hip_max_pool_f32(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w,
+        int32_t pad_h_begin, int32_t pad_w_begin, int32_t pad_h_end, int32_t pad_w_end, int32_t cover_all,
+        chx_hip_tensor* y, void* stream);
+int chx_hip_average_pool_f32(
+        const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w, int32_t pad_h,
+        int32_t pad_w, int32_t count_include_pad, chx_hip_tensor* y, void* stream);
+
 /* ---- pooling on quantized tensors ------------------------------------------------------ */
 
 /* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized

@@ -32,6 +32,11 @@
  *                            ChainerX's Sigmoid routine is not in the tree.
  *   orc_tanh_f32/orc_exp_f32 call the host libm, as std::tanh/std::exp do in
  *                            ChainerX's native kernels.
+ *   orc_max_pool_f32         pinned: numpy restatement over an explicitly padded array (pads, strides,
+ *                            cover_all, whole-image window).
+ *   orc_average_pool_f32     pinned like orc_average_pool_q8 (tap-major numpy loop, both pad-count modes,
+ *                            integer-valued images where every sum is exact, the whole-image window against
+ *                            a sequential running sum); the same PARITY UNPINNED remainder.
  *   orc_gemm_f32             pinned for everything but the order of the fp32 sum:
  *                            float64 numpy within a bound from the row norms,
  *                            bit-equal on integer-valued operands (every sum
@@ -627,6 +632,54 @@ void orc_max_pool_q8(
                     ((uint8_t*)y)[(nc * OH + oh) * OW + ow] = (uint8_t)m;
             }
     }
+}
+
+/* MaxPoolOp / AveragePoolOp::RunImpl on float32 arrays (runtime/ops/pooling.cc:47-75), NCHW dense.
+ * max: padding never wins (a window in the padding altogether gives the lowest finite float, ChainerX's
+ * padding value as recalled); cover_all as above.  average: the window's taps in (kh, kw) order, one float32
+ * addition each starting from 0, divided by the number of taps that count (all kh*kw with count_include_pad,
+ * else those inside the image).  PARITY UNPINNED where orc_average_pool_q8 is: ChainerX's kernels are not in
+ * the tree. */
+void orc_max_pool_f32(
+        const float* x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph0,
+        int64_t pw0, int64_t ph1, int64_t pw1, int cover_all, float* y) {
+    const int64_t OH = pool_out_dim(H, ph0, ph1, kh, sh, cover_all), OW = pool_out_dim(W, pw0, pw1, kw, sw, cover_all);
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t nc = 0; nc < N * C; ++nc)
+        for (int64_t oh = 0; oh < OH; ++oh)
+            for (int64_t ow = 0; ow < OW; ++ow) {
+                float m = -3.402823466e+38f;
+                for (int64_t i = 0; i < kh; ++i)
+                    for (int64_t j = 0; j < kw; ++j) {
+                        const int64_t ih = oh * sh - ph0 + i, iw = ow * sw - pw0 + j;
+                        if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                        const float v = x[(nc * H + ih) * W + iw];
+                        if (v > m) m = v;
+                    }
+                y[(nc * OH + oh) * OW + ow] = m;
+            }
+}
+
+void orc_average_pool_f32(
+        const float* x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t ph,
+        int64_t pw, int count_include_pad, float* y) {
+    const int64_t OH = pool_out_dim(H, ph, ph, kh, sh, 0), OW = pool_out_dim(W, pw, pw, kw, sw, 0);
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t nc = 0; nc < N * C; ++nc)
+        for (int64_t oh = 0; oh < OH; ++oh)
+            for (int64_t ow = 0; ow < OW; ++ow) {
+                float sum = 0.f;
+                int32_t cnt = 0;
+                for (int64_t i = 0; i < kh; ++i)
+                    for (int64_t j = 0; j < kw; ++j) {
+                        const int64_t ih = oh * sh - ph + i, iw = ow * sw - pw + j;
+                        if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                        sum = sum + x[(nc * H + ih) * W + iw];
+                        ++cnt;
+                    }
+                if (count_include_pad) cnt = (int32_t)(kh * kw);
+                y[(nc * OH + oh) * OW + ow] = sum / (float)cnt;
+            }
 }
 
 void orc_average_pool_q8(

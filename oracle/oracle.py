@@ -398,6 +398,32 @@ def max_pool_q8(x, kernel, strides, pads=(0, 0), cover_all=False):
     return y
 
 
+def max_pool(x, kernel, strides, pads=(0, 0), cover_all=False):
+    """MaxPoolOp::RunImpl on float32, runtime/ops/pooling.cc:47-61."""
+    x = _c(x, np.float32)
+    N, C, H, W = x.shape
+    OH = pool_out_dim(H, pads[0], pads[0], kernel[0], strides[0], cover_all)
+    OW = pool_out_dim(W, pads[1], pads[1], kernel[1], strides[1], cover_all)
+    y = np.empty((N, C, OH, OW), dtype=np.float32)
+    i64 = ctypes.c_int64
+    lib().orc_max_pool_f32(_p(x), i64(N), i64(C), i64(H), i64(W), i64(kernel[0]), i64(kernel[1]), i64(strides[0]), i64(strides[1]),
+                           i64(pads[0]), i64(pads[1]), i64(pads[0]), i64(pads[1]), ctypes.c_int(int(cover_all)), _p(y))
+    return y
+
+
+def average_pool(x, kernel, strides, pads=(0, 0), count_include_pad=False):
+    """AveragePoolOp::RunImpl on float32, runtime/ops/pooling.cc:63-75."""
+    x = _c(x, np.float32)
+    N, C, H, W = x.shape
+    OH = pool_out_dim(H, pads[0], pads[0], kernel[0], strides[0])
+    OW = pool_out_dim(W, pads[1], pads[1], kernel[1], strides[1])
+    y = np.empty((N, C, OH, OW), dtype=np.float32)
+    i64 = ctypes.c_int64
+    lib().orc_average_pool_f32(_p(x), i64(N), i64(C), i64(H), i64(W), i64(kernel[0]), i64(kernel[1]), i64(strides[0]), i64(strides[1]),
+                               i64(pads[0]), i64(pads[1]), ctypes.c_int(int(count_include_pad)), _p(y))
+    return y
+
+
 def average_pool_q8(x, x_scale, x_zero_point, kernel, strides, pads, y_scale, y_zero_point, y_dtype=np.uint8,
                     count_include_pad=False, round_mode=ROUND_REFERENCE):
     x = _c(x)

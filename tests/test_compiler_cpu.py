@@ -395,3 +395,21 @@ def test_float_head_nodes_are_emitted_with_the_reference_operand_lists(vm):
     assert [v for _, v in g2[1][2:]] == [-1, 1.0, 1.0, 0, 0]          # no c: the optional operand is -1
     mm = next(i for i in insts if i[0] == "MatMul")
     assert [t for t, _ in mm[1]] == ["ARRAY", "ARRAY"]
+
+
+def test_global_pools_become_pools_over_the_spatial_extent(vm):
+    """ReplaceGlobalPool, compiler/simplifier.cc:272-290: kernel_shape = the input's spatial dimensions, which have to
+    be known; strides 1 and no padding are the pool nodes' defaults."""
+    N = onnx_lite.Node
+    m = model([N("GlobalAveragePool", ["x"], ["a"], {}), N("GlobalMaxPool", ["x"], ["y"], {})], [("x", (2, 8, 7, 5))],
+              [("a", (2, 8, 1, 1)), ("y", (2, 8, 1, 1))])
+    insts = decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))
+    avg = next(i for i in insts if i[0] == "AveragePool")
+    assert [t for t, _ in avg[1]] == ["ARRAY", "INTS", "INTS", "INTS", "INT"]
+    assert [list(v) if isinstance(v, (list, tuple)) else v for _, v in avg[1][1:]] == [[7, 5], [1, 1], [0, 0], 0]
+    mx = next(i for i in insts if i[0] == "MaxPool")
+    assert [list(v) if isinstance(v, (list, tuple)) else v for _, v in mx[1][1:]] == [[7, 5], [1, 1], [0, 0], 0, "NOTSET"]
+    assert avg[2][1] == -1 and mx[2][1] == -1          # the backward context is dropped
+    unknown = model([N("MaxPool", ["x"], ["h"], {"kernel_shape": [2, 2]}), N("GlobalAveragePool", ["h"], ["a"], {})], [("x", (2, 8, 7, 5))], [("a", (2, 8, 1, 1))])
+    with pytest.raises(vm.ChxVMError, match="shape of GlobalAveragePool must be known"):
+        vm.compile_onnx(unknown, {"fuse": "none"})

@@ -292,14 +292,30 @@ def test_residual_group_with_other_constants_runs_unfused(g, vm, oracle):
         np.testing.assert_array_equal(got, oracle.quantize_linear(s_, 0.3, 100, np.uint8))
 
 
-def test_unfused_pool_is_refused_at_load(g, vm):
+def test_unfused_pools_run_as_float_ops(g, vm, oracle):
+    """A MaxPool / AveragePool that is not between a DequantizeLinear and a QuantizeLinear is the float op of
+    runtime/ops/pooling.cc:47-75; asking for its backward context is refused when the program is loaded."""
+    rng = np.random.default_rng(21)
+    xv = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    b = vm.ProgramBuilder()
+    x = b.input("x", "float32", xv.shape)
+    y, a = b.new_slot(), b.new_slot()
+    b.add_raw("MaxPool", [("ARRAY", x), ("INTS", [3, 2]), ("INTS", [2, 2]), ("INTS", [1, 0]), ("INT", 1), ("STRING", "NOTSET")], [y, -1])
+    b.add_raw("AveragePool", [("ARRAY", x), ("INTS", [3, 3]), ("INTS", [2, 1]), ("INTS", [1, 1]), ("INT", 0)], [a, -1])
+    b.output("y", y)
+    b.output("a", a)
+    prog = vm.Program(b.serialize())
+    for xd in (g.dev(xv), g.to_channels_last(g.dev(xv))):
+        out = prog.run({"x": xd})
+        np.testing.assert_array_equal(out["y"], oracle.max_pool(xv, (3, 2), (2, 2), (1, 0), True))
+        np.testing.assert_array_equal(out["a"].view(np.int32), oracle.average_pool(xv, (3, 3), (2, 1), (1, 1), False).view(np.int32))
+    prog.close()
     b = vm.ProgramBuilder()
     x = b.input("x", "float32", (1, 1, 4, 4))
-    y = b.new_slot()
-    b.add_raw("MaxPool", [("ARRAY", x), ("INTS", [2, 2]), ("INTS", [2, 2]), ("INTS", [0, 0]), ("INT", 0), ("STRING", "NOTSET")],
-              [y, -1])
+    y, c = b.new_slot(), b.new_slot()
+    b.add_raw("MaxPool", [("ARRAY", x), ("INTS", [2, 2]), ("INTS", [2, 2]), ("INTS", [0, 0]), ("INT", 0), ("STRING", "NOTSET")], [y, c])
     b.output("y", y)
-    with pytest.raises(vm.ChxVMError, match="MaxPool"):
+    with pytest.raises(vm.ChxVMError, match="backward context"):
         vm.Program(b.serialize())
 
 

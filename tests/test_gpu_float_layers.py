@@ -110,6 +110,31 @@ def test_flatten(g, oracle):
         g.ops.Flatten(g.dev(x), 4)
 
 
+POOL_SHAPES = [
+    # N, C, H, W, kernel, strides, pads
+    (2, 16, 13, 12, (3, 3), (2, 2), (0, 0)), (1, 5, 9, 9, (2, 2), (2, 2), (1, 1)), (2, 3, 7, 7, (7, 7), (1, 1), (0, 0)),
+    (1, 4, 11, 10, (4, 5), (2, 3), (1, 2)), (3, 2, 6, 6, (1, 1), (2, 2), (0, 0)), (64, 8, 28, 28, (3, 3), (2, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", POOL_SHAPES, ids=lambda c: "x".join(str(v) for v in c[:4]) + "_k%dx%d" % c[4])
+def test_float_pools_through_the_c_abi(g, oracle, case):
+    """MaxPool (both cover_all settings) and AveragePool (both pad-count modes) on float32, NCHW and channels-last,
+    bit for bit against the oracle (the sum of a window is taken in the oracle's order)."""
+    N, C, H, W, kernel, strides, pads = case
+    rng = np.random.default_rng(H * 100 + W)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    for xd in (g.dev(x), g.to_channels_last(g.dev(x))):
+        for cover_all in (False, True):
+            got = g.host(g.ops.MaxPool(xd, kernel, strides, pads, cover_all))
+            np.testing.assert_array_equal(got, oracle.max_pool(x, kernel, strides, pads, cover_all))
+        for include_pad in (False, True):
+            got = g.host(g.ops.AveragePool(xd, kernel, strides, pads, include_pad))
+            np.testing.assert_array_equal(bits(got), bits(oracle.average_pool(x, kernel, strides, pads, include_pad)))
+    with pytest.raises(g.capi.ChxHipError, match="float32"):
+        g.ops.MaxPool(g.dev(np.zeros((1, 1, 4, 4), np.uint8)), (2, 2), out=torch.zeros((1, 1, 3, 3), dtype=torch.float32, device="cuda"))
+
+
 def test_float_layers_as_program_instructions(g, vm, oracle):
     """Flatten -> Gemm (Linear route) -> Relu -> MatMul -> Linear in one serialized program, against the
     oracle op by op."""

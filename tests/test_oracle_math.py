@@ -540,3 +540,63 @@ def test_flatten(oracle):
     # a channels-last view flattens in its logical (NCHW) order
     nhwc = np.ascontiguousarray(x.transpose(0, 2, 3, 1)).transpose(0, 3, 1, 2)
     np.testing.assert_array_equal(oracle.flatten(nhwc, 1), x.reshape(2, 60))
+
+
+# --- float pools (runtime/ops/pooling.cc:47-75) ---
+
+def np_max_pool_f32(x, kernel, strides, pads, cover_all):
+    N, C, H, W = x.shape
+    (kh, kw), (sh, sw), (ph, pw) = kernel, strides, pads
+    if cover_all:
+        OH, OW = -((H + 2 * ph - kh) // -sh) + 1, -((W + 2 * pw - kw) // -sw) + 1
+    else:
+        OH, OW = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    lowest = np.finfo(np.float32).min
+    PH, PW = (OH - 1) * sh + kh, (OW - 1) * sw + kw
+    pad = np.full((N, C, max(PH, H + 2 * ph), max(PW, W + 2 * pw)), lowest, np.float32)
+    pad[:, :, ph:ph + H, pw:pw + W] = x
+    out = np.full((N, C, OH, OW), lowest, np.float32)
+    for i in range(kh):
+        for j in range(kw):
+            out = np.maximum(out, pad[:, :, i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw])
+    return out
+
+
+@pytest.mark.parametrize("cover_all", [False, True])
+def test_float_max_pool_vs_numpy(oracle, cover_all):
+    rng = np.random.default_rng(61)
+    for kernel, strides, pads, H, W in POOL_CASES:
+        x = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+        np.testing.assert_array_equal(oracle.max_pool(x, kernel, strides, pads, cover_all), np_max_pool_f32(x, kernel, strides, pads, cover_all),
+                                      err_msg=str((kernel, strides, pads)))
+    x = rng.standard_normal((2, 3, 6, 5)).astype(np.float32)
+    np.testing.assert_array_equal(oracle.max_pool(x, (6, 5), (1, 1), (0, 0), cover_all).reshape(2, 3), x.max(axis=(2, 3)))
+
+
+@pytest.mark.parametrize("include_pad", [False, True])
+def test_float_average_pool_vs_numpy(oracle, include_pad):
+    rng = np.random.default_rng(62)
+    for kernel, strides, pads, H, W in POOL_CASES:
+        x = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+        (kh, kw), (sh, sw), (ph, pw) = kernel, strides, pads
+        OH, OW = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+        val = np.zeros((2, 3, H + 2 * ph, W + 2 * pw), np.float32)
+        val[:, :, ph:ph + H, pw:pw + W] = x
+        inside = np.zeros((H + 2 * ph, W + 2 * pw), np.int64)
+        inside[ph:ph + H, pw:pw + W] = 1
+        total = np.zeros((2, 3, OH, OW), np.float32)
+        count = np.zeros((OH, OW), np.int64)
+        for i in range(kh):                       # taps in (kh, kw) order, one float32 addition each; padding adds 0.0f
+            for j in range(kw):
+                total = total + val[:, :, i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw]
+                count = count + inside[i:i + (OH - 1) * sh + 1:sh, j:j + (OW - 1) * sw + 1:sw]
+        div = np.float32(kh * kw) if include_pad else count.astype(np.float32)
+        np.testing.assert_array_equal(oracle.average_pool(x, kernel, strides, pads, include_pad), total / div, err_msg=str((kernel, strides, pads)))
+    # integer-valued image: every sum is exact, so the mean is numpy's whatever the order
+    xi = rng.integers(-50, 51, size=(1, 2, 9, 9)).astype(np.float32)
+    got = oracle.average_pool(xi, (3, 3), (3, 3), (0, 0), include_pad)
+    np.testing.assert_array_equal(got, (xi.reshape(1, 2, 3, 3, 3, 3).transpose(0, 1, 2, 4, 3, 5).reshape(1, 2, 3, 3, 9).sum(axis=-1) / np.float32(9)).astype(np.float32))
+    # whole-image window: the sequential float32 running sum of the pixels in storage order
+    xg = rng.standard_normal((1, 2, 7, 7)).astype(np.float32)
+    seq = np.cumsum(xg.reshape(1, 2, 49), axis=-1, dtype=np.float32)[..., -1] / np.float32(49)
+    np.testing.assert_array_equal(oracle.average_pool(xg, (7, 7), (1, 1), (0, 0), include_pad).reshape(1, 2), seq)
