@@ -89,17 +89,20 @@ FM_FN float div_in_range(float n, float d) {
 // which changes no result).  Without it every multiply and add rounds on its own.
 // Over all 2^32 inputs the two groupings differ on exactly two, 0x4202422f and
 // 0xc27c65d9, which is how a host's variant can be told.
-template <bool kUseFma>
+// kNegate evaluates expf(-x) (the sigmoid's use) without spending an instruction on the sign.
+// (kd as one fused multiply-add and the cubic in Horner form also give the library's result for
+// every argument, but the device compiler spends more on placing their constants than they save.)
+template <bool kUseFma, bool kNegate = false>
 FM_FN float expf_faithful(float x) {
-    const fm_u32 ux = f2u(x);
-    const fm_u32 abstop = (ux >> 20) & 0x7ff;
+    const fm_u32 abstop = (f2u(x) >> 20) & 0x7ff;
     if (abstop >= 0x42b) {  // |x| >= 88 or NaN
-        if (ux == 0xff800000u) return 0.0f;
-        if (abstop >= 0x7f8) return x + x;
-        if (x > 0x1.62e42ep6f) return u2f(0x7f800000u);  // overflow
-        if (x < -0x1.9fe368p6f) return 0.0f;             // underflow
+        const float v = kNegate ? -x : x;
+        if (f2u(v) == 0xff800000u) return 0.0f;
+        if (abstop >= 0x7f8) return v + v;
+        if (v > 0x1.62e42ep6f) return u2f(0x7f800000u);  // overflow
+        if (v < -0x1.9fe368p6f) return 0.0f;             // underflow
     }
-    const double xd = (double)x;
+    const double xd = kNegate ? -(double)x : (double)x;
     const double InvLn2N = 0x1.71547652b82fep+0 * 32.0;
     const double Shift = 0x1.8p+52;
     const double C0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
@@ -217,12 +220,32 @@ FM_FN float expm1f_faithful(float x) {
 // tanhf, fdlibm, written without data-dependent branches so that a 64-wide wavefront
 // does not serialise the algorithm's many cases: every lane evaluates the one shared
 // expm1f core (argument reduction, polynomial, one division) on the argument its case
-// calls for, all reconstruction formulas, and selects.  Each selected value is produced
-// by exactly the operations fdlibm's tanhf -> expm1f performs for that input:
+// calls for, the reconstruction formulas, and selects:
 //   |x| >= 1 : t = expm1f( 2|x|), z = 1 - 2/(t+2)      (k = 3..63 in expm1f)
 //   |x| <  1 : t = expm1f(-2|x|), z = -t/(t+2)         (k = 0, -1, -2, -3)
 // with k*ln2_hi == +-ln2_hi exactly for k == +-1 and hi == x, lo == 0 for k == 0, so the
 // reduction needs no case split either.
+//
+// Where fdlibm's operation sequence can be shortened without changing the result for any of the
+// 2^32 arguments, it is: the checks named in the header comment compare this function with the C
+// library's tanhf over all of them, on the host and on the device, and each of the following was
+// added only after that comparison came out equal (and others were dropped because it did not:
+// contracting r1, t3, the divisor or e2 changes between 70 and 118718 results):
+//  * k = trunc(invln2*arg +- 0.5) as one fused multiply-add, and without expm1f's special cases
+//    for |arg| < 1.5 ln2 (k = +-1) and |arg| <= 0.5 ln2 (k = 0): the formula gives the same k;
+//  * hi = arg - k*ln2_hi contracted (k*ln2_hi is exact, so this cannot round differently), the
+//    four inner steps of the polynomial contracted, 0.5*(x - e) - 0.5 contracted (the product is
+//    exact);
+//  * for k == 0 the correction c is 0 and fdlibm's x - (x*e - hxs) is -(e2 - x) of the general
+//    path, operation for operation;
+//  * one reconstruction 2^k * (tb - (e - x)) with tb = 1 - 2^-k (1 where 2^-k is below half an ulp
+//    of 1, i.e. k > 24, and for k < 0), minus 1 for negative k.  That is fdlibm's formula for
+//    k <= -2 and for 1 < k < 23.  For k >= 23 fdlibm adds 2^-k last instead of first, or leaves it
+//    out (k > 56); there t is above 2^22 and 1 - 2/(t+2) does not resolve the difference;
+//  * |x| >= 22 and +-inf through the same arithmetic, the argument limited to 88 (k = 127, t about
+//    2^127, z = 1 exactly) instead of a select at the end;
+//  * |x| < 2^-55 (fdlibm: x*(1+x)), +-0 and expm1f's |arg| < 2^-25 through the general path, which
+//    returns the argument itself there; only NaN is selected separately.
 FM_FN float tanhf_faithful(float x) {
     const float one = 1.0f, two = 2.0f;
     const float ln2_hi = u2f(0x3f317180u);
@@ -234,71 +257,52 @@ FM_FN float tanhf_faithful(float x) {
     const float Q4 = u2f(0x36867e54u);
     const float Q5 = u2f(0xb457edbbu);
 
-    const fm_u32 jx = f2u(x);
-    const fm_u32 ix = jx & 0x7fffffffu;
+    const fm_u32 ix = f2u(x) & 0x7fffffffu;
     const float ax = u2f(ix);
     const bool big = ix >= 0x3f800000u;  // |x| >= 1
-    const float arg = big ? two * ax : -two * ax;
+    const float arg = __builtin_fminf(big ? two * ax : -two * ax, 88.0f);
 
     // expm1f(arg)
-    const fm_u32 hx = f2u(arg) & 0x7fffffffu;
-    fm_i32 k = (fm_i32)(invln2 * arg + (big ? 0.5f : -0.5f));
-    k = hx < 0x3F851592u ? (big ? 1 : -1) : k;  // |arg| < 1.5 ln2
-    k = hx > 0x3eb17218u ? k : 0;               // |arg| <= 0.5 ln2
+    const fm_i32 k = (fm_i32)__builtin_fmaf(invln2, arg, big ? 0.5f : -0.5f);
     const float tk = (float)k;
-    const float hi = arg - tk * ln2_hi;
+    const float hi = __builtin_fmaf(-tk, ln2_hi, arg);
     const float lo = tk * ln2_lo;
     const float xr = hi - lo;
     const float c = (hi - xr) - lo;
     const float hfx = 0.5f * xr;
     const float hxs = xr * hfx;
-    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    float p = __builtin_fmaf(hxs, Q5, Q4);
+    p = __builtin_fmaf(hxs, p, Q3);
+    p = __builtin_fmaf(hxs, p, Q2);
+    p = __builtin_fmaf(hxs, p, Q1);
+    const float r1 = one + hxs * p;
     const float t3 = 3.0f - r1 * hfx;
-    // 6 - xr*t3 is within a few percent of 6 and r1 - t3 of -2 for every finite argument (xr is the reduced
-    // argument, |xr| <= 0.35); a non-finite argument is replaced by its case's constant at the end
+    // 6 - xr*t3 is within a few percent of 6 and r1 - t3 of -2 (xr is the reduced argument, |xr| <= 0.35)
     const float e = hxs * div_in_range(r1 - t3, 6.0f - xr * t3);
-    const float y_k0 = xr - (xr * e - hxs);
     float e2 = (xr * (e - c) - c);
     e2 -= hxs;
-    const float y_km1 = 0.5f * (xr - e2) - 0.5f;
     const float emx = e2 - xr;
-    const fm_u32 kshift = (fm_u32)k << 23;
-    // k <= -2 or k > 56
-    float ya = one - emx;
-    ya = u2f(f2u(ya) + kshift);
-    ya = ya - one;
-    // 1 < k < 23
-    const float tb = u2f(0x3f800000u - (0x1000000u >> ((fm_u32)k & 31u)));
-    float yb = tb - emx;
-    yb = u2f(f2u(yb) + kshift);
-    // 23 <= k <= 56
-    const float tc = u2f((fm_u32)(0x7f - k) << 23);
-    float yc = xr - (e2 + tc);
-    yc += one;
-    yc = u2f(f2u(yc) + kshift);
-    float t = k < 23 ? yb : yc;
-    t = (k <= -2 || k > 56) ? ya : t;
-    t = k == -1 ? y_km1 : t;
-    t = k == 0 ? y_k0 : t;
-    t = hx < 0x33000000u ? arg : t;  // |arg| < 2^-25: expm1f returns its argument
+    const fm_u32 sh = (fm_u32)k < 31u ? (fm_u32)k : 31u;  // negative k: 31, tb = 1
+    const float tb = u2f(0x3f800000u - (0x1000000u >> sh));
+    float y = tb - emx;
+    y = u2f(f2u(y) + ((fm_u32)k << 23));
+    float t = big ? y : y - one;
+    t = k == -1 ? __builtin_fmaf(-0.5f, emx, -0.5f) : t;
+    t = k == 0 ? -emx : t;
 
-    // |x| >= 1: 2 / (t + 2) with t = expm1(2|x|) in [6.3, 1.3e19] while |x| < 22 (beyond, z is the constant
-    // below and what this division gives is not used); |x| < 1: t / (t + 2) with t in (-0.87, 0] and
-    // t + 2 in (1.13, 2], the quotient at least 2^-55 in magnitude where it is used
+    // |x| >= 1: 2 / (t + 2) with t = expm1(2|x|) in [6.3, 2^127]; |x| < 1: t / (t + 2) with t in (-0.87, 0] and
+    // t + 2 in (1.13, 2]
     const float q = div_in_range(big ? two : t, t + two);
-    float z = big ? one - q : -q;
-    z = ix >= 0x41b00000u ? one : z;           // |x| >= 22 (and +-inf): one - tiny
-    float r = (jx >> 31) == 0 ? z : -z;
-    r = ix < 0x24000000u ? x : r;              // |x| < 2^-55: x*(1+x) == x; also +-0
-    r = ix > 0x7f800000u ? x + x : r;          // NaN
-    return r;
+    const float z = big ? one - q : -q;  // z >= 0
+    const float r = __builtin_copysignf(z, x);
+    return ix > 0x7f800000u ? x : r;  // NaN
 }
 
 // ChainerX's Sigmoid routine as the oracle restates it: Reciprocal(1 + Exp(-x)),
 // one rounding per operation.
 template <bool kUseFma>
 FM_FN float sigmoid_faithful(float x) {
-    const float e = expf_faithful<kUseFma>(-x);
+    const float e = expf_faithful<kUseFma, true>(x);
     const float d = 1.0f + e;
     // d >= 1; beyond 2^125 (x < -86.6) the reciprocal approaches the denormal range and the plain division takes over
     if (d > 0x1p125f) return 1.0f / d;
