@@ -163,7 +163,9 @@ int float_value(const std::string& tok, float* value) {
 // Value kinds: 'f' float32 value, 'q' 8-bit code held in an int.
 int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* uses_exp_table) {
     std::map<std::string, char> kind;
-    os << "__device__ __forceinline__ void elem(";
+    // kFast: Exp and Sigmoid without their rare cases (arguments beyond +-88, quotients near the denormal range);
+    // `rare` comes back set when an element met one, and the caller evaluates it again with kFast = false
+    os << "template <bool kFast>\n__device__ __forceinline__ void elem(";
     bool first = true;
     for (const Port& p : prog.inputs) {
         CHX_REQUIRE(!kind.count(p.name), "fusion program: duplicate input '%s'", p.name.c_str());
@@ -173,7 +175,7 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
     }
     for (size_t i = 0; i < prog.outputs.size(); ++i)
         os << ", " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float& " : "int& ") << "o_" << i;
-    os << ") {\n";
+    os << ", bool& rare) {\n";
     const char* fma = use_fma ? "true" : "false";
     for (const Stmt& s : prog.stmts) {
         CHX_REQUIRE(!kind.count(s.out), "fusion program: '%s' assigned twice", s.out.c_str());
@@ -238,12 +240,14 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
         } else if (s.op == "Exp") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = chx_fm::expf_faithful<" << fma << ">(" << a << ");\n";
+            os << "  const float " << o << " = kFast ? chx_fm::expf_unless_rare<" << fma << ">(" << a << ", rare) : chx_fm::expf_faithful<"
+               << fma << ">(" << a << ");\n";
             *uses_exp_table = true;
         } else if (s.op == "Sigmoid") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = chx_fm::sigmoid_faithful<" << fma << ">(" << a << ");\n";
+            os << "  const float " << o << " = kFast ? chx_fm::sigmoid_unless_rare<" << fma << ">(" << a
+               << ", rare) : chx_fm::sigmoid_faithful<" << fma << ">(" << a << ");\n";
             *uses_exp_table = true;
         } else if (s.op == "Relu") {
             CHX_PROPAGATE(need(1));
@@ -354,6 +358,7 @@ int generate_source(
     os << "#define FM_FN __device__ __forceinline__\n";
     os << "#define FM_TABLE_QUALIFIER static __device__ const\n";
     os << "#define FM_DEVICE_DIV 1\n";
+    os << "#define FM_ANY_LANE(c) (__builtin_amdgcn_ballot_w64(c) != 0ull)\n";
     std::ostringstream body;
     bool uses_table = false;
     CHX_PROPAGATE(emit_elem(prog, use_fma, body, &uses_table));
@@ -418,10 +423,17 @@ int generate_source(
     }
     for (size_t i = 0; i < nout; ++i)
         os << "  " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float" : "int") << " y" << i << "[" << vec << "];\n";
-    os << "#pragma unroll\n  for (int e = 0; e < " << vec << "; ++e) elem(";
-    for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "x" << i << "[e]";
-    for (size_t i = 0; i < nout; ++i) os << ", y" << i << "[e]";
-    os << ");\n";
+    // all elements of the step without the rare cases first, one wavefront-wide test, and again in full if any lane
+    // met one: a branch per element costs more than the rare cases' few instructions
+    os << "  bool rare = false;\n";
+    for (int fast = 1; fast >= 0; --fast) {
+        if (!fast) os << "  if (__builtin_expect(FM_ANY_LANE(rare), 0)) {\n";
+        os << "#pragma unroll\n  for (int e = 0; e < " << vec << "; ++e) elem<" << (fast ? "true" : "false") << ">(";
+        for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "x" << i << "[e]";
+        for (size_t i = 0; i < nout; ++i) os << ", y" << i << "[e]";
+        os << ", rare);\n";
+        if (!fast) os << "  }\n";
+    }
     for (size_t i = 0; i < nout; ++i) {
         if (prog.outputs[i].dtype == CHX_HIP_FLOAT32) {
             os << "  { v4f* dst = (v4f*)(o" << i << " + base);\n";
@@ -470,10 +482,10 @@ int generate_source(
     os << "    rest = q;\n  }\n";
     for (size_t i = 0; i < nout; ++i)
         os << "  " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float" : "int") << " r" << i << ";\n";
-    os << "  elem(";
+    os << "  bool rare = false;\n  elem<false>(";
     for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "i" << i << "[off[" << i << "]]";
     for (size_t i = 0; i < nout; ++i) os << ", r" << i;
-    os << ");\n";
+    os << ", rare);\n";
     for (size_t i = 0; i < nout; ++i) {
         if (prog.outputs[i].dtype == CHX_HIP_FLOAT32)
             os << "  o" << i << "[idx] = r" << i << ";\n";

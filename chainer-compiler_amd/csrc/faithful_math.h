@@ -27,11 +27,21 @@
 #define FM_FN inline
 #endif
 
+// FM_ANY_LANE(c): c for the calling lane; the run-time compiled device code defines it as "c holds for some lane
+// of the wavefront", which turns the rare-case tests below into branches that a wavefront takes as a whole.  A
+// guarded path therefore has to be right for every lane, not only for those with c (it is the complete routine;
+// the path behind it is the routine without the cases that c excludes).  Data-dependent branches cost this code far
+// more than their instruction count: expf alone over 2^26 floats takes 124 us with the per-lane test and 93 us without.
+#ifndef FM_ANY_LANE
+#define FM_ANY_LANE(c) (c)
+#endif
+
 namespace chx_fm {
 
 typedef unsigned int fm_u32;
 typedef unsigned long long fm_u64;
 typedef int fm_i32;
+typedef fm_u32 fm_u32x2 __attribute__((vector_size(8)));  // a 64-bit pattern as (low, high) words
 
 FM_FN fm_u32 f2u(float f) {
     return __builtin_bit_cast(fm_u32, f);
@@ -92,16 +102,17 @@ FM_FN float div_in_range(float n, float d) {
 // kNegate evaluates expf(-x) (the sigmoid's use) without spending an instruction on the sign.
 // (kd as one fused multiply-add and the cubic in Horner form also give the library's result for
 // every argument, but the device compiler spends more on placing their constants than they save.)
-template <bool kUseFma, bool kNegate = false>
-FM_FN float expf_faithful(float x) {
-    const fm_u32 abstop = (f2u(x) >> 20) & 0x7ff;
-    if (abstop >= 0x42b) {  // |x| >= 88 or NaN
-        const float v = kNegate ? -x : x;
-        if (f2u(v) == 0xff800000u) return 0.0f;
-        if (abstop >= 0x7f8) return v + v;
-        if (v > 0x1.62e42ep6f) return u2f(0x7f800000u);  // overflow
-        if (v < -0x1.9fe368p6f) return 0.0f;             // underflow
-    }
+//
+// The library tests the top 12 bits for |x| >= 88 or NaN (expf_far) and decides those arguments before the
+// arithmetic.  Here the arithmetic (expf_arith) runs for every lane (for such arguments on meaningless operands,
+// which it tolerates: the table index is masked, nothing traps) and the decided values replace its result
+// afterwards (expf_decided).
+FM_FN bool expf_far(float x) {
+    return !(__builtin_fabsf(x) < 88.0f);
+}
+
+template <bool kUseFma, bool kNegate>
+FM_FN float expf_arith(float x) {
     const double xd = kNegate ? -(double)x : (double)x;
     const double InvLn2N = 0x1.71547652b82fep+0 * 32.0;
     const double Shift = 0x1.8p+52;
@@ -113,12 +124,16 @@ FM_FN float expf_faithful(float x) {
     const fm_u64 ki = d2u(kd);
     kd = kd - Shift;
     const double r = kUseFma ? __builtin_fma(InvLn2N, xd, -kd) : z - kd;
-    fm_u64 t = kExp2fTab[ki & 31];
-    t += ki << 47;
-    const double s = u2d(t);
+    // t + (ki << 47): the sum only reaches the upper half, as (low word of ki) << 15
+    const fm_u64 t = kExp2fTab[ki & 31];
+    fm_u32x2 tw = __builtin_bit_cast(fm_u32x2, t);
+    tw[1] += (fm_u32)ki << 15;
+    const double s = __builtin_bit_cast(double, tw);
     double y;
     if (kUseFma) {
-        z = __builtin_fma(C0, r, C1);
+        // not fused, although the library's build fuses it: the result is the same for every argument, and a fused
+        // multiply-add with two constant operands makes the device compiler copy one of them into registers first
+        z = C0 * r + C1;
         const double r2 = r * r;
         y = __builtin_fma(C2, r, 1.0);
         y = __builtin_fma(z, r2, y);
@@ -130,6 +145,30 @@ FM_FN float expf_faithful(float x) {
     }
     y = y * s;
     return (float)y;
+}
+
+template <bool kNegate>
+FM_FN float expf_decided(float x, float res) {
+    const float v = kNegate ? -x : x;
+    float sp = v > 0.0f ? u2f(0x7f800000u) : 0.0f;   // overflow beyond 0x1.62e42ep6, underflow below -0x1.9fe368p6, +-inf
+    sp = (f2u(v) & 0x7fffffffu) > 0x7f800000u ? v + v : sp;  // NaN
+    const bool decided = expf_far(x) && (v > 0x1.62e42ep6f || v < -0x1.9fe368p6f || (f2u(v) & 0x7fffffffu) > 0x7f800000u);
+    return decided ? sp : res;
+}
+
+template <bool kUseFma, bool kNegate = false>
+FM_FN float expf_faithful(float x) {
+    float res = expf_arith<kUseFma, kNegate>(x);
+    if (__builtin_expect(FM_ANY_LANE(expf_far(x)), 0)) res = expf_decided<kNegate>(x, res);
+    return res;
+}
+
+// The same for callers that evaluate several elements before they branch: the result is the library's unless `rare`
+// comes back set, in which case the caller evaluates the element again with expf_faithful.
+template <bool kUseFma, bool kNegate = false>
+FM_FN float expf_unless_rare(float x, bool& rare) {
+    rare = rare || expf_far(x);
+    return expf_arith<kUseFma, kNegate>(x);
 }
 
 // expm1f, fdlibm.
@@ -305,7 +344,16 @@ FM_FN float sigmoid_faithful(float x) {
     const float e = expf_faithful<kUseFma, true>(x);
     const float d = 1.0f + e;
     // d >= 1; beyond 2^125 (x < -86.6) the reciprocal approaches the denormal range and the plain division takes over
-    if (d > 0x1p125f) return 1.0f / d;
+    if (__builtin_expect(FM_ANY_LANE(d > 0x1p125f), 0)) return 1.0f / d;
+    return div_in_range(1.0f, d);
+}
+
+// As expf_unless_rare: valid unless `rare` comes back set.
+template <bool kUseFma>
+FM_FN float sigmoid_unless_rare(float x, bool& rare) {
+    const float e = expf_unless_rare<kUseFma, true>(x, rare);
+    const float d = 1.0f + e;
+    rare = rare || d > 0x1p125f;
     return div_in_range(1.0f, d);
 }
 

@@ -84,6 +84,42 @@ def test_transcendentals_bit_exact_over_every_float(g, oracle, op):
         oracle.set_threads(1)
 
 
+@pytest.mark.parametrize("op", ["Exp", "Sigmoid", "chain"])
+@pytest.mark.parametrize("share", [0.0005, 0.02, 0.5])
+def test_rare_arguments_scattered_among_ordinary_ones(g, oracle, op, share):
+    """The kernels evaluate a step's elements without expf's out-of-range cases and the sigmoid's near-denormal
+    quotients first and repeat the step in full when any lane of the wavefront met one: so arguments of both kinds
+    share wavefronts here (a few, some, half of the lanes), in the vector kernel and in the strided one."""
+    rng = np.random.default_rng(int(share * 1e4) + len(op))
+    n = 1 << 18
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    rare = np.array([np.inf, -np.inf, np.nan, 88.0, -88.0, 88.5, 88.72283, 88.72284, 89.0, 100.0, 1e30, -86.6, -86.7, -87.0,
+                     -87.4, -88.0, -100.0, -103.9, -103.98, -104.5, -150.0, -1e30, 86.6, 87.0, 87.4, 103.9, 104.5],
+                    dtype=np.float32)
+    at = rng.random(n) < share
+    x[at] = rng.choice(rare, int(at.sum()))
+    if op == "chain":
+        c = x
+        xx = rng.standard_normal(n).astype(np.float32)
+        a, b = rng.standard_normal(256).astype(np.float32), rng.standard_normal(256).astype(np.float32)
+        xx2, c2 = xx.reshape(-1, 256), c.reshape(-1, 256)
+        want = oracle.run_chain(ORACLE_CHAIN, dict(x=xx2, a=a, b=b, c=c2))["y"]
+        got = g.host(g.ops.ElementWiseNvrtc([g.dev(xx2), g.dev(a), g.dev(b), g.dev(c2)], 1, chain_program(g.ops), 3)[0])
+        cases = [(got, want)]
+    else:
+        fn = {"Exp": oracle.exp, "Sigmoid": oracle.sigmoid}[op]
+        prog = unary_program(g.ops, op)
+        got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, prog)[0])
+        # every other element of a twice as long array: not contiguous, so the strided kernel runs
+        wide = g.dev(np.repeat(x, 2))
+        got2 = g.host(g.ops.ElementWiseNvrtc([wide[::2]], 1, prog)[0])
+        cases = [(got, fn(x)), (got2, fn(x))]
+    for got, want in cases:
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
 @pytest.mark.parametrize("shape,vec_shape", [((8, 64, 256), (256,)), ((3, 5, 7), (7,)), ((2, 1000), (1000,)),
                                             ((1, 4), (4,)), ((5,), (1,))])
 def test_chain_matches_oracle(g, oracle, shape, vec_shape):
