@@ -619,7 +619,18 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         // requantization instead of in front of every store.
         constexpr int ITER = TN * OUT_CHUNKS / T;
         v4i rres[ITER];
-        if (kRes) {
+        // A tile that lies inside the output altogether, with 16-byte accesses allowed, needs no test per lane
+        // (the operands of this test are the same for the whole work-group); per-lane branches in the loops
+        // below cost far more than the instructions they skip.
+        // (in 32-bit scalar terms: every pixel tile but the last is full, and the last one is when TN divides M)
+        const bool tile_inside = (px_tile + 1 < a.tiles_px || a.M % TN == 0) && oc0 + TM <= a.OC && a.y_vec_ok && (!kRes || a.res.r_vec_ok);
+        if (kRes && tile_inside) {
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                const int q = tid + it * T;
+                rres[it] = *reinterpret_cast<const v4i*>(a.res.r + (m0 + q / OUT_CHUNKS) * a.res.r_px_stride + oc0 + (q % OUT_CHUNKS) * 16);
+            }
+        } else if (kRes) {
 #pragma unroll
             for (int it = 0; it < ITER; ++it) {
                 const int q = tid + it * T;
@@ -653,6 +664,27 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
             }
         }
         __syncthreads();
+        if (tile_inside) {
+            auto store_all = [&](auto mode_tag) {
+                constexpr int kMode = decltype(mode_tag)::value;  // 0: no residual, 1 / 2: the two-multiply-add forms, 3: the exact chain
+#pragma unroll
+                for (int it = 0; it < ITER; ++it) {
+                    const int q = tid + it * T;
+                    const int pxl = q / OUT_CHUNKS;
+                    const int ch = q % OUT_CHUNKS;
+                    v4i val = *reinterpret_cast<const v4i*>(staged(lds_out, pxl, ch * 16));
+                    if constexpr (kMode == 1) val = affine_residual16<false>(val, rres[it], a.res);
+                    if constexpr (kMode == 2) val = affine_residual16<true>(val, rres[it], a.res);
+                    if constexpr (kMode == 3) val = add_residual16_any(val, rres[it], a.res);
+                    *reinterpret_cast<v4i*>(a.y + (m0 + pxl) * a.y_px_stride + oc0 + ch * 16) = val;
+                }
+            };
+            if (!kRes) store_all(std::integral_constant<int, 0>());
+            else if (a.res.affine == 1) store_all(std::integral_constant<int, 1>());
+            else if (a.res.affine == 2) store_all(std::integral_constant<int, 2>());
+            else store_all(std::integral_constant<int, 3>());
+            return;
+        }
 #pragma unroll
         for (int it = 0; it < ITER; ++it) {
             const int q = tid + it * T;
