@@ -362,6 +362,12 @@ private:
             // compiler/chxvm/simple_node_emitter.cc:316-318; attribute defaults of compiler/gen_node.py
             simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true)), FloatIn(n.GetFloat("alpha", 1.f)),
                         FloatIn(n.GetFloat("beta", 1.f)), IntIn(n.GetInt("transA", 0)), IntIn(n.GetInt("transB", 0))});
+        } else if (op == "BatchNormalization" && nin == 5) {
+            // EmitBatchNormalization, compiler/chxvm/emitter.cc:193-206: one output is the inference form
+            CHECK_EQ(1, n.GetInt("spatial", 1)) << "`spatial` for BatchNormalization was removed from ONNX";
+            CHECK_EQ(1u, n.outputs().size()) << "BatchNormalization with the outputs of a training step is not on the quantized-inference path";
+            simple("FixedBatchNormalization", {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), ArrayIn(Operand(n, 2)), ArrayIn(Operand(n, 3)),
+                                               ArrayIn(Operand(n, 4)), FloatIn(n.GetFloat("epsilon", 1e-5f))});
         } else if (op == "Flatten" && nin == 1) {
             // compiler/chxvm/simple_node_emitter.cc:698-701
             simple(op, {ArrayIn(Operand(n, 0)), IntIn(n.GetInt("axis", 1))});

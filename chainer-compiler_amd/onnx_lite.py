@@ -156,6 +156,7 @@ class Graph(object):
         self.name = ""
         self.nodes, self.initializers = [], {}
         self.inputs, self.outputs = [], []       # [(name, elem_type, shape)]
+        self.value_info = []                     # the same for values inside the graph
 
 
 def _parse_attr(b):
@@ -237,6 +238,8 @@ def parse_model(b):
             g.inputs.append(_parse_value_info(v))
         elif f == 12:
             g.outputs.append(_parse_value_info(v))
+        elif f == 13:
+            g.value_info.append(_parse_value_info(v))
     return g
 
 
@@ -274,4 +277,5 @@ def make_model(graph, opset=10):
     g += b"".join(_ld(5, make_tensor(k, v)) for k, v in graph.initializers.items())
     g += b"".join(_ld(11, _make_value_info(*vi)) for vi in graph.inputs)
     g += b"".join(_ld(12, _make_value_info(*vi)) for vi in graph.outputs)
+    g += b"".join(_ld(13, _make_value_info(*vi)) for vi in graph.value_info)
     return _vi(1, 5) + _ld(2, "chainer-compiler_amd") + _ld(7, g) + _ld(8, _ld(1, "") + _vi(2, opset))

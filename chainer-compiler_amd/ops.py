@@ -325,6 +325,16 @@ def AveragePool(x, kernel_shape, strides=(), pads=(), count_include_pad=False, o
     return out
 
 
+def FixedBatchNormalization(x, s, bias, mean, var, epsilon=1e-5, out=None):
+    """FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225: BatchNormalization with stored
+    statistics on a float32 array [N, C, ...]."""
+    if out is None:
+        out = torch.empty_like(x)
+    capi.check(capi.lib().chx_hip_fixed_batch_norm_f32(
+        capi.ref(x), capi.ref(s), capi.ref(bias), capi.ref(mean), capi.ref(var), _f(epsilon), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
 def MaxPoolQ8(x, kernel_shape, strides=(), pads=(), cover_all=False, out=None):
     """DequantizeLinear -> MaxPool (runtime/ops/pooling.cc:47-61) -> QuantizeLinear with equal
     quantization parameters, on the 8-bit codes: their maximum m for uint8, m + (m < 0) for int8 (the

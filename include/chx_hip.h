@@ -271,6 +271,17 @@ int chx_hip_average_pool_f32(
         const chx_hip_tensor* x, int32_t kernel_h, int32_t kernel_w, int32_t stride_h, int32_t stride_w, int32_t pad_h,
         int32_t pad_w, int32_t count_include_pad, chx_hip_tensor* y, void* stream);
 
+/* FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225 (the inference form a
+ * BatchNormalization node with one output is emitted as, compiler/chxvm/emitter.cc:193-206): x float32
+ * [N, C, ...] with any batch and channel strides and the remaining axes one evenly strided run (NCHW,
+ * channels-last); s, bias, mean, var contiguous float32 with C elements each;
+ *   y = ((x - mean) * (1 / sqrt(var + eps))) * s + bias
+ * one float32 rounding per operation in this order, eps <= 1e-5 replaced by (float)(1e-5 + 1e-12) as the op
+ * does.  (The operation order of ChainerX's FixedBatchNorm is not in the reference tree.) */
+int chx_hip_fixed_batch_norm_f32(
+        const chx_hip_tensor* x, const chx_hip_tensor* s, const chx_hip_tensor* bias, const chx_hip_tensor* mean,
+        const chx_hip_tensor* var, float epsilon, chx_hip_tensor* y, void* stream);
+
 /* ---- pooling on quantized tensors ------------------------------------------------------ */
 
 /* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized

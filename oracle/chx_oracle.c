@@ -37,6 +37,10 @@
  *   orc_average_pool_f32     pinned like orc_average_pool_q8 (tap-major numpy loop, both pad-count modes,
  *                            integer-valued images where every sum is exact, the whole-image window against
  *                            a sequential running sum); the same PARITY UNPINNED remainder.
+ *   orc_fixed_batch_norm_f32 pinned against float64 (error bound of its five roundings) and bit for bit on
+ *                            operands for which every step is exact (power-of-two deviations and scales);
+ *                            PARITY UNPINNED for the order of its operations: chainerx::FixedBatchNorm is not
+ *                            in the tree.
  *   orc_gemm_f32             pinned for everything but the order of the fp32 sum:
  *                            float64 numpy within a bound from the row norms,
  *                            bit-equal on integer-valued operands (every sum
@@ -680,6 +684,30 @@ void orc_average_pool_f32(
                 if (count_include_pad) cnt = (int32_t)(kh * kw);
                 y[(nc * OH + oh) * OW + ow] = sum / (float)cnt;
             }
+}
+
+/* FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225, on a contiguous [N, C, inner] float32
+ * array: ((x - mean) * (1 / sqrt(var + eps))) * s + bias, one rounding per operation, eps adjusted as the op does
+ * (lines 217-218).  PARITY UNPINNED for the order of the operations (chainerx::FixedBatchNorm is not in the tree);
+ * pinned against float64 within 4 ulp-sized terms and bit for bit where every step is exact. */
+void orc_fixed_batch_norm_f32(
+        const float* x, const float* s, const float* bias, const float* mean, const float* var, float epsilon, int64_t N, int64_t C,
+        int64_t inner, float* y) {
+    const float eps = epsilon <= 1e-5f ? (float)(1e-5 + 1e-12) : epsilon;
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t nc = 0; nc < N * C; ++nc) {
+        const int64_t c = nc % C;
+        const float ve = var[c] + eps;
+        const float sd = sqrtf(ve);
+        const float inv_std = 1.0f / sd;
+        for (int64_t i = 0; i < inner; ++i) {
+            float r = x[nc * inner + i] - mean[c];
+            r = r * inv_std;
+            r = r * s[c];
+            r = r + bias[c];
+            y[nc * inner + i] = r;
+        }
+    }
 }
 
 void orc_average_pool_q8(

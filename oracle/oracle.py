@@ -424,6 +424,19 @@ def average_pool(x, kernel, strides, pads=(0, 0), count_include_pad=False):
     return y
 
 
+def fixed_batch_norm(x, s, bias, mean, var, epsilon=1e-5):
+    """FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225, x [N, C, ...] float32."""
+    x = _c(x, np.float32)
+    s, bias, mean, var = (_c(np.asarray(v).reshape(-1), np.float32) for v in (s, bias, mean, var))
+    N, C = x.shape[0], x.shape[1]
+    inner = int(np.prod(x.shape[2:], dtype=np.int64))
+    assert s.size == bias.size == mean.size == var.size == C
+    y = np.empty(x.shape, dtype=np.float32)
+    i64 = ctypes.c_int64
+    lib().orc_fixed_batch_norm_f32(_p(x), _p(s), _p(bias), _p(mean), _p(var), ctypes.c_float(epsilon), i64(N), i64(C), i64(inner), _p(y))
+    return y
+
+
 def average_pool_q8(x, x_scale, x_zero_point, kernel, strides, pads, y_scale, y_zero_point, y_dtype=np.uint8,
                     count_include_pad=False, round_mode=ROUND_REFERENCE):
     x = _c(x)

@@ -29,8 +29,9 @@ def vm():
     return mod
 
 
-def model(nodes, inputs, outputs, initializers=None):
+def model(nodes, inputs, outputs, initializers=None, value_info=()):
     g = onnx_lite.Graph()
+    g.value_info = [(n, F, list(s)) for n, s in value_info]
     g.name = "test"
     g.nodes = [onnx_lite.Node(*n) if not isinstance(n, onnx_lite.Node) else n for n in nodes]
     g.inputs = [(n, F, list(s)) for n, s in inputs]
@@ -413,3 +414,19 @@ def test_global_pools_become_pools_over_the_spatial_extent(vm):
     unknown = model([N("MaxPool", ["x"], ["h"], {"kernel_shape": [2, 2]}), N("GlobalAveragePool", ["h"], ["a"], {})], [("x", (2, 8, 7, 5))], [("a", (2, 8, 1, 1))])
     with pytest.raises(vm.ChxVMError, match="shape of GlobalAveragePool must be known"):
         vm.compile_onnx(unknown, {"fuse": "none"})
+
+
+def test_batch_normalization_is_emitted_in_its_inference_form(vm):
+    """EmitBatchNormalization, compiler/chxvm/emitter.cc:193-206: one output -> FixedBatchNormalization(x, s, bias, mean, var,
+    epsilon); the outputs of a training step are not on this path."""
+    N = onnx_lite.Node
+    c4 = {k: np.ones(4, np.float32) for k in ("s", "b", "m", "v")}
+    m = model([N("BatchNormalization", ["x", "s", "b", "m", "v"], ["y"], {"epsilon": 1e-3})], [("x", (2, 4, 3, 3))], [("y", (2, 4, 3, 3))], c4)
+    insts = decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))
+    bn = next(i for i in insts if i[0] == "FixedBatchNormalization")
+    assert [t for t, _ in bn[1]] == ["ARRAY"] * 5 + ["FLOAT"] and abs(bn[1][5][1] - 1e-3) < 1e-9
+    assert not any(i[0] == "BatchNormalization" for i in insts)
+    train = model([N("BatchNormalization", ["x", "s", "b", "m", "v"], ["y", "rm", "rv"], {})], [("x", (2, 4, 3, 3))],
+                  [("y", (2, 4, 3, 3)), ("rm", (4,)), ("rv", (4,))], c4)
+    with pytest.raises(vm.ChxVMError, match=r"1 vs\. 3.*BatchNormalization"):
+        vm.compile_onnx(train, {"fuse": "none"})

@@ -186,3 +186,77 @@ def test_float_layers_from_an_onnx_graph(g, vm, oracle):
     prog.close()
     want = oracle.gemm(oracle.gemm(oracle.flatten(x, 1), w, bias, trans_b=True), w2)
     np.testing.assert_array_equal(bits(got["y"]), bits(want))
+
+
+@pytest.mark.parametrize("shape", [(4, 6, 5, 7), (2, 16, 14, 14), (3, 5), (2, 4, 9), (1, 1, 1, 1)], ids=str)
+def test_fixed_batch_norm_through_the_c_abi(g, oracle, shape):
+    """FixedBatchNormalization on NCHW, channels-last, [N, C] and [N, C, L] arrays, bit for bit against the oracle
+    (square root and reciprocal are correctly rounded on both sides); epsilon at or below 1e-5 is replaced."""
+    rng = np.random.default_rng(sum(shape))
+    C = shape[1]
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    s, bias, mean = (rng.standard_normal(C).astype(np.float32) for _ in range(3))
+    var = rng.uniform(0.0, 4.0, C).astype(np.float32)
+    for eps in (1e-3, 1e-5, 0.0):
+        want = oracle.fixed_batch_norm(x, s, bias, mean, var, eps)
+        layouts = [g.dev(x)] + ([g.to_channels_last(g.dev(x))] if len(shape) == 4 else [])
+        for xd in layouts:
+            got = g.ops.FixedBatchNormalization(xd, g.dev(s), g.dev(bias), g.dev(mean), g.dev(var.reshape(1, C)), eps)
+            assert got.stride() == xd.stride()
+            np.testing.assert_array_equal(bits(g.host(got)), bits(want))
+    with pytest.raises(g.capi.ChxHipError, match="channels"):
+        g.ops.FixedBatchNormalization(g.dev(x), g.dev(s[:-1] if C > 1 else np.zeros(2, np.float32)), g.dev(bias), g.dev(mean), g.dev(var))
+    with pytest.raises(g.capi.ChxHipError, match="float32"):
+        g.ops.FixedBatchNormalization(g.dev(x.astype(np.float64)).to(torch.float64), g.dev(s), g.dev(bias), g.dev(mean), g.dev(var),
+                                      out=torch.empty(shape, dtype=torch.float32, device="cuda"))
+
+
+def test_conv_net_with_batch_normalization_under_the_default_quantization(g, vm, oracle):
+    """What `--quantize` (dynamic parameters, integer ops) leaves of a float CNN: the Conv without a bias becomes
+    QuantizeLinear -> ConvInteger -> Cast -> Mul, and BatchNormalization, Relu, MaxPool, GlobalAveragePool, Flatten and Gemm
+    stay float nodes (compiler/quantize.cc:377-380, compiler/chxvm/emitter.cc:193-206).  The program is compared with
+    the same sequence spelled with numpy and the oracle, and loosely with the float network."""
+    import test_compiler_cpu as cc
+    import test_gpu_compiler as gc
+    onnx_lite = cc.onnx_lite
+    rng = np.random.default_rng(21)
+    N = onnx_lite.Node
+    w = (rng.standard_normal((8, 3, 3, 3)) * 0.3).astype(np.float32)
+    s, bias, mean = (rng.standard_normal(8).astype(np.float32) * 0.5 for _ in range(3))
+    s = s + np.float32(1.5)
+    var = rng.uniform(0.5, 2.0, 8).astype(np.float32)
+    fc = (rng.standard_normal((5, 8)) * 0.4).astype(np.float32)
+    fb = rng.standard_normal(5).astype(np.float32)
+    nodes = [N("Conv", ["x", "w"], ["c"], {"kernel_shape": [3, 3], "strides": [1, 1], "pads": [1, 1, 1, 1]}),
+             N("BatchNormalization", ["c", "s", "bias", "mean", "var"], ["bn"], {"epsilon": 1e-5}),
+             N("Relu", ["bn"], ["r"], {}),
+             N("MaxPool", ["r"], ["p"], {"kernel_shape": [2, 2], "strides": [2, 2]}),
+             N("GlobalAveragePool", ["p"], ["ga"], {}),
+             N("Flatten", ["ga"], ["f"], {}),
+             N("Gemm", ["f", "fc", "fb"], ["y"], {"transB": 1})]
+    x = (rng.standard_normal((2, 3, 12, 12)) * 1.5).astype(np.float32)
+    m = cc.model(nodes, [("x", x.shape)], [("y", (2, 5))], {"w": w, "s": s, "bias": bias, "mean": mean, "var": var, "fc": fc, "fb": fb},
+                 value_info=[("p", (2, 8, 6, 6))])
+    data = vm.compile_onnx(m, {"quantize": {}})
+    names = [i[0] for i in cc.decode_program(vm, data)]
+    assert "ConvInteger" in names and "FixedBatchNormalization" in names and "Gemm" in names and "Conv" not in names
+    prog = vm.Program(data)
+    got = prog.run({"x": torch.from_numpy(x).cuda()})["y"]
+    prog.close()
+    scale, zp = gc._dynamic_uint8_params(x)
+    xq = oracle.quantize_linear(x, scale, int(zp), np.uint8)
+    parts = [cc.numpy_quantize(w[oc], np.uint8) for oc in range(w.shape[0])]     # per output channel: the quantizer's default
+    wq = np.stack([q[0] for q in parts])
+    ws, wz = np.array([q[1] for q in parts], np.float32), np.array([q[2] for q in parts], np.uint8)
+    acc = oracle.conv_integer(xq, wq, int(zp), wz, strides=(1, 1), pads=(1, 1), group=1, auto_pad="")
+    c = acc.astype(np.float32) * (scale * ws).astype(np.float32).reshape(-1, 1, 1)
+    bn = oracle.fixed_batch_norm(c, s, bias, mean, var, 1e-5)
+    p = oracle.max_pool(np.maximum(bn, np.float32(0)), (2, 2), (2, 2), (0, 0), False)
+    ga = oracle.average_pool(p, (6, 6), (1, 1), (0, 0), False)
+    want = oracle.gemm(oracle.flatten(ga, 1), fc, fb, trans_b=True)
+    np.testing.assert_array_equal(bits(got), bits(want))
+    tx = torch.from_numpy
+    ref = torch.nn.functional.conv2d(tx(x), tx(w), padding=1)
+    ref = torch.nn.functional.batch_norm(ref, tx(mean), tx(var), tx(s), tx(bias), eps=1e-5).relu()
+    ref = torch.nn.functional.max_pool2d(ref, 2).mean(dim=(2, 3)) @ tx(fc).T + tx(fb)
+    assert np.abs(got - ref.numpy()).max() < 0.05 * np.abs(ref.numpy()).max() + 0.05

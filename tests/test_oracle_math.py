@@ -600,3 +600,46 @@ def test_float_average_pool_vs_numpy(oracle, include_pad):
     xg = rng.standard_normal((1, 2, 7, 7)).astype(np.float32)
     seq = np.cumsum(xg.reshape(1, 2, 49), axis=-1, dtype=np.float32)[..., -1] / np.float32(49)
     np.testing.assert_array_equal(oracle.average_pool(xg, (7, 7), (1, 1), (0, 0), include_pad).reshape(1, 2), seq)
+
+
+def test_fixed_batch_norm_pins(oracle):
+    """orc_fixed_batch_norm_f32 against float64 (five float32 roundings: the bound below), bit for bit where every
+    step is exact, against the same steps in numpy float32, and the op's adjustment of a small epsilon
+    (runtime/ops/normalization.cc:217-218)."""
+    rng = np.random.default_rng(71)
+    for shape in [(4, 6, 5, 7), (3, 5), (2, 4, 9)]:
+        C = shape[1]
+        x = (rng.standard_normal(shape) * 3).astype(np.float32)
+        s, bias, mean = (rng.standard_normal(C).astype(np.float32) for _ in range(3))
+        var = rng.uniform(0.01, 4.0, C).astype(np.float32)
+        bc = (1, C) + (1,) * (len(shape) - 2)
+        for eps in (1e-3, 1e-5, 0.0):
+            eff = np.float32(eps) if eps > 1e-5 else np.float32(1e-5 + 1e-12)
+            got = oracle.fixed_batch_norm(x, s, bias, mean, var, eps)
+            # the same five operations in numpy float32
+            inv = np.float32(1) / np.sqrt(var + eff)
+            steps = ((x - mean.reshape(bc)) * inv.reshape(bc)) * s.reshape(bc) + bias.reshape(bc)
+            np.testing.assert_array_equal(got, steps)
+            f8 = np.float64
+            scaled = (x.astype(f8) - mean.reshape(bc).astype(f8)) / np.sqrt(var.reshape(bc).astype(f8) + f8(eff)) * s.reshape(bc).astype(f8)
+            exact = scaled + bias.reshape(bc).astype(f8)
+            bound = 2.0 ** -24 * (5 * np.abs(scaled) + np.abs(exact)) + 1e-37
+            assert (np.abs(got - exact) <= bound).all()
+    # exact family: integer deviations, var + eps a power of four, power-of-two scales, integer biases
+    x = rng.integers(-100, 101, size=(2, 4, 3, 3)).astype(np.float32)
+    mean = np.array([3, -7, 0, 12], np.float32)
+    var = np.array([0.0, 0.75, 3.75, 15.75], np.float32)       # + 0.25 = 0.25, 1, 4, 16
+    s = np.array([2.0, -0.5, 4.0, 1.0], np.float32)
+    bias = np.array([5, -3, 0, 100], np.float32)
+    want = (x - mean.reshape(1, 4, 1, 1)) * (s / np.array([0.5, 1, 2, 4], np.float32)).reshape(1, 4, 1, 1) + bias.reshape(1, 4, 1, 1)
+    np.testing.assert_array_equal(oracle.fixed_batch_norm(x, s, bias, mean, var, 0.25), want)
+    # epsilon at or below 1e-5 is replaced: with var = 0 the replaced value shows
+    z = np.zeros(4, np.float32)
+    a = oracle.fixed_batch_norm(x, s, z, z, z, 1e-5)
+    b = oracle.fixed_batch_norm(x, s, z, z, z, float(np.float32(1e-5 + 1e-12)) + 1e-9)   # just above: taken as it is
+    c = oracle.fixed_batch_norm(x, s, z, z, z, 0.0)
+    np.testing.assert_array_equal(a, c)
+    assert np.float32(1e-5 + 1e-12) > np.float32(1e-5)
+    naive = (x * (np.float32(1) / np.sqrt(np.float32(1e-5)))) * s.reshape(1, 4, 1, 1)
+    assert not np.array_equal(a, naive)
+    assert np.allclose(a, b, rtol=1e-3)
