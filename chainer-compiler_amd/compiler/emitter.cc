@@ -362,6 +362,10 @@ private:
             // compiler/chxvm/simple_node_emitter.cc:316-318; attribute defaults of compiler/gen_node.py
             simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true)), FloatIn(n.GetFloat("alpha", 1.f)),
                         FloatIn(n.GetFloat("beta", 1.f)), IntIn(n.GetInt("transA", 0)), IntIn(n.GetInt("transB", 0))});
+        } else if (op == "Conv" && (nin == 2 || nin == 3)) {
+            // compiler/chxvm/simple_node_emitter.cc:213-219: a convolution the quantizer did not rewrite
+            ChxVMInstructionProto* inst = simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true))});
+            ConvAttrs(n, inst);
         } else if (op == "BatchNormalization" && nin == 5) {
             // EmitBatchNormalization, compiler/chxvm/emitter.cc:193-206: one output is the inference form
             CHECK_EQ(1, n.GetInt("spatial", 1)) << "`spatial` for BatchNormalization was removed from ONNX";

@@ -325,6 +325,15 @@ def AveragePool(x, kernel_shape, strides=(), pads=(), count_include_pad=False, o
     return out
 
 
+def Conv(x, w, b=None, strides=(), pads=(), group=1, auto_pad="", out=None):
+    """ConvOp::RunImpl on float32, runtime/ops/connection.cc:24-30."""
+    params, shape = _conv_setup(x, w, strides, pads, group, auto_pad)
+    if out is None:
+        out = _alloc_like_input_layout(x, shape, torch.float32)
+    capi.check(capi.lib().chx_hip_conv_f32(capi.ref(x), capi.ref(w), capi.ref(b), ctypes.byref(params), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
 def FixedBatchNormalization(x, s, bias, mean, var, epsilon=1e-5, out=None):
     """FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225: BatchNormalization with stored
     statistics on a float32 array [N, C, ...]."""

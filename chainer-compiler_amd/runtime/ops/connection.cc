@@ -1,7 +1,8 @@
-// The float layers around a quantized network on the hip backend: GemmOp and MatMulOp
+// The float layers around a quantized network on the hip backend: ConvOp (runtime/ops/connection.cc:24-30), GemmOp and MatMulOp
 // (runtime/ops/math.cc:156-177 of the chainer-compiler tree), LinearOp (runtime/ops/connection.cc:12-15),
 // FlattenOp (runtime/ops/manipulation.cc:20-28).  The products run in chx_hip_gemm_f32 /
 // chx_hip_linear_f32; Flatten is a view, after a device copy when the array is not dense.
+#include "../chainerx_util.h"
 #include "../gen/gen_chxvm_ops.h"
 
 namespace chainer_compiler {
@@ -11,6 +12,12 @@ namespace {
 
 void CheckFloat32(const chainerx::Array& a, const char* op, const char* name) {
     CHECK(a.dtype() == chainerx::Dtype::kFloat32) << op << ": " << name << " must be float32 on the hip backend, not " << a.dtype();
+}
+
+// outputs follow the input's layout: channels-last in, channels-last out
+chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& shape, chainerx::Dtype dtype) {
+    const bool channels_last = x.ndim() == 4 && !x.IsContiguous() && x.strides()[1] == x.GetItemSize();
+    return channels_last ? chainerx::EmptyChannelsLast(shape, dtype) : chainerx::Empty(shape, dtype);
 }
 
 }  // namespace
@@ -37,6 +44,20 @@ chainerx::Array GemmOp::RunImpl(
     if (c.has_value()) ct = c->hip();
     CHXVM_HIP_CALL(chx_hip_gemm_f32(&at, &bt, c.has_value() ? &ct : nullptr, static_cast<float>(alpha), static_cast<float>(beta),
                                     trans_a ? 1 : 0, trans_b ? 1 : 0, &yt, chainerx::CurrentStream()));
+    return y;
+}
+
+// ConvOp::RunImpl, runtime/ops/connection.cc:24-30: a convolution the quantizer left in float (one with a bias).
+chainerx::Array ConvOp::RunImpl(
+        ChxVMState* st, const chainerx::Array& x, const chainerx::Array& w, const absl::optional<chainerx::Array>& b) {
+    CheckFloat32(x, "Conv", "x");
+    CheckFloat32(w, "Conv", "w");
+    if (b.has_value()) CheckFloat32(*b, "Conv", "b");
+    const chx_hip_conv_params p = MakeConvParams(x, w, strides, pads, group, auto_pad);
+    chainerx::Array y = EmptyLike4d(x, ConvOutputShape(x, w, p), chainerx::Dtype::kFloat32);
+    chx_hip_tensor xt = x.hip(), wt = w.hip(), yt = y.hip(), bt;
+    if (b.has_value()) bt = b->hip();
+    CHXVM_HIP_CALL(chx_hip_conv_f32(&xt, &wt, b.has_value() ? &bt : nullptr, &p, &yt, chainerx::CurrentStream()));
     return y;
 }
 

@@ -282,6 +282,17 @@ int chx_hip_fixed_batch_norm_f32(
         const chx_hip_tensor* x, const chx_hip_tensor* s, const chx_hip_tensor* bias, const chx_hip_tensor* mean,
         const chx_hip_tensor* var, float epsilon, chx_hip_tensor* y, void* stream);
 
+/* ConvOp::RunImpl, runtime/ops/connection.cc:24-30 (GroupedConv, runtime/chainerx_util.cc:313-340) on
+ * float32: the convolutions the quantizer does not rewrite (a Conv with a bias, compiler/quantize.cc:376-381).
+ * x [N,C,H,W], w [OC,C/group,KH,KW], b [OC] or NULL, y [N,OC,OH,OW], all float32 with any strides; params as
+ * for chx_hip_qlinear_conv (auto_pad already resolved into explicit pads).  The sum runs over (c, kh, kw) in
+ * this order in float32 from 0, one rounding per multiplication and per addition, b added last.  (The order
+ * of ChainerX's own Conv is not in the reference tree; against the reference the result carries its
+ * tolerance, rtol 1e-4 / atol 1e-6.)  A coverage kernel, not tuned. */
+int chx_hip_conv_f32(
+        const chx_hip_tensor* x, const chx_hip_tensor* w, const chx_hip_tensor* b, const chx_hip_conv_params* params,
+        chx_hip_tensor* y, void* stream);
+
 /* ---- pooling on quantized tensors ------------------------------------------------------ */
 
 /* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized

@@ -37,6 +37,10 @@
  *   orc_average_pool_f32     pinned like orc_average_pool_q8 (tap-major numpy loop, both pad-count modes,
  *                            integer-valued images where every sum is exact, the whole-image window against
  *                            a sequential running sum); the same PARITY UNPINNED remainder.
+ *   orc_conv_f32             pinned against float64 within the bound of a K-term float32 sum, bit for bit on
+ *                            integer-valued operands (groups, strides, pads), against orc_gemm_f32 on the
+ *                            explicitly expanded matrix; PARITY UNPINNED for the order (c, kh, kw):
+ *                            chainerx::Conv is not in the tree.
  *   orc_fixed_batch_norm_f32 pinned against float64 (error bound of its five roundings) and bit for bit on
  *                            operands for which every step is exact (power-of-two deviations and scales);
  *                            PARITY UNPINNED for the order of its operations: chainerx::FixedBatchNorm is not
@@ -684,6 +688,40 @@ void orc_average_pool_f32(
                 if (count_include_pad) cnt = (int32_t)(kh * kw);
                 y[(nc * OH + oh) * OW + ow] = sum / (float)cnt;
             }
+}
+
+/* ConvOp::RunImpl on float32, runtime/ops/connection.cc:24-30 (GroupedConv, runtime/chainerx_util.cc:313-340):
+ * the expanded-matrix product of orc_qlinear_conv_literal without the quantization around it: k = (c, kh, kw) in
+ * order, an fp32 accumulator from 0, a tap in the padding as the product 0 * w, the bias added last.
+ * PARITY UNPINNED for that order (chainerx::Conv is not in the tree); pinned against float64 within the bound of
+ * a K-term float32 sum and bit for bit on integer-valued operands. */
+void orc_conv_f32(const float* x, const float* w, const float* bias, const orc_conv_geom* g, float* y) {
+    const int64_t OH = orc_conv_out_h(g), OW = orc_conv_out_w(g);
+    const int64_t Cg = g->C / g->group, OCg = g->OC / g->group;
+    const int64_t Kdim = Cg * g->KH * g->KW;
+#pragma omp parallel for collapse(2) num_threads(g_threads) if (g_threads > 1)
+    for (int64_t n = 0; n < g->N; ++n)
+        for (int64_t oc = 0; oc < g->OC; ++oc) {
+            const int64_t grp = oc / OCg;
+            const float* wr = w + oc * Kdim;
+            for (int64_t oh = 0; oh < OH; ++oh)
+                for (int64_t ow = 0; ow < OW; ++ow) {
+                    float v = 0.f;
+                    for (int64_t c = 0; c < Cg; ++c)
+                        for (int64_t kh = 0; kh < g->KH; ++kh) {
+                            const int64_t ih = oh * g->sh - g->ph0 + kh;
+                            for (int64_t kw = 0; kw < g->KW; ++kw) {
+                                const int64_t iw = ow * g->sw - g->pw0 + kw;
+                                float xv = 0.f;
+                                if (ih >= 0 && ih < g->H && iw >= 0 && iw < g->W) xv = x[((n * g->C + grp * Cg + c) * g->H + ih) * g->W + iw];
+                                const float prod = xv * wr[(c * g->KH + kh) * g->KW + kw];
+                                v = v + prod;
+                            }
+                        }
+                    if (bias) v = v + bias[oc];
+                    y[((n * g->OC + oc) * OH + oh) * OW + ow] = v;
+                }
+        }
 }
 
 /* FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225, on a contiguous [N, C, inner] float32

@@ -424,6 +424,16 @@ def average_pool(x, kernel, strides, pads=(0, 0), count_include_pad=False):
     return y
 
 
+def conv(x, w, bias=None, strides=(1, 1), pads=(0, 0), group=1, auto_pad=""):
+    """ConvOp::RunImpl on float32, runtime/ops/connection.cc:24-30."""
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    g = conv_geometry(x.shape, w.shape, strides, pads, group, auto_pad)
+    b = None if bias is None else _c(bias, np.float32)
+    y = np.empty(conv_out_shape(g), dtype=np.float32)
+    lib().orc_conv_f32(_p(x), _p(w), _p(b) if b is not None else None, ctypes.byref(g), _p(y))
+    return y
+
+
 def fixed_batch_norm(x, s, bias, mean, var, epsilon=1e-5):
     """FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225, x [N, C, ...] float32."""
     x = _c(x, np.float32)

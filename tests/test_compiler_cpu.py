@@ -430,3 +430,18 @@ def test_batch_normalization_is_emitted_in_its_inference_form(vm):
                   [("y", (2, 4, 3, 3)), ("rm", (4,)), ("rv", (4,))], c4)
     with pytest.raises(vm.ChxVMError, match=r"1 vs\. 3.*BatchNormalization"):
         vm.compile_onnx(train, {"fuse": "none"})
+
+
+def test_float_conv_is_emitted_with_the_reference_operand_list(vm):
+    """compiler/chxvm/simple_node_emitter.cc:213-219: Conv(x, w, b?, strides, pads, group, auto_pad); the quantizer leaves
+    a Conv with a bias as it is (compiler/quantize.cc:376-381) and rewrites the one without."""
+    rng = np.random.default_rng(9)
+    m, _ = conv_model(rng, with_bias=True)
+    insts = decode_program(vm, vm.compile_onnx(m, {"quantize": {}}))
+    conv = next(i for i in insts if i[0] == "Conv")
+    assert [t for t, _ in conv[1]] == ["ARRAY", "ARRAY", "ARRAY", "INTS", "INTS", "INT", "STRING"]
+    assert not any(i[0] == "ConvInteger" for i in insts)
+    m, _ = conv_model(rng, with_bias=False)
+    insts = decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))                     # not quantized at all: a float Conv, no bias
+    conv = next(i for i in insts if i[0] == "Conv")
+    assert conv[1][2][1] == -1

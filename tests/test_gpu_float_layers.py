@@ -211,10 +211,35 @@ def test_fixed_batch_norm_through_the_c_abi(g, oracle, shape):
                                       out=torch.empty(shape, dtype=torch.float32, device="cuda"))
 
 
+FCONV_CASES = [  # N, C, H, W, OC, KH, KW, strides, pads, group, auto_pad
+    (2, 3, 9, 8, 4, 3, 3, (1, 1), (1, 1), 1, ""), (1, 4, 7, 7, 6, 1, 1, (2, 2), (0, 0), 2, ""), (2, 6, 8, 8, 6, 3, 2, (2, 1), (0, 1), 6, ""),
+    (1, 8, 5, 5, 4, 5, 5, (1, 1), (2, 2), 4, ""), (3, 2, 6, 6, 5, 2, 2, (2, 2), (0, 0), 1, ""), (2, 16, 14, 14, 32, 3, 3, (2, 2), (0, 0), 1, "SAME_UPPER"),
+    (4, 3, 32, 32, 16, 7, 7, (2, 2), (3, 3), 1, "")]
+
+
+@pytest.mark.parametrize("case", FCONV_CASES, ids=lambda c: "x".join(str(v) for v in c[:7]) + "_g%d" % c[9])
+def test_float_conv_through_the_c_abi(g, oracle, case):
+    """The float32 Conv the quantizer leaves alone (one with a bias): NCHW and channels-last, with and without the bias,
+    groups, strides, pads and SAME_UPPER; bit for bit against the oracle, whose order of the sum the kernel follows."""
+    N, C, H, W, OC, KH, KW, strides, pads, group, auto_pad = case
+    rng = np.random.default_rng(N * 100 + C * 10 + KH)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    w = rng.standard_normal((OC, C // group, KH, KW)).astype(np.float32)
+    b = rng.standard_normal(OC).astype(np.float32)
+    for bias in (b, None):
+        want = oracle.conv(x, w, bias, strides, pads, group, auto_pad)
+        for xd in (g.dev(x), g.to_channels_last(g.dev(x))):
+            got = g.ops.Conv(xd, g.dev(w), None if bias is None else g.dev(bias), strides, pads, group, auto_pad)
+            assert got.shape == want.shape
+            np.testing.assert_array_equal(bits(g.host(got)), bits(want))
+    with pytest.raises(g.capi.ChxHipError, match="float32"):
+        g.ops.Conv(g.dev(x), g.dev(w.astype(np.float64)).to(torch.float64), None, strides, pads, group, auto_pad)
+
+
 def test_conv_net_with_batch_normalization_under_the_default_quantization(g, vm, oracle):
     """What `--quantize` (dynamic parameters, integer ops) leaves of a float CNN: the Conv without a bias becomes
-    QuantizeLinear -> ConvInteger -> Cast -> Mul, and BatchNormalization, Relu, MaxPool, GlobalAveragePool, Flatten and Gemm
-    stay float nodes (compiler/quantize.cc:377-380, compiler/chxvm/emitter.cc:193-206).  The program is compared with
+    QuantizeLinear -> ConvInteger -> Cast -> Mul, and the Conv with a bias, BatchNormalization, Relu, MaxPool,
+    GlobalAveragePool, Flatten and Gemm stay float nodes (compiler/quantize.cc:377-380, compiler/chxvm/emitter.cc:193-206).  The program is compared with
     the same sequence spelled with numpy and the oracle, and loosely with the float network."""
     import test_compiler_cpu as cc
     import test_gpu_compiler as gc
@@ -225,21 +250,24 @@ def test_conv_net_with_batch_normalization_under_the_default_quantization(g, vm,
     s, bias, mean = (rng.standard_normal(8).astype(np.float32) * 0.5 for _ in range(3))
     s = s + np.float32(1.5)
     var = rng.uniform(0.5, 2.0, 8).astype(np.float32)
+    w2 = (rng.standard_normal((8, 8, 3, 3)) * 0.2).astype(np.float32)
+    b2 = rng.standard_normal(8).astype(np.float32)
     fc = (rng.standard_normal((5, 8)) * 0.4).astype(np.float32)
     fb = rng.standard_normal(5).astype(np.float32)
     nodes = [N("Conv", ["x", "w"], ["c"], {"kernel_shape": [3, 3], "strides": [1, 1], "pads": [1, 1, 1, 1]}),
              N("BatchNormalization", ["c", "s", "bias", "mean", "var"], ["bn"], {"epsilon": 1e-5}),
-             N("Relu", ["bn"], ["r"], {}),
+             N("Relu", ["bn"], ["r0"], {}),
+             N("Conv", ["r0", "w2", "b2"], ["r"], {"kernel_shape": [3, 3], "pads": [1, 1, 1, 1]}),       # with a bias: not rewritten
              N("MaxPool", ["r"], ["p"], {"kernel_shape": [2, 2], "strides": [2, 2]}),
              N("GlobalAveragePool", ["p"], ["ga"], {}),
              N("Flatten", ["ga"], ["f"], {}),
              N("Gemm", ["f", "fc", "fb"], ["y"], {"transB": 1})]
     x = (rng.standard_normal((2, 3, 12, 12)) * 1.5).astype(np.float32)
-    m = cc.model(nodes, [("x", x.shape)], [("y", (2, 5))], {"w": w, "s": s, "bias": bias, "mean": mean, "var": var, "fc": fc, "fb": fb},
+    m = cc.model(nodes, [("x", x.shape)], [("y", (2, 5))], {"w": w, "s": s, "bias": bias, "mean": mean, "var": var, "fc": fc, "fb": fb, "w2": w2, "b2": b2},
                  value_info=[("p", (2, 8, 6, 6))])
     data = vm.compile_onnx(m, {"quantize": {}})
     names = [i[0] for i in cc.decode_program(vm, data)]
-    assert "ConvInteger" in names and "FixedBatchNormalization" in names and "Gemm" in names and "Conv" not in names
+    assert names.count("ConvInteger") == 1 and names.count("Conv") == 1 and "FixedBatchNormalization" in names and "Gemm" in names
     prog = vm.Program(data)
     got = prog.run({"x": torch.from_numpy(x).cuda()})["y"]
     prog.close()
@@ -251,12 +279,14 @@ def test_conv_net_with_batch_normalization_under_the_default_quantization(g, vm,
     acc = oracle.conv_integer(xq, wq, int(zp), wz, strides=(1, 1), pads=(1, 1), group=1, auto_pad="")
     c = acc.astype(np.float32) * (scale * ws).astype(np.float32).reshape(-1, 1, 1)
     bn = oracle.fixed_batch_norm(c, s, bias, mean, var, 1e-5)
-    p = oracle.max_pool(np.maximum(bn, np.float32(0)), (2, 2), (2, 2), (0, 0), False)
+    r = oracle.conv(np.maximum(bn, np.float32(0)), w2, b2, (1, 1), (1, 1))
+    p = oracle.max_pool(r, (2, 2), (2, 2), (0, 0), False)
     ga = oracle.average_pool(p, (6, 6), (1, 1), (0, 0), False)
     want = oracle.gemm(oracle.flatten(ga, 1), fc, fb, trans_b=True)
     np.testing.assert_array_equal(bits(got), bits(want))
     tx = torch.from_numpy
     ref = torch.nn.functional.conv2d(tx(x), tx(w), padding=1)
     ref = torch.nn.functional.batch_norm(ref, tx(mean), tx(var), tx(s), tx(bias), eps=1e-5).relu()
+    ref = torch.nn.functional.conv2d(ref, tx(w2), tx(b2), padding=1)
     ref = torch.nn.functional.max_pool2d(ref, 2).mean(dim=(2, 3)) @ tx(fc).T + tx(fb)
     assert np.abs(got - ref.numpy()).max() < 0.05 * np.abs(ref.numpy()).max() + 0.05

@@ -643,3 +643,38 @@ def test_fixed_batch_norm_pins(oracle):
     naive = (x * (np.float32(1) / np.sqrt(np.float32(1e-5)))) * s.reshape(1, 4, 1, 1)
     assert not np.array_equal(a, naive)
     assert np.allclose(a, b, rtol=1e-3)
+
+
+def test_float_conv_pins(oracle):
+    """orc_conv_f32 against float64 (bound of a K-term float32 sum), bit for bit on integer-valued operands (every
+    sum exact whatever its order) with groups, strides and pads, and against orc_gemm_f32 on the explicitly
+    expanded matrix (the same k order)."""
+    import torch
+    rng = np.random.default_rng(81)
+    cases = [  # N, C, H, W, OC, KH, KW, strides, pads, group
+        (2, 3, 9, 8, 4, 3, 3, (1, 1), (1, 1), 1), (1, 4, 7, 7, 6, 1, 1, (2, 2), (0, 0), 2), (2, 6, 8, 8, 6, 3, 2, (2, 1), (0, 1), 6),
+        (1, 8, 5, 5, 4, 5, 5, (1, 1), (2, 2), 4), (3, 2, 6, 6, 5, 2, 2, (2, 2), (0, 0), 1)]
+    for N, C, H, W, OC, KH, KW, strides, pads, group in cases:
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        w = rng.standard_normal((OC, C // group, KH, KW)).astype(np.float32)
+        b = rng.standard_normal(OC).astype(np.float32)
+        got = oracle.conv(x, w, b, strides, pads, group)
+        tx = torch.from_numpy
+        exact = torch.nn.functional.conv2d(tx(x).double(), tx(w).double(), tx(b).double(), strides, pads, 1, group).numpy()
+        mag = torch.nn.functional.conv2d(tx(np.abs(x)).double(), tx(np.abs(w)).double(), None, strides, pads, 1, group).numpy() + np.abs(b).reshape(1, -1, 1, 1)
+        K = (C // group) * KH * KW
+        assert got.shape == exact.shape and (np.abs(got - exact) <= (K + 2) * 2.0 ** -24 * mag + 1e-30).all()
+        xi = rng.integers(-8, 9, size=x.shape).astype(np.float32)
+        wi = rng.integers(-8, 9, size=w.shape).astype(np.float32)
+        bi = rng.integers(-50, 51, size=OC).astype(np.float32)
+        want = torch.nn.functional.conv2d(tx(xi).double(), tx(wi).double(), tx(bi).double(), strides, pads, 1, group).numpy()
+        np.testing.assert_array_equal(oracle.conv(xi, wi, bi, strides, pads, group), want.astype(np.float32))
+        np.testing.assert_array_equal(oracle.conv(xi, wi, None, strides, pads, group), (want - bi.reshape(1, -1, 1, 1)).astype(np.float32))
+    # the same order as a matrix product over the expanded matrix with k = (c, kh, kw)
+    x = rng.standard_normal((2, 3, 6, 6)).astype(np.float32)
+    w = rng.standard_normal((5, 3, 3, 3)).astype(np.float32)
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    col = np.stack([xp[:, :, i:i + 6, j:j + 6] for i in range(3) for j in range(3)], axis=2)      # [N, C, 9, OH, OW]
+    col = col.transpose(0, 3, 4, 1, 2).reshape(2 * 36, 27)
+    want = oracle.gemm(col, w.reshape(5, 27), trans_b=True).reshape(2, 6, 6, 5).transpose(0, 3, 1, 2)
+    np.testing.assert_array_equal(oracle.conv(x, w, None, (1, 1), (1, 1)), want)
