@@ -366,6 +366,9 @@ private:
             // compiler/chxvm/simple_node_emitter.cc:213-219: a convolution the quantizer did not rewrite
             ChxVMInstructionProto* inst = simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true))});
             ConvAttrs(n, inst);
+        } else if (op == "Softmax" && nin == 1) {
+            // compiler/chxvm/simple_node_emitter.cc:385-386; attribute defaults of compiler/gen_node.py:223
+            simple(op, {ArrayIn(Operand(n, 0)), IntIn(n.GetInt("axis", 1)), IntIn(n.GetInt("chainer_is_onnx_semantics", 1))});
         } else if (op == "BatchNormalization" && nin == 5) {
             // EmitBatchNormalization, compiler/chxvm/emitter.cc:193-206: one output is the inference form
             CHECK_EQ(1, n.GetInt("spatial", 1)) << "`spatial` for BatchNormalization was removed from ONNX";

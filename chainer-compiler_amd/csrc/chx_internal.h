@@ -127,6 +127,10 @@ bool same_dense_layout(const chx_hip_tensor& a, const chx_hip_tensor& b);
 
 int check_tensor(const chx_hip_tensor* t, const char* what);
 
+// Which operation grouping of expf the host C library uses (faithful_math.h): the two groupings differ on
+// exactly two arguments, so evaluating one of them tells.
+bool host_libm_uses_fma();
+
 inline hipStream_t as_stream(void* s) {
     return reinterpret_cast<hipStream_t>(s);
 }

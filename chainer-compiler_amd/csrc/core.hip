@@ -1,4 +1,5 @@
 // Library state, error reporting and the thin device-memory helpers of the C ABI.
+#include <cmath>
 #include <cstring>
 
 #include "chx_internal.h"
@@ -14,6 +15,21 @@ void set_error(const char* fmt, ...) {
     vsnprintf(buf, sizeof(buf), fmt, ap);
     va_end(ap);
     g_last_error = buf;
+}
+
+bool host_libm_uses_fma() {
+    static const bool v = [] {
+        volatile float x = 0.0f;
+        const uint32_t bits = 0x4202422fu;
+        float xf;
+        memcpy(&xf, &bits, 4);
+        x = xf;
+        const float e = expf(x);
+        uint32_t eb;
+        memcpy(&eb, &e, 4);
+        return eb == 0x56fc9f1cu;  // 0x1.f93e38p+46: the fused-reduction result
+    }();
+    return v;
 }
 
 int check_tensor(const chx_hip_tensor* t, const char* what) {

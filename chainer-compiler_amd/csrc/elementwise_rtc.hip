@@ -530,23 +530,6 @@ int compile_source(const std::string& src, const std::string& name, std::vector<
     return CHX_HIP_OK;
 }
 
-// Which operation grouping of expf the host C library uses (see faithful_math.h):
-// the two groupings differ on exactly two inputs, so evaluating one of them tells.
-bool host_libm_uses_fma() {
-    static const bool v = [] {
-        volatile float x = 0.0f;
-        const uint32_t bits = 0x4202422fu;
-        float xf;
-        memcpy(&xf, &bits, 4);
-        x = xf;
-        const float e = expf(x);
-        uint32_t eb;
-        memcpy(&eb, &e, 4);
-        return eb == 0x56fc9f1cu;  // 0x1.f93e38p+46: the fused-reduction result
-    }();
-    return v;
-}
-
 struct Plan {
     std::string modes;             // per input
     bool vector_ok = false;

@@ -334,6 +334,14 @@ def Conv(x, w, b=None, strides=(), pads=(), group=1, auto_pad="", out=None):
     return out
 
 
+def Softmax(x, axis=1, is_onnx_semantics=True, out=None):
+    """SoftmaxOp::RunImpl, runtime/ops/activation.cc:66-95, on a contiguous float32 array."""
+    if out is None:
+        out = torch.empty_like(x)
+    capi.check(capi.lib().chx_hip_softmax_f32(capi.ref(x), _i(axis), _i(1 if is_onnx_semantics else 0), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
 def FixedBatchNormalization(x, s, bias, mean, var, epsilon=1e-5, out=None):
     """FixedBatchNormalizationOp::RunImpl, runtime/ops/normalization.cc:210-225: BatchNormalization with stored
     statistics on a float32 array [N, C, ...]."""

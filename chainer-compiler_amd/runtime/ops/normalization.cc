@@ -1,6 +1,7 @@
 // FixedBatchNormalizationOp (runtime/ops/normalization.cc:210-225 of the chainer-compiler tree) on the hip
 // backend: the inference form of BatchNormalization, which the quantizer leaves in float behind an integer
-// convolution.  The arithmetic is chx_hip_fixed_batch_norm_f32.
+// convolution; and SoftmaxOp (runtime/ops/activation.cc:93-95).  The arithmetic is in chx_hip_fixed_batch_norm_f32
+// and chx_hip_softmax_f32.
 #include "../gen/gen_chxvm_ops.h"
 
 namespace chainer_compiler {
@@ -20,6 +21,20 @@ chainerx::Array FixedBatchNormalizationOp::RunImpl(
                                       : chainerx::Empty(x.shape(), chainerx::Dtype::kFloat32);
     chx_hip_tensor xt = x.hip(), st_ = sd.hip(), bt = bd.hip(), mt = md.hip(), vt = vd.hip(), yt = y.hip();
     CHXVM_HIP_CALL(chx_hip_fixed_batch_norm_f32(&xt, &st_, &bt, &mt, &vt, static_cast<float>(epsilon), &yt, chainerx::CurrentStream()));
+    return y;
+}
+
+// SoftmaxOp::RunImpl, runtime/ops/activation.cc:93-95 (RunSoftmax :66-89): the classifier head's last node.
+chainerx::Array SoftmaxOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
+    CHECK(input.dtype() == chainerx::Dtype::kFloat32) << "Softmax: float32 only on the hip backend, not " << input.dtype();
+    int ax = static_cast<int>(axis);
+    if (ax < 0) ax += input.ndim();
+    CHECK_LE(0, ax);
+    CHECK_GT(input.ndim(), ax);
+    const chainerx::Array x = AsContiguous(input);
+    chainerx::Array y = chainerx::Empty(x.shape(), chainerx::Dtype::kFloat32);
+    chx_hip_tensor xt = x.hip(), yt = y.hip();
+    CHXVM_HIP_CALL(chx_hip_softmax_f32(&xt, ax, is_onnx_semantics ? 1 : 0, &yt, chainerx::CurrentStream()));
     return y;
 }
 

@@ -293,6 +293,13 @@ int chx_hip_conv_f32(
         const chx_hip_tensor* x, const chx_hip_tensor* w, const chx_hip_tensor* b, const chx_hip_conv_params* params,
         chx_hip_tensor* y, void* stream);
 
+/* SoftmaxOp::RunImpl, runtime/ops/activation.cc:66-95 (chainerx::Softmax): x and y contiguous float32 of one
+ * shape; with is_onnx_semantics the axes from `axis` on are reduced together (RunSoftmax's reshape), otherwise
+ * `axis` alone.  m = max over the reduced elements, e = exp(x - m) as the host C library computes expf,
+ * s = the sum of e in ascending order from 0, y = e * (1 / s), one float32 rounding per operation.  (The sequence
+ * inside ChainerX's Softmax is not in the reference tree.) */
+int chx_hip_softmax_f32(const chx_hip_tensor* x, int32_t axis, int32_t is_onnx_semantics, chx_hip_tensor* y, void* stream);
+
 /* ---- pooling on quantized tensors ------------------------------------------------------ */
 
 /* MaxPoolOp::RunImpl, runtime/ops/pooling.cc:47-61, as it occurs in a quantized

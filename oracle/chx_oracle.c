@@ -37,6 +37,10 @@
  *   orc_average_pool_f32     pinned like orc_average_pool_q8 (tap-major numpy loop, both pad-count modes,
  *                            integer-valued images where every sum is exact, the whole-image window against
  *                            a sequential running sum); the same PARITY UNPINNED remainder.
+ *   orc_softmax_f32          pinned against float64 (relative error of a few roundings), rows sum to 1 within
+ *                            len roundings, exact shift invariance, both axis semantics against each other;
+ *                            PARITY UNPINNED for the sequence max / exp / ascending sum / multiply by the
+ *                            reciprocal: chainerx::Softmax is not in the tree.
  *   orc_conv_f32             pinned against float64 within the bound of a K-term float32 sum, bit for bit on
  *                            integer-valued operands (groups, strides, pads), against orc_gemm_f32 on the
  *                            explicitly expanded matrix; PARITY UNPINNED for the order (c, kh, kw):
@@ -688,6 +692,36 @@ void orc_average_pool_f32(
                 if (count_include_pad) cnt = (int32_t)(kh * kw);
                 y[(nc * OH + oh) * OW + ow] = sum / (float)cnt;
             }
+}
+
+/* SoftmaxOp::RunImpl, runtime/ops/activation.cc:66-95, on a dense [outer][len][inner] float32 array, reduced over len:
+ * m = max, e = expf(x - m) (the host libm, as std::exp in ChainerX's native kernel), s = the sum of e in ascending
+ * order from 0, result e * (1 / s); a NaN wins the maximum.  PARITY UNPINNED for this sequence (chainerx::Softmax is
+ * not in the tree); pinned against float64, by the rows summing to 1 within len roundings, and by shift invariance
+ * where the shift is exact. */
+void orc_softmax_f32(const float* x, int64_t outer, int64_t len, int64_t inner, float* y) {
+#pragma omp parallel for collapse(2) num_threads(g_threads) if (g_threads > 1)
+    for (int64_t o = 0; o < outer; ++o)
+        for (int64_t i = 0; i < inner; ++i) {
+            const float* xp = x + o * len * inner + i;
+            float* yp = y + o * len * inner + i;
+            float m = xp[0];
+            for (int64_t k = 1; k < len; ++k) {
+                const float v = xp[k * inner];
+                m = v > m ? v : m;
+                m = v != v ? v : m;
+            }
+            float s = 0.f;
+            for (int64_t k = 0; k < len; ++k) {
+                const float e = expf(xp[k * inner] - m);
+                s = s + e;
+            }
+            const float r = 1.0f / s;
+            for (int64_t k = 0; k < len; ++k) {
+                const float e = expf(xp[k * inner] - m);
+                yp[k * inner] = e * r;
+            }
+        }
 }
 
 /* ConvOp::RunImpl on float32, runtime/ops/connection.cc:24-30 (GroupedConv, runtime/chainerx_util.cc:313-340):

@@ -424,6 +424,22 @@ def average_pool(x, kernel, strides, pads=(0, 0), count_include_pad=False):
     return y
 
 
+def softmax(x, axis=1, is_onnx_semantics=True):
+    """SoftmaxOp::RunImpl, runtime/ops/activation.cc:66-95."""
+    x = _c(x, np.float32)
+    if axis < 0:
+        axis += x.ndim
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    if is_onnx_semantics:
+        length, inner = int(np.prod(x.shape[axis:], dtype=np.int64)), 1
+    else:
+        length, inner = x.shape[axis], int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    y = np.empty(x.shape, dtype=np.float32)
+    i64 = ctypes.c_int64
+    lib().orc_softmax_f32(_p(x), i64(outer), i64(length), i64(inner), _p(y))
+    return y
+
+
 def conv(x, w, bias=None, strides=(1, 1), pads=(0, 0), group=1, auto_pad=""):
     """ConvOp::RunImpl on float32, runtime/ops/connection.cc:24-30."""
     x, w = _c(x, np.float32), _c(w, np.float32)

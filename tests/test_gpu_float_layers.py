@@ -290,3 +290,37 @@ def test_conv_net_with_batch_normalization_under_the_default_quantization(g, vm,
     ref = torch.nn.functional.conv2d(ref, tx(w2), tx(b2), padding=1)
     ref = torch.nn.functional.max_pool2d(ref, 2).mean(dim=(2, 3)) @ tx(fc).T + tx(fb)
     assert np.abs(got - ref.numpy()).max() < 0.05 * np.abs(ref.numpy()).max() + 0.05
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 10), 1), ((3, 5, 7), 1), ((3, 5, 7), 2), ((2, 3, 4, 5), 1), ((6,), 0), ((64, 1000), -1),
+                                        ((2, 3, 4, 5), 0), ((1, 1), 1)], ids=str)
+def test_softmax_through_the_c_abi(g, oracle, shape, axis):
+    """Softmax with both axis semantics, bit for bit against the oracle (exp as the C library's expf on both sides)."""
+    rng = np.random.default_rng(len(shape) * 10 + axis)
+    x = (rng.standard_normal(shape) * 4).astype(np.float32)
+    x.reshape(-1)[::7] *= 12          # arguments far below the maximum: exp underflows to denormals and to 0
+    for onnx in (True, False):
+        got = g.host(g.ops.Softmax(g.dev(x), axis, onnx))
+        np.testing.assert_array_equal(bits(got), bits(oracle.softmax(x, axis, onnx)))
+    with pytest.raises(g.capi.ChxHipError, match="axis"):
+        g.ops.Softmax(g.dev(x), len(shape), True)
+
+
+def test_softmax_from_an_onnx_graph(g, vm, oracle):
+    """Gemm -> Softmax (the head of a classifier) through the emitter: attribute defaults axis = 1 and ONNX semantics,
+    and an explicit axis 0 (everything reduced together)."""
+    import test_compiler_cpu as cc
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((5, 12)).astype(np.float32)
+    w = rng.standard_normal((12, 7)).astype(np.float32)
+    N = cc.onnx_lite.Node
+    m = cc.model([N("Gemm", ["x", "w"], ["h"], {}), N("Softmax", ["h"], ["y"], {}), N("Softmax", ["h"], ["z"], {"axis": 0})],
+                 [("x", x.shape)], [("y", (5, 7)), ("z", (5, 7))], {"w": w})
+    insts = cc.decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))
+    assert [[v for _, v in i[1][1:]] for i in insts if i[0] == "Softmax"] == [[1, 1], [0, 1]]
+    prog = vm.Program(vm.compile_onnx(m, {"fuse": "none"}))
+    out = prog.run({"x": g.dev(x)})
+    prog.close()
+    h = oracle.gemm(x, w)
+    np.testing.assert_array_equal(bits(out["y"]), bits(oracle.softmax(h, 1, True)))
+    np.testing.assert_array_equal(bits(out["z"]), bits(oracle.softmax(h, 0, True)))

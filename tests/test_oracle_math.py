@@ -678,3 +678,34 @@ def test_float_conv_pins(oracle):
     col = col.transpose(0, 3, 4, 1, 2).reshape(2 * 36, 27)
     want = oracle.gemm(col, w.reshape(5, 27), trans_b=True).reshape(2, 6, 6, 5).transpose(0, 3, 1, 2)
     np.testing.assert_array_equal(oracle.conv(x, w, None, (1, 1), (1, 1)), want)
+
+
+def test_softmax_pins(oracle):
+    """orc_softmax_f32 against float64, rows summing to 1 within `len` roundings, shift invariance where the shift is
+    exact, and the two axis semantics of RunSoftmax (runtime/ops/activation.cc:66-89) against each other."""
+    rng = np.random.default_rng(91)
+    for shape, axis in [((4, 10), 1), ((3, 5, 7), 1), ((3, 5, 7), 2), ((2, 3, 4, 5), 1), ((6,), 0), ((2, 1000), -1)]:
+        x = (rng.standard_normal(shape) * 4).astype(np.float32)
+        for onnx in (True, False):
+            got = oracle.softmax(x, axis, onnx)
+            ax = axis % x.ndim
+            red = tuple(range(ax, x.ndim)) if onnx else (ax,)
+            x8 = x.astype(np.float64)
+            e = np.exp(x8 - x8.max(axis=red, keepdims=True))
+            exact = e / e.sum(axis=red, keepdims=True)
+            n = int(np.prod([x.shape[d] for d in red]))
+            assert (np.abs(got - exact) <= (n + 8) * 2.0 ** -24 * exact + 1e-45).all()
+            assert np.abs(got.astype(np.float64).sum(axis=red) - 1).max() <= (2 * n + 8) * 2.0 ** -24
+            # integer-valued rows: adding 16 changes nothing in x - max, so nothing in the result
+            xi = rng.integers(-20, 21, size=shape).astype(np.float32)
+            np.testing.assert_array_equal(oracle.softmax(xi + np.float32(16), axis, onnx), oracle.softmax(xi, axis, onnx))
+    x = (rng.standard_normal((3, 4, 5)) * 2).astype(np.float32)
+    # ONNX semantics at axis 1 = the reduction over the last axis of the array reshaped to [3, 20]
+    np.testing.assert_array_equal(oracle.softmax(x, 1, True), oracle.softmax(x.reshape(3, 20), 1, False).reshape(3, 4, 5))
+    # chainer semantics at axis 1 = over the last axis of the transposed array
+    np.testing.assert_array_equal(oracle.softmax(x, 1, False), oracle.softmax(x.transpose(0, 2, 1), 2, False).transpose(0, 2, 1))
+    # one element: exactly 1; a NaN spreads over its row only
+    assert oracle.softmax(np.array([[3.5]], np.float32), 1).tolist() == [[1.0]]
+    xn = np.array([[1, np.nan, 2], [1, 2, 3]], np.float32)
+    got = oracle.softmax(xn, 1)
+    assert np.isnan(got[0]).all() and not np.isnan(got[1]).any()
