@@ -188,6 +188,25 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         torch.cuda.synchronize()
         conv_ms_per_step += a.elapsed_time(b) / REP
         n_launch += len(fids)
+    # What the event figure contains besides the kernels: in a graph every kernel boundary costs a fixed time
+    # (the device hands one kernel's results to the next).  The same number of launches of a kernel that does
+    # nothing, timed the same way, measures it; a profiler's per-kernel durations leave most of it out, so the
+    # figure without it is the one to hold against profiles/.  frac below keeps the boundaries in.
+    tiny = torch.zeros(64, device="cuda")
+    idle = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(idle):
+        for _ in range(n_launch):
+            tiny.add_(1.0)
+    idle.replay()
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(REP):
+        idle.replay()
+    b.record()
+    torch.cuda.synchronize()
+    boundary_ms_per_step = a.elapsed_time(b) / REP
+    layer_graphs.append(idle)
     if mobilenet:
         achieved = model["depthwise_bytes"] / (conv_ms_per_step * 1e-3) / 1e9
         roofline = dict(bound="hbm", kernel="depthwise3x3_kernel (%d launches per step, summed)" % n_launch,
@@ -198,6 +217,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         roofline = dict(bound="mfma", kernel="QLinearConv launches of one step, summed (%d: conv_mfma_kernel, the first layer conv_stem_kernel)" % n_launch,
                         achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
                         ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
+    roofline["boundary_us_per_launch"] = boundary_ms_per_step * 1e3 / max(n_launch, 1)
+    roofline["kernel_ms_per_step_without_boundaries"] = conv_ms_per_step - boundary_ms_per_step
+    roofline["frac_without_boundaries"] = roofline["frac"] * conv_ms_per_step / max(conv_ms_per_step - boundary_ms_per_step, 1e-9)
     if not mobilenet and batch == 64 and args.parts <= 1:
         # HBM bytes of the same launches from hardware counters (FETCH_SIZE / WRITE_SIZE, scaled by a
         # copy kernel of known size): NOT measured in this run but taken from two separate profiling runs,
