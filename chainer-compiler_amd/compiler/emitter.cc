@@ -1,5 +1,6 @@
 #include "emitter.h"
 
+#include <algorithm>
 #include <map>
 #include <set>
 
@@ -366,6 +367,16 @@ private:
             // compiler/chxvm/simple_node_emitter.cc:213-219: a convolution the quantizer did not rewrite
             ChxVMInstructionProto* inst = simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true))});
             ConvAttrs(n, inst);
+        } else if (op == "Transpose" && nin == 1) {
+            simple(op, {ArrayIn(Operand(n, 0)), IntsIn(n.GetInts("perm"))});  // compiler/chxvm/simple_node_emitter.cc:523-526
+        } else if (op == "Squeeze" && nin == 1) {
+            simple(op, {ArrayIn(Operand(n, 0)), IntsIn(n.GetInts("axes"))});  // :297-300
+        } else if (op == "Unsqueeze" && nin == 1) {
+            // :301-311: the axes sorted; negative and positive ones together are refused
+            std::vector<int64_t> axes = n.GetInts("axes");
+            std::sort(axes.begin(), axes.end());
+            if (!axes.empty()) CHECK(!(axes.front() < 0 && axes.back() > 0)) << "Unsqueeze with negative/positive axes mixed is not supported";
+            simple(op, {ArrayIn(Operand(n, 0)), IntsIn(axes)});
         } else if (op == "Softmax" && nin == 1) {
             // compiler/chxvm/simple_node_emitter.cc:385-386; attribute defaults of compiler/gen_node.py:223
             simple(op, {ArrayIn(Operand(n, 0)), IntIn(n.GetInt("axis", 1)), IntIn(n.GetInt("chainer_is_onnx_semantics", 1))});

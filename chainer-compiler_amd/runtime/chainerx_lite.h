@@ -253,6 +253,9 @@ public:
     }
     // A view with permuted axes (no data movement), as chainerx::Array::Transpose.
     Array Transpose(std::initializer_list<int> perm) const {
+        return Transpose(std::vector<int>(perm));
+    }
+    Array Transpose(const std::vector<int>& perm) const {
         Array r;
         r.body_ = std::make_shared<Body>(*body_);
         r.body_->shape = Shape();

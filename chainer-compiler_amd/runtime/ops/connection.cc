@@ -89,5 +89,55 @@ chainerx::Array FlattenOp::RunImpl(ChxVMState* st, const chainerx::Array& input)
     return AsContiguous(input).Reshape(chainerx::Shape{d0, d1});
 }
 
+// TransposeOp::RunImpl, runtime/ops/manipulation.cc:101-107: a view; no perm reverses the axes, a perm shorter than
+// the rank leaves the remaining axes in place.
+chainerx::Array TransposeOp::RunImpl(ChxVMState* st, const chainerx::Array& data) {
+    std::vector<int> axes;
+    if (perm.empty()) {
+        for (int i = data.ndim() - 1; i >= 0; --i) axes.push_back(i);
+    } else {
+        for (int64_t p : perm) axes.push_back(static_cast<int>(p < 0 ? p + data.ndim() : p));
+        while (data.ndim() > static_cast<int>(axes.size())) axes.push_back(static_cast<int>(axes.size()));
+    }
+    CHECK_EQ(static_cast<size_t>(data.ndim()), axes.size()) << "Transpose: perm longer than the rank";
+    std::vector<bool> seen(axes.size(), false);
+    for (int a : axes) {
+        CHECK(a >= 0 && a < data.ndim() && !seen[a]) << "Transpose: perm is not a permutation of the axes";
+        seen[a] = true;
+    }
+    return data.Transpose(axes);
+}
+
+// SqueezeOp::RunImpl, runtime/ops/manipulation.cc:60-62 (chainerx::Squeeze): the named axes, which must have extent 1,
+// or every axis of extent 1 when none is named.
+chainerx::Array SqueezeOp::RunImpl(ChxVMState* st, const chainerx::Array& data) {
+    std::vector<bool> drop(data.ndim(), false);
+    if (axes.empty()) {
+        for (int i = 0; i < data.ndim(); ++i) drop[i] = data.shape()[i] == 1;
+    } else {
+        for (int64_t a : axes) {
+            const int ax = static_cast<int>(a < 0 ? a + data.ndim() : a);
+            CHECK(ax >= 0 && ax < data.ndim()) << "Squeeze: axis " << a << " out of range";
+            CHECK_EQ(1, data.shape()[ax]) << "Squeeze: axis " << a << " has extent " << data.shape()[ax];
+            drop[ax] = true;
+        }
+    }
+    chainerx::Shape shape;
+    for (int i = 0; i < data.ndim(); ++i)
+        if (!drop[i]) shape.push_back(data.shape()[i]);
+    return AsContiguous(data).Reshape(shape);
+}
+
+// UnsqueezeOp::RunImpl, runtime/ops/manipulation.cc:64-72.
+chainerx::Array UnsqueezeOp::RunImpl(ChxVMState* st, const chainerx::Array& data) {
+    std::vector<int64_t> dims(data.shape().begin(), data.shape().end());
+    for (int64_t a : axes) {
+        const int64_t d = a < 0 ? static_cast<int64_t>(dims.size() + axes.size()) + a : a;
+        CHECK(d >= 0 && d <= static_cast<int64_t>(dims.size())) << "Unsqueezing axis out of bound: " << d;
+        dims.insert(dims.begin() + d, 1);
+    }
+    return AsContiguous(data).Reshape(chainerx::Shape(dims.begin(), dims.end()));
+}
+
 }  // namespace runtime
 }  // namespace chainer_compiler

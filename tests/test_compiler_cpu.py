@@ -445,3 +445,17 @@ def test_float_conv_is_emitted_with_the_reference_operand_list(vm):
     insts = decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))                     # not quantized at all: a float Conv, no bias
     conv = next(i for i in insts if i[0] == "Conv")
     assert conv[1][2][1] == -1
+
+
+def test_view_nodes_are_emitted_with_the_reference_operand_lists(vm):
+    """Transpose(data, perm), Squeeze(data, axes), Unsqueeze(data, sorted axes): compiler/chxvm/simple_node_emitter.cc:297-311,
+    523-526; Unsqueeze refuses negative and positive axes together."""
+    N = onnx_lite.Node
+    m = model([N("Transpose", ["x"], ["t"], {"perm": [1, 0, 2]}), N("Squeeze", ["t"], ["s"], {"axes": [2]}), N("Unsqueeze", ["s"], ["y"], {"axes": [3, 0]})],
+              [("x", (2, 3, 1))], [("y", (1, 3, 2, 1))])
+    insts = {i[0]: i for i in decode_program(vm, vm.compile_onnx(m, {"fuse": "none"}))}
+    assert list(insts["Transpose"][1][1][1]) == [1, 0, 2] and list(insts["Squeeze"][1][1][1]) == [2]
+    assert list(insts["Unsqueeze"][1][1][1]) == [0, 3]
+    mixed = model([N("Unsqueeze", ["x"], ["y"], {"axes": [-1, 1]})], [("x", (2, 3))], [("y", (2, 1, 3, 1))])
+    with pytest.raises(vm.ChxVMError, match="mixed"):
+        vm.compile_onnx(mixed, {"fuse": "none"})

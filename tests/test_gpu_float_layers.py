@@ -324,3 +324,35 @@ def test_softmax_from_an_onnx_graph(g, vm, oracle):
     h = oracle.gemm(x, w)
     np.testing.assert_array_equal(bits(out["y"]), bits(oracle.softmax(h, 1, True)))
     np.testing.assert_array_equal(bits(out["z"]), bits(oracle.softmax(h, 0, True)))
+
+
+def test_views_between_the_float_layers(g, vm, oracle):
+    """Transpose (a view, no perm = reversed axes), Squeeze (named axes, or every axis of extent 1) and Unsqueeze
+    (runtime/ops/manipulation.cc:60-72, 101-107) as they occur between a pooled feature map and a classifier head:
+    GlobalAveragePool -> Squeeze -> Gemm -> Transpose -> Softmax over the other axis -> Unsqueeze."""
+    import test_compiler_cpu as cc
+    rng = np.random.default_rng(41)
+    N = cc.onnx_lite.Node
+    x = rng.standard_normal((4, 6, 3, 5)).astype(np.float32)
+    w = rng.standard_normal((6, 7)).astype(np.float32)
+    nodes = [N("GlobalAveragePool", ["x"], ["p"], {}), N("Squeeze", ["p"], ["s"], {"axes": [2, 3]}), N("Squeeze", ["p"], ["s_all"], {}),
+             N("Gemm", ["s", "w"], ["h"], {}), N("Transpose", ["h"], ["t"], {}), N("Softmax", ["t"], ["sm"], {"axis": 1}),
+             N("Unsqueeze", ["sm"], ["u"], {"axes": [0, 3]}), N("Transpose", ["x"], ["xt"], {"perm": [0, 2, 3, 1]}),
+             N("Unsqueeze", ["s_all"], ["u2"], {"axes": [-1]})]
+    outs = [("s_all", (4, 6)), ("t", (7, 4)), ("u", (1, 7, 4, 1)), ("xt", (4, 3, 5, 6)), ("u2", (4, 6, 1))]
+    m = cc.model(nodes, [("x", x.shape)], outs, {"w": w})
+    prog = vm.Program(vm.compile_onnx(m, {"fuse": "none"}))
+    out = prog.run({"x": g.dev(x)})
+    prog.close()
+    pooled = oracle.average_pool(x, (3, 5), (1, 1), (0, 0), False).reshape(4, 6)
+    h = oracle.gemm(pooled, w)
+    np.testing.assert_array_equal(out["s_all"], pooled)
+    np.testing.assert_array_equal(bits(out["t"]), bits(np.ascontiguousarray(h.T)))
+    np.testing.assert_array_equal(bits(out["u"]), bits(oracle.softmax(np.ascontiguousarray(h.T), 1, True).reshape(1, 7, 4, 1)))
+    np.testing.assert_array_equal(out["xt"], x.transpose(0, 2, 3, 1))
+    np.testing.assert_array_equal(out["u2"], pooled.reshape(4, 6, 1))
+    bad = cc.model([N("Squeeze", ["x"], ["y"], {"axes": [1]})], [("x", x.shape)], [("y", (4, 3, 5))])
+    prog = vm.Program(vm.compile_onnx(bad, {"fuse": "none"}))
+    with pytest.raises(vm.ChxVMError, match="extent 6"):
+        prog.run({"x": g.dev(x)})
+    prog.close()
