@@ -556,9 +556,12 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
             constexpr int kPath = decltype(path_tag)::value;
+            // a block of 32 output channels that lies beyond OC altogether (OC = 96 in a 128-wide tile, say) is not
+            // requantized: nobody reads its staged bytes (the test is the same for the whole wavefront)
             if constexpr (kPath == 0) {
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
+                for (int i = 0; i < FM; ++i) {
+                    if (oc0 + wm * 32 * FM + i * 32 >= a.OC) continue;
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
                         const int ocl = wm * 32 * FM + i * 32 + g * 8 + (lane >> 5) * 4;
@@ -578,11 +581,13 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                             *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
                         }
                     }
+                }
             } else {
                 // sixteen values (4 / FN row groups of the accumulator) per switch of the rounding mode
                 constexpr int G = 4 / FN;
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
+                for (int i = 0; i < FM; ++i) {
+                    if (oc0 + wm * 32 * FM + i * 32 >= a.OC) continue;
 #pragma unroll
                     for (int gb = 0; gb < 4; gb += G) {
                         float pre[16];
@@ -613,6 +618,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                                 *reinterpret_cast<uint32_t*>(staged(lds_out, wn * 32 * FN + j * 32 + (lane & 31), ocl)) = word[gl * FN + j];
                         }
                     }
+                }
             }
         };
         // The residual chunks this thread will add are requested now: their latency runs under the
