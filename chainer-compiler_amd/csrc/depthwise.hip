@@ -57,12 +57,15 @@ __global__ __launch_bounds__(256) void pack_depthwise_kernel(
 // Output rows per thread.  More rows spread the per-thread set-up (index arithmetic, masks, filter
 // rows and constants) and the two halo rows over more outputs, at the price of registers for the
 // loads in flight: stride 1 takes 14 rows when the output height is a multiple of 14 (224 / 2^k
-// images), otherwise 8.
-constexpr int rows_per_thread(int step, bool tall) { return step == 1 ? (tall ? 14 : 8) : step == 2 ? 4 : 1; }
+// images) and the image is at least 56 rows high; 7 when it is a multiple of 7 (the 28x28, 14x14 and 7x7 images: with 14
+// rows per thread a 14x14 layer at batch 128 is 2.6 wavefronts per SIMD, which is launch and memory latency and nothing
+// else; measured on MobileNetV2: the 17 launches 0.306 -> 0.292 ms); otherwise 8.
+// kStrip: 0 = 8 rows, 1 = 14, 2 = 7.
+constexpr int rows_per_thread(int step, int strip) { return step == 1 ? (strip == 1 ? 14 : strip == 2 ? 7 : 8) : step == 2 ? 4 : 1; }
 constexpr int kDwThreads = 64;  // small groups: (output columns x channel groups) of a row is rarely a multiple of 256
-template <bool kRne, bool kFloatBias, int kStep, int kPath, bool kTall>
+template <bool kRne, bool kFloatBias, int kStep, int kPath, int kStrip>
 __global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs a) {
-    constexpr int kRows = rows_per_thread(kStep, kTall);
+    constexpr int kRows = rows_per_thread(kStep, kStrip);
     constexpr int kInRows = kStep == 1 ? kRows + 2 : kStep == 2 ? 2 * kRows + 1 : 3;
     // grid: x over (output column, channel group) of one strip of output rows, y the strip, z the image
     const uint32_t idx = blockIdx.x * kDwThreads + threadIdx.x;
@@ -210,8 +213,8 @@ int pack_depthwise(const chx_hip_tensor& w, int32_t* rows, int32_t* wsum, hipStr
 
 int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
     const int step = a.sh == 1 ? 1 : a.sh == 2 ? 2 : 0;
-    const bool tall = step == 1 && a.OH % 14 == 0;
-    const int rows = rows_per_thread(step, tall);
+    const int strip = step != 1 ? 0 : (a.OH % 14 == 0 && a.OH >= 56) ? 1 : a.OH % 7 == 0 ? 2 : 0;
+    const int rows = rows_per_thread(step, strip);
     a.oh_blocks = (a.OH + rows - 1) / rows;
     a.total = (int64_t)a.N * a.oh_blocks * a.OW * (a.C / 4);
     if (a.total == 0) return CHX_HIP_OK;
@@ -231,10 +234,11 @@ int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
     } while (0)
 #define CHX_DW_S(RN, FB)                               \
     do {                                               \
-        if (tall) CHX_DW_P(RN, FB, 1, true);           \
-        else if (step == 1) CHX_DW_P(RN, FB, 1, false); \
-        else if (step == 2) CHX_DW_P(RN, FB, 2, false); \
-        else CHX_DW_P(RN, FB, 0, false);               \
+        if (strip == 1) CHX_DW_P(RN, FB, 1, 1);        \
+        else if (strip == 2) CHX_DW_P(RN, FB, 1, 2);   \
+        else if (step == 1) CHX_DW_P(RN, FB, 1, 0);    \
+        else if (step == 2) CHX_DW_P(RN, FB, 2, 0);    \
+        else CHX_DW_P(RN, FB, 0, 0);                   \
     } while (0)
     if (rne) {
         if (fbias) CHX_DW_S(true, true);

@@ -235,8 +235,9 @@ def test_errors(g):
 @pytest.mark.parametrize("case", [
     # N, C, H, W, stride, pad
     (2, 32, 9, 10, 1, 1), (1, 96, 13, 12, 2, 1), (2, 16, 7, 7, 1, 0), (1, 144, 5, 6, 2, 0), (1, 48, 4, 4, 1, 1),
-    # 14 and 28 output rows (the 14-row strips), a stride the row reuse does not cover, strides that differ
-    (1, 16, 14, 5, 1, 1), (1, 16, 30, 3, 1, 0), (1, 32, 11, 10, 3, 1), (1, 16, 12, 9, (2, 1), 1), (1, 16, 9, 12, (1, 3), 1)])
+    # 14, 28, 21 and 7 output rows (strips of 7), 56 (strips of 14), a stride the row reuse does not cover, strides that differ
+    (1, 16, 14, 5, 1, 1), (1, 16, 30, 3, 1, 0), (1, 16, 21, 4, 1, 1), (1, 16, 7, 9, 1, 1), (1, 16, 58, 3, 1, 0),
+    (1, 32, 11, 10, 3, 1), (1, 16, 12, 9, (2, 1), 1), (1, 16, 9, 12, (1, 3), 1)])
 def test_depthwise_qlinear_conv(g, oracle, case, xdt):
     """Depthwise 3x3 on channels-last operands (the row-packing kernel), stateless call and plan,
     both bias modes, fused Relu in both roundings; NCHW operands take the generic kernel and must
