@@ -367,6 +367,10 @@ private:
             // compiler/chxvm/simple_node_emitter.cc:213-219: a convolution the quantizer did not rewrite
             ChxVMInstructionProto* inst = simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), OptionalArrayIn(Operand(n, 2, true))});
             ConvAttrs(n, inst);
+        } else if (op == "Concat" && nin >= 1) {
+            std::vector<int> ins;  // compiler/chxvm/simple_node_emitter.cc:490-494
+            for (size_t i = 0; i < nin; ++i) ins.push_back(Operand(n, i));
+            simple(op, {ArrayListIn(ins), IntIn(n.GetInt("axis", 1))});
         } else if (op == "Transpose" && nin == 1) {
             simple(op, {ArrayIn(Operand(n, 0)), IntsIn(n.GetInts("perm"))});  // compiler/chxvm/simple_node_emitter.cc:523-526
         } else if (op == "Squeeze" && nin == 1) {

@@ -267,6 +267,15 @@ public:
         return r;
     }
 
+    // A view of `length` positions of one axis from `start` on (no data movement).
+    Array Narrow(int axis, int64_t start, int64_t length) const {
+        Array r;
+        r.body_ = std::make_shared<Body>(*body_);
+        r.body_->offset = body_->offset + start * body_->strides[axis];
+        r.body_->shape[axis] = length;
+        return r;
+    }
+
     // A view of a contiguous array with another shape of the same size.
     Array Reshape(const Shape& to) const;
 

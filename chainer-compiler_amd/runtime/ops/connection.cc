@@ -89,6 +89,38 @@ chainerx::Array FlattenOp::RunImpl(ChxVMState* st, const chainerx::Array& input)
     return AsContiguous(input).Reshape(chainerx::Shape{d0, d1});
 }
 
+// ConcatOp::RunImpl, runtime/ops/manipulation.cc:74-76 (chainerx::Concatenate): every input is copied into its span of
+// the result (a strided device copy each); the result is laid out like the first input when all of them are
+// channels-last feature maps, dense otherwise.
+chainerx::Array ConcatOp::RunImpl(ChxVMState* st, const std::vector<chainerx::Array>& inputs) {
+    CHECK(!inputs.empty()) << "Concat: no inputs";
+    const chainerx::Array& first = inputs[0];
+    const int ax = static_cast<int>(axis < 0 ? axis + first.ndim() : axis);
+    CHECK(ax >= 0 && ax < first.ndim()) << "Concat: axis " << axis << " out of range";
+    chainerx::Shape shape = first.shape();
+    int64_t total = 0;
+    bool channels_last = true;
+    for (const chainerx::Array& a : inputs) {
+        CHECK(a.dtype() == first.dtype()) << "Concat: inputs of different types";
+        CHECK_EQ(first.ndim(), a.ndim()) << "Concat: inputs of different rank";
+        for (int d = 0; d < a.ndim(); ++d)
+            if (d != ax) CHECK_EQ(first.shape()[d], a.shape()[d]) << "Concat: extents differ on axis " << d;
+        total += a.shape()[ax];
+        channels_last = channels_last && a.ndim() == 4 && !a.IsContiguous() && a.strides()[1] == a.GetItemSize();
+    }
+    shape[ax] = total;
+    chainerx::Array y = channels_last ? chainerx::EmptyChannelsLast(shape, first.dtype()) : chainerx::Empty(shape, first.dtype());
+    int64_t at = 0;
+    for (const chainerx::Array& a : inputs) {
+        if (a.shape()[ax] == 0) continue;
+        const chainerx::Array span = y.Narrow(ax, at, a.shape()[ax]);
+        chx_hip_tensor xt = a.hip(), yt = span.hip();
+        CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, chainerx::CurrentStream()));  // same element type on both sides: a strided copy
+        at += a.shape()[ax];
+    }
+    return y;
+}
+
 // TransposeOp::RunImpl, runtime/ops/manipulation.cc:101-107: a view; no perm reverses the axes, a perm shorter than
 // the rank leaves the remaining axes in place.
 chainerx::Array TransposeOp::RunImpl(ChxVMState* st, const chainerx::Array& data) {

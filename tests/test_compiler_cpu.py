@@ -459,3 +459,11 @@ def test_view_nodes_are_emitted_with_the_reference_operand_lists(vm):
     mixed = model([N("Unsqueeze", ["x"], ["y"], {"axes": [-1, 1]})], [("x", (2, 3))], [("y", (2, 1, 3, 1))])
     with pytest.raises(vm.ChxVMError, match="mixed"):
         vm.compile_onnx(mixed, {"fuse": "none"})
+
+
+def test_concat_is_emitted_with_an_array_list(vm):
+    """compiler/chxvm/simple_node_emitter.cc:490-494: Concat(inputs as one list, axis)."""
+    N = onnx_lite.Node
+    m = model([N("Concat", ["a", "b", "a"], ["y"], {"axis": 2})], [("a", (2, 3, 1)), ("b", (2, 3, 4))], [("y", (2, 3, 6))])
+    cat = next(i for i in decode_program(vm, vm.compile_onnx(m, {"fuse": "none"})) if i[0] == "Concat")
+    assert [t for t, _ in cat[1]] == ["ARRAY_LIST", "INT"] and len(cat[1][0][1]) == 3 and cat[1][1][1] == 2

@@ -356,3 +356,38 @@ def test_views_between_the_float_layers(g, vm, oracle):
     with pytest.raises(vm.ChxVMError, match="extent 6"):
         prog.run({"x": g.dev(x)})
     prog.close()
+
+
+def test_concat_as_a_program_instruction(g, vm):
+    """ConcatOp::RunImpl (runtime/ops/manipulation.cc:74-76): along the channel axis of NCHW and of channels-last feature
+    maps, along the first and the last axis, float32 and uint8; inputs of different extents on the axis."""
+    import test_compiler_cpu as cc
+    rng = np.random.default_rng(51)
+    N = cc.onnx_lite.Node
+    a = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    b = rng.standard_normal((2, 5, 4, 5)).astype(np.float32)
+    c = rng.standard_normal((2, 1, 4, 5)).astype(np.float32)
+    m = cc.model([N("Concat", ["a", "b", "c"], ["ch"], {"axis": 1}), N("Concat", ["a", "a"], ["n"], {"axis": 0}),
+                  N("Concat", ["a", "a", "a"], ["w"], {"axis": -1})],
+                 [("a", a.shape), ("b", b.shape), ("c", c.shape)], [("ch", (2, 9, 4, 5)), ("n", (4, 3, 4, 5)), ("w", (2, 3, 4, 15))])
+    prog = vm.Program(vm.compile_onnx(m, {"fuse": "none"}))
+    for lay in (g.dev, lambda t: g.to_channels_last(g.dev(t))):
+        out = prog.run({"a": lay(a), "b": lay(b), "c": lay(c)})
+        np.testing.assert_array_equal(out["ch"], np.concatenate([a, b, c], axis=1))
+        np.testing.assert_array_equal(out["n"], np.concatenate([a, a], axis=0))
+        np.testing.assert_array_equal(out["w"], np.concatenate([a, a, a], axis=3))
+    prog.close()
+    # codes: a builder program, since ONNX value infos of the test helper are float
+    qa = rng.integers(0, 256, size=(1, 16, 3, 3)).astype(np.uint8)
+    qb = rng.integers(0, 256, size=(1, 32, 3, 3)).astype(np.uint8)
+    bld = vm.ProgramBuilder()
+    sa, sb = bld.input("a", "uint8", qa.shape), bld.input("b", "uint8", qb.shape)
+    y = bld.new_slot()
+    bld.add_raw("Concat", [("ARRAY_LIST", [sa, sb]), ("INT", 1)], [y])
+    bld.output("y", y)
+    prog = vm.Program(bld.serialize())
+    out = prog.run({"a": g.to_channels_last(g.dev(qa)), "b": g.to_channels_last(g.dev(qb))})
+    np.testing.assert_array_equal(out["y"], np.concatenate([qa, qb], axis=1))
+    with pytest.raises(vm.ChxVMError, match="extents differ"):
+        prog.run({"a": g.dev(qa), "b": g.dev(qb[:, :, :2])})
+    prog.close()
