@@ -68,6 +68,7 @@ struct ConvMfmaArgs {
     int32_t tiles_oc, tiles_px;  // filled by the launcher
     uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
     uint32_t row_unit;           // bit i*KW set for every filter row i (when KH*KW <= 32), filled by the launcher
+    int32_t px_linear;           // 1x1, stride 1, no padding over a dense image: input pixel m is at x + m * x_w_stride (launcher)
     ResidualAdd res;             // res.r == nullptr: plain QLinearConv
 };
 

@@ -393,6 +393,12 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
             const bool row_ok = m < a.M && ld_tile < px_hi;
             // rows past the end re-read the last pixel; they are never written back
             const uint32_t mm = m < a.M ? (uint32_t)m : (uint32_t)(a.M - 1);  // M fits 31 bits (checked on the host)
+            if (a.px_linear) {
+                // output pixel m reads input pixel m: no decomposition into (n, oh, ow), one multiplication
+                xb[j] = a.x + (int64_t)mm * a.x_w_stride + kc * 16;
+                if (kPad) tapmask[j] = row_ok ? 1u : 0u;  // the one tap is inside the image
+                continue;
+            }
             const uint32_t r = fast_div(mm, a.ow_mul, a.ow_shift);
             const uint32_t ow = mm - r * (uint32_t)a.OW;
             const uint32_t n = fast_div(r, a.oh_mul, a.oh_shift);
@@ -977,6 +983,8 @@ int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_c
     if (a.M == 0 || a.OC == 0) return CHX_HIP_OK;
     magic_divisor((uint32_t)a.OW, &a.ow_mul, &a.ow_shift);
     magic_divisor((uint32_t)a.OH, &a.oh_mul, &a.oh_shift);
+    a.px_linear = a.KH == 1 && a.KW == 1 && a.sh == 1 && a.sw == 1 && a.ph == 0 && a.pw == 0 && a.OH == a.H && a.OW == a.W &&
+                  a.x_h_stride == (int64_t)a.W * a.x_w_stride && a.x_n_stride == (int64_t)a.H * a.x_h_stride;
     a.row_unit = 0;
     if (a.KH * a.KW <= 32)
         for (int i = 0; i < a.KH; ++i) a.row_unit |= 1u << (i * a.KW);
