@@ -187,7 +187,7 @@ chainerx::Array MatMulIntegerOp::RunImpl(
     if (a_zero_point.has_value()) azt = a_zero_point->hip();
     if (b_zero_point.has_value()) bzt = b_zero_point->hip();
     CHXVM_HIP_CALL(chx_hip_matmul_integer(&at, &bt, a_zero_point.has_value() ? &azt : nullptr,
-                                          b_zero_point.has_value() ? &bzt : nullptr, &yt, nullptr));
+                                          b_zero_point.has_value() ? &bzt : nullptr, &yt, chainerx::CurrentStream()));
     return y;
 }
 
@@ -202,7 +202,7 @@ chainerx::Array ConvIntegerOp::RunImpl(
     chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), yt = y.hip(), zt;
     if (w_zero_point_opt.has_value()) zt = w_zero_point_opt->hip();
     const int32_t xz = x_zero_point.has_value() ? static_cast<int32_t>(static_cast<int64_t>(*x_zero_point)) : 0;
-    CHXVM_HIP_CALL(chx_hip_conv_integer(&xt, &wt, xz, w_zero_point_opt.has_value() ? &zt : nullptr, &p, &yt, nullptr));
+    CHXVM_HIP_CALL(chx_hip_conv_integer(&xt, &wt, xz, w_zero_point_opt.has_value() ? &zt : nullptr, &p, &yt, chainerx::CurrentStream()));
     return y;
 }
 
