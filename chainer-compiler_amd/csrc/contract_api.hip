@@ -532,6 +532,17 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
         return rc;
     }
     a.C16 = C16eff;
+    {
+        // bytes from x to the end of the last pixel's C16 channels (the strides of the three cases above are positive)
+        const int64_t n_img = pw.dense ? 1 : cs.N, h_img = pw.dense ? 1 : H, w_img = pw.dense ? (int64_t)cs.N * cs.OH * cs.OW : W;
+        const int64_t span = (n_img - 1) * a.x_n_stride + (h_img - 1) * a.x_h_stride + (w_img - 1) * a.x_w_stride + C16eff;
+        if (span >= (int64_t(1) << 31) - (int64_t(1) << 24)) {
+            release_scratch(c.cache, x_scratch, s);
+            release_scratch(c.cache, y_scratch, s);
+            CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv: the activations span 2 GB or more, which the MFMA kernel does not address");
+        }
+        a.x_bytes = (uint32_t)span;
+    }
     a.C64 = pw.C64;
     a.H = H; a.W = W; a.KH = KH; a.KW = KW;
     a.OH = pw.dense ? 1 : cs.OH;

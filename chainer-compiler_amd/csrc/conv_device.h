@@ -46,6 +46,64 @@ __device__ __forceinline__ void async_copy16(const void* src, uint32_t lds_addr)
             : "memory", "m0");
 }
 
+// Raw buffer resource over `bytes` bytes at `base` (no stride, no swizzle): an access at byte offset
+// voffset + soffset + immediate that does not lie inside [0, bytes) reads zeros, and an asynchronous
+// copy writes those zeros into LDS.
+__device__ __forceinline__ v4i buffer_resource(const void* base, uint32_t bytes) {
+    const uint64_t p = (uint64_t)base;
+    v4i r;
+    r[0] = (int)(uint32_t)p;
+    r[1] = (int)((uint32_t)(p >> 32) & 0xffffu);
+    r[2] = (int)bytes;
+    r[3] = 0x00020000;
+    // The resource is the same in every lane; saying so here makes the compiler keep it in scalar registers, where the
+    // "s" operands of the copies below need it (the constraint alone does not: the compiler has handed over vector
+    // registers for values it had decided to hold in them, which the assembler refuses).
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = __builtin_amdgcn_readfirstlane(r[i]);
+    return r;
+}
+
+// The same for a 32-bit value that is the same in every lane.
+__device__ __forceinline__ void keep_scalar(uint32_t& v) { v = (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ void keep_scalar(int& v) { v = __builtin_amdgcn_readfirstlane(v); }
+
+// Per-lane byte offsets handed to buffer copies carry this bit when the lane must not fetch anything:
+// the offset then lies beyond any resource this library builds (at most 2^31 - 1 bytes).
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+// Copies Q0 .. Q0+N-1 of a wave's group of up to four asynchronous 16-byte-per-lane copies through a buffer
+// resource into LDS, as one statement so that nothing can touch M0 between them.  Copy q reads byte offset
+// voff[q] + soff + q*1024 of the resource and lane i writes LDS bytes [lds_addr + q*1024 + 16*i, + 16): the
+// immediate of the instruction is added on both sides, so the per-lane offsets handed in have q*1024
+// subtracted already.
+template <int N, int Q0>
+__device__ __forceinline__ void buffer_copy16_run(const uint32_t (&voff)[4], v4i srd, uint32_t soff, uint32_t lds_addr) {
+    static_assert(N >= 1 && Q0 >= 0 && Q0 + N <= 4, "the 12-bit immediate reaches four copies of 1 KB");
+    if constexpr (N == 1)
+        asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                     "buffer_load_dwordx4 %0, %1, %2 offen offset:%4 lds"
+                     : : "v"(voff[Q0]), "s"(srd), "s"(soff), "s"(lds_addr), "n"(Q0 * 1024) : "memory", "m0");
+    else if constexpr (N == 2)
+        asm volatile("s_mov_b32 m0, %4\n\ts_nop 0\n\t"
+                     "buffer_load_dwordx4 %0, %2, %3 offen offset:%5 lds\n\t"
+                     "buffer_load_dwordx4 %1, %2, %3 offen offset:%6 lds"
+                     : : "v"(voff[Q0]), "v"(voff[Q0 + 1]), "s"(srd), "s"(soff), "s"(lds_addr), "n"(Q0 * 1024), "n"(Q0 * 1024 + 1024) : "memory", "m0");
+    else if constexpr (N == 3)
+        asm volatile("s_mov_b32 m0, %5\n\ts_nop 0\n\t"
+                     "buffer_load_dwordx4 %0, %3, %4 offen offset:%6 lds\n\t"
+                     "buffer_load_dwordx4 %1, %3, %4 offen offset:%7 lds\n\t"
+                     "buffer_load_dwordx4 %2, %3, %4 offen offset:%8 lds"
+                     : : "v"(voff[Q0]), "v"(voff[Q0 + 1]), "v"(voff[Q0 + 2]), "s"(srd), "s"(soff), "s"(lds_addr), "n"(Q0 * 1024), "n"(Q0 * 1024 + 1024), "n"(Q0 * 1024 + 2048) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %6\n\ts_nop 0\n\t"
+                     "buffer_load_dwordx4 %0, %4, %5 offen lds\n\t"
+                     "buffer_load_dwordx4 %1, %4, %5 offen offset:1024 lds\n\t"
+                     "buffer_load_dwordx4 %2, %4, %5 offen offset:2048 lds\n\t"
+                     "buffer_load_dwordx4 %3, %4, %5 offen offset:3072 lds"
+                     : : "v"(voff[0]), "v"(voff[1]), "v"(voff[2]), "v"(voff[3]), "s"(srd), "s"(soff), "s"(lds_addr) : "memory", "m0");
+}
+
 // Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
 // (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
 // reference's order, one IEEE operation each.

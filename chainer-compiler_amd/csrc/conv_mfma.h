@@ -40,8 +40,12 @@ constexpr int kAffineCandidates = 5 * 5 * 13;
 
 struct ConvMfmaArgs {
     // activations, channels-last: element (n, c, ih, iw) at x + n*x_n_stride + ih*x_h_stride + iw*x_w_stride + c
+    // The bytes [x, x + x_bytes) hold every element of x and nothing the kernel may not read; x_bytes and every
+    // stride are below 2^31 (the kernel addresses x with 32-bit offsets through a buffer resource).
     const char* x;
     int64_t x_n_stride, x_h_stride, x_w_stride;
+    uint32_t x_bytes;
+    uint32_t x_bias;  // filled by the launcher: what the kernel adds to every offset into x so that taps in the padding stay non-negative
     int32_t C16;  // channels rounded up to 16; the pixel pitch covers at least this many bytes
     int32_t C64;  // channels rounded up to 64 (K bytes per filter tap in the packed weights)
     int32_t H, W, OH, OW, KH, KW, sh, sw, ph, pw;
@@ -68,6 +72,10 @@ struct ConvMfmaArgs {
     int32_t tiles_oc, tiles_px;  // filled by the launcher
     uint32_t ow_mul, ow_shift, oh_mul, oh_shift;  // magic_divisor(OW), magic_divisor(OH), filled by the launcher
     uint32_t row_unit;           // bit i*KW set for every filter row i (when KH*KW <= 32), filled by the launcher
+    uint32_t tiles_oc_mul, tiles_oc_shift;  // magic_divisor(tiles_oc), filled by the launcher
+    int32_t px_slots;                       // pixel-tile slots per XCD of the launch's grid: gridDim.x / 8 / tiles_oc (launcher)
+    uint32_t px_slots_mul, px_slots_shift;  // magic_divisor(px_slots)
+    uint32_t tap_step_col, tap_step_row;  // what the scalar offset into x gains from the last K step of a filter tap to the first of the next: one pixel to the right, or to the first column of the next filter row (launcher)
     int32_t px_linear;           // 1x1, stride 1, no padding over a dense image: input pixel m is at x + m * x_w_stride (launcher)
     ResidualAdd res;             // res.r == nullptr: plain QLinearConv
 };
@@ -134,6 +142,16 @@ int launch_conv_stem(ConvStemArgs a, bool rne, hipStream_t s);
 // p->affine (1 when a candidate without mismatch exists; then kc, kr, k0, floor_pre are filled in).  Only for uint8
 // sums without the range guard; otherwise p->affine stays 0.  `scratch` holds kAffineCandidates int32 on the device.
 int find_affine_residual(ResidualAdd* p, int32_t* scratch, hipStream_t s);
+
+// One launcher per tile shape (FM x FN MFMA tiles per wavefront, K bytes per step, wavefronts along the pixels), each
+// in a translation unit of its own (conv_mfma_t*.hip).
+#define CHX_CONV_MFMA_TILES(X) \
+    X(2, 1, 128, 4) X(2, 1, 64, 4) X(2, 2, 128, 4) X(1, 1, 128, 4) X(2, 2, 128, 2) X(2, 2, 64, 2) X(1, 2, 128, 2) X(1, 2, 64, 2) \
+    X(2, 1, 128, 2) X(2, 1, 64, 2) X(1, 1, 128, 2) X(1, 1, 64, 2)
+#define CHX_CONV_MFMA_DECLARE(FM, FN, BK, NWN) \
+    int launch_conv_mfma_##FM##_##FN##_##BK##_##NWN(const ConvMfmaArgs& a, bool x_unsigned, bool out_int32, bool rne, int max_wgs_per_cu, hipStream_t s);
+CHX_CONV_MFMA_TILES(CHX_CONV_MFMA_DECLARE)
+#undef CHX_CONV_MFMA_DECLARE
 
 int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_cu, int waves, bool x_unsigned, bool out_int32, bool rne,
                      hipStream_t s);
