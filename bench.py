@@ -47,6 +47,8 @@ def parse():
                     help="network workloads: chxvm = the serialized ChxVMProgramProto through the C++ VM of the runtime library "
                          "(libchxvm_hip_runtime.so), its run recorded into a device graph and replayed; python = the op program "
                          "driven from Python through the C ABI (ops.py), also replayed as a graph")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default workload only: do not append the short runs of the other configurations (other_workloads)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one plain copy kernel (fused Identity on float32) over this many MiB: the known traffic "
                          "that hardware counters of a profiling run are scaled against")
@@ -217,6 +219,21 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         roofline = dict(bound="mfma", kernel="QLinearConv launches of one step, summed (%d: conv_mfma_kernel, the first layer conv_stem_kernel)" % n_launch,
                         achieved=achieved, peak=INT8_PEAK_TOPS, unit="TOP/s", frac=achieved / INT8_PEAK_TOPS, traffic=None,
                         ops_per_step=conv_ops, kernel_ms_per_step=conv_ms_per_step)
+    # The same launches against BOTH roofs: a launch is priced at the roof that takes longer for its algorithmic
+    # operations and bytes (input pixels it needs, weights, output, residual operand; workloads.conv_layer_table);
+    # most 1x1 layers of these networks are below the ridge of 625 op/byte and belong to the HBM roof.  For
+    # MobileNetV2 the figure covers every QLinearConv launch, not only the depthwise ones timed above.
+    table = wl.conv_layer_table(model, fuse)
+    floor_s = sum(max(r["ops"] / (INT8_PEAK_TOPS * 1e12), r["bytes"] / (HBM_PEAK_GBS * 1e9)) for r in table)
+    n_mfma = sum(1 for r in table if r["ops"] / (INT8_PEAK_TOPS * 1e12) >= r["bytes"] / (HBM_PEAK_GBS * 1e9))
+    roofline["mixed"] = dict(
+        floor_ms=floor_s * 1e3, mfma_only_ms=sum(r["ops"] for r in table) / (INT8_PEAK_TOPS * 1e12) * 1e3,
+        hbm_only_ms=sum(r["bytes"] for r in table) / (HBM_PEAK_GBS * 1e9) * 1e3,
+        algorithmic_bytes_per_step=sum(r["bytes"] for r in table), launches=len(table),
+        launches_mfma_class=n_mfma, launches_hbm_class=len(table) - n_mfma)
+    if not mobilenet:
+        roofline["mixed"]["frac"] = floor_s * 1e3 / conv_ms_per_step
+    roofline["launches_per_step"] = len(model["program"]) - (sum(1 for r in table if r["residual"]) if fuse else 0)
     roofline["boundary_us_per_launch"] = boundary_ms_per_step * 1e3 / max(n_launch, 1)
     roofline["kernel_ms_per_step_without_boundaries"] = conv_ms_per_step - boundary_ms_per_step
     roofline["frac_without_boundaries"] = roofline["frac"] * conv_ms_per_step / max(conv_ms_per_step - boundary_ms_per_step, 1e-9)
@@ -246,6 +263,8 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
                 key = "%s/%s/w%s%s" % (f.get("tile"), f.get("wgs_per_cu"), f.get("waves", "4"), "+res" if f.get("res") == "1" else "")
                 hist[key] = hist.get(key, 0) + 1
     roofline["configs"] = hist
+    roofline["configs_source"] = ("plans of the Python runner (ops.py), whose launches the kernel time above is measured on; the "
+                                  "plans inside the C++ VM measure their own configurations and may choose differently")
     if forms:
         roofline["residual_sums"] = forms
     res = dict(metric="images/sec %s int8 bs%d @1 GPU" % ("MobileNetV2" if mobilenet else "ResNet-50", batch),
@@ -272,8 +291,16 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         t0 = time.perf_counter()
         wl.run_reference(many, lit, many["input"])
         dtn = time.perf_counter() - t0
+        # Where the integer-accumulating restatement (which the device is held to, bit for bit) and the literal fp32
+        # restatement of QLinearConvOp differ: every convolution of three images computed both ways on the same
+        # input.  Reported, not gated.
+        three = build(batch=3)
+        cnt = _MismatchCounter(orc)
+        wl.run_reference(three, cnt, three["input"])
         orc.set_threads(1)
-        return dict(value=nb / dtn, unit="images/sec", cores=cores, kind="port", single_thread_value=1.0 / dt1,
+        parity = dict(images=3, elements=cnt.elements, literal_differs_from_int=cnt.differ,
+                      largest_difference_in_codes=cnt.largest, layers_with_a_difference=cnt.layers)
+        return dict(value=nb / dtn, unit="images/sec", cores=cores, kind="port", single_thread_value=1.0 / dt1, literal_vs_int=parity,
                     sample="%d images of the same network (batch %d), restated reference op sequence (fp32 dequantize, "
                            "im2col + sequential-k fp32 GEMM, quantize) with OpenMP over %d threads: %.1f s; one image "
                            "single-threaded, as ChainerX's native device runs: %.1f s" % (nb, nb, cores, dtn, dt1))
@@ -295,6 +322,28 @@ def _literal_executor(orc):
         def qlinear_conv_int(self, *a, **k):
             return orc.qlinear_conv_literal(*a, **k)
     return Lit()
+
+
+class _MismatchCounter(object):
+    """The oracle with QLinearConv computed both ways: returns the integer-accumulating result, counts the output
+    elements on which the literal fp32 restatement differs from it."""
+
+    def __init__(self, orc):
+        self.orc, self.elements, self.differ, self.largest, self.layers = orc, 0, 0, 0, 0
+
+    def __getattr__(self, name):
+        return getattr(self.orc, name)
+
+    def qlinear_conv_int(self, *a, **k):
+        import numpy as np
+        yi = self.orc.qlinear_conv_int(*a, **k)
+        yl = self.orc.qlinear_conv_literal(*a, **k)
+        d = np.abs(yi.astype(np.int32) - yl.astype(np.int32))
+        self.elements += d.size
+        self.differ += int(np.count_nonzero(d))
+        self.largest = max(self.largest, int(d.max()) if d.size else 0)
+        self.layers += 1 if d.any() else 0
+        return yi
 
 
 def bench_conv3x3(args, torch, pkg):
@@ -350,7 +399,12 @@ def bench_conv3x3(args, torch, pkg):
         orc.qlinear_conv_literal(x, 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1),
                                  bias_mode=orc.BIAS_ONNX_INT32)
         dt1 = time.perf_counter() - t1
-        return dict(value=reps * n / dt, unit="images/sec", cores=cores, kind="port", single_thread_value=n / dt1,
+        orc.set_threads(cores)
+        cnt = _MismatchCounter(orc)
+        cnt.qlinear_conv_int(x, 0.02, 128, w, ws, wz, 0.05, 128, np.uint8, bias=bias, pads=(1, 1), bias_mode=orc.BIAS_ONNX_INT32)
+        orc.set_threads(1)
+        parity = dict(elements=cnt.elements, literal_differs_from_int=cnt.differ, largest_difference_in_codes=cnt.largest)
+        return dict(value=reps * n / dt, unit="images/sec", cores=cores, kind="port", single_thread_value=n / dt1, literal_vs_int=parity,
                     sample="%d passes over all %d images, literal fp32 restatement of QLinearConvOp (dequantize, im2col + "
                            "sequential-k GEMM, quantize), %d threads: %.1f s; one pass single-threaded: %.1f s" % (
                                reps, n, cores, dt, dt1))
@@ -436,7 +490,31 @@ def main():
         code = pkg.ops.fusion_program([("x", torch.float32)], [("y", "Identity", "x")], [("y", torch.float32)])
         pkg.ops.ElementWiseNvrtc([src], 1, code, 9999)
         torch.cuda.synchronize()
+    others = None
+    if args.workload == "resnet50" and not args.no_other_workloads and not args.batch and not args.no_graph:
+        # the other configurations, shortly, so that one run reports all of them (their own --workload runs time them longer)
+        import copy
+        close()
+        close = lambda: None
+        others = []
+        for name in ("conv3x3", "fusion", "qdq", "mobilenetv2"):
+            a2 = copy.copy(args)
+            a2.workload, a2.steps, a2.warmup = name, 10, 3
+            torch.cuda.empty_cache()
+            if name == "mobilenetv2":
+                r2, roof2, _cpu2, close2 = bench_resnet50(a2, torch, pkg, mobilenet=True)
+            elif name == "conv3x3":
+                r2, roof2, _cpu2, close2 = bench_conv3x3(a2, torch, pkg)
+            else:
+                r2, roof2, _cpu2, close2 = bench_fusion(a2, torch, pkg, qdq=name == "qdq")
+            close2()
+            others.append(dict(workload=r2["config"]["workload"], metric=r2["metric"], value=r2["value"], unit=r2["unit"],
+                               ms_per_step=r2["ms_per_step"], steps=a2.steps, warmup=a2.warmup,
+                               roofline=dict(bound=roof2["bound"], kernel=roof2["kernel"], frac=roof2["frac"], achieved=roof2["achieved"],
+                                             unit=roof2["unit"], kernel_us=roof2.get("launch_us", roof2.get("kernel_ms_per_step", 0.0) * 1e3 if "kernel_ms_per_step" in roof2 else None))))
     out = dict(res)
+    if others is not None:
+        out["other_workloads"] = others
     out.update(n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak", vs_baseline=None,
                data="synthetic", roofline=roofline)
     if not args.no_cpu_baseline:

@@ -259,15 +259,6 @@ bool autotune_enabled() {
     return !(e && e[0] == '0') && !getenv("CHX_HIP_TILE");
 }
 
-bool stream_is_capturing(hipStream_t s) {
-    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
-        (void)hipGetLastError();
-        return true;  // when in doubt, do not time
-    }
-    return st != hipStreamCaptureStatusNone;
-}
-
 // Times every launch configuration on the call's operands and keeps the fastest in *best.
 int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hipStream_t s, TunedConfig* best) {
     // tile (output channels x pixels), wavefronts; the eight-wavefront kernels take the compute unit alone
@@ -1086,7 +1077,8 @@ extern "C" int chx_hip_conv_integer(
         a.w_zp_stride = stride;
     }
     hipStream_t s = as_stream(stream);
-    if (weights_fit_mfma(*w, params->group)) {
+    // (a recorded run takes the kernel without scratch memory: the weights of this entry point are packed per call)
+    if (weights_fit_mfma(*w, params->group) && !stream_is_capturing(s)) {
         bool zero = true;
         if (w_zero_point) {
             std::vector<uint8_t> zp;
@@ -1123,6 +1115,7 @@ int matmul_via_mfma(
     const int nd = a.ndim;
     if (ms.batch != 1 || b.dtype != CHX_HIP_INT8 || ms.M > INT32_MAX || ms.K > (1 << 20) || ms.N >= (1 << 24))
         return CHX_HIP_EUNSUPPORTED;
+    if (stream_is_capturing(s)) return CHX_HIP_EUNSUPPORTED;  // b is packed into scratch memory per call: not inside a recorded run
     chx_hip_tensor x4, w4, y4;
     memset(&x4, 0, sizeof(x4));
     memset(&w4, 0, sizeof(w4));
@@ -1227,7 +1220,7 @@ extern "C" int chx_hip_matmul_integer(
         m.b_zp_signed = b_zero_point->dtype == CHX_HIP_INT8;
     }
     hipStream_t s = as_stream(stream);
-    if (ms.batch == 1 && b->dtype == CHX_HIP_INT8 && ms.M * ms.N * ms.K >= (int64_t(1) << 22)) {
+    if (ms.batch == 1 && b->dtype == CHX_HIP_INT8 && ms.M * ms.N * ms.K >= (int64_t(1) << 22) && !stream_is_capturing(s)) {
         bool a_scalar, b_scalar;
         int32_t az, bz;
         CHX_PROPAGATE(scalar_zero_point(a_zero_point, s, &a_scalar, &az));

@@ -79,9 +79,22 @@ int launch_check(const char* kernel) {
     return CHX_HIP_OK;
 }
 
+bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;  // when in doubt, behave as if it were
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
 int scratch_alloc(void** p, size_t bytes, hipStream_t s) {
     *p = nullptr;
     if (bytes == 0) return CHX_HIP_OK;
+    // A stream-ordered allocation on a capturing stream would become a memory node of the graph, whose replays then
+    // run kernels on addresses that are not mapped (a device fault).  Callers that may be captured keep their scratch
+    // between calls (plans) or take a path without scratch.
+    if (stream_is_capturing(s)) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "scratch memory cannot be allocated while the stream is being captured into a graph");
     CHX_HIP_CALL(hipMallocAsync(p, bytes, s));
     return CHX_HIP_OK;
 }

@@ -609,6 +609,35 @@ class ConcurrentRunner(object):
             r.close()
 
 
+def conv_layer_table(model, fuse_residual=True):
+    """One row per QLinearConv launch of the program, in program order: the algorithmic work that prices it against
+    the two roofs.  ops = 2 * MACs.  bytes = what the launch must move at least: the input pixels it needs (a 1x1
+    convolution with stride s reads every s-th pixel of every s-th row only), the weights, the output, and with
+    `fuse_residual` the residual operand of the Add(+Relu) group behind it (whose sum is then the output).  All tensors
+    are 8-bit.  A launch belongs to the roof that takes longer at the published peaks."""
+    prog, convs, shapes = model["program"], model["convs"], model["shapes"]
+    rows = []
+    for i, ins in enumerate(prog):
+        if ins[0] != "QLinearConv":
+            continue
+        c = convs[ins[3]]
+        n, cin, h, w = shapes[ins[2]]
+        _, oc, oh, ow = shapes[ins[1]]
+        k = c.wq.shape[2]
+        x_bytes = n * cin * (oh * ow if k == 1 else h * w)
+        nbytes = x_bytes + c.wq.size + n * oc * oh * ow
+        residual = False
+        if fuse_residual and i + 1 < len(prog) and prog[i + 1][0] in ("AddRelu", "Add") and ins[1] in prog[i + 1][2:4]:
+            # the group is computed in this launch when the convolution result has no other reader
+            readers = [j for j in prog if ins[1] in j[2:]]
+            if len(readers) == 1:
+                residual = True
+                nbytes += n * oc * oh * ow
+        rows.append(dict(name=c.name, cin=cin, cout=oc, k=k, stride=c.stride, group=c.group, out_hw=oh, ops=2.0 * c.macs(shapes[ins[1]]),
+                         bytes=float(nbytes), residual=residual))
+    return rows
+
+
 def run_reference(model, orc, x, keep=None):
     """Executes the program with a CPU executor `orc` that offers the oracle's functions
     (quantize_linear, qlinear_conv_int, max_pool_q8, ...).  Test and benchmark code passes

@@ -579,6 +579,36 @@ def test_recorded_run_replays_with_new_inputs(g, vm, oracle):
         prog.close()
 
 
+def test_recorded_integer_ops_follow_the_input(g, vm, oracle):
+    """ConvInteger and MatMulInteger inside a recorded run: they are launched on the recording stream like every
+    other op, so each replay computes them from what the input buffers hold then (on the null stream they would
+    run once while recording, and every replay would return those first results)."""
+    rng = np.random.default_rng(21)
+    x, w = rand_q(rng, (2, 32, 9, 8), np.uint8), rand_q(rng, (16, 32, 3, 3), np.int8)
+    a_, b_ = rand_q(rng, (24, 64), np.uint8), rand_q(rng, (64, 40), np.int8)
+    b = vm.ProgramBuilder()
+    xi = b.input("x", "uint8", x.shape)
+    b.output("y", b.ConvInteger(xi, b.constant(w), b.scalar(77, "uint8"), None, [1, 1], [1, 1], 1, ""))
+    ai = b.input("a", "uint8", a_.shape)
+    b.output("m", b.MatMulInteger(ai, b.constant(b_), b.constant(np.array([3], np.uint8)), None))
+    prog = vm.Program(b.serialize())
+    xd, ad = g.dev(x), g.dev(a_)
+    replay = prog.capture({"x": xd, "a": ad})
+    for i in range(3):
+        xv, av = rand_q(rng, x.shape, np.uint8), rand_q(rng, a_.shape, np.uint8)
+        xd.copy_(torch.from_numpy(xv))
+        ad.copy_(torch.from_numpy(av))
+        torch.cuda.synchronize()
+        replay.launch()
+        replay.synchronize()
+        got = replay.outputs()
+        np.testing.assert_array_equal(got["y"], oracle.conv_integer(xv, w, 77, None, strides=(1, 1), pads=(1, 1), group=1),
+                                      err_msg="replay %d" % i)
+        np.testing.assert_array_equal(got["m"], oracle.matmul_integer(av, b_, np.array([3], np.uint8), None), err_msg="replay %d" % i)
+    replay.close()
+    prog.close()
+
+
 def test_a_program_that_reads_results_back_cannot_be_recorded(g, vm):
     """A dynamically quantized graph computes its scales on the device and reads them back as scalars: the
     capture fails with the reason, and the program still runs eagerly afterwards."""

@@ -181,6 +181,31 @@ def test_fused_quantize_dequantize_round_trip(g, oracle):
     np.testing.assert_array_equal(got, oracle.dequantize_linear(oracle.quantize_linear(x, 0.05, 0, np.int8), 0.05, 0))
 
 
+def test_full_size_fused_quantize_dequantize(g, oracle):
+    """The fused QuantizeLinear -> DequantizeLinear group on [64,1024,1024] (int8, scale 0.05, zero point 0), the kernel
+    the benchmark times: sampled rows against the oracle, every element against the two separate kernels and through
+    properties that need no oracle."""
+    torch.manual_seed(1)
+    x = torch.randn(64, 1024, 1024, device="cuda")
+    prog = g.ops.fusion_program([("x", F32)], [("q", "QuantizeLinear", "x", 0.05, 0, "int8"),
+                                               ("y", "DequantizeLinear", "q", 0.05, 0)], [("y", F32)])
+    y = g.ops.ElementWiseNvrtc([x], 1, prog, 3)[0]
+    torch.cuda.synchronize()
+    assert y.shape == x.shape and y.dtype == torch.float32
+    # the two ops as kernels of their own give the same bits
+    assert torch.equal(y, g.ops.DequantizeLinear(g.ops.QuantizeLinear(x, 0.05, 0, torch.int8), 0.05, 0))
+    # every result is a code times the scale, codes within [-127, 127]
+    codes = torch.round(y / 0.05)
+    assert torch.equal(codes * 0.05, y) and float(codes.min()) >= -127 and float(codes.max()) <= 127
+    # "+0.5f then truncate": error <= scale/2 for x >= 0, < 1.5 scale below
+    err = (y - x).abs()
+    assert err[x >= 0].max().item() <= 0.05 * 0.5 * 1.0001 and err.max().item() <= 0.05 * 1.5 * 1.0001
+    rows = torch.randint(0, 64 * 1024, (96,), device="cuda")
+    xs = x.view(-1, 1024)[rows].cpu().numpy()
+    want = oracle.dequantize_linear(oracle.quantize_linear(xs, 0.05, 0, np.int8), 0.05, 0)
+    np.testing.assert_array_equal(y.view(-1, 1024)[rows].cpu().numpy(), want)
+
+
 def test_full_size_chain(g, oracle):
     """x, c [64,1024,1024], a, b [1024]: sampled rows against the oracle plus properties that do
     not depend on the size."""
