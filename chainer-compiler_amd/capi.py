@@ -29,7 +29,7 @@ EXPORTS = [
     "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_describe", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
-    "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_match_residual_add",
+    "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_output_dtypes", "chx_hip_elementwise_match_residual_add",
     "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_reduce_min_max_noalloc", "chx_hip_cast", "chx_hip_count_nonfinite",
     "chx_hip_stream_create", "chx_hip_stream_destroy", "chx_hip_capture_begin", "chx_hip_capture_end", "chx_hip_stream_is_capturing",
     "chx_hip_graph_launch", "chx_hip_graph_destroy", "chx_hip_gemm_f32", "chx_hip_linear_f32", "chx_hip_max_pool_f32", "chx_hip_average_pool_f32", "chx_hip_fixed_batch_norm_f32", "chx_hip_conv_f32", "chx_hip_softmax_f32",
@@ -133,6 +133,14 @@ def make_desc(data_ptr, dtype, shape, strides_bytes):
         d.shape[i] = n
         d.strides[i] = st
     return d
+
+
+def elementwise_output_dtypes(code):
+    """chx_hip_elementwise_output_dtypes: the dtype codes of a fusion program's outputs, in order."""
+    codes = (ctypes.c_int32 * 64)()
+    count = ctypes.c_int32(0)
+    check(lib().chx_hip_elementwise_output_dtypes(code.encode(), codes, ctypes.c_int32(64), ctypes.byref(count)))
+    return [int(codes[i]) for i in range(count.value)]
 
 
 def elementwise_source(code, fusion_id, in_descs, out_descs, compile=False):

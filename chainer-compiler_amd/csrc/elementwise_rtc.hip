@@ -18,7 +18,7 @@
 //
 // Program text (one statement per line, '#' starts a comment):
 //   chxhip-fusion 1
-//   in  <name>:<dtype> ...            dtype: float32 | uint8 | int8
+//   in  <name>:<dtype> ...            dtype: float32 | float16 | float64 | uint8 | int8
 //   <name> = <Op> <operand> ...       operands are earlier names or, where noted, literals
 //   out <name>:<dtype> ...
 // Ops: Identity a | Neg a | Abs a | Floor a | Round a | Add a b | Sub a b | Mul a b | Div a b | Max a b | Min a b
@@ -26,6 +26,16 @@
 //      QuantizeLinear a <scale> <zero_point> <uint8|int8> [rne]   (float -> 8-bit code)
 //      DequantizeLinear q <scale> <zero_point>                    (8-bit code -> float)
 // Float literals are decimal or 0x######## (the bit pattern of the float32).
+// The arithmetic type of a program is that of its floating-point ports (one type per program, as the reference's
+// `typedef ... T`, compiler/nvrtc_builder.cc:118-127): float32; float16, where every node computes in float32 and
+// rounds to float16 (what a half-precision operation is); or float64.  The 8-bit ops go with float32 only, and only
+// float32 programs have the vector kernel; the other two types run on the general kernel.
+//
+// The CUDA C text that the reference's compiler emits for a group (BuildNvrtcProgram, nvrtc_builder.cc:91-206) is
+// accepted as well and turned into the same internal program: `typedef half|float|double T;`, the kernel's
+// parameters `T* i_<name>` / `T* o_<name>`, one `const T <name> = <expression>;` per node (a + b, a - b, a * b,
+// a / b, tanh(a), exp(a), sigmoid(a), a, or a number) and `o_<name>[tid] = <name>;` per output.  Its sigmoid is the
+// helper that text defines, tanh(x * 0.5) * 0.5 + 0.5, one rounding per operation.
 #include <hip/hiprtc.h>
 
 #include <cmath>
@@ -59,10 +69,17 @@ struct Port {
 struct Program {
     std::vector<Port> inputs, outputs;
     std::vector<Stmt> stmts;
+    int32_t arith = CHX_HIP_FLOAT32;  // type of the floating-point values: float32, float16 or float64
 };
+
+bool is_float_dtype(int32_t dt) {
+    return dt == CHX_HIP_FLOAT32 || dt == CHX_HIP_FLOAT16 || dt == CHX_HIP_FLOAT64;
+}
 
 bool parse_dtype(const std::string& s, int32_t* dt) {
     if (s == "float32") *dt = CHX_HIP_FLOAT32;
+    else if (s == "float16") *dt = CHX_HIP_FLOAT16;
+    else if (s == "float64") *dt = CHX_HIP_FLOAT64;
     else if (s == "uint8") *dt = CHX_HIP_UINT8;
     else if (s == "int8") *dt = CHX_HIP_INT8;
     else return false;
@@ -85,8 +102,32 @@ int parse_port(const std::string& tok, Port* p) {
     return CHX_HIP_OK;
 }
 
+int parse_nvrtc_source(const char* code, Program* prog);
+
+// One floating-point type per program; 8-bit ports only beside float32.
+int settle_arithmetic_type(Program* prog) {
+    int32_t arith = 0;
+    bool any8 = false;
+    auto see = [&](const Port& p) -> int {
+        if (!is_float_dtype(p.dtype)) {
+            any8 = true;
+            return CHX_HIP_OK;
+        }
+        CHX_REQUIRE(arith == 0 || arith == p.dtype, "fusion program: ports of two floating-point types (%s and %s)", dtype_name(arith),
+                    dtype_name(p.dtype));
+        arith = p.dtype;
+        return CHX_HIP_OK;
+    };
+    for (const Port& p : prog->inputs) CHX_PROPAGATE(see(p));
+    for (const Port& p : prog->outputs) CHX_PROPAGATE(see(p));
+    prog->arith = arith ? arith : CHX_HIP_FLOAT32;
+    CHX_REQUIRE(!any8 || prog->arith == CHX_HIP_FLOAT32, "fusion program: 8-bit ports go with float32 arithmetic, not %s", dtype_name(prog->arith));
+    return CHX_HIP_OK;
+}
+
 int parse_program(const char* code, Program* prog) {
     CHX_REQUIRE(code != nullptr, "fusion program: null code");
+    if (strstr(code, "__global__") != nullptr && strstr(code, "typedef") != nullptr) return parse_nvrtc_source(code, prog);
     std::istringstream iss(code);
     std::string line;
     bool header = false;
@@ -119,7 +160,175 @@ int parse_program(const char* code, Program* prog) {
     CHX_REQUIRE(header, "fusion program: empty");
     CHX_REQUIRE(!prog->inputs.empty(), "fusion program: no inputs");
     CHX_REQUIRE(!prog->outputs.empty(), "fusion program: no outputs");
-    return CHX_HIP_OK;
+    return settle_arithmetic_type(prog);
+}
+
+std::string trimmed(const std::string& s) {
+    size_t a = 0, b = s.size();
+    while (a < b && isspace((unsigned char)s[a])) ++a;
+    while (b > a && isspace((unsigned char)s[b - 1])) --b;
+    return s.substr(a, b - a);
+}
+
+bool is_identifier(const std::string& s) {
+    if (s.empty() || !(isalpha((unsigned char)s[0]) || s[0] == '_')) return false;
+    for (char c : s)
+        if (!(isalnum((unsigned char)c) || c == '_')) return false;
+    return true;
+}
+
+// The CUDA C text of BuildNvrtcProgram (compiler/nvrtc_builder.cc:91-206).  Port names are the variables the kernel
+// loads its inputs into / stores its outputs from; inputs and outputs keep the order of the kernel's parameters,
+// which is the order the op hands its arrays over in (runtime/ops/nvrtc.cc:134-150).
+int parse_nvrtc_source(const char* code, Program* prog) {
+    std::vector<std::string> lines;
+    {
+        std::istringstream iss(code);
+        std::string line;
+        while (std::getline(iss, line)) {
+            const size_t c = line.find("//");
+            if (c != std::string::npos) line.resize(c);
+            line = trimmed(line);
+            if (!line.empty()) lines.push_back(line);
+        }
+    }
+    int32_t arith = 0;
+    size_t i = 0;
+    for (; i < lines.size(); ++i) {
+        if (lines[i].compare(0, 8, "typedef ") != 0) continue;
+        const std::vector<std::string> t = split_ws(lines[i]);
+        CHX_REQUIRE(t.size() == 3 && t[2] == "T;", "fusion source: expected 'typedef <type> T;', got '%s'", lines[i].c_str());
+        if (t[1] == "half") arith = CHX_HIP_FLOAT16;
+        else if (t[1] == "float") arith = CHX_HIP_FLOAT32;
+        else if (t[1] == "double") arith = CHX_HIP_FLOAT64;
+        else CHX_FAIL(CHX_HIP_EUNSUPPORTED, "fusion source: element type '%s' (half, float or double expected)", t[1].c_str());
+        ++i;
+        break;
+    }
+    CHX_REQUIRE(arith != 0, "fusion source: no 'typedef ... T;'");
+    // the sigmoid helper, when the group has one
+    if (i < lines.size() && lines[i].compare(0, 10, "__device__") == 0) {
+        CHX_REQUIRE(lines[i].find("T sigmoid(T x)") != std::string::npos, "fusion source: unknown helper '%s'", lines[i].c_str());
+        bool body = false;
+        for (++i; i < lines.size() && lines[i] != "}"; ++i)
+            if (lines[i].find("tanh(x * half) * half + half") != std::string::npos) body = true;
+        CHX_REQUIRE(body && i < lines.size(), "fusion source: the sigmoid helper is not tanh(x * half) * half + half");
+        ++i;
+    }
+    // extern "C" __global__ / void fusionN(size_t n, T* i_a, ..., T* o_y) {
+    std::string sig;
+    for (; i < lines.size(); ++i) {
+        if (lines[i].compare(0, 5, "void ") == 0) {
+            sig = lines[i++];
+            break;
+        }
+        CHX_REQUIRE(lines[i].find("__global__") != std::string::npos, "fusion source: unexpected line '%s' in front of the kernel", lines[i].c_str());
+    }
+    const size_t lp = sig.find('('), rp = sig.rfind(')');
+    CHX_REQUIRE(!sig.empty() && lp != std::string::npos && rp != std::string::npos && rp > lp, "fusion source: no kernel signature");
+    std::vector<std::string> in_params, out_params;
+    {
+        std::istringstream ps(sig.substr(lp + 1, rp - lp - 1));
+        std::string param;
+        bool first = true;
+        while (std::getline(ps, param, ',')) {
+            param = trimmed(param);
+            if (first) {
+                CHX_REQUIRE(param == "size_t n", "fusion source: the first kernel parameter is '%s', not 'size_t n'", param.c_str());
+                first = false;
+                continue;
+            }
+            CHX_REQUIRE(param.compare(0, 3, "T* ") == 0, "fusion source: kernel parameter '%s' is not a T*", param.c_str());
+            const std::string name = trimmed(param.substr(3));
+            if (name.compare(0, 2, "i_") == 0) in_params.push_back(name);
+            else if (name.compare(0, 2, "o_") == 0) out_params.push_back(name);
+            else CHX_FAIL(CHX_HIP_EINVAL, "fusion source: kernel parameter '%s' is neither an input (i_) nor an output (o_)", name.c_str());
+        }
+    }
+    CHX_REQUIRE(!in_params.empty() && !out_params.empty(), "fusion source: the kernel needs inputs and outputs");
+    std::vector<std::string> in_var(in_params.size()), out_var(out_params.size());
+    for (; i < lines.size(); ++i) {
+        std::string line = lines[i];
+        if (line == "}") break;
+        if (line.compare(0, 11, "size_t tid ") == 0 || line.compare(0, 13, "if (tid >= n)") == 0) continue;
+        CHX_REQUIRE(line.back() == ';', "fusion source: statement without ';': '%s'", line.c_str());
+        line.resize(line.size() - 1);
+        const size_t eq = line.find(" = ");
+        CHX_REQUIRE(eq != std::string::npos, "fusion source: cannot parse '%s'", lines[i].c_str());
+        const std::string lhs = trimmed(line.substr(0, eq)), rhs = trimmed(line.substr(eq + 3));
+        if (lhs.compare(0, 8, "const T ") != 0) {
+            // o_<name>[tid] = <name>
+            const size_t br = lhs.find("[tid]");
+            CHX_REQUIRE(br != std::string::npos && br + 5 == lhs.size(), "fusion source: cannot parse '%s'", lines[i].c_str());
+            const std::string param = lhs.substr(0, br);
+            size_t k = 0;
+            while (k < out_params.size() && out_params[k] != param) ++k;
+            CHX_REQUIRE(k < out_params.size() && is_identifier(rhs), "fusion source: '%s' stores to something that is not an output", lines[i].c_str());
+            out_var[k] = rhs;
+            continue;
+        }
+        const std::string out = trimmed(lhs.substr(8));
+        CHX_REQUIRE(is_identifier(out), "fusion source: '%s' does not define a variable", lines[i].c_str());
+        const size_t br = rhs.find("[tid]");
+        if (br != std::string::npos) {
+            // <name> = i_<name>[tid]
+            const std::string param = rhs.substr(0, br);
+            size_t k = 0;
+            while (k < in_params.size() && in_params[k] != param) ++k;
+            CHX_REQUIRE(k < in_params.size() && br + 5 == rhs.size(), "fusion source: '%s' loads from something that is not an input", lines[i].c_str());
+            CHX_REQUIRE(in_var[k].empty(), "fusion source: input '%s' is loaded twice", param.c_str());
+            in_var[k] = out;
+            continue;
+        }
+        Stmt st;
+        st.out = out;
+        const std::vector<std::string> t = split_ws(rhs);
+        const size_t call = rhs.find('(');
+        if (t.size() == 3 && t[1].size() == 1 && strchr("+-*/", t[1][0]) && is_identifier(t[0]) && is_identifier(t[2])) {
+            st.op = t[1] == "+" ? "Add" : t[1] == "-" ? "Sub" : t[1] == "*" ? "Mul" : "Div";
+            st.args = {t[0], t[2]};
+            prog->stmts.push_back(st);
+        } else if (call != std::string::npos && rhs.back() == ')') {
+            const std::string fn = rhs.substr(0, call), arg = trimmed(rhs.substr(call + 1, rhs.size() - call - 2));
+            CHX_REQUIRE(is_identifier(arg), "fusion source: cannot parse the argument of '%s'", lines[i].c_str());
+            if (fn == "tanh" || fn == "exp") {
+                st.op = fn == "tanh" ? "Tanh" : "Exp";
+                st.args = {arg};
+                prog->stmts.push_back(st);
+            } else if (fn == "sigmoid") {
+                // the helper of this text, operation by operation: tanh(x * half) * half + half with half = 0.5
+                const std::string h = out + "__half", a = out + "__arg", th = out + "__tanh", m = out + "__scaled";
+                prog->stmts.push_back(Stmt{h, "Const", {"0.5"}});
+                prog->stmts.push_back(Stmt{a, "Mul", {arg, h}});
+                prog->stmts.push_back(Stmt{th, "Tanh", {a}});
+                prog->stmts.push_back(Stmt{m, "Mul", {th, h}});
+                prog->stmts.push_back(Stmt{out, "Add", {m, h}});
+            } else {
+                CHX_FAIL(CHX_HIP_EUNSUPPORTED, "fusion source: function '%s' is not one the reference's builder emits", fn.c_str());
+            }
+        } else if (t.size() == 1 && is_identifier(t[0])) {
+            st.op = "Identity";
+            st.args = {t[0]};
+            prog->stmts.push_back(st);
+        } else {
+            char* end = nullptr;
+            (void)strtod(rhs.c_str(), &end);
+            CHX_REQUIRE(end && *end == 0 && end != rhs.c_str(), "fusion source: cannot parse the expression of '%s'", lines[i].c_str());
+            st.op = "Const";
+            st.args = {rhs};
+            prog->stmts.push_back(st);
+        }
+    }
+    CHX_REQUIRE(i < lines.size(), "fusion source: the kernel body does not end");
+    for (size_t k = 0; k < in_params.size(); ++k) {
+        // an input that the kernel never loads keeps its place in the argument list
+        prog->inputs.push_back(Port{in_var[k].empty() ? in_params[k] + "__unused" : in_var[k], arith});
+    }
+    for (size_t k = 0; k < out_params.size(); ++k) {
+        CHX_REQUIRE(!out_var[k].empty(), "fusion source: output '%s' is never stored", out_params[k].c_str());
+        prog->outputs.push_back(Port{out_var[k], arith});
+    }
+    return settle_arithmetic_type(prog);
 }
 
 std::string ident(const std::string& s) {
@@ -130,12 +339,38 @@ std::string ident(const std::string& s) {
 
 int float_value(const std::string& tok, float* value);
 
-int float_literal(const std::string& tok, std::string* out) {
+// A literal of the program's arithmetic type, as source text that reproduces its bits: float32 and float64 by their
+// bit patterns; float16 as the float32 that equals the literal rounded to float16.
+int float_literal(const std::string& tok, std::string* out, int32_t arith = CHX_HIP_FLOAT32) {
+    char buf[80];
+    if (arith == CHX_HIP_FLOAT64 || arith == CHX_HIP_FLOAT16) {
+        double d;
+        if (tok.size() == 10 && tok[0] == '0' && (tok[1] == 'x' || tok[1] == 'X')) {
+            float f;
+            CHX_PROPAGATE(float_value(tok, &f));
+            d = f;
+        } else {
+            char* end = nullptr;
+            d = strtod(tok.c_str(), &end);
+            CHX_REQUIRE(end && *end == 0 && end != tok.c_str(), "fusion program: bad float literal '%s'", tok.c_str());
+        }
+        if (arith == CHX_HIP_FLOAT64) {
+            uint64_t bits;
+            memcpy(&bits, &d, 8);
+            snprintf(buf, sizeof(buf), "__builtin_bit_cast(double, 0x%016llxull)", (unsigned long long)bits);
+        } else {
+            const float f = (float)(_Float16)d;
+            uint32_t bits;
+            memcpy(&bits, &f, 4);
+            snprintf(buf, sizeof(buf), "__builtin_bit_cast(float, 0x%08xu)", bits);
+        }
+        *out = buf;
+        return CHX_HIP_OK;
+    }
     float f;
     CHX_PROPAGATE(float_value(tok, &f));
     uint32_t bits;
     memcpy(&bits, &f, 4);
-    char buf[64];
     snprintf(buf, sizeof(buf), "__builtin_bit_cast(float, 0x%08xu)", bits);
     *out = buf;
     return CHX_HIP_OK;
@@ -160,21 +395,28 @@ int float_value(const std::string& tok, float* value) {
 }
 
 // Emits the per-element device function:  elem(in..., &out...).
-// Value kinds: 'f' float32 value, 'q' 8-bit code held in an int.
+// Value kinds: 'f' floating-point value, 'q' 8-bit code held in an int.  A floating-point value is held as TY:
+// float for float32 and for float16 programs (in the latter every node's result goes through R(), the rounding
+// to float16, so that it is a float16 value at all times), double for float64 programs.
 int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* uses_exp_table) {
     std::map<std::string, char> kind;
+    const bool f64 = prog.arith == CHX_HIP_FLOAT64, f16 = prog.arith == CHX_HIP_FLOAT16;
+    const std::string TY = f64 ? "double" : "float";
+    const std::string decl = "  const " + TY + " ";
+    const char* R0 = f16 ? "chx_round_f16(" : "(";
+    const std::string zero = f64 ? "0.0" : "0.0f";
     // kFast: Exp and Sigmoid without their rare cases (arguments beyond +-88, quotients near the denormal range);
     // `rare` comes back set when an element met one, and the caller evaluates it again with kFast = false
     os << "template <bool kFast>\n__device__ __forceinline__ void elem(";
     bool first = true;
     for (const Port& p : prog.inputs) {
         CHX_REQUIRE(!kind.count(p.name), "fusion program: duplicate input '%s'", p.name.c_str());
-        kind[p.name] = p.dtype == CHX_HIP_FLOAT32 ? 'f' : 'q';
-        os << (first ? "" : ", ") << (p.dtype == CHX_HIP_FLOAT32 ? "const float " : "const int ") << ident(p.name);
+        kind[p.name] = is_float_dtype(p.dtype) ? 'f' : 'q';
+        os << (first ? "" : ", ") << (is_float_dtype(p.dtype) ? "const " + TY + " " : std::string("const int ")) << ident(p.name);
         first = false;
     }
     for (size_t i = 0; i < prog.outputs.size(); ++i)
-        os << ", " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float& " : "int& ") << "o_" << i;
+        os << ", " << (is_float_dtype(prog.outputs[i].dtype) ? TY + "& " : std::string("int& ")) << "o_" << i;
     os << ", bool& rare) {\n";
     const char* fma = use_fma ? "true" : "false";
     for (const Stmt& s : prog.stmts) {
@@ -201,72 +443,89 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             CHX_PROPAGATE(need(2));
             CHX_PROPAGATE(val(0, 'f', &a));
             CHX_PROPAGATE(val(1, 'f', &b));
-            os << "  const float " << o << " = " << a << " " << binops.at(s.op) << " " << b << ";\n";
+            os << decl << o << " = " << R0 << a << " " << binops.at(s.op) << " " << b << ");\n";
         } else if (s.op == "Max" || s.op == "Min") {
             CHX_PROPAGATE(need(2));
             CHX_PROPAGATE(val(0, 'f', &a));
             CHX_PROPAGATE(val(1, 'f', &b));
             if (s.op == "Max")
-                os << "  const float " << o << " = " << a << " < " << b << " ? " << b << " : " << a << ";\n";
+                os << decl << o << " = " << a << " < " << b << " ? " << b << " : " << a << ";\n";
             else
-                os << "  const float " << o << " = " << b << " < " << a << " ? " << b << " : " << a << ";\n";
+                os << decl << o << " = " << b << " < " << a << " ? " << b << " : " << a << ";\n";
         } else if (s.op == "Identity") {
             CHX_PROPAGATE(need(1));
             auto it = kind.find(s.args[0]);
             CHX_REQUIRE(it != kind.end(), "fusion program: '%s' used before definition", s.args[0].c_str());
             out_kind = it->second;
-            os << "  const " << (out_kind == 'f' ? "float " : "int ") << o << " = " << ident(s.args[0]) << ";\n";
+            os << "  const " << (out_kind == 'f' ? TY + " " : std::string("int ")) << o << " = " << ident(s.args[0]) << ";\n";
         } else if (s.op == "Neg") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = -" << a << ";\n";
+            os << decl << o << " = -" << a << ";\n";
         } else if (s.op == "Abs") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = __builtin_fabsf(" << a << ");\n";
+            os << decl << o << " = " << (f64 ? "__builtin_fabs(" : "__builtin_fabsf(") << a << ");\n";
         } else if (s.op == "Floor") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = __builtin_floorf(" << a << ");\n";
+            os << decl << o << " = " << (f64 ? "__builtin_floor(" : "__builtin_floorf(") << a << ");\n";
         } else if (s.op == "Round") {
             // to the nearest integer, ties to even (RoundOp, runtime/ops/quantize.cc:148-151)
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = __builtin_rintf(" << a << ");\n";
+            os << decl << o << " = " << (f64 ? "__builtin_rint(" : "__builtin_rintf(") << a << ");\n";
         } else if (s.op == "Tanh") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = chx_fm::tanhf_faithful(" << a << ");\n";
+            if (f64) os << decl << o << " = ::tanh(" << a << ");\n";
+            else os << decl << o << " = " << R0 << "chx_fm::tanhf_faithful(" << a << "));\n";
         } else if (s.op == "Exp") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = kFast ? chx_fm::expf_unless_rare<" << fma << ">(" << a << ", rare) : chx_fm::expf_faithful<"
-               << fma << ">(" << a << ");\n";
-            *uses_exp_table = true;
+            if (f64) {
+                os << decl << o << " = ::exp(" << a << ");\n";
+            } else {
+                os << decl << o << " = " << R0 << "kFast ? chx_fm::expf_unless_rare<" << fma << ">(" << a << ", rare) : chx_fm::expf_faithful<"
+                   << fma << ">(" << a << "));\n";
+                *uses_exp_table = true;
+            }
         } else if (s.op == "Sigmoid") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = kFast ? chx_fm::sigmoid_unless_rare<" << fma << ">(" << a
-               << ", rare) : chx_fm::sigmoid_faithful<" << fma << ">(" << a << ");\n";
-            *uses_exp_table = true;
+            if (f64) {
+                // 1 / (1 + exp(-x)), as the CPU path spells it
+                os << decl << o << " = 1.0 / (1.0 + ::exp(-" << a << "));\n";
+            } else if (f16) {
+                // the same, every operation a float16 operation
+                os << decl << o << "_e = chx_round_f16(chx_fm::expf_faithful<" << fma << ">(-" << a << "));\n";
+                os << decl << o << "_d = chx_round_f16(1.0f + " << o << "_e);\n";
+                os << decl << o << " = chx_round_f16(1.0f / " << o << "_d);\n";
+                *uses_exp_table = true;
+            } else {
+                os << decl << o << " = kFast ? chx_fm::sigmoid_unless_rare<" << fma << ">(" << a
+                   << ", rare) : chx_fm::sigmoid_faithful<" << fma << ">(" << a << ");\n";
+                *uses_exp_table = true;
+            }
         } else if (s.op == "Relu") {
             CHX_PROPAGATE(need(1));
             CHX_PROPAGATE(val(0, 'f', &a));
-            os << "  const float " << o << " = " << a << " < 0.0f ? 0.0f : " << a << ";\n";
+            os << decl << o << " = " << a << " < " << zero << " ? " << zero << " : " << a << ";\n";
         } else if (s.op == "Clip") {
             CHX_PROPAGATE(need(3));
             CHX_PROPAGATE(val(0, 'f', &a));
-            CHX_PROPAGATE(float_literal(s.args[1], &l0));
-            CHX_PROPAGATE(float_literal(s.args[2], &l1));
-            os << "  const float " << o << "_lo = " << a << " < " << l0 << " ? " << l0 << " : " << a << ";\n";
-            os << "  const float " << o << " = " << o << "_lo < " << l1 << " ? " << o << "_lo : " << l1 << ";\n";
+            CHX_PROPAGATE(float_literal(s.args[1], &l0, prog.arith));
+            CHX_PROPAGATE(float_literal(s.args[2], &l1, prog.arith));
+            os << decl << o << "_lo = " << a << " < " << l0 << " ? " << l0 << " : " << a << ";\n";
+            os << decl << o << " = " << o << "_lo < " << l1 << " ? " << o << "_lo : " << l1 << ";\n";
         } else if (s.op == "Const") {
             CHX_PROPAGATE(need(1));
-            CHX_PROPAGATE(float_literal(s.args[0], &l0));
-            os << "  const float " << o << " = " << l0 << ";\n";
+            CHX_PROPAGATE(float_literal(s.args[0], &l0, prog.arith));
+            os << decl << o << " = " << l0 << ";\n";
         } else if (s.op == "QuantizeLinear") {
             CHX_REQUIRE(s.args.size() == 4 || (s.args.size() == 5 && s.args[4] == "rne"),
                         "fusion program: QuantizeLinear a scale zero_point dtype [rne]");
+            CHX_REQUIRE(prog.arith == CHX_HIP_FLOAT32, "fusion program: QuantizeLinear inside a %s program", dtype_name(prog.arith));
             CHX_PROPAGATE(val(0, 'f', &a));
             CHX_PROPAGATE(float_literal(s.args[1], &l0));
             char* end = nullptr;
@@ -314,6 +573,7 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
             out_kind = 'q';
         } else if (s.op == "DequantizeLinear") {
             CHX_PROPAGATE(need(3));
+            CHX_REQUIRE(prog.arith == CHX_HIP_FLOAT32, "fusion program: DequantizeLinear inside a %s program", dtype_name(prog.arith));
             CHX_PROPAGATE(val(0, 'q', &a));
             CHX_PROPAGATE(float_literal(s.args[1], &l0));
             char* end = nullptr;
@@ -330,7 +590,7 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
     for (size_t i = 0; i < prog.outputs.size(); ++i) {
         auto it = kind.find(prog.outputs[i].name);
         CHX_REQUIRE(it != kind.end(), "fusion program: output '%s' is never defined", prog.outputs[i].name.c_str());
-        const char want = prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? 'f' : 'q';
+        const char want = is_float_dtype(prog.outputs[i].dtype) ? 'f' : 'q';
         CHX_REQUIRE(it->second == want, "fusion program: output '%s' is declared %s but computed as %s",
                     prog.outputs[i].name.c_str(), dtype_name(prog.outputs[i].dtype), it->second == 'f' ? "float" : "code");
         os << "  o_" << i << " = " << ident(prog.outputs[i].name) << ";\n";
@@ -342,7 +602,8 @@ int emit_elem(const Program& prog, bool use_fma, std::ostringstream& os, bool* u
 enum Mode : char { kFull = 'F', kScalar = 'S', kPeriodic = 'P' };
 
 const char* ctype_of(int32_t dt) {
-    return dt == CHX_HIP_FLOAT32 ? "float" : (dt == CHX_HIP_INT8 ? "signed char" : "unsigned char");
+    return dt == CHX_HIP_FLOAT32 ? "float" : dt == CHX_HIP_FLOAT16 ? "_Float16" : dt == CHX_HIP_FLOAT64 ? "double"
+           : dt == CHX_HIP_INT8 ? "signed char" : "unsigned char";
 }
 
 // Source of both kernels for one (program, operand modes) combination.
@@ -363,6 +624,7 @@ int generate_source(
     bool uses_table = false;
     CHX_PROPAGATE(emit_elem(prog, use_fma, body, &uses_table));
     os << kFaithfulMathText << "\n";
+    os << "__device__ __forceinline__ float chx_round_f16(float x) { return (float)(_Float16)x; }\n";
     os << "typedef float v4f __attribute__((ext_vector_type(4)));\n";
     os << "typedef unsigned int v4u __attribute__((ext_vector_type(4)));\n";
     os << "namespace {\n" << body.str() << "}\n";
@@ -374,6 +636,11 @@ int generate_source(
     // of them are 8-bit (one 128-bit access each).  kSteps steps per thread at a stride of
     // one block keep every access instruction of a wavefront on one contiguous span.
     const int steps = 2;
+    const std::string VT = prog.arith == CHX_HIP_FLOAT64 ? "double" : "float";  // what elem() takes and gives
+    if (prog.arith != CHX_HIP_FLOAT32) {
+        // float16 and float64 programs run on the general kernel; this one is never launched
+        os << "extern \"C\" __global__ void " << name << "_vec(unsigned int n_vec) {}\n";
+    } else {
     os << "extern \"C\" __global__ __launch_bounds__(256) void " << name << "_vec(unsigned int n_vec";
     for (size_t i = 0; i < nin; ++i) os << ", const " << ctype_of(prog.inputs[i].dtype) << "* __restrict__ i" << i;
     for (size_t i = 0; i < nout; ++i) os << ", " << ctype_of(prog.outputs[i].dtype) << "* __restrict__ o" << i;
@@ -461,6 +728,7 @@ int generate_source(
         }
     }
     os << "  }\n  }\n}\n";
+    }
 
     // ---- general kernel ----
     os << "struct GenDesc { int ndim; int pad; long long shape[" << CHX_HIP_MAX_NDIM << "]; long long istr[" << nin << "]["
@@ -481,16 +749,14 @@ int generate_source(
     os << "    for (int i = 0; i < " << nin << "; ++i) off[i] += r * d.istr[i][a];\n";
     os << "    rest = q;\n  }\n";
     for (size_t i = 0; i < nout; ++i)
-        os << "  " << (prog.outputs[i].dtype == CHX_HIP_FLOAT32 ? "float" : "int") << " r" << i << ";\n";
+        os << "  " << (is_float_dtype(prog.outputs[i].dtype) ? VT : std::string("int")) << " r" << i << ";\n";
     os << "  bool rare = false;\n  elem<false>(";
-    for (size_t i = 0; i < nin; ++i) os << (i ? ", " : "") << "i" << i << "[off[" << i << "]]";
+    for (size_t i = 0; i < nin; ++i)
+        os << (i ? ", " : "") << "(" << (is_float_dtype(prog.inputs[i].dtype) ? VT : std::string("int")) << ")i" << i << "[off[" << i << "]]";
     for (size_t i = 0; i < nout; ++i) os << ", r" << i;
     os << ", rare);\n";
     for (size_t i = 0; i < nout; ++i) {
-        if (prog.outputs[i].dtype == CHX_HIP_FLOAT32)
-            os << "  o" << i << "[idx] = r" << i << ";\n";
-        else
-            os << "  o" << i << "[idx] = (" << ctype_of(prog.outputs[i].dtype) << ")r" << i << ";\n";
+        os << "  o" << i << "[idx] = (" << ctype_of(prog.outputs[i].dtype) << ")r" << i << ";\n";
     }
     os << "}\n";
     *out = os.str();
@@ -682,7 +948,7 @@ int make_plan(
     }
     for (int k = 0; k < n_outputs; ++k)
         if (!aligned(outputs[k]->data, 16)) ok = false;
-    plan->vector_ok = ok && n >= plan->vec;
+    plan->vector_ok = ok && n >= plan->vec && prog.arith == CHX_HIP_FLOAT32;
     if (!plan->vector_ok) {
         // the general kernel ignores modes; use one canonical key
         plan->modes.assign(n_inputs, kFull);
@@ -757,6 +1023,15 @@ int launch(hipFunction_t f, unsigned grid, ArgPacker& args, hipStream_t s) {
 }  // namespace chx
 
 using namespace chx;
+
+extern "C" int chx_hip_elementwise_output_dtypes(const char* code, int32_t* dtypes, int32_t capacity, int32_t* count) {
+    CHX_REQUIRE(count != nullptr && (dtypes != nullptr || capacity == 0), "elementwise_output_dtypes: null output");
+    Program prog;
+    CHX_PROPAGATE(parse_program(code, &prog));
+    *count = (int32_t)prog.outputs.size();
+    for (int32_t i = 0; i < *count && i < capacity; ++i) dtypes[i] = prog.outputs[(size_t)i].dtype;
+    return CHX_HIP_OK;
+}
 
 extern "C" int chx_hip_elementwise_source(
         const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,

@@ -51,7 +51,7 @@ def DequantizeLinear(x, x_scale, x_zero_point=None, out=None):
     return out
 
 
-_DTYPE_NAMES = {torch.float32: "float32", torch.uint8: "uint8", torch.int8: "int8"}
+_DTYPE_NAMES = {torch.float32: "float32", torch.float16: "float16", torch.float64: "float64", torch.uint8: "uint8", torch.int8: "int8"}
 
 
 def fusion_program(inputs, statements, outputs):
@@ -68,12 +68,9 @@ def fusion_program(inputs, statements, outputs):
 
 
 def _program_output_dtypes(code):
-    names = {v: k for k, v in _DTYPE_NAMES.items()}
-    for line in code.splitlines():
-        t = line.split()
-        if t and t[0] == "out":
-            return [names[p.split(":")[1]] for p in t[1:]]
-    raise ValueError("fusion program has no 'out' line")
+    """Result types of a fusion program: this library's program text or the CUDA C text the reference's compiler emits."""
+    torch_of = {v: k for k, v in capi._TORCH_TO_CHX.items()}
+    return [torch_of[c] for c in capi.elementwise_output_dtypes(code)]
 
 
 def ElementWiseNvrtc(inputs, num_outputs, code, fusion_id=0, outs=None):

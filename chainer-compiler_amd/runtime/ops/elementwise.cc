@@ -15,25 +15,15 @@ chainerx::Array AsContiguous(const chainerx::Array& a);  // ops/connection.cc
 
 namespace {
 
-// dtypes of the outputs, from the program's `out name:dtype ...` line
+// dtypes of the outputs: those the program declares (either form of program text: this library's, or the CUDA C
+// that the reference's compiler emits, whose results have the type of its `typedef ... T`)
 std::vector<chainerx::Dtype> OutputDtypes(const std::string& code) {
+    int32_t codes[64];
+    int32_t count = 0;
+    CHXVM_HIP_CALL(chx_hip_elementwise_output_dtypes(code.c_str(), codes, 64, &count));
+    CHECK_LE(count, 64) << "a fusion program with more than 64 outputs";
     std::vector<chainerx::Dtype> out;
-    std::istringstream iss(code);
-    std::string line;
-    while (std::getline(iss, line)) {
-        std::istringstream ls(line);
-        std::string tok;
-        if (!(ls >> tok) || tok != "out") continue;
-        while (ls >> tok) {
-            const size_t c = tok.find(':');
-            CHECK(c != std::string::npos) << "bad output declaration in fusion program: " << tok;
-            const std::string dt = tok.substr(c + 1);
-            if (dt == "float32") out.push_back(chainerx::Dtype::kFloat32);
-            else if (dt == "uint8") out.push_back(chainerx::Dtype::kUInt8);
-            else if (dt == "int8") out.push_back(chainerx::Dtype::kInt8);
-            else CHECK(false) << "unsupported dtype in fusion program: " << dt;
-        }
-    }
+    for (int32_t i = 0; i < count; ++i) out.push_back(static_cast<chainerx::Dtype>(codes[i]));
     return out;
 }
 

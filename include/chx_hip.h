@@ -337,6 +337,13 @@ int chx_hip_elementwise(
         const char* code, int32_t fusion_id, const chx_hip_tensor* const* inputs, int32_t n_inputs,
         chx_hip_tensor* const* outputs, int32_t n_outputs, void* stream);
 
+/* The result types of a FusionGroup program, in the order of its outputs: what
+ * ElementWiseNvrtcOp::RunImpl needs to allocate its results (the reference allocates
+ * them with the type of the inputs, runtime/ops/nvrtc.cc:138-141; a program of this
+ * library may also end in a QuantizeLinear).  Writes at most `capacity` codes; *count
+ * receives the number of outputs.  Touches no device memory. */
+int chx_hip_elementwise_output_dtypes(const char* code, int32_t* dtypes, int32_t capacity, int32_t* count);
+
 /* Diagnostics for the same op: writes the HIP source that chx_hip_elementwise would
  * generate for these operands into `buffer` (truncated to buffer_size, always
  * terminated; *needed receives the full size) and, when `compile` is non-zero, also

@@ -69,7 +69,8 @@ def test_quantized_chain_uses_16_wide_vectors():
     ("chxhip-fusion 1\nin x:float32\ny = Add x z\nout y:float32\n", "before definition"),
     ("chxhip-fusion 1\nin x:float32\ny = Add x\nout y:float32\n", "takes 2 operands"),
     ("chxhip-fusion 1\nin x:float32\ny = Tanh x\nout y:uint8\n", "declared uint8"),
-    ("chxhip-fusion 1\nin x:float64\ny = Tanh x\nout y:float32\n", "unsupported dtype"),
+    ("chxhip-fusion 1\nin x:int32\ny = Tanh x\nout y:float32\n", "unsupported dtype"),
+    ("chxhip-fusion 1\nin x:float64\ny = Tanh x\nout y:float32\n", "two floating-point types"),
     ("chxhip-fusion 1\nin x:uint8\ny = Tanh x\nout y:float32\n", "wrong kind"),
     ("chxhip-fusion 1\nin x:float32\ny = QuantizeLinear x 0.1 300 uint8\nout y:uint8\n", "out of range"),
 ])
@@ -122,3 +123,64 @@ def test_residual_sum_groups_are_recognised():
     assert capi.match_residual_add(CHAIN) is None                                 # float chain
     with pytest.raises(capi.ChxHipError):
         capi.match_residual_add("not a program")
+
+
+# ---- the CUDA C text of the reference's BuildNvrtcProgram as program text ----------------------------------
+
+def _nvrtc_sources():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "nvrtc_fusion_sources.json")) as f:
+        return json.load(f)
+
+
+def test_reference_kernel_text_is_accepted():
+    src = _nvrtc_sources()
+    assert capi.elementwise_output_dtypes(src["tanh_sigmoid_float"]) == [capi.FLOAT32]
+    text = capi.elementwise_source(src["tanh_sigmoid_float"], 1, [fake((4, 8))], [fake((4, 8))], compile=True)
+    # tanh through the C library's arithmetic; the sigmoid is that text's helper, operation by operation
+    assert text.count("tanhf_faithful") >= 2 and "sigmoid_faithful<" not in text.split("namespace {")[-1]
+    full = (16, 64)
+    chain = src["chain_T"].replace("@T@", "float")
+    text = capi.elementwise_source(chain, 3, [fake(full), fake((64,)), fake((64,)), fake(full)], [fake(full)], compile=True)
+    assert "modes=FPPF vector" in text.splitlines()[0]
+    two = src["const_sub_div_exp_identity_float"]
+    assert capi.elementwise_output_dtypes(two) == [capi.FLOAT32, capi.FLOAT32]
+    capi.elementwise_source(two, 12, [fake((5,)), fake((5,))], [fake((5,)), fake((5,))], compile=True)
+
+
+@pytest.mark.parametrize("ctype,code,es", [("half", capi.FLOAT16, 2), ("double", capi.FLOAT64, 8)])
+def test_half_and_double_programs_compile_for_the_general_kernel(ctype, code, es):
+    chain = _nvrtc_sources()["chain_T"].replace("@T@", ctype)
+    assert capi.elementwise_output_dtypes(chain) == [code]
+    full = (16, 64)
+    t = dict(dtype=code, es=es)
+    text = capi.elementwise_source(chain, 3, [fake(full, **t), fake((64,), **t), fake((64,), **t), fake(full, **t)], [fake(full, **t)],
+                                   compile=True)
+    assert "general" in text.splitlines()[0]
+    assert ("chx_round_f16(" in text.split("namespace {")[-1]) == (ctype == "half")
+    # this library's own program text in the same types
+    dt = {"half": torch.float16, "double": torch.float64}[ctype]
+    own = ops.fusion_program([("x", dt), ("y", dt)], [("s", "Add", "x", "y"), ("r", "Relu", "s"), ("c", "Clip", "r", 0.25, 6.0)], [("c", dt)])
+    capi.elementwise_source(own, 4, [fake(full, **t), fake(full, **t)], [fake(full, **t)], compile=True)
+
+
+@pytest.mark.parametrize("bad,msg", [
+    ("typedef int T;\nextern \"C\" __global__\nvoid fusion1(size_t n, T* i_a, T* o_b) {\nconst T v_a = i_a[tid];\no_b[tid] = v_a;\n}\n", "half, float or double"),
+    ("typedef float T;\nextern \"C\" __global__\nvoid fusion1(size_t n, T* i_a, T* o_b) {\nconst T v_a = i_a[tid];\nconst T v_b = erf(v_a);\no_b[tid] = v_b;\n}\n", "not one the reference"),
+    ("typedef float T;\nextern \"C\" __global__\nvoid fusion1(size_t n, T* i_a, T* o_b) {\nconst T v_a = i_a[tid];\n}\n", "never stored"),
+])
+def test_reference_kernel_text_errors(bad, msg):
+    with pytest.raises(capi.ChxHipError) as e:
+        capi.elementwise_source(bad, 1, [fake((4,))], [fake((4,))])
+    assert msg in str(e.value)
+
+
+def test_mixed_float_types_and_quantization_outside_float32_are_refused():
+    with pytest.raises(capi.ChxHipError) as e:
+        capi.elementwise_output_dtypes(ops.fusion_program([("x", torch.float16), ("y", torch.float32)], [("s", "Add", "x", "y")], [("s", torch.float32)]))
+    assert "two floating-point types" in str(e.value)
+    prog = ops.fusion_program([("x", torch.float64)], [("q", "QuantizeLinear", "x", 0.05, 0, "int8")], [("q", torch.int8)])
+    with pytest.raises(capi.ChxHipError) as e:
+        capi.elementwise_source(prog, 1, [fake((4,), dtype=capi.FLOAT64, es=8)], [fake((4,), dtype=capi.INT8, es=1)])
+    assert "8-bit ports go with float32" in str(e.value)

@@ -674,3 +674,27 @@ def test_benchmark_networks_at_full_size_through_the_vm(g, vm, oracle, net, batc
         np.testing.assert_array_equal(again[name], out[name][perm.numpy()], err_msg=name)
     replay.close()
     prog.close()
+
+
+def test_fusion_group_with_the_reference_kernel_text(g, vm, oracle):
+    """An ElementWiseNvrtc instruction whose `code` is the CUDA C text that the reference's compiler emits (the group of
+    compiler/fusion_test.cc, Tanh -> Sigmoid): it loads and runs; the sigmoid is that text's helper."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "nvrtc_fusion_sources.json")) as f:
+        src = json.load(f)
+    b = vm.ProgramBuilder()
+    (y,) = b.ElementWiseNvrtc([b.input("input")], 1, src["tanh_sigmoid_float"], 1, num_list_outputs=1)
+    b.output("output", y)
+    prog = vm.Program(b.serialize())
+    x = (np.random.default_rng(41).standard_normal((2, 50, 30)) * 3).astype(np.float32)
+    out = prog.run({"input": g.dev(x)})
+    np.testing.assert_array_equal(out["output"], oracle.sigmoid_tanh_form(oracle.tanh(x)))
+    # in half precision the results are float16 arrays
+    bh = vm.ProgramBuilder()
+    (yh,) = bh.ElementWiseNvrtc([bh.input("x", "float16"), bh.input("a", "float16"), bh.input("b", "float16"), bh.input("c", "float16")], 1,
+                                src["chain_T"].replace("@T@", "half"), 3, num_list_outputs=1)
+    bh.output("y", yh)
+    xs = [torch.from_numpy(np.random.default_rng(42 + i).standard_normal((4, 16)).astype(np.float16)).cuda() for i in range(4)]
+    out = vm.Program(bh.serialize()).run(dict(zip("xabc", xs)))
+    assert out["y"].dtype == np.float16 and out["y"].shape == (4, 16)

@@ -299,3 +299,89 @@ def test_random_programs(g, oracle):
             want = np.broadcast_to(env[o], full_shape)
             assert not np.isnan(want).any()
             np.testing.assert_array_equal(g.host(t), want, err_msg="trial %d, %s of %s" % (trial, o, stmts))
+
+
+# ---- the CUDA C text of the reference's BuildNvrtcProgram (compiler/nvrtc_builder.cc:91-206) as the program ----
+
+def _nvrtc_sources():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "nvrtc_fusion_sources.json")) as f:
+        return json.load(f)
+
+
+def _chain_of_the_reference_text(orc, x, a, b, c, rnd):
+    """The chain fixture operation by operation; `rnd` rounds every result to the program's type (identity for
+    float32).  The sigmoid is that text's helper: tanh(x * 0.5) * 0.5 + 0.5."""
+    half = rnd(np.float32(0.5))
+    t0 = rnd(orc.binary(orc.MUL, x, a))
+    s = rnd(orc.binary(orc.ADD, rnd(orc.binary(orc.MUL, rnd(orc.tanh(rnd(orc.binary(orc.MUL, c, half)))), half)), half))
+    t1 = rnd(orc.binary(orc.ADD, t0, b))
+    t2 = rnd(orc.tanh(t1))
+    t4 = rnd(orc.binary(orc.MUL, t2, s))
+    return rnd(orc.binary(orc.ADD, t4, x))
+
+
+def test_reference_kernel_text_in_float(g, oracle):
+    src = _nvrtc_sources()
+    rng = np.random.default_rng(31)
+    x = (rng.standard_normal((3, 40, 64)) * 2).astype(np.float32)
+    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x)], 1, src["tanh_sigmoid_float"], 1)[0])
+    np.testing.assert_array_equal(got, oracle.sigmoid_tanh_form(oracle.tanh(x)))
+    # how far that spelling of the sigmoid is from the CPU path's 1 / (1 + exp(-x)): reported by the oracle, a few ulp
+    a, b = rng.standard_normal(64).astype(np.float32), rng.standard_normal(64).astype(np.float32)
+    c = rng.standard_normal((3, 40, 64)).astype(np.float32)
+    chain = src["chain_T"].replace("@T@", "float")
+    got = g.host(g.ops.ElementWiseNvrtc([g.dev(x), g.dev(a), g.dev(b), g.dev(c)], 1, chain, 3)[0])
+    np.testing.assert_array_equal(got, _chain_of_the_reference_text(oracle, x, a, b, c, lambda v: v))
+    p, q = rng.standard_normal((7, 33)).astype(np.float32), rng.standard_normal((7, 33)).astype(np.float32)
+    r, s = g.ops.ElementWiseNvrtc([g.dev(p), g.dev(q)], 2, src["const_sub_div_exp_identity_float"], 12)
+    d = oracle.binary(oracle.SUB, p, q)
+    want_r = oracle.binary(oracle.MUL, oracle.binary(oracle.DIV, oracle.exp(d), np.float32(2)), np.float32(0.333333))
+    np.testing.assert_array_equal(g.host(r), want_r)
+    np.testing.assert_array_equal(g.host(s), d)
+
+
+def test_reference_kernel_text_in_half(g, oracle):
+    """typedef half T: every node is a half-precision operation, i.e. the float32 operation rounded to float16
+    (numpy's float16 arithmetic is defined the same way); tanh is the C library's float32 tanh, rounded."""
+    rng = np.random.default_rng(32)
+    h = lambda v: np.asarray(v, np.float32).astype(np.float16).astype(np.float32)
+    x, c = h(rng.standard_normal((5, 24, 64)) * 2), h(rng.standard_normal((5, 24, 64)))
+    a, b = h(rng.standard_normal(64)), h(rng.standard_normal(64))
+    chain = _nvrtc_sources()["chain_T"].replace("@T@", "half")
+    dev = [torch.from_numpy(v.astype(np.float16)).cuda() for v in (x, a, b, c)]
+    got = g.ops.ElementWiseNvrtc(dev, 1, chain, 3)[0]
+    assert got.dtype == torch.float16
+    want = _chain_of_the_reference_text(oracle, x, a, b, c, h)
+    np.testing.assert_array_equal(got.cpu().numpy(), want.astype(np.float16))
+    # the exact operations, straight against numpy's float16 arithmetic
+    xh, ah, bh = x.astype(np.float16), a.astype(np.float16), b.astype(np.float16)
+    own = g.ops.fusion_program([("x", torch.float16), ("a", torch.float16), ("b", torch.float16)],
+                               [("m", "Mul", "x", "a"), ("s", "Add", "m", "b"), ("d", "Div", "s", "a"), ("r", "Relu", "d")], [("r", torch.float16)])
+    got = g.ops.ElementWiseNvrtc(dev[:3], 1, own, 4)[0].cpu().numpy()
+    with np.errstate(all="ignore"):
+        np.testing.assert_array_equal(got, np.maximum((xh * ah + bh) / ah, np.float16(0)))
+
+
+def test_reference_kernel_text_in_double(g):
+    """typedef double T: the arithmetic operations bit for bit against numpy's float64; tanh within 2 ulp of the C
+    library's double-precision tanh (its bits are not pinned: the device's double tanh is the ROCm math library's)."""
+    rng = np.random.default_rng(33)
+    x, c = rng.standard_normal((5, 24, 64)) * 2, rng.standard_normal((5, 24, 64))
+    a, b = rng.standard_normal(64), rng.standard_normal(64)
+    own = g.ops.fusion_program([("x", torch.float64), ("a", torch.float64), ("b", torch.float64)],
+                               [("m", "Mul", "x", "a"), ("s", "Add", "m", "b"), ("d", "Div", "s", "a"), ("u", "Sub", "d", "x"), ("r", "Relu", "u")],
+                               [("r", torch.float64)])
+    dev = [torch.from_numpy(v).cuda() for v in (x, a, b, c)]
+    got = g.ops.ElementWiseNvrtc(dev[:3], 1, own, 5)[0]
+    assert got.dtype == torch.float64
+    np.testing.assert_array_equal(got.cpu().numpy(), np.maximum((x * a + b) / a - x, 0.0))
+    chain = _nvrtc_sources()["chain_T"].replace("@T@", "double")
+    got = g.ops.ElementWiseNvrtc(dev, 1, chain, 3)[0].cpu().numpy()
+    want = np.tanh(x * a + b) * (np.tanh(c * 0.5) * 0.5 + 0.5) + x
+    # two tanh results within 2 ulp each, carried through a product and two sums of magnitude <= 1 + |x|
+    assert np.all(np.abs(got - want) <= 6 * np.spacing(1.0 + np.abs(x)))
+    single = "typedef double T;\nextern \"C\" __global__\nvoid fusion9(size_t n, T* i_x, T* o_y) {\nconst T v_x = i_x[tid];\nconst T v_y = tanh(v_x);\no_y[tid] = v_y;\n}\n"
+    got = g.ops.ElementWiseNvrtc(dev[:1], 1, single, 9)[0].cpu().numpy()
+    assert np.all(np.abs(got - np.tanh(x)) <= 2 * np.spacing(np.abs(np.tanh(x))))
