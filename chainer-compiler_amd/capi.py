@@ -27,10 +27,10 @@ EINVAL, EUNSUPPORTED, ERUNTIME = 1, 2, 3
 EXPORTS = [
     "chx_hip_init", "chx_hip_last_error", "chx_hip_version", "chx_hip_get_device_props", "chx_hip_malloc",
     "chx_hip_free", "chx_hip_memcpy_h2d", "chx_hip_memcpy_d2h", "chx_hip_memset", "chx_hip_stream_synchronize",
-    "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qconv_plan_create",
+    "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qlinear_conv_nd", "chx_hip_conv_integer_nd", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_describe", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
     "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_output_dtypes", "chx_hip_elementwise_match_residual_add",
-    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_reduce_min_max_noalloc", "chx_hip_cast", "chx_hip_count_nonfinite",
+    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_reduce_min_max_noalloc", "chx_hip_cast", "chx_hip_bit_shift", "chx_hip_count_nonfinite",
     "chx_hip_stream_create", "chx_hip_stream_destroy", "chx_hip_capture_begin", "chx_hip_capture_end", "chx_hip_stream_is_capturing",
     "chx_hip_graph_launch", "chx_hip_graph_destroy", "chx_hip_gemm_f32", "chx_hip_linear_f32", "chx_hip_max_pool_f32", "chx_hip_average_pool_f32", "chx_hip_fixed_batch_norm_f32", "chx_hip_conv_f32", "chx_hip_softmax_f32",
 ]
@@ -44,6 +44,22 @@ class Tensor(ctypes.Structure):
 class ConvParams(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "stride_h", "stride_w", "pad_h_begin", "pad_w_begin", "pad_h_end", "pad_w_end", "group")]
+
+
+class ConvNdParams(ctypes.Structure):
+    _fields_ = [("n_spatial", ctypes.c_int32), ("stride", ctypes.c_int32 * 3), ("pad_begin", ctypes.c_int32 * 3),
+                ("pad_end", ctypes.c_int32 * 3), ("group", ctypes.c_int32)]
+
+
+def conv_nd_params(strides, begin, end, group):
+    p = ConvNdParams()
+    p.n_spatial = len(strides)
+    for i in range(3):
+        p.stride[i], p.pad_begin[i], p.pad_end[i] = 1, 0, 0
+    for i, (s, b, e) in enumerate(list(zip(strides, begin, end))[:3]):   # more than three axes: the library refuses n_spatial
+        p.stride[i], p.pad_begin[i], p.pad_end[i] = int(s), int(b), int(e)
+    p.group = int(group)
+    return p
 
 
 class DeviceProps(ctypes.Structure):

@@ -406,6 +406,10 @@ private:
         } else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div") {
             CHECK_EQ(2UL, nin) << n.ToString();
             simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1))});
+        } else if (op == "BitShift") {
+            // compiler/chxvm/simple_node_emitter.cc:681-684
+            CHECK_EQ(2UL, nin) << n.ToString();
+            simple(op, {ArrayIn(Operand(n, 0)), ArrayIn(Operand(n, 1)), StringIn(n.GetString("direction", ""))});
         } else {
             CHECK(false) << "node type " << op << " (" << nin << " inputs) is not on the quantized-inference path";
         }

@@ -546,7 +546,7 @@ void InferDtypes(Graph* graph) {
         };
         static const std::set<std::string> unary = {"Identity", "Neg", "Abs", "Floor", "Round", "Exp", "Tanh", "Sigmoid", "Relu", "Cast", "Clip",
                                                     "QuantizeLinear", "DequantizeLinear"};
-        static const std::set<std::string> binary = {"Add", "Sub", "Mul", "Div", "Max", "Min"};
+        static const std::set<std::string> binary = {"Add", "Sub", "Mul", "Div", "Max", "Min", "BitShift"};
         std::vector<int64_t> dims;
         bool has_dims = false;
         if (op == "Constant") {

@@ -14,6 +14,9 @@ struct ConvDirectArgs {
     int64_t xs[4], ws[4], ys[4];  // byte strides of NCHW / OIHW / NCHW axes
     int32_t N, C, H, W, OC, Cg, KH, KW, OH, OW;
     int32_t sh, sw, ph, pw, group;
+    // a third (outermost) spatial axis, for 3-D convolutions; D = KD = OD = 1, sd = 1, pd = 0 otherwise
+    int32_t D, KD, OD, sd, pd;
+    int64_t xsd, wsd, ysd;  // byte strides of that axis in x, w and y
     int32_t x_signed, w_signed;
     int32_t x_zp;
     const char* w_zp;  // device, dtype of w

@@ -80,6 +80,7 @@ void fill_conv_args(
     a->x_signed = x.dtype == CHX_HIP_INT8;
     a->w_signed = w.dtype == CHX_HIP_INT8;
     a->total = (int64_t)cs.N * cs.OC * cs.OH * cs.OW;
+    a->D = a->KD = a->OD = a->sd = 1;  // no third spatial axis
 }
 
 int fill_requant(
@@ -852,6 +853,139 @@ extern "C" int chx_hip_qlinear_conv(
         }
     }
     return launch_conv_direct(q.direct, rne, s);
+}
+
+namespace chx {
+namespace {
+
+// Rank-generic convolutions (ComplementStride / ComplementPad and GroupedConv are rank-generic in the reference,
+// runtime/chainerx_util.cc:180-200,313-340).  One spatial axis is a 2-D convolution over images one pixel high and
+// takes every kernel the 2-D entry points have; three spatial axes run on the direct kernel, whose outermost spatial
+// axis is described here beside the 4-D views (n, c, h, w) that the 2-D checks and argument blocks are made from.
+struct ConvNdViews {
+    chx_hip_tensor x, w, y;
+    chx_hip_conv_params p;
+};
+
+chx_hip_tensor drop_axis(const chx_hip_tensor& t, int axis) {
+    chx_hip_tensor r = t;
+    r.ndim = t.ndim - 1;
+    for (int i = axis; i < r.ndim; ++i) {
+        r.shape[i] = t.shape[i + 1];
+        r.strides[i] = t.strides[i + 1];
+    }
+    return r;
+}
+
+chx_hip_tensor insert_unit_axis(const chx_hip_tensor& t, int axis) {
+    chx_hip_tensor r = t;
+    r.ndim = t.ndim + 1;
+    for (int i = r.ndim - 1; i > axis; --i) {
+        r.shape[i] = t.shape[i - 1];
+        r.strides[i] = t.strides[i - 1];
+    }
+    r.shape[axis] = 1;
+    r.strides[axis] = t.shape[axis] * t.strides[axis];  // any value serves an axis of extent 1; this one keeps the view dense
+    return r;
+}
+
+int conv_nd_views(const chx_hip_tensor* x, const chx_hip_tensor* w, const chx_hip_tensor* y, const chx_hip_conv_nd_params* p, const char* op,
+                  ConvNdViews* v) {
+    CHX_PROPAGATE(check_tensor(x, op));
+    CHX_PROPAGATE(check_tensor(w, op));
+    CHX_PROPAGATE(check_tensor(y, op));
+    CHX_REQUIRE(p != nullptr, "%s: null params", op);
+    CHX_REQUIRE(p->n_spatial >= 1 && p->n_spatial <= 3, "%s: %d spatial axes (1, 2 or 3 are computed)", op, p->n_spatial);
+    const int nd = p->n_spatial + 2;
+    CHX_REQUIRE(x->ndim == nd && w->ndim == nd && y->ndim == nd, "%s: x, w and y must have %d axes for %d spatial ones", op, nd, p->n_spatial);
+    const int lead = 3 - p->n_spatial;  // entries of the 2-D parameter block that stay at their neutral values
+    int32_t st[3] = {1, 1, 1}, pb[3] = {0, 0, 0}, pe[3] = {0, 0, 0};
+    for (int i = 0; i < p->n_spatial; ++i) {
+        st[lead + i] = p->stride[i];
+        pb[lead + i] = p->pad_begin[i];
+        pe[lead + i] = p->pad_end[i];
+    }
+    v->p.stride_h = st[1]; v->p.stride_w = st[2];
+    v->p.pad_h_begin = pb[1]; v->p.pad_w_begin = pb[2];
+    v->p.pad_h_end = pe[1]; v->p.pad_w_end = pe[2];
+    v->p.group = p->group;
+    if (p->n_spatial == 1) {
+        v->x = insert_unit_axis(*x, 2);
+        v->w = insert_unit_axis(*w, 2);
+        v->y = insert_unit_axis(*y, 2);
+    } else if (p->n_spatial == 2) {
+        v->x = *x; v->w = *w; v->y = *y;
+    } else {
+        v->x = drop_axis(*x, 2);
+        v->w = drop_axis(*w, 2);
+        v->y = drop_axis(*y, 2);
+    }
+    return CHX_HIP_OK;
+}
+
+// the outermost spatial axis of a 3-D convolution into the argument block of the direct kernel
+int add_depth_axis(const chx_hip_tensor& x, const chx_hip_tensor& w, const chx_hip_tensor& y, const chx_hip_conv_nd_params& p, const char* op,
+                   ConvDirectArgs* a) {
+    CHX_REQUIRE(p.stride[0] >= 1 && p.pad_begin[0] >= 0 && p.pad_end[0] >= 0, "%s: strides must be positive and pads non-negative", op);
+    CHX_REQUIRE(x.shape[2] <= INT32_MAX && w.shape[2] <= INT32_MAX, "%s: extent too large", op);
+    const int64_t ed = x.shape[2] + p.pad_begin[0] + p.pad_end[0] - w.shape[2];
+    CHX_REQUIRE(ed >= 0, "%s: kernel deeper than the padded input", op);
+    const int64_t od = ed / p.stride[0] + 1;
+    CHX_REQUIRE(y.shape[2] == od, "%s: y has depth %lld, expected %lld", op, (long long)y.shape[2], (long long)od);
+    a->D = (int32_t)x.shape[2];
+    a->KD = (int32_t)w.shape[2];
+    a->OD = (int32_t)od;
+    a->sd = p.stride[0];
+    a->pd = p.pad_begin[0];
+    a->xsd = x.strides[2];
+    a->wsd = w.strides[2];
+    a->ysd = y.strides[2];
+    a->total *= od;
+    return CHX_HIP_OK;
+}
+
+}  // namespace
+}  // namespace chx
+
+extern "C" int chx_hip_qlinear_conv_nd(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w, const chx_hip_tensor* w_scale,
+        const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point, const chx_hip_tensor* bias,
+        const chx_hip_conv_nd_params* params, uint32_t flags, chx_hip_tensor* y, void* stream) {
+    ConvNdViews v;
+    CHX_PROPAGATE(conv_nd_views(x, w, y, params, "QLinearConv", &v));
+    if (params->n_spatial < 3) {
+        const int rc = chx_hip_qlinear_conv(&v.x, x_scale, x_zero_point, &v.w, w_scale, w_zero_point, y_scale, y_zero_point, bias, &v.p, flags, &v.y, stream);
+        return rc;
+    }
+    QConvChecked q;
+    CHX_PROPAGATE(check_qconv(&v.x, x_scale, x_zero_point, &v.w, w_scale, w_zero_point, y_scale, y_zero_point, bias, &v.p, flags, &v.y, &q));
+    CHX_PROPAGATE(add_depth_axis(*x, *w, *y, *params, "QLinearConv", &q.direct));
+    return launch_conv_direct(q.direct, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0, as_stream(stream));
+}
+
+extern "C" int chx_hip_conv_integer_nd(
+        const chx_hip_tensor* x, const chx_hip_tensor* w, int32_t x_zero_point, const chx_hip_tensor* w_zero_point,
+        const chx_hip_conv_nd_params* params, chx_hip_tensor* y, void* stream) {
+    ConvNdViews v;
+    CHX_PROPAGATE(conv_nd_views(x, w, y, params, "ConvInteger", &v));
+    if (params->n_spatial < 3) return chx_hip_conv_integer(&v.x, &v.w, x_zero_point, w_zero_point, &v.p, &v.y, stream);
+    CHX_REQUIRE(y->dtype == CHX_HIP_INT32, "ConvInteger: y must be int32, got %s", dtype_name(y->dtype));
+    ConvShape cs;
+    CHX_PROPAGATE(conv_shape(v.x, v.w, v.p, v.y, "ConvInteger", &cs));
+    ConvDirectArgs a;
+    fill_conv_args(v.x, v.w, v.p, v.y, cs, &a);
+    a.x_zp = x_zero_point;
+    if (w_zero_point) {
+        CHX_PROPAGATE(check_tensor(w_zero_point, "ConvInteger w_zero_point"));
+        CHX_REQUIRE(w_zero_point->dtype == w->dtype, "ConvInteger: w_zero_point must have the dtype of w");
+        int64_t len, stride;
+        CHX_PROPAGATE(param_vector(*w_zero_point, cs.OC, "ConvInteger w_zero_point", &len, &stride));
+        a.w_zp = static_cast<const char*>(w_zero_point->data);
+        a.w_zp_len = (int32_t)len;
+        a.w_zp_stride = stride;
+    }
+    CHX_PROPAGATE(add_depth_axis(*x, *w, *y, *params, "ConvInteger", &a));
+    return launch_conv_direct(a, false, as_stream(stream));
 }
 
 extern "C" int chx_hip_qconv_plan_create(

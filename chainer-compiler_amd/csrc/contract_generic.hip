@@ -21,13 +21,15 @@ template <bool kRne>
 __global__ __launch_bounds__(kThreads) void conv_direct_kernel(ConvDirectArgs a) {
     const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= a.total) return;
-    // idx enumerates (n, oh, ow, oc) with oc fastest: neighbouring lanes share the input window
+    // idx enumerates (n, od, oh, ow, oc) with oc fastest: neighbouring lanes share the input window
     const int oc = (int)(idx % a.OC);
     int64_t rest = idx / a.OC;
     const int ow = (int)(rest % a.OW);
     rest /= a.OW;
     const int oh = (int)(rest % a.OH);
-    const int n = (int)(rest / a.OH);
+    rest /= a.OH;
+    const int od = (int)(rest % a.OD);
+    const int n = (int)(rest / a.OD);
     const int OCg = a.OC / a.group;
     const int grp = oc / OCg;
     int32_t wz = 0;
@@ -38,19 +40,23 @@ __global__ __launch_bounds__(kThreads) void conv_direct_kernel(ConvDirectArgs a)
     for (int c = 0; c < a.Cg; ++c) {
         const char* xc = a.x + (int64_t)n * a.xs[0] + (int64_t)(grp * a.Cg + c) * a.xs[1];
         const char* wc = wbase + (int64_t)c * a.ws[1];
-        for (int kh = 0; kh < a.KH; ++kh) {
-            const int ih = oh * a.sh - a.ph + kh;
-            if (ih < 0 || ih >= a.H) continue;
-            for (int kw = 0; kw < a.KW; ++kw) {
-                const int iw = ow * a.sw - a.pw + kw;
-                if (iw < 0 || iw >= a.W) continue;
-                const int32_t xv = load8(xc + (int64_t)ih * a.xs[2] + (int64_t)iw * a.xs[3], a.x_signed) - a.x_zp;
-                const int32_t wv = load8(wc + (int64_t)kh * a.ws[2] + (int64_t)kw * a.ws[3], a.w_signed) - wz;
-                acc += xv * wv;
+        for (int kd = 0; kd < a.KD; ++kd) {
+            const int id = od * a.sd - a.pd + kd;
+            if (id < 0 || id >= a.D) continue;
+            for (int kh = 0; kh < a.KH; ++kh) {
+                const int ih = oh * a.sh - a.ph + kh;
+                if (ih < 0 || ih >= a.H) continue;
+                for (int kw = 0; kw < a.KW; ++kw) {
+                    const int iw = ow * a.sw - a.pw + kw;
+                    if (iw < 0 || iw >= a.W) continue;
+                    const int32_t xv = load8(xc + (int64_t)id * a.xsd + (int64_t)ih * a.xs[2] + (int64_t)iw * a.xs[3], a.x_signed) - a.x_zp;
+                    const int32_t wv = load8(wc + (int64_t)kd * a.wsd + (int64_t)kh * a.ws[2] + (int64_t)kw * a.ws[3], a.w_signed) - wz;
+                    acc += xv * wv;
+                }
             }
         }
     }
-    char* yp = a.y + (int64_t)n * a.ys[0] + (int64_t)oc * a.ys[1] + (int64_t)oh * a.ys[2] + (int64_t)ow * a.ys[3];
+    char* yp = a.y + (int64_t)n * a.ys[0] + (int64_t)oc * a.ys[1] + (int64_t)od * a.ysd + (int64_t)oh * a.ys[2] + (int64_t)ow * a.ys[3];
     if (!a.requant) {
         *reinterpret_cast<int32_t*>(yp) = acc;
         return;

@@ -7,6 +7,8 @@
 #include <mutex>
 #include <vector>
 
+#include <type_traits>
+
 #include "chx_internal.h"
 
 namespace chx {
@@ -211,6 +213,85 @@ extern "C" int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* st
         case CHX_HIP_UINT8: return cast_from<uint8_t>(*x, *y, n, s);
         case CHX_HIP_INT8: return cast_from<int8_t>(*x, *y, n, s);
         default: CHX_FAIL(CHX_HIP_EUNSUPPORTED, "Cast: no conversion from %s on the device", dtype_name(x->dtype));
+    }
+}
+
+namespace chx {
+namespace {
+
+// z = x << y or x >> y over the broadcast of x and y (strides of 0 on broadcast axes), one lane per element.
+// A count of the element width or more shifts every bit out: 0, or for a negative x shifted right the sign (-1), as
+// numpy defines it (C leaves it undefined); a right shift of a signed type is arithmetic.
+template <typename T, bool kLeft>
+__global__ __launch_bounds__(kThreads) void bit_shift_kernel(
+        const char* __restrict__ x, StridedDesc xd, const char* __restrict__ y, StridedDesc yd, char* __restrict__ z, StridedDesc zd, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    typedef typename std::make_unsigned<T>::type U;
+    const T a = *reinterpret_cast<const T*>(x + strided_offset(i, xd));
+    const T c = *reinterpret_cast<const T*>(y + strided_offset(i, yd));
+    const int bits = (int)sizeof(T) * 8;
+    T r;
+    if (c < 0 || (uint64_t)c >= (uint64_t)bits) r = (!kLeft && a < 0) ? (T)-1 : (T)0;
+    else if (kLeft) r = (T)((U)a << (int)c);
+    else r = (T)(a >> (int)c);
+    *reinterpret_cast<T*>(z + strided_offset(i, zd)) = r;
+}
+
+template <typename T>
+int launch_bit_shift(const chx_hip_tensor& x, const StridedDesc& xd, const chx_hip_tensor& y, const StridedDesc& yd, chx_hip_tensor& z, bool left,
+                     int64_t n, hipStream_t s) {
+    const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads);
+    const StridedDesc zd = make_desc(z);
+    if (left)
+        bit_shift_kernel<T, true><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x.data), xd, static_cast<const char*>(y.data), yd,
+                                                               static_cast<char*>(z.data), zd, n);
+    else
+        bit_shift_kernel<T, false><<<blocks, kThreads, 0, s>>>(static_cast<const char*>(x.data), xd, static_cast<const char*>(y.data), yd,
+                                                                static_cast<char*>(z.data), zd, n);
+    return launch_check("bit_shift_kernel");
+}
+
+// the descriptor of t seen through the shape of z: strides 0 where t broadcasts
+int broadcast_desc(const chx_hip_tensor& t, const chx_hip_tensor& z, const char* what, StridedDesc* d) {
+    CHX_REQUIRE(t.ndim <= z.ndim, "BitShift: %s has more axes than the result", what);
+    d->ndim = z.ndim;
+    for (int a = 0; a < z.ndim; ++a) {
+        const int ta = a - (z.ndim - t.ndim);
+        d->shape[a] = z.shape[a];
+        if (ta < 0 || t.shape[ta] == 1) {
+            d->strides[a] = 0;
+        } else {
+            CHX_REQUIRE(t.shape[ta] == z.shape[a], "BitShift: %s does not broadcast to the result (axis %d: %lld vs %lld)", what, a,
+                        (long long)t.shape[ta], (long long)z.shape[a]);
+            d->strides[a] = t.strides[ta];
+        }
+    }
+    return CHX_HIP_OK;
+}
+
+}  // namespace
+}  // namespace chx
+
+extern "C" int chx_hip_bit_shift(const chx_hip_tensor* x, const chx_hip_tensor* y, int32_t left, chx_hip_tensor* z, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "BitShift x"));
+    CHX_PROPAGATE(check_tensor(y, "BitShift y"));
+    CHX_PROPAGATE(check_tensor(z, "BitShift z"));
+    CHX_REQUIRE(x->dtype == y->dtype && x->dtype == z->dtype, "BitShift: x, y and z must have one integer type, got %s, %s and %s",
+                dtype_name(x->dtype), dtype_name(y->dtype), dtype_name(z->dtype));
+    StridedDesc xd, yd;
+    CHX_PROPAGATE(broadcast_desc(*x, *z, "x", &xd));
+    CHX_PROPAGATE(broadcast_desc(*y, *z, "y", &yd));
+    const int64_t n = numel(*z);
+    if (n == 0) return CHX_HIP_OK;
+    hipStream_t s = as_stream(stream);
+    switch (x->dtype) {
+        case CHX_HIP_UINT8: return launch_bit_shift<uint8_t>(*x, xd, *y, yd, *z, left != 0, n, s);
+        case CHX_HIP_INT8: return launch_bit_shift<int8_t>(*x, xd, *y, yd, *z, left != 0, n, s);
+        case CHX_HIP_INT16: return launch_bit_shift<int16_t>(*x, xd, *y, yd, *z, left != 0, n, s);
+        case CHX_HIP_INT32: return launch_bit_shift<int32_t>(*x, xd, *y, yd, *z, left != 0, n, s);
+        case CHX_HIP_INT64: return launch_bit_shift<int64_t>(*x, xd, *y, yd, *z, left != 0, n, s);
+        default: CHX_FAIL(CHX_HIP_EINVAL, "BitShift: %s is not an integer type", dtype_name(x->dtype));  // CHECK(!IsFloat(...)), quantize.cc:154-155
     }
 }
 

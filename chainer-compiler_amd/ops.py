@@ -120,15 +120,19 @@ def _auto_pad(auto_pad, in_shape, kernel, strides, pads):
 
 
 def _conv_setup(x, w, strides, pads, group, auto_pad):
-    strides = _complement(strides, x.dim() - 2, 1)
-    pads = _complement(pads, x.dim() - 2, 0)
-    if len(pads) == 2 * (x.dim() - 2):    # explicit begin/end list (what ApplyAsymmetricPad handles)
-        begin, end = pads[:x.dim() - 2], pads[x.dim() - 2:]
+    """Completed attributes and the result shape; x [N,C,H,W] gives the 2-D parameter block, x with one or three spatial
+    axes the rank-generic one."""
+    ns = x.dim() - 2
+    strides = _complement(strides, ns, 1)
+    pads = _complement(pads, ns, 0)
+    if len(pads) == 2 * ns:    # explicit begin/end list (what ApplyAsymmetricPad handles)
+        begin, end = pads[:ns], pads[ns:]
     else:
         begin, end = _auto_pad(auto_pad, x.shape[2:], w.shape[2:], strides, pads)
-    oh = (x.shape[2] + begin[0] + end[0] - w.shape[2]) // strides[0] + 1
-    ow = (x.shape[3] + begin[1] + end[1] - w.shape[3]) // strides[1] + 1
-    return capi.conv_params(strides, begin, end, group), (x.shape[0], w.shape[0], oh, ow)
+    out = tuple((x.shape[2 + i] + begin[i] + end[i] - w.shape[2 + i]) // strides[i] + 1 for i in range(ns))
+    if ns == 2:
+        return capi.conv_params(strides, begin, end, group), (x.shape[0], w.shape[0]) + out
+    return capi.conv_nd_params(strides, begin, end, group), (x.shape[0], w.shape[0]) + out
 
 
 def _alloc_like_input_layout(x, shape, dtype):
@@ -144,7 +148,8 @@ def QLinearConv(x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_z
     params, shape = _conv_setup(x, w, strides, pads, group, auto_pad)
     if out is None:
         out = _alloc_like_input_layout(x, shape, zero_point_dtype)
-    capi.check(capi.lib().chx_hip_qlinear_conv(
+    entry = capi.lib().chx_hip_qlinear_conv if x.dim() == 4 else capi.lib().chx_hip_qlinear_conv_nd
+    capi.check(entry(
         capi.ref(x), _f(x_scale), _i(x_zero_point), capi.ref(w), capi.ref(w_scale), capi.ref(w_zero_point),
         _f(y_scale), _i(y_zero_point), capi.ref(b), ctypes.byref(params), ctypes.c_uint32(flags), capi.ref(out),
         capi.stream_ptr()))
@@ -156,7 +161,8 @@ def ConvInteger(x, w, x_zero_point=None, w_zero_point=None, strides=(), pads=(),
     params, shape = _conv_setup(x, w, strides, pads, group, auto_pad)
     if out is None:
         out = _alloc_like_input_layout(x, shape, torch.int32)
-    capi.check(capi.lib().chx_hip_conv_integer(
+    entry = capi.lib().chx_hip_conv_integer if x.dim() == 4 else capi.lib().chx_hip_conv_integer_nd
+    capi.check(entry(
         capi.ref(x), capi.ref(w), _i(0 if x_zero_point is None else x_zero_point), capi.ref(w_zero_point),
         ctypes.byref(params), capi.ref(out), capi.stream_ptr()))
     return out
@@ -182,6 +188,17 @@ def QLinearMatMul(a, a_scale, a_zero_point, b, b_scale, b_zero_point, y_scale, y
         capi.ref(a), _f(a_scale), _i(a_zero_point), capi.ref(b), _f(b_scale), _i(b_zero_point), _f(y_scale),
         _i(y_zero_point), capi.ref(bias), ctypes.c_uint32(flags), capi.ref(out), capi.stream_ptr()))
     return out
+
+
+def BitShift(x, y, direction):
+    """BitShiftOp::RunImpl, runtime/ops/quantize.cc:153-163: x << y ("LEFT") or x >> y ("RIGHT") over the broadcast of
+    two integer arrays of one type."""
+    assert direction in ("LEFT", "RIGHT")
+    shape = torch.broadcast_shapes(tuple(x.shape), tuple(y.shape))
+    z = torch.empty(shape, dtype=x.dtype, device=x.device)
+    capi.check(capi.lib().chx_hip_bit_shift(capi.ref(x), capi.ref(y), ctypes.c_int32(1 if direction == "LEFT" else 0),
+                                            capi.ref(z), capi.stream_ptr()))
+    return z
 
 
 def Gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=0, trans_b=0, out=None):

@@ -1,5 +1,7 @@
 #include "chainerx_util.h"
 
+#include <cstring>
+
 namespace chainer_compiler {
 namespace runtime {
 
@@ -71,6 +73,40 @@ chainerx::Shape ConvOutputShape(const chainerx::Array& x, const chainerx::Array&
     const int64_t oh = (x.shape()[2] + p.pad_h_begin + p.pad_h_end - w.shape()[2]) / p.stride_h + 1;
     const int64_t ow = (x.shape()[3] + p.pad_w_begin + p.pad_w_end - w.shape()[3]) / p.stride_w + 1;
     return chainerx::Shape{x.shape()[0], w.shape()[0], oh, ow};
+}
+
+chx_hip_conv_nd_params MakeConvNdParams(
+        const chainerx::Array& x, const chainerx::Array& w, const Int64StackVector& strides, const Int64StackVector& pads,
+        int group, const std::string& auto_pad, chainerx::Shape* y_shape) {
+    const int ns = x.ndim() - 2;
+    CHECK(ns >= 1 && ns <= 3) << "convolutions over 1, 2 or 3 spatial axes on the hip backend, got an input of shape " << x.shape();
+    CHECK_EQ(x.ndim(), w.ndim());
+    const Int64StackVector st = ComplementStride(strides, x);
+    const Int64StackVector pd = ComplementPad(pads, x);
+    CHECK_EQ(static_cast<size_t>(ns), st.size());
+    Int64StackVector kernel, begin_in;
+    for (int i = 0; i < ns; ++i) kernel.push_back(w.shape()[2 + i]);
+    // an explicit begin/end list passes through; a begin list goes through the auto-pad completion
+    Int64StackVector full;
+    if (pd.size() == static_cast<size_t>(2 * ns)) {
+        full = pd;
+    } else {
+        CHECK_EQ(static_cast<size_t>(ns), pd.size());
+        full = CalculateAutoPad(auto_pad, x, kernel, st, pd);
+    }
+    chx_hip_conv_nd_params p;
+    memset(&p, 0, sizeof(p));
+    p.n_spatial = ns;
+    p.group = group;
+    *y_shape = chainerx::Shape{x.shape()[0], w.shape()[0]};
+    for (int i = 0; i < 3; ++i) p.stride[i] = 1;
+    for (int i = 0; i < ns; ++i) {
+        p.stride[i] = static_cast<int32_t>(st[i]);
+        p.pad_begin[i] = static_cast<int32_t>(full[i]);
+        p.pad_end[i] = static_cast<int32_t>(full.size() == static_cast<size_t>(2 * ns) ? full[ns + i] : full[i]);
+        y_shape->push_back((x.shape()[2 + i] + p.pad_begin[i] + p.pad_end[i] - w.shape()[2 + i]) / p.stride[i] + 1);
+    }
+    return p;
 }
 
 }  // namespace runtime

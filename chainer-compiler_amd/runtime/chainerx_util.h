@@ -30,5 +30,11 @@ chx_hip_conv_params MakeConvParams(
 
 chainerx::Shape ConvOutputShape(const chainerx::Array& x, const chainerx::Array& w, const chx_hip_conv_params& p);
 
+// The same for one or three spatial axes (the completion helpers above are rank-generic, as in the reference), with
+// the result shape.
+chx_hip_conv_nd_params MakeConvNdParams(
+        const chainerx::Array& x, const chainerx::Array& w, const Int64StackVector& strides, const Int64StackVector& pads,
+        int group, const std::string& auto_pad, chainerx::Shape* y_shape);
+
 }  // namespace runtime
 }  // namespace chainer_compiler

@@ -224,6 +224,17 @@ chainerx::Array CastOp::RunImpl(ChxVMState* st, const chainerx::Array& input) {
     return y;
 }
 
+// chainerx::LeftShift / RightShift over the broadcast of x and y (runtime/ops/quantize.cc:153-163)
+chainerx::Array BitShiftOp::RunImpl(ChxVMState* st, const chainerx::Array& x, const chainerx::Array& y) {
+    CHECK(chainerx::GetKind(x.dtype()) != chainerx::DtypeKind::kFloat) << "BitShift of " << x.dtype();
+    CHECK(chainerx::GetKind(y.dtype()) != chainerx::DtypeKind::kFloat) << "BitShift by " << y.dtype();
+    CHECK(direction == "LEFT" || direction == "RIGHT") << "BitShift direction " << direction;
+    chainerx::Array z = chainerx::Empty(chainerx::internal::BroadcastShapes(x.shape(), y.shape()), x.dtype());
+    chx_hip_tensor xt = x.hip(), yt = y.hip(), zt = z.hip();
+    CHXVM_HIP_CALL(chx_hip_bit_shift(&xt, &yt, direction == "LEFT" ? 1 : 0, &zt, chainerx::CurrentStream()));
+    return z;
+}
+
 // a view of the same memory, after a dense copy where the array is not dense (runtime/ops/manipulation.cc:30-53);
 // -1 and 0 entries as ONNX defines them
 chainerx::Array ReshapeOp::RunImpl(ChxVMState* st, const chainerx::Array& data, const chainerx::Shape& shape) {

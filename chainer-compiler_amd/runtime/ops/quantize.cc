@@ -111,6 +111,21 @@ chainerx::Array QLinearConvOp::RunImpl(
     CHECK_EQ(w_scale.GetTotalSize(), w_zero_point.GetTotalSize());
     CHECK_EQ(w_scale.shape().size(), w_zero_point.shape().size());
     CheckQuantizedDtype(y_zero_point.dtype(), "QLinearConv y_zero_point");
+    if (q_x.ndim() != 4) {
+        // one or three spatial axes: the rank-generic entry point, operands as they are, a dense result
+        chainerx::Shape nd_shape;
+        const chx_hip_conv_nd_params np = MakeConvNdParams(q_x, q_w, strides, pads, group, auto_pad, &nd_shape);
+        const uint32_t nd_flags =
+                CHX_HIP_ROUND_REFERENCE | (st->options().qlinearconv_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
+        chainerx::Array y = chainerx::Empty(nd_shape, y_zero_point.dtype());
+        chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), yt = y.hip(), bt;
+        if (b.has_value()) bt = b->hip();
+        CHXVM_HIP_CALL(chx_hip_qlinear_conv_nd(
+                &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &wt, &st2, &zt,
+                static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), b.has_value() ? &bt : nullptr, &np,
+                nd_flags, &yt, chainerx::CurrentStream()));
+        return y;
+    }
     const chx_hip_conv_params p = MakeConvParams(q_x, q_w, strides, pads, group, auto_pad);
     const chainerx::Shape y_shape = ConvOutputShape(q_x, q_w, p);
     // The reference adds the bias as an unscaled float after the convolution (runtime/ops/quantize.cc:93);
@@ -197,6 +212,16 @@ chainerx::Array ConvIntegerOp::RunImpl(
         const chainerx::Array& q_w,
         const absl::optional<StrictScalar>& x_zero_point,
         const absl::optional<chainerx::Array>& w_zero_point_opt) {
+    if (q_x.ndim() != 4) {
+        chainerx::Shape nd_shape;
+        const chx_hip_conv_nd_params np = MakeConvNdParams(q_x, q_w, strides, pads, group, auto_pad, &nd_shape);
+        chainerx::Array y = chainerx::Empty(nd_shape, chainerx::Dtype::kInt32);
+        chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), yt = y.hip(), zt;
+        if (w_zero_point_opt.has_value()) zt = w_zero_point_opt->hip();
+        const int32_t xz = x_zero_point.has_value() ? static_cast<int32_t>(static_cast<int64_t>(*x_zero_point)) : 0;
+        CHXVM_HIP_CALL(chx_hip_conv_integer_nd(&xt, &wt, xz, w_zero_point_opt.has_value() ? &zt : nullptr, &np, &yt, chainerx::CurrentStream()));
+        return y;
+    }
     const chx_hip_conv_params p = MakeConvParams(q_x, q_w, strides, pads, group, auto_pad);
     chainerx::Array y = EmptyLike4d(q_x, ConvOutputShape(q_x, q_w, p), chainerx::Dtype::kInt32);
     chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), yt = y.hip(), zt;

@@ -88,6 +88,16 @@ typedef struct chx_hip_conv_params {
     int32_t group;
 } chx_hip_conv_params;
 
+/* The same for convolutions over 1, 2 or 3 spatial axes (ComplementStride, ComplementPad and GroupedConv are
+ * rank-generic, runtime/chainerx_util.cc:180-200,313-340): entry i describes spatial axis i of x, outermost first. */
+typedef struct chx_hip_conv_nd_params {
+    int32_t n_spatial;
+    int32_t stride[3];
+    int32_t pad_begin[3];
+    int32_t pad_end[3];
+    int32_t group;
+} chx_hip_conv_nd_params;
+
 typedef struct chx_hip_device_props {
     int32_t compute_units;
     int32_t clock_khz;
@@ -163,6 +173,18 @@ int chx_hip_qlinear_conv(
         const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
         const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
         const chx_hip_tensor* bias, const chx_hip_conv_params* params, uint32_t flags, chx_hip_tensor* y, void* stream);
+
+/* QLinearConvOp::RunImpl and ConvIntegerOp::RunImpl (runtime/ops/quantize.cc:62-94,116-146) for x [N,C,L],
+ * [N,C,H,W] or [N,C,D,H,W] with w and y of the same rank.  One spatial axis runs as a 2-D convolution over images one
+ * pixel high (every kernel of the 2-D entry points); three run on the direct kernel (one lane per output element,
+ * exact int32 accumulation, the same requantization). */
+int chx_hip_qlinear_conv_nd(
+        const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, const chx_hip_tensor* w,
+        const chx_hip_tensor* w_scale, const chx_hip_tensor* w_zero_point, float y_scale, int32_t y_zero_point,
+        const chx_hip_tensor* bias, const chx_hip_conv_nd_params* params, uint32_t flags, chx_hip_tensor* y, void* stream);
+int chx_hip_conv_integer_nd(
+        const chx_hip_tensor* x, const chx_hip_tensor* w, int32_t x_zero_point, const chx_hip_tensor* w_zero_point,
+        const chx_hip_conv_nd_params* params, chx_hip_tensor* y, void* stream);
 
 /* The same op with the weight-side work (repacking for the MFMA kernel, per-channel
  * sums, the zero-point read-back) done once.  The reference redoes its weight
@@ -367,6 +389,12 @@ int chx_hip_reduce_min_max(const chx_hip_tensor* x, int32_t is_max, chx_hip_tens
  * (two streams, two threads) share the array and race: keep them in one stream's order.  Results are
  * identical to chx_hip_reduce_min_max's. */
 int chx_hip_reduce_min_max_noalloc(const chx_hip_tensor* x, int32_t is_max, chx_hip_tensor* y, void* stream);
+
+/* BitShiftOp::RunImpl, runtime/ops/quantize.cc:153-163 (chainerx::LeftShift / RightShift): z = x << y when `left`
+ * is non-zero, x >> y otherwise, over the broadcast of x and y; one integer type (uint8, int8, int16, int32, int64)
+ * for x, y and z; z has the broadcast shape.  The right shift of a signed type is arithmetic; a count of the element
+ * width or more (which C leaves undefined) gives 0, or -1 for a negative x shifted right. */
+int chx_hip_bit_shift(const chx_hip_tensor* x, const chx_hip_tensor* y, int32_t left, chx_hip_tensor* z, void* stream);
 
 /* The scan behind ChxVMState::CheckNans / CheckInfs (runtime/chxvm_state.cc:215-263: chainerx::IsNan / IsInf,
  * Sum, AsScalar): *count receives the number of NaN elements of x (infinities = 0) or of +-Inf elements

@@ -698,3 +698,37 @@ def test_fusion_group_with_the_reference_kernel_text(g, vm, oracle):
     xs = [torch.from_numpy(np.random.default_rng(42 + i).standard_normal((4, 16)).astype(np.float16)).cuda() for i in range(4)]
     out = vm.Program(bh.serialize()).run(dict(zip("xabc", xs)))
     assert out["y"].dtype == np.float16 and out["y"].shape == (4, 16)
+
+
+def test_bit_shift_instruction(g, vm):
+    """BitShift as a VM instruction (IDL row of runtime/chxvm_defs.py:471): direction is a string attribute."""
+    x = np.arange(24, dtype=np.uint8).reshape(2, 3, 4) * 9
+    y = np.array([1, 0, 3, 7], np.uint8)
+    for direction, fn in (("LEFT", np.left_shift), ("RIGHT", np.right_shift)):
+        b = vm.ProgramBuilder()
+        b.output("z", b.BitShift(b.input("x", "uint8"), b.constant(y), direction))
+        out = vm.Program(b.serialize()).run({"x": g.dev(x)})
+        np.testing.assert_array_equal(out["z"], fn(x, y))
+    b = vm.ProgramBuilder()
+    b.output("z", b.BitShift(b.input("x", "uint8"), b.constant(y), "UP"))
+    with pytest.raises(vm.ChxVMError) as e:
+        vm.Program(b.serialize()).run({"x": g.dev(x)})
+    assert "direction" in str(e.value)
+
+
+def test_convolution_over_one_spatial_axis_as_an_instruction(g, vm, oracle):
+    """QLinearConv and ConvInteger on x [N,C,L]: the attributes are completed for one spatial axis
+    (ComplementStride / ComplementPad, runtime/chainerx_util.cc:180-200) and the result has three axes."""
+    rng = np.random.default_rng(71)
+    x, w = rand_q(rng, (2, 64, 40), np.uint8), rand_q(rng, (16, 64, 3), np.int8)
+    ws, wz = rng.uniform(0.001, 0.01, 16).astype(np.float32), np.zeros(16, np.int8)
+    b = vm.ProgramBuilder()
+    xi = b.input("x", "uint8", x.shape)
+    y = b.QLinearConv(xi, b.scalar(0.02, "float32"), b.scalar(3, "uint8"), b.constant(w), b.constant(ws), b.constant(wz),
+                      b.scalar(0.05, "float32"), b.scalar(128, "uint8"), None, [], [1], 1, "")
+    b.output("y", y)
+    b.output("yi", b.ConvInteger(xi, b.constant(w), b.scalar(3, "uint8"), None, [2], [], 1, ""))
+    out = vm.Program(b.serialize()).run({"x": g.dev(x)})
+    want = oracle.qlinear_conv_int(x[:, :, None, :], 0.02, 3, w[:, :, None, :], ws, wz, 0.05, 128, np.uint8, strides=(1, 1), pads=(0, 1))
+    np.testing.assert_array_equal(out["y"], want[:, :, 0, :])
+    np.testing.assert_array_equal(out["yi"], oracle.conv_integer(x[:, :, None, :], w[:, :, None, :], 3, None, strides=(1, 2), pads=(0, 0))[:, :, 0, :])

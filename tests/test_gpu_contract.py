@@ -619,3 +619,55 @@ def test_random_matmul_sweep(g, oracle):
         want = oracle.qlinear_matmul_int(a, 0.02, a_zp, b, b_scale, b_zp, y_scale, y_zp, ydt)
         got = g.ops.QLinearMatMul(g.dev(a), 0.02, a_zp, bd, b_scale, b_zp, y_scale, y_zp, zero_point_dtype=TDT[ydt])
         np.testing.assert_array_equal(g.host(got), want, err_msg=tag + " QLinearMatMul -> " + ydt.__name__)
+
+
+def _depth_folded(x, w, zp, sd, pd_b, pd_e, od):
+    """The 2-D problem that output depth `od` of a 3-D convolution is: the KD input slices under the window stacked
+    along the channels (channel c, tap kd -> c*KD + kd, so groups stay contiguous), depth padding filled with the zero
+    point (x - zero_point = 0 there: the reference's zero padding of the zero-point-subtracted tensor)."""
+    n, c, d, h, wd = x.shape
+    kd = w.shape[2]
+    xp = np.full((n, c, d + pd_b + pd_e, h, wd), zp, x.dtype)
+    xp[:, :, pd_b:pd_b + d] = x
+    x2 = xp[:, :, od * sd:od * sd + kd].reshape(n, c * kd, h, wd)
+    w2 = w.reshape(w.shape[0], w.shape[1] * kd, w.shape[3], w.shape[4])
+    return np.ascontiguousarray(x2), np.ascontiguousarray(w2)
+
+
+def test_convolutions_over_one_and_three_spatial_axes(g, oracle):
+    """ComplementStride / ComplementPad / GroupedConv are rank-generic (runtime/chainerx_util.cc:180-200,313-340): x [N,C,L]
+    against the 2-D oracle on images one pixel high; x [N,C,D,H,W] against the 2-D oracle on the depth-folded problem."""
+    rng = np.random.default_rng(61)
+    # one spatial axis: reaches the matrix-core kernel (64 channels) and the direct kernel (groups)
+    for c, oc, group in ((64, 32, 1), (12, 8, 2)):
+        x, w = rand_q(rng, (3, c, 50), np.uint8), rand_q(rng, (oc, c // group, 5), np.int8)
+        ws, wz = rng.uniform(0.001, 0.01, oc).astype(np.float32), np.zeros(oc, np.int8)
+        bias = rng.integers(-500, 500, oc).astype(np.int32)
+        got = g.ops.QLinearConv(g.dev(x), 0.02, 120, g.dev(w), g.dev(ws), g.dev(wz), 0.05, 128, g.dev(bias), strides=[2], pads=[2, 1],
+                                group=group, flags=g.capi.BIAS_ONNX_INT32)
+        want = oracle.qlinear_conv_int(x[:, :, None, :], 0.02, 120, w[:, :, None, :], ws, wz, 0.05, 128, np.uint8, bias=bias, strides=(1, 2),
+                                       pads=(0, 2, 0, 1), group=group, bias_mode=oracle.BIAS_ONNX_INT32)
+        assert tuple(got.shape) == (3, oc, want.shape[3])
+        np.testing.assert_array_equal(g.host(got), want[:, :, 0, :])
+        goti = g.ops.ConvInteger(g.dev(x), g.dev(w), 120, None, strides=[2], pads=[2, 1], group=group)
+        np.testing.assert_array_equal(g.host(goti), oracle.conv_integer(x[:, :, None, :], w[:, :, None, :], 120, None, strides=(1, 2),
+                                                                         pads=(0, 2, 0, 1), group=group)[:, :, 0, :])
+    # three spatial axes
+    for group in (1, 2):
+        x, w = rand_q(rng, (2, 6, 7, 9, 8), np.uint8), rand_q(rng, (4, 6 // group, 3, 2, 3), np.int8)
+        ws, wz = rng.uniform(0.001, 0.01, 4).astype(np.float32), rand_q(rng, (4,), np.int8)
+        strides, pb, pe = (2, 1, 2), (1, 0, 2), (1, 1, 0)
+        got = g.ops.QLinearConv(g.dev(x), 0.03, 7, g.dev(w), g.dev(ws), g.dev(wz), 0.04, 100, None, strides=list(strides),
+                                pads=list(pb) + list(pe), group=group)
+        goti = g.ops.ConvInteger(g.dev(x), g.dev(w), 7, g.dev(wz), strides=list(strides), pads=list(pb) + list(pe), group=group)
+        od_n = (7 + pb[0] + pe[0] - 3) // strides[0] + 1
+        assert got.shape[2] == od_n and goti.dtype == torch.int32
+        for od in range(od_n):
+            x2, w2 = _depth_folded(x, w, 7, strides[0], pb[0], pe[0], od)
+            want = oracle.qlinear_conv_int(x2, 0.03, 7, w2, ws, wz, 0.04, 100, np.uint8, strides=strides[1:], pads=(pb[1], pb[2], pe[1], pe[2]),
+                                           group=group, bias_mode=oracle.BIAS_REFERENCE_FLOAT)
+            np.testing.assert_array_equal(g.host(got)[:, :, od], want, err_msg="group %d depth %d" % (group, od))
+            wanti = oracle.conv_integer(x2, w2, 7, wz, strides=strides[1:], pads=(pb[1], pb[2], pe[1], pe[2]), group=group)
+            np.testing.assert_array_equal(g.host(goti)[:, :, od], wanti)
+    with pytest.raises(g.capi.ChxHipError):
+        g.ops.ConvInteger(g.dev(rand_q(rng, (1, 2, 3, 3, 3, 3), np.uint8)), g.dev(rand_q(rng, (1, 2, 1, 1, 1, 1), np.int8)))

@@ -121,3 +121,30 @@ def test_errors(g):
         g.ops.QuantizeLinear(x, 1.0, 0, torch.uint8, out=torch.empty(9, dtype=torch.uint8, device="cuda"))
     # empty input is fine
     assert g.ops.QuantizeLinear(torch.zeros(0, device="cuda"), 1.0).numel() == 0
+
+
+def test_bit_shift_against_numpy(g, vm=None):
+    """BitShiftOp (runtime/ops/quantize.cc:153-163): both directions, every integer type of the array library, with
+    broadcasting; counts below the element width, where numpy, C and the ONNX operator agree, plus numpy's results
+    for counts of the width and beyond."""
+    rng = np.random.default_rng(51)
+    for dt, lo, hi in ((np.uint8, 0, 256), (np.int8, -128, 128), (np.int16, -2 ** 15, 2 ** 15), (np.int32, -2 ** 31, 2 ** 31),
+                       (np.int64, -2 ** 62, 2 ** 62)):
+        bits = np.dtype(dt).itemsize * 8
+        x = rng.integers(lo, hi, size=(3, 5, 17)).astype(dt)
+        y = rng.integers(0, bits, size=(5, 1)).astype(dt)
+        for direction, fn in (("LEFT", np.left_shift), ("RIGHT", np.right_shift)):
+            got = g.ops.BitShift(g.dev(x), g.dev(y), direction)
+            assert tuple(got.shape) == (3, 5, 17)
+            np.testing.assert_array_equal(g.host(got), fn(x, y), err_msg="%s %s" % (np.dtype(dt).name, direction))
+            # a strided operand, and counts from the width upwards
+            big = np.array([bits, bits + 3, 100 if bits > 8 else 77], dt)
+            got = g.ops.BitShift(g.dev(x).permute(2, 0, 1)[:3], g.dev(big).reshape(3, 1, 1), direction)
+            want = np.where(np.transpose(x, (2, 0, 1))[:3] < 0, -1, 0).astype(dt) if direction == "RIGHT" else np.zeros((3, 3, 5), dt)
+            np.testing.assert_array_equal(g.host(got), want)
+    # the ONNX operator's own examples (uint8)
+    x, y = np.array([16, 4, 1], np.uint8), np.array([1, 2, 3], np.uint8)
+    assert g.host(g.ops.BitShift(g.dev(x), g.dev(y), "RIGHT")).tolist() == [8, 1, 0]
+    assert g.host(g.ops.BitShift(g.dev(x), g.dev(y), "LEFT")).tolist() == [32, 16, 8]
+    with pytest.raises(g.capi.ChxHipError):
+        g.ops.BitShift(g.dev(np.zeros(3, np.float32)), g.dev(np.zeros(3, np.float32)), "LEFT")
