@@ -142,6 +142,8 @@ inline bool aligned(const void* p, size_t a) {
 int launch_check(const char* kernel);
 
 // Stream-ordered scratch memory for one call.
+// device address of the scratch array of chx_hip_reduce_min_max_noalloc on the current device, looked up once (reduce_cast.hip)
+int prepare_noalloc_scratch();
 // whether work submitted to s is being recorded into a graph instead of executed
 bool stream_is_capturing(hipStream_t s);
 int scratch_alloc(void** p, size_t bytes, hipStream_t s);

@@ -371,6 +371,7 @@ bool byte_ranges_overlap(const chx_hip_tensor& a, const chx_hip_tensor& b) {
 struct ScratchCache {
     void* ptr[2] = {nullptr, nullptr};
     size_t size[2] = {0, 0};
+    bool pinned = false;  // a recorded run holds these addresses: the buffers must not move
 };
 
 struct ConvCall {
@@ -397,6 +398,10 @@ struct ConvCall {
 int acquire_scratch(ScratchCache* cache, int slot, size_t bytes, hipStream_t s, void** out) {
     if (!cache) return scratch_alloc(out, bytes, s);
     if (cache->size[slot] < bytes) {
+        if (cache->pinned)
+            CHX_FAIL(CHX_HIP_EPINNED,
+                     "this convolution plan is pinned by a recorded run and would have to move its scratch memory (%zu bytes needed, %zu held): "
+                     "run larger inputs before recording, or after the recording has been destroyed", bytes, cache->size[slot]);
         // the old buffer may still be in use by work queued on the stream
         CHX_HIP_CALL(hipStreamSynchronize(s));
         if (cache->ptr[slot]) CHX_HIP_CALL(hipFree(cache->ptr[slot]));
@@ -484,9 +489,10 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     } else if (is_contiguous(y) && !c.out_int32 && !c.res) {
         const int64_t OHW = (int64_t)cs.OH * cs.OW;
         const int pitch = round_up(cs.OC, 16);
-        if (acquire_scratch(c.cache, 1, (size_t)cs.N * OHW * pitch, s, &y_scratch) != CHX_HIP_OK) {
+        const int rc_y = acquire_scratch(c.cache, 1, (size_t)cs.N * OHW * pitch, s, &y_scratch);
+        if (rc_y != CHX_HIP_OK) {
             release_scratch(c.cache, x_scratch, s);
-            return CHX_HIP_ERUNTIME;
+            return rc_y;
         }
         a.y = static_cast<char*>(y_scratch);
         a.y_px_stride = pitch;
@@ -819,6 +825,9 @@ struct chx_hip_qconv_plan {
     // with which its two-multiply-add form is exact (find_affine_residual); kept so that the search runs once
     bool res_known = false;
     chx::ResidualAdd res_key, res_found;
+    // recorded runs (HIP graphs) that hold addresses of this plan's packed weights and scratch memory
+    int pins = 0;
+    bool destroy_when_unpinned = false;
 };
 
 extern "C" int chx_hip_qlinear_conv(
@@ -1179,8 +1188,25 @@ extern "C" int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char*
     return CHX_HIP_OK;
 }
 
+extern "C" int chx_hip_qconv_plan_pin(chx_hip_qconv_plan* plan, int32_t delta) {
+    CHX_REQUIRE(plan != nullptr && (delta == 1 || delta == -1), "QLinearConv plan pin: a plan and +1 or -1");
+    CHX_REQUIRE(plan->pins + delta >= 0, "QLinearConv plan pin: released more often than pinned");
+    plan->pins += delta;
+    plan->scratch.pinned = plan->pins > 0;
+    if (plan->pins == 0 && plan->destroy_when_unpinned) {
+        plan->destroy_when_unpinned = false;
+        chx_hip_qconv_plan_destroy(plan);
+    }
+    return CHX_HIP_OK;
+}
+
 extern "C" void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan) {
     if (!plan) return;
+    if (plan->pins > 0) {
+        // a recorded run still launches kernels on this plan's memory: it goes when the last pin does
+        plan->destroy_when_unpinned = true;
+        return;
+    }
     chx::release_packed(&plan->pw, true, nullptr);
     chx::release_depthwise(&plan->dw, true, nullptr);
     for (int i = 0; i < 2; ++i)

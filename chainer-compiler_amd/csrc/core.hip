@@ -130,7 +130,7 @@ int chx_hip_init(int device) {
     CHX_HIP_CALL(hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
-    return CHX_HIP_OK;
+    return prepare_noalloc_scratch();
 }
 
 int chx_hip_get_device_props(chx_hip_device_props* out) {

@@ -42,6 +42,17 @@ int noalloc_scratch(float** out) {
     return CHX_HIP_OK;
 }
 
+}  // namespace
+
+// chx_hip_init asks for the address on its device, so that the first call of the entry point on a capturing
+// stream finds it known (the lookup is no stream operation, but it need not happen inside a recording).
+int prepare_noalloc_scratch() {
+    float* p = nullptr;
+    return noalloc_scratch(&p);
+}
+
+namespace {
+
 __device__ __forceinline__ int64_t strided_offset(int64_t flat, const StridedDesc& d) {
     int64_t off = 0;
     for (int a = d.ndim - 1; a >= 0; --a) {

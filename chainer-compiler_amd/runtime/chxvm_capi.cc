@@ -60,9 +60,11 @@ struct chxvm_replay {
     chx_hip_graph* graph = nullptr;
     chxvm_outputs outputs;
     int32_t warm_runs = 0;
+    std::vector<chx_hip_qconv_plan*> pinned_plans;  // whose memory the graph's kernels address
 
     ~chxvm_replay() {
         chx_hip_graph_destroy(graph);
+        for (chx_hip_qconv_plan* plan : pinned_plans) (void)chx_hip_qconv_plan_pin(plan, -1);
         outputs.arrays.clear();
         outputs.keep_inputs.clear();
         if (stream) (void)chx_hip_stream_destroy(stream);
@@ -211,7 +213,9 @@ int32_t chxvm_program_capture(
         InOuts result;
         try {
             chainerx::DeviceContextScope scope(r->stream, r->pool.get());
-            result = program->vm->Run(in, options);
+            ChxVMOptions recorded = options;
+            recorded.pinned_plans = &r->pinned_plans;
+            result = program->vm->Run(in, recorded);
         } catch (...) {
             chx_hip_graph* dropped = nullptr;
             (void)chx_hip_capture_end(r->stream, &dropped);

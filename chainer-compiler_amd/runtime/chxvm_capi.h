@@ -62,7 +62,13 @@ void chxvm_outputs_destroy(chxvm_outputs* outputs);
  * recording.  launch() enqueues the recorded run on `stream`, or on the replay's own stream when that is
  * null (synchronize() waits for it); the outputs (same names and shapes on every launch) are device memory of
  * the replay, valid until destroy, rewritten by every launch.  One replay must not be launched concurrently
- * with itself. */
+ * with itself.
+ * The recorded kernels address memory of the program's convolution plans (packed weights, transposition and
+ * expansion scratch), which eager runs of the same program share.  The plans a recording has used are therefore
+ * pinned until the replay is destroyed: an eager run of the program on larger inputs, which would have to move
+ * that scratch memory, fails with an error instead (run the largest inputs before capture()), and a plan that
+ * the program gives up (other weight operands) is released only with the replay.  Eager runs and launches of a
+ * replay of one program must not overlap in time: both write that scratch memory. */
 typedef struct chxvm_replay chxvm_replay;
 int32_t chxvm_program_capture(
         chxvm_program* program, const char* const* input_names, const chx_hip_tensor* inputs, int32_t num_inputs, chxvm_replay** out);

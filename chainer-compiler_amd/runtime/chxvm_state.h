@@ -37,6 +37,9 @@ struct ChxVMOptions {
     // QLinearConv bias: false = the reference's unscaled float bias added after the convolution
     // (runtime/ops/quantize.cc:93), true = the ONNX operator's int32 bias added to the accumulator
     bool qlinearconv_onnx_int32_bias = false;
+    // set while a run is being recorded into a device graph: every convolution plan the run uses is pinned and listed
+    // here, so that the recording can release them when it is destroyed (chx_hip_qconv_plan_pin)
+    std::vector<struct chx_hip_qconv_plan*>* pinned_plans = nullptr;
 };
 
 class ChxVMState {

@@ -156,6 +156,11 @@ chainerx::Array QLinearConvOp::RunImpl(
         impl_->w_zero_point = w_zero_point;
         impl_->bias = b.has_value() ? *b : chainerx::Array();
     }
+    if (std::vector<chx_hip_qconv_plan*>* pinned = st->options().pinned_plans) {
+        // this run is being recorded: the recording holds addresses inside the plan
+        CHXVM_HIP_CALL(chx_hip_qconv_plan_pin(impl_->plan, 1));
+        pinned->push_back(impl_->plan);
+    }
     if (QLinearConvResidualRequest* req = st->residual_request()) {
         const bool same_quantization = static_cast<float>(y_scale) == req->y_scale &&
                                        static_cast<int64_t>(y_zero_point) == req->y_zero_point && y_zero_point.dtype() == req->y_dtype;

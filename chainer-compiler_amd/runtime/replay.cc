@@ -12,6 +12,7 @@ PoolAllocator::~PoolAllocator() {
 std::shared_ptr<void> PoolAllocator::Allocate(size_t bytes) {
     const size_t want = (bytes + 255) / 256 * 256;
     size_t index = 0;
+    void* ptr = nullptr;  // read under the lock: a concurrent Allocate may grow (move) the vector
     {
         std::lock_guard<std::mutex> lock(mu_);
         size_t best = blocks_.size();
@@ -28,9 +29,10 @@ std::shared_ptr<void> PoolAllocator::Allocate(size_t bytes) {
             blocks_[best].free = false;
         }
         index = best;
+        ptr = blocks_[index].ptr;
     }
     std::shared_ptr<PoolAllocator> self = shared_from_this();
-    return std::shared_ptr<void>(blocks_[index].ptr, [self, index](void*) { self->Release(index); });
+    return std::shared_ptr<void>(ptr, [self, index](void*) { self->Release(index); });
 }
 
 void PoolAllocator::Release(size_t index) {

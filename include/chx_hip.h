@@ -55,7 +55,8 @@ enum {
     CHX_HIP_EINVAL = 1,      /* bad argument: dtype, shape, stride, null pointer */
     CHX_HIP_EUNSUPPORTED = 2,/* valid for the reference op but not implemented on the device */
     CHX_HIP_ERUNTIME = 3,    /* a HIP / hiprtc call failed */
-    CHX_HIP_ECOMPILE = 4     /* run-time compilation of a fused kernel failed */
+    CHX_HIP_ECOMPILE = 4,    /* run-time compilation of a fused kernel failed */
+    CHX_HIP_EPINNED = 5      /* the call would have to move memory that a recorded run (HIP graph) addresses */
 };
 
 /* Behaviour switches.  0 is always the reference's behaviour. */
@@ -229,6 +230,12 @@ int chx_hip_qconv_plan_run_add(
         const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
         int32_t y_zero_point, int32_t y_dtype, uint32_t flags, const chx_hip_tensor* r, float r_scale, int32_t r_zero_point,
         float out_scale, int32_t out_zero_point, int32_t relu, chx_hip_tensor* out, void* stream);
+/* Pins (delta = +1) or releases (-1) the plan's device memory for a recorded run: a HIP graph captured over
+ * chx_hip_qconv_plan_run holds the addresses of the packed weights and of the scratch memory.  While a plan is
+ * pinned, a run that would have to enlarge (move) the scratch memory fails with CHX_HIP_EPINNED, and
+ * chx_hip_qconv_plan_destroy is deferred until the last pin is released.  No counterpart in the reference (it has
+ * no recorded runs); the ChxVM runtime pins every plan a recorded program run has used. */
+int chx_hip_qconv_plan_pin(chx_hip_qconv_plan* plan, int32_t delta);
 void chx_hip_qconv_plan_destroy(chx_hip_qconv_plan* plan);
 
 /* ---- integer contractions ------------------------------------------------------------- */

@@ -732,3 +732,34 @@ def test_convolution_over_one_spatial_axis_as_an_instruction(g, vm, oracle):
     want = oracle.qlinear_conv_int(x[:, :, None, :], 0.02, 3, w[:, :, None, :], ws, wz, 0.05, 128, np.uint8, strides=(1, 1), pads=(0, 1))
     np.testing.assert_array_equal(out["y"], want[:, :, 0, :])
     np.testing.assert_array_equal(out["yi"], oracle.conv_integer(x[:, :, None, :], w[:, :, None, :], 3, None, strides=(1, 2), pads=(0, 0))[:, :, 0, :])
+
+
+def test_a_recording_pins_the_plans_it_has_used(g, vm, oracle):
+    """The kernels of a recorded run address the scratch memory of the convolution plans.  An eager run of the same
+    program on a larger input, which would have to move that memory, is refused while the recording lives; the
+    recording keeps giving the right values, and after its destruction the larger run goes through."""
+    rng = np.random.default_rng(81)
+    w = rand_q(rng, (32, 64, 3, 3), np.int8)
+    ws, wz = rng.uniform(0.001, 0.01, 32).astype(np.float32), np.zeros(32, np.int8)
+    b = vm.ProgramBuilder()
+    y = b.QLinearConv(b.input("x", "uint8"), b.scalar(0.02, "float32"), b.scalar(0, "uint8"), b.constant(w), b.constant(ws), b.constant(wz),
+                      b.scalar(0.05, "float32"), b.scalar(128, "uint8"), None, [], [1, 1], 1, "")
+    b.output("y", y)
+    prog = vm.Program(b.serialize())
+    small, large = rand_q(rng, (1, 64, 12, 12), np.uint8), rand_q(rng, (4, 64, 20, 20), np.uint8)
+    want = lambda x: oracle.qlinear_conv_int(x, 0.02, 0, w, ws, wz, 0.05, 128, np.uint8, pads=(1, 1))
+    xd = g.dev(small)   # NCHW-contiguous: the plan transposes it into scratch memory of its own
+    replay = prog.capture({"x": xd})
+    with pytest.raises(vm.ChxVMError) as e:
+        prog.run({"x": g.dev(large)})
+    assert "pinned by a recorded run" in str(e.value)
+    again = rand_q(rng, small.shape, np.uint8)
+    xd.copy_(torch.from_numpy(again))
+    torch.cuda.synchronize()
+    replay.launch()
+    replay.synchronize()
+    np.testing.assert_array_equal(replay.outputs()["y"], want(again))
+    np.testing.assert_array_equal(prog.run({"x": g.dev(small)})["y"], want(small))   # the recorded size still runs eagerly
+    replay.close()
+    np.testing.assert_array_equal(prog.run({"x": g.dev(large)})["y"], want(large))
+    prog.close()

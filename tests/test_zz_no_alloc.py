@@ -44,6 +44,37 @@ def test_sizes_beyond_the_limit_are_refused(g):
     rc = g.capi.lib().chx_hip_reduce_min_max_noalloc(g.capi.ref(huge), ctypes.c_int32(1), g.capi.ref(y), g.capi.stream_ptr())
     assert rc == g.capi.EINVAL
     assert b"at most" in g.capi.lib().chx_hip_last_error()
-    # the limit itself passes the check (and reads the one element 2^30 times)
-    ok = one.expand(1 << 20)
+    # the limit itself passes (the one element is read 2^30 times)
+    ok = one.expand(1 << 30)
     assert _reduce(g, "chx_hip_reduce_min_max_noalloc", ok, True) == 0.0
+
+
+def test_inside_a_recording(g):
+    """What the entry point is for: between capture_begin and capture_end on a created stream it is recorded (it
+    allocates nothing), and every replay reduces what the input holds then; the allocating entry point is refused
+    there."""
+    lib = g.capi.lib()
+    stream = ctypes.c_void_p()
+    g.capi.check(lib.chx_hip_stream_create(ctypes.byref(stream)))
+    rng = np.random.default_rng(43)
+    x = torch.from_numpy(rng.standard_normal((300, 1000)).astype(np.float32)).cuda()
+    y = torch.full((), float("nan"), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    g.capi.check(lib.chx_hip_capture_begin(stream))
+    rc_alloc = lib.chx_hip_reduce_min_max(g.capi.ref(x), ctypes.c_int32(1), g.capi.ref(y), stream)
+    rc = lib.chx_hip_reduce_min_max_noalloc(g.capi.ref(x), ctypes.c_int32(1), g.capi.ref(y), stream)
+    graph = ctypes.c_void_p()
+    g.capi.check(lib.chx_hip_capture_end(stream, ctypes.byref(graph)))
+    assert rc_alloc == g.capi.EUNSUPPORTED and rc == 0
+    try:
+        for i in range(3):
+            x.copy_(torch.from_numpy(rng.standard_normal((300, 1000)).astype(np.float32) * (i + 1)))
+            torch.cuda.synchronize()
+            g.capi.check(lib.chx_hip_graph_launch(graph, stream))
+            g.capi.check(lib.chx_hip_stream_synchronize(stream))
+            assert float(y) == float(x.max())
+            # eager work of the same entry point between the replays (it shares the scratch array, one call at a time)
+            assert _reduce(g, "chx_hip_reduce_min_max_noalloc", x[:7], False) == x[:7].min().cpu().numpy()
+    finally:
+        lib.chx_hip_graph_destroy(graph)
+        g.capi.check(lib.chx_hip_stream_destroy(stream))
