@@ -211,20 +211,52 @@ bool weights_fit_mfma(const chx_hip_tensor& w, int group) {
     return (int64_t)pw.KP * 128 * 128 < (int64_t(1) << 31) && w.shape[0] < (1 << 24);
 }
 
-// Tile shape: the largest tile that still gives every compute unit a work-group.
-void pick_tile(int OC, int64_t M, int bk, int* tile_oc, int* tile_px, int* max_wgs_per_cu, int* waves) {
-    // CHX_HIP_TILE=<oc>,<px>[,<work-groups per compute unit>[,<wavefronts: 4 or 8>]] forces a launch configuration
-    // (read on every call: a tuning aid, and how the tests reach every configuration the tuner may choose)
-    *waves = 4;
+// How a convolution is launched, beyond what its operands decide.  The defaults are what a host wants; the
+// environment variables are overrides for tuning and for tests (which reach every launch configuration through them),
+// read when a plan is created or a one-shot entry point is called, never on the path of a plan's runs.
+//   CHX_HIP_TILE=<oc>,<px>[,<work-groups per compute unit>[,<wavefronts: 4 or 8>]]  forces a launch configuration
+//   CHX_HIP_AUTOTUNE=0          keeps the heuristic tile choice instead of timing the configurations
+//   CHX_HIP_NO_STEM=1           keeps few-channel first layers off the planar-input kernel
+//   CHX_HIP_AFFINE_RESIDUAL=0   keeps fused residual sums on the operation-by-operation arithmetic
+struct LaunchOptions {
+    bool forced_tile = false;
+    int tile_oc = 0, tile_px = 0, max_wgs_per_cu = 0, waves = 4;
+    bool autotune = true;
+    bool stem_kernel = true;
+    bool affine_residual = true;
+};
+
+LaunchOptions read_launch_options() {
+    LaunchOptions o;
     if (const char* env = getenv("CHX_HIP_TILE")) {
         int toc = 0, tpx = 0, cap = 0, wv = 4;
         const int got = sscanf(env, "%d,%d,%d,%d", &toc, &tpx, &cap, &wv);
+        if (got >= 2 && cap >= 0) {
+            o.forced_tile = true;
+            o.tile_oc = toc;
+            o.tile_px = tpx;
+            o.max_wgs_per_cu = got >= 3 ? cap : 0;
+            o.waves = wv;
+            o.autotune = false;
+        }
+    }
+    if (const char* e = getenv("CHX_HIP_AUTOTUNE")) o.autotune = o.autotune && e[0] != '0';
+    o.stem_kernel = getenv("CHX_HIP_NO_STEM") == nullptr;
+    if (const char* e = getenv("CHX_HIP_AFFINE_RESIDUAL")) o.affine_residual = e[0] != '0';
+    return o;
+}
+
+// Tile shape: the largest tile that still gives every compute unit a work-group.
+void pick_tile(const LaunchOptions& opt, int OC, int64_t M, int bk, int* tile_oc, int* tile_px, int* max_wgs_per_cu, int* waves) {
+    *waves = 4;
+    if (opt.forced_tile) {
+        const int toc = opt.tile_oc, tpx = opt.tile_px, wv = opt.waves;
         const bool four = wv == 4 && (toc == 64 || toc == 128) && (tpx == 64 || tpx == 128);
         const bool eight = wv == 8 && ((toc == 128 && tpx == 128) || (bk == 128 && ((toc == 128 && tpx == 256) || (toc == 64 && tpx == 128))));
-        if (got >= 2 && (four || eight) && cap >= 0) {
+        if (four || eight) {
             *tile_oc = toc;
             *tile_px = tpx;
-            *max_wgs_per_cu = got >= 3 ? cap : 0;
+            *max_wgs_per_cu = opt.max_wgs_per_cu;
             *waves = wv;
             return;
         }
@@ -254,11 +286,6 @@ struct TunedConfig {
 struct TuneCache {
     std::vector<TunedConfig> entries;
 };
-
-bool autotune_enabled() {
-    const char* e = getenv("CHX_HIP_AUTOTUNE");  // CHX_HIP_AUTOTUNE=0 keeps the heuristic
-    return !(e && e[0] == '0') && !getenv("CHX_HIP_TILE");
-}
 
 // Times every launch configuration on the call's operands and keeps the fastest in *best.
 int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hipStream_t s, TunedConfig* best) {
@@ -389,6 +416,7 @@ struct ConvCall {
     const int32_t* bias;
     RequantParams rq;
     const ResidualAdd* res = nullptr;  // a residual sum fused behind the requantization
+    LaunchOptions opt;                 // the plan's, or read for this one-shot call
 };
 
 // Runs the MFMA kernel on packed weights.  x may be channels-last (used in place) or
@@ -433,7 +461,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     const bool stem = pw.dense && pw.wd && !c.out_int32 && x.strides[3] == 1 &&
                       stem_patch_fits(cs.C, cs.KH, cs.KW, sh, sw) && ph < 64 && pw_ < 64 &&
                       (int64_t)cs.C * (x.strides[1] < 0 ? -x.strides[1] : x.strides[1]) < (int64_t(1) << 30) &&
-                      x.strides[2] > 0 && (int64_t)cs.H * x.strides[2] < (int64_t(1) << 30) && getenv("CHX_HIP_NO_STEM") == nullptr;
+                      x.strides[2] > 0 && (int64_t)cs.H * x.strides[2] < (int64_t(1) << 30) && c.opt.stem_kernel;
     if (stem && c.res) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "the planar-input kernel has no fused residual sum");
     if (stem) {
         // x is used in place
@@ -565,13 +593,13 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     if (c.res) a.res = *c.res;
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64, cap = 0, waves = 4;
-    pick_tile(cs.OC, a.M, a.bk, &toc, &tpx, &cap, &waves);
+    pick_tile(c.opt, cs.OC, a.M, a.bk, &toc, &tpx, &cap, &waves);
     int rc = CHX_HIP_OK;
     const TunedConfig* tuned = nullptr;
     if (c.tune) {
         for (const TunedConfig& t : c.tune->entries)
             if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW && t.with_res == (c.res != nullptr)) tuned = &t;
-        if (!tuned && autotune_enabled() && !stream_is_capturing(s)) {
+        if (!tuned && c.opt.autotune && !stream_is_capturing(s)) {
             TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, 4, c.res != nullptr};
             rc = tune_conv_mfma(a, xu, c.out_int32, c.rne, s, &best);
             if (rc == CHX_HIP_OK) {
@@ -753,8 +781,9 @@ int check_qconv(
 }
 
 ConvCall conv_call_from(const QConvChecked& q, const chx_hip_tensor* x, chx_hip_tensor* y, const chx_hip_conv_params* p,
-                        bool rne) {
+                        bool rne, const LaunchOptions& opt) {
     ConvCall c;
+    c.opt = opt;
     c.cache = nullptr;
     c.tune = nullptr;
     c.x = x;
@@ -821,10 +850,15 @@ struct chx_hip_qconv_plan {
     chx::PackedWeights pw;
     chx::ScratchCache scratch;  // makes run() unsafe to call concurrently on one plan
     chx::TuneCache tune;
-    // the residual sum last fused behind this convolution (run_add): its parameters, and whether constants were found
-    // with which its two-multiply-add form is exact (find_affine_residual); kept so that the search runs once
-    bool res_known = false;
-    chx::ResidualAdd res_key, res_found;
+    // the residual sums fused behind this convolution so far (run_add): each one's parameters, and whether constants
+    // were found with which its two-multiply-add form is exact (find_affine_residual); kept so that the search runs
+    // once per set of parameters, also for a caller that alternates between a few of them.  Oldest dropped first.
+    struct SearchedResidual {
+        chx::ResidualAdd key, found;
+    };
+    static constexpr size_t kMaxSearchedResiduals = 8;
+    std::vector<SearchedResidual> searched;
+    chx::LaunchOptions opt;  // read once, when the plan is created
     // recorded runs (HIP graphs) that hold addresses of this plan's packed weights and scratch memory
     int pins = 0;
     bool destroy_when_unpinned = false;
@@ -845,7 +879,7 @@ extern "C" int chx_hip_qlinear_conv(
         if (all_zero(zp)) {
             PackedWeights pw;
             CHX_PROPAGATE(make_packed(*w, false, s, &pw));
-            const int rc = run_conv_mfma(conv_call_from(q, x, y, params, rne), pw, s);
+            const int rc = run_conv_mfma(conv_call_from(q, x, y, params, rne, read_launch_options()), pw, s);
             release_packed(&pw, false, s);
             if (rc != CHX_HIP_EUNSUPPORTED) return rc;
         }
@@ -856,7 +890,7 @@ extern "C" int chx_hip_qlinear_conv(
         if (all_zero(zp)) {
             DepthwiseState st;
             CHX_PROPAGATE(make_depthwise(*w, false, s, &st));
-            const int rc = run_depthwise(conv_call_from(q, x, y, params, rne), st, s);
+            const int rc = run_depthwise(conv_call_from(q, x, y, params, rne, read_launch_options()), st, s);
             release_depthwise(&st, false, s);
             if (rc != CHX_HIP_EUNSUPPORTED) return rc;
         }
@@ -1018,6 +1052,7 @@ extern "C" int chx_hip_qconv_plan_create(
     p->params = *params;
     p->mfma = false;
     p->depthwise = false;
+    p->opt = chx::read_launch_options();
     if (weights_fit_depthwise(*w, params->group) && w_zero_point->dtype == w->dtype && w_zero_point->ndim <= 1) {
         std::vector<uint8_t> zp;
         int rc = read_back(*w_zero_point, &zp, s);
@@ -1066,14 +1101,14 @@ extern "C" int chx_hip_qconv_plan_run(
     hipStream_t s = as_stream(stream);
     const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
     if (plan->mfma) {
-        ConvCall call = conv_call_from(q, x, y, &plan->params, rne);
+        ConvCall call = conv_call_from(q, x, y, &plan->params, rne, plan->opt);
         call.cache = const_cast<ScratchCache*>(&plan->scratch);
         call.tune = const_cast<TuneCache*>(&plan->tune);
         const int rc = run_conv_mfma(call, plan->pw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
     if (plan->depthwise) {
-        const int rc = run_depthwise(conv_call_from(q, x, y, &plan->params, rne), plan->dw, s);
+        const int rc = run_depthwise(conv_call_from(q, x, y, &plan->params, rne, plan->opt), plan->dw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
     return launch_conv_direct(q.direct, rne, s);
@@ -1140,14 +1175,16 @@ extern "C" int chx_hip_qconv_plan_run_add(
         key.r = nullptr;
         key.r_px_stride = 0;
         key.r_vec_ok = 0;
-        const char* env = getenv("CHX_HIP_AFFINE_RESIDUAL");
-        const bool wanted = !(env && env[0] == '0');
-        if (wanted && mp->res_known && memcmp(&key, &mp->res_key, sizeof(key)) == 0) {
-            res.affine = mp->res_found.affine;
-            res.kc = mp->res_found.kc;
-            res.kr = mp->res_found.kr;
-            res.k0 = mp->res_found.k0;
-            res.floor_pre = mp->res_found.floor_pre;
+        const bool wanted = plan->opt.affine_residual;
+        const ResidualAdd* known = nullptr;
+        for (const chx_hip_qconv_plan::SearchedResidual& e : mp->searched)
+            if (memcmp(&key, &e.key, sizeof(key)) == 0) known = &e.found;
+        if (wanted && known) {
+            res.affine = known->affine;
+            res.kc = known->kc;
+            res.kr = known->kr;
+            res.k0 = known->k0;
+            res.floor_pre = known->floor_pre;
         } else if (wanted && !stream_is_capturing(s)) {
             int32_t* counts = nullptr;
             CHX_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&counts), kAffineCandidates * sizeof(int32_t)));
@@ -1156,9 +1193,10 @@ extern "C" int chx_hip_qconv_plan_run_add(
             const int rc = find_affine_residual(&found, counts, s);
             (void)hipFree(counts);
             CHX_PROPAGATE(rc);
-            memcpy(&mp->res_key, &key, sizeof(key));
-            memcpy(&mp->res_found, &found, sizeof(found));
-            mp->res_known = true;
+            if (mp->searched.size() == chx_hip_qconv_plan::kMaxSearchedResiduals) mp->searched.erase(mp->searched.begin());
+            mp->searched.emplace_back();
+            memcpy(&mp->searched.back().key, &key, sizeof(key));
+            memcpy(&mp->searched.back().found, &found, sizeof(found));
             res.affine = found.affine;
             res.kc = found.kc;
             res.kr = found.kr;
@@ -1166,7 +1204,7 @@ extern "C" int chx_hip_qconv_plan_run_add(
             res.floor_pre = found.floor_pre;
         }
     }
-    ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0);
+    ConvCall call = conv_call_from(q, x, &y, &plan->params, (flags & CHX_HIP_ROUND_ONNX_RNE) != 0, plan->opt);
     call.cache = const_cast<ScratchCache*>(&plan->scratch);
     call.tune = const_cast<TuneCache*>(&plan->tune);
     call.res = &res;
@@ -1182,7 +1220,7 @@ extern "C" int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char*
                  t.tile_oc, t.tile_px, t.max_wgs_per_cu, t.waves);
         text += line;
     }
-    if (plan->res_known) text += plan->res_found.affine ? "residual=affine\n" : "residual=exact\n";
+    if (!plan->searched.empty()) text += plan->searched.back().found.affine ? "residual=affine\n" : "residual=exact\n";
     strncpy(buf, text.c_str(), buf_size - 1);
     buf[buf_size - 1] = 0;
     return CHX_HIP_OK;
@@ -1248,6 +1286,7 @@ extern "C" int chx_hip_conv_integer(
         if (zero) {
             ConvCall c;
             memset(&c, 0, sizeof(c));
+            c.opt = read_launch_options();
             c.x = x;
             c.y = y;
             c.p = params;
@@ -1295,6 +1334,7 @@ int matmul_via_mfma(
     chx_hip_conv_params p = {1, 1, 0, 0, 0, 0, 1};
     ConvCall c;
     memset(&c, 0, sizeof(c));
+    c.opt = read_launch_options();
     c.x = &x4;
     c.y = &y4;
     c.p = &p;

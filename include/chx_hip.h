@@ -221,7 +221,7 @@ int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_
  * constants with which floor(y*kc + (r*kr + k0)), two fused multiply-adds, gives the same byte as that
  * arithmetic on every one of the 65536 pairs of codes, checks each candidate on the device against
  * the arithmetic itself, and uses the short form from then on if one passes (CHX_HIP_AFFINE_RESIDUAL=0
- * in the environment keeps the long one).  r and out: same shape as y, channels-last, uint8 or int8.
+ * in the environment when the plan is created keeps the long one).  r and out: same shape as y, channels-last, uint8 or int8.
  * `out` must not overlap x or r in memory (the first call on a new shape may run the kernel several
  * times on the call's operands to pick a launch configuration): CHX_HIP_EINVAL when it does.
  * CHX_HIP_EUNSUPPORTED when the plan's weights or the layouts do not fit the matrix-core kernel;

@@ -425,6 +425,14 @@ def test_qlinear_conv_with_fused_residual_sum(g, oracle, case, ydt, rdt, odt, fo
         assert forms and forms[-1] in ("residual=affine", "residual=exact")
         if odt == np.int8:
             assert forms[-1] == "residual=exact"
+    # a caller that alternates between sets of parameters gets each one's own arithmetic back (the plan keeps what
+    # it found for several of them): the first set again, after the others
+    want = _residual_sum(oracle, conv, ys, yz, r, rs, rz, False, os_, oz, odt)
+    rd = g.to_channels_last(g.dev(r))
+    for _ in range(2):
+        got = plan.run_add(xd, 0.02, 101, ys, yz, rd, rs, rz, os_, oz, False, zero_point_dtype=TDT[ydt],
+                           flags=g.capi.BIAS_ONNX_INT32, out=torch.zeros_like(rd, dtype=TDT[odt]))
+        np.testing.assert_array_equal(g.host(got), want)
     # operands that are not channels-last are refused, not converted
     with pytest.raises(g.capi.ChxHipError) as e:
         plan.run_add(xd, 0.02, 101, ys, yz, g.dev(r), rs, rz, os_, oz, True, zero_point_dtype=TDT[ydt],
