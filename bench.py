@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget for the CPU baseline")
     ap.add_argument("--no-fuse-residual", action="store_true",
                     help="run the residual Add(+Relu) groups as kernels of their own instead of inside the convolution before them")
+    ap.add_argument("--no-pair-convs", action="store_true",
+                    help="run the two convolutions that read a down-sampling block's input as two launches instead of one")
     ap.add_argument("--parts", type=int, default=1,
                     help="run the batch as this many concurrent slices on separate streams (network workloads)")
     ap.add_argument("--runner", default="chxvm", choices=["chxvm", "python"],
@@ -121,8 +123,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # default is the plain whole-batch runner, whose launches are the ones the roofline figure
     # below prices.
     fuse = not args.no_fuse_residual
+    pair = fuse and not args.no_pair_convs and args.parts <= 1
     # values share memory once their last reader has run, as in the VM (whose allocator reuses freed slots)
-    runner = wl.DeviceRunner(model, pkg, fuse, reuse_buffers=True) if args.parts <= 1 else None
+    runner = wl.DeviceRunner(model, pkg, fuse, reuse_buffers=True, pair_convs=pair) if args.parts <= 1 else None
     timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts, fuse)
 
     def step(_timer):
@@ -136,6 +139,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         # the drop-in itself: the network as one serialized program in the C++ VM
         import importlib
         vm = importlib.import_module(pkg.__name__ + ".chxvm")
+        vm.set_option("pair_convolutions", "on" if pair else "off")
         vm_prog = vm.Program(wl.program_to_chxvm(model, vm, ops, keep=("logits",)).serialize())
         vm_prog.set_option("qlinearconv_bias", "onnx_int32")
         if args.no_graph:
@@ -169,8 +173,8 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         torch.cuda.synchronize()
         vals = dict(rn.bufs, x=xs)   # every value's buffer (with reuse_buffers several share memory, as in the timed step)
         fids = []
-        for fid, ins in enumerate(model["program"]):
-            if ins[0] != "QLinearConv":
+        for fid, ins in enumerate(rn.program):
+            if ins[0] not in ("QLinearConv", "QLinearConvPair"):
                 continue
             if mobilenet and model["convs"][ins[3]].group == 1:
                 continue  # MobileNetV2: the roofline figure is the depthwise kernel's
@@ -223,7 +227,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # operations and bytes (input pixels it needs, weights, output, residual operand; workloads.conv_layer_table);
     # most 1x1 layers of these networks are below the ridge of 625 op/byte and belong to the HBM roof.  For
     # MobileNetV2 the figure covers every QLinearConv launch, not only the depthwise ones timed above.
-    table = wl.conv_layer_table(model, fuse)
+    table = wl.conv_layer_table(model, fuse, pair)
     floor_s = sum(max(r["ops"] / (INT8_PEAK_TOPS * 1e12), r["bytes"] / (HBM_PEAK_GBS * 1e9)) for r in table)
     n_mfma = sum(1 for r in table if r["ops"] / (INT8_PEAK_TOPS * 1e12) >= r["bytes"] / (HBM_PEAK_GBS * 1e9))
     roofline["mixed"] = dict(
@@ -233,7 +237,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         launches_mfma_class=n_mfma, launches_hbm_class=len(table) - n_mfma)
     if not mobilenet:
         roofline["mixed"]["frac"] = floor_s * 1e3 / conv_ms_per_step
-    roofline["launches_per_step"] = len(model["program"]) - (sum(1 for r in table if r["residual"]) if fuse else 0)
+    roofline["launches_per_step"] = len(model["program"]) - (sum(1 for r in table if r["residual"]) if fuse else 0) - (
+        len(wl.conv_layer_table(model, fuse)) - len(table))
+    roofline["paired_convolutions"] = len(wl.conv_layer_table(model, fuse)) - len(table)
     roofline["boundary_us_per_launch"] = boundary_ms_per_step * 1e3 / max(n_launch, 1)
     roofline["kernel_ms_per_step_without_boundaries"] = conv_ms_per_step - boundary_ms_per_step
     roofline["frac_without_boundaries"] = roofline["frac"] * conv_ms_per_step / max(conv_ms_per_step - boundary_ms_per_step, 1e-9)

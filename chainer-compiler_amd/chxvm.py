@@ -494,6 +494,8 @@ def decode_program(data):
 def set_option(name, value):
     """Runtime switches: "qlinearconv_bias" = "reference" (default) | "onnx_int32";
     "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards);
+    "pair_convolutions" = "on" (default) | "off": two QLinearConv of one value with the same geometry as one launch
+    (applies to programs loaded afterwards);
     "chrome_tracing" = file that every later run writes its per-instruction timeline to, "" = off;
     "dump_outputs_dir" = directory that every later run writes the instructions' named array
     outputs to as .npy files, "" = off;

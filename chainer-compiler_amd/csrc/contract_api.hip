@@ -282,6 +282,7 @@ struct TunedConfig {
     int tile_oc, tile_px, max_wgs_per_cu;
     int waves;      // wavefronts per work-group: 4 or 8
     bool with_res;  // measured with a fused residual sum (an entry of its own: the epilogue differs)
+    int32_t oc_split = 0;  // measured as two convolutions in one launch, split here (restricts the tiles)
 };
 struct TuneCache {
     std::vector<TunedConfig> entries;
@@ -299,6 +300,7 @@ int tune_conv_mfma(const ConvMfmaArgs& a, bool xu, bool out_int32, bool rne, hip
     int rc = CHX_HIP_OK;
     for (int t = 0; t < 7 && rc == CHX_HIP_OK; ++t) {
         if (a.OC <= 64 && tiles[t][0] > 64) continue;
+        if (a.oc_split % tiles[t][0] != 0) continue;  // two outputs: a tile belongs to one of them whole
         if (tiles[t][2] == 8 && (tiles[t][0] == 64 || tiles[t][1] == 256) && a.bk != 128) continue;
         for (int c = 0; c < (tiles[t][2] == 8 ? 1 : 3) && rc == CHX_HIP_OK; ++c) {
             const int reps = 3;
@@ -417,6 +419,10 @@ struct ConvCall {
     RequantParams rq;
     const ResidualAdd* res = nullptr;  // a residual sum fused behind the requantization
     LaunchOptions opt;                 // the plan's, or read for this one-shot call
+    // two convolutions of x in one launch (ConvMfmaArgs::oc_split): the second one's output and requantization
+    const chx_hip_tensor* y2 = nullptr;
+    int32_t oc_split = 0;
+    RequantParams rq2;
 };
 
 // Runs the MFMA kernel on packed weights.  x may be channels-last (used in place) or
@@ -531,6 +537,21 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     }
     a.y_vec_ok = aligned(a.y, 16) && (a.y_px_stride % 16 == 0) ? 1 : 0;
     (void)es;
+    if (c.y2) {
+        int64_t y2_px = 0;
+        if (stem || pw.dense || x_scratch || y_post || c.out_int32 || c.res || !y_is_pixel_major(*c.y2, &y2_px)) {
+            release_scratch(c.cache, x_scratch, s);
+            release_scratch(c.cache, y_scratch, s);
+            CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv pair: needs channels-last x, y1 and y2 and at least 16 input channels");
+        }
+        a.oc_split = c.oc_split;
+        a.y2 = static_cast<char*>(c.y2->data);
+        a.y2_px_stride = y2_px;
+        a.y2_vec_ok = aligned(a.y2, 16) && (y2_px % 16 == 0) ? 1 : 0;
+        a.q2 = c.rq2.q;
+        a.inv_y_scale2 = 1.0f / c.rq2.q.scale;
+        a.lo_folded2 = fold_relu_floor(c.rq2.q, c.rq2.relu_floor, c.rne);
+    }
     if (stem) {
         ConvStemArgs sa;
         memset(&sa, 0, sizeof(sa));
@@ -594,13 +615,14 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     CHX_REQUIRE(a.M < (int64_t(1) << 31), "QLinearConv: too many output pixels for the MFMA kernel");
     int toc = 64, tpx = 64, cap = 0, waves = 4;
     pick_tile(c.opt, cs.OC, a.M, a.bk, &toc, &tpx, &cap, &waves);
+    if (a.oc_split % toc != 0) toc = 64, waves = 4, tpx = tpx > 128 ? 128 : tpx;  // (the split is a multiple of 64)
     int rc = CHX_HIP_OK;
     const TunedConfig* tuned = nullptr;
     if (c.tune) {
         for (const TunedConfig& t : c.tune->entries)
-            if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW && t.with_res == (c.res != nullptr)) tuned = &t;
+            if (t.M == a.M && t.H == a.H && t.W == a.W && t.OH == a.OH && t.OW == a.OW && t.with_res == (c.res != nullptr) && t.oc_split == a.oc_split) tuned = &t;
         if (!tuned && c.opt.autotune && !stream_is_capturing(s)) {
-            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, 4, c.res != nullptr};
+            TunedConfig best = {a.M, a.H, a.W, a.OH, a.OW, toc, tpx, 0, waves, c.res != nullptr, a.oc_split};
             rc = tune_conv_mfma(a, xu, c.out_int32, c.rne, s, &best);
             if (rc == CHX_HIP_OK) {
                 c.tune->entries.push_back(best);
@@ -1112,6 +1134,46 @@ extern "C" int chx_hip_qconv_plan_run(
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
     }
     return launch_conv_direct(q.direct, rne, s);
+}
+
+extern "C" int chx_hip_qconv_plan_run_pair(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, int32_t split,
+        float y1_scale, int32_t y1_zero_point, uint32_t flags1, chx_hip_tensor* y1, float y2_scale, int32_t y2_zero_point,
+        uint32_t flags2, chx_hip_tensor* y2, void* stream) {
+    CHX_REQUIRE(plan != nullptr, "QLinearConv pair: null plan");
+    CHX_PROPAGATE(check_tensor(y1, "QLinearConv pair y1"));
+    CHX_PROPAGATE(check_tensor(y2, "QLinearConv pair y2"));
+    CHX_REQUIRE(y1->ndim == 4 && y2->ndim == 4, "QLinearConv pair: y1 and y2 must be 4-D");
+    const int64_t OC = plan->w.shape[0];
+    CHX_REQUIRE(split > 0 && split < OC && y1->shape[1] == split && y2->shape[1] == OC - split,
+                "QLinearConv pair: y1 and y2 must hold the first %d and the other %lld of the plan's %lld output channels", split,
+                (long long)(OC - split), (long long)OC);
+    for (int ax : {0, 2, 3}) CHX_REQUIRE(y1->shape[ax] == y2->shape[ax], "QLinearConv pair: y1 and y2 differ in batch or image size");
+    const uint32_t shared = CHX_HIP_BIAS_ONNX_INT32 | CHX_HIP_ROUND_ONNX_RNE;
+    CHX_REQUIRE((flags1 & shared) == (flags2 & shared), "QLinearConv pair: the two halves must agree on the bias and rounding flags");
+    CHX_PROPAGATE(check_tensor(x, "QLinearConv pair x"));
+    CHX_REQUIRE(!byte_ranges_overlap(*y1, *x) && !byte_ranges_overlap(*y2, *x) && !byte_ranges_overlap(*y1, *y2),
+                "QLinearConv pair: x, y1 and y2 must not overlap in memory");
+    if (split % 64 != 0) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv pair: the first convolution must have a multiple of 64 output channels");
+    if (!plan->mfma) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv pair: these weights do not run on the matrix-core kernel");
+    // shapes and parameters as for one convolution with all output channels, laid out like y1
+    chx_hip_tensor y_all = *y1;
+    y_all.shape[1] = OC;
+    QConvChecked q;
+    CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, &plan->w, &plan->w_scale, &plan->w_zero_point, y1_scale, y1_zero_point,
+                              plan->has_bias ? &plan->bias : nullptr, &plan->params, flags1, &y_all, &q));
+    RequantParams rq2;
+    const int32_t* bias2 = nullptr;
+    CHX_PROPAGATE(fill_requant(x_scale, y2_scale, y2_zero_point, *y2, plan->has_bias ? &plan->bias : nullptr, OC, flags2,
+                               "QLinearConv pair", &rq2, &bias2));
+    hipStream_t s = as_stream(stream);
+    ConvCall call = conv_call_from(q, x, y1, &plan->params, (flags1 & CHX_HIP_ROUND_ONNX_RNE) != 0, plan->opt);
+    call.cache = const_cast<ScratchCache*>(&plan->scratch);
+    call.tune = const_cast<TuneCache*>(&plan->tune);
+    call.y2 = y2;
+    call.oc_split = split;
+    call.rq2 = rq2;
+    return run_conv_mfma(call, plan->pw, s);
 }
 
 extern "C" int chx_hip_qconv_plan_run_add(

@@ -104,6 +104,26 @@ __device__ __forceinline__ void buffer_copy16_run(const uint32_t (&voff)[4], v4i
                      : : "v"(voff[0]), "v"(voff[1]), "v"(voff[2]), "v"(voff[3]), "s"(srd), "s"(soff), "s"(lds_addr) : "memory", "m0");
 }
 
+// The fields of a residual sum that its per-element arithmetic reads.
+__device__ __forceinline__ ResidualAdd in_vector_registers(const ResidualAdd& p) {
+    ResidualAdd v = p;
+    v.c_flip = in_vector_register(p.c_flip);
+    v.r_flip = in_vector_register(p.r_flip);
+    v.c_zpf = in_vector_register(p.c_zpf);
+    v.c_scale = in_vector_register(p.c_scale);
+    v.r_zpf = in_vector_register(p.r_zpf);
+    v.r_scale = in_vector_register(p.r_scale);
+    v.big = in_vector_register(p.big);
+    v.inv_out_scale = in_vector_register(p.inv_out_scale);
+    v.out = in_vector_registers(p.out);
+    v.out.lo = p.out.lo;  // selects the variant (a uniform branch) and bounds the int8 path only
+    v.kc = in_vector_register(p.kc);
+    v.kr = in_vector_register(p.kr);
+    v.k0 = in_vector_register(p.k0);
+    v.floor_pre = in_vector_register(p.floor_pre);
+    return v;
+}
+
 // Sixteen codes of the convolution and sixteen of the residual -> sixteen codes of the sum
 // (see ResidualAdd): the DequantizeLinear, Add, Relu and QuantizeLinear of quant_math.h in the
 // reference's order, one IEEE operation each.

@@ -78,6 +78,17 @@ struct ConvMfmaArgs {
     uint32_t tap_step_col, tap_step_row;  // what the scalar offset into x gains from the last K step of a filter tap to the first of the next: one pixel to the right, or to the first column of the next filter row (launcher)
     int32_t px_linear;           // 1x1, stride 1, no padding over a dense image: input pixel m is at x + m * x_w_stride (launcher)
     ResidualAdd res;             // res.r == nullptr: plain QLinearConv
+    // Two convolutions of the same input in one launch (oc_split > 0): the weights hold both filter sets one after the
+    // other; output channels [0, oc_split) are the first convolution's and go to y with rq.q / inv_y_scale /
+    // lo_folded, channels [oc_split, OC) are the second's and go to y2 (its channel oc - oc_split) with the set below.
+    // oc_split is a multiple of the tile's output channels, so a tile belongs to one of the two whole.
+    int32_t oc_split;
+    char* y2;
+    int64_t y2_px_stride;
+    int32_t y2_vec_ok;
+    QuantParams q2;
+    float inv_y_scale2;
+    float lo_folded2;
 };
 
 // Direct convolution over planar activations with few channels (conv_stem.hip).

@@ -344,6 +344,8 @@ int launch_conv_mfma(ConvMfmaArgs a, int tile_oc, int tile_px, int max_wgs_per_c
     a.tiles_oc = (a.OC + tile_oc - 1) / tile_oc;
     a.tiles_px = (int)((a.M + tile_px - 1) / tile_px);
     if (a.M == 0 || a.OC == 0) return CHX_HIP_OK;
+    if (a.oc_split != 0 && (a.oc_split < 0 || a.oc_split >= a.OC || a.oc_split % tile_oc != 0 || out_int32 || a.res.r))
+        CHX_FAIL(CHX_HIP_EINVAL, "conv_mfma: two outputs split at channel %d do not fit tiles of %d output channels", a.oc_split, tile_oc);
     // 32-bit offsets into x: the bias keeps the offset of a tap in the padding of the first image non-negative
     // (and leaves room for the immediates the copies subtract); a tap that is fetched lies inside x
     const int64_t bias = 4096 + (int64_t)a.ph * a.x_h_stride + (int64_t)a.pw * a.x_w_stride;

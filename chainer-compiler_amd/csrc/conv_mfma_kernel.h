@@ -52,20 +52,21 @@ template <int BYTES>
 __device__ __forceinline__ void warm_kernel_arguments() {
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
     constexpr int LINES = (BYTES + 63) / 64;
-    static_assert(LINES >= 4 && LINES <= 6, "between four and six lines are touched");
+    static_assert(LINES >= 4 && LINES <= 7, "between four and seven lines are touched");
     // offsets of the last lines, clamped into the block so that nothing outside it is read
-    constexpr int L4 = LINES > 4 ? 0x100 : 0xc0, L5 = LINES > 5 ? 0x140 : L4;
-    int t0, t1, t2, t3, t4, t5;
+    constexpr int L4 = LINES > 4 ? 0x100 : 0xc0, L5 = LINES > 5 ? 0x140 : L4, L6 = LINES > 6 ? 0x180 : L5;
+    int t0, t1, t2, t3, t4, t5, t6;
     asm volatile(
-            "s_load_dword %0, %6, 0x0\n\t"
-            "s_load_dword %1, %6, 0x40\n\t"
-            "s_load_dword %2, %6, 0x80\n\t"
-            "s_load_dword %3, %6, 0xc0\n\t"
-            "s_load_dword %4, %6, %7\n\t"
-            "s_load_dword %5, %6, %8\n\t"
+            "s_load_dword %0, %7, 0x0\n\t"
+            "s_load_dword %1, %7, 0x40\n\t"
+            "s_load_dword %2, %7, 0x80\n\t"
+            "s_load_dword %3, %7, 0xc0\n\t"
+            "s_load_dword %4, %7, %8\n\t"
+            "s_load_dword %5, %7, %9\n\t"
+            "s_load_dword %6, %7, %10\n\t"
             "s_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5)
-            : "s"(ka), "n"(L4), "n"(L5)
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6)
+            : "s"(ka), "n"(L4), "n"(L5), "n"(L6)
             : "memory");
 }
 
@@ -433,7 +434,21 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         return slot + pxl * TM + ((((ocl >> 4) ^ (pxl >> 1)) & (OUT_CHUNKS - 1)) << 4) + (ocl & 15);
     };
     auto epilogue = [&](int px_tile, char* lds_out) {
-        const ConvMfmaArgs a = kernel_arguments_again<ConvMfmaArgs>();
+        ConvMfmaArgs a = kernel_arguments_again<ConvMfmaArgs>();
+        if (a.oc_split > 0) {
+            // two convolutions in this launch: the tile is one of the second's (its output and quantization take the
+            // first's place, its channel 0 is this launch's channel oc_split), or the first's channels end at oc_split
+            if (oc0 >= a.oc_split) {
+                a.y = a.y2 - a.oc_split;
+                a.y_px_stride = a.y2_px_stride;
+                a.y_vec_ok = a.y2_vec_ok;
+                a.rq.q = a.q2;
+                a.inv_y_scale = a.inv_y_scale2;
+                a.lo_folded = a.lo_folded2;
+            } else {
+                a.OC = a.oc_split;
+            }
+        }
         const int64_t m0 = (int64_t)px_tile * TN;
         if (kOutInt32) {
 #pragma unroll
@@ -465,6 +480,10 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         // branches are uniform).  kPath 0: any 8-bit type and rounding; 1: uint8 in the reference's
         // rounding through floor_sat_u8x16; 2: the same with a lower bound above 0 (a folded Relu);
         // 3: as 1 with a zero point of 0.
+        // the constants of the per-element arithmetic in vector registers (in_vector_register says why)
+        const QuantParams rq_q = in_vector_registers(a.rq.q);
+        const float inv_y_scale = in_vector_register(a.inv_y_scale);
+        const float lo_folded = in_vector_register(a.lo_folded);
         auto requantize_tile = [&](auto float_bias_tag, auto path_tag) {
             constexpr bool kFloatBias = decltype(float_bias_tag)::value;
             constexpr int kPath = decltype(path_tag)::value;
@@ -488,7 +507,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                             for (int e = 0; e < 4; ++e) {
                                 float v = (float)acc[i][j][g * 4 + e] * sc[e];
                                 if (kFloatBias) v = v + fb[e];  // reference mode: float bias after the scale multiply
-                                code[e] = quantize_value_folded<kRne>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                                code[e] = quantize_value_folded<kRne>(v, rq_q, inv_y_scale, lo_folded);
                             }
                             *reinterpret_cast<uint32_t*>(staged(lds_out, pxl, ocl)) = pack4(code[0], code[1], code[2], code[3]);
                         }
@@ -517,7 +536,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                                     float v = (float)acc[i][j][g * 4 + e] * sc[e];
                                     if (kFloatBias) v = v + fb[e];
                                     pre[(gl * FN + j) * 4 + e] =
-                                            quantize_prefloor_u8<kPath == 2, kPath != 3>(v, a.rq.q, a.inv_y_scale, a.lo_folded);
+                                            quantize_prefloor_u8<kPath == 2, kPath != 3>(v, rq_q, inv_y_scale, lo_folded);
                                 }
                         }
                         uint32_t word[4];
@@ -584,15 +603,17 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         if (tile_inside) {
             auto store_all = [&](auto mode_tag) {
                 constexpr int kMode = decltype(mode_tag)::value;  // 0: no residual, 1 / 2: the two-multiply-add forms, 3: the exact chain
+                ResidualAdd res;
+                if constexpr (kMode != 0) res = in_vector_registers(a.res);
 #pragma unroll
                 for (int it = 0; it < ITER; ++it) {
                     const int q = tid + it * T;
                     const int pxl = q / OUT_CHUNKS;
                     const int ch = q % OUT_CHUNKS;
                     v4i val = *reinterpret_cast<const v4i*>(staged(lds_out, pxl, ch * 16));
-                    if constexpr (kMode == 1) val = affine_residual16<false>(val, rres[it], a.res);
-                    if constexpr (kMode == 2) val = affine_residual16<true>(val, rres[it], a.res);
-                    if constexpr (kMode == 3) val = add_residual16_any(val, rres[it], a.res);
+                    if constexpr (kMode == 1) val = affine_residual16<false>(val, rres[it], res);
+                    if constexpr (kMode == 2) val = affine_residual16<true>(val, rres[it], res);
+                    if constexpr (kMode == 3) val = add_residual16_any(val, rres[it], res);
                     *reinterpret_cast<v4i*>(a.y + (m0 + pxl) * a.y_px_stride + oc0 + ch * 16) = val;
                 }
             };
@@ -661,8 +682,8 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
     constexpr int NM = FM * FN;          // MFMAs per extent
     constexpr int READS = FM + FN;       // fragment reads per extent
     v4i fa[NB][FM], fb[NB][FN];
-    int flip;  // in a scalar register: a literal would make every flip an eight-byte instruction
-    asm volatile("s_mov_b32 %0, 0x80808080" : "=s"(flip));
+    int flip;  // in a vector register: a literal would make every flip an eight-byte instruction, a scalar register a four-cycle one
+    asm volatile("v_mov_b32 %0, 0x80808080" : "=v"(flip));
     auto read_one = [&](auto buf_c, auto sub_c, auto r_c, uint32_t slot_off) {
         constexpr int buf = decltype(buf_c)::value, sub = decltype(sub_c)::value, r = decltype(r_c)::value;
         if constexpr (r < FM) fa[buf][r] = lds_read16_nowait<r * 32 * BK>(wave_a + slot_off + lane_off[sub]);

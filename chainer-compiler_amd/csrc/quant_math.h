@@ -27,6 +27,28 @@ inline QuantParams make_quant_params(float scale, int32_t zero_point, bool int8_
     return q;
 }
 
+// A wave-uniform constant held in a vector register.  Measured on gfx950 with a loop of independent instructions:
+// one wavefront issues a vector instruction every 4.5 cycles whatever it is; two wavefronts of a SIMD run float32
+// multiply / add / fused multiply-add, v_xor, v_mov and compares side by side (0.94 ns per instruction and SIMD)
+// when all operands are vector registers, inline constants or literals, but take turns (1.77 ns) as soon as one
+// operand is a scalar register; conversions, v_perm, v_med3, v_cvt_pk_u8, dot products and float64 always take
+// turns.  So the constants of per-element float arithmetic that several wavefronts of a SIMD execute at once are
+// copied into vector registers, once per tile.  (The convolution epilogue gains 2-3 % on 1x1 layers with few
+// multiply-adds per output from it and nothing elsewhere: one wavefront's own issue rate is the usual limit.)
+// The copy is opaque to the compiler, which would otherwise fold it back.
+__device__ __forceinline__ float in_vector_register(float s) {
+    float v;
+    asm("v_mov_b32 %0, %1" : "=v"(v) : "v"(s));
+    return v;
+}
+__device__ __forceinline__ uint32_t in_vector_register(uint32_t s) {
+    uint32_t v;
+    asm("v_mov_b32 %0, %1" : "=v"(v) : "v"(s));
+    return v;
+}
+__device__ __forceinline__ QuantParams in_vector_registers(const QuantParams& q) {
+    return QuantParams{in_vector_register(q.scale), in_vector_register(q.zpf), in_vector_register(q.lo), in_vector_register(q.hi)};
+}
 // quantize_array, runtime/ops/quantize.cc:29-34:
 //   scaled = v / y_scale; if (zp != 0) scaled += zp;
 //   AsType(Maximum(lo, Minimum(scaled, hi)) + 0.5f)          (AsType truncates)

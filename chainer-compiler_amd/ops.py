@@ -283,6 +283,22 @@ class QLinearConvPlan(object):
             _f(out_scale), _i(out_zero_point), _i(1 if relu else 0), capi.ref(out), capi.stream_ptr()))
         return out
 
+    def run_pair(self, x, x_scale, x_zero_point, split, y1_scale, y1_zero_point, y2_scale, y2_zero_point,
+                 zero_point_dtypes=(torch.uint8, torch.uint8), flags=(0, 0), outs=None):
+        """Two QLinearConv of the same x in one launch (chx_hip_qconv_plan_run_pair): this plan holds both filter sets
+        concatenated along the output channels; the first `split` channels go to the first result with the first
+        quantization, the others to the second.  Raises ChxHipError with code EUNSUPPORTED when the weights or layouts
+        do not fit; run two plans then."""
+        handle, shape = self._plan_for(x)
+        if outs is None:
+            outs = (_alloc_like_input_layout(x, (shape[0], split) + tuple(shape[2:]), zero_point_dtypes[0]),
+                    _alloc_like_input_layout(x, (shape[0], shape[1] - split) + tuple(shape[2:]), zero_point_dtypes[1]))
+        capi.check(capi.lib().chx_hip_qconv_plan_run_pair(
+            handle, capi.ref(x), _f(x_scale), _i(x_zero_point), _i(split), _f(y1_scale), _i(y1_zero_point),
+            ctypes.c_uint32(flags[0]), capi.ref(outs[0]), _f(y2_scale), _i(y2_zero_point), ctypes.c_uint32(flags[1]),
+            capi.ref(outs[1]), capi.stream_ptr()))
+        return outs
+
     def describe(self):
         """The launch configurations measured so far (chx_hip_qconv_plan_describe), one per line."""
         lines = []

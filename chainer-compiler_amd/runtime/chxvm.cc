@@ -1,5 +1,6 @@
 #include "chxvm.h"
 
+#include <algorithm>
 #include <cstring>
 #include <fstream>
 #include <iomanip>
@@ -168,6 +169,7 @@ private:
 // when it does not (other quantization constants at run time, operands the kernel does not take),
 // both instructions run as they are.
 bool g_fuse_residual = true;
+bool g_pair_convolutions = true;
 
 struct ResidualFusionState {
     bool fused = false;  // of the current run
@@ -333,10 +335,70 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
         fused_inputs[q] = std::make_pair(da, db);
         role[m] = role[da] = role[db] = 1;
     }
+    // Two QLinearConv that read the same value with the same activation quantization, strides, pads and kernel size
+    // (the main-path and the shortcut convolution of a down-sampling block): the second moves up to the first and the
+    // two run as one launch (role 6 = the first, now the pair; role 7 = the second, now nothing).  Every operand of the
+    // second must exist where the first stands, or be a literal constant that stands between the two (the compiler
+    // emits a constant in front of its first reader): those constants move up as well (role 7, run in front of the
+    // pair).  The second's result then exists from the first's place on (`position` says where a value is produced
+    // after this move).
+    const int kQLinearConv = OpNumber("QLinearConv");
+    const std::set<int> literal_ops = {OpNumber("FloatScalarConstant"), OpNumber("IntScalarConstant"), OpNumber("FloatConstant"),
+                                       OpNumber("IntConstant")};
+    std::vector<int> position(n);
+    for (int i = 0; i < n; ++i) position[i] = i;
+    std::vector<int> pair_second(n, -1);
+    std::vector<std::vector<int>> pair_constants(n);
+    for (int i = 0; i < n && g_pair_convolutions; ++i) {
+        const ChxVMInstructionProto& ai = program.instructions[i];
+        if (ai.op != kQLinearConv || role[i] != 0 || ai.inputs.size() != 13 || ai.outputs.empty()) continue;
+        for (int j = i + 1; j < n; ++j) {
+            const ChxVMInstructionProto& bi = program.instructions[j];
+            if (bi.op == kFree && bi.inputs.size() == 1 && bi.inputs[0].array == ai.inputs[0].array) break;  // x ends here
+            if (bi.op != kQLinearConv || role[j] != 0 || bi.inputs.size() != 13 || bi.outputs.empty()) continue;
+            if (bi.inputs[0].array != ai.inputs[0].array) continue;
+            bool same = bi.inputs[9].ints == ai.inputs[9].ints && bi.inputs[10].ints == ai.inputs[10].ints &&
+                        bi.inputs[11].i == 1 && ai.inputs[11].i == 1 && bi.inputs[12].s == ai.inputs[12].s;
+            // the second one's operands: produced before the first, or literal constants in between that can move up
+            std::vector<int> moved;
+            auto available = [&](int slot) {
+                if (slot < 0 || producer[slot] < 0) return false;
+                const int pr = producer[slot];
+                if (pr < i) return role[pr] == 0 || position[pr] < i;
+                if (pr > j || role[pr] != 0 || !literal_ops.count(program.instructions[pr].op) || program.instructions[pr].outputs.size() != 1) return false;
+                moved.push_back(pr);
+                return true;
+            };
+            for (int k : {1, 2, 6, 7}) same = same && available(bi.inputs[k].scalar);
+            for (int k : {3, 4, 5}) same = same && available(bi.inputs[k].array);
+            if (bi.inputs[8].array >= 0) same = same && available(bi.inputs[8].array);
+            // nothing between the two may free one of them (the compiler frees a value after its last reader, which
+            // the second convolution is at the latest)
+            for (int f = i; f < j && same; ++f) {
+                const ChxVMInstructionProto& fi = program.instructions[f];
+                if (fi.op != kFree || fi.inputs.size() != 1) continue;
+                for (int k : {3, 4, 5, 8}) same = same && fi.inputs[0].array != bi.inputs[k].array;
+                for (int k : {1, 2, 6, 7}) same = same && fi.inputs[0].array != bi.inputs[k].scalar;
+            }
+            if (!same) continue;
+            role[i] = 6;
+            role[j] = 7;
+            pair_second[i] = j;
+            position[j] = i;
+            std::sort(moved.begin(), moved.end());
+            moved.erase(std::unique(moved.begin(), moved.end()), moved.end());
+            for (int c : moved) {
+                role[c] = 7;
+                position[c] = i;
+            }
+            pair_constants[i] = moved;
+            break;
+        }
+    }
     // Residual sums: an ElementWiseNvrtc group of the form Q(act(DQ(a) + DQ(b))) one of whose operands
     // is the result of a QLinearConv that nobody else reads, with the other operand produced
     // before that convolution.  role 4 = the convolution, role 5 = the group.
-    const int kQLinearConv = OpNumber("QLinearConv"), kElementWise = OpNumber("ElementWiseNvrtc");
+    const int kElementWise = OpNumber("ElementWiseNvrtc");
     std::vector<int> partner(n, -1), conv_operand(n, 0);
     std::vector<chx_hip_residual_group> groups(n);
     for (int e = 0; e < n && g_fuse_residual; ++e) {
@@ -352,7 +414,7 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
             if (slot < 0 || other < 0 || slot == other) continue;
             const int c = producer[slot];
             if (c < 0 || program.instructions[c].op != kQLinearConv || role[c] != 0 || !single_use(slot)) continue;
-            if (producer[other] >= c) continue;  // the other operand must exist when the convolution runs
+            if (producer[other] < 0 || position[producer[other]] >= c) continue;  // the other operand must exist when the convolution runs
             bool other_alive = true;             // ... and still exist: no Free of it before the group
             for (int i = c; i < e; ++i)
                 if (program.instructions[i].op == kFree && program.instructions[i].inputs[0].array == other) other_alive = false;
@@ -401,8 +463,13 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
     for (int i = 0; i < n; ++i) {
         const ChxVMInstructionProto& inst = program.instructions[i];
         const bool frees_dead = inst.op == kFree && inst.inputs.size() == 1 && inst.inputs[0].array >= 0 && dead[inst.inputs[0].array];
-        if (role[i] == 1 || frees_dead || deferred[i]) {
+        if (role[i] == 1 || role[i] == 7 || frees_dead || deferred[i]) {
             program_.emplace_back(new NopOp(inst));
+        } else if (role[i] == 6) {
+            std::vector<std::unique_ptr<ChxVMOp>> seq;
+            for (int c : pair_constants[i]) seq.emplace_back(MakeChxVMOp(program.instructions[c]));
+            seq.emplace_back(MakeQLinearConvPairOp(inst, program.instructions[pair_second[i]]));
+            program_.emplace_back(new SequenceOp(inst, std::move(seq)));
         } else if (role[i] == 3) {
             const ChxVMInstructionProto& pool = program.instructions[fused_inputs[i].second];
             program_.emplace_back(new FusedQuantizedPoolOp(inst, pool, program.instructions[fused_inputs[i].first], pool.op == kMaxPool));
@@ -435,6 +502,10 @@ ChxVM::~ChxVM() = default;
 
 void SetFuseResidual(bool on) {
     g_fuse_residual = on;
+}
+
+void SetPairConvolutions(bool on) {
+    g_pair_convolutions = on;
 }
 
 namespace {

@@ -29,6 +29,15 @@ int64_t QLinearConvResidualFusions();  // requests taken so far, process-wide (a
 // Whether programs loaded from now on pair such convolutions and groups at all (default: yes).
 void SetFuseResidual(bool on);
 
+// Two QLinearConv instructions that read the same value with the same geometry (the main-path and the shortcut
+// convolution of a down-sampling block), run as one launch where the second one's operands allow it
+// (chx_hip_qconv_plan_run_pair) and one after the other otherwise; it stands at the place of the first and writes
+// both results.
+std::unique_ptr<ChxVMOp> MakeQLinearConvPairOp(const ChxVMInstructionProto& first, const ChxVMInstructionProto& second);
+int64_t QLinearConvPairFusions();  // pairs run as one launch so far, process-wide
+// Whether programs loaded from now on pair such convolutions at all (default: yes).
+void SetPairConvolutions(bool on);
+
 class ChxVM {
 public:
     explicit ChxVM(const ChxVMProgramProto& program);

@@ -291,6 +291,9 @@ int32_t chxvm_set_option(const char* name, const char* value) {
         } else if (n == "fuse_residual") {
             CHECK(v == "on" || v == "off") << "fuse_residual is 'on' or 'off', got " << v;
             SetFuseResidual(v == "on");
+        } else if (n == "pair_convolutions") {
+            CHECK(v == "on" || v == "off") << "pair_convolutions is 'on' or 'off', got " << v;
+            SetPairConvolutions(v == "on");
         } else if (n == "chrome_tracing") {
             g_chrome_tracing_path = v;
         } else if (n == "dump_outputs_dir") {
@@ -329,6 +332,7 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name) {
 int64_t chxvm_counter(const char* name) {
     const std::string n = name ? name : "";
     if (n == "qlinearconv_residual_fusions") return QLinearConvResidualFusions();
+    if (n == "qlinearconv_pair_fusions") return QLinearConvPairFusions();
     return -1;
 }
 

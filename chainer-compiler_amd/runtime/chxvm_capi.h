@@ -90,6 +90,9 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
  * name "qlinearconv_bias": value "reference" (unscaled float bias, the default) or "onnx_int32";
  * name "fuse_residual": value "on" (default) or "off": whether a QLinearConv read only by a
  * residual-sum group computes that group inside its kernel (decided when a program is loaded);
+ * name "pair_convolutions": value "on" (default) or "off": whether two QLinearConv that read the same
+ * value with the same strides, pads and kernel size (the main-path and the shortcut convolution of a
+ * down-sampling block) run as one launch (decided when a program is loaded);
  * name "chrome_tracing": value a file name; every later chxvm_program_run writes its
  * per-instruction timeline there in the Chrome tracing format (the device is synchronized after
  * each instruction while this is on), "" switches it off;
@@ -97,7 +100,8 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
  * each instruction there as <5-digit instruction id>_<name>.npy, "" switches it off. */
 int32_t chxvm_set_option(const char* name, const char* value);
 /* Process-wide event counts.  name "qlinearconv_residual_fusions": runs of a QLinearConv that
- * computed the residual-sum group behind it inside its kernel.  Unknown names give -1. */
+ * computed the residual-sum group behind it inside its kernel; "qlinearconv_pair_fusions": pairs of
+ * QLinearConv that ran as one launch.  Unknown names give -1. */
 int64_t chxvm_counter(const char* name);
 
 /* BackendConfig queries.  `config` is a built-in name ("chxvm", "chxvm_test", "hip") or, with

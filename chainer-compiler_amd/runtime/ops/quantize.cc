@@ -6,6 +6,7 @@
 #include "../chxvm.h"
 
 #include <atomic>
+#include <iostream>
 
 namespace chainer_compiler {
 namespace runtime {
@@ -188,6 +189,182 @@ chainerx::Array QLinearConvOp::RunImpl(
             impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
             static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, chainerx::CurrentStream()));
     return y;
+}
+
+namespace {
+
+std::atomic<int64_t> g_pair_fusions{0};
+
+// b appended to a along the first axis, dense
+chainerx::Array ConcatFirstAxis(const chainerx::Array& a, const chainerx::Array& b) {
+    chainerx::Shape shape = a.shape();
+    shape[0] += b.shape()[0];
+    chainerx::Array y = chainerx::Empty(shape, a.dtype());
+    const chainerx::Array* parts[2] = {&a, &b};
+    int64_t at = 0;
+    for (const chainerx::Array* part : parts) {
+        const chainerx::Array span = y.Narrow(0, at, part->shape()[0]);
+        chx_hip_tensor xt = part->hip(), yt = span.hip();
+        CHXVM_HIP_CALL(chx_hip_cast(&xt, &yt, chainerx::CurrentStream()));  // same element type on both sides: a copy
+        at += part->shape()[0];
+    }
+    return y;
+}
+
+// The variable slots and attributes of a QLinearConv instruction (the op class keeps its own private).
+struct QLinearConvSlots {
+    explicit QLinearConvSlots(const ChxVMInstructionProto& inst)
+        : x(inst.inputs[0].array), x_scale(inst.inputs[1].scalar), x_zero_point(inst.inputs[2].scalar), w(inst.inputs[3].array),
+          w_scale(inst.inputs[4].array), w_zero_point(inst.inputs[5].array), y_scale(inst.inputs[6].scalar),
+          y_zero_point(inst.inputs[7].scalar), b(inst.inputs[8].array), strides(inst.inputs[9].ints.begin(), inst.inputs[9].ints.end()),
+          pads(inst.inputs[10].ints.begin(), inst.inputs[10].ints.end()), group(static_cast<int>(inst.inputs[11].i)),
+          auto_pad(inst.inputs[12].s), y(inst.outputs[0]) {
+    }
+    int x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_zero_point, b;
+    chainerx::StackVector<int64_t, chainerx::kMaxNdim> strides, pads;
+    int group;
+    std::string auto_pad;
+    int y;
+};
+
+class QLinearConvPairOp : public ChxVMOp {
+public:
+    QLinearConvPairOp(const ChxVMInstructionProto& first, const ChxVMInstructionProto& second)
+        : ChxVMOp(first), first_(new QLinearConvOp(first)), second_(new QLinearConvOp(second)), a_(new QLinearConvSlots(first)),
+          b_(new QLinearConvSlots(second)) {
+    }
+    ~QLinearConvPairOp() override {
+        chx_hip_qconv_plan_destroy(plan_);
+    }
+    void InitImpl() override {
+        first_->InitImpl();
+        second_->InitImpl();
+    }
+    void Run(ChxVMState* st) override {
+        if (!RunAsOne(st)) {
+            first_->Run(st);
+            second_->Run(st);
+        }
+    }
+
+private:
+    struct Operands {
+        chainerx::Array w, w_scale, w_zero_point;
+        absl::optional<chainerx::Array> bias;
+    };
+    static bool Same(const chainerx::Array& kept, const chainerx::Array& now) {
+        return !kept.IsNullHandle() && kept.raw_data() == now.raw_data() && kept.offset() == now.offset() && kept.shape() == now.shape() &&
+               kept.strides() == now.strides() && kept.dtype() == now.dtype();
+    }
+    static bool Same(const Operands& kept, const Operands& now) {
+        if (!Same(kept.w, now.w) || !Same(kept.w_scale, now.w_scale) || !Same(kept.w_zero_point, now.w_zero_point)) return false;
+        if (kept.bias.has_value() != now.bias.has_value()) return false;
+        return !kept.bias.has_value() || Same(*kept.bias, *now.bias);
+    }
+    static bool Constants(const Operands& o) {
+        return !o.w.IsBorrowed() && !o.w_scale.IsBorrowed() && !o.w_zero_point.IsBorrowed() && !(o.bias.has_value() && o.bias->IsBorrowed());
+    }
+    static Operands Fetch(ChxVMState* st, const QLinearConvSlots& op) {
+        return Operands{st->GetArray(op.w), st->GetArray(op.w_scale), st->GetArray(op.w_zero_point), st->GetOptionalArray(op.b)};
+    }
+
+    // false: the two instructions have to run on their own (nothing has been written)
+    bool RunAsOne(ChxVMState* st) {
+        for (const QLinearConvSlots* op : {a_.get(), b_.get()})
+            for (int slot : {op->x, op->w, op->w_scale, op->w_zero_point})
+                if (slot < 0 || st->GetVar(slot)->IsNull()) return false;
+        const chainerx::Array x = st->GetArray(a_->x);
+        const Operands oa = Fetch(st, *a_), ob = Fetch(st, *b_);
+        const StrictScalar x_scale = st->GetScalar(a_->x_scale), x_zero_point = st->GetScalar(a_->x_zero_point);
+        const StrictScalar y1_scale = st->GetScalar(a_->y_scale), y1_zero_point = st->GetScalar(a_->y_zero_point);
+        const StrictScalar y2_scale = st->GetScalar(b_->y_scale), y2_zero_point = st->GetScalar(b_->y_zero_point);
+        // the same activation quantization on both (they read the same value: anything else would be a program that
+        // interprets one tensor in two ways), per-channel weight scales, weights that are constants of the program
+        if (static_cast<float>(x_scale) != static_cast<float>(st->GetScalar(b_->x_scale)) ||
+            static_cast<int64_t>(x_zero_point) != static_cast<int64_t>(st->GetScalar(b_->x_zero_point)))
+            return false;
+        if (x.ndim() != 4 || oa.w.ndim() != 4 || ob.w.ndim() != 4 || oa.w.dtype() != ob.w.dtype() || !Constants(oa) || !Constants(ob)) return false;
+        for (int d = 1; d < 4; ++d)
+            if (oa.w.shape()[d] != ob.w.shape()[d]) return false;
+        const int64_t oc1 = oa.w.shape()[0], oc2 = ob.w.shape()[0];
+        auto per_channel = [](const Operands& o, int64_t oc) {
+            return o.w_scale.ndim() == 1 && o.w_scale.shape()[0] == oc && o.w_zero_point.ndim() == 1 && o.w_zero_point.shape()[0] == oc &&
+                   (!o.bias.has_value() || (o.bias->ndim() == 1 && o.bias->shape()[0] == oc));
+        };
+        if (oc1 % 64 != 0 || !per_channel(oa, oc1) || !per_channel(ob, oc2) || oa.bias.has_value() != ob.bias.has_value()) return false;
+        if (oa.w_zero_point.dtype() != ob.w_zero_point.dtype() || oa.w_scale.dtype() != ob.w_scale.dtype()) return false;
+        const bool is_q8 = (y1_zero_point.dtype() == chainerx::Dtype::kUInt8 || y1_zero_point.dtype() == chainerx::Dtype::kInt8) &&
+                           (y2_zero_point.dtype() == chainerx::Dtype::kUInt8 || y2_zero_point.dtype() == chainerx::Dtype::kInt8);
+        if (!is_q8) return false;
+        const chx_hip_conv_params p = MakeConvParams(x, oa.w, a_->strides, a_->pads, a_->group, a_->auto_pad);
+        const chx_hip_conv_params p2 = MakeConvParams(x, ob.w, b_->strides, b_->pads, b_->group, b_->auto_pad);
+        if (memcmp(&p, &p2, sizeof(p)) != 0 || p.group != 1) return false;
+        if (plan_ && !(Same(kept_a_, oa) && Same(kept_b_, ob) && memcmp(&p, &params_, sizeof(p)) == 0)) {
+            chx_hip_qconv_plan_destroy(plan_);
+            plan_ = nullptr;
+        }
+        if (!plan_) {
+            if (failed_ && Same(kept_a_, oa) && Same(kept_b_, ob)) return false;  // these operands were refused before
+            w_ = ConcatFirstAxis(oa.w, ob.w);
+            w_scale_ = ConcatFirstAxis(oa.w_scale, ob.w_scale);
+            w_zero_point_ = ConcatFirstAxis(oa.w_zero_point, ob.w_zero_point);
+            bias_ = oa.bias.has_value() ? ConcatFirstAxis(*oa.bias, *ob.bias) : chainerx::Array();
+            chx_hip_tensor wt = w_.hip(), st2 = w_scale_.hip(), zt = w_zero_point_.hip(), bt;
+            if (oa.bias.has_value()) bt = bias_.hip();
+            CHXVM_HIP_CALL(chx_hip_qconv_plan_create(&wt, &st2, &zt, oa.bias.has_value() ? &bt : nullptr, &p, nullptr, &plan_));
+            params_ = p;
+            kept_a_ = oa;
+            kept_b_ = ob;
+            failed_ = false;
+        }
+        const uint32_t flags =
+                CHX_HIP_ROUND_REFERENCE | (st->options().qlinearconv_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
+        chainerx::Shape y1_shape = ConvOutputShape(x, oa.w, p), y2_shape = ConvOutputShape(x, ob.w, p);
+        chainerx::Array y1 = chainerx::EmptyChannelsLastPadded(y1_shape, y1_zero_point.dtype());
+        chainerx::Array y2 = chainerx::EmptyChannelsLastPadded(y2_shape, y2_zero_point.dtype());
+        chx_hip_tensor xt = x.hip(), y1t = y1.hip(), y2t = y2.hip();
+        const int rc = chx_hip_qconv_plan_run_pair(
+                plan_, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), static_cast<int32_t>(oc1),
+                static_cast<float>(y1_scale), static_cast<int32_t>(static_cast<int64_t>(y1_zero_point)), flags, &y1t,
+                static_cast<float>(y2_scale), static_cast<int32_t>(static_cast<int64_t>(y2_zero_point)), flags, &y2t, chainerx::CurrentStream());
+        if (rc == CHX_HIP_EUNSUPPORTED) {
+            // layouts or weights the one-launch kernel does not take: remembered, so that the weights are not joined again
+            chx_hip_qconv_plan_destroy(plan_);
+            plan_ = nullptr;
+            failed_ = true;
+            return false;
+        }
+        CHECK_EQ(CHX_HIP_OK, rc) << chx_hip_last_error();
+        if (std::vector<chx_hip_qconv_plan*>* pinned = st->options().pinned_plans) {
+            // this run is being recorded: the recording holds addresses inside the plan
+            CHXVM_HIP_CALL(chx_hip_qconv_plan_pin(plan_, 1));
+            pinned->push_back(plan_);
+        }
+        if (st->trace_level())
+            std::cerr << "$" << a_->y << ", $" << b_->y << " = QLinearConv x 2 in one launch($" << a_->x << ")" << std::endl;
+        st->SetArray(a_->y, y1);
+        st->SetArray(b_->y, y2);
+        ++g_pair_fusions;
+        return true;
+    }
+
+    std::unique_ptr<QLinearConvOp> first_, second_;  // the instructions as they are, for operands the one launch does not take
+    std::unique_ptr<QLinearConvSlots> a_, b_;
+    chx_hip_qconv_plan* plan_ = nullptr;
+    chx_hip_conv_params params_;
+    Operands kept_a_, kept_b_;               // what the plan was built from
+    chainerx::Array w_, w_scale_, w_zero_point_, bias_;  // the joined operands the plan points into
+    bool failed_ = false;
+};
+
+}  // namespace
+
+std::unique_ptr<ChxVMOp> MakeQLinearConvPairOp(const ChxVMInstructionProto& first, const ChxVMInstructionProto& second) {
+    return std::unique_ptr<ChxVMOp>(new QLinearConvPairOp(first, second));
+}
+
+int64_t QLinearConvPairFusions() {
+    return g_pair_fusions.load();
 }
 
 chainerx::Array MatMulIntegerOp::RunImpl(

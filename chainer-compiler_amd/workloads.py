@@ -276,20 +276,51 @@ def add_relu_program(ops, qa, qb, qy):
         [("q", u8)])
 
 
+def pair_convolutions(program, convs):
+    """The program with every two QLinearConv that read the same value with the same geometry (the main-path and the
+    shortcut convolution of a down-sampling block) replaced by one instruction
+    ("QLinearConvPair", out1, x, conv1, out2, conv2) at the place of the first: one launch computes both
+    (chx_hip_qconv_plan_run_pair).  The first one's output channels must be a multiple of 64."""
+    out, taken = [], set()
+    for i, ins in enumerate(program):
+        if i in taken:
+            continue
+        if ins[0] == "QLinearConv":
+            a = convs[ins[3]]
+            for j in range(i + 1, len(program)):
+                other = program[j]
+                if other[0] != "QLinearConv" or other[2] != ins[2] or j in taken:
+                    continue
+                b = convs[other[3]]
+                same = (a.stride, a.pad, a.group, a.wq.shape[1:]) == (b.stride, b.pad, 1, b.wq.shape[1:])
+                if same and a.wq.shape[0] % 64 == 0 and a.wq.shape[1] >= 16:
+                    out.append(("QLinearConvPair", ins[1], ins[2], ins[3], other[1], other[3]))
+                    taken.add(j)
+                    break
+            else:
+                out.append(ins)
+            continue
+        out.append(ins)
+    return out
+
+
 class DeviceRunner(object):
     """Runs a program on the MI355X: weights resident, one plan per QLinearConv, every
     activation channels-last, all intermediate buffers allocated once."""
 
-    def __init__(self, model, pkg, fuse_residual=False, reuse_buffers=False):
+    def __init__(self, model, pkg, fuse_residual=False, reuse_buffers=False, pair_convs=False):
         """fuse_residual: a QLinearConv whose only reader is the residual Add(+Relu) of its block runs
         as one kernel with it; the convolution's own output is then not materialised.
         reuse_buffers: a value's memory goes back to a pool after its last reader and is handed to later
         values (as the VM's allocator does when the program frees a slot): the working set of a step is
         then a few tensors instead of every tensor of the network, and run() returns only values that are
-        still live at the end (the program's last result is)."""
+        still live at the end (the program's last result is).
+        pair_convs: two convolutions of the same value with the same geometry run as one launch (pair_convolutions);
+        self.program is the instruction list the runner executes."""
         self.m, self.ops, self.capi = model, pkg.ops, pkg.capi
         self.fused_into = {}   # conv output name -> the Add instruction that absorbs it
-        program = model["program"]
+        program = pair_convolutions(model["program"], model["convs"]) if pair_convs else model["program"]
+        self.program = program
         if fuse_residual:
             for i, ins in enumerate(program):
                 if ins[0] in ("AddRelu", "Add") and i > 0:
@@ -308,6 +339,14 @@ class DeviceRunner(object):
             self.dev[name] = t
             self.plans[name] = self.ops.QLinearConvPlan(t[0], t[1], t[2], t[3], strides=(c.stride, c.stride),
                                                         pads=(c.pad, c.pad), group=c.group)
+        for ins in program:
+            if ins[0] == "QLinearConvPair":
+                # both filter sets one after the other along the output channels
+                t = [torch.cat([a, b]) for a, b in zip(self.dev[ins[3]], self.dev[ins[5]])]
+                c = model["convs"][ins[3]]
+                self.dev[ins[3] + "+" + ins[5]] = t
+                self.plans[ins[3] + "+" + ins[5]] = self.ops.QLinearConvPlan(t[0], t[1], t[2], t[3], strides=(c.stride, c.stride),
+                                                                          pads=(c.pad, c.pad), group=1)
         # raw byte blocks: fresh per value, or from the pool of released ones (the smallest that fits)
         free_blocks = []
 
@@ -354,6 +393,8 @@ class DeviceRunner(object):
                 make(add[1], add[0])     # the fused convolution writes the sum here, one instruction early
             elif out not in self.bufs:
                 make(out, kind)
+            if kind == "QLinearConvPair":
+                make(ins[4], kind)
             q = model["qparams"]
             if kind == "AddRelu":
                 self.fusion[out] = add_relu_program(self.ops, q[ins[2]], q[ins[3]], q[out])
@@ -368,7 +409,7 @@ class DeviceRunner(object):
     def launch(self, fid, v):
         """Launches instruction number `fid` of the program on the values `v` (name -> tensor)."""
         ops, q, m = self.ops, self.m["qparams"], self.m
-        ins = m["program"][fid]
+        ins = self.program[fid]
         kind, out = ins[0], ins[1]
         buf = self.bufs.get(out)   # none for a convolution whose result only exists inside the fused residual sum
         if kind == "QuantizeLinear":
@@ -389,6 +430,12 @@ class DeviceRunner(object):
             c = m["convs"][ins[3]]
             self.plans[ins[3]].run(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
                                    flags=self.capi.BIAS_ONNX_INT32, out=buf)
+        elif kind == "QLinearConvPair":
+            c1, c2 = m["convs"][ins[3]], m["convs"][ins[5]]
+            self.plans[ins[3] + "+" + ins[5]].run_pair(
+                v[ins[2]], c1.x_scale, c1.x_zp, c1.wq.shape[0], c1.y_scale, c1.y_zp, c2.y_scale, c2.y_zp,
+                flags=(self.capi.BIAS_ONNX_INT32, self.capi.BIAS_ONNX_INT32), outs=(buf, self.bufs[ins[4]]))
+            v[ins[4]] = self.bufs[ins[4]]
         elif kind == "MaxPool":
             ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)
         elif kind in ("AddRelu", "Add"):
@@ -404,7 +451,7 @@ class DeviceRunner(object):
 
     def run(self, x):
         v = {"x": x}
-        for fid, ins in enumerate(self.m["program"]):
+        for fid, ins in enumerate(self.program):
             buf = self.launch(fid, v)
             if buf is not None:
                 v[ins[1]] = buf
@@ -609,16 +656,18 @@ class ConcurrentRunner(object):
             r.close()
 
 
-def conv_layer_table(model, fuse_residual=True):
+def conv_layer_table(model, fuse_residual=True, pair_convs=False):
     """One row per QLinearConv launch of the program, in program order: the algorithmic work that prices it against
     the two roofs.  ops = 2 * MACs.  bytes = what the launch must move at least: the input pixels it needs (a 1x1
     convolution with stride s reads every s-th pixel of every s-th row only), the weights, the output, and with
-    `fuse_residual` the residual operand of the Add(+Relu) group behind it (whose sum is then the output).  All tensors
+    `fuse_residual` the residual operand of the Add(+Relu) group behind it (whose sum is then the output).  With
+    `pair_convs` two convolutions of one value are one launch (pair_convolutions): the input counts once.  All tensors
     are 8-bit.  A launch belongs to the roof that takes longer at the published peaks."""
-    prog, convs, shapes = model["program"], model["convs"], model["shapes"]
+    convs, shapes = model["convs"], model["shapes"]
+    prog = pair_convolutions(model["program"], convs) if pair_convs else model["program"]
     rows = []
     for i, ins in enumerate(prog):
-        if ins[0] != "QLinearConv":
+        if ins[0] not in ("QLinearConv", "QLinearConvPair"):
             continue
         c = convs[ins[3]]
         n, cin, h, w = shapes[ins[2]]
@@ -626,14 +675,23 @@ def conv_layer_table(model, fuse_residual=True):
         k = c.wq.shape[2]
         x_bytes = n * cin * (oh * ow if k == 1 else h * w)
         nbytes = x_bytes + c.wq.size + n * oc * oh * ow
+        ops = 2.0 * c.macs(shapes[ins[1]])
+        name = c.name
+        if ins[0] == "QLinearConvPair":
+            c2 = convs[ins[5]]
+            oc2 = shapes[ins[4]][1]
+            nbytes += c2.wq.size + n * oc2 * oh * ow
+            ops += 2.0 * c2.macs(shapes[ins[4]])
+            oc += oc2
+            name += "+" + c2.name
         residual = False
-        if fuse_residual and i + 1 < len(prog) and prog[i + 1][0] in ("AddRelu", "Add") and ins[1] in prog[i + 1][2:4]:
+        if ins[0] == "QLinearConv" and fuse_residual and i + 1 < len(prog) and prog[i + 1][0] in ("AddRelu", "Add") and ins[1] in prog[i + 1][2:4]:
             # the group is computed in this launch when the convolution result has no other reader
             readers = [j for j in prog if ins[1] in j[2:]]
             if len(readers) == 1:
                 residual = True
                 nbytes += n * oc * oh * ow
-        rows.append(dict(name=c.name, cin=cin, cout=oc, k=k, stride=c.stride, group=c.group, out_hw=oh, ops=2.0 * c.macs(shapes[ins[1]]),
+        rows.append(dict(name=name, cin=cin, cout=oc, k=k, stride=c.stride, group=c.group, out_hw=oh, ops=ops,
                          bytes=float(nbytes), residual=residual))
     return rows
 

@@ -211,6 +211,19 @@ int chx_hip_qconv_plan_run(
  * does not run on the matrix-core kernel or has not run eagerly yet.  No counterpart in the reference; benchmarks
  * report it next to their timings. */
 int chx_hip_qconv_plan_describe(const chx_hip_qconv_plan* plan, char* buf, size_t buf_size);
+/* Two QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94, twice) that read the same x with the same
+ * activation quantization, kernel size, strides and pads, as ONE launch: the main-path and the shortcut convolution
+ * of a down-sampling residual block.  The plan is created from both filter sets concatenated along the output
+ * channels (w [OC1 + OC2, C, KH, KW]; w_scale, w_zero_point and bias likewise); output channels [0, split) are
+ * requantized with (y1_scale, y1_zero_point, flags1) into y1 [N, split, OH, OW], the others with the second set into
+ * y2 [N, OC - split, OH, OW].  The bytes are those of the two ops run one after the other; x is read once and one
+ * kernel boundary disappears.  flags1 and flags2 may differ in CHX_HIP_FUSE_RELU only.  x, y1 and y2 must not
+ * overlap (CHX_HIP_EINVAL).  CHX_HIP_EUNSUPPORTED when split is not a multiple of 64, when the weights do not run on
+ * the matrix-core kernel or an operand is not channels-last: the caller then runs two plans. */
+int chx_hip_qconv_plan_run_pair(
+        const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, int32_t split,
+        float y1_scale, int32_t y1_zero_point, uint32_t flags1, chx_hip_tensor* y1, float y2_scale, int32_t y2_zero_point,
+        uint32_t flags2, chx_hip_tensor* y2, void* stream);
 /* A QLinearConv (QLinearConvOp::RunImpl, runtime/ops/quantize.cc:62-94) whose only reader is the
  * element-wise group  QuantizeLinear(act(DequantizeLinear(y) + DequantizeLinear(r)))  of a
  * residual block (ElementWiseNvrtcOp::RunImpl, runtime/ops/nvrtc.cc:90-161, act = Relu or

@@ -202,9 +202,10 @@ def test_errors_name_the_instruction(g, vm):
         vm.Program(b.serialize()).run({"x": g.dev(np.zeros(4, np.float32))})
 
 
-def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None):
+def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None, paired=None):
     wl = g.pkg.workloads
     before = vm.counter("qlinearconv_residual_fusions")
+    pairs_before = vm.counter("qlinearconv_pair_fusions")
     serialized = wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize()
     assert vm.proto_roundtrip(serialized) == serialized
     vm.set_option("qlinearconv_bias", "onnx_int32")
@@ -224,6 +225,8 @@ def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None):
         np.testing.assert_array_equal(got[name], ref[name], err_msg="value %s" % name)
     if fused_residuals is not None:
         assert vm.counter("qlinearconv_residual_fusions") - before == fused_residuals
+    if paired is not None:
+        assert vm.counter("qlinearconv_pair_fusions") - pairs_before == paired
 
 
 def test_small_resnet_as_one_program(g, vm, oracle):
@@ -231,20 +234,27 @@ def test_small_resnet_as_one_program(g, vm, oracle):
     operands, DequantizeLinear -> MaxPool / AveragePool -> QuantizeLinear fused at load,
     FusionGroups for the residual sums, Free after the last reader.  Every value, then only the logits."""
     model = g.pkg.workloads.build_resnet50(batch=2, image=64, seed=5, width=16, blocks=(2, 1, 1, 1), classes=10)
+    # The two convolutions that read a down-sampling block's input run as one launch where the first has a multiple of
+    # 64 output channels (the blocks with 64 and 128 channels here; the other two pairs run one after the other).
+    wl = g.pkg.workloads
+    pairs = sum(1 for ins in wl.pair_convolutions(model["program"], model["convs"]) if ins[0] == "QLinearConvPair")
+    assert pairs == 2
     # every value is a program output: nothing may be absorbed into another instruction
-    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0)
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0, paired=pairs)
     # only the logits: each of the five residual sums is computed by the convolution before it
     blocks = sum(1 for ins in model["program"] if ins[0] == "AddRelu")
     assert blocks == 5
-    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks)
+    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks, paired=pairs)
     # the block outputs too: the sums are still absorbed (their convolutions' results are not outputs)
     keep = ["logits"] + [ins[1] for ins in model["program"] if ins[0] == "AddRelu"]
-    _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=blocks)
+    _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=blocks, paired=pairs)
     vm.set_option("fuse_residual", "off")
+    vm.set_option("pair_convolutions", "off")
     try:
-        _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=0)
+        _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=0, paired=0)
     finally:
         vm.set_option("fuse_residual", "on")
+        vm.set_option("pair_convolutions", "on")
 
 
 def test_small_mobilenetv2_as_one_program(g, vm, oracle):

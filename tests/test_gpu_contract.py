@@ -538,6 +538,65 @@ def test_every_launch_configuration_of_the_matrix_core_kernel(g, oracle, tile):
             os.environ["CHX_HIP_TILE"] = before
 
 
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, OC1, OC2, K, stride, pad
+    (2, 256, 14, 14, 128, 512, 1, 2, 0),    # a down-sampling block: main path and shortcut, stride 2
+    (3, 64, 9, 11, 64, 256, 1, 1, 0),       # the first block: 64-channel tiles only, a 64-byte K step
+    (1, 128, 7, 6, 192, 72, 3, 1, 1),       # padded taps, a ragged second half, a split that only 64-channel tiles divide
+    (16, 64, 40, 41, 128, 128, 1, 1, 0)])   # more pixel tiles than resident work-groups
+def test_two_convolutions_of_one_input_in_one_launch(g, oracle, case):
+    """chx_hip_qconv_plan_run_pair against the two QLinearConv on the CPU oracle, each with its own output quantization
+    (and one of them with a fused Relu): the tuner's choice and every launch configuration whose tile divides the split."""
+    import os
+    N, C, H, W, OC1, OC2, K, stride, pad = case
+    rng = np.random.default_rng(97)
+    x = rand_q(rng, (N, C, H, W), np.uint8)
+    w = rng.integers(-127, 128, size=(OC1 + OC2, C, K, K)).astype(np.int8)
+    ws = rng.uniform(0.002, 0.02, size=OC1 + OC2).astype(np.float32)
+    wz = np.zeros(OC1 + OC2, np.int8)
+    bias = rng.integers(-500, 501, size=OC1 + OC2).astype(np.int32)
+    ys1 = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C * K * K) / 40)
+    ys2 = np.float32(ys1 * 1.7)
+    kw = dict(strides=(stride, stride), pads=(pad, pad))
+    want1 = oracle.qlinear_conv_int(x, 0.02, 101, w[:OC1], ws[:OC1], wz[:OC1], ys1, 0, np.uint8, bias=bias[:OC1],
+                                    bias_mode=oracle.BIAS_ONNX_INT32, **kw)
+    want2 = oracle.qlinear_conv_int(x, 0.02, 101, w[OC1:], ws[OC1:], wz[OC1:], ys2, -9, np.int8, bias=bias[OC1:],
+                                    bias_mode=oracle.BIAS_ONNX_INT32, **kw)
+    assert want1.min() < want1.max() and want2.min() < want2.max()
+    xd = g.to_channels_last(g.dev(x))
+    flags = (g.capi.BIAS_ONNX_INT32 | g.capi.FUSE_RELU, g.capi.BIAS_ONNX_INT32)
+    before = os.environ.get("CHX_HIP_TILE")
+    try:
+        for tile in (None, "128,128,0,4", "64,128,0,4", "128,64,2,4", "64,64,1,4", "128,128,0,8", "128,256,0,8", "64,128,0,8"):
+            if tile is None:
+                os.environ.pop("CHX_HIP_TILE", None)
+            else:
+                os.environ["CHX_HIP_TILE"] = tile       # a tile that does not divide the split falls back to 64 channels
+            plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), **kw)
+            for _ in range(2):
+                got1, got2 = plan.run_pair(xd, 0.02, 101, OC1, ys1, 0, ys2, -9, zero_point_dtypes=(torch.uint8, torch.int8), flags=flags)
+                np.testing.assert_array_equal(g.host(got1), want1, err_msg="tile %s first" % tile)
+                np.testing.assert_array_equal(g.host(got2), want2, err_msg="tile %s second" % tile)
+            plan.close()
+    finally:
+        if before is None:
+            os.environ.pop("CHX_HIP_TILE", None)
+        else:
+            os.environ["CHX_HIP_TILE"] = before
+    # what the entry point refuses
+    plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), **kw)
+    with pytest.raises(g.capi.ChxHipError) as e:
+        plan.run_pair(xd, 0.02, 101, OC1 - 32, ys1, 0, ys2, -9, zero_point_dtypes=(torch.uint8, torch.int8), flags=flags)          # not a multiple of 64
+    assert e.value.code == g.capi.EUNSUPPORTED
+    with pytest.raises(g.capi.ChxHipError) as e:
+        plan.run_pair(xd, 0.02, 101, OC1, ys1, 0, ys2, -9, zero_point_dtypes=(torch.uint8, torch.int8), flags=(g.capi.BIAS_ONNX_INT32, 0))    # the halves differ in the bias mode
+    assert e.value.code == g.capi.EINVAL
+    with pytest.raises(g.capi.ChxHipError) as e:
+        plan.run_pair(g.dev(x), 0.02, 101, OC1, ys1, 0, ys2, -9, zero_point_dtypes=(torch.uint8, torch.int8), flags=flags)          # NCHW operands are not converted
+    assert e.value.code == g.capi.EUNSUPPORTED
+    plan.close()
+
+
 def test_random_convolution_sweep(g, oracle):
     """Seeded random QLinearConv / ConvInteger configurations across every dispatch path (matrix-core
     tiles, first-layer kernel, depthwise kernel, generic kernel): shapes, kernel sizes, strides, pads,

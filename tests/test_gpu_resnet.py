@@ -22,20 +22,24 @@ def check_model(g, oracle, model, threads=16):
         ref = wl.run_reference(model, oracle, model["input"])
     finally:
         oracle.set_threads(1)
-    # every op a kernel of its own, then with the residual sums inside the convolutions before them
-    # (those convolutions' own outputs are then not materialised)
-    for fuse in (False, True):
-        runner = wl.DeviceRunner(model, g.pkg, fuse_residual=fuse)
+    # every op a kernel of its own; then with the residual sums inside the convolutions before them (those
+    # convolutions' own outputs are then not materialised); then also with the two convolutions that read a
+    # down-sampling block's input as one launch
+    paired = 0
+    for fuse, pair in ((False, False), (True, False), (True, True)):
+        runner = wl.DeviceRunner(model, g.pkg, fuse_residual=fuse, pair_convs=pair)
         dev = runner.run(torch.from_numpy(model["input"]).cuda())
         torch.cuda.synchronize()
         assert bool(runner.fused_into) == (fuse and any(i[0] in ("Add", "AddRelu") for i in model["program"]))
+        paired = sum(1 for i in runner.program if i[0] == "QLinearConvPair")
+        assert (paired > 0) == (pair and len(runner.program) < len(model["program"]))
         for ins in model["program"]:
             name = ins[1]
             if name in runner.fused_into:
                 assert name not in dev
                 continue
             got = dev[name].cpu().numpy()
-            np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s (fused residual: %s)" % (name, ins[0], fuse))
+            np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s (fused residual: %s, paired: %s)" % (name, ins[0], fuse, pair))
         runner.close()
     return ref
 
