@@ -26,6 +26,11 @@ struct DepthwiseArgs {
     float inv_y_scale;
     float lo_folded;
     int32_t oh_blocks;      // filled by the launcher
+    // The launch is one-dimensional: work-group b of the device's dispatch order (which deals work-groups out to the 8
+    // XCDs in turn) takes block (b % 8) * xcd_chunk + b / 8 of the (x blocks of a row strip, row strips, images) order, so
+    // that each XCD works through a contiguous run of blocks and the input lines that neighbouring blocks share (the
+    // filter's three columns, the halo rows of a strip) are found in that XCD's own L2.  Filled by the launcher.
+    uint32_t grid_x, grid_xy, blocks, xcd_chunk;
     int64_t total;          // filled by the launcher
 };
 

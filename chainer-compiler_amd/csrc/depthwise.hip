@@ -67,14 +67,19 @@ template <bool kRne, bool kFloatBias, int kStep, int kPath, int kStrip>
 __global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs a) {
     constexpr int kRows = rows_per_thread(kStep, kStrip);
     constexpr int kInRows = kStep == 1 ? kRows + 2 : kStep == 2 ? 2 * kRows + 1 : 3;
-    // grid: x over (output column, channel group) of one strip of output rows, y the strip, z the image
-    const uint32_t idx = blockIdx.x * kDwThreads + threadIdx.x;
+    // blocks: x over (output column, channel group) of one strip of output rows, then the strips, then the images;
+    // which block this work-group takes: see DepthwiseArgs
+    const uint32_t block = (blockIdx.x & 7u) * a.xcd_chunk + (blockIdx.x >> 3);
+    if (block >= a.blocks) return;
+    const uint32_t bz = block / a.grid_xy, bxy = block - bz * a.grid_xy;
+    const uint32_t by = bxy / a.grid_x, bx = bxy - by * a.grid_x;
+    const uint32_t idx = bx * kDwThreads + threadIdx.x;
     const uint32_t cgs = (uint32_t)a.C >> 2;
     if (idx >= (uint32_t)a.OW * cgs) return;
     const int ow = (int)(idx / cgs);
     const int cg = (int)(idx - (uint32_t)ow * cgs);
-    const int ohb = blockIdx.y;
-    const int n = blockIdx.z;
+    const int ohb = (int)by;
+    const int n = (int)bz;
     const int c0 = cg * 4;
 
     v4i wq[3];
@@ -220,7 +225,14 @@ int launch_depthwise3x3(DepthwiseArgs a, bool rne, hipStream_t s) {
     if (a.total == 0) return CHX_HIP_OK;
     if (a.oh_blocks > 65535 || a.N > 65535 || (int64_t)a.OW * (a.C / 4) >= (int64_t(1) << 31))
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: more than 65535 images or row strips, or a row of 2^31 channel groups");
-    const dim3 blocks((unsigned)(((int64_t)a.OW * (a.C / 4) + kDwThreads - 1) / kDwThreads), (unsigned)a.oh_blocks, (unsigned)a.N);
+    const int64_t grid_x = ((int64_t)a.OW * (a.C / 4) + kDwThreads - 1) / kDwThreads;
+    const int64_t all_blocks = grid_x * a.oh_blocks * a.N;
+    if (all_blocks >= (int64_t(1) << 31) - 8) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "depthwise kernel: 2^31 work-groups or more");
+    a.grid_x = (uint32_t)grid_x;
+    a.grid_xy = (uint32_t)(grid_x * a.oh_blocks);
+    a.blocks = (uint32_t)all_blocks;
+    a.xcd_chunk = (uint32_t)((all_blocks + 7) / 8);
+    const dim3 blocks(a.xcd_chunk * 8u);
     const bool fbias = a.bias != nullptr && a.float_bias != 0;
     const bool u8_reference = !rne && a.q.lo == 0.f && a.q.hi == 255.f;
     const int path = !u8_reference ? 0 : a.lo_folded > 0.f ? 2 : a.q.zpf == 0.f ? 3 : 1;
