@@ -186,8 +186,15 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
             pv[j] = v;
         }
     };
-    if ((int)blockIdx.x < a.tiles) fetch_patch((int)blockIdx.x);
-    for (int t = blockIdx.x; t < a.tiles; t += gridDim.x) {
+    // The device deals work-groups out to its 8 XCDs in turn: the work-groups of XCD x (blockIdx.x % 8 == x; the grid's
+    // x extent is a multiple of 8) share the tiles [x * chunk, (x + 1) * chunk), so that the input rows neighbouring tiles
+    // have in common (15 of a tile's 21 rows for a 7x7 filter with stride 2) are found in that XCD's own L2.
+    const int t_step = (int)(gridDim.x >> 3);
+    const int chunk = (a.tiles + 7) >> 3;
+    const int t_first = (int)(blockIdx.x & 7u) * chunk + (int)(blockIdx.x >> 3);
+    const int t_end = min(((int)(blockIdx.x & 7u) + 1) * chunk, a.tiles);
+    if (t_first < t_end) fetch_patch(t_first);
+    for (int t = t_first; t < t_end; t += t_step) {
         const int n = (int)magic_div((uint32_t)t, a.tpi_mul, a.tpi_shift);
         const int r = t - n * tiles_per_image;
         const int th = (int)magic_div((uint32_t)r, a.tw_mul, a.tw_shift), tw = r - th * a.tiles_w;
@@ -200,7 +207,7 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(ConvStemArgs a) {
             if (tid + 256 * j < patch_dwords) reinterpret_cast<uint32_t*>(s_patch)[tid + 256 * j] = pv[j];
         }
         __syncthreads();
-        if (t + (int)gridDim.x < a.tiles) fetch_patch(t + (int)gridDim.x);
+        if (t + t_step < t_end) fetch_patch(t + t_step);
 
         // lane holds, per 32x32 MFMA tile: pixel column p, output-channel rows (v/4)*8 + (lane>>5)*4 + v%4
         v16i acc[2];
@@ -380,7 +387,9 @@ int launch_conv_stem(ConvStemArgs a, bool rne, hipStream_t s) {
     const int oc_blocks = (a.OC + 63) / 64;
     int per_block = cus * per_cu / oc_blocks;
     if (per_block < 1) per_block = 1;
-    const dim3 grid((unsigned)(a.tiles < per_block ? a.tiles : per_block), (unsigned)oc_blocks);
+    // (a multiple of 8 work-groups along x: see the kernel's tile order)
+    const int along_x = ((a.tiles < per_block ? a.tiles : per_block) + 7) / 8 * 8;
+    const dim3 grid((unsigned)along_x, (unsigned)oc_blocks);
     const bool kwp4 = a.KW <= 4;
     if (kwp4) {
         if (rne) conv_stem_kernel<4, true><<<grid, 256, lds, s>>>(a);
