@@ -43,6 +43,8 @@ def parse():
                     help="run the residual Add(+Relu) groups as kernels of their own instead of inside the convolution before them")
     ap.add_argument("--no-pair-convs", action="store_true",
                     help="run the two convolutions that read a down-sampling block's input as two launches instead of one")
+    ap.add_argument("--no-minus-128", action="store_true",
+                    help="keep every 8-bit value between two convolutions as uint8 codes instead of codes minus 128 in int8 arrays")
     ap.add_argument("--parts", type=int, default=1,
                     help="run the batch as this many concurrent slices on separate streams (network workloads)")
     ap.add_argument("--runner", default="chxvm", choices=["chxvm", "python"],
@@ -124,8 +126,9 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
     # below prices.
     fuse = not args.no_fuse_residual
     pair = fuse and not args.no_pair_convs and args.parts <= 1
+    signed = fuse and not args.no_minus_128 and args.parts <= 1
     # values share memory once their last reader has run, as in the VM (whose allocator reuses freed slots)
-    runner = wl.DeviceRunner(model, pkg, fuse, reuse_buffers=True, pair_convs=pair) if args.parts <= 1 else None
+    runner = wl.DeviceRunner(model, pkg, fuse, reuse_buffers=True, pair_convs=pair, minus_128=signed) if args.parts <= 1 else None
     timed_runner = runner if args.parts <= 1 else wl.ConcurrentRunner(model, pkg, args.parts, fuse)
 
     def step(_timer):

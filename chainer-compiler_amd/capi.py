@@ -22,6 +22,7 @@ ROUND_ONNX_RNE = 1
 BIAS_REFERENCE_FLOAT = 0
 BIAS_ONNX_INT32 = 2
 FUSE_RELU = 4
+STORE_MINUS_128 = 8
 EINVAL, EUNSUPPORTED, ERUNTIME = 1, 2, 3
 
 EXPORTS = [

@@ -423,6 +423,8 @@ struct ConvCall {
     const chx_hip_tensor* y2 = nullptr;
     int32_t oc_split = 0;
     RequantParams rq2;
+    // CHX_HIP_STORE_MINUS_128 for y / y2: the stored byte is the uint8 code minus 128
+    bool y_minus_128 = false, y2_minus_128 = false;
 };
 
 // Runs the MFMA kernel on packed weights.  x may be channels-last (used in place) or
@@ -537,6 +539,14 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     }
     a.y_vec_ok = aligned(a.y, 16) && (a.y_px_stride % 16 == 0) ? 1 : 0;
     (void)es;
+    if (c.y_minus_128 || c.y2_minus_128) {
+        if (stem || y_post || c.out_int32) {
+            release_scratch(c.cache, x_scratch, s);
+            release_scratch(c.cache, y_scratch, s);
+            CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv: codes minus 128 are stored by the matrix-core kernel into channels-last results only");
+        }
+        a.y_flip = c.y_minus_128 ? 0x80808080u : 0u;
+    }
     if (c.y2) {
         int64_t y2_px = 0;
         if (stem || pw.dense || x_scratch || y_post || c.out_int32 || c.res || !y_is_pixel_major(*c.y2, &y2_px)) {
@@ -548,6 +558,7 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
         a.y2 = static_cast<char*>(c.y2->data);
         a.y2_px_stride = y2_px;
         a.y2_vec_ok = aligned(a.y2, 16) && (y2_px % 16 == 0) ? 1 : 0;
+        a.y2_flip = c.y2_minus_128 ? 0x80808080u : 0u;
         a.q2 = c.rq2.q;
         a.inv_y_scale2 = 1.0f / c.rq2.q.scale;
         a.lo_folded2 = fold_relu_floor(c.rq2.q, c.rq2.relu_floor, c.rne);
@@ -1113,22 +1124,44 @@ extern "C" int chx_hip_qconv_plan_create(
     return CHX_HIP_OK;
 }
 
+namespace chx {
+namespace {
+// CHX_HIP_STORE_MINUS_128: the array is int8, its quantization is that of the uint8 array it stands for.  *view is what
+// the checks and the requantization parameters are derived from.
+int result_view(const chx_hip_tensor* y, uint32_t flags, const char* op, chx_hip_tensor* view, bool* minus_128) {
+    CHX_PROPAGATE(check_tensor(y, op));
+    *view = *y;
+    *minus_128 = (flags & CHX_HIP_STORE_MINUS_128) != 0;
+    if (*minus_128) {
+        CHX_REQUIRE(y->dtype == CHX_HIP_INT8, "%s: codes minus 128 are stored into an int8 array, got %s", op, dtype_name(y->dtype));
+        view->dtype = CHX_HIP_UINT8;
+    }
+    return CHX_HIP_OK;
+}
+}  // namespace
+}  // namespace chx
+
 extern "C" int chx_hip_qconv_plan_run(
         const chx_hip_qconv_plan* plan, const chx_hip_tensor* x, float x_scale, int32_t x_zero_point, float y_scale,
         int32_t y_zero_point, uint32_t flags, chx_hip_tensor* y, void* stream) {
     CHX_REQUIRE(plan != nullptr, "QLinearConv plan: null plan");
+    chx_hip_tensor yv;
+    bool minus_128 = false;
+    CHX_PROPAGATE(result_view(y, flags, "QLinearConv y", &yv, &minus_128));
     QConvChecked q;
     CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, &plan->w, &plan->w_scale, &plan->w_zero_point, y_scale,
-                              y_zero_point, plan->has_bias ? &plan->bias : nullptr, &plan->params, flags, y, &q));
+                              y_zero_point, plan->has_bias ? &plan->bias : nullptr, &plan->params, flags, &yv, &q));
     hipStream_t s = as_stream(stream);
     const bool rne = (flags & CHX_HIP_ROUND_ONNX_RNE) != 0;
     if (plan->mfma) {
-        ConvCall call = conv_call_from(q, x, y, &plan->params, rne, plan->opt);
+        ConvCall call = conv_call_from(q, x, &yv, &plan->params, rne, plan->opt);
         call.cache = const_cast<ScratchCache*>(&plan->scratch);
         call.tune = const_cast<TuneCache*>(&plan->tune);
+        call.y_minus_128 = minus_128;
         const int rc = run_conv_mfma(call, plan->pw, s);
-        if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        if (rc != CHX_HIP_EUNSUPPORTED || minus_128) return rc;
     }
+    if (minus_128) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv: codes minus 128 are stored by the matrix-core kernel only");
     if (plan->depthwise) {
         const int rc = run_depthwise(conv_call_from(q, x, y, &plan->params, rne, plan->opt), plan->dw, s);
         if (rc != CHX_HIP_EUNSUPPORTED) return rc;
@@ -1141,8 +1174,10 @@ extern "C" int chx_hip_qconv_plan_run_pair(
         float y1_scale, int32_t y1_zero_point, uint32_t flags1, chx_hip_tensor* y1, float y2_scale, int32_t y2_zero_point,
         uint32_t flags2, chx_hip_tensor* y2, void* stream) {
     CHX_REQUIRE(plan != nullptr, "QLinearConv pair: null plan");
-    CHX_PROPAGATE(check_tensor(y1, "QLinearConv pair y1"));
-    CHX_PROPAGATE(check_tensor(y2, "QLinearConv pair y2"));
+    chx_hip_tensor y1v, y2v;
+    bool y1_minus_128 = false, y2_minus_128 = false;
+    CHX_PROPAGATE(result_view(y1, flags1, "QLinearConv pair y1", &y1v, &y1_minus_128));
+    CHX_PROPAGATE(result_view(y2, flags2, "QLinearConv pair y2", &y2v, &y2_minus_128));
     CHX_REQUIRE(y1->ndim == 4 && y2->ndim == 4, "QLinearConv pair: y1 and y2 must be 4-D");
     const int64_t OC = plan->w.shape[0];
     CHX_REQUIRE(split > 0 && split < OC && y1->shape[1] == split && y2->shape[1] == OC - split,
@@ -1157,20 +1192,22 @@ extern "C" int chx_hip_qconv_plan_run_pair(
     if (split % 64 != 0) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv pair: the first convolution must have a multiple of 64 output channels");
     if (!plan->mfma) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv pair: these weights do not run on the matrix-core kernel");
     // shapes and parameters as for one convolution with all output channels, laid out like y1
-    chx_hip_tensor y_all = *y1;
+    chx_hip_tensor y_all = y1v;
     y_all.shape[1] = OC;
     QConvChecked q;
     CHX_PROPAGATE(check_qconv(x, x_scale, x_zero_point, &plan->w, &plan->w_scale, &plan->w_zero_point, y1_scale, y1_zero_point,
                               plan->has_bias ? &plan->bias : nullptr, &plan->params, flags1, &y_all, &q));
     RequantParams rq2;
     const int32_t* bias2 = nullptr;
-    CHX_PROPAGATE(fill_requant(x_scale, y2_scale, y2_zero_point, *y2, plan->has_bias ? &plan->bias : nullptr, OC, flags2,
+    CHX_PROPAGATE(fill_requant(x_scale, y2_scale, y2_zero_point, y2v, plan->has_bias ? &plan->bias : nullptr, OC, flags2,
                                "QLinearConv pair", &rq2, &bias2));
     hipStream_t s = as_stream(stream);
-    ConvCall call = conv_call_from(q, x, y1, &plan->params, (flags1 & CHX_HIP_ROUND_ONNX_RNE) != 0, plan->opt);
+    ConvCall call = conv_call_from(q, x, &y1v, &plan->params, (flags1 & CHX_HIP_ROUND_ONNX_RNE) != 0, plan->opt);
     call.cache = const_cast<ScratchCache*>(&plan->scratch);
     call.tune = const_cast<TuneCache*>(&plan->tune);
-    call.y2 = y2;
+    call.y2 = &y2v;
+    call.y_minus_128 = y1_minus_128;
+    call.y2_minus_128 = y2_minus_128;
     call.oc_split = split;
     call.rq2 = rq2;
     return run_conv_mfma(call, plan->pw, s);
@@ -1182,13 +1219,17 @@ extern "C" int chx_hip_qconv_plan_run_add(
         float out_scale, int32_t out_zero_point, int32_t relu, chx_hip_tensor* out, void* stream) {
     CHX_REQUIRE(plan != nullptr, "QLinearConv+Add: null plan");
     CHX_PROPAGATE(check_tensor(r, "QLinearConv+Add r"));
-    CHX_PROPAGATE(check_tensor(out, "QLinearConv+Add out"));
-    CHX_REQUIRE(is_q8(y_dtype) && is_q8(r->dtype) && is_q8(out->dtype), "QLinearConv+Add: y, r and out must be uint8 or int8");
+    // (with CHX_HIP_STORE_MINUS_128 `out` is an int8 array that holds the codes of a uint8 sum minus 128)
+    chx_hip_tensor outv;
+    bool out_minus_128 = false;
+    CHX_PROPAGATE(result_view(out, flags, "QLinearConv+Add out", &outv, &out_minus_128));
+    const int32_t out_dtype = outv.dtype;
+    CHX_REQUIRE(is_q8(y_dtype) && is_q8(r->dtype) && is_q8(out_dtype), "QLinearConv+Add: y, r and out must be uint8 or int8");
     CHX_REQUIRE(r->ndim == 4 && out->ndim == 4, "QLinearConv+Add: r and out must be 4-D");
     for (int i = 0; i < 4; ++i)
         CHX_REQUIRE(r->shape[i] == out->shape[i], "QLinearConv+Add: r and out differ in shape (no broadcasting)");
     auto in_range = [](int32_t zp, int32_t dt) { return dt == CHX_HIP_INT8 ? zp >= -128 && zp <= 127 : zp >= 0 && zp <= 255; };
-    CHX_REQUIRE(in_range(r_zero_point, r->dtype) && in_range(out_zero_point, out->dtype),
+    CHX_REQUIRE(in_range(r_zero_point, r->dtype) && in_range(out_zero_point, out_dtype),
                 "QLinearConv+Add: zero point out of the range of its type");
     if (!(out_scale >= 0x1p-60f && out_scale <= 0x1p60f))
         CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv+Add: out_scale outside [2^-60, 2^60]");
@@ -1218,13 +1259,14 @@ extern "C" int chx_hip_qconv_plan_run_add(
     res.r_zpf = (float)(r_zero_point + (r->dtype == CHX_HIP_INT8 ? 128 : 0));
     res.r_scale = r_scale;
     res.relu = relu ? 1 : 0;
-    res.out = make_quant_params(out_scale, out_zero_point, out->dtype == CHX_HIP_INT8);
+    res.out = make_quant_params(out_scale, out_zero_point, out_dtype == CHX_HIP_INT8);
     res.inv_out_scale = 1.0f / out_scale;
     res.big = 0x1p40f * out_scale;
     // |DQ(y) + DQ(r)| <= 511 * (|y_scale| + |r_scale|): when that is far below `big`, limiting is the identity
     const double reach = 511.0 * (fabs((double)y_scale) + fabs((double)r_scale));
     res.guard = (reach == reach && reach < 0.25 * (double)res.big) ? 0 : 1;
-    res.lean = out->dtype == CHX_HIP_UINT8 && r->dtype == CHX_HIP_UINT8 && r_zero_point == 0 && out_zero_point == 0 ? 1 : 0;
+    // (r's zero point in the unsigned range: a uint8 r with zero point 0, or the same codes stored minus 128 as int8)
+    res.lean = out_dtype == CHX_HIP_UINT8 && res.r_zpf == 0.f && out_zero_point == 0 ? 1 : 0;
     hipStream_t s = as_stream(stream);
     // The cheaper form of the sum, where the search over its constants has shown it exact for these parameters.  The
     // search runs on the first call with new parameters (it synchronizes the stream and allocates, so not while the
@@ -1270,6 +1312,7 @@ extern "C" int chx_hip_qconv_plan_run_add(
     call.cache = const_cast<ScratchCache*>(&plan->scratch);
     call.tune = const_cast<TuneCache*>(&plan->tune);
     call.res = &res;
+    call.y_minus_128 = out_minus_128;
     return run_conv_mfma(call, plan->pw, s);
 }
 

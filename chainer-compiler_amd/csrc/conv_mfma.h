@@ -62,6 +62,7 @@ struct ConvMfmaArgs {
     char* y;
     int64_t y_px_stride;
     int32_t y_vec_ok;     // 16-byte stores allowed (base and pitch aligned)
+    uint32_t y_flip;      // 0x80808080: every stored byte is the code minus 128 (CHX_HIP_STORE_MINUS_128), else 0
     // epilogue
     const float* w_scale;
     int32_t w_scale_len;
@@ -86,6 +87,7 @@ struct ConvMfmaArgs {
     char* y2;
     int64_t y2_px_stride;
     int32_t y2_vec_ok;
+    uint32_t y2_flip;
     QuantParams q2;
     float inv_y_scale2;
     float lo_folded2;

@@ -442,6 +442,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                 a.y = a.y2 - a.oc_split;
                 a.y_px_stride = a.y2_px_stride;
                 a.y_vec_ok = a.y2_vec_ok;
+                a.y_flip = a.y2_flip;
                 a.rq.q = a.q2;
                 a.inv_y_scale = a.inv_y_scale2;
                 a.lo_folded = a.lo_folded2;
@@ -605,6 +606,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                 constexpr int kMode = decltype(mode_tag)::value;  // 0: no residual, 1 / 2: the two-multiply-add forms, 3: the exact chain
                 ResidualAdd res;
                 if constexpr (kMode != 0) res = in_vector_registers(a.res);
+                const int store_flip = (int)in_vector_register(a.y_flip);
 #pragma unroll
                 for (int it = 0; it < ITER; ++it) {
                     const int q = tid + it * T;
@@ -614,6 +616,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                     if constexpr (kMode == 1) val = affine_residual16<false>(val, rres[it], res);
                     if constexpr (kMode == 2) val = affine_residual16<true>(val, rres[it], res);
                     if constexpr (kMode == 3) val = add_residual16_any(val, rres[it], res);
+                    val ^= store_flip;
                     *reinterpret_cast<v4i*>(a.y + (m0 + pxl) * a.y_px_stride + oc0 + ch * 16) = val;
                 }
             };
@@ -649,8 +652,9 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                 if (a.res.affine == 1) val = affine_residual16<false>(val, rv, a.res);
                 else if (a.res.affine == 2) val = affine_residual16<true>(val, rv, a.res);
                 else val = add_residual16_any(val, rv, a.res);
-                if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
             }
+            val ^= (int)a.y_flip;
+            if (!(a.y_vec_ok && whole)) *reinterpret_cast<v4i*>(src) = val;  // the byte loop below reads LDS
             char* dst = a.y + m * a.y_px_stride + oc;
             if (a.y_vec_ok && whole) {
                 *reinterpret_cast<v4i*>(dst) = val;

@@ -304,11 +304,48 @@ def pair_convolutions(program, convs):
     return out
 
 
+def minus_128_values(program, convs, fused_into):
+    """The values of `program` that can be stored as code - 128 in int8 arrays (CHX_HIP_STORE_MINUS_128): written by the
+    matrix-core convolution kernel (a QLinearConv that is not grouped and has at least 16 input channels, a pair of them,
+    or the residual sum inside one) and read only by convolutions, as their input or as the residual operand of a sum
+    that one of them computes.  A reading convolution with padding must find the padding value, its input's zero point,
+    stored as the byte 0 (a uint8 zero point of 128), or it does not run with the padding that costs nothing; a value
+    with such a reader and another zero point keeps its uint8 array.
+    `fused_into`: convolution result -> the Add instruction computed inside that convolution."""
+    fused_adds = set(add[1] for add in fused_into.values())
+    producers = {}
+    for ins in program:
+        if ins[0] == "QLinearConv" and convs[ins[3]].group == 1 and convs[ins[3]].wq.shape[1] >= 16:
+            producers[fused_into[ins[1]][1] if ins[1] in fused_into else ins[1]] = ins
+        if ins[0] == "QLinearConvPair":
+            producers[ins[1]] = producers[ins[4]] = ins
+    keep = set()
+    for name in producers:
+        ok, readers = True, 0
+        for ins in program:
+            if ins[0] in ("QLinearConv", "QLinearConvPair"):
+                if ins[2] == name:
+                    readers += 1
+                    c = convs[ins[3]]
+                    if c.pad and c.x_zp != 128:
+                        ok = False
+            elif ins[0] in ("Add", "AddRelu") and ins[1] in fused_adds:
+                # computed inside a convolution: `name` may be its residual operand, not the convolution's own result
+                conv_out = [k for k, add in fused_into.items() if add[1] == ins[1]][0]
+                if name in ins[2:4] and name != conv_out:
+                    readers += 1
+            elif name in [a for a in ins[2:4] if isinstance(a, str)]:
+                ok = False
+        if ok and readers:
+            keep.add(name)
+    return keep
+
+
 class DeviceRunner(object):
     """Runs a program on the MI355X: weights resident, one plan per QLinearConv, every
     activation channels-last, all intermediate buffers allocated once."""
 
-    def __init__(self, model, pkg, fuse_residual=False, reuse_buffers=False, pair_convs=False):
+    def __init__(self, model, pkg, fuse_residual=False, reuse_buffers=False, pair_convs=False, minus_128=False):
         """fuse_residual: a QLinearConv whose only reader is the residual Add(+Relu) of its block runs
         as one kernel with it; the convolution's own output is then not materialised.
         reuse_buffers: a value's memory goes back to a pool after its last reader and is handed to later
@@ -316,6 +353,8 @@ class DeviceRunner(object):
         then a few tensors instead of every tensor of the network, and run() returns only values that are
         still live at the end (the program's last result is).
         pair_convs: two convolutions of the same value with the same geometry run as one launch (pair_convolutions);
+        minus_128: values that only convolutions read are stored as code - 128 in int8 arrays (minus_128_values; the
+        entries of run()'s result for them are int8 tensors), which spares the reading kernel the sign flips;
         self.program is the instruction list the runner executes."""
         self.m, self.ops, self.capi = model, pkg.ops, pkg.capi
         self.fused_into = {}   # conv output name -> the Add instruction that absorbs it
@@ -328,6 +367,7 @@ class DeviceRunner(object):
                     readers = sum(1 for other in program if prev[1] in other[2:4] and other[0] != "QuantizeLinear")
                     if prev[0] == "QLinearConv" and prev[1] in ins[2:4] and readers == 1 and model["convs"][prev[3]].group == 1:
                         self.fused_into[prev[1]] = ins
+        self.minus_128 = minus_128_values(program, model["convs"], self.fused_into) if minus_128 else set()
         self.dev = {}
         self.plans = {}
         self.bufs = {}
@@ -383,6 +423,8 @@ class DeviceRunner(object):
                 pitch = (c + 15) // 16 * 16
                 block_of[out] = take(n * h * w * pitch)
                 full = block_of[out][:n * h * w * pitch].view(n, h, w, pitch)
+                if out in self.minus_128:
+                    full = full.view(torch.int8)
                 self.bufs[out] = full[..., :c].permute(0, 3, 1, 2)
                 # element-wise groups run over the padded pixels as they lie in memory (dense)
                 self.full[out] = full.permute(0, 3, 1, 2)
@@ -412,6 +454,10 @@ class DeviceRunner(object):
         ins = self.program[fid]
         kind, out = ins[0], ins[1]
         buf = self.bufs.get(out)   # none for a convolution whose result only exists inside the fused residual sum
+        S = self.minus_128
+        zp_of = lambda name, zp: zp - 128 if name in S else zp                    # an int8 array of codes minus 128
+        dt_of = lambda name: torch.int8 if name in S else torch.uint8
+        fl_of = lambda name: self.capi.BIAS_ONNX_INT32 | (self.capi.STORE_MINUS_128 if name in S else 0)
         if kind == "QuantizeLinear":
             ops.QuantizeLinear(v[ins[2]], ins[3], ins[4], torch.uint8, out=buf)
         elif kind == "QLinearConv" and out in self.fused_into:
@@ -420,21 +466,20 @@ class DeviceRunner(object):
             c = m["convs"][ins[3]]
             # DequantizeLinear(a) + DequantizeLinear(b) is commutative bit for bit, so the
             # convolution may be either operand of the Add
-            self.plans[ins[3]].run_add(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, v[other], q[other][0], q[other][1],
-                                       q[add[1]][0], q[add[1]][1], add[0] == "AddRelu", torch.uint8,
-                                       flags=self.capi.BIAS_ONNX_INT32, out=self.bufs[add[1]])
+            self.plans[ins[3]].run_add(v[ins[2]], c.x_scale, zp_of(ins[2], c.x_zp), c.y_scale, c.y_zp, v[other], q[other][0],
+                                       zp_of(other, q[other][1]), q[add[1]][0], q[add[1]][1], add[0] == "AddRelu", torch.uint8,
+                                       flags=fl_of(add[1]), out=self.bufs[add[1]])
             return None
         elif kind in ("AddRelu", "Add") and (ins[2] in self.fused_into or ins[3] in self.fused_into):
             pass   # written by the fused convolution
         elif kind == "QLinearConv":
             c = m["convs"][ins[3]]
-            self.plans[ins[3]].run(v[ins[2]], c.x_scale, c.x_zp, c.y_scale, c.y_zp, torch.uint8,
-                                   flags=self.capi.BIAS_ONNX_INT32, out=buf)
+            self.plans[ins[3]].run(v[ins[2]], c.x_scale, zp_of(ins[2], c.x_zp), c.y_scale, c.y_zp, dt_of(out), flags=fl_of(out), out=buf)
         elif kind == "QLinearConvPair":
             c1, c2 = m["convs"][ins[3]], m["convs"][ins[5]]
             self.plans[ins[3] + "+" + ins[5]].run_pair(
-                v[ins[2]], c1.x_scale, c1.x_zp, c1.wq.shape[0], c1.y_scale, c1.y_zp, c2.y_scale, c2.y_zp,
-                flags=(self.capi.BIAS_ONNX_INT32, self.capi.BIAS_ONNX_INT32), outs=(buf, self.bufs[ins[4]]))
+                v[ins[2]], c1.x_scale, zp_of(ins[2], c1.x_zp), c1.wq.shape[0], c1.y_scale, c1.y_zp, c2.y_scale, c2.y_zp,
+                flags=(fl_of(out), fl_of(ins[4])), outs=(buf, self.bufs[ins[4]]))
             v[ins[4]] = self.bufs[ins[4]]
         elif kind == "MaxPool":
             ops.MaxPoolQ8(v[ins[2]], (ins[3], ins[3]), (ins[4], ins[4]), (ins[5], ins[5]), ins[6], out=buf)

@@ -68,7 +68,14 @@ enum {
     CHX_HIP_BIAS_REFERENCE_FLOAT = 0u,/* float(b) added unscaled to the fp32 result: runtime/ops/quantize.cc:93 */
     CHX_HIP_BIAS_ONNX_INT32 = 2u,     /* b added to the int32 accumulator (scale x_scale*w_scale) */
     /* Q(Relu(DQ(q))) folded into the epilogue: output clamped below at y_zero_point */
-    CHX_HIP_FUSE_RELU = 4u
+    CHX_HIP_FUSE_RELU = 4u,
+    /* chx_hip_qconv_plan_run / _run_add / _run_pair only: the result is quantized as uint8 (its zero point is given in
+     * the uint8 range) but every byte is stored as code - 128, in an array of dtype int8.  An int8 array with zero point
+     * zp - 128 denotes the same numbers, so a later QLinearConv reads it as its int8 x (or a fused residual sum as its
+     * int8 r) with that zero point and gives the bytes it would give on the uint8 array, without flipping sign bits in
+     * its inner loop.  No counterpart in the reference; a storage convention between the convolutions of one host.
+     * CHX_HIP_EUNSUPPORTED where the matrix-core kernel does not run (store uint8 then). */
+    CHX_HIP_STORE_MINUS_128 = 8u
 };
 
 typedef struct chx_hip_tensor {

@@ -597,6 +597,72 @@ def test_two_convolutions_of_one_input_in_one_launch(g, oracle, case):
     plan.close()
 
 
+def test_results_stored_minus_128(g, oracle):
+    """CHX_HIP_STORE_MINUS_128: a uint8 result stored as code - 128 in an int8 array is the same tensor as an int8 one
+    with zero point zp - 128.  The flag on the three plan entry points gives the bytes of the plain result with the top
+    bit flipped, and a convolution (or a fused residual sum) that reads such an array as int8 gives the bytes it gives
+    on the uint8 array: a chain of two convolutions with a residual sum, every intermediate in both storages."""
+    rng = np.random.default_rng(151)
+    N, C, H, W, OC = 2, 64, 9, 10, 128
+    x = rand_q(rng, (N, C, H, W), np.uint8)
+    w1 = rng.integers(-127, 128, size=(OC, C, 3, 3)).astype(np.int8)
+    w2 = rng.integers(-127, 128, size=(C, OC, 1, 1)).astype(np.int8)
+    ws1, ws2 = rng.uniform(0.002, 0.02, size=OC).astype(np.float32), rng.uniform(0.002, 0.02, size=C).astype(np.float32)
+    b1, b2 = rng.integers(-500, 501, size=OC).astype(np.int32), rng.integers(-500, 501, size=C).astype(np.int32)
+    y1s, y1z = np.float32(0.02 * 0.01 * 74 * 74 * np.sqrt(C * 9) / 40), 17
+    y2s, y2z = np.float32(y1s * 0.01 * 74 * np.sqrt(OC) / 3), 119
+    os_, oz = np.float32(0.05), 0
+    kw1 = dict(strides=(1, 1), pads=(1, 1))
+    a = oracle.qlinear_conv_int(x, 0.02, 101, w1, ws1, np.zeros(OC, np.int8), y1s, y1z, np.uint8, bias=b1, bias_mode=oracle.BIAS_ONNX_INT32, **kw1)
+    c = oracle.qlinear_conv_int(a, y1s, y1z, w2, ws2, np.zeros(C, np.int8), y2s, y2z, np.uint8, bias=b2, bias_mode=oracle.BIAS_ONNX_INT32)
+    for relu in (True, False):
+        want_sum = _residual_sum(oracle, c, y2s, y2z, x, np.float32(0.02), 101, relu, os_, oz, np.uint8)
+        assert a.min() < a.max() and c.min() < c.max() and want_sum.min() < want_sum.max()
+        flip = lambda t: (t.view(torch.uint8) ^ 0x80)       # int8 storage -> the uint8 codes it stands for
+        F = g.capi.BIAS_ONNX_INT32
+        S = F | g.capi.STORE_MINUS_128
+        p1 = g.ops.QLinearConvPlan(g.dev(w1), g.dev(ws1), g.dev(np.zeros(OC, np.int8)), g.dev(b1), **kw1)
+        p2 = g.ops.QLinearConvPlan(g.dev(w2), g.dev(ws2), g.dev(np.zeros(C, np.int8)), g.dev(b2))
+        xd = g.to_channels_last(g.dev(x))
+        xs = (xd.view(torch.uint8) ^ 0x80).view(torch.int8)        # the input stored minus 128
+        for x_in, x_zp in ((xd, 101), (xs, 101 - 128)):
+            # first convolution, result in either storage
+            a_u = p1.run(x_in, 0.02, x_zp, y1s, y1z, torch.uint8, flags=F)
+            a_s = p1.run(x_in, 0.02, x_zp, y1s, y1z, torch.int8, flags=S)
+            np.testing.assert_array_equal(g.host(a_u), a)
+            assert a_s.dtype == torch.int8
+            np.testing.assert_array_equal(g.host(flip(a_s)), a)
+            for a_in, a_zp in ((a_u, y1z), (a_s, y1z - 128)):
+                # second convolution with the block's residual sum (the residual in either storage too), result in either storage
+                for r_in, r_zp in ((xd, 101), (xs, 101 - 128)):
+                    got = p2.run_add(a_in, y1s, a_zp, y2s, y2z, r_in, 0.02, r_zp, os_, oz, relu, zero_point_dtype=torch.uint8, flags=F,
+                                     out=torch.zeros_like(xd))
+                    np.testing.assert_array_equal(g.host(got), want_sum)
+                    got = p2.run_add(a_in, y1s, a_zp, y2s, y2z, r_in, 0.02, r_zp, os_, oz, relu, zero_point_dtype=torch.uint8, flags=S,
+                                     out=torch.zeros_like(xs))
+                    np.testing.assert_array_equal(g.host(flip(got)), want_sum)
+        # two convolutions in one launch, one result in each storage
+        wp = np.concatenate([w1, w1[::-1]])
+        pp = g.ops.QLinearConvPlan(g.dev(wp), g.dev(np.concatenate([ws1, ws1[::-1]])), g.dev(np.zeros(2 * OC, np.int8)), g.dev(np.concatenate([b1, b1[::-1]])), **kw1)
+        a_rev = oracle.qlinear_conv_int(x, 0.02, 101, w1[::-1].copy(), ws1[::-1].copy(), np.zeros(OC, np.int8), y1s, 33, np.uint8, bias=b1[::-1].copy(),
+                                        bias_mode=oracle.BIAS_ONNX_INT32, **kw1)
+        o1, o2 = pp.run_pair(xs, 0.02, 101 - 128, OC, y1s, y1z, y1s, 33, zero_point_dtypes=(torch.int8, torch.uint8), flags=(S, F))
+        np.testing.assert_array_equal(g.host(flip(o1)), a)
+        np.testing.assert_array_equal(g.host(o2), a_rev)
+        o1, o2 = pp.run_pair(xd, 0.02, 101, OC, y1s, y1z, y1s, 33, zero_point_dtypes=(torch.uint8, torch.int8), flags=(F, S))
+        np.testing.assert_array_equal(g.host(o1), a)
+        np.testing.assert_array_equal(g.host(flip(o2)), a_rev)
+        # the flag wants an int8 array, and a kernel that can honour it
+        with pytest.raises(g.capi.ChxHipError) as e:
+            p1.run(xd, 0.02, 101, y1s, y1z, torch.uint8, flags=S)
+        assert e.value.code == g.capi.EINVAL
+        with pytest.raises(g.capi.ChxHipError) as e:
+            p1.run(g.dev(x), 0.02, 101, y1s, y1z, torch.int8, flags=S)        # NCHW: the result would be transposed afterwards
+        assert e.value.code == g.capi.EUNSUPPORTED
+        for p in (p1, p2, pp):
+            p.close()
+
+
 def test_random_convolution_sweep(g, oracle):
     """Seeded random QLinearConv / ConvInteger configurations across every dispatch path (matrix-core
     tiles, first-layer kernel, depthwise kernel, generic kernel): shapes, kernel sizes, strides, pads,

@@ -25,21 +25,26 @@ def check_model(g, oracle, model, threads=16):
     # every op a kernel of its own; then with the residual sums inside the convolutions before them (those
     # convolutions' own outputs are then not materialised); then also with the two convolutions that read a
     # down-sampling block's input as one launch
-    paired = 0
-    for fuse, pair in ((False, False), (True, False), (True, True)):
-        runner = wl.DeviceRunner(model, g.pkg, fuse_residual=fuse, pair_convs=pair)
+    for fuse, pair, signed in ((False, False, False), (True, False, False), (True, True, False), (True, True, True), (False, False, True)):
+        runner = wl.DeviceRunner(model, g.pkg, fuse_residual=fuse, pair_convs=pair, minus_128=signed)
         dev = runner.run(torch.from_numpy(model["input"]).cuda())
         torch.cuda.synchronize()
         assert bool(runner.fused_into) == (fuse and any(i[0] in ("Add", "AddRelu") for i in model["program"]))
         paired = sum(1 for i in runner.program if i[0] == "QLinearConvPair")
-        assert (paired > 0) == (pair and len(runner.program) < len(model["program"]))
+        assert (paired > 0) == (pair and len(wl.pair_convolutions(model["program"], model["convs"])) < len(model["program"]))
+        assert bool(runner.minus_128) == signed
         for ins in model["program"]:
             name = ins[1]
             if name in runner.fused_into:
                 assert name not in dev
                 continue
-            got = dev[name].cpu().numpy()
-            np.testing.assert_array_equal(got, ref[name], err_msg="value %s after %s (fused residual: %s, paired: %s)" % (name, ins[0], fuse, pair))
+            got = dev[name]
+            if name in runner.minus_128:
+                # codes minus 128 in an int8 array: the values only convolutions read
+                assert got.dtype == torch.int8
+                got = got.view(torch.uint8) ^ 0x80
+            np.testing.assert_array_equal(got.cpu().numpy(), ref[name],
+                                          err_msg="value %s after %s (fused residual: %s, paired: %s, minus 128: %s)" % (name, ins[0], fuse, pair, signed))
         runner.close()
     return ref
 
