@@ -143,6 +143,7 @@ def bench_resnet50(args, torch, pkg, mobilenet=False):
         import importlib
         vm = importlib.import_module(pkg.__name__ + ".chxvm")
         vm.set_option("pair_convolutions", "on" if pair else "off")
+        vm.set_option("store_minus_128", "on" if signed else "off")
         vm_prog = vm.Program(wl.program_to_chxvm(model, vm, ops, keep=("logits",)).serialize())
         vm_prog.set_option("qlinearconv_bias", "onnx_int32")
         if args.no_graph:

@@ -31,7 +31,7 @@ EXPORTS = [
     "chx_hip_quantize_linear", "chx_hip_dequantize_linear", "chx_hip_qlinear_conv", "chx_hip_qlinear_conv_nd", "chx_hip_conv_integer_nd", "chx_hip_qconv_plan_create",
     "chx_hip_qconv_plan_run", "chx_hip_qconv_plan_run_add", "chx_hip_qconv_plan_run_pair", "chx_hip_qconv_plan_describe", "chx_hip_qconv_plan_pin", "chx_hip_qconv_plan_destroy", "chx_hip_conv_integer", "chx_hip_matmul_integer",
     "chx_hip_qlinear_matmul", "chx_hip_elementwise", "chx_hip_elementwise_source", "chx_hip_elementwise_output_dtypes", "chx_hip_elementwise_match_residual_add",
-    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_reduce_min_max_noalloc", "chx_hip_cast", "chx_hip_bit_shift", "chx_hip_count_nonfinite",
+    "chx_hip_max_pool_q8", "chx_hip_average_pool_q8", "chx_hip_reduce_min_max", "chx_hip_reduce_min_max_noalloc", "chx_hip_cast", "chx_hip_codes_minus_128", "chx_hip_bit_shift", "chx_hip_count_nonfinite",
     "chx_hip_stream_create", "chx_hip_stream_destroy", "chx_hip_capture_begin", "chx_hip_capture_end", "chx_hip_stream_is_capturing",
     "chx_hip_graph_launch", "chx_hip_graph_destroy", "chx_hip_gemm_f32", "chx_hip_linear_f32", "chx_hip_max_pool_f32", "chx_hip_average_pool_f32", "chx_hip_fixed_batch_norm_f32", "chx_hip_conv_f32", "chx_hip_softmax_f32",
 ]

@@ -230,6 +230,34 @@ extern "C" int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* st
 namespace chx {
 namespace {
 
+// y = x with bit 7 of every byte inverted, one lane per element, any strides on both sides
+__global__ __launch_bounds__(kThreads) void flip_sign_bits_kernel(const char* __restrict__ x, StridedDesc xd, char* __restrict__ y, StridedDesc yd, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    y[strided_offset(i, yd)] = (char)(x[strided_offset(i, xd)] ^ 0x80);
+}
+
+}  // namespace
+}  // namespace chx
+
+extern "C" int chx_hip_codes_minus_128(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream) {
+    CHX_PROPAGATE(check_tensor(x, "codes minus 128: x"));
+    CHX_PROPAGATE(check_tensor(y, "codes minus 128: y"));
+    CHX_REQUIRE((x->dtype == CHX_HIP_UINT8 && y->dtype == CHX_HIP_INT8) || (x->dtype == CHX_HIP_INT8 && y->dtype == CHX_HIP_UINT8),
+                "codes minus 128: uint8 -> int8 (code - 128) or int8 -> uint8 (code + 128), got %s -> %s", dtype_name(x->dtype), dtype_name(y->dtype));
+    CHX_REQUIRE(x->ndim == y->ndim, "codes minus 128: x and y differ in rank");
+    for (int i = 0; i < x->ndim; ++i) CHX_REQUIRE(x->shape[i] == y->shape[i], "codes minus 128: x and y differ in shape");
+    const int64_t n = numel(*x);
+    if (n == 0) return CHX_HIP_OK;
+    const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads);
+    flip_sign_bits_kernel<<<blocks, kThreads, 0, as_stream(stream)>>>(static_cast<const char*>(x->data), make_desc(*x), static_cast<char*>(y->data),
+                                                                      make_desc(*y), n);
+    return launch_check("flip_sign_bits_kernel");
+}
+
+namespace chx {
+namespace {
+
 // z = x << y or x >> y over the broadcast of x and y (strides of 0 on broadcast axes), one lane per element.
 // A count of the element width or more shifts every bit out: 0, or for a negative x shifted right the sign (-1), as
 // numpy defines it (C leaves it undefined); a right shift of a signed type is arithmetic.

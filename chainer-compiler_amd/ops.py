@@ -201,6 +201,15 @@ def BitShift(x, y, direction):
     return z
 
 
+def codes_minus_128(x, out=None):
+    """chx_hip_codes_minus_128: a uint8 tensor as int8 codes minus 128 (the storage CHX_HIP_STORE_MINUS_128 writes), or
+    such an int8 tensor back as uint8.  No counterpart in the reference."""
+    if out is None:
+        out = torch.empty_like(x, dtype=torch.int8 if x.dtype == torch.uint8 else torch.uint8)
+    capi.check(capi.lib().chx_hip_codes_minus_128(capi.ref(x), capi.ref(out), capi.stream_ptr()))
+    return out
+
+
 def Gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_a=0, trans_b=0, out=None):
     """GemmOp::RunImpl, runtime/ops/math.cc:160-177, on float32 matrices."""
     if out is None:

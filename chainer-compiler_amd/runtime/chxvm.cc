@@ -170,6 +170,7 @@ private:
 // both instructions run as they are.
 bool g_fuse_residual = true;
 bool g_pair_convolutions = true;
+bool g_store_minus_128 = true;
 
 struct ResidualFusionState {
     bool fused = false;  // of the current run
@@ -194,7 +195,15 @@ public:
         req.r_scale = g_.in_scale[1 - k_]; req.r_zero_point = g_.in_zero_point[1 - k_];
         req.out_scale = g_.out_scale; req.out_zero_point = g_.out_zero_point; req.out_dtype = dt(g_.out_dtype);
         req.relu = g_.relu != 0;
-        const bool r_fits = !req.r.IsNullHandle() && req.r.dtype() == dt(g_.in_dtype[1 - k_]);
+        req.out_slot = group_out_;
+        bool r_fits = !req.r.IsNullHandle() && req.r.dtype() == dt(g_.in_dtype[1 - k_]);
+        // the other operand kept as code - 128: an int8 tensor with the zero point 128 lower
+        const bool r_minus_128 = !req.r.IsNullHandle() && st->store_minus_128(other_) && req.r.dtype() == chainerx::Dtype::kInt8 &&
+                                 dt(g_.in_dtype[1 - k_]) == chainerx::Dtype::kUInt8;
+        if (r_minus_128) {
+            req.r_zero_point -= 128;
+            r_fits = true;
+        }
         st->set_residual_request(r_fits ? &req : nullptr);
         try {
             conv_->Run(st);
@@ -208,6 +217,11 @@ public:
             if (st->trace_level()) std::cerr << "  (residual sum $" << group_out_ << " computed by the convolution)" << std::endl;
             st->FreeVar(conv_out_);  // holds a null array: the convolution's own result was never written
             st->SetArray(group_out_, req.out);
+        } else if (r_minus_128) {
+            // the group instruction will run as the program wrote it: it reads plain codes
+            const chainerx::Array plain = PlainCodes(req.r);
+            st->FreeVar(other_);
+            st->SetArray(other_, plain);
         }
     }
 
@@ -428,6 +442,62 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
             break;
         }
     }
+    // Values that may be kept as code - 128 in int8 arrays (ChxVMState::store_minus_128): every writer is a QLinearConv
+    // or a residual-sum group computed inside one (the producers that know the storage; a writer that runs some other
+    // way stores plain codes and the readers see that from the array's type), and every reader is a QLinearConv that
+    // takes the value as its input, or a residual-sum group computed inside a convolution that takes it as the other
+    // operand (QLinearConvWithResidualOp puts plain codes back when its convolution does not compute the group after
+    // all).  A reading convolution with padding is left out: it pads with its input's zero point, and only a zero
+    // point stored as the byte 0 comes from the padding that costs nothing; the codes of a zero point of 0, the usual
+    // one behind a Relu, are stored as 0x80.
+    minus_128_slots_.assign(num_variables_ > 0 ? num_variables_ : 1, false);
+    if (g_store_minus_128) {
+        std::vector<int> verdict(minus_128_slots_.size(), 0);  // 0 unseen, 1 possible so far, -1 no
+        auto rule_out = [&](int slot) {
+            if (slot >= 0 && slot < static_cast<int>(verdict.size())) verdict[slot] = -1;
+        };
+        auto candidate = [&](int slot) {
+            if (slot >= 0 && slot < static_cast<int>(verdict.size()) && verdict[slot] == 0) verdict[slot] = 1;
+        };
+        for (int i = 0; i < n; ++i) {
+            const ChxVMInstructionProto& inst = program.instructions[i];
+            const bool conv = inst.op == kQLinearConv && inst.inputs.size() == 13 && !inst.outputs.empty();
+            // writers
+            for (size_t o = 0; o < inst.outputs.size(); ++o) {
+                const bool knows = (conv && o == 0 && role[i] != 1) || (role[i] == 5 && o == 0);
+                if (knows) candidate(inst.outputs[o]);
+                else rule_out(inst.outputs[o]);
+            }
+            // readers
+            if (inst.op == kFree) continue;
+            int conv_input = -1, residual_operand = -1;
+            if (conv && role[i] != 1) {
+                bool unpadded = inst.inputs[12].s.empty() || inst.inputs[12].s == "NOTSET" || inst.inputs[12].s == "VALID";
+                for (int64_t pad : inst.inputs[10].ints) unpadded = unpadded && pad == 0;
+                if (unpadded) conv_input = inst.inputs[0].array;
+            }
+            if (role[i] == 5) residual_operand = inst.inputs[0].array_list[1 - conv_operand[partner[i]]];
+            for (const ChxVMValueProto& v : inst.inputs) {
+                switch (v.type) {
+                    case ChxVMValueProto::ARRAY:
+                    case ChxVMValueProto::OPTIONAL_ARRAY:
+                        if (!(v.array == conv_input && &v == &inst.inputs[0])) rule_out(v.array);
+                        break;
+                    case ChxVMValueProto::ARRAY_LIST:
+                        for (int id : v.array_list)
+                            if (!(id == residual_operand && id != inst.inputs[0].array_list[conv_operand[partner[i]]])) rule_out(id);
+                        break;
+                    case ChxVMValueProto::SEQUENCE: rule_out(v.sequence); break;
+                    case ChxVMValueProto::OPAQUE: rule_out(v.opaque); break;
+                    case ChxVMValueProto::SHAPE: rule_out(v.shape); break;
+                    case ChxVMValueProto::SCALAR:
+                    case ChxVMValueProto::OPTIONAL_SCALAR: rule_out(v.scalar); break;
+                    default: break;
+                }
+            }
+        }
+        for (size_t v = 0; v < verdict.size(); ++v) minus_128_slots_[v] = verdict[v] == 1;
+    }
     // A fused op runs where its last instruction stood but reads the operands of the earlier ones: a
     // Free of such an operand between the two (the compiler frees a value right after its last
     // reader) moves behind the fused op.
@@ -506,6 +576,10 @@ void SetFuseResidual(bool on) {
 
 void SetPairConvolutions(bool on) {
     g_pair_convolutions = on;
+}
+
+void SetStoreMinus128(bool on) {
+    g_store_minus_128 = on;
 }
 
 namespace {
@@ -623,6 +697,8 @@ InOuts ChxVM::Run(const InOuts& program_inputs, const ChxVMOptions& options) {
         }
     }
     ChxVMState state(options, num_variables_, program_inputs);
+    // (a run that checks result types against the program's or writes results to files sees plain codes everywhere)
+    if (!options.check_types && options.dump_outputs_dir.empty()) state.set_minus_128_slots(&minus_128_slots_);
     int64_t peak_used_mbs = 0;
     while (state.pc() < static_cast<int>(program_.size())) {
         const int pc = state.pc();

@@ -22,6 +22,7 @@ struct QLinearConvResidualRequest {
     int32_t y_zero_point = 0, r_zero_point = 0, out_zero_point = 0;
     chainerx::Dtype y_dtype = chainerx::Dtype::kUInt8, out_dtype = chainerx::Dtype::kUInt8;
     bool relu = false;
+    int out_slot = -1;  // the variable the sum goes to (ChxVMState::store_minus_128 says how it may be stored)
     chainerx::Array out;
     bool done = false;
 };
@@ -37,6 +38,14 @@ std::unique_ptr<ChxVMOp> MakeQLinearConvPairOp(const ChxVMInstructionProto& firs
 int64_t QLinearConvPairFusions();  // pairs run as one launch so far, process-wide
 // Whether programs loaded from now on pair such convolutions at all (default: yes).
 void SetPairConvolutions(bool on);
+
+// Values that only convolutions read (as their input, or as the residual operand of a sum computed inside one) are
+// stored as code - 128 in int8 arrays (CHX_HIP_STORE_MINUS_128 of the device library): the reading kernel then
+// needs no sign flips in its inner loop.  Whether programs loaded from now on do so at all (default: yes).
+void SetStoreMinus128(bool on);
+int64_t Minus128Stores();  // results written in that storage so far, process-wide
+// The plain uint8 array of a value held in that storage (chx_hip_codes_minus_128).
+chainerx::Array PlainCodes(const chainerx::Array& minus_128);
 
 class ChxVM {
 public:
@@ -66,6 +75,7 @@ private:
     std::vector<ChxVMTypeProto> input_types_;
     int num_variables_ = 0;
     int64_t residual_fusions_ = 0;
+    std::vector<bool> minus_128_slots_;  // per variable: see ChxVMState::store_minus_128
 };
 
 }  // namespace runtime

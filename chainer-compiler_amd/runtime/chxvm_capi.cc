@@ -294,6 +294,9 @@ int32_t chxvm_set_option(const char* name, const char* value) {
         } else if (n == "pair_convolutions") {
             CHECK(v == "on" || v == "off") << "pair_convolutions is 'on' or 'off', got " << v;
             SetPairConvolutions(v == "on");
+        } else if (n == "store_minus_128") {
+            CHECK(v == "on" || v == "off") << "store_minus_128 is 'on' or 'off', got " << v;
+            SetStoreMinus128(v == "on");
         } else if (n == "chrome_tracing") {
             g_chrome_tracing_path = v;
         } else if (n == "dump_outputs_dir") {
@@ -333,6 +336,7 @@ int64_t chxvm_counter(const char* name) {
     const std::string n = name ? name : "";
     if (n == "qlinearconv_residual_fusions") return QLinearConvResidualFusions();
     if (n == "qlinearconv_pair_fusions") return QLinearConvPairFusions();
+    if (n == "minus_128_stores") return Minus128Stores();
     return -1;
 }
 

@@ -93,6 +93,10 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
  * name "pair_convolutions": value "on" (default) or "off": whether two QLinearConv that read the same
  * value with the same strides, pads and kernel size (the main-path and the shortcut convolution of a
  * down-sampling block) run as one launch (decided when a program is loaded);
+ * name "store_minus_128": value "on" (default) or "off": whether a uint8 value that only unpadded QLinearConv
+ * read (as input, or as the residual operand of a sum computed inside one) is kept as code - 128 in an int8
+ * array between them, which spares the reading kernel its sign flips (decided when a program is loaded; a
+ * run with check_types or dump_outputs_dir stores plain codes);
  * name "chrome_tracing": value a file name; every later chxvm_program_run writes its
  * per-instruction timeline there in the Chrome tracing format (the device is synchronized after
  * each instruction while this is on), "" switches it off;
@@ -101,7 +105,7 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
 int32_t chxvm_set_option(const char* name, const char* value);
 /* Process-wide event counts.  name "qlinearconv_residual_fusions": runs of a QLinearConv that
  * computed the residual-sum group behind it inside its kernel; "qlinearconv_pair_fusions": pairs of
- * QLinearConv that ran as one launch.  Unknown names give -1. */
+ * QLinearConv that ran as one launch; "minus_128_stores": results written as code - 128.  Unknown names give -1. */
 int64_t chxvm_counter(const char* name);
 
 /* BackendConfig queries.  `config` is a built-in name ("chxvm", "chxvm_test", "hip") or, with

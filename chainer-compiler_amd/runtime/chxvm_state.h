@@ -126,6 +126,16 @@ public:
         ++residual_fusions_;
     }
 
+    // Whether the uint8 value of variable `slot` may be stored as code - 128 in an int8 array in this run (the
+    // program's analysis found only readers that take that storage, and no option of the run looks at raw values);
+    // an int8 array found in such a slot where the program's types say uint8 holds that storage.
+    bool store_minus_128(int slot) const {
+        return minus_128_slots_ && slot >= 0 && slot < static_cast<int>(minus_128_slots_->size()) && (*minus_128_slots_)[slot];
+    }
+    void set_minus_128_slots(const std::vector<bool>* slots) {
+        minus_128_slots_ = slots;
+    }
+
 private:
     void CheckNonFinite(const std::vector<int>& inputs, const std::vector<int>& outputs, bool infinities);
 
@@ -136,6 +146,7 @@ private:
     ChxVMOptions options_;
     QLinearConvResidualRequest* residual_request_ = nullptr;
     int64_t residual_fusions_ = 0;
+    const std::vector<bool>* minus_128_slots_ = nullptr;
 };
 
 }  // namespace runtime

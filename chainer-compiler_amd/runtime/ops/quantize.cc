@@ -14,6 +14,13 @@ namespace runtime {
 namespace {
 
 std::atomic<int64_t> g_residual_fusions{0};
+std::atomic<int64_t> g_minus_128_stores{0};
+
+// A uint8 value kept as code - 128 in an int8 array: what a producer leaves in a variable for which
+// ChxVMState::store_minus_128 holds.  Such an array is an int8 tensor with the zero point lowered by 128.
+bool HoldsCodesMinus128(ChxVMState* st, int slot, const chainerx::Array& a, chainerx::Dtype type_in_program) {
+    return st->store_minus_128(slot) && a.dtype() == chainerx::Dtype::kInt8 && type_in_program == chainerx::Dtype::kUInt8;
+}
 
 StrictScalar DefaultZeroPoint() {
     // an absent zero point is uint8 0 (runtime/ops/quantize.cc:50-51,57-58)
@@ -34,6 +41,20 @@ chainerx::Array EmptyLike4d(const chainerx::Array& x, const chainerx::Shape& sha
 
 int64_t QLinearConvResidualFusions() {
     return g_residual_fusions.load();
+}
+
+int64_t Minus128Stores() {
+    return g_minus_128_stores.load();
+}
+
+chainerx::Array PlainCodes(const chainerx::Array& minus_128) {
+    CHECK(minus_128.dtype() == chainerx::Dtype::kInt8);
+    const bool channels_last = minus_128.ndim() == 4 && !minus_128.IsContiguous() && minus_128.strides()[1] == minus_128.GetItemSize();
+    chainerx::Array plain = channels_last ? chainerx::EmptyChannelsLastPadded(minus_128.shape(), chainerx::Dtype::kUInt8)
+                                          : chainerx::Empty(minus_128.shape(), chainerx::Dtype::kUInt8);
+    chx_hip_tensor xt = minus_128.hip(), yt = plain.hip();
+    CHXVM_HIP_CALL(chx_hip_codes_minus_128(&xt, &yt, chainerx::CurrentStream()));
+    return plain;
 }
 
 chainerx::Array QuantizeLinearOp::RunImpl(
@@ -70,6 +91,7 @@ public:
     chx_hip_qconv_plan* plan = nullptr;
     chx_hip_conv_params params;
     chainerx::Array w, w_scale, w_zero_point, bias;  // what the plan was built from
+    bool minus_128_refused = false;  // the kernel that runs this plan does not write the minus-128 storage
 
     bool Matches(const chainerx::Array& q_w, const chainerx::Array& s, const chainerx::Array& z, const absl::optional<chainerx::Array>& b,
                  const chx_hip_conv_params& p) const {
@@ -86,6 +108,7 @@ public:
         chx_hip_qconv_plan_destroy(plan);
         plan = nullptr;
         w = w_scale = w_zero_point = bias = chainerx::Array();
+        minus_128_refused = false;
     }
 };
 
@@ -112,6 +135,8 @@ chainerx::Array QLinearConvOp::RunImpl(
     CHECK_EQ(w_scale.GetTotalSize(), w_zero_point.GetTotalSize());
     CHECK_EQ(w_scale.shape().size(), w_zero_point.shape().size());
     CheckQuantizedDtype(y_zero_point.dtype(), "QLinearConv y_zero_point");
+    // (an input kept as code - 128 is an int8 tensor with the zero point 128 lower: every kernel takes it as that)
+    const int32_t x_zp = static_cast<int32_t>(static_cast<int64_t>(x_zero_point)) - (HoldsCodesMinus128(st, this->x, q_x, x_zero_point.dtype()) ? 128 : 0);
     if (q_x.ndim() != 4) {
         // one or three spatial axes: the rank-generic entry point, operands as they are, a dense result
         chainerx::Shape nd_shape;
@@ -122,7 +147,7 @@ chainerx::Array QLinearConvOp::RunImpl(
         chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), yt = y.hip(), bt;
         if (b.has_value()) bt = b->hip();
         CHXVM_HIP_CALL(chx_hip_qlinear_conv_nd(
-                &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &wt, &st2, &zt,
+                &xt, static_cast<float>(x_scale), x_zp, &wt, &st2, &zt,
                 static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), b.has_value() ? &bt : nullptr, &np,
                 nd_flags, &yt, chainerx::CurrentStream()));
         return y;
@@ -141,7 +166,7 @@ chainerx::Array QLinearConvOp::RunImpl(
         chx_hip_tensor xt = q_x.hip(), wt = q_w.hip(), st2 = w_scale.hip(), zt = w_zero_point.hip(), yt = y.hip(), bt;
         if (b.has_value()) bt = b->hip();
         CHXVM_HIP_CALL(chx_hip_qlinear_conv(
-                &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), &wt, &st2, &zt,
+                &xt, static_cast<float>(x_scale), x_zp, &wt, &st2, &zt,
                 static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), b.has_value() ? &bt : nullptr, &p,
                 flags, &yt, chainerx::CurrentStream()));
         return y;
@@ -166,28 +191,49 @@ chainerx::Array QLinearConvOp::RunImpl(
         const bool same_quantization = static_cast<float>(y_scale) == req->y_scale &&
                                        static_cast<int64_t>(y_zero_point) == req->y_zero_point && y_zero_point.dtype() == req->y_dtype;
         if (same_quantization && !req->r.IsNullHandle() && req->r.shape() == y_shape) {
-            chainerx::Array out = chainerx::EmptyChannelsLastPadded(y_shape, req->out_dtype);
-            chx_hip_tensor xt = q_x.hip(), rt = req->r.hip(), ot = out.hip();
-            const int rc = chx_hip_qconv_plan_run_add(
-                    impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
-                    req->y_scale, req->y_zero_point, static_cast<int32_t>(req->y_dtype), flags, &rt, req->r_scale, req->r_zero_point,
-                    req->out_scale, req->out_zero_point, req->relu ? 1 : 0, &ot, chainerx::CurrentStream());
-            if (rc == CHX_HIP_OK) {
-                req->out = out;
-                req->done = true;
-                ++g_residual_fusions;
-                st->count_residual_fusion();
-                return chainerx::Array();
+            // the sum in the minus-128 storage where its variable allows it; the kernel's refusal of that storage
+            // (remembered) is not a refusal of the sum
+            const bool minus_128 = st->store_minus_128(req->out_slot) && req->out_dtype == chainerx::Dtype::kUInt8 && !impl_->minus_128_refused;
+            for (int attempt = minus_128 ? 0 : 1; attempt < 2; ++attempt) {
+                const bool signed_storage = attempt == 0;
+                chainerx::Array out = chainerx::EmptyChannelsLastPadded(y_shape, signed_storage ? chainerx::Dtype::kInt8 : req->out_dtype);
+                chx_hip_tensor xt = q_x.hip(), rt = req->r.hip(), ot = out.hip();
+                const int rc = chx_hip_qconv_plan_run_add(
+                        impl_->plan, &xt, static_cast<float>(x_scale), x_zp, req->y_scale, req->y_zero_point, static_cast<int32_t>(req->y_dtype),
+                        flags | (signed_storage ? CHX_HIP_STORE_MINUS_128 : 0u), &rt, req->r_scale, req->r_zero_point, req->out_scale,
+                        req->out_zero_point, req->relu ? 1 : 0, &ot, chainerx::CurrentStream());
+                if (rc == CHX_HIP_OK) {
+                    req->out = out;
+                    req->done = true;
+                    ++g_residual_fusions;
+                    if (signed_storage) ++g_minus_128_stores;
+                    st->count_residual_fusion();
+                    return chainerx::Array();
+                }
+                CHECK_EQ(CHX_HIP_EUNSUPPORTED, rc) << chx_hip_last_error();  // unsupported: run the ops one by one
+                if (signed_storage) impl_->minus_128_refused = true;
             }
-            CHECK_EQ(CHX_HIP_EUNSUPPORTED, rc) << chx_hip_last_error();  // unsupported: run the ops one by one
         }
     }
     // 8-bit activations leave a convolution channels-last, whatever layout came in
+    if (st->store_minus_128(this->y) && y_zero_point.dtype() == chainerx::Dtype::kUInt8 && !impl_->minus_128_refused) {
+        chainerx::Array y_minus_128 = chainerx::EmptyChannelsLastPadded(y_shape, chainerx::Dtype::kInt8);
+        chx_hip_tensor xt = q_x.hip(), yt = y_minus_128.hip();
+        const int rc = chx_hip_qconv_plan_run(
+                impl_->plan, &xt, static_cast<float>(x_scale), x_zp, static_cast<float>(y_scale),
+                static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags | CHX_HIP_STORE_MINUS_128, &yt, chainerx::CurrentStream());
+        if (rc == CHX_HIP_OK) {
+            ++g_minus_128_stores;
+            return y_minus_128;
+        }
+        CHECK_EQ(CHX_HIP_EUNSUPPORTED, rc) << chx_hip_last_error();  // a kernel that writes plain codes only
+        impl_->minus_128_refused = true;
+    }
     chainerx::Array y = chainerx::EmptyChannelsLastPadded(y_shape, y_zero_point.dtype());
     chx_hip_tensor xt = q_x.hip(), yt = y.hip();
     CHXVM_HIP_CALL(chx_hip_qconv_plan_run(
-            impl_->plan, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)),
-            static_cast<float>(y_scale), static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, chainerx::CurrentStream()));
+            impl_->plan, &xt, static_cast<float>(x_scale), x_zp, static_cast<float>(y_scale),
+            static_cast<int32_t>(static_cast<int64_t>(y_zero_point)), flags, &yt, chainerx::CurrentStream()));
     return y;
 }
 
@@ -320,13 +366,19 @@ private:
         const uint32_t flags =
                 CHX_HIP_ROUND_REFERENCE | (st->options().qlinearconv_onnx_int32_bias ? CHX_HIP_BIAS_ONNX_INT32 : CHX_HIP_BIAS_REFERENCE_FLOAT);
         chainerx::Shape y1_shape = ConvOutputShape(x, oa.w, p), y2_shape = ConvOutputShape(x, ob.w, p);
-        chainerx::Array y1 = chainerx::EmptyChannelsLastPadded(y1_shape, y1_zero_point.dtype());
-        chainerx::Array y2 = chainerx::EmptyChannelsLastPadded(y2_shape, y2_zero_point.dtype());
+        const int32_t x_zp = static_cast<int32_t>(static_cast<int64_t>(x_zero_point)) - (HoldsCodesMinus128(st, a_->x, x, x_zero_point.dtype()) ? 128 : 0);
+        // each result in the minus-128 storage where its variable allows it
+        const bool s1 = st->store_minus_128(a_->y) && y1_zero_point.dtype() == chainerx::Dtype::kUInt8;
+        const bool s2 = st->store_minus_128(b_->y) && y2_zero_point.dtype() == chainerx::Dtype::kUInt8;
+        chainerx::Array y1 = chainerx::EmptyChannelsLastPadded(y1_shape, s1 ? chainerx::Dtype::kInt8 : y1_zero_point.dtype());
+        chainerx::Array y2 = chainerx::EmptyChannelsLastPadded(y2_shape, s2 ? chainerx::Dtype::kInt8 : y2_zero_point.dtype());
         chx_hip_tensor xt = x.hip(), y1t = y1.hip(), y2t = y2.hip();
         const int rc = chx_hip_qconv_plan_run_pair(
-                plan_, &xt, static_cast<float>(x_scale), static_cast<int32_t>(static_cast<int64_t>(x_zero_point)), static_cast<int32_t>(oc1),
-                static_cast<float>(y1_scale), static_cast<int32_t>(static_cast<int64_t>(y1_zero_point)), flags, &y1t,
-                static_cast<float>(y2_scale), static_cast<int32_t>(static_cast<int64_t>(y2_zero_point)), flags, &y2t, chainerx::CurrentStream());
+                plan_, &xt, static_cast<float>(x_scale), x_zp, static_cast<int32_t>(oc1), static_cast<float>(y1_scale),
+                static_cast<int32_t>(static_cast<int64_t>(y1_zero_point)), flags | (s1 ? CHX_HIP_STORE_MINUS_128 : 0u), &y1t,
+                static_cast<float>(y2_scale), static_cast<int32_t>(static_cast<int64_t>(y2_zero_point)),
+                flags | (s2 ? CHX_HIP_STORE_MINUS_128 : 0u), &y2t, chainerx::CurrentStream());
+        if (rc == CHX_HIP_OK) g_minus_128_stores += (s1 ? 1 : 0) + (s2 ? 1 : 0);
         if (rc == CHX_HIP_EUNSUPPORTED) {
             // layouts or weights the one-launch kernel does not take: remembered, so that the weights are not joined again
             chx_hip_qconv_plan_destroy(plan_);

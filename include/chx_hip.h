@@ -434,6 +434,12 @@ int chx_hip_count_nonfinite(const chx_hip_tensor* x, int32_t infinities, int64_t
  * int32, uint8, int8 on either side; float -> integer truncates toward zero. */
 int chx_hip_cast(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream);
 
+/* Moves 8-bit codes between the two storages that CHX_HIP_STORE_MINUS_128 distinguishes; it has no counterpart
+ * in the reference, whose uint8 tensors have one storage.  x uint8, y int8: y = code - 128; x int8, y uint8:
+ * y = code + 128 (either way bit 7 of every byte inverted).  Same shape, any strides.  A runtime that keeps
+ * some values in the minus-128 storage uses it when such a value reaches a reader that wants plain codes. */
+int chx_hip_codes_minus_128(const chx_hip_tensor* x, chx_hip_tensor* y, void* stream);
+
 /* Says whether a fusion program (the `code` of an ElementWiseNvrtc instruction, emitted per
  * FusionGroup by compiler/chxvm/emitter.cc:621-729) is exactly the residual sum of a quantized
  * network,  out = QuantizeLinear(act(DequantizeLinear(in0) + DequantizeLinear(in1)))  with

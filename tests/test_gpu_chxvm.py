@@ -202,10 +202,11 @@ def test_errors_name_the_instruction(g, vm):
         vm.Program(b.serialize()).run({"x": g.dev(np.zeros(4, np.float32))})
 
 
-def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None, paired=None):
+def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None, paired=None, minus_128=None):
     wl = g.pkg.workloads
     before = vm.counter("qlinearconv_residual_fusions")
     pairs_before = vm.counter("qlinearconv_pair_fusions")
+    stores_before = vm.counter("minus_128_stores")
     serialized = wl.program_to_chxvm(model, vm, g.pkg.ops, keep=keep).serialize()
     assert vm.proto_roundtrip(serialized) == serialized
     vm.set_option("qlinearconv_bias", "onnx_int32")
@@ -227,6 +228,8 @@ def _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=None, pa
         assert vm.counter("qlinearconv_residual_fusions") - before == fused_residuals
     if paired is not None:
         assert vm.counter("qlinearconv_pair_fusions") - pairs_before == paired
+    if minus_128 is not None:
+        assert vm.counter("minus_128_stores") - stores_before == minus_128
 
 
 def test_small_resnet_as_one_program(g, vm, oracle):
@@ -240,18 +243,33 @@ def test_small_resnet_as_one_program(g, vm, oracle):
     pairs = sum(1 for ins in wl.pair_convolutions(model["program"], model["convs"]) if ins[0] == "QLinearConvPair")
     assert pairs == 2
     # every value is a program output: nothing may be absorbed into another instruction
-    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0, paired=pairs)
+    # (a program output is read as plain codes: no value is kept as code - 128)
+    _run_network_through_vm(g, vm, oracle, model, [ins[1] for ins in model["program"]], fused_residuals=0, paired=pairs, minus_128=0)
     # only the logits: each of the five residual sums is computed by the convolution before it
     blocks = sum(1 for ins in model["program"] if ins[0] == "AddRelu")
     assert blocks == 5
-    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks, paired=pairs)
-    # the block outputs too: the sums are still absorbed (their convolutions' results are not outputs)
+    # The values only unpadded convolutions read (as input or as the residual operand of an absorbed sum) are kept as
+    # code - 128: what the Python runner's analysis finds on the same program with the same fusions.
+    runner = wl.DeviceRunner(model, g.pkg, fuse_residual=True, pair_convs=True, minus_128=True)
+    kept_minus_128 = len(runner.minus_128)
+    runner.close()
+    assert kept_minus_128 >= 8
+    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks, paired=pairs, minus_128=kept_minus_128)
+    # the block outputs too: the sums are still absorbed (their convolutions' results are not outputs), and come out
+    # as plain codes
     keep = ["logits"] + [ins[1] for ins in model["program"] if ins[0] == "AddRelu"]
     _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=blocks, paired=pairs)
+    vm.set_option("store_minus_128", "off")
+    try:
+        _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=blocks, paired=pairs, minus_128=0)
+    finally:
+        vm.set_option("store_minus_128", "on")
+    # residual sums as instructions of their own: the operand a sum reads is then not one only convolutions read
     vm.set_option("fuse_residual", "off")
     vm.set_option("pair_convolutions", "off")
     try:
         _run_network_through_vm(g, vm, oracle, model, keep, fused_residuals=0, paired=0)
+        _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=0, paired=0)
     finally:
         vm.set_option("fuse_residual", "on")
         vm.set_option("pair_convolutions", "on")
@@ -300,6 +318,57 @@ def test_residual_group_with_other_constants_runs_unfused(g, vm, oracle):
         conv = oracle.qlinear_conv_int(x, 0.02, 128, w, ws, np.zeros(32, np.int8), np.float32(0.25), 120, np.uint8)
         s_ = oracle.binary(oracle.ADD, oracle.dequantize_linear(r, 0.1, 3), oracle.dequantize_linear(conv, group_scale, 120))
         np.testing.assert_array_equal(got, oracle.quantize_linear(s_, 0.3, 100, np.uint8))
+
+
+def test_value_kept_minus_128_reaches_a_group_that_runs_unfused(g, vm, oracle):
+    """A value only convolutions read is kept as code - 128; when the residual sum that reads it is, at run time, not
+    the convolution's to compute after all (other constants), the group instruction gets plain codes back."""
+    rng = np.random.default_rng(78)
+    x = rand_q(rng, (2, 16, 6, 5), np.uint8)
+    w0 = rng.integers(-127, 128, size=(32, 16, 1, 1)).astype(np.int8)
+    w1 = rng.integers(-127, 128, size=(32, 32, 1, 1)).astype(np.int8)
+    ws0 = rng.uniform(0.002, 0.01, size=32).astype(np.float32)
+    ws1 = rng.uniform(0.002, 0.01, size=32).astype(np.float32)
+    zeros = np.zeros(32, np.int8)
+    u8 = torch.uint8
+
+    def scale_bits(v):
+        return "0x%08x" % np.float32(v).view(np.uint32)
+    for group_scale, fused in ((0.25, 1), (0.26, 0)):
+        code = g.ops.fusion_program(
+            [("a", u8), ("b", u8)],
+            [("fa", "DequantizeLinear", "a", scale_bits(group_scale), 120), ("fb", "DequantizeLinear", "b", scale_bits(0.1), 3),
+             ("s", "Add", "fb", "fa"), ("q", "QuantizeLinear", "s", scale_bits(0.3), 100, "uint8")], [("q", u8)])
+        b = vm.ProgramBuilder()
+        xs = b.input("x", "uint8", x.shape)
+        r = b.QLinearConv(xs, b.scalar(0.02, "float32"), b.scalar(128, "uint8"), b.constant(w0), b.constant(ws0), b.constant(zeros),
+                          b.scalar(0.1, "float32"), b.scalar(3, "uint8"), None, [1, 1], [0, 0], 1, "")
+        y = b.QLinearConv(r, b.scalar(0.1, "float32"), b.scalar(3, "uint8"), b.constant(w1), b.constant(ws1), b.constant(zeros),
+                          b.scalar(0.25, "float32"), b.scalar(120, "uint8"), None, [1, 1], [0, 0], 1, "")
+        out = b.ElementWiseNvrtc([y, r], 1, code, 7, num_list_outputs=1)[0]
+        b.Free(y)
+        b.Free(r)
+        b.output("out", out)
+        fusions, stores = vm.counter("qlinearconv_residual_fusions"), vm.counter("minus_128_stores")
+        prog = vm.Program(b.serialize())
+        got = prog.run({"x": g.to_channels_last(g.dev(x))})["out"]
+        prog.close()
+        assert vm.counter("qlinearconv_residual_fusions") - fusions == fused
+        assert vm.counter("minus_128_stores") - stores == 1   # r; `out` is read by the caller
+        rv = oracle.qlinear_conv_int(x, 0.02, 128, w0, ws0, zeros, np.float32(0.1), 3, np.uint8)
+        conv = oracle.qlinear_conv_int(rv, 0.1, 3, w1, ws1, zeros, np.float32(0.25), 120, np.uint8)
+        s_ = oracle.binary(oracle.ADD, oracle.dequantize_linear(rv, 0.1, 3), oracle.dequantize_linear(conv, group_scale, 120))
+        np.testing.assert_array_equal(got, oracle.quantize_linear(s_, 0.3, 100, np.uint8))
+    # with type checks on, the run keeps plain codes (the program's types say uint8)
+    stores = vm.counter("minus_128_stores")
+    prog = vm.Program(b.serialize())
+    vm.set_option("check_types", "on")
+    try:
+        prog.run({"x": g.to_channels_last(g.dev(x))})
+    finally:
+        vm.set_option("check_types", "off")
+    prog.close()
+    assert vm.counter("minus_128_stores") == stores
 
 
 def test_unfused_pools_run_as_float_ops(g, vm, oracle):

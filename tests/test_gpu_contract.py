@@ -804,3 +804,28 @@ def test_convolutions_over_one_and_three_spatial_axes(g, oracle):
             np.testing.assert_array_equal(g.host(goti)[:, :, od], wanti)
     with pytest.raises(g.capi.ChxHipError):
         g.ops.ConvInteger(g.dev(rand_q(rng, (1, 2, 3, 3, 3, 3), np.uint8)), g.dev(rand_q(rng, (1, 2, 1, 1, 1, 1), np.int8)))
+
+
+def test_codes_minus_128_both_ways(g):
+    """chx_hip_codes_minus_128: uint8 -> int8 is code - 128, int8 -> uint8 code + 128, through any strides; other
+    pairs of types and differing shapes are refused."""
+    rng = np.random.default_rng(152)
+    u = rng.integers(0, 256, size=(3, 5, 7, 16)).astype(np.uint8)
+    want = (u.astype(np.int16) - 128).astype(np.int8)
+    du = torch.from_numpy(u).cuda()
+    s = g.ops.codes_minus_128(du)
+    assert s.dtype == torch.int8
+    np.testing.assert_array_equal(s.cpu().numpy(), want)
+    np.testing.assert_array_equal(g.ops.codes_minus_128(s).cpu().numpy(), u)
+    # channels-last source, dense destination; a sliced destination
+    cl = du.permute(0, 3, 1, 2)
+    np.testing.assert_array_equal(g.ops.codes_minus_128(cl.contiguous(memory_format=torch.channels_last)).cpu().numpy(), want.transpose(0, 3, 1, 2))
+    wide = torch.zeros((3, 5, 7, 32), dtype=torch.int8, device="cuda")
+    g.ops.codes_minus_128(du, out=wide[..., 8:24])
+    np.testing.assert_array_equal(wide[..., 8:24].cpu().numpy(), want)
+    assert not wide[..., :8].any() and not wide[..., 24:].any()
+    assert g.ops.codes_minus_128(torch.empty((0, 4), dtype=torch.uint8, device="cuda")).shape == (0, 4)
+    for bad_out in (torch.empty_like(du), torch.empty((3, 5, 7, 16), dtype=torch.int32, device="cuda"),
+                    torch.empty((3, 5, 7, 8), dtype=torch.int8, device="cuda")):
+        with pytest.raises(g.capi.ChxHipError):
+            g.ops.codes_minus_128(du, out=bad_out)
