@@ -496,7 +496,7 @@ def set_option(name, value):
     "fuse_residual" = "on" (default) | "off" (applies to programs loaded afterwards);
     "pair_convolutions" = "on" (default) | "off": two QLinearConv of one value with the same geometry as one launch
     (applies to programs loaded afterwards);
-    "store_minus_128" = "on" (default) | "off": uint8 values that only unpadded QLinearConv read are kept as
+    "store_minus_128" = "on" (default) | "off": uint8 values that only QLinearConv with pads of at most 1 read are kept as
     code - 128 in int8 arrays between them (applies to programs loaded afterwards);
     "chrome_tracing" = file that every later run writes its per-instruction timeline to, "" = off;
     "dump_outputs_dir" = directory that every later run writes the instructions' named array

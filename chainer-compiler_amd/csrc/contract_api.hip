@@ -176,6 +176,7 @@ inline int round_up(int v, int m) {
 struct PackedWeights {
     int8_t* wp = nullptr;
     int32_t* wsum = nullptr;
+    int32_t* padsum = nullptr;  // ConvMfmaArgs::padsum (inside wsum's allocation), null for dense packing and for more than 32 taps
     int C64 = 0, OCpad = 0, KP = 0;
     int BK = 64;         // K bytes per kernel step; the packed layout depends on it
     bool dense = false;  // taps packed densely; activations go through an explicit im2col
@@ -613,6 +614,8 @@ int run_conv_mfma(const ConvCall& c, const PackedWeights& pw, hipStream_t s) {
     a.nk = pw.KP / pw.BK;
     a.wp = pw.wp;
     a.wsum = pw.wsum;
+    a.padsum = pw.padsum;
+    a.padsum_stride = pw.OCpad;
     a.x_zp = c.x_zp;
     const bool xu = x.dtype == CHX_HIP_UINT8;
     a.corr_mult = xu ? 128 - c.x_zp : -c.x_zp;
@@ -694,27 +697,31 @@ int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedW
     const size_t stem_bytes =
             stem ? (size_t)(pw->OCpad / 64) * stem_k_blocks((int)w.shape[1], (int)w.shape[2], (int)w.shape[3]) * 2048 : 0;
     const size_t bytes = mfma_bytes + stem_bytes;
+    // the per-channel sums, and behind them the sixteen classes of border sums
+    const bool border_sums = !pw->dense && w.shape[2] * w.shape[3] <= 32;
+    const size_t sums_bytes = sizeof(int32_t) * pw->OCpad * (border_sums ? 17 : 1);
     void* p0 = nullptr;
     void* p1 = nullptr;
     if (persistent) {
         CHX_HIP_CALL(hipMalloc(&p0, bytes));
-        if (hipMalloc(&p1, sizeof(int32_t) * pw->OCpad) != hipSuccess) {
+        if (hipMalloc(&p1, sums_bytes) != hipSuccess) {
             (void)hipFree(p0);
             CHX_FAIL(CHX_HIP_ERUNTIME, "hipMalloc failed for the per-channel weight sums");
         }
     } else {
         CHX_PROPAGATE(scratch_alloc(&p0, bytes, s));
-        if (scratch_alloc(&p1, sizeof(int32_t) * pw->OCpad, s) != CHX_HIP_OK) {
+        if (scratch_alloc(&p1, sums_bytes, s) != CHX_HIP_OK) {
             scratch_free(p0, s);
             return CHX_HIP_ERUNTIME;
         }
     }
     pw->wp = static_cast<int8_t*>(p0);
     pw->wsum = static_cast<int32_t*>(p1);
+    pw->padsum = border_sums ? pw->wsum + pw->OCpad : nullptr;
     pw->wd = stem ? pw->wp + mfma_bytes : nullptr;
     if (stem) CHX_PROPAGATE(pack_weights_stem(w, pw->OCpad, pw->wd, s));
     if (pw->dense) return pack_weights_dense(w, pw->KP, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
-    return pack_weights(w, pw->C64, pw->BK, pw->OCpad, pw->wp, pw->wsum, s);
+    return pack_weights(w, pw->C64, pw->BK, pw->OCpad, pw->wp, pw->wsum, pw->padsum, s);
 }
 
 void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
@@ -727,6 +734,7 @@ void release_packed(PackedWeights* pw, bool persistent, hipStream_t s) {
     }
     pw->wp = nullptr;
     pw->wsum = nullptr;
+    pw->padsum = nullptr;
     pw->wd = nullptr;
 }
 

@@ -56,8 +56,15 @@ struct ConvMfmaArgs {
     int32_t KP;   // packed row length: KH * KW * C64
     const int8_t* wp;     // [OCpad / 64][nk][64][bk]
     const int32_t* wsum;  // [OCpad]
+    // [16][OCpad]: the sum of a filter's weights over the taps of its first row (class bit 3), last row (bit 2), first
+    // column (bit 1) and last column (bit 0), each tap once: what a pixel whose window leaves the image on those sides
+    // misses when the taps outside arrive as zeros (pack_weights); null when the packing did not compute it
+    const int32_t* padsum;
+    int32_t padsum_stride;  // channels per class of padsum
     int32_t x_zp;
     int32_t corr_mult;    // (128 - x_zp) for uint8 x, (-x_zp) for int8 x
+    int32_t tap_corr;     // not 0: taps outside the image arrive as zeros although the zero point is not the byte 0, and the accumulators start from the pixel's class of padsum; the number of classes other than 0 that occur (launcher)
+    uint64_t tap_classes; // those classes, four bits each from bit 0 up (launcher)
     // output, pixel-major: element (m, oc) at y + m*y_px_stride + oc*elemsize
     char* y;
     int64_t y_px_stride;
@@ -140,7 +147,7 @@ inline void magic_divisor(uint32_t d, uint32_t* mul, uint32_t* shift) {
 
 int pack_weights_dense(const chx_hip_tensor& w, int Kd, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
 int launch_im2col_dense(const Im2colArgs& a, hipStream_t s);
-int pack_weights(const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s);
+int pack_weights(const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, int32_t* padsum, hipStream_t s);
 // the stem kernel: weights [C][KH][KW] with C*KH <= 32 and KW <= 8; patch = LDS bytes of a tile's input rows
 bool stem_shape_fits(int C, int KH, int KW);
 bool stem_patch_fits(int C, int KH, int KW, int sh, int sw);

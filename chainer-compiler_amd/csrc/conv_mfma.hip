@@ -48,12 +48,16 @@ __host__ __device__ __forceinline__ int64_t packed_offset(int oc, int k, int KP,
 // ---------------------------------------------------------------------------------------------
 // Weight repacking: w [OC][C][KH][KW] (any strides) -> Wp, K index k = (kh*KW + kw)*C64 + c with
 // C64 = C rounded up to 64 (zero filled), and wsum[oc] = sum of the row.  One work-group per
-// output channel.
+// output channel.  padsum (when not null; at most 32 taps): [16][gridDim.x] sums of the row over the taps of the
+// filter's border rows and columns that the class names (ConvMfmaArgs::padsum).
 __global__ __launch_bounds__(256) void pack_weights_kernel(
         const char* __restrict__ w, int64_t s_oc, int64_t s_c, int64_t s_kh, int64_t s_kw, int OC, int C, int KH, int KW,
-        int C64, int BK, int8_t* __restrict__ wp, int32_t* __restrict__ wsum) {
+        int C64, int BK, int8_t* __restrict__ wp, int32_t* __restrict__ wsum, int32_t* __restrict__ padsum) {
     const int oc = blockIdx.x;
     const int KP = KH * KW * C64;
+    __shared__ int32_t tap_sum[32];
+    if (threadIdx.x < 32) tap_sum[threadIdx.x] = 0;
+    __syncthreads();
     int32_t local = 0;
     for (int k = threadIdx.x; k < KP; k += 256) {
         const int c = k % C64;
@@ -65,6 +69,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
         }
         wp[packed_offset(oc, k, KP, BK)] = v;
         local += v;
+        if (padsum && v != 0) atomicAdd(&tap_sum[pos], (int32_t)v);
     }
     __shared__ int32_t red[256];
     red[threadIdx.x] = local;
@@ -74,6 +79,16 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
         __syncthreads();
     }
     if (threadIdx.x == 0) wsum[oc] = red[0];
+    if (padsum && threadIdx.x < 16) {
+        const int cls = threadIdx.x;
+        int32_t sum = 0;
+        for (int i = 0; i < KH; ++i)
+            for (int j = 0; j < KW; ++j) {
+                const bool outside = ((cls & 8) && i == 0) || ((cls & 4) && i == KH - 1) || ((cls & 2) && j == 0) || ((cls & 1) && j == KW - 1);
+                if (outside) sum += tap_sum[i * KW + j];
+            }
+        padsum[(int64_t)cls * gridDim.x + oc] = sum;
+    }
 }
 
 // Few input channels (the 3-channel stem): padding each filter tap to 64 K-bytes would waste
@@ -220,10 +235,10 @@ __global__ __launch_bounds__(256) void im2col_dense_lds_kernel(Im2colArgs a, int
 }  // namespace
 
 int pack_weights(
-        const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, hipStream_t s) {
+        const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, int32_t* padsum, hipStream_t s) {
     pack_weights_kernel<<<OCpad, 256, 0, s>>>(
             static_cast<const char*>(w.data), w.strides[0], w.strides[1], w.strides[2], w.strides[3], (int)w.shape[0],
-            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, BK, wp, wsum);
+            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, BK, wp, wsum, w.shape[2] * w.shape[3] <= 32 ? padsum : nullptr);
     return launch_check("pack_weights_kernel");
 }
 

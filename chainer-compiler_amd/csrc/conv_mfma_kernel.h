@@ -52,21 +52,22 @@ template <int BYTES>
 __device__ __forceinline__ void warm_kernel_arguments() {
     const uint64_t ka = (uint64_t)__builtin_amdgcn_kernarg_segment_ptr();
     constexpr int LINES = (BYTES + 63) / 64;
-    static_assert(LINES >= 4 && LINES <= 7, "between four and seven lines are touched");
+    static_assert(LINES >= 4 && LINES <= 8, "between four and eight lines are touched");
     // offsets of the last lines, clamped into the block so that nothing outside it is read
-    constexpr int L4 = LINES > 4 ? 0x100 : 0xc0, L5 = LINES > 5 ? 0x140 : L4, L6 = LINES > 6 ? 0x180 : L5;
-    int t0, t1, t2, t3, t4, t5, t6;
+    constexpr int L4 = LINES > 4 ? 0x100 : 0xc0, L5 = LINES > 5 ? 0x140 : L4, L6 = LINES > 6 ? 0x180 : L5, L7 = LINES > 7 ? 0x1c0 : L6;
+    int t0, t1, t2, t3, t4, t5, t6, t7;
     asm volatile(
-            "s_load_dword %0, %7, 0x0\n\t"
-            "s_load_dword %1, %7, 0x40\n\t"
-            "s_load_dword %2, %7, 0x80\n\t"
-            "s_load_dword %3, %7, 0xc0\n\t"
-            "s_load_dword %4, %7, %8\n\t"
-            "s_load_dword %5, %7, %9\n\t"
-            "s_load_dword %6, %7, %10\n\t"
+            "s_load_dword %0, %8, 0x0\n\t"
+            "s_load_dword %1, %8, 0x40\n\t"
+            "s_load_dword %2, %8, 0x80\n\t"
+            "s_load_dword %3, %8, 0xc0\n\t"
+            "s_load_dword %4, %8, %9\n\t"
+            "s_load_dword %5, %8, %10\n\t"
+            "s_load_dword %6, %8, %11\n\t"
+            "s_load_dword %7, %8, %12\n\t"
             "s_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6)
-            : "s"(ka), "n"(L4), "n"(L5), "n"(L6)
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            : "s"(ka), "n"(L4), "n"(L5), "n"(L6), "n"(L7)
             : "memory");
 }
 
@@ -144,7 +145,10 @@ __device__ __forceinline__ int row_swizzle(int row) {
 // mask of its taps (computed once per pixel tile).  1: at most 32 taps and the activation zero point is the byte 0, so
 // a tap outside the image is fetched from outside the resource (one shift and one and-or on the
 // lane's offset): zeros contribute (0 - 0) * w, the reference's zero padding of the already
-// zero-point-subtracted tensor.  2: any zero point; the pixel copies use flat addresses and fetch
+// zero-point-subtracted tensor.  With another zero point z each such zero stands for a z and the sum misses z * w
+// per tap outside: the accumulators of a pixel then start from z times the sum of the weights of its taps outside
+// (ConvMfmaArgs::tap_corr; the copy side leaves each staged pixel's class of taps in LDS, the seeding reads it).
+// 2: any zero point, any window; the pixel copies use flat addresses and fetch
 // an invalid chunk from a 64-byte row holding the zero point instead (g_fill_rows).
 //
 // NWN: wavefronts along the pixel axis (two along the output channels).  2: four wavefronts, two
@@ -171,7 +175,11 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
     static_assert(TN * TM <= STAGE_BYTES, "the output tile is staged in one ring slot");
     __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) float s_scale[TM];
-    __shared__ __attribute__((aligned(16))) int32_t s_add[TM];
+    // what the accumulators start from, per output channel; kPad 1: sixteen rows, one per class of taps outside the image
+    // (ConvMfmaArgs::padsum), row 0 for a pixel whose taps are all inside, and each staged pixel's class
+    constexpr int ADD_ROW = TM + 8;  // (rows 32 bytes off a multiple of the bank width: lanes that read different rows do not meet on a bank)
+    __shared__ __attribute__((aligned(16))) int32_t s_add[kPad == 1 ? 16 * ADD_ROW : TM];
+    __shared__ int32_t s_cls[kPad == 1 ? TN : 1];
     __shared__ __attribute__((aligned(16))) float s_fbias[TM];
 
     warm_kernel_arguments<sizeof(ConvMfmaArgs)>();
@@ -272,6 +280,11 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                         const uint32_t below_hi = hi_bit >= 32 ? ~0u : (1u << hi_bit) - 1u;
                         const uint32_t rows = r_hi > r_lo ? below_hi & ~((1u << lo_bit) - 1u) : 0u;
                         mask = (cols * a.row_unit) & rows;
+                        if constexpr (kPad == 1) {
+                            // which sides the window leaves the image on (at most one row or column per side: the launcher
+                            // has checked); every lane of the row writes the same word
+                            s_cls[rowB] = a.tap_corr ? r_lo * 8 + (a.KH - r_hi) * 4 + c_lo * 2 + (a.KW - c_hi) : 0;
+                        }
                     } else {
                         const uint64_t below_hi = c_hi >= 64 ? ~(uint64_t)0 : ((uint64_t)1 << c_hi) - 1;  // a 1x64 filter fills the mask
                         const uint64_t cols = c_hi > c_lo ? below_hi & ~(((uint64_t)1 << c_lo) - 1) : 0;
@@ -372,6 +385,25 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         keep_scalar(tap);
     };
 
+    // kPad 1 with a zero point that is not the byte 0: the sums over the border taps of each class in use
+    // (a.tap_classes: their numbers, four bits each; a.tap_corr: how many), requested first of all so that they travel
+    // together with the first copies.  The T / TM threads of an output channel share the classes out (a wavefront
+    // holds one share); every instruction here delays the work-group's first matrix instruction.
+    constexpr int SHARES = T / TM;
+    constexpr int SHARE_MAX = (15 + SHARES - 1) / SHARES;
+    static_assert(T % TM == 0 && TM % 64 == 0, "whole wavefronts per share of the classes");
+    int32_t border[SHARE_MAX];
+    if constexpr (kPad == 1) {
+        if (a.tap_corr) {
+            const int share = __builtin_amdgcn_readfirstlane(tid / TM);
+            const int32_t* mine = a.padsum + min(oc0 + tid % TM, a.OC - 1);
+#pragma unroll
+            for (int k = 0; k < SHARE_MAX; ++k) {
+                border[k] = 0;
+                if (k * SHARES + share < a.tap_corr) border[k] = mine[(int64_t)((a.tap_classes >> (4 * (k * SHARES + share))) & 15) * a.padsum_stride];
+            }
+        }
+    }
     // the first NS-1 stages go out before anything else touches memory; the weight rows of the very first one
     // do not wait for the pixel addresses
     issue_weights(std::integral_constant<int, 0>(), std::integral_constant<int, CA>());
@@ -385,8 +417,11 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
         advance_stage();
     }
 
-    // per-channel epilogue constants; s_add seeds the accumulators
-    for (int i = tid; i < TM; i += T) {
+    // per-channel epilogue constants; s_add seeds the accumulators.  One thread per output channel; with class rows
+    // to fill (kPad 1, see `border`) every share of the threads works the channel's constant out for itself.
+    const bool all_shares = kPad == 1 && a.tap_corr;
+    if (tid < TM || all_shares) {
+        const int i = tid % TM;
         const int oc = oc0 + i;
         float sc = 0.f, fb = 0.f;
         int32_t add = 0;
@@ -401,9 +436,22 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                 }
             }
         }
-        s_scale[i] = sc;
-        s_add[i] = add;
-        s_fbias[i] = fb;
+        if (tid < TM) {
+            s_scale[i] = sc;
+            s_add[i] = add;
+            s_fbias[i] = fb;
+        }
+        if constexpr (kPad == 1) {
+            // taps outside the image arrive as the byte 0 where the tensor would hold the zero point: each contributes
+            // w * x_zp too little.  Row c of s_add = row 0 + x_zp * the border sums of class c.
+            if (a.tap_corr) {
+                const int share = __builtin_amdgcn_readfirstlane(tid / TM);
+#pragma unroll
+                for (int k = 0; k < SHARE_MAX; ++k)
+                    if (k * SHARES + share < a.tap_corr)
+                        s_add[(int)((a.tap_classes >> (4 * (k * SHARES + share))) & 15) * ADD_ROW + i] = add + a.x_zp * border[k];
+            }
+        }
     }
     __syncthreads();
 
@@ -411,6 +459,24 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
     // (v / 4) * 8 + (lane >> 5) * 4 + (v % 4)
     v16i acc[FM][FN];
     auto seed_acc = [&]() {
+        if constexpr (kPad == 1) {
+            // the row of the pixel's class (s_cls holds the classes of the tile about to be computed: the copy side wrote
+            // them when it turned to that tile, at least one barrier ago, and turns to the tile after it only once this
+            // one is under way)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const int32_t* row = &s_add[s_cls[wn * 32 * FN + j * 32 + (lane & 31)] * ADD_ROW + wm * 32 * FM + (lane >> 5) * 4];
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const v4i ad = *reinterpret_cast<const v4i*>(&row[i * 32 + g * 8]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] = ad[e];
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -823,7 +889,34 @@ int launch_config(const ConvMfmaArgs& a_in, bool x_unsigned, bool out_int32, boo
     // no tap can leave the image: 0; else 1 when the zero point is the byte 0 and 32 bits hold a pixel's tap mask (a tap
     // outside the image is fetched as zeros), 2 otherwise (it is fetched from a row of zero points)
     const bool pad = a.ph != 0 || a.pw != 0 || (int64_t)(a.OH - 1) * a.sh + a.KH > a.H || (int64_t)(a.OW - 1) * a.sw + a.KW > a.W;
-    const int pad_mode = !pad ? 0 : ((a.x_zp & 0xff) == 0 && a.KH * a.KW <= 32) ? 1 : 2;
+    // (with another zero point still 1 when the accumulators can start from what the zeros miss: border sums packed, the
+    // window leaves the image by at most one row or column per side, and enough K steps per tile that the copy side is
+    // never more than one tile ahead of the seeding, which reads the classes it leaves in LDS)
+    const int last_ih0 = (a.OH - 1) * a.sh - a.ph, last_iw0 = (a.OW - 1) * a.sw - a.pw;
+    const int below = a.KH - (a.H - last_ih0 < 0 ? 0 : a.H - last_ih0 > a.KH ? a.KH : a.H - last_ih0);
+    const int right = a.KW - (a.W - last_iw0 < 0 ? 0 : a.W - last_iw0 > a.KW ? a.KW : a.W - last_iw0);
+    const bool class_seeds = a.padsum != nullptr && a.ph <= 1 && a.pw <= 1 && below <= 1 && right <= 1 && a.nk >= 4;
+    const int pad_mode = !pad ? 0 : (a.KH * a.KW <= 32 && ((a.x_zp & 0xff) == 0 || class_seeds)) ? 1 : 2;
+    a.tap_corr = 0;
+    a.tap_classes = 0;
+    if (pad_mode == 1 && (a.x_zp & 0xff) != 0) {
+        // the classes in use: 4 * (2 * rows outside above + rows outside below) + 2 * columns outside left + columns outside
+        // right, over the output rows and columns that can differ from the interior (the first and the last few)
+        auto sides = [](int O, int stride, int p, int I, int K) {
+            uint32_t seen = 0;
+            for (int o = 0; o < O; ++o) {
+                if (o == 4 && O > 8) o = O - 4;
+                const int i0 = o * stride - p;
+                const int lo = -i0 < 0 ? 0 : -i0 > K ? K : -i0, hi = I - i0 < 0 ? 0 : I - i0 > K ? K : I - i0;
+                seen |= 1u << ((lo * 2 + (K - hi)) & 3);
+            }
+            return seen;
+        };
+        const uint32_t rows = sides(a.OH, a.sh, a.ph, a.H, a.KH), cols = sides(a.OW, a.sw, a.pw, a.W, a.KW);
+        for (int cls = 1; cls < 16; ++cls)
+            if (((rows >> (cls >> 2)) & 1) && ((cols >> (cls & 3)) & 1)) a.tap_classes |= (uint64_t)cls << (4 * a.tap_corr++);
+        // (padding means that some pixel has a tap outside: at least one class besides 0)
+    }
 #define CHX_LAUNCH_R(XU, OI, RN, RS)                                                    \
     do {                                                                                \
         if (pad_mode == 0)                                                              \

@@ -447,9 +447,9 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
     // way stores plain codes and the readers see that from the array's type), and every reader is a QLinearConv that
     // takes the value as its input, or a residual-sum group computed inside a convolution that takes it as the other
     // operand (QLinearConvWithResidualOp puts plain codes back when its convolution does not compute the group after
-    // all).  A reading convolution with padding is left out: it pads with its input's zero point, and only a zero
-    // point stored as the byte 0 comes from the padding that costs nothing; the codes of a zero point of 0, the usual
-    // one behind a Relu, are stored as 0x80.
+    // all).  A reading convolution with pads above 1 is left out: it pads with its input's zero point, and beyond one
+    // row or column per side only a zero point stored as the byte 0 comes from the padding that costs nothing; the
+    // codes of a zero point of 0, the usual one behind a Relu, are stored as 0x80.
     minus_128_slots_.assign(num_variables_ > 0 ? num_variables_ : 1, false);
     if (g_store_minus_128) {
         std::vector<int> verdict(minus_128_slots_.size(), 0);  // 0 unseen, 1 possible so far, -1 no
@@ -472,9 +472,9 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
             if (inst.op == kFree) continue;
             int conv_input = -1, residual_operand = -1;
             if (conv && role[i] != 1) {
-                bool unpadded = inst.inputs[12].s.empty() || inst.inputs[12].s == "NOTSET" || inst.inputs[12].s == "VALID";
-                for (int64_t pad : inst.inputs[10].ints) unpadded = unpadded && pad == 0;
-                if (unpadded) conv_input = inst.inputs[0].array;
+                bool small_pads = inst.inputs[12].s.empty() || inst.inputs[12].s == "NOTSET" || inst.inputs[12].s == "VALID";
+                for (int64_t pad : inst.inputs[10].ints) small_pads = small_pads && pad >= 0 && pad <= 1;
+                if (small_pads) conv_input = inst.inputs[0].array;
             }
             if (role[i] == 5) residual_operand = inst.inputs[0].array_list[1 - conv_operand[partner[i]]];
             for (const ChxVMValueProto& v : inst.inputs) {

@@ -93,7 +93,7 @@ int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
  * name "pair_convolutions": value "on" (default) or "off": whether two QLinearConv that read the same
  * value with the same strides, pads and kernel size (the main-path and the shortcut convolution of a
  * down-sampling block) run as one launch (decided when a program is loaded);
- * name "store_minus_128": value "on" (default) or "off": whether a uint8 value that only unpadded QLinearConv
+ * name "store_minus_128": value "on" (default) or "off": whether a uint8 value that only QLinearConv with pads of at most 1
  * read (as input, or as the residual operand of a sum computed inside one) is kept as code - 128 in an int8
  * array between them, which spares the reading kernel its sign flips (decided when a program is loaded; a
  * run with check_types or dump_outputs_dir stores plain codes);

@@ -248,7 +248,7 @@ def test_small_resnet_as_one_program(g, vm, oracle):
     # only the logits: each of the five residual sums is computed by the convolution before it
     blocks = sum(1 for ins in model["program"] if ins[0] == "AddRelu")
     assert blocks == 5
-    # The values only unpadded convolutions read (as input or as the residual operand of an absorbed sum) are kept as
+    # The values only convolutions read (as input or as the residual operand of an absorbed sum) are kept as
     # code - 128: what the Python runner's analysis finds on the same program with the same fusions.
     runner = wl.DeviceRunner(model, g.pkg, fuse_residual=True, pair_convs=True, minus_128=True)
     kept_minus_128 = len(runner.minus_128)

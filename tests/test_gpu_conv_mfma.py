@@ -144,3 +144,70 @@ def test_full_size_conv_properties(g, oracle):
     ones = torch.ones_like(xd)
     taps = g.ops.ConvInteger(ones, g.dev(w), 0, None, pads=(1, 1))   # per-position sum of in-image taps
     assert torch.equal(ci(w, 100) - full, 28 * taps)
+
+
+PADDED_WINDOWS = [
+    # N, C, H, W, OC, KH, KW, strides, pads
+    (2, 32, 1, 1, 32, 3, 3, (1, 1), (1, 1)),      # a window that leaves the image on all four sides
+    (2, 64, 2, 5, 48, 3, 3, (1, 1), (1, 1)),      # ... above and below at once
+    (1, 64, 8, 8, 64, 3, 3, (2, 2), (1, 1)),      # stride 2 over an even image: nothing below or to the right
+    (1, 64, 9, 7, 64, 3, 3, (2, 2), (1, 1)),      # ... over an odd one
+    (1, 256, 6, 6, 64, 1, 1, (1, 1), (1, 1)),     # a single tap that can lie outside altogether
+    (1, 64, 6, 6, 32, 2, 2, (1, 1), (1, 1)),
+    (1, 16, 10, 10, 32, 5, 5, (1, 1), (1, 1)),    # 25 taps, one row or column outside per side
+    (1, 16, 10, 10, 32, 5, 5, (1, 1), (2, 2)),    # two outside: the copies fetch rows of zero points
+    (1, 64, 6, 6, 32, 3, 1, (1, 1), (1, 0)),
+    (1, 64, 6, 6, 32, 1, 3, (1, 1), (0, 1)),
+    (24, 16, 56, 56, 32, 3, 3, (1, 1), (1, 1)),   # more pixel tiles than resident work-groups: each walks over several
+]
+
+
+@pytest.mark.parametrize("case", PADDED_WINDOWS)
+@pytest.mark.parametrize("xdt", [np.uint8, np.int8])
+def test_padding_with_any_zero_point(g, oracle, case, xdt):
+    """Taps outside the image count as the activation zero point.  The matrix-core kernel fetches them as zeros and,
+    for a zero point that is not the byte 0, starts each pixel's accumulators from what those zeros miss (windows that
+    leave the image by at most one row or column per side); QLinearConv and ConvInteger against the oracle for zero
+    points at both ends and inside the range, every tile shape on one of the cases."""
+    import os
+    N, C, H, W, OC, KH, KW, strides, pads = case
+    rng = np.random.default_rng(41)
+    x, w, ws, wz, bias, ys = make_case(rng, N, C, H, W, OC, KH, KW, xdt)
+    zps = (0, 1, 128, 255) if xdt == np.uint8 else (-128, -1, 0, 5, 127)
+    big = N * H * W > 10000
+    if big:
+        zps = zps[1:3]
+        oracle.set_threads(16)
+    xd = g.to_channels_last(g.dev(x))
+    plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), strides=strides, pads=pads)
+    try:
+        for zp in zps:
+            want = oracle.qlinear_conv_int(x, 0.02, zp, w, ws, wz, ys, 128, np.uint8, bias=bias, strides=strides, pads=pads,
+                                           bias_mode=oracle.BIAS_ONNX_INT32)
+            got = plan.run(xd, 0.02, zp, ys, 128, torch.uint8, flags=g.capi.BIAS_ONNX_INT32)
+            np.testing.assert_array_equal(g.host(got), want, err_msg="zero point %d" % zp)
+            if not big:
+                want_int = oracle.conv_integer(x, w, zp, None, strides=strides, pads=pads)
+                np.testing.assert_array_equal(g.host(g.ops.ConvInteger(xd, g.dev(w), zp, None, strides=strides, pads=pads)), want_int,
+                                              err_msg="ConvInteger, zero point %d" % zp)
+    finally:
+        plan.close()
+        oracle.set_threads(1)
+    if case != PADDED_WINDOWS[3]:
+        return
+    zp = zps[1]
+    want = oracle.qlinear_conv_int(x, 0.02, zp, w, ws, wz, ys, 128, np.uint8, bias=bias, strides=strides, pads=pads,
+                                   bias_mode=oracle.BIAS_ONNX_INT32)
+    before = os.environ.get("CHX_HIP_TILE")
+    try:
+        for tile in ("128,128,0,4", "128,64,0,4", "64,128,0,4", "64,64,0,4", "128,128,0,8", "128,256,0,8", "64,128,0,8"):
+            os.environ["CHX_HIP_TILE"] = tile
+            plan = g.ops.QLinearConvPlan(g.dev(w), g.dev(ws), g.dev(wz), g.dev(bias), strides=strides, pads=pads)
+            got = plan.run(xd, 0.02, zp, ys, 128, torch.uint8, flags=g.capi.BIAS_ONNX_INT32)
+            plan.close()
+            np.testing.assert_array_equal(g.host(got), want, err_msg="tile %s" % tile)
+    finally:
+        if before is None:
+            os.environ.pop("CHX_HIP_TILE", None)
+        else:
+            os.environ["CHX_HIP_TILE"] = before
