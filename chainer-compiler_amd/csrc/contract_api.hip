@@ -875,6 +875,7 @@ int run_depthwise(const ConvCall& c, const DepthwiseState& st, hipStream_t s) {
     a.q = c.rq.q;
     a.inv_y_scale = 1.0f / c.rq.q.scale;
     a.lo_folded = fold_relu_floor(c.rq.q, c.rq.relu_floor, c.rne);
+    a.y_flip = c.y_minus_128 ? 0x80808080u : 0u;  // (c.y is then the uint8 view of the caller's int8 array)
     return launch_depthwise3x3(a, c.rne, s);
 }
 
@@ -1169,11 +1170,13 @@ extern "C" int chx_hip_qconv_plan_run(
         const int rc = run_conv_mfma(call, plan->pw, s);
         if (rc != CHX_HIP_EUNSUPPORTED || minus_128) return rc;
     }
-    if (minus_128) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv: codes minus 128 are stored by the matrix-core kernel only");
     if (plan->depthwise) {
-        const int rc = run_depthwise(conv_call_from(q, x, y, &plan->params, rne, plan->opt), plan->dw, s);
-        if (rc != CHX_HIP_EUNSUPPORTED) return rc;
+        ConvCall call = conv_call_from(q, x, &yv, &plan->params, rne, plan->opt);
+        call.y_minus_128 = minus_128;
+        const int rc = run_depthwise(call, plan->dw, s);
+        if (rc != CHX_HIP_EUNSUPPORTED || minus_128) return rc;
     }
+    if (minus_128) CHX_FAIL(CHX_HIP_EUNSUPPORTED, "QLinearConv: codes minus 128 are stored by the matrix-core and the depthwise kernel only");
     return launch_conv_direct(q.direct, rne, s);
 }
 

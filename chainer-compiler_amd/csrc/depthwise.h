@@ -25,6 +25,7 @@ struct DepthwiseArgs {
     QuantParams q;
     float inv_y_scale;
     float lo_folded;
+    uint32_t y_flip;        // 0x80808080: every stored byte is the uint8 code minus 128 (CHX_HIP_STORE_MINUS_128), else 0
     int32_t oh_blocks;      // filled by the launcher
     // The launch is one-dimensional: work-group b of the device's dispatch order (which deals work-groups out to the 8
     // XCDs in turn) takes block (b % 8) * xcd_chunk + b / 8 of the (x blocks of a row strip, row strips, images) order, so

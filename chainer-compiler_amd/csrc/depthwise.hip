@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kDwThreads) void depthwise3x3_kernel(DepthwiseArgs 
             else code[e] = quantize_value_folded<kRne>(v, a.q, a.inv_y_scale, a.lo_folded);
         }
         const uint32_t o = kPath ? floor_sat_u8x4(pre[0], pre[1], pre[2], pre[3]) : pack4(code[0], code[1], code[2], code[3]);
-        if (oh < a.OH) *reinterpret_cast<uint32_t*>(yn + (int64_t)oh * a.y_h_stride + y_off) = o;
+        if (oh < a.OH) *reinterpret_cast<uint32_t*>(yn + (int64_t)oh * a.y_h_stride + y_off) = o ^ a.y_flip;
     };
 
     // filter rows and per-channel constants; requested after the strip's input rows so that all of it is in flight together

@@ -445,7 +445,7 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
     // Values that may be kept as code - 128 in int8 arrays (ChxVMState::store_minus_128): every writer is a QLinearConv
     // or a residual-sum group computed inside one (the producers that know the storage; a writer that runs some other
     // way stores plain codes and the readers see that from the array's type), and every reader is a QLinearConv that
-    // takes the value as its input, or a residual-sum group computed inside a convolution that takes it as the other
+    // without groups that takes the value as its input, or a residual-sum group computed inside a convolution that takes it as the other
     // operand (QLinearConvWithResidualOp puts plain codes back when its convolution does not compute the group after
     // all).  A reading convolution with pads above 1 is left out: it pads with its input's zero point, and beyond one
     // row or column per side only a zero point stored as the byte 0 comes from the padding that costs nothing; the
@@ -474,7 +474,8 @@ ChxVM::ChxVM(const ChxVMProgramProto& program) : input_names_(program.input_name
             if (conv && role[i] != 1) {
                 bool small_pads = inst.inputs[12].s.empty() || inst.inputs[12].s == "NOTSET" || inst.inputs[12].s == "VALID";
                 for (int64_t pad : inst.inputs[10].ints) small_pads = small_pads && pad >= 0 && pad <= 1;
-                if (small_pads) conv_input = inst.inputs[0].array;
+                // (a grouped convolution gains nothing from the storage)
+                if (small_pads && inst.inputs[11].i == 1) conv_input = inst.inputs[0].array;
             }
             if (role[i] == 5) residual_operand = inst.inputs[0].array_list[1 - conv_operand[partner[i]]];
             for (const ChxVMValueProto& v : inst.inputs) {

@@ -307,15 +307,18 @@ def pair_convolutions(program, convs):
 def minus_128_values(program, convs, fused_into):
     """The values of `program` that can be stored as code - 128 in int8 arrays (CHX_HIP_STORE_MINUS_128): written by the
     matrix-core convolution kernel (a QLinearConv that is not grouped and has at least 16 input channels, a pair of them,
-    or the residual sum inside one) and read only by convolutions, as their input or as the residual operand of a sum
-    that one of them computes.  A reading convolution whose window leaves the image by more than one row or column
+    or the residual sum inside one) or by the depthwise 3x3 kernel, and read only by convolutions that are not grouped (the
+    depthwise kernel gains nothing from the storage), as their input or as the residual operand of a sum that one of
+    them computes.  A reading convolution whose window leaves the image by more than one row or column
     must find the padding value, its input's zero point, stored as the byte 0 (a uint8 zero point of 128), or it does
     not run with the padding that costs nothing; a value with such a reader and another zero point keeps its uint8 array.
     `fused_into`: convolution result -> the Add instruction computed inside that convolution."""
     fused_adds = set(add[1] for add in fused_into.values())
     producers = {}
     for ins in program:
-        if ins[0] == "QLinearConv" and convs[ins[3]].group == 1 and convs[ins[3]].wq.shape[1] >= 16:
+        c = convs[ins[3]] if ins[0] == "QLinearConv" else None
+        depthwise = c is not None and c.group > 1 and c.group % 16 == 0 and tuple(c.wq.shape) == (c.group, 1, 3, 3)
+        if c is not None and ((c.group == 1 and c.wq.shape[1] >= 16) or depthwise):
             producers[fused_into[ins[1]][1] if ins[1] in fused_into else ins[1]] = ins
         if ins[0] == "QLinearConvPair":
             producers[ins[1]] = producers[ins[4]] = ins
@@ -327,7 +330,7 @@ def minus_128_values(program, convs, fused_into):
                 if ins[2] == name:
                     readers += 1
                     c = convs[ins[3]]
-                    if c.pad > 1 and c.x_zp != 128:
+                    if (c.pad > 1 and c.x_zp != 128) or c.group != 1:
                         ok = False
             elif ins[0] in ("Add", "AddRelu") and ins[1] in fused_adds:
                 # computed inside a convolution: `name` may be its residual operand, not the convolution's own result

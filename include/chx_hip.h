@@ -74,7 +74,7 @@ enum {
      * zp - 128 denotes the same numbers, so a later QLinearConv reads it as its int8 x (or a fused residual sum as its
      * int8 r) with that zero point and gives the bytes it would give on the uint8 array, without flipping sign bits in
      * its inner loop.  No counterpart in the reference; a storage convention between the convolutions of one host.
-     * CHX_HIP_EUNSUPPORTED where the matrix-core kernel does not run (store uint8 then). */
+     * CHX_HIP_EUNSUPPORTED where neither the matrix-core kernel nor the depthwise 3x3 kernel runs (store uint8 then). */
     CHX_HIP_STORE_MINUS_128 = 8u
 };
 

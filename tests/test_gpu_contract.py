@@ -661,6 +661,28 @@ def test_results_stored_minus_128(g, oracle):
         assert e.value.code == g.capi.EUNSUPPORTED
         for p in (p1, p2, pp):
             p.close()
+        # the depthwise 3x3 kernel stores the codes minus 128 as well; a grouped convolution of another shape does not
+        Cd = 32
+        xdw = rand_q(rng, (2, Cd, 9, 10), np.uint8)
+        wdw = rng.integers(-127, 128, size=(Cd, 1, 3, 3)).astype(np.int8)
+        wsd = rng.uniform(0.002, 0.02, size=Cd).astype(np.float32)
+        bd = rng.integers(-500, 501, size=Cd).astype(np.int32)
+        yds = np.float32(0.02 * 0.01 * 74 * 74 * 3 / 40)
+        kwd = dict(strides=(1, 1), pads=(1, 1), group=Cd)
+        want_dw = oracle.qlinear_conv_int(xdw, 0.02, 101, wdw, wsd, np.zeros(Cd, np.int8), yds, 119, np.uint8, bias=bd,
+                                          bias_mode=oracle.BIAS_ONNX_INT32, **kwd)
+        pd = g.ops.QLinearConvPlan(g.dev(wdw), g.dev(wsd), g.dev(np.zeros(Cd, np.int8)), g.dev(bd), **kwd)
+        xdd = g.to_channels_last(g.dev(xdw))
+        np.testing.assert_array_equal(g.host(pd.run(xdd, 0.02, 101, yds, 119, torch.uint8, flags=F)), want_dw)
+        np.testing.assert_array_equal(g.host(flip(pd.run(xdd, 0.02, 101, yds, 119, torch.int8, flags=S))), want_dw)
+        np.testing.assert_array_equal(g.host(flip(pd.run(g.ops.codes_minus_128(xdd), 0.02, 101 - 128, yds, 119, torch.int8, flags=S))), want_dw)
+        pd.close()
+        wg = rng.integers(-127, 128, size=(Cd, 2, 3, 3)).astype(np.int8)
+        pg = g.ops.QLinearConvPlan(g.dev(wg), g.dev(wsd), g.dev(np.zeros(Cd, np.int8)), g.dev(bd), strides=(1, 1), pads=(1, 1), group=Cd // 2)
+        with pytest.raises(g.capi.ChxHipError) as e:
+            pg.run(xdd, 0.02, 101, yds, 119, torch.int8, flags=S)
+        assert e.value.code == g.capi.EUNSUPPORTED
+        pg.close()
 
 
 def test_random_convolution_sweep(g, oracle):
