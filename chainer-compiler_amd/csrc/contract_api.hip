@@ -698,7 +698,9 @@ int make_packed(const chx_hip_tensor& w, bool persistent, hipStream_t s, PackedW
             stem ? (size_t)(pw->OCpad / 64) * stem_k_blocks((int)w.shape[1], (int)w.shape[2], (int)w.shape[3]) * 2048 : 0;
     const size_t bytes = mfma_bytes + stem_bytes;
     // the per-channel sums, and behind them the sixteen classes of border sums
-    const bool border_sums = !pw->dense && w.shape[2] * w.shape[3] <= 32;
+    // (between 2 and 32 taps: the kernel's tap masks hold 32, and a single tap that can lie outside is rare enough for
+    // the flat-address padding)
+    const bool border_sums = !pw->dense && w.shape[2] * w.shape[3] <= 32 && w.shape[2] * w.shape[3] > 1;
     const size_t sums_bytes = sizeof(int32_t) * pw->OCpad * (border_sums ? 17 : 1);
     void* p0 = nullptr;
     void* p1 = nullptr;

@@ -59,6 +59,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
     if (threadIdx.x < 32) tap_sum[threadIdx.x] = 0;
     __syncthreads();
     int32_t local = 0;
+    int32_t run = 0, run_pos = 0;  // this thread's sum over its elements of tap run_pos so far
     for (int k = threadIdx.x; k < KP; k += 256) {
         const int c = k % C64;
         const int pos = k / C64;
@@ -69,8 +70,16 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(
         }
         wp[packed_offset(oc, k, KP, BK)] = v;
         local += v;
-        if (padsum && v != 0) atomicAdd(&tap_sum[pos], (int32_t)v);
+        if (padsum) {
+            if (pos != run_pos) {
+                if (run != 0) atomicAdd(&tap_sum[run_pos], run);
+                run = 0;
+                run_pos = pos;
+            }
+            run += v;
+        }
     }
+    if (padsum && run != 0) atomicAdd(&tap_sum[run_pos], run);
     __shared__ int32_t red[256];
     red[threadIdx.x] = local;
     __syncthreads();
@@ -238,7 +247,7 @@ int pack_weights(
         const chx_hip_tensor& w, int C64, int BK, int OCpad, int8_t* wp, int32_t* wsum, int32_t* padsum, hipStream_t s) {
     pack_weights_kernel<<<OCpad, 256, 0, s>>>(
             static_cast<const char*>(w.data), w.strides[0], w.strides[1], w.strides[2], w.strides[3], (int)w.shape[0],
-            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, BK, wp, wsum, w.shape[2] * w.shape[3] <= 32 ? padsum : nullptr);
+            (int)w.shape[1], (int)w.shape[2], (int)w.shape[3], C64, BK, wp, wsum, padsum);
     return launch_check("pack_weights_kernel");
 }
 
