@@ -64,7 +64,8 @@ struct ConvMfmaArgs {
     int32_t x_zp;
     int32_t corr_mult;    // (128 - x_zp) for uint8 x, (-x_zp) for int8 x
     int32_t tap_corr;     // not 0: taps outside the image arrive as zeros although the zero point is not the byte 0, and the accumulators start from the pixel's class of padsum; the number of classes other than 0 that occur (launcher)
-    uint64_t tap_classes; // those classes, four bits each from bit 0 up (launcher)
+    uint64_t tap_classes; // those classes (at most eight), four bits each from bit 0 up (launcher)
+    uint64_t tap_rows;    // per class (four bits each, class c at bit 4c): its row of the work-group's seed table, the class's place in tap_classes + 1; 0 for class 0 (launcher)
     // output, pixel-major: element (m, oc) at y + m*y_px_stride + oc*elemsize
     char* y;
     int64_t y_px_stride;

@@ -175,10 +175,10 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
     static_assert(TN * TM <= STAGE_BYTES, "the output tile is staged in one ring slot");
     __shared__ __attribute__((aligned(16))) char ring[NS * STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) float s_scale[TM];
-    // what the accumulators start from, per output channel; kPad 1: sixteen rows, one per class of taps outside the image
-    // (ConvMfmaArgs::padsum), row 0 for a pixel whose taps are all inside, and each staged pixel's class
+    // what the accumulators start from, per output channel; kPad 1: up to nine rows, one per class of taps outside the
+    // image that occurs (ConvMfmaArgs::padsum), row 0 for a pixel whose taps are all inside, and each staged pixel's row
     constexpr int ADD_ROW = TM + 8;  // (rows 32 bytes off a multiple of the bank width: lanes that read different rows do not meet on a bank)
-    __shared__ __attribute__((aligned(16))) int32_t s_add[kPad == 1 ? 16 * ADD_ROW : TM];
+    __shared__ __attribute__((aligned(16))) int32_t s_add[kPad == 1 ? 9 * ADD_ROW : TM];
     __shared__ int32_t s_cls[kPad == 1 ? TN : 1];
     __shared__ __attribute__((aligned(16))) float s_fbias[TM];
 
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
                         if constexpr (kPad == 1) {
                             // which sides the window leaves the image on (at most one row or column per side: the launcher
                             // has checked); every lane of the row writes the same word
-                            s_cls[rowB] = a.tap_corr ? r_lo * 8 + (a.KH - r_hi) * 4 + c_lo * 2 + (a.KW - c_hi) : 0;
+                            s_cls[rowB] = a.tap_corr ? (int)((a.tap_rows >> (4 * (r_lo * 8 + (a.KH - r_hi) * 4 + c_lo * 2 + (a.KW - c_hi)))) & 15) : 0;
                         }
                     } else {
                         const uint64_t below_hi = c_hi >= 64 ? ~(uint64_t)0 : ((uint64_t)1 << c_hi) - 1;  // a 1x64 filter fills the mask
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
     // together with the first copies.  The T / TM threads of an output channel share the classes out (a wavefront
     // holds one share); every instruction here delays the work-group's first matrix instruction.
     constexpr int SHARES = T / TM;
-    constexpr int SHARE_MAX = (15 + SHARES - 1) / SHARES;
+    constexpr int SHARE_MAX = (8 + SHARES - 1) / SHARES;
     static_assert(T % TM == 0 && TM % 64 == 0, "whole wavefronts per share of the classes");
     int32_t border[SHARE_MAX];
     if constexpr (kPad == 1) {
@@ -449,7 +449,7 @@ __global__ __launch_bounds__(128 * NWN) __attribute__((amdgpu_waves_per_eu(2))) 
 #pragma unroll
                 for (int k = 0; k < SHARE_MAX; ++k)
                     if (k * SHARES + share < a.tap_corr)
-                        s_add[(int)((a.tap_classes >> (4 * (k * SHARES + share))) & 15) * ADD_ROW + i] = add + a.x_zp * border[k];
+                        s_add[(k * SHARES + share + 1) * ADD_ROW + i] = add + a.x_zp * border[k];  // the class's row: its place in the list + 1
             }
         }
     }
@@ -895,11 +895,12 @@ int launch_config(const ConvMfmaArgs& a_in, bool x_unsigned, bool out_int32, boo
     const int last_ih0 = (a.OH - 1) * a.sh - a.ph, last_iw0 = (a.OW - 1) * a.sw - a.pw;
     const int below = a.KH - (a.H - last_ih0 < 0 ? 0 : a.H - last_ih0 > a.KH ? a.KH : a.H - last_ih0);
     const int right = a.KW - (a.W - last_iw0 < 0 ? 0 : a.W - last_iw0 > a.KW ? a.KW : a.W - last_iw0);
-    const bool class_seeds = a.padsum != nullptr && a.ph <= 1 && a.pw <= 1 && below <= 1 && right <= 1 && a.nk >= 4;
-    const int pad_mode = !pad ? 0 : (a.KH * a.KW <= 32 && ((a.x_zp & 0xff) == 0 || class_seeds)) ? 1 : 2;
     a.tap_corr = 0;
     a.tap_classes = 0;
-    if (pad_mode == 1 && (a.x_zp & 0xff) != 0) {
+    a.tap_rows = 0;
+    bool class_seeds = pad && (a.x_zp & 0xff) != 0 && a.KH * a.KW <= 32 && a.padsum != nullptr && a.ph <= 1 && a.pw <= 1 && below <= 1 &&
+                       right <= 1 && a.nk >= 4;
+    if (class_seeds) {
         // the classes in use: 4 * (2 * rows outside above + rows outside below) + 2 * columns outside left + columns outside
         // right, over the output rows and columns that can differ from the interior (the first and the last few)
         auto sides = [](int O, int stride, int p, int I, int K) {
@@ -913,10 +914,24 @@ int launch_config(const ConvMfmaArgs& a_in, bool x_unsigned, bool out_int32, boo
             return seen;
         };
         const uint32_t rows = sides(a.OH, a.sh, a.ph, a.H, a.KH), cols = sides(a.OW, a.sw, a.pw, a.W, a.KW);
+        int count = 0;
+        uint64_t classes = 0, table_rows = 0;
         for (int cls = 1; cls < 16; ++cls)
-            if (((rows >> (cls >> 2)) & 1) && ((cols >> (cls & 3)) & 1)) a.tap_classes |= (uint64_t)cls << (4 * a.tap_corr++);
-        // (padding means that some pixel has a tap outside: at least one class besides 0)
+            if (((rows >> (cls >> 2)) & 1) && ((cols >> (cls & 3)) & 1)) {
+                classes |= (uint64_t)cls << (4 * count);
+                ++count;
+                table_rows |= (uint64_t)(count & 15) << (4 * cls);
+            }
+        // (padding means that some pixel has a tap outside: at least one class besides 0; more than eight only where a
+        // window leaves the image on opposite sides at once, images one or two pixels high or wide)
+        class_seeds = count >= 1 && count <= 8;
+        if (class_seeds) {
+            a.tap_corr = count;
+            a.tap_classes = classes;
+            a.tap_rows = table_rows;
+        }
     }
+    const int pad_mode = !pad ? 0 : (a.KH * a.KW <= 32 && ((a.x_zp & 0xff) == 0 || class_seeds)) ? 1 : 2;
 #define CHX_LAUNCH_R(XU, OI, RN, RS)                                                    \
     do {                                                                                \
         if (pad_mode == 0)                                                              \
