@@ -399,7 +399,8 @@ class Program:
         _check(runtime().chxvm_program_set_option(self._h, name.encode(), value.encode()))
 
     def counter(self, name):
-        """Event counts of this program over all its runs, e.g. "qlinearconv_residual_fusions"."""
+        """Event counts of this program over all its runs, e.g. "qlinearconv_residual_fusions"; "minus_128_variables" is
+        the number of variables the loader marked to be kept as code - 128 between convolutions."""
         return runtime().chxvm_program_counter(self._h, name.encode())
 
     def close(self):

@@ -59,6 +59,13 @@ public:
         return residual_fusions_;
     }
 
+    // variables of the program that its convolutions keep as code - 128 between them (ChxVMState::store_minus_128)
+    int64_t minus_128_variables() const {
+        int64_t n = 0;
+        for (bool marked : minus_128_slots_) n += marked ? 1 : 0;
+        return n;
+    }
+
     int num_variables() const {
         return num_variables_;
     }

@@ -329,6 +329,7 @@ int32_t chxvm_program_set_option(chxvm_program* program, const char* name, const
 int64_t chxvm_program_counter(const chxvm_program* program, const char* name) {
     const std::string n = name ? name : "";
     if (program && n == "qlinearconv_residual_fusions") return program->vm->residual_fusions();
+    if (program && n == "minus_128_variables") return program->vm->minus_128_variables();
     return -1;
 }
 

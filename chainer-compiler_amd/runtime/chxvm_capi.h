@@ -83,7 +83,8 @@ void chxvm_replay_destroy(chxvm_replay* replay);
  * "reference", "onnx_int32", or "default" (follow chxvm_set_option again).  Programs with different
  * settings may run in one process, also concurrently. */
 int32_t chxvm_program_set_option(chxvm_program* program, const char* name, const char* value);
-/* Event counts of one program over all its runs; names as for chxvm_counter. */
+/* Event counts of one program over all its runs; names as for chxvm_counter.  "minus_128_variables": how many
+ * variables of the program the loader marked to be kept as code - 128 between convolutions (fixed at load). */
 int64_t chxvm_program_counter(const chxvm_program* program, const char* name);
 
 /* Process-wide defaults, read when a run starts.

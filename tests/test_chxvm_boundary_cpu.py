@@ -388,3 +388,85 @@ def test_whole_network_as_one_program(chxvm):
     ctx.output("y", y)
     with pytest.raises(chxvm.ChxVMError, match="backward context"):
         chxvm.Program(ctx.serialize())
+
+
+def test_loader_marks_values_only_convolutions_read(chxvm):
+    """Which variables a program's convolutions may keep as code - 128 between them is decided when the program is
+    loaded: written by a QLinearConv, read only by QLinearConv without groups and with pads of at most 1 (as input),
+    and by nothing else; not a program output."""
+    def program(second_pads=(1, 1), second_group=1, extra_reader=False):
+        b = chxvm.ProgramBuilder()
+        x = b.input("x", "uint8", (1, 16, 8, 8))
+        ws = [b.input("w%d" % i, "int8", (16, 16 // (second_group if i == 1 else 1), 3, 3)) for i in range(3)]
+        sc, zp = b.input("w_scale", "float32", (16,)), b.input("w_zero_point", "int8", (16,))
+
+        def conv(v, w, pads, group=1):
+            return b.QLinearConv(v, b.scalar(0.02, "float32"), b.scalar(3, "uint8"), w, sc, zp, b.scalar(0.05, "float32"),
+                                 b.scalar(7, "uint8"), None, [1, 1], list(pads), group, "")
+        a = conv(x, ws[0], (1, 1))
+        c = conv(a, ws[1], second_pads, second_group)
+        d = conv(c, ws[2], (1, 1))
+        if extra_reader:
+            b.output("a_float", b.DequantizeLinear(a, b.scalar(0.05, "float32"), b.scalar(7, "uint8")))
+        b.output("d", d)
+        return b.serialize()
+
+    def marked(data):
+        prog = chxvm.Program(data)
+        n = prog.counter("minus_128_variables")
+        prog.close()
+        return n
+    assert marked(program()) == 2                       # a and c; x is the caller's, d goes back to the caller
+    assert marked(program(second_pads=(2, 2))) == 1     # a's reader pads by two rows: a keeps plain codes
+    assert marked(program(second_group=2)) == 1         # a grouped reader
+    assert marked(program(extra_reader=True)) == 1      # a DequantizeLinear reads a as well
+    chxvm.set_option("store_minus_128", "off")
+    try:
+        assert marked(program()) == 0
+    finally:
+        chxvm.set_option("store_minus_128", "on")
+
+
+def test_loader_marks_the_operands_of_absorbed_residual_sums(chxvm):
+    """A value that a residual-sum group reads as its other operand stays markable while the group is computed inside
+    the convolution before it (the group's own result is then a convolution's result too); with that fusion switched
+    off the group is a reader of its own and neither value is marked."""
+    import numpy as np
+    import torch
+    pkg = entry.load_package()
+    from importlib import import_module
+    ops = import_module(pkg.__name__ + ".ops")
+    u8 = torch.uint8
+
+    def scale_bits(v):
+        return "0x%08x" % np.float32(v).view(np.uint32)
+    code = ops.fusion_program(
+        [("a", u8), ("b", u8)],
+        [("fa", "DequantizeLinear", "a", scale_bits(0.05), 7), ("fb", "DequantizeLinear", "b", scale_bits(0.05), 7),
+         ("s", "Add", "fb", "fa"), ("r", "Relu", "s"), ("q", "QuantizeLinear", "r", scale_bits(0.05), 7, "uint8")], [("q", u8)])
+
+    def marked():
+        b = chxvm.ProgramBuilder()
+        x = b.input("x", "uint8", (1, 16, 8, 8))
+        ws = [b.input("w%d" % i, "int8", (16, 16, 1, 1)) for i in range(3)]
+        sc, zp = b.input("w_scale", "float32", (16,)), b.input("w_zero_point", "int8", (16,))
+
+        def conv(v, w):
+            return b.QLinearConv(v, b.scalar(0.02, "float32"), b.scalar(3, "uint8"), w, sc, zp, b.scalar(0.05, "float32"),
+                                 b.scalar(7, "uint8"), None, [1, 1], [0, 0], 1, "")
+        a = conv(x, ws[0])
+        y = conv(a, ws[1])
+        out = b.ElementWiseNvrtc([y, a], 1, code, 3, num_list_outputs=1)[0]
+        b.Free(y)
+        b.Free(a)
+        b.output("d", conv(out, ws[2]))
+        prog = chxvm.Program(b.serialize())
+        n = prog.counter("minus_128_variables")
+        prog.close()
+        return n
+    assert marked() == 2            # a (input of a convolution, other operand of the absorbed sum) and the sum
+    chxvm.set_option("fuse_residual", "off")
+    try:
+        assert marked() == 0
+    finally:
+        chxvm.set_option("fuse_residual", "on")
