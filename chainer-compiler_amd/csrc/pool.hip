@@ -37,15 +37,8 @@ __device__ __forceinline__ uint32_t max4_u8(uint32_t a, uint32_t b) {
     return r;
 }
 
-// Byte-wise maximum of two dwords kept as two dwords of 16-bit lanes (even bytes, odd bytes): the
-// packed 16-bit maximum then does two bytes per instruction.
+// The packed 16-bit maximum of two dwords (two 16-bit lanes per instruction).
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
-struct SplitBytes {
-    uint32_t even, odd;
-};
-__device__ __forceinline__ SplitBytes split_bytes(uint32_t x) {
-    return SplitBytes{x & 0x00ff00ffu, (x >> 8) & 0x00ff00ffu};
-}
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2us, a), __builtin_bit_cast(v2us, b)));
 }
@@ -55,6 +48,11 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
 // unconditional loads: a tap outside the image reads the nearest pixel inside instead, which
 // belongs to the same window whenever the window touches the image at all, so it does not change
 // the maximum (a branch around the load would make every load wait for the one before).
+// The maximum of the bytes of two dwords in three instructions: as 16-bit lanes the dwords compare by
+// their high (odd) bytes first, so the packed maximum of the raw dwords carries the maximum of the odd
+// bytes in its high bytes whatever the low bytes are; the even bytes are masked out and compared on
+// their own.
+template <bool kSigned>
 __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
     const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= a.total) return;
@@ -65,11 +63,11 @@ __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
     r /= a.OW;
     const int oh = (int)(r % a.OH);
     const int n = (int)(r / a.OH);
-    const uint32_t flip = a.is_signed ? 0x80808080u : 0u;
+    const uint32_t flip = kSigned ? 0x80808080u : 0u;
     const int ih0 = oh * a.sh - a.ph, iw0 = ow * a.sw - a.pw;
     const bool touches = ih0 < a.H && ih0 + a.kh > 0 && iw0 < a.W && iw0 + a.kw > 0;
     const char* xn = a.x + n * a.xs[0] + cg * 16;
-    SplitBytes m[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+    uint32_t m_odd[4] = {0, 0, 0, 0}, m_even[4] = {0, 0, 0, 0};
     const int taps = a.kh * a.kw;
     int i = 0, j = 0;
     for (int t0 = 0; t0 < taps; t0 += 9) {
@@ -88,9 +86,9 @@ __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
         for (int t = 0; t < 9; ++t)
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                const SplitBytes x = split_bytes(v[t][d] ^ flip);
-                m[d].even = pk_max_u16(m[d].even, x.even);
-                m[d].odd = pk_max_u16(m[d].odd, x.odd);
+                const uint32_t x = kSigned ? v[t][d] ^ flip : v[t][d];
+                m_odd[d] = pk_max_u16(m_odd[d], x);
+                m_even[d] = pk_max_u16(m_even[d], x & 0x00ff00ffu);
             }
     }
     // int8: the QuantizeLinear behind the pool adds 0.5 and truncates toward zero, so a negative code
@@ -99,8 +97,8 @@ __global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
     v4u out;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        uint32_t u = touches ? m[d].even | (m[d].odd << 8) : 0u;
-        if (a.is_signed) u += (~u >> 7) & 0x01010101u;
+        uint32_t u = touches ? m_even[d] | (m_odd[d] & 0xff00ff00u) : 0u;
+        if (kSigned) u += (~u >> 7) & 0x01010101u;
         out[d] = u ^ flip;
     }
     *reinterpret_cast<v4u*>(a.y + n * a.ys[0] + oh * a.ys[2] + ow * a.ys[3] + cg * 16) = out;
@@ -364,7 +362,8 @@ extern "C" int chx_hip_max_pool_q8(
                       aligned(y->data, 16) && px % 16 == 0 && py % 16 == 0;
     if (cl16) {
         a.total = (int64_t)a.N * a.OH * a.OW * (a.C / 16);
-        max_pool_cl16_kernel<<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
+        if (a.is_signed) max_pool_cl16_kernel<true><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
+        else max_pool_cl16_kernel<false><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
         return launch_check("max_pool_cl16_kernel");
     }
     max_pool_generic_kernel<<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
