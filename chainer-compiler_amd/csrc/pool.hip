@@ -52,9 +52,12 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
 // their high (odd) bytes first, so the packed maximum of the raw dwords carries the maximum of the odd
 // bytes in its high bytes whatever the low bytes are; the even bytes are masked out and compared on
 // their own.
+// The device deals work-groups out to its 8 XCDs in turn, each with its own L2: work-group b takes block
+// (b % 8) * xcd_chunk + b / 8, so that an XCD works through a contiguous run of output rows and finds the input rows
+// that neighbouring output rows share in its own L2 (the launch is xcd_chunk * 8 work-groups).
 template <bool kSigned>
-__global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a) {
-    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+__global__ __launch_bounds__(kThreads) void max_pool_cl16_kernel(PoolArgs a, uint32_t xcd_chunk) {
+    const int64_t idx = (int64_t)((blockIdx.x & 7u) * xcd_chunk + (blockIdx.x >> 3)) * kThreads + threadIdx.x;
     if (idx >= a.total) return;
     const int cgroups = a.C / 16;
     const int cg = (int)(idx % cgroups);
@@ -362,8 +365,11 @@ extern "C" int chx_hip_max_pool_q8(
                       aligned(y->data, 16) && px % 16 == 0 && py % 16 == 0;
     if (cl16) {
         a.total = (int64_t)a.N * a.OH * a.OW * (a.C / 16);
-        if (a.is_signed) max_pool_cl16_kernel<true><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
-        else max_pool_cl16_kernel<false><<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
+        const int64_t blocks = (a.total + kThreads - 1) / kThreads;
+        CHX_REQUIRE(blocks < (int64_t(1) << 31) - 8, "MaxPool: 2^31 work-groups or more");
+        const uint32_t xcd_chunk = (uint32_t)((blocks + 7) / 8);
+        if (a.is_signed) max_pool_cl16_kernel<true><<<xcd_chunk * 8, kThreads, 0, s>>>(a, xcd_chunk);
+        else max_pool_cl16_kernel<false><<<xcd_chunk * 8, kThreads, 0, s>>>(a, xcd_chunk);
         return launch_check("max_pool_cl16_kernel");
     }
     max_pool_generic_kernel<<<(unsigned)((a.total + kThreads - 1) / kThreads), kThreads, 0, s>>>(a);
