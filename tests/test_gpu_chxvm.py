@@ -283,6 +283,15 @@ def test_small_mobilenetv2_as_one_program(g, vm, oracle):
     adds = [ins[1] for ins in model["program"] if ins[0] == "Add"]
     assert len(adds) >= 1
     _run_network_through_vm(g, vm, oracle, model, ["logits"] + adds, fused_residuals=len(adds))
+    # only the logits: the block outputs and the depthwise results are kept as code - 128 between the convolutions, the
+    # values the Python runner's analysis names on the same program (the expansion results, which a depthwise
+    # convolution reads, keep plain codes)
+    runner = g.pkg.workloads.DeviceRunner(model, g.pkg, fuse_residual=True, pair_convs=True, minus_128=True)
+    kept_minus_128 = len(runner.minus_128)
+    runner.close()
+    depthwise = sum(1 for c in model["convs"].values() if c.group > 1)
+    assert kept_minus_128 >= depthwise >= 3
+    _run_network_through_vm(g, vm, oracle, model, ["logits"], fused_residuals=len(adds), minus_128=kept_minus_128)
 
 
 def test_residual_group_with_other_constants_runs_unfused(g, vm, oracle):
